@@ -1,0 +1,240 @@
+/*
+ * mongoose_hip.h -- C ABI of libmongoose_hip.so, the MI355X (gfx950) backend
+ * for mongoose's batch-1 fused quantized decode path.
+ *
+ * Plain C: pointers, sizes and ints only.  A "device pointer" is memory
+ * obtained from tw_gpu_alloc (or any hipMalloc); `stream` is a hipStream_t
+ * passed as void* (NULL = the default stream), exactly where the reference
+ * passes a cudaStream_t.  Reference paths are relative to the mongoose
+ * checkout.
+ *
+ * Three groups, mirroring what the reference's cgo blocks bind:
+ *   1. tw_gpu_*        device memory shim            (cuda_tensor.go:19-52)
+ *   2. mongoose_*      one launch per decode op      (kernels.go:12-72, 150-226;
+ *                                                     bodies kernels/mongoose.cu)
+ *   3. mg_*            fused-inference context: what CUDAFusedInference,
+ *                      CUDAStreamInfer and CUDAGraph do behind their Go methods
+ *                      (cuda_fused_infer.go, cuda_fused_infer_q4.go,
+ *                       cuda_q4_0.go, cuda_fused_stream.go, cuda_graph.go)
+ *
+ * Error convention.  The reference's kernels return void and report nothing;
+ * its Go methods return -1 when the object is not built.  Here mongoose_*
+ * keep the void signatures (so a dlsym table binds them unchanged) and record
+ * failures for mongoose_check(); mg_* return 0 on success and a negative
+ * MG_E_* code otherwise, with text in mg_last_error().
+ */
+#ifndef MONGOOSE_HIP_H
+#define MONGOOSE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MG_OK            0
+#define MG_E_NOT_BUILT  (-1)   /* same value the Go methods return when !built */
+#define MG_E_ARG        (-2)
+#define MG_E_HIP        (-3)
+#define MG_E_STATE      (-4)
+#define MG_E_UNSUPPORTED (-5)
+
+/* ------------------------------------------------------------------ */
+/* 1. Device memory shim                      cuda_tensor.go:19-52      */
+/* ------------------------------------------------------------------ */
+void* tw_gpu_alloc(size_t bytes);                               /* :19-28  NULL on failure (message on stderr) */
+void  tw_gpu_free(void* ptr);                                   /* :30-32 */
+void  tw_gpu_upload(void* dst, const void* src, size_t bytes);  /* :34-36  synchronous H2D */
+void  tw_gpu_download(void* dst, const void* src, size_t bytes);/* :38-40  synchronous D2H */
+void  tw_gpu_zero(void* ptr, size_t bytes);                     /* :42-44 */
+void* tw_gpu_alloc_pinned(size_t bytes);                        /* :47-52  page-locked host memory */
+void  tw_gpu_free_pinned(void* ptr);
+/* cuda.go:30-56 tw_cuda_init_device: select device, 0 on success. */
+int   tw_hip_init_device(int device);
+/* cuda.go:58-75: device name / total memory. */
+int   tw_hip_device_info(char* name, size_t nameLen, uint64_t* totalMem);
+
+/* ------------------------------------------------------------------ */
+/* 2. Per-op kernels                           kernels.go:12-72         */
+/*    Same symbol names and argument order as libmongoose_kernels.so.   */
+/* ------------------------------------------------------------------ */
+
+/* kernels.go:13, mongoose.cu:145-179.  out = in * rsqrt(mean(in^2)+1e-6) * w, per row of [seqLen, dim]. */
+void mongoose_rmsnorm_out(const float* in, float* out, const float* w, int seqLen, int dim, void* stream);
+/* Same with eps as an argument (cpu.go:36 and the Metal path take it as a
+ * parameter; the CUDA kernel hard-codes 1e-6). */
+void mongoose_rmsnorm_out_eps(const float* in, float* out, const float* w, int seqLen, int dim, float eps, void* stream);
+
+/* kernels.go:62, mongoose.cu:1556-1595.  out[r] = sum_k act[k]*w[r,k] * (scales[r]/127):
+ * the reference kernel's convention, `scales` holding per-row absmax
+ * (producer: mongoose_requant_fp32_to_int8, mongoose.cu:1501-1545). */
+void mongoose_q8_matvec(const float* act, const void* w_int8, const float* scales, float* out, int N, int K, void* stream);
+/* Per-row-scale form: out[r] = sum_k act[k]*w[r,k] * scales[r], with
+ * scales[r] = absmax/127 as quantizeQ8 stores them (cuda_fused_infer.go:373-374,
+ * metal_impl_darwin.m:5533-5535).  This is what the mg_* context uses. */
+void mongoose_q8_matvec_rowscale(const float* act, const void* w_int8, const float* scales, float* out, int N, int K, void* stream);
+
+/* kernels.go:65.  w is raw GGUF block_q4_0 (18-byte blocks: fp16 d, 16 bytes of
+ * nibbles; low nibble = element j, high nibble = element j+16; value (nib-8)*d),
+ * rows of K/32 blocks (cuda_q4_0.go:13-17).  fp32 activations, fp32 accumulate. */
+void mongoose_q4_0_matvec(const float* act, const void* w_q4_0, float* out, int N, int K, void* stream);
+/* Device-side repack of raw GGUF rows into the split layout the fast kernel
+ * reads: N*K/2 bytes of nibbles (16 per block, rows contiguous) followed by
+ * N*K/32 fp16 scales.  `planar` needs N*K/2 + N*K/16 bytes. */
+void mongoose_q4_0_repack(const void* w_q4_0, void* planar, int N, int K, void* stream);
+void mongoose_q4_0_matvec_planar(const float* act, const void* planar, float* out, int N, int K, void* stream);
+
+/* kernels.go:31, mongoose.cu:991-1013.  In place on x[seqLen, dim]; rotate-half
+ * pairs (j, j+headDim/2); row `pos` of x uses table row `pos`. */
+void mongoose_rope(float* x, const float* cosTab, const float* sinTab, int seqLen, int dim, int headDim, int nHeads, void* stream);
+/* kernels.go:64, mongoose.cu:1644-1653.  cache[pos*kvDim + i] = src[i]. */
+void mongoose_kv_cache_write(float* cache, const float* src, int pos, int kvDim, void* stream);
+/* kernels.go:38, mongoose.cu:856-945.  Single query against [cacheLen, kvDim] caches, GQA. */
+void mongoose_decode_attention(const float* Q, const float* K, const float* V, float* out,
+                               int cacheLen, int dim, int kvDim, int nHeads, int nKVHeads, void* stream);
+/* kernels.go:29, mongoose.cu:949-960.  out = gate * sigmoid(gate) * up. */
+void mongoose_silu_gate_mul(const float* gate, const float* up, float* out, int n, void* stream);
+/* kernels.go:17, mongoose.cu:212-219.  a += b. */
+void mongoose_add_inplace(float* a, const float* b, int n, void* stream);
+/* kernels.go:34, mongoose.cu:1052-1064.  out[p,:] = embed[tokens[p],:] (fp32 table). */
+void mongoose_embed_gather(float* out, const float* embed, const int* tokens, int seqLen, int dim, void* stream);
+/* kernels.go:41, mongoose.cu:1475-1499 (absmax convention: q * scales[r]/127). */
+void mongoose_dequant_int8_to_fp32(const void* w_int8, const float* scales, float* out, int rows, int cols, void* stream);
+/* q * scales[r] (per-row-scale convention) and GGUF Q4_0 blocks -> fp32. */
+void mongoose_dequant_q8_rowscale(const void* w_int8, const float* scales, float* out, int rows, int cols, void* stream);
+void mongoose_dequant_q4_0(const void* w_q4_0, float* out, int rows, int cols, void* stream);
+/* kernels.go:24-26, mongoose.cu:356-368. */
+void mongoose_copy(void* dst, const void* src, size_t bytes, void* stream);
+void mongoose_zero(void* ptr, size_t bytes, void* stream);
+void mongoose_sync(void* stream);
+/* kernels.go:326-330 (CUDACheck -> cudaPeekAtLastError): 0 when no launch has
+ * failed since the last call, else the HIP error code; clears the record. */
+int  mongoose_check(void);
+
+/* ------------------------------------------------------------------ */
+/* 3. Fused-inference context                                           */
+/* ------------------------------------------------------------------ */
+typedef struct mg_ctx mg_ctx;
+
+/* NewCUDAFusedInference, cuda_fused_infer.go:144-229.  eps is the RMSNorm
+ * epsilon (a parameter here; cpu.go:36).  NULL on failure. */
+mg_ctx* mg_create(int dim, int kvDim, int headDim, int nHeads, int nKVHeads, int ffnDim,
+                  int vocabSize, int nLayers, int maxSeq, double ropeTheta, float eps);
+void    mg_destroy(mg_ctx* ctx);
+const char* mg_last_error(void);
+
+/* NumWeights, cuda_fused_infer.go:231-233: nLayers*12 + 2.  Slot map (:241-272):
+ * l*12 + {0 norm1, 1 wq, 2 wk, 3 wv, 4 bq, 5 bk, 6 bv, 7 wo, 8 norm2, 9 gate,
+ * 10 up, 11 down}; nLayers*12 final norm; nLayers*12+1 lm_head. */
+int mg_num_weights(const mg_ctx* ctx);
+
+/* SetWeight, cuda_fused_infer.go:241-272 + quantizeQ8 :363-390: fp32 in; matrix
+ * slots are quantized to per-row int8 on the host and uploaded, norm gains
+ * are uploaded as fp32.  Unlike the resident CUDA path (:255 skips them) bias
+ * slots 4/5/6 are kept and added before RoPE, as cuda_fused_stream.go:319-321. */
+int mg_set_weight(mg_ctx* ctx, int idx, const float* data, size_t n);
+/* Already-quantized rows (same layout quantizeQ8 produces). */
+int mg_set_weight_q8(mg_ctx* ctx, int idx, const int8_t* q, const float* scales);
+/* SetWeightQ4_0, cuda_fused_infer_q4.go:46-90 + UploadQ4_0 cuda_q4_0.go:15-26:
+ * raw GGUF block_q4_0 bytes, rows*(cols/32)*18. */
+int mg_set_weight_q4_0(mg_ctx* ctx, int idx, const uint8_t* q4Data, size_t nbytes);
+/* Q8 rounding used by mg_set_weight: 0 = truncate toward zero
+ * (cuda_fused_infer.go:378), 1 = round half away from zero
+ * (metal_impl_darwin.m:5776-5778).  Default 0. */
+int mg_set_quant_rounding(mg_ctx* ctx, int mode);
+
+/* Embedding table for mg_decode_token / mg_generate (the reference leaves the
+ * lookup to its caller).  Without one, the lm_head row is used (tied weights). */
+int mg_set_embedding_f16(mg_ctx* ctx, const uint16_t* table /* [vocab, dim] */);
+int mg_set_embedding_f32(mg_ctx* ctx, const float* table /* [vocab, dim] */);
+
+/* SetLayerRange :542-554 (allocates the fp32 KV caches of the owned layers),
+ * ResetKV :530-537. */
+int mg_set_layer_range(mg_ctx* ctx, int layerStart, int layerEnd);
+int mg_reset_kv(mg_ctx* ctx);
+
+/* PartialStep :392-452 / PartialStepQ4 cuda_fused_infer_q4.go:92.  hiddenIn
+ * [dim] host floats, or NULL for the ...Continue forms (:456, q4:272) that keep
+ * the device-resident hidden state.  logitsOut [vocab] is written when
+ * layerEnd >= nLayers and it is not NULL; hiddenOut [dim] when
+ * layerEnd < nLayers and it is not NULL. */
+int mg_partial_step(mg_ctx* ctx, const float* hiddenIn, int pos, int layerStart, int layerEnd,
+                    float* hiddenOut, float* logitsOut);
+/* StepLayerResident, cuda_fused_infer_q4.go:451-605: one layer, with host
+ * snapshots of the hidden state before (preOut) and after (postOut) it;
+ * hiddenIn is uploaded when layer == 0; logitsOut as above. */
+int mg_step_layer_resident(mg_ctx* ctx, int layer, int pos, const float* hiddenIn,
+                           float* preOut, float* postOut, float* logitsOut);
+/* ExportHidden :235-239. */
+int mg_export_hidden(mg_ctx* ctx, float* out /* [dim] */);
+
+/* Execution mode of the layer loop: 0 = one launch per reference op, in the
+ * reference's order (cuda_fused_infer.go:417-443, 17 launches a layer);
+ * 1 = fused launches (default).  Both give the same results to rounding. */
+int mg_set_exec_mode(mg_ctx* ctx, int mode);
+
+/* Whole token on the device: embedding gather -> layers -> final norm ->
+ * lm_head -> greedy argmax (lowest index on ties).  logitsOut may be NULL. */
+int mg_decode_token(mg_ctx* ctx, int token, int pos, int* nextToken, float* logitsOut);
+/* Greedy generation: prompt tokens occupy positions 0..nPrompt-1, then
+ * nDecode tokens are produced; outTokens [nDecode].  useGraph != 0 replays a
+ * captured hipGraph per token (CaptureGraph / Launch, cuda_graph.go:315-669);
+ * the position and the token stay in device memory between steps. */
+int mg_generate(mg_ctx* ctx, const int* prompt, int nPrompt, int nDecode, int* outTokens, int useGraph);
+
+/* CUDAGraph, cuda_graph.go:286-739.  Capture once; every launch advances the
+ * device-resident position by one.  mg_graph_validate replays one step both
+ * ways and returns the largest absolute logit difference (the reference's
+ * criterion is < 1e-3, cuda_graph.go:590-597). */
+int mg_graph_capture(mg_ctx* ctx);
+int mg_graph_launch(mg_ctx* ctx, int token, int pos, int* nextToken);
+int mg_graph_validate(mg_ctx* ctx, int token, int pos, float* maxAbsDiff);
+
+/* Timed decode for measurement: runs `steps` graph (or eager) decode steps
+ * starting at device state (token, pos), bracketed by events on the context's
+ * stream; returns elapsed milliseconds.  Inputs are resident before the timed
+ * region starts. */
+int mg_timed_decode(mg_ctx* ctx, int token, int pos, int steps, int useGraph, float* elapsedMs);
+
+/* Bytes of weights, scales and norm gains one token reads (the figure the
+ * bandwidth roofline is computed from), and the KV bytes read at position pos. */
+uint64_t mg_weight_bytes_per_token(const mg_ctx* ctx);
+uint64_t mg_kv_bytes_at(const mg_ctx* ctx, int pos);
+
+/* ------------------------------------------------------------------ */
+/* Streaming inference (weights larger than device memory)              */
+/* CUDAStreamInfer, cuda_fused_stream.go:98-726                         */
+/* ------------------------------------------------------------------ */
+typedef struct mg_stream mg_stream;
+/* StreamBuild :127-198: two device weight sets + two pinned staging buffers. */
+mg_stream* mg_stream_build(mg_ctx* ctx);
+void       mg_stream_destroy(mg_stream* s);
+/* StreamForwardToken :559-670.  layerPtrs[i*12+k] are host pointers to the
+ * tensors of layer i in slot order (norm1, wq, wk, wv, bq, bk, bv, wo, norm2,
+ * gate, up, down; bias pointers may be NULL), layerSizes[i*7+m] the byte sizes
+ * of its seven Q4_0 matrices (wq, wk, wv, wo, gate, up, down).  The final norm
+ * and lm_head come from the context (slots nLayers*12, +1). */
+int mg_stream_forward_token(mg_stream* s, int pos, const float* embHidden, int nLayers,
+                            const void* const* layerPtrs, const int32_t* layerSizes,
+                            float* logitsOut);
+
+/* ------------------------------------------------------------------ */
+/* Host-side helpers shared with the loaders                            */
+/* ------------------------------------------------------------------ */
+/* quantizeQ8 (cuda_fused_infer.go:363-390) on the host; mode as mg_set_quant_rounding. */
+void mg_quantize_q8(const float* w, int rows, int cols, int mode, int8_t* q, float* scales);
+/* GGML quantize_row_q4_0 over rows*(cols/32) blocks -> 18-byte blocks. */
+void mg_quantize_q4_0(const float* w, int rows, int cols, uint8_t* blocks);
+uint16_t mg_f32_to_f16(float f);
+float    mg_f16_to_f32(uint16_t h);
+/* Deterministic synthetic weights: n samples of N(0, std) for stream (seed, idx),
+ * identical on every machine (integer generator + fixed-order arithmetic). */
+void mg_synth_normal(uint64_t seed, uint64_t idx, float std, float* out, size_t n);
+/* n uniform ints in [0, bound). */
+void mg_synth_tokens(uint64_t seed, uint64_t idx, int bound, int* out, size_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MONGOOSE_HIP_H */

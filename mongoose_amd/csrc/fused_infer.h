@@ -1,0 +1,122 @@
+// fused_infer.h -- HIPFusedInference: the MI355X counterpart of the Go type
+// CUDAFusedInference (cuda_fused_infer.go:56-142).  It owns the quantized
+// weights, the fp32 KV caches, the scratch vectors and the RoPE tables, and
+// runs the batch-1 decode step.  Method names follow the Go methods they
+// stand in for; the mg_* C functions are thin wrappers over them.
+#pragma once
+#include "kernels.h"
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+namespace mg {
+
+struct DevMat {
+    int kind = -1;          // -1 none, WF_Q8, WF_Q4P
+    void* w = nullptr;      // Q8: int8 [rows, cols]; Q4P: nibble plane + fp16 d plane
+    float* scales = nullptr;
+    int rows = 0, cols = 0;
+    size_t bytes = 0;       // bytes a token reads from this matrix (weights + scales)
+};
+
+struct LayerWeights {
+    float* norm1 = nullptr;
+    float* norm2 = nullptr;
+    float* bq = nullptr;
+    float* bk = nullptr;
+    float* bv = nullptr;
+    DevMat wq, wk, wv, wo, gate, up, down;
+};
+
+void set_error(const std::string& s);
+const std::string& get_error();
+
+class HIPFusedInference {
+public:
+    // NewCUDAFusedInference, cuda_fused_infer.go:144-229
+    static HIPFusedInference* New(int dim, int kvDim, int headDim, int nHeads, int nKVHeads, int ffnDim,
+                                  int vocabSize, int nLayers, int maxSeq, double ropeTheta, float eps);
+    ~HIPFusedInference();
+
+    int NumWeights() const { return nLayers * 12 + 2; }                           // :231
+    int SetWeight(int idx, const float* data, size_t n);                          // :241
+    int SetWeightQ8(int idx, const int8_t* q, const float* scales);
+    int SetWeightQ4_0(int idx, const uint8_t* q4Data, size_t nbytes);             // cuda_fused_infer_q4.go:46
+    int SetEmbeddingF16(const uint16_t* table);
+    int SetEmbeddingF32(const float* table);
+    int SetLayerRange(int layerStart, int layerEnd);                              // :542
+    int ResetKV();                                                                // :530
+    int PartialStep(const float* hiddenIn, int pos, int layerStart, int layerEnd,
+                    float* hiddenOut, float* logitsOut);                          // :392, :456, q4:92, q4:272
+    int StepLayerResident(int layer, int pos, const float* hiddenIn, float* preOut,
+                          float* postOut, float* logitsOut);                      // cuda_fused_infer_q4.go:451
+    int ExportHidden(float* out);                                                 // :235
+    int DecodeToken(int token, int pos, int* nextToken, float* logitsOut);
+    int Generate(const int* prompt, int nPrompt, int nDecode, int* outTokens, bool useGraph);
+    int GraphCapture();                                                           // cuda_graph.go:315
+    int GraphLaunch(int token, int pos, int* nextToken);                          // cuda_graph.go:663
+    int GraphValidate(int token, int pos, float* maxAbsDiff);                     // cuda_graph.go:554
+    int TimedDecode(int token, int pos, int steps, bool useGraph, float* elapsedMs);
+    uint64_t WeightBytesPerToken() const;
+    uint64_t KVBytesAt(int pos) const { return (uint64_t)2 * nLayers * (uint64_t)(pos + 1) * kvDim * 4; }
+
+    int quantRounding = 0;
+    int execMode = 1;
+
+    // shape
+    int dim, kvDim, headDim, nHeads, nKVHeads, ffnDim, vocabSize, nLayers, maxSeq;
+    double ropeTheta;
+    float eps;
+
+    // used by the streaming front end
+    hipStream_t stream = nullptr;
+    std::vector<LayerWeights> layers;
+    std::vector<float*> kCache, vCache;
+    float* hidden[2] = {nullptr, nullptr};
+    int hiddenIdx = 0;
+    int enqueueLayer(const LayerWeights& L, int layer, const StepState* st, int posImm);
+    int enqueueFinal(bool withArgmax);
+    float* logits = nullptr;
+    float* finalNorm = nullptr;
+    DevMat lmHead;
+
+private:
+    HIPFusedInference() = default;
+    bool built = false;
+    int invalidateGraphs();
+    int uploadMat(DevMat& m, int rows, int cols, const int8_t* q, const float* scales);
+    int uploadMatQ4(DevMat& m, int rows, int cols, const uint8_t* raw, size_t nbytes);
+    int setVec(float*& dst, const float* data, size_t n, size_t expect);
+    DevMat* matSlot(int idx, int* rows, int* cols);
+    int enqueueLayerFused(const LayerWeights& L, int layer, const StepState* st, int posImm);
+    int enqueueLayerPerOp(const LayerWeights& L, int layer, int pos);
+    int enqueueEmbed();
+    int enqueueToken(bool withHead);      // embed -> layers -> final(+argmax) / advance, all from device state
+    int freeMat(DevMat& m);
+
+    // scratch (cuda_fused_infer.go:56-69, :626)
+    float *normed = nullptr, *Q = nullptr, *K = nullptr, *V = nullptr, *attnOut = nullptr, *proj = nullptr;
+    float *normed2 = nullptr, *gatePre = nullptr, *upOut = nullptr, *ffnMid = nullptr;
+    float *cosTab = nullptr, *sinTab = nullptr;
+    // split-KV attention partials
+    float *pm = nullptr, *pl = nullptr, *pacc = nullptr;
+    int smax = 1, minSplit = 256;
+    // embedding table (optional)
+    int embedKind = -1;       // -1: tied lm_head
+    void* embedTable = nullptr;
+    // token-level state
+    StepState* dState = nullptr;
+    StepState* hState = nullptr;    // pinned mirror
+    float* amaxVal = nullptr;
+    int* amaxIdx = nullptr;
+    int amaxParts = 0;
+    int* dHistory = nullptr;
+    int* dPrompt = nullptr;
+    int* hTokens = nullptr;         // pinned
+    hipGraph_t graphFull = nullptr, graphPrompt = nullptr;
+    hipGraphExec_t execFull = nullptr, execPrompt = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+};
+
+}  // namespace mg

@@ -1,0 +1,767 @@
+// fused_infer.hip -- HIPFusedInference and the mg_* C entry points over it.
+// Host code only (no kernels here); compiled with hipcc for the runtime API.
+#include "fused_infer.h"
+#include "../../include/mongoose_hip.h"
+#include "host_util.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+namespace mg {
+
+static thread_local std::string g_err;
+void set_error(const std::string& s) { g_err = s; }
+const std::string& get_error() { return g_err; }
+
+#define HIPCHK(expr)                                                                      \
+    do {                                                                                  \
+        hipError_t e_ = (expr);                                                           \
+        if (e_ != hipSuccess) {                                                           \
+            set_error(std::string(#expr) + ": " + hipGetErrorString(e_));                 \
+            (void)hipGetLastError();                                                      \
+            return MG_E_HIP;                                                              \
+        }                                                                                 \
+    } while (0)
+
+#define ARGCHK(cond, msg)                                                                 \
+    do {                                                                                  \
+        if (!(cond)) { set_error(msg); return MG_E_ARG; }                                 \
+    } while (0)
+
+template <typename T>
+static int devAlloc(T*& p, size_t count, bool zero) {
+    void* v = nullptr;
+    HIPCHK(hipMalloc(&v, count * sizeof(T) ? count * sizeof(T) : 1));
+    if (zero) HIPCHK(hipMemset(v, 0, count * sizeof(T)));
+    p = static_cast<T*>(v);
+    return MG_OK;
+}
+
+HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int nHeads, int nKVHeads, int ffnDim,
+                                          int vocabSize, int nLayers, int maxSeq, double ropeTheta, float eps) {
+    if (dim <= 0 || kvDim <= 0 || nHeads <= 0 || nKVHeads <= 0 || ffnDim <= 0 || vocabSize <= 0 || nLayers <= 0 ||
+        maxSeq <= 0) { set_error("mg_create: non-positive dimension"); return nullptr; }
+    if (headDim != 64 && headDim != 128) { set_error("mg_create: headDim must be 64 or 128"); return nullptr; }
+    if (nHeads * headDim != dim || nKVHeads * headDim != kvDim || nHeads % nKVHeads != 0) {
+        set_error("mg_create: dim/kvDim must equal heads*headDim and nHeads must be a multiple of nKVHeads");
+        return nullptr;
+    }
+    if (dim % 32 != 0 || ffnDim % 32 != 0 || dim > 16384 || ffnDim > 16384) {
+        set_error("mg_create: dim and ffnDim must be multiples of 32 and at most 16384");
+        return nullptr;
+    }
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
+        (void)hipGetLastError();
+        set_error("mg_create: no HIP device");
+        return nullptr;
+    }
+    auto* f = new HIPFusedInference();
+    f->dim = dim; f->kvDim = kvDim; f->headDim = headDim; f->nHeads = nHeads; f->nKVHeads = nKVHeads;
+    f->ffnDim = ffnDim; f->vocabSize = vocabSize; f->nLayers = nLayers; f->maxSeq = maxSeq;
+    f->ropeTheta = ropeTheta; f->eps = eps;
+    f->layers.resize(nLayers);
+    f->kCache.assign(nLayers, nullptr);
+    f->vCache.assign(nLayers, nullptr);
+
+    auto fail = [&](const char* what) -> HIPFusedInference* {
+        if (get_error().empty()) set_error(what);
+        delete f;
+        return nullptr;
+    };
+    if (hipStreamCreateWithFlags(&f->stream, hipStreamNonBlocking) != hipSuccess) return fail("stream create failed");
+    if (hipEventCreate(&f->ev0) != hipSuccess || hipEventCreate(&f->ev1) != hipSuccess) return fail("event create failed");
+
+    bool ok = devAlloc(f->hidden[0], dim, true) == 0 && devAlloc(f->hidden[1], dim, true) == 0 &&
+              devAlloc(f->logits, vocabSize, true) == 0 && devAlloc(f->normed, dim, true) == 0 &&
+              devAlloc(f->Q, dim, true) == 0 && devAlloc(f->K, kvDim, true) == 0 && devAlloc(f->V, kvDim, true) == 0 &&
+              devAlloc(f->attnOut, dim, true) == 0 && devAlloc(f->proj, dim, true) == 0 &&
+              devAlloc(f->normed2, dim, true) == 0 && devAlloc(f->gatePre, ffnDim, true) == 0 &&
+              devAlloc(f->upOut, ffnDim, true) == 0 && devAlloc(f->ffnMid, ffnDim, true) == 0;
+    if (!ok) return fail("scratch alloc failed");
+
+    // RoPE tables, cuda_fused_infer.go:181-192: angle in double, stored as float.
+    const int half = headDim / 2;
+    std::vector<float> cosD((size_t)maxSeq * half), sinD((size_t)maxSeq * half);
+    std::vector<double> freq(half);
+    for (int j = 0; j < half; j++) freq[j] = 1.0 / std::pow(ropeTheta, (double)(2 * j) / (double)headDim);
+    for (int pos = 0; pos < maxSeq; pos++) {
+        for (int j = 0; j < half; j++) {
+            double angle = (double)pos * freq[j];
+            cosD[(size_t)pos * half + j] = (float)std::cos(angle);
+            sinD[(size_t)pos * half + j] = (float)std::sin(angle);
+        }
+    }
+    if (devAlloc(f->cosTab, cosD.size(), false) != 0 || devAlloc(f->sinTab, sinD.size(), false) != 0) return fail("rope alloc");
+    if (hipMemcpy(f->cosTab, cosD.data(), cosD.size() * 4, hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(f->sinTab, sinD.data(), sinD.size() * 4, hipMemcpyHostToDevice) != hipSuccess) return fail("rope upload");
+
+    // split-KV partials: one tile of 256 positions per split at full context, at most 64 splits
+    f->minSplit = 256;
+    f->smax = (maxSeq + 255) / 256;
+    if (f->smax > 64) f->smax = 64;
+    if (f->smax < 1) f->smax = 1;
+    if (devAlloc(f->pm, (size_t)nHeads * f->smax, true) != 0 || devAlloc(f->pl, (size_t)nHeads * f->smax, true) != 0 ||
+        devAlloc(f->pacc, (size_t)nHeads * f->smax * headDim, true) != 0) return fail("attention partial alloc");
+
+    f->amaxParts = 2048;
+    if (devAlloc(f->amaxVal, f->amaxParts, true) != 0 || devAlloc(f->amaxIdx, f->amaxParts, true) != 0 ||
+        devAlloc(f->dState, 1, true) != 0 || devAlloc(f->dHistory, (size_t)maxSeq + 1, true) != 0 ||
+        devAlloc(f->dPrompt, (size_t)maxSeq + 1, true) != 0) return fail("state alloc");
+    void* hp = nullptr;
+    if (hipHostMalloc(&hp, sizeof(StepState), hipHostMallocDefault) != hipSuccess) return fail("pinned alloc");
+    f->hState = static_cast<StepState*>(hp);
+    if (hipHostMalloc(&hp, sizeof(int) * ((size_t)maxSeq + 1), hipHostMallocDefault) != hipSuccess) return fail("pinned alloc");
+    f->hTokens = static_cast<int*>(hp);
+
+    f->built = true;
+    return f;
+}
+
+int HIPFusedInference::freeMat(DevMat& m) {
+    if (m.w) (void)hipFree(m.w);
+    if (m.scales) (void)hipFree(m.scales);
+    m = DevMat();
+    return MG_OK;
+}
+
+HIPFusedInference::~HIPFusedInference() {
+    if (stream) (void)hipStreamSynchronize(stream);
+    invalidateGraphs();
+    for (auto& L : layers) {
+        for (float* p : {L.norm1, L.norm2, L.bq, L.bk, L.bv}) if (p) (void)hipFree(p);
+        for (DevMat* m : {&L.wq, &L.wk, &L.wv, &L.wo, &L.gate, &L.up, &L.down}) freeMat(*m);
+    }
+    freeMat(lmHead);
+    for (float* p : kCache) if (p) (void)hipFree(p);
+    for (float* p : vCache) if (p) (void)hipFree(p);
+    for (float* p : {hidden[0], hidden[1], logits, finalNorm, normed, Q, K, V, attnOut, proj, normed2, gatePre, upOut,
+                     ffnMid, cosTab, sinTab, pm, pl, pacc, amaxVal}) if (p) (void)hipFree(p);
+    if (amaxIdx) (void)hipFree(amaxIdx);
+    if (dState) (void)hipFree(dState);
+    if (dHistory) (void)hipFree(dHistory);
+    if (dPrompt) (void)hipFree(dPrompt);
+    if (embedTable) (void)hipFree(embedTable);
+    if (hState) (void)hipHostFree(hState);
+    if (hTokens) (void)hipHostFree(hTokens);
+    if (ev0) (void)hipEventDestroy(ev0);
+    if (ev1) (void)hipEventDestroy(ev1);
+    if (stream) (void)hipStreamDestroy(stream);
+}
+
+int HIPFusedInference::invalidateGraphs() {
+    if (execFull) { (void)hipGraphExecDestroy(execFull); execFull = nullptr; }
+    if (execPrompt) { (void)hipGraphExecDestroy(execPrompt); execPrompt = nullptr; }
+    if (graphFull) { (void)hipGraphDestroy(graphFull); graphFull = nullptr; }
+    if (graphPrompt) { (void)hipGraphDestroy(graphPrompt); graphPrompt = nullptr; }
+    return MG_OK;
+}
+
+// Slot map, cuda_fused_infer.go:241-272.
+DevMat* HIPFusedInference::matSlot(int idx, int* rows, int* cols) {
+    if (idx < 0) return nullptr;
+    if (idx < nLayers * 12) {
+        LayerWeights& L = layers[idx / 12];
+        switch (idx % 12) {
+        case 1: *rows = dim; *cols = dim; return &L.wq;
+        case 2: *rows = kvDim; *cols = dim; return &L.wk;
+        case 3: *rows = kvDim; *cols = dim; return &L.wv;
+        case 7: *rows = dim; *cols = dim; return &L.wo;
+        case 9: *rows = ffnDim; *cols = dim; return &L.gate;
+        case 10: *rows = ffnDim; *cols = dim; return &L.up;
+        case 11: *rows = dim; *cols = ffnDim; return &L.down;
+        default: return nullptr;
+        }
+    }
+    if (idx == nLayers * 12 + 1) { *rows = vocabSize; *cols = dim; return &lmHead; }
+    return nullptr;
+}
+
+int HIPFusedInference::setVec(float*& dst, const float* data, size_t n, size_t expect) {
+    ARGCHK(n == expect, "SetWeight: wrong element count for a norm/bias slot");
+    if (!dst) { int rc = devAlloc(dst, expect, false); if (rc) return rc; }
+    HIPCHK(hipStreamSynchronize(stream));
+    HIPCHK(hipMemcpy(dst, data, expect * sizeof(float), hipMemcpyHostToDevice));
+    return MG_OK;
+}
+
+int HIPFusedInference::uploadMat(DevMat& m, int rows, int cols, const int8_t* q, const float* scales) {
+    HIPCHK(hipStreamSynchronize(stream));
+    invalidateGraphs();
+    freeMat(m);
+    void* w = nullptr;
+    HIPCHK(hipMalloc(&w, (size_t)rows * cols));
+    m.w = w;
+    HIPCHK(hipMemcpy(m.w, q, (size_t)rows * cols, hipMemcpyHostToDevice));
+    int rc = devAlloc(m.scales, rows, false);
+    if (rc) return rc;
+    HIPCHK(hipMemcpy(m.scales, scales, (size_t)rows * 4, hipMemcpyHostToDevice));
+    m.kind = WF_Q8; m.rows = rows; m.cols = cols;
+    m.bytes = (size_t)rows * cols + (size_t)rows * 4;
+    return MG_OK;
+}
+
+int HIPFusedInference::uploadMatQ4(DevMat& m, int rows, int cols, const uint8_t* raw, size_t nbytes) {
+    ARGCHK(cols % 32 == 0, "SetWeightQ4_0: cols must be a multiple of 32");
+    size_t expect = (size_t)rows * (cols / 32) * 18;          // cuda_q4_0.go:16-19
+    ARGCHK(nbytes == expect, "SetWeightQ4_0: byte count is not rows*(cols/32)*18");
+    HIPCHK(hipStreamSynchronize(stream));
+    invalidateGraphs();
+    freeMat(m);
+    std::vector<uint8_t> planar(expect);
+    repack_q4_0_host(raw, rows, cols, planar.data());
+    void* w = nullptr;
+    HIPCHK(hipMalloc(&w, expect));
+    m.w = w;
+    HIPCHK(hipMemcpy(m.w, planar.data(), expect, hipMemcpyHostToDevice));
+    m.kind = WF_Q4P; m.rows = rows; m.cols = cols; m.bytes = expect;
+    return MG_OK;
+}
+
+int HIPFusedInference::SetWeight(int idx, const float* data, size_t n) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(data != nullptr && idx >= 0 && idx < NumWeights(), "SetWeight: bad slot or NULL data");
+    int rows = 0, cols = 0;
+    DevMat* m = matSlot(idx, &rows, &cols);
+    if (m) {
+        ARGCHK(n == (size_t)rows * cols, "SetWeight: wrong element count for a matrix slot");
+        std::vector<int8_t> q((size_t)rows * cols);
+        std::vector<float> sc(rows);
+        mg_quantize_q8(data, rows, cols, quantRounding, q.data(), sc.data());
+        return uploadMat(*m, rows, cols, q.data(), sc.data());
+    }
+    if (idx == nLayers * 12) return setVec(finalNorm, data, n, dim);
+    LayerWeights& L = layers[idx / 12];
+    switch (idx % 12) {
+    case 0: return setVec(L.norm1, data, n, dim);
+    case 8: return setVec(L.norm2, data, n, dim);
+    case 4: invalidateGraphs(); return setVec(L.bq, data, n, dim);
+    case 5: invalidateGraphs(); return setVec(L.bk, data, n, kvDim);
+    case 6: invalidateGraphs(); return setVec(L.bv, data, n, kvDim);
+    }
+    set_error("SetWeight: unreachable slot");
+    return MG_E_ARG;
+}
+
+int HIPFusedInference::SetWeightQ8(int idx, const int8_t* q, const float* scales) {
+    if (!built) return MG_E_NOT_BUILT;
+    int rows = 0, cols = 0;
+    DevMat* m = matSlot(idx, &rows, &cols);
+    ARGCHK(m && q && scales, "SetWeightQ8: not a matrix slot or NULL data");
+    return uploadMat(*m, rows, cols, q, scales);
+}
+
+int HIPFusedInference::SetWeightQ4_0(int idx, const uint8_t* q4Data, size_t nbytes) {
+    if (!built) return MG_E_NOT_BUILT;
+    int rows = 0, cols = 0;
+    DevMat* m = matSlot(idx, &rows, &cols);
+    // cuda_fused_infer_q4.go:52,66,78: norm, bias and final-norm slots are not Q4 and are ignored
+    if (!m) return (idx >= 0 && idx < NumWeights()) ? MG_OK : MG_E_ARG;
+    ARGCHK(q4Data != nullptr, "SetWeightQ4_0: NULL data");
+    return uploadMatQ4(*m, rows, cols, q4Data, nbytes);
+}
+
+int HIPFusedInference::SetEmbeddingF16(const uint16_t* table) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(table, "SetEmbeddingF16: NULL table");
+    HIPCHK(hipStreamSynchronize(stream));
+    invalidateGraphs();
+    if (embedTable) { (void)hipFree(embedTable); embedTable = nullptr; }
+    size_t bytes = (size_t)vocabSize * dim * 2;
+    HIPCHK(hipMalloc(&embedTable, bytes));
+    HIPCHK(hipMemcpy(embedTable, table, bytes, hipMemcpyHostToDevice));
+    embedKind = 1;
+    return MG_OK;
+}
+
+int HIPFusedInference::SetEmbeddingF32(const float* table) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(table, "SetEmbeddingF32: NULL table");
+    HIPCHK(hipStreamSynchronize(stream));
+    invalidateGraphs();
+    if (embedTable) { (void)hipFree(embedTable); embedTable = nullptr; }
+    size_t bytes = (size_t)vocabSize * dim * 4;
+    HIPCHK(hipMalloc(&embedTable, bytes));
+    HIPCHK(hipMemcpy(embedTable, table, bytes, hipMemcpyHostToDevice));
+    embedKind = 2;
+    return MG_OK;
+}
+
+int HIPFusedInference::SetLayerRange(int layerStart, int layerEnd) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(layerStart >= 0 && layerStart <= layerEnd, "SetLayerRange: bad range");
+    for (int l = layerStart; l < layerEnd && l < nLayers; l++) {
+        if (!kCache[l]) {
+            invalidateGraphs();
+            int rc = devAlloc(kCache[l], (size_t)maxSeq * kvDim, true);
+            if (rc) return rc;
+            rc = devAlloc(vCache[l], (size_t)maxSeq * kvDim, true);
+            if (rc) return rc;
+        }
+    }
+    return MG_OK;
+}
+
+// cuda_fused_infer.go:530-537 uploads zeros over K only; V is cleared as well
+// here (a fresh sequence never reads V rows it has not written).
+int HIPFusedInference::ResetKV() {
+    if (!built) return MG_E_NOT_BUILT;
+    HIPCHK(hipStreamSynchronize(stream));
+    for (int l = 0; l < nLayers; l++) {
+        if (kCache[l]) HIPCHK(hipMemset(kCache[l], 0, (size_t)maxSeq * kvDim * 4));
+        if (vCache[l]) HIPCHK(hipMemset(vCache[l], 0, (size_t)maxSeq * kvDim * 4));
+    }
+    return MG_OK;
+}
+
+uint64_t HIPFusedInference::WeightBytesPerToken() const {
+    uint64_t b = 0;
+    for (const auto& L : layers) {
+        b += L.wq.bytes + L.wk.bytes + L.wv.bytes + L.wo.bytes + L.gate.bytes + L.up.bytes + L.down.bytes;
+        if (L.norm1) b += (uint64_t)dim * 4;
+        if (L.norm2) b += (uint64_t)dim * 4;
+    }
+    b += lmHead.bytes;
+    if (finalNorm) b += (uint64_t)dim * 4;
+    return b;
+}
+
+static bool layerComplete(const LayerWeights& L) {
+    return L.norm1 && L.norm2 && L.wq.w && L.wk.w && L.wv.w && L.wo.w && L.gate.w && L.up.w && L.down.w;
+}
+
+// One launch per reference op, in the reference's order
+// (cuda_fused_infer.go:417-443; bias adds cuda_fused_stream.go:319-321).
+int HIPFusedInference::enqueueLayerPerOp(const LayerWeights& L, int layer, int pos) {
+    float* h = hidden[hiddenIdx];
+    const int half = headDim / 2;
+    auto mv = [&](const DevMat& m, const float* act, float* out) -> hipError_t {
+        MvParams p{};
+        p.seg[0] = MvSeg{m.w, m.scales, nullptr, out, m.rows};
+        p.nseg = 1; p.K = m.cols; p.act = act;
+        return launch_matvec(m.kind, EPI_STORE, PRO_PLAIN, p, nullptr, stream);
+    };
+    HIPCHK(launch_rmsnorm_out(h, normed, L.norm1, 1, dim, eps, stream));
+    HIPCHK(mv(L.wq, normed, Q));
+    HIPCHK(mv(L.wk, normed, K));
+    HIPCHK(mv(L.wv, normed, V));
+    if (L.bq) HIPCHK(launch_add_inplace(Q, L.bq, dim, stream));
+    if (L.bk) HIPCHK(launch_add_inplace(K, L.bk, kvDim, stream));
+    if (L.bv) HIPCHK(launch_add_inplace(V, L.bv, kvDim, stream));
+    const float* cosRow = cosTab + (size_t)pos * half;      // cuda_fused_infer.go:423-424
+    const float* sinRow = sinTab + (size_t)pos * half;
+    HIPCHK(launch_rope(Q, cosRow, sinRow, 1, dim, headDim, nHeads, stream));
+    HIPCHK(launch_rope(K, cosRow, sinRow, 1, kvDim, headDim, nKVHeads, stream));
+    HIPCHK(launch_kv_cache_write(kCache[layer], K, pos, kvDim, stream));
+    HIPCHK(launch_kv_cache_write(vCache[layer], V, pos, kvDim, stream));
+    AttnParams a{};
+    a.q = Q; a.Kc = kCache[layer]; a.Vc = vCache[layer]; a.posImm = pos;
+    a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
+    a.fused = 0; a.direct = 1; a.out = attnOut; a.smax = 1; a.minSplit = 1;
+    HIPCHK(launch_attention(a, stream));
+    HIPCHK(mv(L.wo, attnOut, proj));
+    HIPCHK(launch_add_inplace(h, proj, dim, stream));
+    HIPCHK(launch_rmsnorm_out(h, normed2, L.norm2, 1, dim, eps, stream));
+    HIPCHK(mv(L.gate, normed2, gatePre));
+    HIPCHK(mv(L.up, normed2, upOut));
+    HIPCHK(launch_silu_gate_mul(gatePre, upOut, ffnMid, ffnDim, stream));
+    HIPCHK(mv(L.down, ffnMid, proj));
+    HIPCHK(launch_add_inplace(h, proj, dim, stream));
+    return MG_OK;
+}
+
+// Five launches a layer: [norm1+QKV+bias] [RoPE+KV write+attention]
+// [combine+Wo+residual] [norm2+gate/up+SiLU*mul] [down+residual].
+int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const StepState* st, int posImm) {
+    float* h = hidden[hiddenIdx];
+    {
+        MvParams p{};
+        p.K = dim; p.act = h; p.gain = L.norm1; p.eps = eps;
+        if (L.wq.kind == L.wk.kind && L.wk.kind == L.wv.kind) {
+            p.seg[0] = MvSeg{L.wq.w, L.wq.scales, L.bq, Q, dim};
+            p.seg[1] = MvSeg{L.wk.w, L.wk.scales, L.bk, K, kvDim};
+            p.seg[2] = MvSeg{L.wv.w, L.wv.scales, L.bv, V, kvDim};
+            p.nseg = 3;
+            HIPCHK(launch_matvec(L.wq.kind, EPI_STORE, PRO_RMS, p, nullptr, stream));
+        } else {
+            const DevMat* ms[3] = {&L.wq, &L.wk, &L.wv};
+            const float* bs[3] = {L.bq, L.bk, L.bv};
+            float* outs[3] = {Q, K, V};
+            for (int i = 0; i < 3; i++) {
+                p.seg[0] = MvSeg{ms[i]->w, ms[i]->scales, bs[i], outs[i], ms[i]->rows};
+                p.nseg = 1;
+                HIPCHK(launch_matvec(ms[i]->kind, EPI_STORE, PRO_RMS, p, nullptr, stream));
+            }
+        }
+    }
+    {
+        AttnParams a{};
+        a.q = Q; a.kNew = K; a.vNew = V; a.Kc = kCache[layer]; a.Vc = vCache[layer];
+        a.cosTab = cosTab; a.sinTab = sinTab; a.state = st; a.posImm = posImm;
+        a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
+        a.fused = 1; a.direct = 0; a.smax = smax; a.minSplit = minSplit;
+        a.pm = pm; a.pl = pl; a.pacc = pacc;
+        HIPCHK(launch_attention(a, stream));
+    }
+    {
+        MvParams p{};
+        p.seg[0] = MvSeg{L.wo.w, L.wo.scales, nullptr, h, dim};
+        p.nseg = 1; p.K = dim;
+        p.pm = pm; p.pl = pl; p.pacc = pacc; p.nHeads = nHeads; p.headDim = headDim; p.smax = smax; p.minSplit = minSplit;
+        p.state = st; p.posImm = posImm; p.resid = h;
+        HIPCHK(launch_matvec(L.wo.kind, EPI_RESID, PRO_ATTN, p, nullptr, stream));
+    }
+    if (L.gate.kind == L.up.kind) {
+        MvParams p{};
+        p.seg[0] = MvSeg{L.gate.w, L.gate.scales, nullptr, ffnMid, ffnDim};
+        p.seg[1] = MvSeg{L.up.w, L.up.scales, nullptr, nullptr, ffnDim};
+        p.nseg = 2; p.K = dim; p.act = h; p.gain = L.norm2; p.eps = eps;
+        HIPCHK(launch_matvec(L.gate.kind, EPI_SWIGLU, PRO_RMS, p, nullptr, stream));
+    } else {
+        MvParams p{};
+        p.K = dim; p.act = h; p.gain = L.norm2; p.eps = eps; p.nseg = 1;
+        p.seg[0] = MvSeg{L.gate.w, L.gate.scales, nullptr, gatePre, ffnDim};
+        HIPCHK(launch_matvec(L.gate.kind, EPI_STORE, PRO_RMS, p, nullptr, stream));
+        p.seg[0] = MvSeg{L.up.w, L.up.scales, nullptr, upOut, ffnDim};
+        HIPCHK(launch_matvec(L.up.kind, EPI_STORE, PRO_RMS, p, nullptr, stream));
+        HIPCHK(launch_silu_gate_mul(gatePre, upOut, ffnMid, ffnDim, stream));
+    }
+    {
+        MvParams p{};
+        p.seg[0] = MvSeg{L.down.w, L.down.scales, nullptr, h, dim};
+        p.nseg = 1; p.K = ffnDim; p.act = ffnMid; p.resid = h;
+        HIPCHK(launch_matvec(L.down.kind, EPI_RESID, PRO_PLAIN, p, nullptr, stream));
+    }
+    return MG_OK;
+}
+
+int HIPFusedInference::enqueueLayer(const LayerWeights& L, int layer, const StepState* st, int posImm) {
+    if (!kCache[layer] || !vCache[layer]) { set_error("layer has no KV cache: call SetLayerRange first"); return MG_E_STATE; }
+    if (!layerComplete(L)) { set_error("layer weights incomplete"); return MG_E_STATE; }
+    if (execMode == 0) {
+        if (st) { set_error("per-op mode needs a host-side position"); return MG_E_STATE; }
+        return enqueueLayerPerOp(L, layer, posImm);
+    }
+    return enqueueLayerFused(L, layer, st, posImm);
+}
+
+// Final norm + lm_head (cuda_fused_infer.go:446-448) with the per-workgroup
+// argmax folded into the matvec epilogue.
+int HIPFusedInference::enqueueFinal(bool withArgmax) {
+    if (!finalNorm || !lmHead.w) { set_error("final norm / lm_head not set"); return MG_E_STATE; }
+    MvParams p{};
+    p.seg[0] = MvSeg{lmHead.w, lmHead.scales, nullptr, logits, vocabSize};
+    p.nseg = 1; p.K = dim; p.act = hidden[hiddenIdx]; p.gain = finalNorm; p.eps = eps;
+    p.amaxVal = amaxVal; p.amaxIdx = amaxIdx;
+    MvConfig c{0, 0, 0};
+    HIPCHK(launch_matvec(lmHead.kind, withArgmax ? EPI_ARGMAX : EPI_STORE, PRO_RMS, p, &c, stream));
+    if (withArgmax) {
+        if (c.grid > amaxParts) { set_error("argmax partial buffer too small"); return MG_E_STATE; }
+        HIPCHK(launch_argmax_finish(amaxVal, amaxIdx, c.grid, dState, nullptr, dHistory, maxSeq + 1, vocabSize, stream));
+    }
+    return MG_OK;
+}
+
+int HIPFusedInference::PartialStep(const float* hiddenIn, int pos, int layerStart, int layerEnd, float* hiddenOut,
+                                   float* logitsOut) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(pos >= 0 && pos < maxSeq, "PartialStep: pos out of range");
+    ARGCHK(layerStart >= 0, "PartialStep: negative layerStart");
+    float* h = hidden[hiddenIdx];
+    if (hiddenIn) {
+        HIPCHK(hipStreamSynchronize(stream));
+        HIPCHK(hipMemcpy(h, hiddenIn, (size_t)dim * 4, hipMemcpyHostToDevice));      // :395
+    }
+    for (int l = layerStart; l < layerEnd && l < nLayers; l++) {
+        if (!layers[l].norm1) continue;                                               // :415
+        int rc = enqueueLayer(layers[l], l, nullptr, pos);
+        if (rc) return rc;
+    }
+    if (layerEnd >= nLayers && logitsOut && finalNorm) {                              // :446
+        int rc = enqueueFinal(false);
+        if (rc) return rc;
+        HIPCHK(hipStreamSynchronize(stream));
+        HIPCHK(hipMemcpy(logitsOut, logits, (size_t)vocabSize * 4, hipMemcpyDeviceToHost));
+    }
+    if (hiddenOut && layerEnd < nLayers) {                                            // :452
+        HIPCHK(hipStreamSynchronize(stream));
+        HIPCHK(hipMemcpy(hiddenOut, h, (size_t)dim * 4, hipMemcpyDeviceToHost));
+    }
+    HIPCHK(hipStreamSynchronize(stream));
+    return MG_OK;
+}
+
+int HIPFusedInference::StepLayerResident(int layer, int pos, const float* hiddenIn, float* preOut, float* postOut,
+                                         float* logitsOut) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(layer >= 0 && layer < nLayers && pos >= 0 && pos < maxSeq, "StepLayerResident: bad layer or pos");
+    float* h = hidden[hiddenIdx];
+    if (layer == 0) {
+        ARGCHK(hiddenIn, "StepLayerResident: layer 0 needs hiddenIn");
+        HIPCHK(hipStreamSynchronize(stream));
+        HIPCHK(hipMemcpy(h, hiddenIn, (size_t)dim * 4, hipMemcpyHostToDevice));
+    }
+    if (preOut) {
+        HIPCHK(hipStreamSynchronize(stream));
+        HIPCHK(hipMemcpy(preOut, h, (size_t)dim * 4, hipMemcpyDeviceToHost));
+    }
+    int rc = enqueueLayer(layers[layer], layer, nullptr, pos);
+    if (rc) return rc;
+    if (postOut) {
+        HIPCHK(hipStreamSynchronize(stream));
+        HIPCHK(hipMemcpy(postOut, h, (size_t)dim * 4, hipMemcpyDeviceToHost));
+    }
+    if (logitsOut) {
+        rc = enqueueFinal(false);
+        if (rc) return rc;
+        HIPCHK(hipStreamSynchronize(stream));
+        HIPCHK(hipMemcpy(logitsOut, logits, (size_t)vocabSize * 4, hipMemcpyDeviceToHost));
+    }
+    HIPCHK(hipStreamSynchronize(stream));
+    return MG_OK;
+}
+
+int HIPFusedInference::ExportHidden(float* out) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(out, "ExportHidden: NULL out");
+    HIPCHK(hipStreamSynchronize(stream));
+    HIPCHK(hipMemcpy(out, hidden[hiddenIdx], (size_t)dim * 4, hipMemcpyDeviceToHost));
+    return MG_OK;
+}
+
+int HIPFusedInference::enqueueEmbed() {
+    float* h = hidden[hiddenIdx];
+    if (embedKind == 1 || embedKind == 2) {
+        HIPCHK(launch_embed_token(embedKind, embedTable, nullptr, dState, h, dim, vocabSize, stream));
+    } else {
+        if (!lmHead.w) { set_error("no embedding table and no lm_head to tie to"); return MG_E_STATE; }
+        int kind = lmHead.kind == WF_Q8 ? 0 : 3;
+        HIPCHK(launch_embed_token(kind, lmHead.w, lmHead.scales, dState, h, dim, vocabSize, stream));
+    }
+    return MG_OK;
+}
+
+// One whole token from the device-resident state.
+int HIPFusedInference::enqueueToken(bool withHead) {
+    int rc = enqueueEmbed();
+    if (rc) return rc;
+    for (int l = 0; l < nLayers; l++) {
+        rc = enqueueLayerFused(layers[l], l, dState, 0);
+        if (rc) return rc;
+    }
+    if (withHead) return enqueueFinal(true);
+    HIPCHK(launch_advance_prompt(dState, dPrompt, stream));
+    return MG_OK;
+}
+
+static int checkReady(HIPFusedInference* f) {
+    for (int l = 0; l < f->nLayers; l++) {
+        if (!layerComplete(f->layers[l])) { set_error("decode: layer weights incomplete"); return MG_E_STATE; }
+        if (!f->kCache[l]) { set_error("decode: KV cache missing, call SetLayerRange(0, nLayers)"); return MG_E_STATE; }
+    }
+    if (!f->finalNorm || !f->lmHead.w) { set_error("decode: final norm / lm_head not set"); return MG_E_STATE; }
+    return MG_OK;
+}
+
+int HIPFusedInference::DecodeToken(int token, int pos, int* nextToken, float* logitsOut) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(pos >= 0 && pos < maxSeq && token >= 0 && token < vocabSize, "DecodeToken: token or pos out of range");
+    int rc = checkReady(this);
+    if (rc) return rc;
+    HIPCHK(launch_set_state(dState, pos, token, 0, 0, stream));
+    if (execMode == 0) {
+        rc = enqueueEmbed();
+        if (rc) return rc;
+        for (int l = 0; l < nLayers; l++) {
+            rc = enqueueLayerPerOp(layers[l], l, pos);
+            if (rc) return rc;
+        }
+        rc = enqueueFinal(true);
+    } else {
+        rc = enqueueToken(true);
+    }
+    if (rc) return rc;
+    HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int), hipMemcpyDeviceToHost, stream));
+    HIPCHK(hipStreamSynchronize(stream));
+    if (nextToken) *nextToken = hTokens[0];
+    if (logitsOut) HIPCHK(hipMemcpy(logitsOut, logits, (size_t)vocabSize * 4, hipMemcpyDeviceToHost));
+    return MG_OK;
+}
+
+int HIPFusedInference::GraphCapture() {
+    if (!built) return MG_E_NOT_BUILT;
+    int rc = checkReady(this);
+    if (rc) return rc;
+    if (execFull && execPrompt) return MG_OK;
+    invalidateGraphs();
+    HIPCHK(hipStreamSynchronize(stream));
+    for (int which = 0; which < 2; which++) {
+        HIPCHK(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));
+        rc = enqueueToken(which == 0);
+        hipGraph_t g = nullptr;
+        hipError_t e = hipStreamEndCapture(stream, &g);
+        if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
+        HIPCHK(e);
+        hipGraphExec_t ex = nullptr;
+        HIPCHK(hipGraphInstantiate(&ex, g, nullptr, nullptr, 0));
+        if (which == 0) { graphFull = g; execFull = ex; } else { graphPrompt = g; execPrompt = ex; }
+    }
+    return MG_OK;
+}
+
+int HIPFusedInference::GraphLaunch(int token, int pos, int* nextToken) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(pos >= 0 && pos < maxSeq && token >= 0 && token < vocabSize, "GraphLaunch: token or pos out of range");
+    int rc = GraphCapture();
+    if (rc) return rc;
+    HIPCHK(launch_set_state(dState, pos, token, 0, 0, stream));
+    HIPCHK(hipGraphLaunch(execFull, stream));
+    HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int), hipMemcpyDeviceToHost, stream));
+    HIPCHK(hipStreamSynchronize(stream));
+    if (nextToken) *nextToken = hTokens[0];
+    return MG_OK;
+}
+
+int HIPFusedInference::GraphValidate(int token, int pos, float* maxAbsDiff) {
+    if (!built) return MG_E_NOT_BUILT;
+    std::vector<float> a(vocabSize), b(vocabSize);
+    int t0 = -1, t1 = -1;
+    int saved = execMode;
+    execMode = 1;
+    int rc = DecodeToken(token, pos, &t0, a.data());
+    execMode = saved;
+    if (rc) return rc;
+    rc = GraphLaunch(token, pos, &t1);
+    if (rc) return rc;
+    HIPCHK(hipMemcpy(b.data(), logits, (size_t)vocabSize * 4, hipMemcpyDeviceToHost));
+    float md = 0.f;
+    for (int i = 0; i < vocabSize; i++) md = std::fmax(md, std::fabs(a[i] - b[i]));
+    if (t0 != t1) md = std::fmax(md, 1.0f);
+    if (maxAbsDiff) *maxAbsDiff = md;
+    return MG_OK;
+}
+
+int HIPFusedInference::Generate(const int* prompt, int nPrompt, int nDecode, int* outTokens, bool useGraph) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(prompt && nPrompt >= 1 && nDecode >= 0 && outTokens, "Generate: bad arguments");
+    ARGCHK(nPrompt + nDecode <= maxSeq + 1 && nPrompt <= maxSeq, "Generate: prompt + decode exceeds maxSeq");
+    for (int i = 0; i < nPrompt; i++) ARGCHK(prompt[i] >= 0 && prompt[i] < vocabSize, "Generate: prompt token out of range");
+    int rc = checkReady(this);
+    if (rc) return rc;
+    if (execMode == 0) {
+        // per-op mode: host-driven loop, one synchronisation per token
+        int tok = prompt[0];
+        for (int pos = 0; pos < nPrompt - 1 + nDecode; pos++) {
+            int next = -1;
+            rc = DecodeToken(tok, pos, &next, nullptr);
+            if (rc) return rc;
+            if (pos + 1 < nPrompt) tok = prompt[pos + 1];
+            else { outTokens[pos + 1 - nPrompt] = next; tok = next; }
+        }
+        return MG_OK;
+    }
+    if (useGraph) { rc = GraphCapture(); if (rc) return rc; }
+    HIPCHK(hipStreamSynchronize(stream));
+    HIPCHK(hipMemcpy(dPrompt, prompt, sizeof(int) * (size_t)nPrompt, hipMemcpyHostToDevice));
+    HIPCHK(launch_set_state(dState, 0, prompt[0], 0, nPrompt, stream));
+    for (int i = 0; i < nPrompt - 1; i++) {
+        if (useGraph) HIPCHK(hipGraphLaunch(execPrompt, stream));
+        else { rc = enqueueToken(false); if (rc) return rc; }
+    }
+    for (int i = 0; i < nDecode; i++) {
+        if (useGraph) HIPCHK(hipGraphLaunch(execFull, stream));
+        else { rc = enqueueToken(true); if (rc) return rc; }
+    }
+    if (nDecode > 0) HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int) * (size_t)nDecode, hipMemcpyDeviceToHost, stream));
+    HIPCHK(hipStreamSynchronize(stream));
+    for (int i = 0; i < nDecode; i++) outTokens[i] = hTokens[i];
+    return MG_OK;
+}
+
+int HIPFusedInference::TimedDecode(int token, int pos, int steps, bool useGraph, float* elapsedMs) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(steps >= 1 && pos >= 0 && pos + steps <= maxSeq && token >= 0 && token < vocabSize, "TimedDecode: bad arguments");
+    int rc = checkReady(this);
+    if (rc) return rc;
+    if (useGraph) { rc = GraphCapture(); if (rc) return rc; }
+    HIPCHK(launch_set_state(dState, pos, token, 0, 0, stream));
+    HIPCHK(hipStreamSynchronize(stream));
+    HIPCHK(hipEventRecord(ev0, stream));
+    for (int i = 0; i < steps; i++) {
+        if (useGraph) HIPCHK(hipGraphLaunch(execFull, stream));
+        else { rc = enqueueToken(true); if (rc) return rc; }
+    }
+    HIPCHK(hipEventRecord(ev1, stream));
+    HIPCHK(hipEventSynchronize(ev1));
+    float ms = 0.f;
+    HIPCHK(hipEventElapsedTime(&ms, ev0, ev1));
+    if (elapsedMs) *elapsedMs = ms;
+    return MG_OK;
+}
+
+}  // namespace mg
+
+// ---------------------------------------------------------------------------
+// C entry points
+// ---------------------------------------------------------------------------
+using mg::HIPFusedInference;
+struct mg_ctx { HIPFusedInference* f; };
+
+extern "C" {
+
+const char* mg_last_error(void) { return mg::get_error().c_str(); }
+
+mg_ctx* mg_create(int dim, int kvDim, int headDim, int nHeads, int nKVHeads, int ffnDim, int vocabSize, int nLayers,
+                  int maxSeq, double ropeTheta, float eps) {
+    mg::set_error("");
+    HIPFusedInference* f = HIPFusedInference::New(dim, kvDim, headDim, nHeads, nKVHeads, ffnDim, vocabSize, nLayers,
+                                                  maxSeq, ropeTheta, eps);
+    if (!f) return nullptr;
+    return new mg_ctx{f};
+}
+void mg_destroy(mg_ctx* c) { if (c) { delete c->f; delete c; } }
+
+#define CTX(c) if (!(c) || !(c)->f) { mg::set_error("NULL context"); return MG_E_NOT_BUILT; } HIPFusedInference* f = (c)->f
+
+int mg_num_weights(const mg_ctx* c) { return c && c->f ? c->f->NumWeights() : 0; }
+int mg_set_weight(mg_ctx* c, int idx, const float* data, size_t n) { CTX(c); return f->SetWeight(idx, data, n); }
+int mg_set_weight_q8(mg_ctx* c, int idx, const int8_t* q, const float* scales) { CTX(c); return f->SetWeightQ8(idx, q, scales); }
+int mg_set_weight_q4_0(mg_ctx* c, int idx, const uint8_t* d, size_t n) { CTX(c); return f->SetWeightQ4_0(idx, d, n); }
+int mg_set_quant_rounding(mg_ctx* c, int mode) {
+    CTX(c);
+    if (mode != 0 && mode != 1) { mg::set_error("rounding mode must be 0 or 1"); return MG_E_ARG; }
+    f->quantRounding = mode;
+    return MG_OK;
+}
+int mg_set_embedding_f16(mg_ctx* c, const uint16_t* t) { CTX(c); return f->SetEmbeddingF16(t); }
+int mg_set_embedding_f32(mg_ctx* c, const float* t) { CTX(c); return f->SetEmbeddingF32(t); }
+int mg_set_layer_range(mg_ctx* c, int a, int b) { CTX(c); return f->SetLayerRange(a, b); }
+int mg_reset_kv(mg_ctx* c) { CTX(c); return f->ResetKV(); }
+int mg_partial_step(mg_ctx* c, const float* hiddenIn, int pos, int l0, int l1, float* hiddenOut, float* logitsOut) {
+    CTX(c); return f->PartialStep(hiddenIn, pos, l0, l1, hiddenOut, logitsOut);
+}
+int mg_step_layer_resident(mg_ctx* c, int layer, int pos, const float* hiddenIn, float* preOut, float* postOut, float* logitsOut) {
+    CTX(c); return f->StepLayerResident(layer, pos, hiddenIn, preOut, postOut, logitsOut);
+}
+int mg_export_hidden(mg_ctx* c, float* out) { CTX(c); return f->ExportHidden(out); }
+int mg_set_exec_mode(mg_ctx* c, int mode) {
+    CTX(c);
+    if (mode != 0 && mode != 1) { mg::set_error("exec mode must be 0 or 1"); return MG_E_ARG; }
+    f->execMode = mode;
+    return MG_OK;
+}
+int mg_decode_token(mg_ctx* c, int token, int pos, int* next, float* logitsOut) { CTX(c); return f->DecodeToken(token, pos, next, logitsOut); }
+int mg_generate(mg_ctx* c, const int* prompt, int nPrompt, int nDecode, int* out, int useGraph) {
+    CTX(c); return f->Generate(prompt, nPrompt, nDecode, out, useGraph != 0);
+}
+int mg_graph_capture(mg_ctx* c) { CTX(c); return f->GraphCapture(); }
+int mg_graph_launch(mg_ctx* c, int token, int pos, int* next) { CTX(c); return f->GraphLaunch(token, pos, next); }
+int mg_graph_validate(mg_ctx* c, int token, int pos, float* md) { CTX(c); return f->GraphValidate(token, pos, md); }
+int mg_timed_decode(mg_ctx* c, int token, int pos, int steps, int useGraph, float* ms) {
+    CTX(c); return f->TimedDecode(token, pos, steps, useGraph != 0, ms);
+}
+uint64_t mg_weight_bytes_per_token(const mg_ctx* c) { return c && c->f ? c->f->WeightBytesPerToken() : 0; }
+uint64_t mg_kv_bytes_at(const mg_ctx* c, int pos) { return c && c->f ? c->f->KVBytesAt(pos) : 0; }
+
+}  // extern "C"

@@ -1,0 +1,131 @@
+// kernels.h -- launcher prototypes shared by the C ABI (abi.hip) and the
+// fused-inference context (fused_infer.hip).  Device code lives in kernels.hip.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mg {
+
+// Weight formats the matvec kernel reads.
+enum WeightFormat {
+    WF_Q8 = 0,      // int8 [N,K] + per-row float scale
+    WF_Q4P = 1,     // Q4_0 split layout: nibbles [N,K/2] then fp16 d [N,K/32]
+    WF_Q4RAW = 2,   // raw GGUF block_q4_0, 18-byte blocks
+};
+
+// How the activation vector reaches LDS.
+enum Prologue {
+    PRO_PLAIN = 0,  // act[K] copied
+    PRO_RMS = 1,    // act = rmsnorm(x, gain, eps)
+    PRO_ATTN = 2,   // act = combined split-KV attention partials
+};
+
+// What happens to each finished row.
+enum Epilogue {
+    EPI_STORE = 0,   // out[r] = v (+ bias[r])
+    EPI_RESID = 1,   // out[r] = resid[r] + v
+    EPI_SWIGLU = 2,  // seg0 = gate, seg1 = up: out[r] = silu(g) * u
+    EPI_ARGMAX = 3,  // out[r] = v and a per-workgroup running (max, index)
+};
+
+// Device-resident step state, so that a captured graph needs no new arguments
+// per token (what tw_graph_params was meant for, cuda_graph.go:181-205).
+struct StepState {
+    int pos;        // position of the token being processed
+    int token;      // its id
+    int count;      // tokens emitted so far into the history buffer
+    int nPrompt;    // prompt length (tokens < nPrompt come from the prompt buffer)
+};
+
+struct MvSeg {
+    const void* w;        // weights (format WF)
+    const void* aux;      // Q8: float scales[rows]; Q4P: unused (d follows the nibbles); Q4RAW: unused
+    const float* bias;    // optional
+    float* out;
+    int rows;
+};
+
+struct MvParams {
+    MvSeg seg[3];
+    int nseg;
+    int K;
+    int ngroups;          // row groups over all segments
+    int segGroup0[3];     // first group of each segment
+    // prologue
+    const float* act;     // PRO_PLAIN: activation; PRO_RMS: x
+    const float* gain;
+    float eps;
+    // PRO_ATTN: split-KV partials
+    const float* pm;      // [nHeads, smax]
+    const float* pl;      // [nHeads, smax]
+    const float* pacc;    // [nHeads, smax, headDim]
+    int nHeads, headDim, smax, minSplit;
+    const StepState* state;  // position source for PRO_ATTN (may be NULL -> posImm)
+    int posImm;
+    // epilogue
+    const float* resid;
+    int div127;           // Q8: multiply by scales[r]/127 instead of scales[r]
+    float* amaxVal;       // EPI_ARGMAX partials [gridDim.x]
+    int* amaxIdx;
+};
+
+struct MvConfig { int nr; int ks; int grid; };
+
+// Positions per split so that ceil(len/splitLen) <= smax; shared by the
+// attention kernel and the combining prologue.
+__host__ __device__ inline int attn_split_len(int len, int smax, int minSplit) {
+    int s = (len + smax - 1) / smax;
+    if (s < minSplit) s = minSplit;
+    return s;
+}
+
+MvConfig pick_config(int wf, int epi, int totalRows, int K);
+// Launch the matvec; returns hipSuccess or the launch error.  cfgInOut may be
+// NULL or have nr == 0 (pick automatically); the configuration used, with the
+// grid size, is written back.
+hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInOut, hipStream_t s);
+
+struct AttnParams {
+    const float* q;       // [dim]   (raw, bias added, not rotated when fused)
+    const float* kNew;    // [kvDim] (fused only)
+    const float* vNew;    // [kvDim] (fused only)
+    float* Kc;            // [maxSeq, kvDim]
+    float* Vc;
+    const float* cosTab;  // [maxSeq, headDim/2] (fused only)
+    const float* sinTab;
+    const StepState* state;   // position source (NULL -> posImm)
+    int posImm;
+    int kvDim, nHeads, nKVHeads, headDim;
+    int fused;            // 1: rotate q, rotate+store k, store v at pos
+    int smax, minSplit;
+    float* pm; float* pl; float* pacc;   // partial outputs (direct == 0)
+    float* out;           // direct == 1: final [dim] output, single split
+    int direct;
+};
+hipError_t launch_attention(const AttnParams& p, hipStream_t s);
+
+hipError_t launch_rmsnorm_out(const float* in, float* out, const float* w, int seqLen, int dim, float eps, hipStream_t s);
+hipError_t launch_rope(float* x, const float* cosTab, const float* sinTab, int seqLen, int dim, int headDim, int nHeads, hipStream_t s);
+hipError_t launch_kv_cache_write(float* cache, const float* src, int pos, int kvDim, hipStream_t s);
+hipError_t launch_silu_gate_mul(const float* gate, const float* up, float* out, int n, hipStream_t s);
+hipError_t launch_add_inplace(float* a, const float* b, int n, hipStream_t s);
+hipError_t launch_embed_gather_f32(float* out, const float* embed, const int* tokens, int seqLen, int dim, hipStream_t s);
+hipError_t launch_dequant_q8(const void* w, const float* scales, float* out, int rows, int cols, int div127, hipStream_t s);
+hipError_t launch_dequant_q4_0(const void* w, float* out, int rows, int cols, hipStream_t s);
+hipError_t launch_q4_0_repack(const void* raw, void* planar, int N, int K, hipStream_t s);
+hipError_t launch_matvec_generic_q8(const float* act, const void* w, const float* scales, float* out, int N, int K, int div127, hipStream_t s);
+hipError_t launch_fill_zero(void* ptr, size_t bytes, hipStream_t s);
+
+// Embedding row of state->token into x[dim]: kind 0 = Q8 row * scale (tied
+// lm_head), 1 = fp16 table, 2 = fp32 table, 3 = Q4_0 split-layout row.
+hipError_t launch_embed_token(int kind, const void* table, const float* scales, const StepState* state,
+                              float* x, int dim, int vocab, hipStream_t s);
+// Reduce the lm_head partials to a token, append it to the history and
+// advance the step state (next token comes from the prompt while pos+1 < nPrompt).
+hipError_t launch_argmax_finish(const float* pv, const int* pi, int nparts, StepState* state,
+                                const int* prompt, int* history, int historyCap, int vocab, hipStream_t s);
+hipError_t launch_set_state(StepState* state, int pos, int token, int count, int nPrompt, hipStream_t s);
+// Advance state without an lm_head (prompt positions): pos++, token = prompt[pos].
+hipError_t launch_advance_prompt(StepState* state, const int* prompt, hipStream_t s);
+
+}  // namespace mg

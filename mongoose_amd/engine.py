@@ -1,0 +1,403 @@
+"""Host-side mirror of mongoose's Go API for the fused quantized decode path.
+
+Same names, argument meaning and error behaviour as the Go types they stand
+in for, so that tests read like the reference's:
+
+    HIP / NewHIP               Engine + the TensorEngine memory calls
+                               (engine.go:7-29, tensor.go:29-49, cuda.go:198-223)
+    Tensor                     tensor.go:15-89
+    K* functions               kernels.go:600-1136 wrappers over the per-op launches
+    HIPFusedInference          CUDAFusedInference (cuda_fused_infer.go,
+                               cuda_fused_infer_q4.go, cuda_fused_infer_stub.go:7-49)
+    HIPStreamInfer             CUDAStreamInfer (cuda_fused_stream.go)
+
+Everything here is a thin ctypes call into libmongoose_hip.so; there is no
+computation in Python and no CPU fallback.
+"""
+import ctypes
+
+import numpy as np
+
+from .lib import lib, last_error
+
+_f = ctypes.POINTER(ctypes.c_float)
+_i = ctypes.POINTER(ctypes.c_int)
+
+
+def _fp(a):
+    return a.ctypes.data_as(_f) if a is not None else None
+
+
+def _ip(a):
+    return a.ctypes.data_as(_i) if a is not None else None
+
+
+def _as_f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+class Tensor:
+    """Device buffer owned by an engine (tensor.go:15-27)."""
+
+    def __init__(self, eng, ptr, nbytes, shape):
+        self.eng, self._ptr, self.nbytes, self.Shape = eng, ptr, nbytes, list(shape)
+
+    def DevicePtr(self):
+        return self._ptr
+
+    def Size(self):
+        n = 1
+        for s in self.Shape:
+            n *= s
+        return n
+
+    def Release(self):
+        if self._ptr:
+            lib.tw_gpu_free(self._ptr)
+            self._ptr = None
+
+
+def ptrAdd(ptr, nbytes):
+    """kernel_tensor.go:9-11."""
+    return ctypes.c_void_p(ptr.value + nbytes if isinstance(ptr, ctypes.c_void_p) else ptr + nbytes)
+
+
+class HIP:
+    """The engine object NewHIP() returns (cuda.go:198-223 for CUDA)."""
+
+    def __init__(self, name, vram):
+        self._name, self._vram = name, vram
+
+    def Name(self):
+        return "hip/" + self._name
+
+    def VRAM(self):
+        return self._vram
+
+    # TensorEngine memory calls (cuda_tensor.go:563-627, 980-990)
+    def FromHost(self, data, shape):
+        a = _as_f32(data)
+        ptr = lib.tw_gpu_alloc(a.nbytes)
+        if not ptr:
+            return None
+        lib.tw_gpu_upload(ptr, a.ctypes.data, a.nbytes)
+        return Tensor(self, ptr, a.nbytes, shape)
+
+    def Zeros(self, shape):
+        n = int(np.prod(shape))
+        ptr = lib.tw_gpu_alloc(n * 4)
+        if not ptr:
+            return None
+        lib.tw_gpu_zero(ptr, n * 4)
+        return Tensor(self, ptr, n * 4, shape)
+
+    def ToHost(self, t):
+        out = np.empty(t.Size(), dtype=np.float32)
+        lib.tw_gpu_download(out.ctypes.data, t.DevicePtr(), out.nbytes)
+        return out
+
+    def UploadInto(self, t, data):
+        a = _as_f32(data)
+        lib.tw_gpu_upload(t.DevicePtr(), a.ctypes.data, a.nbytes)
+
+    def UploadRawBytes(self, data):
+        a = np.ascontiguousarray(data).view(np.uint8).ravel()
+        ptr = lib.tw_gpu_alloc(a.nbytes)
+        if not ptr:
+            return None
+        lib.tw_gpu_upload(ptr, a.ctypes.data, a.nbytes)
+        return Tensor(self, ptr, a.nbytes, [a.nbytes])
+
+    def DownloadRawBytes(self, t, nbytes=None):
+        out = np.empty(nbytes if nbytes is not None else t.nbytes, dtype=np.uint8)
+        lib.tw_gpu_download(out.ctypes.data, t.DevicePtr(), out.nbytes)
+        return out
+
+    def UploadQ4_0(self, q4Data, rows, cols):
+        """cuda_q4_0.go:15-26: raw GGUF block_q4_0 bytes."""
+        return self.UploadRawBytes(np.asarray(q4Data, dtype=np.uint8)[: rows * (cols // 32) * 18])
+
+
+def NewHIP(device=0):
+    """nil (None) when no device is present, as NewCUDA (cuda.go:209-217)."""
+    if lib.tw_hip_init_device(device) != 0:
+        return None
+    name = ctypes.create_string_buffer(256)
+    mem = ctypes.c_uint64(0)
+    if lib.tw_hip_device_info(name, 256, ctypes.byref(mem)) != 0:
+        return None
+    return HIP(name.value.decode(), mem.value)
+
+
+def KernelsLoaded():
+    return True
+
+
+# ---- kernels.go:600-1136 style wrappers (default stream, void) ----
+def _p(x):
+    return x.DevicePtr() if isinstance(x, Tensor) else x
+
+
+def KRMSNormOut(inp, out, w, seqLen, dim):
+    lib.mongoose_rmsnorm_out(_p(inp), _p(out), _p(w), seqLen, dim, None)
+
+
+def KRMSNormOutEps(inp, out, w, seqLen, dim, eps):
+    lib.mongoose_rmsnorm_out_eps(_p(inp), _p(out), _p(w), seqLen, dim, eps, None)
+
+
+def KQ8Matvec(act, w, scales, out, N, K):
+    lib.mongoose_q8_matvec(_p(act), _p(w), _p(scales), _p(out), N, K, None)
+
+
+def KQ8MatvecRowScale(act, w, scales, out, N, K):
+    lib.mongoose_q8_matvec_rowscale(_p(act), _p(w), _p(scales), _p(out), N, K, None)
+
+
+def KQ4_0Matvec(act, w, out, N, K):
+    lib.mongoose_q4_0_matvec(_p(act), _p(w), _p(out), N, K, None)
+
+
+def KQ4_0Repack(w, planar, N, K):
+    lib.mongoose_q4_0_repack(_p(w), _p(planar), N, K, None)
+
+
+def KQ4_0MatvecPlanar(act, planar, out, N, K):
+    lib.mongoose_q4_0_matvec_planar(_p(act), _p(planar), _p(out), N, K, None)
+
+
+def KRoPE(x, cos, sin, seqLen, dim, headDim, nHeads):
+    lib.mongoose_rope(_p(x), _p(cos), _p(sin), seqLen, dim, headDim, nHeads, None)
+
+
+def KKVCacheWrite(cache, src, pos, kvDim):
+    lib.mongoose_kv_cache_write(_p(cache), _p(src), pos, kvDim, None)
+
+
+def KDecodeAttention(Q, K, V, out, cacheLen, dim, kvDim, nHeads, nKVHeads):
+    lib.mongoose_decode_attention(_p(Q), _p(K), _p(V), _p(out), cacheLen, dim, kvDim, nHeads, nKVHeads, None)
+
+
+def KSiLUGateMul(gate, up, out, n):
+    lib.mongoose_silu_gate_mul(_p(gate), _p(up), _p(out), n, None)
+
+
+def KAddInPlace(a, b, n):
+    lib.mongoose_add_inplace(_p(a), _p(b), n, None)
+
+
+def KEmbedGather2(out, embed, tokens, seqLen, dim):
+    lib.mongoose_embed_gather(_p(out), _p(embed), _p(tokens), seqLen, dim, None)
+
+
+def KDequantInt8ToFP32(w, scales, out, rows, cols):
+    lib.mongoose_dequant_int8_to_fp32(_p(w), _p(scales), _p(out), rows, cols, None)
+
+
+def KDequantQ8RowScale(w, scales, out, rows, cols):
+    lib.mongoose_dequant_q8_rowscale(_p(w), _p(scales), _p(out), rows, cols, None)
+
+
+def KDequantQ4_0(w, out, rows, cols):
+    lib.mongoose_dequant_q4_0(_p(w), _p(out), rows, cols, None)
+
+
+def KCopy(dst, src, nbytes):
+    lib.mongoose_copy(_p(dst), _p(src), nbytes, None)
+
+
+def KZero(ptr, nbytes):
+    lib.mongoose_zero(_p(ptr), nbytes, None)
+
+
+def KSync():
+    lib.mongoose_sync(None)
+
+
+def HIPCheck():
+    """kernels.go:732-736 CUDACheck: 0 when no launch failed."""
+    return lib.mongoose_check()
+
+
+# ---- host helpers ----
+def quantize_q8(w, mode=0):
+    w = _as_f32(w)
+    rows, cols = w.shape
+    q = np.empty((rows, cols), dtype=np.int8)
+    s = np.empty(rows, dtype=np.float32)
+    lib.mg_quantize_q8(_fp(w), rows, cols, mode, q.ctypes.data_as(ctypes.POINTER(ctypes.c_int8)), _fp(s))
+    return q, s
+
+
+def quantize_q4_0(w):
+    w = _as_f32(w)
+    rows, cols = w.shape
+    out = np.empty(rows * (cols // 32) * 18, dtype=np.uint8)
+    lib.mg_quantize_q4_0(_fp(w), rows, cols, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)))
+    return out
+
+
+def synth_normal(seed, idx, std, shape):
+    out = np.empty(shape, dtype=np.float32)
+    lib.mg_synth_normal(seed, idx, std, _fp(out), out.size)
+    return out
+
+
+def synth_tokens(seed, idx, bound, n):
+    out = np.empty(n, dtype=np.int32)
+    lib.mg_synth_tokens(seed, idx, bound, _ip(out), n)
+    return out
+
+
+class HIPFusedInference:
+    """Method set of CUDAFusedInference (cuda_fused_infer_stub.go:11-49)."""
+
+    def __init__(self, handle, shape):
+        self._h = handle
+        (self.dim, self.kvDim, self.headDim, self.nHeads, self.nKVHeads, self.ffnDim, self.vocabSize,
+         self.nLayers, self.maxSeq) = shape
+
+    def Close(self):
+        if self._h:
+            lib.mg_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.Close()
+        except Exception:
+            pass
+
+    def NumWeights(self):
+        return lib.mg_num_weights(self._h)
+
+    def SetWeight(self, idx, data):
+        a = _as_f32(data).ravel()
+        return lib.mg_set_weight(self._h, idx, _fp(a), a.size)
+
+    def SetWeightQ8(self, idx, q, scales):
+        q = np.ascontiguousarray(q, dtype=np.int8)
+        s = _as_f32(scales)
+        return lib.mg_set_weight_q8(self._h, idx, q.ctypes.data_as(ctypes.POINTER(ctypes.c_int8)), _fp(s))
+
+    def SetWeightQ4_0(self, idx, q4Data):
+        a = np.ascontiguousarray(q4Data, dtype=np.uint8).ravel()
+        return lib.mg_set_weight_q4_0(self._h, idx, a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), a.size)
+
+    def SetQuantRounding(self, mode):
+        return lib.mg_set_quant_rounding(self._h, mode)
+
+    def SetEmbeddingF16(self, table):
+        a = np.ascontiguousarray(table).view(np.uint16)
+        return lib.mg_set_embedding_f16(self._h, a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint16)))
+
+    def SetEmbeddingF32(self, table):
+        a = _as_f32(table)
+        return lib.mg_set_embedding_f32(self._h, _fp(a))
+
+    def SetLayerRange(self, layerStart, layerEnd):
+        return lib.mg_set_layer_range(self._h, layerStart, layerEnd)
+
+    def ResetKV(self):
+        return lib.mg_reset_kv(self._h)
+
+    def SetExecMode(self, mode):
+        return lib.mg_set_exec_mode(self._h, mode)
+
+    def PartialStep(self, hiddenIn, pos, layerStart, layerEnd, hiddenOut, logitsOut):
+        h = _as_f32(hiddenIn) if hiddenIn is not None else None
+        return lib.mg_partial_step(self._h, _fp(h), pos, layerStart, layerEnd, _fp(hiddenOut), _fp(logitsOut))
+
+    def PartialStepContinue(self, pos, layerStart, layerEnd, hiddenOut, logitsOut):
+        return lib.mg_partial_step(self._h, None, pos, layerStart, layerEnd, _fp(hiddenOut), _fp(logitsOut))
+
+    # the Q4 step is the same entry point: the weight format is a property of each matrix
+    PartialStepQ4 = PartialStep
+    PartialStepQ4Continue = PartialStepContinue
+
+    def StepLayerResident(self, layer, pos, hiddenIn, preOut, postOut, logitsOut):
+        h = _as_f32(hiddenIn) if hiddenIn is not None else None
+        return lib.mg_step_layer_resident(self._h, layer, pos, _fp(h), _fp(preOut), _fp(postOut), _fp(logitsOut))
+
+    def ExportHidden(self):
+        out = np.empty(self.dim, dtype=np.float32)
+        rc = lib.mg_export_hidden(self._h, _fp(out))
+        return out if rc == 0 else None
+
+    def DecodeToken(self, token, pos, logitsOut=None):
+        nxt = ctypes.c_int(-1)
+        rc = lib.mg_decode_token(self._h, token, pos, ctypes.byref(nxt), _fp(logitsOut))
+        return rc, nxt.value
+
+    def Generate(self, prompt, nDecode, useGraph=True):
+        p = np.ascontiguousarray(prompt, dtype=np.int32)
+        out = np.empty(max(nDecode, 1), dtype=np.int32)
+        rc = lib.mg_generate(self._h, _ip(p), p.size, nDecode, _ip(out), 1 if useGraph else 0)
+        return rc, out[:nDecode]
+
+    def CaptureGraph(self):
+        return lib.mg_graph_capture(self._h)
+
+    def GraphLaunch(self, token, pos):
+        nxt = ctypes.c_int(-1)
+        rc = lib.mg_graph_launch(self._h, token, pos, ctypes.byref(nxt))
+        return rc, nxt.value
+
+    def ValidateGraph(self, token, pos):
+        md = ctypes.c_float(0)
+        rc = lib.mg_graph_validate(self._h, token, pos, ctypes.byref(md))
+        return rc, md.value
+
+    def TimedDecode(self, token, pos, steps, useGraph=True):
+        ms = ctypes.c_float(0)
+        rc = lib.mg_timed_decode(self._h, token, pos, steps, 1 if useGraph else 0, ctypes.byref(ms))
+        return rc, ms.value
+
+    def WeightBytesPerToken(self):
+        return lib.mg_weight_bytes_per_token(self._h)
+
+    def KVBytesAt(self, pos):
+        return lib.mg_kv_bytes_at(self._h, pos)
+
+    def StreamBuild(self):
+        h = lib.mg_stream_build(self._h)
+        return HIPStreamInfer(h, self) if h else None
+
+
+def NewHIPFusedInference(eng, dim, kvDim, headDim, nHeads, nKVHeads, ffnDim, vocabSize, nLayers, maxSeq,
+                         ropeTheta, eps=1e-6):
+    """NewCUDAFusedInference (cuda_fused_infer.go:144): None on failure."""
+    if eng is None:
+        return None
+    h = lib.mg_create(dim, kvDim, headDim, nHeads, nKVHeads, ffnDim, vocabSize, nLayers, maxSeq,
+                      float(ropeTheta), float(eps))
+    if not h:
+        return None
+    return HIPFusedInference(h, (dim, kvDim, headDim, nHeads, nKVHeads, ffnDim, vocabSize, nLayers, maxSeq))
+
+
+class HIPStreamInfer:
+    """CUDAStreamInfer (cuda_fused_stream.go:98-126)."""
+
+    def __init__(self, handle, parent):
+        self._h, self._parent = handle, parent
+
+    def Close(self):
+        if self._h:
+            lib.mg_stream_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.Close()
+        except Exception:
+            pass
+
+    def StreamForwardToken(self, pos, embHidden, nLayers, layerPtrs, layerSizes, logitsOut):
+        """layerPtrs: list of nLayers*12 numpy arrays or None; layerSizes: nLayers*7 ints."""
+        keep = [np.ascontiguousarray(a) if a is not None else None for a in layerPtrs]
+        arr = (ctypes.c_void_p * len(keep))(*[a.ctypes.data if a is not None else None for a in keep])
+        sizes = np.ascontiguousarray(layerSizes, dtype=np.int32)
+        h = _as_f32(embHidden)
+        return lib.mg_stream_forward_token(self._h, pos, _fp(h), nLayers, arr,
+                                           sizes.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), _fp(logitsOut))

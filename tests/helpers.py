@@ -1,0 +1,134 @@
+"""Shared test helpers: deterministic synthetic models loaded into the CPU
+oracle and/or the HIP context with identical quantized bytes."""
+import numpy as np
+
+from mongoose_amd import configs
+from mongoose_amd import engine as E
+from oracle import binding as ob
+
+MATRIX_SLOTS = (1, 2, 3, 7, 9, 10, 11)
+
+
+def slot_shape(s, idx):
+    """(rows, cols) of a weight slot; cols == 1 for vectors (cuda_fused_infer.go:241-272)."""
+    kv = configs.kv_dim(s)
+    nL = s.nLayers
+    if idx < nL * 12:
+        w = idx % 12
+        return {0: (s.dim, 1), 1: (s.dim, s.dim), 2: (kv, s.dim), 3: (kv, s.dim), 4: (s.dim, 1), 5: (kv, 1),
+                6: (kv, 1), 7: (s.dim, s.dim), 8: (s.dim, 1), 9: (s.ffnDim, s.dim), 10: (s.ffnDim, s.dim),
+                11: (s.dim, s.ffnDim)}[w]
+    if idx == nL * 12:
+        return (s.dim, 1)
+    return (s.vocab, s.dim)
+
+
+def gen_slot(s, seed, idx):
+    """fp32 data of a slot: matrices and biases N(0, 0.02), norm gains 1 + N(0, 0.02)
+    (not exactly 1, so that a dropped or misplaced gain would show)."""
+    rows, cols = slot_shape(s, idx)
+    a = E.synth_normal(seed, idx, 0.02, (rows, cols) if cols > 1 else (rows,))
+    w = idx % 12 if idx < s.nLayers * 12 else -1
+    if cols == 1 and (w in (0, 8) or idx == s.nLayers * 12):
+        a = (a + np.float32(1.0)).astype(np.float32)
+    return a
+
+
+def all_slots(s):
+    for idx in range(s.nLayers * 12 + 2):
+        w = idx % 12 if idx < s.nLayers * 12 else -1
+        if w in (4, 5, 6) and not s.bias:
+            continue
+        yield idx
+
+
+def with_layers(s, n):
+    return s._replace(nLayers=n, name=f"{s.name}-L{n}")
+
+
+class Model:
+    """Oracle and/or HIP context holding the same synthetic model."""
+
+    def __init__(self, s, seed, maxSeq, eng=None, oracle=True, threads=8, fmt=None, keep_dequant=False):
+        self.s, self.seed, self.maxSeq = s, seed, maxSeq
+        fmt = fmt or s.fmt
+        kv = configs.kv_dim(s)
+        self.orc = ob.Oracle(s.dim, kv, s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab, s.nLayers, maxSeq,
+                             s.theta, s.eps, threads=threads) if oracle else None
+        self.hip = None
+        if eng is not None:
+            self.hip = E.NewHIPFusedInference(eng, s.dim, kv, s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab,
+                                              s.nLayers, maxSeq, s.theta, s.eps)
+            assert self.hip is not None, E.last_error()
+            assert self.hip.SetLayerRange(0, s.nLayers) == 0, E.last_error()
+        self.dequant = {} if keep_dequant else None
+        self.vecs = {}
+        for idx in all_slots(s):
+            rows, cols = slot_shape(s, idx)
+            data = gen_slot(s, seed, idx)
+            if cols == 1:
+                self.vecs[idx] = data
+                if self.orc:
+                    self.orc.set_f32(idx, data)
+                if self.hip:
+                    assert self.hip.SetWeight(idx, data) == 0, E.last_error()
+                continue
+            if fmt == "q8":
+                q, sc = ob.quantize_q8(data, 0)
+                if self.orc:
+                    self.orc.set_q8(idx, q, sc)
+                if self.hip:
+                    assert self.hip.SetWeightQ8(idx, q, sc) == 0, E.last_error()
+                if keep_dequant:
+                    self.dequant[idx] = ob.dequant_q8(q, sc)
+            else:
+                blocks = ob.quantize_q4_0(data)
+                if self.orc:
+                    self.orc.set_q4_0(idx, blocks)
+                if self.hip:
+                    assert self.hip.SetWeightQ4_0(idx, blocks) == 0, E.last_error()
+                if keep_dequant:
+                    self.dequant[idx] = ob.dequant_q4_0(blocks, rows, cols)
+        if not s.tied:
+            # separate fp16 embedding table (the Q4_0 configuration keeps embeddings in fp16)
+            emb = E.synth_normal(seed, 10_000_019, 0.02, (s.vocab, s.dim)).astype(np.float16)
+            self.embed16 = emb
+            if self.orc:
+                self.orc.set_embed_f16(emb)
+            if self.hip:
+                assert self.hip.SetEmbeddingF16(emb) == 0, E.last_error()
+
+    def prompt(self, n):
+        return E.synth_tokens(self.seed, 20_000_003, self.s.vocab, n)
+
+    def close(self):
+        if self.hip:
+            self.hip.Close()
+        if self.orc:
+            self.orc.close()
+
+
+def rel_err(a, b):
+    """max |a-b| / max |b|: error relative to the largest entry of the reference vector."""
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    den = np.abs(b).max()
+    return float(np.abs(a - b).max() / den) if den > 0 else float(np.abs(a - b).max())
+
+
+def oracle_generate(m, prompt, nDecode, want=None, shadow=False):
+    """Greedy decode on the oracle; returns (tokens, per-position records)."""
+    m.orc.reset_kv()
+    toks, rec = [], {}
+    tok = int(prompt[0])
+    nP = len(prompt)
+    for pos in range(nP - 1 + nDecode):
+        nxt, logits, layers = m.orc.decode_token(tok, pos, shadow=shadow, want_layers=want is not None and pos in want)
+        if want is not None and pos in want:
+            rec[pos] = (logits.copy(), layers.copy())
+        if pos + 1 < nP:
+            tok = int(prompt[pos + 1])
+        else:
+            toks.append(nxt)
+            tok = nxt
+    return np.array(toks, np.int32), rec
