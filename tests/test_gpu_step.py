@@ -1,0 +1,280 @@
+"""End-to-end parity of the decode step on the GPU against the CPU oracle on
+identical seeded, identically quantized weights.
+
+Bars (the ones the benchmark definition states): per-layer hidden state within
+1e-4 relative, final logits within 1e-3 relative, greedy token sequences
+identical.  "Relative" is max|gpu-ref| / max|ref| over the vector.  The
+reference for the tolerances is the oracle's double-precision shadow, which
+separates summation-order noise from defects; the float path (the Go CPU
+engine's arithmetic) is checked to the same bars."""
+import numpy as np
+import pytest
+
+from mongoose_amd import configs
+from mongoose_amd import engine as E
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+HID_TOL = 1e-4
+LOGIT_TOL = 1e-3
+
+
+def _gpu_layers(m, tok_hidden, pos):
+    """Per-layer hidden states through StepLayerResident snapshots, plus logits."""
+    s = m.s
+    layers = np.empty((s.nLayers, s.dim), np.float32)
+    logits = np.empty(s.vocab, np.float32)
+    for l in range(s.nLayers):
+        post = np.empty(s.dim, np.float32)
+        rc = m.hip.StepLayerResident(l, pos, tok_hidden if l == 0 else None, None, post,
+                                     logits if l == s.nLayers - 1 else None)
+        assert rc == 0, E.last_error()
+        layers[l] = post
+    return layers, logits
+
+
+def _compare_sequence(m, prompt, nDecode, check_positions):
+    """Greedy tokens identical + hidden/logit bars at selected positions."""
+    toks_ref, rec = H.oracle_generate(m, prompt, nDecode, want=set(check_positions))
+    toks_ref64, rec64 = H.oracle_generate(m, prompt, nDecode, want=set(check_positions), shadow=True)
+    # GPU: whole loop on the device, graph replay
+    assert m.hip.ResetKV() == 0
+    rc, toks = m.hip.Generate(prompt, nDecode, useGraph=True)
+    assert rc == 0, E.last_error()
+    # and eagerly (no graph)
+    assert m.hip.ResetKV() == 0
+    rc, toks_eager = m.hip.Generate(prompt, nDecode, useGraph=False)
+    assert rc == 0, E.last_error()
+    assert (toks == toks_eager).all()
+    assert (toks_ref == toks_ref64).all(), "oracle float and double paths disagree: a near-tie, pick another seed"
+    assert (toks == toks_ref).all(), (toks.tolist(), toks_ref.tolist())
+    # per-layer hidden + logits: replay the same token stream one position at a time
+    assert m.hip.ResetKV() == 0
+    stream = list(prompt) + list(toks_ref)
+    for pos in range(len(prompt) - 1 + nDecode):
+        h = m.orc.embed(stream[pos])
+        if pos in check_positions:
+            layers, logits = _gpu_layers(m, h, pos)
+            lg32, ly32 = rec[pos]
+            lg64, ly64 = rec64[pos]
+            for l in range(m.s.nLayers):
+                assert H.rel_err(layers[l], ly64[l]) < HID_TOL, (pos, l)
+                assert H.rel_err(layers[l], ly32[l]) < HID_TOL, (pos, l)
+            assert H.rel_err(logits, lg64) < LOGIT_TOL and H.rel_err(logits, lg32) < LOGIT_TOL, pos
+            assert int(np.argmax(logits)) == int(np.argmax(lg32))
+        else:
+            assert m.hip.PartialStep(h, pos, 0, m.s.nLayers, None, None) == 0, E.last_error()
+
+
+def test_toy_q8_full_workload(hip):
+    """Toy configuration exactly as stated: 8-token prompt, 64 greedy tokens."""
+    s = configs.TOY
+    m = H.Model(s, seed=1, maxSeq=72, eng=hip, threads=8)
+    prompt = m.prompt(8)
+    _compare_sequence(m, prompt, 64, check_positions=[0, 7, 40, 70])
+    m.close()
+
+
+def test_toy_q8_against_golden_fixture(hip):
+    import os
+    fx = np.load(os.path.join(os.path.dirname(__file__), "golden", "toy_q8.npz"))
+    s = configs.TOY
+    m = H.Model(s, seed=int(fx["seed"]), maxSeq=72, eng=hip, oracle=False)
+    rc, toks = m.hip.Generate(fx["prompt"], 64, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert (toks == fx["tokens"]).all()
+    assert m.hip.ResetKV() == 0
+    stream = list(fx["prompt"]) + list(fx["tokens"])
+    # logits at the recorded positions, replaying the recorded token stream
+    want = {int(p): i for i, p in enumerate(fx["positions"])}
+    for pos in range(8 - 1 + 64):
+        logits = np.empty(s.vocab, np.float32)
+        rc, nxt = m.hip.DecodeToken(int(stream[pos]), pos, logits)
+        assert rc == 0, E.last_error()
+        if pos in want:
+            assert H.rel_err(logits, fx["logits"][want[pos]]) < LOGIT_TOL
+            hid = m.hip.ExportHidden()
+            assert H.rel_err(hid, fx["hidden_last"][want[pos]]) < HID_TOL
+    m.close()
+
+
+def test_qwen_shape_q8_short(hip):
+    """Qwen2.5-0.5B shape (GQA 14/2, QKV bias, tied 151936-row lm_head): 4-token prompt, 4 tokens."""
+    s = configs.QWEN
+    m = H.Model(s, seed=2, maxSeq=16, eng=hip, threads=8)
+    prompt = m.prompt(4)
+    _compare_sequence(m, prompt, 4, check_positions=[0, 3, 6])
+    assert m.hip.WeightBytesPerToken() == configs.weight_bytes_per_token(s) == 495961088
+    m.close()
+
+
+def test_qwen_shape_q4_0_short(hip):
+    """Same shape, Q4_0 linears, fp16 embedding table."""
+    s = configs.QWEN_Q4
+    m = H.Model(s, seed=3, maxSeq=16, eng=hip, threads=8)
+    prompt = m.prompt(4)
+    _compare_sequence(m, prompt, 4, check_positions=[0, 5])
+    assert m.hip.WeightBytesPerToken() == configs.weight_bytes_per_token(s) == 278028800
+    m.close()
+
+
+def test_tinyllama_shape_q8_two_layers(hip):
+    """TinyLlama shape (dim 2048, GQA 32/4, untied head), 2 of 22 layers so the oracle stays fast."""
+    s = H.with_layers(configs.TINYLLAMA, 2)
+    m = H.Model(s, seed=4, maxSeq=16, eng=hip, threads=8)
+    prompt = m.prompt(4)
+    _compare_sequence(m, prompt, 4, check_positions=[0, 6])
+    m.close()
+
+
+def test_llama3_8b_shape_q8_one_layer(hip):
+    """Llama-3-8B shape (dim 4096, head 128, GQA 32/8, ffn 14336), 1 layer, vocab cut to 8192 rows."""
+    s = H.with_layers(configs.LLAMA3_8B, 1)._replace(vocab=8192)
+    m = H.Model(s, seed=5, maxSeq=12, eng=hip, threads=8)
+    prompt = m.prompt(3)
+    _compare_sequence(m, prompt, 3, check_positions=[0, 4])
+    m.close()
+
+
+def test_per_op_mode_matches_fused_mode(hip):
+    """The 17-launch reference order and the fused launches agree to rounding."""
+    s = H.with_layers(configs.QWEN, 2)._replace(vocab=4096)
+    m = H.Model(s, seed=6, maxSeq=12, eng=hip, oracle=True, threads=8)
+    prompt = m.prompt(5)
+    outs = {}
+    for mode in (0, 1):
+        assert m.hip.SetExecMode(mode) == 0
+        assert m.hip.ResetKV() == 0
+        res = []
+        for pos in range(5):
+            logits = np.empty(s.vocab, np.float32)
+            hid = np.empty(s.dim, np.float32)
+            assert m.hip.PartialStep(m.orc.embed(prompt[pos]), pos, 0, 1, hid, None) == 0, E.last_error()
+            assert m.hip.PartialStepContinue(pos, 1, 2, None, logits) == 0, E.last_error()
+            res.append((hid.copy(), logits.copy()))
+        outs[mode] = res
+    for (h0, l0), (h1, l1) in zip(outs[0], outs[1]):
+        assert H.rel_err(h0, h1) < 1e-5 and H.rel_err(l0, l1) < 1e-5
+    # and both against the oracle at the last position
+    m.orc.reset_kv()
+    for pos in range(5):
+        _, lg, _ = m.orc.step(m.orc.embed(prompt[pos]), pos, shadow=True)
+    assert H.rel_err(outs[0][4][1], lg) < LOGIT_TOL and H.rel_err(outs[1][4][1], lg) < LOGIT_TOL
+    m.close()
+
+
+def test_graph_replay_matches_eager(hip):
+    """cuda_graph.go:554-598: graph vs non-graph, max abs logit difference < 1e-3 (here: equal)."""
+    s = H.with_layers(configs.QWEN, 3)._replace(vocab=8192)
+    m = H.Model(s, seed=7, maxSeq=32, eng=hip, oracle=False)
+    prompt = m.prompt(6)
+    rc, _ = m.hip.Generate(prompt, 4, useGraph=False)
+    assert rc == 0, E.last_error()
+    assert m.hip.CaptureGraph() == 0, E.last_error()
+    for rep in range(3):                       # several replays with eager work in between
+        rc, md = m.hip.ValidateGraph(int(prompt[rep]), 9 + rep)
+        assert rc == 0, E.last_error()
+        assert md < 1e-3, md
+        assert md == 0.0
+    m.close()
+
+
+def test_long_context_split_kv(hip):
+    """Context long enough for several KV splits (GQA 7 heads per KV head);
+    logits and hidden still match the oracle at the split boundaries and at the end."""
+    s = H.with_layers(configs.QWEN, 1)._replace(vocab=2048)
+    maxSeq = 1100
+    m = H.Model(s, seed=8, maxSeq=maxSeq, eng=hip, threads=8)
+    prompt = m.prompt(maxSeq)
+    m.orc.reset_kv()
+    assert m.hip.ResetKV() == 0
+    check = {0, 255, 256, 257, 511, 512, 768, 1023, 1024, 1098, 1099}
+    for pos in range(maxSeq):
+        h = m.orc.embed(prompt[pos])
+        want = pos in check
+        hid64, lg, _ = m.orc.step(h, pos, shadow=True, want_logits=want)
+        logits = np.empty(s.vocab, np.float32) if want else None
+        assert m.hip.PartialStep(h, pos, 0, 1, None, logits) == 0, E.last_error()
+        if want:
+            assert H.rel_err(logits, lg) < LOGIT_TOL, pos
+            assert H.rel_err(m.hip.ExportHidden(), hid64) < HID_TOL, pos
+    m.close()
+
+
+def test_edge_cases_and_errors(hip):
+    s = H.with_layers(configs.TOY, 1)
+    kv = configs.kv_dim(s)
+    f = E.NewHIPFusedInference(hip, s.dim, kv, s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab, 1, 8, s.theta, s.eps)
+    assert f is not None and f.NumWeights() == 14
+    h = np.zeros(s.dim, np.float32)
+    # a layer without norm1 is skipped (cuda_fused_infer.go:415): hidden passes through
+    h[:] = 0.5
+    assert f.PartialStep(h, 0, 0, 1, None, None) == 0
+    assert (f.ExportHidden() == 0.5).all()
+    # bad arguments
+    assert f.PartialStep(h, 8, 0, 1, None, None) != 0          # pos == maxSeq
+    assert f.PartialStep(h, -1, 0, 1, None, None) != 0
+    assert f.SetWeight(1, np.zeros(7, np.float32)) != 0         # wrong element count
+    assert f.SetWeight(99, np.zeros(7, np.float32)) != 0        # no such slot
+    assert f.SetWeightQ4_0(1, np.zeros(5, np.uint8)) != 0       # wrong byte count
+    assert f.SetWeightQ4_0(0, np.zeros(5, np.uint8)) == 0       # norm slot: ignored (cuda_fused_infer_q4.go:52)
+    rc, _ = f.DecodeToken(0, 0)
+    assert rc != 0                                              # weights incomplete
+    assert "incomplete" in E.last_error() or "KV" in E.last_error()
+    f.Close()
+    # unsupported head size and inconsistent dims: nil constructor
+    assert E.NewHIPFusedInference(hip, 96, 96, 96, 1, 1, 128, 64, 1, 8, 1e4) is None
+    assert E.NewHIPFusedInference(hip, 512, 512, 64, 7, 7, 1376, 256, 1, 8, 1e4) is None
+
+
+def test_last_position_of_the_cache(hip):
+    """pos == maxSeq-1 is the last legal position; generating up to it works."""
+    s = H.with_layers(configs.TOY, 2)
+    m = H.Model(s, seed=9, maxSeq=12, eng=hip, threads=4)
+    prompt = m.prompt(4)
+    toks_ref, _ = H.oracle_generate(m, prompt, 9)          # positions 0..11
+    rc, toks = m.hip.Generate(prompt, 9, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert (toks == toks_ref).all()
+    rc, _ = m.hip.Generate(prompt, 10, useGraph=True)       # would need position 12
+    assert rc != 0
+    m.close()
+
+
+def test_streaming_matches_resident(hip):
+    """StreamForwardToken (weights staged from host memory per layer) == resident Q4_0 step."""
+    s = H.with_layers(configs.QWEN_Q4, 4)._replace(vocab=4096)
+    m = H.Model(s, seed=10, maxSeq=8, eng=hip, threads=8)
+    st = m.hip.StreamBuild()
+    assert st is not None, E.last_error()
+    from oracle import binding as ob
+    ptrs, sizes = [], []
+    for l in range(s.nLayers):
+        for w in range(12):
+            idx = l * 12 + w
+            rows, cols = H.slot_shape(s, idx)
+            data = H.gen_slot(s, m.seed, idx)
+            if cols == 1:
+                ptrs.append(data if (w not in (4, 5, 6) or s.bias) else None)
+            else:
+                blk = ob.quantize_q4_0(data)
+                ptrs.append(blk)
+                sizes.append(blk.size)
+    prompt = m.prompt(5)
+    m.orc.reset_kv()
+    for pos in range(5):
+        h = m.orc.embed(prompt[pos])
+        _, lg, _ = m.orc.step(h, pos, shadow=True)
+        logits = np.empty(s.vocab, np.float32)
+        rc = st.StreamForwardToken(pos, h, s.nLayers, ptrs, sizes, logits)
+        assert rc == 0, E.last_error()
+        assert H.rel_err(logits, lg) < LOGIT_TOL, pos
+    # resident path on the same positions gives the same logits as streaming
+    assert m.hip.ResetKV() == 0
+    for pos in range(5):
+        logits2 = np.empty(s.vocab, np.float32)
+        assert m.hip.PartialStepQ4(m.orc.embed(prompt[pos]), pos, 0, s.nLayers, None, logits2) == 0
+    assert (logits2 == logits).all()
+    st.Close()
+    m.close()
