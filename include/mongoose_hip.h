@@ -197,6 +197,15 @@ int mg_graph_validate(mg_ctx* ctx, int token, int pos, float* maxAbsDiff);
  * region starts. */
 int mg_timed_decode(mg_ctx* ctx, int token, int pos, int steps, int useGraph, float* elapsedMs);
 
+/* Per-launch-class timing inside a token, for the roofline report: `steps`
+ * (<= 64) tokens from (token, pos) are issued launch by launch with an event
+ * between every two launches, queued behind a gate so that the GPU never
+ * waits for the host.  classMs[8] = mean milliseconds per launch
+ * of class {0 embedding gather, 1 norm+QKV(+bias), 2 RoPE+KV write+attention,
+ * 3 Wo+residual, 4 norm+gate/up+SiLU*mul, 5 down+residual, 6 final norm+lm_head
+ * (+argmax partials), 7 argmax finish}; classLaunches[8] = launches per token. */
+int mg_profile_decode(mg_ctx* ctx, int token, int pos, int steps, float* classMs, int* classLaunches);
+
 /* Bytes of weights, scales and norm gains one token reads (the figure the
  * bandwidth roofline is computed from), and the KV bytes read at position pos. */
 uint64_t mg_weight_bytes_per_token(const mg_ctx* ctx);

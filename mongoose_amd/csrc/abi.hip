@@ -111,11 +111,11 @@ void mongoose_decode_attention(const float* Q, const float* K, const float* V, f
                                int nHeads, int nKVHeads, void* stream) {
     if (cacheLen <= 0 || nHeads <= 0) return;
     mg::AttnParams p{};
-    p.q = Q; p.Kc = const_cast<float*>(K); p.Vc = const_cast<float*>(V);
+    p.q = Q; p.Kc = K; p.Vc = V;
     p.posImm = cacheLen - 1;
     p.kvDim = kvDim; p.nHeads = nHeads; p.nKVHeads = nKVHeads;
     p.headDim = dim / nHeads;                                    // mongoose.cu:939
-    p.fused = 0; p.direct = 1; p.out = out; p.smax = 1; p.minSplit = 1;
+    p.direct = 1; p.out = out; p.smax = 1; p.minSplit = 1;
     note(mg::launch_attention(p, S(stream)));
 }
 void mongoose_silu_gate_mul(const float* gate, const float* up, float* out, int n, void* stream) {

@@ -58,6 +58,7 @@ public:
     int GraphLaunch(int token, int pos, int* nextToken);                          // cuda_graph.go:663
     int GraphValidate(int token, int pos, float* maxAbsDiff);                     // cuda_graph.go:554
     int TimedDecode(int token, int pos, int steps, bool useGraph, float* elapsedMs);
+    int ProfileDecode(int token, int pos, int steps, float* classMs, int* classLaunches);
     uint64_t WeightBytesPerToken() const;
     uint64_t KVBytesAt(int pos) const { return (uint64_t)2 * nLayers * (uint64_t)(pos + 1) * kvDim * 4; }
 
@@ -108,6 +109,7 @@ private:
     // token-level state
     StepState* dState = nullptr;
     StepState* hState = nullptr;    // pinned mirror
+    int* hGate = nullptr;           // pinned flag the timing gate kernel polls
     float* amaxVal = nullptr;
     int* amaxIdx = nullptr;
     int amaxParts = 0;
@@ -117,6 +119,11 @@ private:
     hipGraph_t graphFull = nullptr, graphPrompt = nullptr;
     hipGraphExec_t execFull = nullptr, execPrompt = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    // instrumented run: an event between every two launches of a token
+    std::vector<hipEvent_t> profEvents;
+    std::vector<int> profClass;       // class of the launch that follows event i
+    bool profiling = false;
+    int mark(int cls);
 };
 
 }  // namespace mg

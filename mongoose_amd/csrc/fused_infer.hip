@@ -112,6 +112,9 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
     void* hp = nullptr;
     if (hipHostMalloc(&hp, sizeof(StepState), hipHostMallocDefault) != hipSuccess) return fail("pinned alloc");
     f->hState = static_cast<StepState*>(hp);
+    if (hipHostMalloc(&hp, 64, hipHostMallocDefault) != hipSuccess) return fail("pinned alloc");
+    f->hGate = static_cast<int*>(hp);
+    *f->hGate = 1;
     if (hipHostMalloc(&hp, sizeof(int) * ((size_t)maxSeq + 1), hipHostMallocDefault) != hipSuccess) return fail("pinned alloc");
     f->hTokens = static_cast<int*>(hp);
 
@@ -144,7 +147,9 @@ HIPFusedInference::~HIPFusedInference() {
     if (dPrompt) (void)hipFree(dPrompt);
     if (embedTable) (void)hipFree(embedTable);
     if (hState) (void)hipHostFree(hState);
+    if (hGate) (void)hipHostFree(hGate);
     if (hTokens) (void)hipHostFree(hTokens);
+    for (hipEvent_t e : profEvents) (void)hipEventDestroy(e);
     if (ev0) (void)hipEventDestroy(ev0);
     if (ev1) (void)hipEventDestroy(ev1);
     if (stream) (void)hipStreamDestroy(stream);
@@ -327,6 +332,18 @@ uint64_t HIPFusedInference::WeightBytesPerToken() const {
     return b;
 }
 
+// While the instrumented graph is being captured: an event before the launch
+// of class `cls` (the previous launch's end).  No-op otherwise.
+int HIPFusedInference::mark(int cls) {
+    if (!profiling) return MG_OK;
+    hipEvent_t e = nullptr;
+    HIPCHK(hipEventCreate(&e));
+    profEvents.push_back(e);
+    profClass.push_back(cls);
+    HIPCHK(hipEventRecord(e, stream));
+    return MG_OK;
+}
+
 static bool layerComplete(const LayerWeights& L) {
     return L.norm1 && L.norm2 && L.wq.w && L.wk.w && L.wv.w && L.wo.w && L.gate.w && L.up.w && L.down.w;
 }
@@ -358,7 +375,7 @@ int HIPFusedInference::enqueueLayerPerOp(const LayerWeights& L, int layer, int p
     AttnParams a{};
     a.q = Q; a.Kc = kCache[layer]; a.Vc = vCache[layer]; a.posImm = pos;
     a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
-    a.fused = 0; a.direct = 1; a.out = attnOut; a.smax = 1; a.minSplit = 1;
+    a.direct = 1; a.out = attnOut; a.smax = 1; a.minSplit = 1;
     HIPCHK(launch_attention(a, stream));
     HIPCHK(mv(L.wo, attnOut, proj));
     HIPCHK(launch_add_inplace(h, proj, dim, stream));
@@ -371,39 +388,33 @@ int HIPFusedInference::enqueueLayerPerOp(const LayerWeights& L, int layer, int p
     return MG_OK;
 }
 
-// Five launches a layer: [norm1+QKV+bias] [RoPE+KV write+attention]
-// [combine+Wo+residual] [norm2+gate/up+SiLU*mul] [down+residual].
+// Five launches a layer: [norm1 + QKV + bias + RoPE + KV-cache write] [attention]
+// [combine + Wo + residual] [norm2 + gate/up + SiLU*mul] [down + residual].
 int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const StepState* st, int posImm) {
     float* h = hidden[hiddenIdx];
+    if (mark(1)) return MG_E_HIP;
     {
         MvParams p{};
         p.K = dim; p.act = h; p.gain = L.norm1; p.eps = eps;
-        if (L.wq.kind == L.wk.kind && L.wk.kind == L.wv.kind) {
-            p.seg[0] = MvSeg{L.wq.w, L.wq.scales, L.bq, Q, dim};
-            p.seg[1] = MvSeg{L.wk.w, L.wk.scales, L.bk, K, kvDim};
-            p.seg[2] = MvSeg{L.wv.w, L.wv.scales, L.bv, V, kvDim};
-            p.nseg = 3;
-            HIPCHK(launch_matvec(L.wq.kind, EPI_STORE, PRO_RMS, p, nullptr, stream));
-        } else {
-            const DevMat* ms[3] = {&L.wq, &L.wk, &L.wv};
-            const float* bs[3] = {L.bq, L.bk, L.bv};
-            float* outs[3] = {Q, K, V};
-            for (int i = 0; i < 3; i++) {
-                p.seg[0] = MvSeg{ms[i]->w, ms[i]->scales, bs[i], outs[i], ms[i]->rows};
-                p.nseg = 1;
-                HIPCHK(launch_matvec(ms[i]->kind, EPI_STORE, PRO_RMS, p, nullptr, stream));
-            }
-        }
+        p.seg[0] = MvSeg{L.wq.w, L.wq.scales, L.bq, Q, dim};
+        p.seg[1] = MvSeg{L.wk.w, L.wk.scales, L.bk, kCache[layer], kvDim};
+        p.seg[2] = MvSeg{L.wv.w, L.wv.scales, L.bv, vCache[layer], kvDim};
+        p.nseg = 3;
+        p.headDim = headDim; p.kvDim = kvDim; p.cosTab = cosTab; p.sinTab = sinTab;
+        p.state = st; p.posImm = posImm;
+        HIPCHK(launch_matvec(L.wq.kind, EPI_QKV, PRO_RMS, p, nullptr, stream));
     }
+    if (mark(2)) return MG_E_HIP;
     {
         AttnParams a{};
-        a.q = Q; a.kNew = K; a.vNew = V; a.Kc = kCache[layer]; a.Vc = vCache[layer];
-        a.cosTab = cosTab; a.sinTab = sinTab; a.state = st; a.posImm = posImm;
+        a.q = Q; a.Kc = kCache[layer]; a.Vc = vCache[layer];
+        a.state = st; a.posImm = posImm;
         a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
-        a.fused = 1; a.direct = 0; a.smax = smax; a.minSplit = minSplit;
+        a.direct = 0; a.smax = smax; a.minSplit = minSplit;
         a.pm = pm; a.pl = pl; a.pacc = pacc;
         HIPCHK(launch_attention(a, stream));
     }
+    if (mark(3)) return MG_E_HIP;
     {
         MvParams p{};
         p.seg[0] = MvSeg{L.wo.w, L.wo.scales, nullptr, h, dim};
@@ -412,21 +423,15 @@ int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const
         p.state = st; p.posImm = posImm; p.resid = h;
         HIPCHK(launch_matvec(L.wo.kind, EPI_RESID, PRO_ATTN, p, nullptr, stream));
     }
-    if (L.gate.kind == L.up.kind) {
+    if (mark(4)) return MG_E_HIP;
+    {
         MvParams p{};
         p.seg[0] = MvSeg{L.gate.w, L.gate.scales, nullptr, ffnMid, ffnDim};
         p.seg[1] = MvSeg{L.up.w, L.up.scales, nullptr, nullptr, ffnDim};
         p.nseg = 2; p.K = dim; p.act = h; p.gain = L.norm2; p.eps = eps;
         HIPCHK(launch_matvec(L.gate.kind, EPI_SWIGLU, PRO_RMS, p, nullptr, stream));
-    } else {
-        MvParams p{};
-        p.K = dim; p.act = h; p.gain = L.norm2; p.eps = eps; p.nseg = 1;
-        p.seg[0] = MvSeg{L.gate.w, L.gate.scales, nullptr, gatePre, ffnDim};
-        HIPCHK(launch_matvec(L.gate.kind, EPI_STORE, PRO_RMS, p, nullptr, stream));
-        p.seg[0] = MvSeg{L.up.w, L.up.scales, nullptr, upOut, ffnDim};
-        HIPCHK(launch_matvec(L.up.kind, EPI_STORE, PRO_RMS, p, nullptr, stream));
-        HIPCHK(launch_silu_gate_mul(gatePre, upOut, ffnMid, ffnDim, stream));
     }
+    if (mark(5)) return MG_E_HIP;
     {
         MvParams p{};
         p.seg[0] = MvSeg{L.down.w, L.down.scales, nullptr, h, dim};
@@ -439,8 +444,10 @@ int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const
 int HIPFusedInference::enqueueLayer(const LayerWeights& L, int layer, const StepState* st, int posImm) {
     if (!kCache[layer] || !vCache[layer]) { set_error("layer has no KV cache: call SetLayerRange first"); return MG_E_STATE; }
     if (!layerComplete(L)) { set_error("layer weights incomplete"); return MG_E_STATE; }
-    if (execMode == 0) {
-        if (st) { set_error("per-op mode needs a host-side position"); return MG_E_STATE; }
+    // the fused QKV and gate/up launches read their matrices with one kernel: same format needed
+    const bool uniform = L.wq.kind == L.wk.kind && L.wk.kind == L.wv.kind && L.gate.kind == L.up.kind;
+    if (execMode == 0 || !uniform) {
+        if (st) { set_error("per-op launches need a host-side position (mixed weight formats in a layer, or exec mode 0)"); return MG_E_STATE; }
         return enqueueLayerPerOp(L, layer, posImm);
     }
     return enqueueLayerFused(L, layer, st, posImm);
@@ -455,7 +462,9 @@ int HIPFusedInference::enqueueFinal(bool withArgmax) {
     p.nseg = 1; p.K = dim; p.act = hidden[hiddenIdx]; p.gain = finalNorm; p.eps = eps;
     p.amaxVal = amaxVal; p.amaxIdx = amaxIdx;
     MvConfig c{0, 0, 0};
-    HIPCHK(launch_matvec(lmHead.kind, withArgmax ? EPI_ARGMAX : EPI_STORE, PRO_RMS, p, &c, stream));
+    if (mark(6)) return MG_E_HIP;
+    HIPCHK(launch_matvec(lmHead.kind, EPI_ARGMAX, PRO_RMS, p, &c, stream));
+    if (mark(7)) return MG_E_HIP;
     if (withArgmax) {
         if (c.grid > amaxParts) { set_error("argmax partial buffer too small"); return MG_E_STATE; }
         HIPCHK(launch_argmax_finish(amaxVal, amaxIdx, c.grid, dState, nullptr, dHistory, maxSeq + 1, vocabSize, stream));
@@ -532,6 +541,7 @@ int HIPFusedInference::ExportHidden(float* out) {
 
 int HIPFusedInference::enqueueEmbed() {
     float* h = hidden[hiddenIdx];
+    if (mark(0)) return MG_E_HIP;
     if (embedKind == 1 || embedKind == 2) {
         HIPCHK(launch_embed_token(embedKind, embedTable, nullptr, dState, h, dim, vocabSize, stream));
     } else {
@@ -547,7 +557,7 @@ int HIPFusedInference::enqueueToken(bool withHead) {
     int rc = enqueueEmbed();
     if (rc) return rc;
     for (int l = 0; l < nLayers; l++) {
-        rc = enqueueLayerFused(layers[l], l, dState, 0);
+        rc = enqueueLayer(layers[l], l, dState, 0);
         if (rc) return rc;
     }
     if (withHead) return enqueueFinal(true);
@@ -700,6 +710,53 @@ int HIPFusedInference::TimedDecode(int token, int pos, int steps, bool useGraph,
     return MG_OK;
 }
 
+// Per-launch-class durations inside a token.  Events cannot be read back from
+// graph nodes, so the same launches are issued eagerly with an event between
+// every two of them -- behind a gate kernel that holds the stream until the
+// host has queued the whole batch, so the GPU never waits for the host.
+// classMs[c] = mean milliseconds from the end of the previous launch to the
+// end of a launch of class c (0 embed, 1 norm+QKV, 2 attention, 3 Wo,
+// 4 gate/up, 5 down, 6 lm_head, 7 argmax finish); classLaunches[c] = launches per token.
+int HIPFusedInference::ProfileDecode(int token, int pos, int steps, float* classMs, int* classLaunches) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(steps >= 1 && steps <= 64 && pos >= 0 && pos + steps <= maxSeq && token >= 0 && token < vocabSize &&
+           classMs && classLaunches, "ProfileDecode: bad arguments (1 <= steps <= 64)");
+    int rc = checkReady(this);
+    if (rc) return rc;
+    HIPCHK(hipStreamSynchronize(stream));
+    for (hipEvent_t e : profEvents) (void)hipEventDestroy(e);
+    profEvents.clear(); profClass.clear();
+    int* gate = hGate;
+    *reinterpret_cast<volatile int*>(gate) = 0;
+    HIPCHK(launch_set_state(dState, pos, token, 0, 0, stream));
+    HIPCHK(launch_gate(gate, 100LL * 1000 * 500, stream));   // at most 0.5 s
+    profiling = true;
+    for (int i = 0; i < steps && rc == 0; i++) {
+        rc = enqueueToken(true);
+        if (rc == 0) rc = mark(8);
+    }
+    profiling = false;
+    *reinterpret_cast<volatile int*>(gate) = 1;
+    HIPCHK(hipStreamSynchronize(stream));
+    if (rc) return rc;
+    double acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (size_t k = 0; k + 1 < profEvents.size(); k++) {
+        int c = profClass[k];
+        if (c < 0 || c >= 8) continue;
+        float ms = 0.f;
+        HIPCHK(hipEventElapsedTime(&ms, profEvents[k], profEvents[k + 1]));
+        acc[c] += ms; cnt[c]++;
+    }
+    for (int c = 0; c < 8; c++) {
+        classMs[c] = cnt[c] ? (float)(acc[c] / cnt[c]) : 0.f;
+        classLaunches[c] = cnt[c] / steps;
+    }
+    for (hipEvent_t e : profEvents) (void)hipEventDestroy(e);
+    profEvents.clear(); profClass.clear();
+    return MG_OK;
+}
+
 }  // namespace mg
 
 // ---------------------------------------------------------------------------
@@ -760,6 +817,9 @@ int mg_graph_launch(mg_ctx* c, int token, int pos, int* next) { CTX(c); return f
 int mg_graph_validate(mg_ctx* c, int token, int pos, float* md) { CTX(c); return f->GraphValidate(token, pos, md); }
 int mg_timed_decode(mg_ctx* c, int token, int pos, int steps, int useGraph, float* ms) {
     CTX(c); return f->TimedDecode(token, pos, steps, useGraph != 0, ms);
+}
+int mg_profile_decode(mg_ctx* c, int token, int pos, int steps, float* classMs, int* classLaunches) {
+    CTX(c); return f->ProfileDecode(token, pos, steps, classMs, classLaunches);
 }
 uint64_t mg_weight_bytes_per_token(const mg_ctx* c) { return c && c->f ? c->f->WeightBytesPerToken() : 0; }
 uint64_t mg_kv_bytes_at(const mg_ctx* c, int pos) { return c && c->f ? c->f->KVBytesAt(pos) : 0; }

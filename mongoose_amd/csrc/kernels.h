@@ -26,6 +26,7 @@ enum Epilogue {
     EPI_RESID = 1,   // out[r] = resid[r] + v
     EPI_SWIGLU = 2,  // seg0 = gate, seg1 = up: out[r] = silu(g) * u
     EPI_ARGMAX = 3,  // out[r] = v and a per-workgroup running (max, index)
+    EPI_QKV = 4,     // seg0 = q, seg1 = k, seg2 = v: bias, RoPE on q/k, k/v stored into the caches at pos
 };
 
 // Device-resident step state, so that a captured graph needs no new arguments
@@ -60,8 +61,12 @@ struct MvParams {
     const float* pl;      // [nHeads, smax]
     const float* pacc;    // [nHeads, smax, headDim]
     int nHeads, headDim, smax, minSplit;
-    const StepState* state;  // position source for PRO_ATTN (may be NULL -> posImm)
+    const StepState* state;  // position source for PRO_ATTN / EPI_QKV (may be NULL -> posImm)
     int posImm;
+    // EPI_QKV: RoPE tables [maxSeq, headDim/2]; seg1.out / seg2.out are the K / V caches [maxSeq, kvDim]
+    const float* cosTab;
+    const float* sinTab;
+    int kvDim;
     // epilogue
     const float* resid;
     int div127;           // Q8: multiply by scales[r]/127 instead of scales[r]
@@ -86,17 +91,12 @@ MvConfig pick_config(int wf, int epi, int totalRows, int K);
 hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInOut, hipStream_t s);
 
 struct AttnParams {
-    const float* q;       // [dim]   (raw, bias added, not rotated when fused)
-    const float* kNew;    // [kvDim] (fused only)
-    const float* vNew;    // [kvDim] (fused only)
-    float* Kc;            // [maxSeq, kvDim]
-    float* Vc;
-    const float* cosTab;  // [maxSeq, headDim/2] (fused only)
-    const float* sinTab;
+    const float* q;       // [dim], rotated
+    const float* Kc;      // [maxSeq, kvDim], row pos already written
+    const float* Vc;
     const StepState* state;   // position source (NULL -> posImm)
     int posImm;
     int kvDim, nHeads, nKVHeads, headDim;
-    int fused;            // 1: rotate q, rotate+store k, store v at pos
     int smax, minSplit;
     float* pm; float* pl; float* pacc;   // partial outputs (direct == 0)
     float* out;           // direct == 1: final [dim] output, single split
@@ -127,5 +127,8 @@ hipError_t launch_argmax_finish(const float* pv, const int* pi, int nparts, Step
 hipError_t launch_set_state(StepState* state, int pos, int token, int count, int nPrompt, hipStream_t s);
 // Advance state without an lm_head (prompt positions): pos++, token = prompt[pos].
 hipError_t launch_advance_prompt(StepState* state, const int* prompt, hipStream_t s);
+
+// Stream gate for timing runs: waits for *flag != 0 (host-pinned) or limitTicks of the 100 MHz wall clock.
+hipError_t launch_gate(const int* flag, long long limitTicks, hipStream_t s);
 
 }  // namespace mg

@@ -63,26 +63,49 @@ __device__ __forceinline__ int act_slot4(int k4, int nch) {   // k4 = k/4 -> flo
     return p * nch + c;
 }
 
-template <int CH>
-__device__ void stage_activation(const MvParams& p, int pro, float4* a4, float* red) {
+// All global loads of a prologue are issued before anything waits on them; the
+// caller has already issued its first weight loads, so the activation latency
+// and the weight latency overlap instead of adding up.
+template <int CH, int PRO>
+__device__ __forceinline__ void stage_activation(const MvParams& p, float4* a4, float* red) {
     const int K4 = p.K >> 2;
     const int nch = p.K / CH;
     const int tid = threadIdx.x;
-    if (pro == PRO_PLAIN) {
+    if (PRO == PRO_PLAIN) {
         const float4* x4 = reinterpret_cast<const float4*>(p.act);
         for (int i = tid; i < K4; i += WG) a4[act_slot4<CH>(i, nch)] = x4[i];
-    } else if (pro == PRO_RMS) {
+    } else if (PRO == PRO_RMS) {
         // mongoose.cu:145-174 / cpu.go:36-47: x * (1/sqrt(mean(x^2)+eps)) * g
+        constexpr int XR = 4;                       // float4s kept in registers per thread (K <= 4096)
         const float4* x4 = reinterpret_cast<const float4*>(p.act);
         const float4* g4 = reinterpret_cast<const float4*>(p.gain);
+        float4 xv[XR], gv[XR];
+#pragma unroll
+        for (int r = 0; r < XR; r++) {
+            int i = tid + r * WG;
+            if (i < K4) { xv[r] = x4[i]; gv[r] = g4[i]; }
+            else { xv[r] = make_float4(0.f, 0.f, 0.f, 0.f); gv[r] = xv[r]; }
+        }
         float ss = 0.f;
-        for (int i = tid; i < K4; i += WG) {
+#pragma unroll
+        for (int r = 0; r < XR; r++) ss += xv[r].x * xv[r].x + xv[r].y * xv[r].y + xv[r].z * xv[r].z + xv[r].w * xv[r].w;
+        for (int i = tid + XR * WG; i < K4; i += WG) {
             float4 v = x4[i];
             ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
         }
         float tot = block_sum(ss, red);
         float rs = 1.0f / sqrtf(tot / (float)p.K + p.eps);
-        for (int i = tid; i < K4; i += WG) {
+#pragma unroll
+        for (int r = 0; r < XR; r++) {
+            int i = tid + r * WG;
+            if (i < K4) {
+                float4 o;
+                o.x = xv[r].x * rs * gv[r].x; o.y = xv[r].y * rs * gv[r].y;
+                o.z = xv[r].z * rs * gv[r].z; o.w = xv[r].w * rs * gv[r].w;
+                a4[act_slot4<CH>(i, nch)] = o;
+            }
+        }
+        for (int i = tid + XR * WG; i < K4; i += WG) {
             float4 v = x4[i], g = g4[i], o;
             o.x = v.x * rs * g.x; o.y = v.y * rs * g.y; o.z = v.z * rs * g.z; o.w = v.w * rs * g.w;
             a4[act_slot4<CH>(i, nch)] = o;
@@ -98,18 +121,24 @@ __device__ void stage_activation(const MvParams& p, int pro, float4* a4, float* 
             int h = i / hd4, d4 = i % hd4;
             const float* pm = p.pm + (size_t)h * p.smax;
             const float* pl = p.pl + (size_t)h * p.smax;
-            float M = pm[0];
-            for (int s = 1; s < nsplit; s++) M = fmaxf(M, pm[s]);
-            float den = 0.f;
-            float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
-            for (int s = 0; s < nsplit; s++) {
-                float w = nsplit == 1 ? 1.0f : expf(pm[s] - M);
-                den += w * pl[s];
-                float4 a = reinterpret_cast<const float4*>(p.pacc + ((size_t)h * p.smax + s) * p.headDim)[d4];
-                num.x += w * a.x; num.y += w * a.y; num.z += w * a.z; num.w += w * a.w;
-            }
             float4 o;
-            o.x = num.x / den; o.y = num.y / den; o.z = num.z / den; o.w = num.w / den;
+            if (nsplit == 1) {
+                float den = pl[0];
+                float4 a = reinterpret_cast<const float4*>(p.pacc + (size_t)h * p.smax * p.headDim)[d4];
+                o.x = a.x / den; o.y = a.y / den; o.z = a.z / den; o.w = a.w / den;
+            } else {
+                float M = pm[0];
+                for (int s = 1; s < nsplit; s++) M = fmaxf(M, pm[s]);
+                float den = 0.f;
+                float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
+                for (int s = 0; s < nsplit; s++) {
+                    float w = expf(pm[s] - M);
+                    den += w * pl[s];
+                    float4 a = reinterpret_cast<const float4*>(p.pacc + ((size_t)h * p.smax + s) * p.headDim)[d4];
+                    num.x += w * a.x; num.y += w * a.y; num.z += w * a.z; num.w += w * a.w;
+                }
+                o.x = num.x / den; o.y = num.y / den; o.z = num.z / den; o.w = num.w / den;
+            }
             a4[act_slot4<CH>(i, nch)] = o;
         }
     }
@@ -204,15 +233,59 @@ template <> struct Fmt<WF_Q4RAW> {
 };
 
 // ---------------------------------------------------------------------------
-// The matvec.  One "group" is NR rows that share every activation read.
-// KS == 1: each of the 4 waves owns a group and strides K by 64 chunks.
-// KS == 4: the 4 waves share one group and stride K by 256 chunks (few rows,
-//          long K: keeps every CU loading).
+// The matvec.  A "group" is NR rows that share every activation read; KS == 1:
+// each of the 4 waves owns a group (64 lanes stride K), KS == 4: the 4 waves
+// share one group (256 lanes stride K; few rows, long K).
+//
+// Work of a wave is a stream of items (group, chunk iteration).  Items are
+// loaded D ahead of the one being consumed (register ring), the first D of
+// them before the activation vector is even staged, so the kernel's critical
+// path is one memory latency, not prologue + weights + scales in sequence.
+// Per-row epilogue operands (scale, bias, residual, RoPE factors) ride in the
+// same ring.
 // ---------------------------------------------------------------------------
-template <int WF, int NR, int KS>
-__global__ __launch_bounds__(WG) void matvec_kernel(MvParams p, int pro, int epi) {
+struct RowRef { int seg; int row; bool valid; };
+
+template <int NR, int EPI>
+__device__ __forceinline__ RowRef resolve_row(const MvParams& p, int g, int i) {
+    RowRef r;
+    if (EPI == EPI_SWIGLU) {
+        constexpr int H = NR / 2 > 0 ? NR / 2 : 1;
+        r.seg = i < H ? 0 : 1;
+        r.row = g * H + (i < H ? i : i - H);
+        r.valid = r.row < p.seg[0].rows;
+    } else if (EPI == EPI_QKV) {
+        // pairs (j, j + headDim/2) of one head for q and k, consecutive rows for v
+        int s = 0;
+        if (g >= p.segGroup0[1]) s = 1;
+        if (g >= p.segGroup0[2]) s = 2;
+        int gi = g - p.segGroup0[s];
+        r.seg = s;
+        if (s < 2) {
+            int half = p.headDim >> 1;
+            int head = gi / half, j = gi % half;
+            r.row = head * p.headDim + j + (i ? half : 0);
+        } else {
+            r.row = gi * 2 + i;
+        }
+        r.valid = r.row < p.seg[s].rows;
+    } else {
+        int s = 0;
+        if (p.nseg > 1 && g >= p.segGroup0[1]) s = 1;
+        if (p.nseg > 2 && g >= p.segGroup0[2]) s = 2;
+        r.seg = s;
+        r.row = (g - p.segGroup0[s]) * NR + i;
+        r.valid = r.row < p.seg[s].rows;
+    }
+    return r;
+}
+
+template <int WF, int NR, int KS, int PRO, int EPI>
+__global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     using F = Fmt<WF>;
     constexpr int CH = F::CH;
+    constexpr int LPG = KS == 1 ? 64 : WG;           // lanes per group
+    constexpr int D = NR >= 4 ? 2 : 4;               // items in flight per wave
     extern __shared__ float4 a4[];
     __shared__ float red[4];
     __shared__ float part[4][NR];
@@ -221,125 +294,144 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p, int pro, int epi
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lig = KS == 1 ? lane : (int)threadIdx.x;       // lane within the group
     const int nch = p.K / CH;
+    const int iters = (nch + LPG - 1) / LPG;
+    const int gStart = KS == 1 ? blockIdx.x * 4 + wave : blockIdx.x;
+    const int gStep = KS == 1 ? gridDim.x * 4 : gridDim.x;
+    const int myGroups = gStart < p.ngroups ? (p.ngroups - gStart + gStep - 1) / gStep : 0;
+    const int nItems = myGroups * iters;
 
-    stage_activation<CH>(p, pro, a4, red);
+    int pos = 0;
+    if (EPI == EPI_QKV) pos = p.state ? p.state->pos : p.posImm;
+
+    typename F::Chunk ring[D][NR];
+    float rSc[D], rBi[D], rRe[D], rCs[D], rSn[D];            // epilogue operands of the lane's row
+
+    auto issue = [&](int slot, int item) {
+        if (item >= nItems) return;
+        const int g = gStart + (item / iters) * gStep;
+        const int it = item % iters;
+        const int c = lig + it * LPG;
+#pragma unroll
+        for (int i = 0; i < NR; i++) {
+            RowRef rr = resolve_row<NR, EPI>(p, g, i);
+            if (c < nch) ring[slot][i] = F::load(F::row(p.seg[rr.seg], rr.valid ? rr.row : 0, p.K), c);
+        }
+        if (it == 0) {
+            rSc[slot] = 1.0f; rBi[slot] = 0.f; rRe[slot] = 0.f; rCs[slot] = 1.0f; rSn[slot] = 0.f;
+            if (lane < NR) {
+                RowRef rr = resolve_row<NR, EPI>(p, g, lane < NR ? lane : 0);
+                if (rr.valid) {
+                    const MvSeg& sg = p.seg[rr.seg];
+                    if (WF == WF_Q8) rSc[slot] = static_cast<const float*>(sg.aux)[rr.row];
+                    if (sg.bias) rBi[slot] = sg.bias[rr.row];
+                    if (EPI == EPI_RESID) rRe[slot] = p.resid[rr.row];
+                    if (EPI == EPI_QKV && rr.seg < 2 && lane == 0) {
+                        int half = p.headDim >> 1;
+                        int j = (g - p.segGroup0[rr.seg]) % half;
+                        rCs[slot] = p.cosTab[(size_t)pos * half + j];
+                        rSn[slot] = p.sinTab[(size_t)pos * half + j];
+                    }
+                }
+            }
+        }
+    };
+
+    // first loads go out before the activation vector is staged
+#pragma unroll
+    for (int s = 0; s < D; s++) issue(s, s);
+
+    stage_activation<CH, PRO>(p, a4, red);
     __syncthreads();
 
     float myBestV = -INFINITY;
     int myBestI = INT_MAX;
+    float acc[NR];
+#pragma unroll
+    for (int i = 0; i < NR; i++) acc[i] = 0.f;
+    float sc = 1.0f, bi = 0.f, re = 0.f, cs = 1.0f, sn = 0.f;
 
-    const int gStart = KS == 1 ? blockIdx.x * 4 + wave : blockIdx.x;
-    const int gStep = KS == 1 ? gridDim.x * 4 : gridDim.x;
-    const int c0 = KS == 1 ? lane : (int)threadIdx.x;
-    constexpr int cStep = KS == 1 ? 64 : 256;
-
-    for (int g = gStart; g < p.ngroups; g += gStep) {
-        // resolve the NR rows of this group
-        int segOf[NR], rowOf[NR];
-        bool valid[NR];
-        typename F::Row rows[NR];
-        if (epi == EPI_SWIGLU) {
-            constexpr int H = NR / 2 > 0 ? NR / 2 : 1;
+    for (int base = 0; base < nItems; base += D) {
 #pragma unroll
-            for (int i = 0; i < NR; i++) {
-                segOf[i] = i < H ? 0 : 1;
-                rowOf[i] = g * H + (i < H ? i : i - H);
-                valid[i] = rowOf[i] < p.seg[0].rows;
-            }
-        } else {
-            int s = 0;
-            if (p.nseg > 1 && g >= p.segGroup0[1]) s = 1;
-            if (p.nseg > 2 && g >= p.segGroup0[2]) s = 2;
-            int r0 = (g - p.segGroup0[s]) * NR;
+        for (int s = 0; s < D; s++) {
+            const int item = base + s;
+            if (item < nItems) {
+                const int g = gStart + (item / iters) * gStep;
+                const int it = item % iters;
+                const int c = lig + it * LPG;
+                if (c < nch) {
 #pragma unroll
-            for (int i = 0; i < NR; i++) {
-                segOf[i] = s;
-                rowOf[i] = r0 + i;
-                valid[i] = rowOf[i] < p.seg[s].rows;
-            }
-        }
+                    for (int i = 0; i < NR; i++) acc[i] = F::dot(ring[s][i], a4, nch, c, acc[i]);
+                }
+                // operands arrive with the group's first item and are held until its last
+                if (it == 0) { sc = rSc[s]; bi = rBi[s]; re = rRe[s]; cs = rCs[s]; sn = rSn[s]; }
+                if (it == iters - 1) {
+                    // ---- group finished: reduce and write ----
 #pragma unroll
-        for (int i = 0; i < NR; i++) {
-            int r = valid[i] ? rowOf[i] : 0;          // clamp: loads stay in bounds, result dropped
-            rows[i] = F::row(p.seg[segOf[i]], r, p.K);
-        }
-
-        float acc[NR];
+                    for (int i = 0; i < NR; i++) acc[i] = wave_sum(acc[i]);
+                    bool finisher = true;
+                    if (KS == 4) {
+                        if (lane == 0) {
 #pragma unroll
-        for (int i = 0; i < NR; i++) acc[i] = 0.f;
-
-#pragma unroll 2
-        for (int c = c0; c < nch; c += cStep) {
-            typename F::Chunk ck[NR];
+                            for (int i = 0; i < NR; i++) part[wave][i] = acc[i];
+                        }
+                        __syncthreads();
+                        finisher = wave == 0;
+                        if (finisher) {
 #pragma unroll
-            for (int i = 0; i < NR; i++) ck[i] = F::load(rows[i], c);
-#pragma unroll
-            for (int i = 0; i < NR; i++) acc[i] = F::dot(ck[i], a4, nch, c, acc[i]);
-        }
-
-#pragma unroll
-        for (int i = 0; i < NR; i++) acc[i] = wave_sum(acc[i]);
-
-        bool finisher = true;
-        if (KS == 4) {
-            if (lane == 0) {
-#pragma unroll
-                for (int i = 0; i < NR; i++) part[wave][i] = acc[i];
-            }
-            __syncthreads();
-            finisher = wave == 0;
-            if (finisher) {
-#pragma unroll
-                for (int i = 0; i < NR; i++) acc[i] = (part[0][i] + part[1][i]) + (part[2][i] + part[3][i]);
-            }
-        }
-
-        if (finisher) {
-            // lane i finishes row i
-            float v = acc[0];
-            int seg = segOf[0], r = rowOf[0];
-            bool ok = valid[0];
-#pragma unroll
-            for (int i = 1; i < NR; i++) {
-                if (lane == i) { v = acc[i]; seg = segOf[i]; r = rowOf[i]; ok = valid[i]; }
-            }
-            if (epi == EPI_SWIGLU) {
-                constexpr int H = NR / 2 > 0 ? NR / 2 : 1;
-                float u = acc[H < NR ? H : 0];
-#pragma unroll
-                for (int i = 1; i < H; i++) if (lane == i) u = acc[(H + i) < NR ? (H + i) : 0];
-                if (lane < H && ok) {
-                    float gs = 1.0f, us = 1.0f;
-                    if (WF == WF_Q8) {
-                        gs = static_cast<const float*>(p.seg[0].aux)[r];
-                        us = static_cast<const float*>(p.seg[1].aux)[r];
+                            for (int i = 0; i < NR; i++) acc[i] = (part[0][i] + part[1][i]) + (part[2][i] + part[3][i]);
+                        }
                     }
-                    float gv = v * gs, uv = u * us;
-                    // mongoose.cu:949-956
-                    float sig = 1.0f / (1.0f + expf(-gv));
-                    p.seg[0].out[r] = gv * sig * uv;
-                }
-            } else if (lane < NR && ok) {
-                const MvSeg& sg = p.seg[seg];
-                if (WF == WF_Q8) {
-                    float sc = static_cast<const float*>(sg.aux)[r];
-                    if (p.div127) sc = sc / 127.0f;     // mongoose.cu:1561
-                    v *= sc;
-                }
-                if (sg.bias) v += sg.bias[r];
-                if (epi == EPI_RESID) v = p.resid[r] + v;
-                sg.out[r] = v;
-                if (epi == EPI_ARGMAX) {
-                    if (v > myBestV || (v == myBestV && r < myBestI)) { myBestV = v; myBestI = r; }
+                    if (finisher) {
+                        float v = acc[0];
+#pragma unroll
+                        for (int i = 1; i < NR; i++) if (lane == i) v = acc[i];
+                        if (WF == WF_Q8) {
+                            if (p.div127) sc = sc / 127.0f;      // mongoose.cu:1561
+                            v *= sc;
+                        }
+                        v += bi;
+                        RowRef rr = resolve_row<NR, EPI>(p, g, lane < NR ? lane : 0);
+                        if (EPI == EPI_SWIGLU) {
+                            constexpr int H = NR / 2 > 0 ? NR / 2 : 1;
+                            float u = __shfl(v, lane + H, 64);
+                            if (lane < H && rr.valid) {
+                                float sig = 1.0f / (1.0f + expf(-v));          // mongoose.cu:949-956
+                                p.seg[0].out[rr.row] = v * sig * u;
+                            }
+                        } else if (EPI == EPI_QKV) {
+                            float v1 = __shfl(v, 1, 64);
+                            if (lane == 0 && rr.valid) {
+                                const MvSeg& sg = p.seg[rr.seg];
+                                float* dst = rr.seg == 0 ? sg.out : sg.out + (size_t)pos * p.kvDim;
+                                if (rr.seg < 2) {                               // mongoose.cu:991-1006
+                                    int half = p.headDim >> 1;
+                                    dst[rr.row] = v * cs - v1 * sn;
+                                    dst[rr.row + half] = v * sn + v1 * cs;
+                                } else {                                        // mongoose.cu:1644-1647
+                                    dst[rr.row] = v;
+                                    if (rr.row + 1 < sg.rows) dst[rr.row + 1] = v1;
+                                }
+                            }
+                        } else if (lane < NR && rr.valid) {
+                            if (EPI == EPI_RESID) v = re + v;
+                            p.seg[rr.seg].out[rr.row] = v;
+                            if (EPI == EPI_ARGMAX) {
+                                if (v > myBestV || (v == myBestV && rr.row < myBestI)) { myBestV = v; myBestI = rr.row; }
+                            }
+                        }
+                    }
+                    if (KS == 4) __syncthreads();
+#pragma unroll
+                    for (int i = 0; i < NR; i++) acc[i] = 0.f;
                 }
             }
+            issue(s, item + D);
         }
-        if (KS == 4) __syncthreads();
     }
 
-    if (epi == EPI_ARGMAX) {
-        // lanes 0..NR-1 of each finishing wave hold candidates
+    if (EPI == EPI_ARGMAX) {
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
             float ov = __shfl_xor(myBestV, o, 64);
@@ -365,35 +457,56 @@ MvConfig pick_config(int wf, int epi, int totalRows, int K) {
     c.ks = 1;
     // Long rows and few of them: split K over the workgroup.
     if (nch > 128 && totalRows <= 8192) c.ks = 4;
-    if (epi == EPI_SWIGLU) {
-        // totalRows counts gate rows; each group carries a gate and an up row
+    if (epi == EPI_QKV) {
+        c.nr = 2;
+    } else if (epi == EPI_SWIGLU) {
+        // totalRows counts gate rows; each group carries gate and up rows
         c.nr = totalRows >= 8192 ? 4 : 2;
     } else if (c.ks == 4) {
         c.nr = totalRows >= 4096 ? 2 : 1;
     } else {
         c.nr = totalRows >= 16384 ? 4 : (totalRows >= 4096 ? 2 : 1);
     }
+    if (epi == EPI_RESID && c.nr > 2) c.nr = 2;
     c.grid = 0;   // filled by the launcher from the group count
     return c;
 }
 
-template <int WF, int NR, int KS>
-static hipError_t launch_t(MvParams& p, int pro, int epi, int grid, hipStream_t s) {
+template <int WF, int NR, int KS, int PRO, int EPI>
+static hipError_t launch_t(MvParams& p, int grid, hipStream_t s) {
     size_t lds = (size_t)p.K * sizeof(float);
-    hipLaunchKernelGGL((matvec_kernel<WF, NR, KS>), dim3(grid), dim3(WG), lds, s, p, pro, epi);
+    hipLaunchKernelGGL((matvec_kernel<WF, NR, KS, PRO, EPI>), dim3(grid), dim3(WG), lds, s, p);
     return hipGetLastError();
 }
 
-template <int WF>
-static hipError_t launch_wf(MvParams& p, int pro, int epi, const MvConfig& c, hipStream_t s) {
-    if (c.ks == 4) {
-        if (c.nr == 1) return launch_t<WF, 1, 4>(p, pro, epi, c.grid, s);
-        if (c.nr == 2) return launch_t<WF, 2, 4>(p, pro, epi, c.grid, s);
-        return launch_t<WF, 4, 4>(p, pro, epi, c.grid, s);
+#define MV_CASE(NRV, KSV)                                                           \
+    if (c.nr == NRV && c.ks == KSV) return launch_t<WF, NRV, KSV, PRO, EPI>(p, c.grid, s);
+
+template <int WF, int PRO, int EPI>
+static hipError_t launch_pe(MvParams& p, const MvConfig& c, hipStream_t s) {
+    if (EPI == EPI_QKV) {
+        MV_CASE(2, 1) MV_CASE(2, 4)
+    } else if (EPI == EPI_SWIGLU) {
+        MV_CASE(2, 1) MV_CASE(2, 4) MV_CASE(4, 1) MV_CASE(4, 4)
+    } else if (EPI == EPI_RESID) {
+        MV_CASE(1, 1) MV_CASE(1, 4) MV_CASE(2, 1) MV_CASE(2, 4)
+    } else {
+        MV_CASE(1, 1) MV_CASE(1, 4) MV_CASE(2, 1) MV_CASE(2, 4) MV_CASE(4, 1) MV_CASE(4, 4)
     }
-    if (c.nr == 1) return launch_t<WF, 1, 1>(p, pro, epi, c.grid, s);
-    if (c.nr == 2) return launch_t<WF, 2, 1>(p, pro, epi, c.grid, s);
-    return launch_t<WF, 4, 1>(p, pro, epi, c.grid, s);
+    return hipErrorInvalidValue;
+}
+#undef MV_CASE
+
+template <int WF>
+static hipError_t launch_wf(int pro, int epi, MvParams& p, const MvConfig& c, hipStream_t s) {
+    if (pro == PRO_PLAIN && epi == EPI_STORE) return launch_pe<WF, PRO_PLAIN, EPI_STORE>(p, c, s);
+    if (WF == WF_Q4RAW) return hipErrorInvalidValue;             // raw GGUF rows: per-op entry point only
+    if (pro == PRO_RMS && epi == EPI_QKV) return launch_pe<WF == WF_Q4RAW ? WF_Q4P : WF, PRO_RMS, EPI_QKV>(p, c, s);
+    if (pro == PRO_ATTN && epi == EPI_RESID) return launch_pe<WF == WF_Q4RAW ? WF_Q4P : WF, PRO_ATTN, EPI_RESID>(p, c, s);
+    if (pro == PRO_RMS && epi == EPI_SWIGLU) return launch_pe<WF == WF_Q4RAW ? WF_Q4P : WF, PRO_RMS, EPI_SWIGLU>(p, c, s);
+    if (pro == PRO_PLAIN && epi == EPI_RESID) return launch_pe<WF == WF_Q4RAW ? WF_Q4P : WF, PRO_PLAIN, EPI_RESID>(p, c, s);
+    if (pro == PRO_RMS && epi == EPI_ARGMAX) return launch_pe<WF == WF_Q4RAW ? WF_Q4P : WF, PRO_RMS, EPI_ARGMAX>(p, c, s);
+    return hipErrorInvalidValue;
 }
 
 hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInOut, hipStream_t s) {
@@ -409,6 +522,14 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
         int h = c.nr / 2;
         p.ngroups = (p.seg[0].rows + h - 1) / h;
         p.segGroup0[0] = 0; p.segGroup0[1] = p.ngroups; p.segGroup0[2] = p.ngroups;
+    } else if (epi == EPI_QKV) {
+        // q and k rows pair up inside a head, so both need whole heads; v rows pair up consecutively
+        if (p.nseg != 3 || p.headDim <= 0 || p.seg[0].rows % p.headDim || p.seg[1].rows % p.headDim || p.seg[2].rows % 2)
+            return hipErrorInvalidValue;
+        c.nr = 2;
+        int g = 0;
+        for (int i = 0; i < 3; i++) { p.segGroup0[i] = g; g += p.seg[i].rows / 2; }
+        p.ngroups = g;
     } else {
         int g = 0;
         for (int i = 0; i < 3; i++) {
@@ -422,9 +543,9 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
     int cap = 2048;
     if (c.grid <= 0 || c.grid > wgs) c.grid = wgs < cap ? wgs : cap;
     if (cfgInOut) *cfgInOut = c;
-    if (wf == WF_Q8) return launch_wf<WF_Q8>(p, pro, epi, c, s);
-    if (wf == WF_Q4P) return launch_wf<WF_Q4P>(p, pro, epi, c, s);
-    return launch_wf<WF_Q4RAW>(p, pro, epi, c, s);
+    if (wf == WF_Q8) return launch_wf<WF_Q8>(pro, epi, p, c, s);
+    if (wf == WF_Q4P) return launch_wf<WF_Q4P>(pro, epi, p, c, s);
+    return launch_wf<WF_Q4RAW>(pro, epi, p, c, s);
 }
 
 // Any K, any alignment: one wave per row, byte loads.  Only used by the
@@ -456,23 +577,25 @@ hipError_t launch_matvec_generic_q8(const float* act, const void* w, const float
 // ---------------------------------------------------------------------------
 // Decode attention (mongoose.cu:856-933), split over the KV range.
 // One workgroup = one KV head (all its GQA query heads, so K/V rows are read
-// once) x one split of the positions.  Online softmax over 256-position
-// tiles; scores: one lane per position; P.V: one lane per float4 of the head.
-// Fused form also applies RoPE (mongoose.cu:991-1006) to q and the new k and
-// stores the new k/v rows (mongoose.cu:1644-1647).
+// once) x one split of the positions.  q arrives rotated and the K/V rows of
+// the current position are already in the caches (the QKV matvec's epilogue
+// did both).  Online softmax over 256-position tiles; scores: one lane per
+// position with the whole K row in registers; P.V: one lane per float4 of the
+// head, V rows prefetched while the scores are being computed.
 // ---------------------------------------------------------------------------
 template <int HD, int GMAX>
 __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     constexpr int LPR = HD / 4;        // lanes per V row
     constexpr int TG = WG / LPR;       // position groups in the P.V phase
-    constexpr int HALF = HD / 2;
+    constexpr int VU = 4;              // V rows in flight per thread
+    constexpr int KQ = 16;             // K float4s held in registers at a time
     __shared__ float4 q_s4[GMAX * HD / 4];
     __shared__ float sc[GMAX][WG];
-    __shared__ float red[4];
+    __shared__ float wred[2][GMAX][4];
     __shared__ float4 accbuf[TG][GMAX][LPR];
-    float* q_s = reinterpret_cast<float*>(q_s4);
 
     const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
     const int G = p.nHeads / p.nKVHeads;
     const int nChunks = (G + GMAX - 1) / GMAX;
     const int kvh = blockIdx.x / nChunks;
@@ -480,6 +603,12 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     const int h0 = kvh * G + chunk * GMAX;
     const int gn = min(GMAX, G - chunk * GMAX);
     const int split = blockIdx.y;
+    const int kvOff = kvh * HD;
+    const int tg = tid / LPR, dl = tid % LPR;
+
+    // q does not depend on the position: issue it first
+    float4 qv = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (tid < gn * (HD / 4)) qv = reinterpret_cast<const float4*>(p.q + (size_t)h0 * HD)[tid];
 
     const int pos = p.state ? p.state->pos : p.posImm;
     const int len = pos + 1;
@@ -492,36 +621,8 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     if (split >= nsplit) return;
     const int t0 = split * splitLen;
     const int t1 = min(len, t0 + splitLen);
-    const int kvOff = kvh * HD;
 
-    // q (rotated when fused) -> LDS
-    for (int i = tid; i < gn * HALF; i += WG) {
-        int g = i / HALF, j = i % HALF;
-        float x0 = p.q[(h0 + g) * HD + j];
-        float x1 = p.q[(h0 + g) * HD + HALF + j];
-        if (p.fused) {
-            float c = p.cosTab[(size_t)pos * HALF + j], s = p.sinTab[(size_t)pos * HALF + j];
-            q_s[g * HD + j] = x0 * c - x1 * s;
-            q_s[g * HD + HALF + j] = x0 * s + x1 * c;
-        } else {
-            q_s[g * HD + j] = x0;
-            q_s[g * HD + HALF + j] = x1;
-        }
-    }
-    // new k/v row: the split that contains `pos` stores it, then reads it back
-    // like any other row (same workgroup: visible after the barrier).
-    if (p.fused && t1 == len) {
-        for (int j = tid; j < HALF; j += WG) {
-            float c = p.cosTab[(size_t)pos * HALF + j], s = p.sinTab[(size_t)pos * HALF + j];
-            float x0 = p.kNew[kvOff + j], x1 = p.kNew[kvOff + HALF + j];
-            p.Kc[(size_t)pos * p.kvDim + kvOff + j] = x0 * c - x1 * s;
-            p.Kc[(size_t)pos * p.kvDim + kvOff + HALF + j] = x0 * s + x1 * c;
-            p.Vc[(size_t)pos * p.kvDim + kvOff + j] = p.vNew[kvOff + j];
-            p.Vc[(size_t)pos * p.kvDim + kvOff + HALF + j] = p.vNew[kvOff + HALF + j];
-        }
-    }
-    __threadfence_block();
-    __syncthreads();
+    if (tid < gn * (HD / 4)) q_s4[tid] = qv;
 
     const float scale = 1.0f / sqrtf((float)HD);     // mongoose.cu:867 rsqrtf(headDim)
     float m[GMAX], l[GMAX];
@@ -529,62 +630,109 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
     for (int g = 0; g < GMAX; g++) { m[g] = -INFINITY; l[g] = 0.f; acc[g] = make_float4(0.f, 0.f, 0.f, 0.f); }
 
-    const int tg = tid / LPR, dl = tid % LPR;
+    const float4* Vbase = reinterpret_cast<const float4*>(p.Vc + kvOff) + dl;
+    const size_t vStride = (size_t)p.kvDim / 4;
 
     for (int tile = t0; tile < t1; tile += WG) {
         const int t = tile + tid;
         const bool active = t < t1;
+        const int tileLen = min(WG, t1 - tile);
+        // K row of this lane's position and the first V rows of this thread: all loads go out together
+        const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)(active ? t : tile) * p.kvDim + kvOff);
+        float4 kreg[KQ];
+#pragma unroll
+        for (int d4 = 0; d4 < KQ; d4++) kreg[d4] = krow[d4];
+        float4 vreg[VU];
+#pragma unroll
+        for (int u = 0; u < VU; u++) {
+            int tt = tg + u * TG;
+            vreg[u] = Vbase[(size_t)(tile + (tt < tileLen ? tt : 0)) * vStride];
+        }
+        if (tile == t0) __syncthreads();              // q_s4 staged
         float s[GMAX];
 #pragma unroll
         for (int g = 0; g < GMAX; g++) s[g] = 0.f;
-        if (active) {
-            const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)t * p.kvDim + kvOff);
-#pragma unroll 8
-            for (int d4 = 0; d4 < HD / 4; d4++) {
-                float4 kv = krow[d4];
+#pragma unroll
+        for (int part = 0; part < HD / 4; part += KQ) {
+            if (part > 0) {
+#pragma unroll
+                for (int d4 = 0; d4 < KQ; d4++) kreg[d4] = krow[part + d4];
+            }
+#pragma unroll
+            for (int d4 = 0; d4 < KQ; d4++) {
 #pragma unroll
                 for (int g = 0; g < GMAX; g++) {
                     if (g < gn) {
-                        float4 qv = q_s4[g * (HD / 4) + d4];
-                        s[g] = fmaf(qv.x, kv.x, s[g]);
-                        s[g] = fmaf(qv.y, kv.y, s[g]);
-                        s[g] = fmaf(qv.z, kv.z, s[g]);
-                        s[g] = fmaf(qv.w, kv.w, s[g]);
+                        float4 q4 = q_s4[g * (HD / 4) + part + d4];
+                        s[g] = fmaf(q4.x, kreg[d4].x, s[g]);
+                        s[g] = fmaf(q4.y, kreg[d4].y, s[g]);
+                        s[g] = fmaf(q4.z, kreg[d4].z, s[g]);
+                        s[g] = fmaf(q4.w, kreg[d4].w, s[g]);
                     }
                 }
             }
         }
+        // tile maxima of all heads with one barrier, then the sums with another
+        float sv[GMAX];
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
-            if (g < gn) {                                  // gn is uniform: barriers inside are safe
-                float sv = active ? s[g] * scale : -INFINITY;
-                float tmax = block_max(sv, red);
+            sv[g] = active ? s[g] * scale : -INFINITY;
+            if (g < gn) {
+                float wm = wave_max(sv[g]);
+                if (lane == 0) wred[0][g][wave] = wm;
+            }
+        }
+        __syncthreads();
+        float corr[GMAX];
+#pragma unroll
+        for (int g = 0; g < GMAX; g++) {
+            if (g < gn) {
+                float tmax = fmaxf(fmaxf(wred[0][g][0], wred[0][g][1]), fmaxf(wred[0][g][2], wred[0][g][3]));
                 float mNew = fmaxf(m[g], tmax);
-                float corr = expf(m[g] - mNew);            // first tile: exp(-inf) = 0
-                float pv = active ? expf(sv - mNew) : 0.f;
+                corr[g] = expf(m[g] - mNew);               // first tile: exp(-inf) = 0
+                float pv = active ? expf(sv[g] - mNew) : 0.f;
                 sc[g][tid] = pv;
-                float tsum = block_sum(pv, red);
-                l[g] = l[g] * corr + tsum;
-                acc[g].x *= corr; acc[g].y *= corr; acc[g].z *= corr; acc[g].w *= corr;
+                float ws = wave_sum(pv);
+                if (lane == 0) wred[1][g][wave] = ws;
                 m[g] = mNew;
             }
         }
         __syncthreads();
-        const int tileLen = min(WG, t1 - tile);
-        for (int tt = tg; tt < tileLen; tt += TG) {
-            float4 v = reinterpret_cast<const float4*>(p.Vc + (size_t)(tile + tt) * p.kvDim + kvOff)[dl];
 #pragma unroll
-            for (int g = 0; g < GMAX; g++) {
-                if (g < gn) {
-                    float w = sc[g][tt];
-                    acc[g].x = fmaf(w, v.x, acc[g].x);
-                    acc[g].y = fmaf(w, v.y, acc[g].y);
-                    acc[g].z = fmaf(w, v.z, acc[g].z);
-                    acc[g].w = fmaf(w, v.w, acc[g].w);
+        for (int g = 0; g < GMAX; g++) {
+            if (g < gn) {
+                float tsum = (wred[1][g][0] + wred[1][g][1]) + (wred[1][g][2] + wred[1][g][3]);
+                l[g] = l[g] * corr[g] + tsum;
+                acc[g].x *= corr[g]; acc[g].y *= corr[g]; acc[g].z *= corr[g]; acc[g].w *= corr[g];
+            }
+        }
+        // P.V
+        for (int k0 = 0; k0 * TG < tileLen; k0 += VU) {
+            if (k0 > 0) {
+#pragma unroll
+                for (int u = 0; u < VU; u++) {
+                    int tt = tg + (k0 + u) * TG;
+                    vreg[u] = Vbase[(size_t)(tile + (tt < tileLen ? tt : 0)) * vStride];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < VU; u++) {
+                int tt = tg + (k0 + u) * TG;
+                if (tt < tileLen) {
+#pragma unroll
+                    for (int g = 0; g < GMAX; g++) {
+                        if (g < gn) {
+                            float w = sc[g][tt];
+                            acc[g].x = fmaf(w, vreg[u].x, acc[g].x);
+                            acc[g].y = fmaf(w, vreg[u].y, acc[g].y);
+                            acc[g].z = fmaf(w, vreg[u].z, acc[g].z);
+                            acc[g].w = fmaf(w, vreg[u].w, acc[g].w);
+                        }
+                    }
                 }
             }
         }
-        __syncthreads();
+        __syncthreads();                               // sc and wred are reused by the next tile
     }
 
 #pragma unroll
@@ -593,6 +741,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     for (int i = tid; i < gn * LPR; i += WG) {
         int g = i / LPR, d4 = i % LPR;
         float4 r = accbuf[0][g][d4];
+#pragma unroll
         for (int k = 1; k < TG; k++) {
             float4 a = accbuf[k][g][d4];
             r.x += a.x; r.y += a.y; r.z += a.z; r.w += a.w;
@@ -884,6 +1033,21 @@ __global__ void advance_prompt_kernel(StepState* state, const int* prompt) {
 }
 hipError_t launch_advance_prompt(StepState* state, const int* prompt, hipStream_t s) {
     hipLaunchKernelGGL(advance_prompt_kernel, dim3(1), dim3(1), 0, s, state, prompt);
+    return hipGetLastError();
+}
+
+// Holds the stream until the host sets *flag (or the tick limit passes), so
+// that the host can queue a whole batch of launches ahead of the GPU.  One
+// lane; always exits.
+__global__ void gate_kernel(const volatile int* flag, long long limitTicks) {
+    const long long t0 = wall_clock64();
+    while (*flag == 0) {
+        if (wall_clock64() - t0 > limitTicks) break;
+        __builtin_amdgcn_s_sleep(32);
+    }
+}
+hipError_t launch_gate(const int* flag, long long limitTicks, hipStream_t s) {
+    hipLaunchKernelGGL(gate_kernel, dim3(1), dim3(1), 0, s, flag, limitTicks);
     return hipGetLastError();
 }
 
