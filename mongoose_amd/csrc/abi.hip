@@ -113,9 +113,10 @@ void mongoose_decode_attention(const float* Q, const float* K, const float* V, f
     mg::AttnParams p{};
     p.q = Q; p.Kc = K; p.Vc = V;
     p.posImm = cacheLen - 1;
+    p.rowLimit = cacheLen;
     p.kvDim = kvDim; p.nHeads = nHeads; p.nKVHeads = nKVHeads;
     p.headDim = dim / nHeads;                                    // mongoose.cu:939
-    p.direct = 1; p.out = out; p.smax = 1; p.minSplit = 1;
+    p.out = out; p.smax = 1; p.splitLen = 0;
     note(mg::launch_attention(p, S(stream)));
 }
 void mongoose_silu_gate_mul(const float* gate, const float* up, float* out, int n, void* stream) {

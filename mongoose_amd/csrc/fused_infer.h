@@ -102,7 +102,10 @@ private:
     float *cosTab = nullptr, *sinTab = nullptr;
     // split-KV attention partials
     float *pm = nullptr, *pl = nullptr, *pacc = nullptr;
-    int smax = 1, minSplit = 256;
+    int smax = 1, splitLen = 256, attnHeadsPerWG = 0;
+    int* attnCounters = nullptr;
+    float* ropeCur = nullptr;        // cos then sin row of the device-resident position
+    RopeCur ropeRef() const;
     // embedding table (optional)
     int embedKind = -1;       // -1: tied lm_head
     void* embedTable = nullptr;

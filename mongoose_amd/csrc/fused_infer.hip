@@ -97,13 +97,15 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
     if (hipMemcpy(f->cosTab, cosD.data(), cosD.size() * 4, hipMemcpyHostToDevice) != hipSuccess ||
         hipMemcpy(f->sinTab, sinD.data(), sinD.size() * 4, hipMemcpyHostToDevice) != hipSuccess) return fail("rope upload");
 
-    // split-KV partials: one tile of 256 positions per split at full context, at most 64 splits
-    f->minSplit = 256;
-    f->smax = (maxSeq + 255) / 256;
-    if (f->smax > 64) f->smax = 64;
-    if (f->smax < 1) f->smax = 1;
+    // split-KV geometry, fixed for the context: splits of a multiple of 256 positions, at most 32 of them
+    f->splitLen = 256 * ((maxSeq + 256 * 32 - 1) / (256 * 32));
+    f->smax = (maxSeq + f->splitLen - 1) / f->splitLen;
+    // short contexts: latency-bound, spread the GQA group over workgroups; long: read K/V once per group
+    f->attnHeadsPerWG = maxSeq <= 1024 ? 2 : 0;
     if (devAlloc(f->pm, (size_t)nHeads * f->smax, true) != 0 || devAlloc(f->pl, (size_t)nHeads * f->smax, true) != 0 ||
-        devAlloc(f->pacc, (size_t)nHeads * f->smax * headDim, true) != 0) return fail("attention partial alloc");
+        devAlloc(f->pacc, (size_t)nHeads * f->smax * headDim, true) != 0 ||
+        devAlloc(f->attnCounters, (size_t)attention_columns(nHeads, nKVHeads, 1), true) != 0 ||
+        devAlloc(f->ropeCur, (size_t)headDim, true) != 0) return fail("attention partial alloc");
 
     f->amaxParts = 2048;
     if (devAlloc(f->amaxVal, f->amaxParts, true) != 0 || devAlloc(f->amaxIdx, f->amaxParts, true) != 0 ||
@@ -112,7 +114,7 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
     void* hp = nullptr;
     if (hipHostMalloc(&hp, sizeof(StepState), hipHostMallocDefault) != hipSuccess) return fail("pinned alloc");
     f->hState = static_cast<StepState*>(hp);
-    if (hipHostMalloc(&hp, 64, hipHostMallocDefault) != hipSuccess) return fail("pinned alloc");
+    if (hipHostMalloc(&hp, 64, hipHostMallocCoherent | hipHostMallocMapped) != hipSuccess) return fail("pinned alloc");
     f->hGate = static_cast<int*>(hp);
     *f->hGate = 1;
     if (hipHostMalloc(&hp, sizeof(int) * ((size_t)maxSeq + 1), hipHostMallocDefault) != hipSuccess) return fail("pinned alloc");
@@ -142,6 +144,8 @@ HIPFusedInference::~HIPFusedInference() {
     for (float* p : {hidden[0], hidden[1], logits, finalNorm, normed, Q, K, V, attnOut, proj, normed2, gatePre, upOut,
                      ffnMid, cosTab, sinTab, pm, pl, pacc, amaxVal}) if (p) (void)hipFree(p);
     if (amaxIdx) (void)hipFree(amaxIdx);
+    if (attnCounters) (void)hipFree(attnCounters);
+    if (ropeCur) (void)hipFree(ropeCur);
     if (dState) (void)hipFree(dState);
     if (dHistory) (void)hipFree(dHistory);
     if (dPrompt) (void)hipFree(dPrompt);
@@ -344,6 +348,10 @@ int HIPFusedInference::mark(int cls) {
     return MG_OK;
 }
 
+RopeCur HIPFusedInference::ropeRef() const {
+    return RopeCur{cosTab, sinTab, ropeCur, headDim / 2, maxSeq};
+}
+
 static bool layerComplete(const LayerWeights& L) {
     return L.norm1 && L.norm2 && L.wq.w && L.wk.w && L.wv.w && L.wo.w && L.gate.w && L.up.w && L.down.w;
 }
@@ -373,9 +381,9 @@ int HIPFusedInference::enqueueLayerPerOp(const LayerWeights& L, int layer, int p
     HIPCHK(launch_kv_cache_write(kCache[layer], K, pos, kvDim, stream));
     HIPCHK(launch_kv_cache_write(vCache[layer], V, pos, kvDim, stream));
     AttnParams a{};
-    a.q = Q; a.Kc = kCache[layer]; a.Vc = vCache[layer]; a.posImm = pos;
+    a.q = Q; a.Kc = kCache[layer]; a.Vc = vCache[layer]; a.posImm = pos; a.rowLimit = maxSeq;
     a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
-    a.direct = 1; a.out = attnOut; a.smax = 1; a.minSplit = 1;
+    a.out = attnOut; a.smax = 1; a.splitLen = 0;
     HIPCHK(launch_attention(a, stream));
     HIPCHK(mv(L.wo, attnOut, proj));
     HIPCHK(launch_add_inplace(h, proj, dim, stream));
@@ -389,7 +397,7 @@ int HIPFusedInference::enqueueLayerPerOp(const LayerWeights& L, int layer, int p
 }
 
 // Five launches a layer: [norm1 + QKV + bias + RoPE + KV-cache write] [attention]
-// [combine + Wo + residual] [norm2 + gate/up + SiLU*mul] [down + residual].
+// [Wo + residual] [norm2 + gate/up + SiLU*mul] [down + residual].
 int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const StepState* st, int posImm) {
     float* h = hidden[hiddenIdx];
     if (mark(1)) return MG_E_HIP;
@@ -400,28 +408,29 @@ int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const
         p.seg[1] = MvSeg{L.wk.w, L.wk.scales, L.bk, kCache[layer], kvDim};
         p.seg[2] = MvSeg{L.wv.w, L.wv.scales, L.bv, vCache[layer], kvDim};
         p.nseg = 3;
-        p.headDim = headDim; p.kvDim = kvDim; p.cosTab = cosTab; p.sinTab = sinTab;
+        p.headDim = headDim; p.kvDim = kvDim;
         p.state = st; p.posImm = posImm;
+        const int half = headDim / 2;
+        p.cosRow = st ? ropeCur : cosTab + (size_t)posImm * half;
+        p.sinRow = st ? ropeCur + half : sinTab + (size_t)posImm * half;
         HIPCHK(launch_matvec(L.wq.kind, EPI_QKV, PRO_RMS, p, nullptr, stream));
     }
     if (mark(2)) return MG_E_HIP;
     {
         AttnParams a{};
         a.q = Q; a.Kc = kCache[layer]; a.Vc = vCache[layer];
-        a.state = st; a.posImm = posImm;
+        a.state = st; a.posImm = posImm; a.rowLimit = maxSeq;
         a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
-        a.direct = 0; a.smax = smax; a.minSplit = minSplit;
-        a.pm = pm; a.pl = pl; a.pacc = pacc;
+        a.smax = smax; a.splitLen = splitLen; a.headsPerWG = attnHeadsPerWG;
+        a.pm = pm; a.pl = pl; a.pacc = pacc; a.counters = attnCounters; a.out = attnOut;
         HIPCHK(launch_attention(a, stream));
     }
     if (mark(3)) return MG_E_HIP;
     {
         MvParams p{};
         p.seg[0] = MvSeg{L.wo.w, L.wo.scales, nullptr, h, dim};
-        p.nseg = 1; p.K = dim;
-        p.pm = pm; p.pl = pl; p.pacc = pacc; p.nHeads = nHeads; p.headDim = headDim; p.smax = smax; p.minSplit = minSplit;
-        p.state = st; p.posImm = posImm; p.resid = h;
-        HIPCHK(launch_matvec(L.wo.kind, EPI_RESID, PRO_ATTN, p, nullptr, stream));
+        p.nseg = 1; p.K = dim; p.act = attnOut; p.resid = h;
+        HIPCHK(launch_matvec(L.wo.kind, EPI_RESID, PRO_PLAIN, p, nullptr, stream));
     }
     if (mark(4)) return MG_E_HIP;
     {
@@ -467,7 +476,7 @@ int HIPFusedInference::enqueueFinal(bool withArgmax) {
     if (mark(7)) return MG_E_HIP;
     if (withArgmax) {
         if (c.grid > amaxParts) { set_error("argmax partial buffer too small"); return MG_E_STATE; }
-        HIPCHK(launch_argmax_finish(amaxVal, amaxIdx, c.grid, dState, nullptr, dHistory, maxSeq + 1, vocabSize, stream));
+        HIPCHK(launch_argmax_finish(amaxVal, amaxIdx, c.grid, dState, nullptr, dHistory, maxSeq + 1, vocabSize, ropeRef(), stream));
     }
     return MG_OK;
 }
@@ -561,7 +570,7 @@ int HIPFusedInference::enqueueToken(bool withHead) {
         if (rc) return rc;
     }
     if (withHead) return enqueueFinal(true);
-    HIPCHK(launch_advance_prompt(dState, dPrompt, stream));
+    HIPCHK(launch_advance_prompt(dState, dPrompt, ropeRef(), stream));
     return MG_OK;
 }
 
@@ -579,7 +588,7 @@ int HIPFusedInference::DecodeToken(int token, int pos, int* nextToken, float* lo
     ARGCHK(pos >= 0 && pos < maxSeq && token >= 0 && token < vocabSize, "DecodeToken: token or pos out of range");
     int rc = checkReady(this);
     if (rc) return rc;
-    HIPCHK(launch_set_state(dState, pos, token, 0, 0, stream));
+    HIPCHK(launch_set_state(dState, pos, token, 0, 0, ropeRef(), stream));
     if (execMode == 0) {
         rc = enqueueEmbed();
         if (rc) return rc;
@@ -625,7 +634,7 @@ int HIPFusedInference::GraphLaunch(int token, int pos, int* nextToken) {
     ARGCHK(pos >= 0 && pos < maxSeq && token >= 0 && token < vocabSize, "GraphLaunch: token or pos out of range");
     int rc = GraphCapture();
     if (rc) return rc;
-    HIPCHK(launch_set_state(dState, pos, token, 0, 0, stream));
+    HIPCHK(launch_set_state(dState, pos, token, 0, 0, ropeRef(), stream));
     HIPCHK(hipGraphLaunch(execFull, stream));
     HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int), hipMemcpyDeviceToHost, stream));
     HIPCHK(hipStreamSynchronize(stream));
@@ -674,7 +683,7 @@ int HIPFusedInference::Generate(const int* prompt, int nPrompt, int nDecode, int
     if (useGraph) { rc = GraphCapture(); if (rc) return rc; }
     HIPCHK(hipStreamSynchronize(stream));
     HIPCHK(hipMemcpy(dPrompt, prompt, sizeof(int) * (size_t)nPrompt, hipMemcpyHostToDevice));
-    HIPCHK(launch_set_state(dState, 0, prompt[0], 0, nPrompt, stream));
+    HIPCHK(launch_set_state(dState, 0, prompt[0], 0, nPrompt, ropeRef(), stream));
     for (int i = 0; i < nPrompt - 1; i++) {
         if (useGraph) HIPCHK(hipGraphLaunch(execPrompt, stream));
         else { rc = enqueueToken(false); if (rc) return rc; }
@@ -695,7 +704,7 @@ int HIPFusedInference::TimedDecode(int token, int pos, int steps, bool useGraph,
     int rc = checkReady(this);
     if (rc) return rc;
     if (useGraph) { rc = GraphCapture(); if (rc) return rc; }
-    HIPCHK(launch_set_state(dState, pos, token, 0, 0, stream));
+    HIPCHK(launch_set_state(dState, pos, token, 0, 0, ropeRef(), stream));
     HIPCHK(hipStreamSynchronize(stream));
     HIPCHK(hipEventRecord(ev0, stream));
     for (int i = 0; i < steps; i++) {
@@ -728,7 +737,7 @@ int HIPFusedInference::ProfileDecode(int token, int pos, int steps, float* class
     profEvents.clear(); profClass.clear();
     int* gate = hGate;
     *reinterpret_cast<volatile int*>(gate) = 0;
-    HIPCHK(launch_set_state(dState, pos, token, 0, 0, stream));
+    HIPCHK(launch_set_state(dState, pos, token, 0, 0, ropeRef(), stream));
     HIPCHK(launch_gate(gate, 100LL * 1000 * 500, stream));   // at most 0.5 s
     profiling = true;
     for (int i = 0; i < steps && rc == 0; i++) {

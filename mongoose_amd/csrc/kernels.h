@@ -17,7 +17,6 @@ enum WeightFormat {
 enum Prologue {
     PRO_PLAIN = 0,  // act[K] copied
     PRO_RMS = 1,    // act = rmsnorm(x, gain, eps)
-    PRO_ATTN = 2,   // act = combined split-KV attention partials
 };
 
 // What happens to each finished row.
@@ -56,17 +55,13 @@ struct MvParams {
     const float* act;     // PRO_PLAIN: activation; PRO_RMS: x
     const float* gain;
     float eps;
-    // PRO_ATTN: split-KV partials
-    const float* pm;      // [nHeads, smax]
-    const float* pl;      // [nHeads, smax]
-    const float* pacc;    // [nHeads, smax, headDim]
-    int nHeads, headDim, smax, minSplit;
-    const StepState* state;  // position source for PRO_ATTN / EPI_QKV (may be NULL -> posImm)
+    // EPI_QKV: cos/sin row of the current position [headDim/2] (no dependence on the
+    // position load); seg1.out / seg2.out are the K / V caches [maxSeq, kvDim], row `pos` is written
+    const StepState* state;  // position source (may be NULL -> posImm)
     int posImm;
-    // EPI_QKV: RoPE tables [maxSeq, headDim/2]; seg1.out / seg2.out are the K / V caches [maxSeq, kvDim]
-    const float* cosTab;
-    const float* sinTab;
-    int kvDim;
+    const float* cosRow;
+    const float* sinRow;
+    int headDim, kvDim;
     // epilogue
     const float* resid;
     int div127;           // Q8: multiply by scales[r]/127 instead of scales[r]
@@ -76,14 +71,6 @@ struct MvParams {
 
 struct MvConfig { int nr; int ks; int grid; };
 
-// Positions per split so that ceil(len/splitLen) <= smax; shared by the
-// attention kernel and the combining prologue.
-__host__ __device__ inline int attn_split_len(int len, int smax, int minSplit) {
-    int s = (len + smax - 1) / smax;
-    if (s < minSplit) s = minSplit;
-    return s;
-}
-
 MvConfig pick_config(int wf, int epi, int totalRows, int K);
 // Launch the matvec; returns hipSuccess or the launch error.  cfgInOut may be
 // NULL or have nr == 0 (pick automatically); the configuration used, with the
@@ -92,17 +79,21 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
 
 struct AttnParams {
     const float* q;       // [dim], rotated
-    const float* Kc;      // [maxSeq, kvDim], row pos already written
+    const float* Kc;      // [rowLimit, kvDim], row pos already written
     const float* Vc;
     const StepState* state;   // position source (NULL -> posImm)
     int posImm;
+    int rowLimit;         // rows that may be touched (maxSeq, or cacheLen for the per-op call)
     int kvDim, nHeads, nKVHeads, headDim;
-    int smax, minSplit;
-    float* pm; float* pl; float* pacc;   // partial outputs (direct == 0)
-    float* out;           // direct == 1: final [dim] output, single split
-    int direct;
+    int splitLen;         // positions per split, fixed for the context (multiple of 256); 0 = one split
+    int smax;             // number of splits launched
+    float* pm; float* pl; float* pacc;   // partials [nHeads, smax(, headDim)] when smax > 1
+    int* counters;        // one per workgroup column, zero between launches (smax > 1)
+    int headsPerWG;       // query heads of a GQA group per workgroup (0 = the whole group, up to 8)
+    float* out;           // [dim]
 };
 hipError_t launch_attention(const AttnParams& p, hipStream_t s);
+int attention_columns(int nHeads, int nKVHeads, int headsPerWG);
 
 hipError_t launch_rmsnorm_out(const float* in, float* out, const float* w, int seqLen, int dim, float eps, hipStream_t s);
 hipError_t launch_rope(float* x, const float* cosTab, const float* sinTab, int seqLen, int dim, int headDim, int nHeads, hipStream_t s);
@@ -122,11 +113,15 @@ hipError_t launch_embed_token(int kind, const void* table, const float* scales, 
                               float* x, int dim, int vocab, hipStream_t s);
 // Reduce the lm_head partials to a token, append it to the history and
 // advance the step state (next token comes from the prompt while pos+1 < nPrompt).
+// Every kernel that sets the position also copies that position's cos/sin row
+// into rope.cur (cos then sin, headDim/2 each), so that the next token's
+// kernels read it without first waiting for the position.
+struct RopeCur { const float* cosTab; const float* sinTab; float* cur; int half; int maxSeq; };
 hipError_t launch_argmax_finish(const float* pv, const int* pi, int nparts, StepState* state,
-                                const int* prompt, int* history, int historyCap, int vocab, hipStream_t s);
-hipError_t launch_set_state(StepState* state, int pos, int token, int count, int nPrompt, hipStream_t s);
+                                const int* prompt, int* history, int historyCap, int vocab, RopeCur rope, hipStream_t s);
+hipError_t launch_set_state(StepState* state, int pos, int token, int count, int nPrompt, RopeCur rope, hipStream_t s);
 // Advance state without an lm_head (prompt positions): pos++, token = prompt[pos].
-hipError_t launch_advance_prompt(StepState* state, const int* prompt, hipStream_t s);
+hipError_t launch_advance_prompt(StepState* state, const int* prompt, RopeCur rope, hipStream_t s);
 
 // Stream gate for timing runs: waits for *flag != 0 (host-pinned) or limitTicks of the 100 MHz wall clock.
 hipError_t launch_gate(const int* flag, long long limitTicks, hipStream_t s);

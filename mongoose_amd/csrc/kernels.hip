@@ -19,14 +19,28 @@ constexpr int WG = 256;
 // ---------------------------------------------------------------------------
 // wave64 / workgroup reductions
 // ---------------------------------------------------------------------------
+// Lane exchange inside a row of 16 lanes through DPP (no LDS traffic):
+// quad_perm [1,0,3,2] = 0xB1, quad_perm [2,3,0,1] = 0x4E, row_ror:4 = 0x124, row_ror:8 = 0x128.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    v += dpp_f<0xB1>(v);
+    v += dpp_f<0x4E>(v);
+    v += dpp_f<0x124>(v);
+    v += dpp_f<0x128>(v);
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
     return v;
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    v = fmaxf(v, dpp_f<0xB1>(v));
+    v = fmaxf(v, dpp_f<0x4E>(v));
+    v = fmaxf(v, dpp_f<0x124>(v));
+    v = fmaxf(v, dpp_f<0x128>(v));
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
     return v;
 }
 // Sum over the 256 threads of a workgroup; every thread gets the result.
@@ -108,37 +122,6 @@ __device__ __forceinline__ void stage_activation(const MvParams& p, float4* a4, 
         for (int i = tid + XR * WG; i < K4; i += WG) {
             float4 v = x4[i], g = g4[i], o;
             o.x = v.x * rs * g.x; o.y = v.y * rs * g.y; o.z = v.z * rs * g.z; o.w = v.w * rs * g.w;
-            a4[act_slot4<CH>(i, nch)] = o;
-        }
-    } else {
-        // Combine split-KV attention partials: out = sum_s e^(m_s-M) acc_s / sum_s e^(m_s-M) l_s
-        int pos = p.state ? p.state->pos : p.posImm;
-        int len = pos + 1;
-        int splitLen = attn_split_len(len, p.smax, p.minSplit);
-        int nsplit = (len + splitLen - 1) / splitLen;
-        const int hd4 = p.headDim >> 2;
-        for (int i = tid; i < K4; i += WG) {
-            int h = i / hd4, d4 = i % hd4;
-            const float* pm = p.pm + (size_t)h * p.smax;
-            const float* pl = p.pl + (size_t)h * p.smax;
-            float4 o;
-            if (nsplit == 1) {
-                float den = pl[0];
-                float4 a = reinterpret_cast<const float4*>(p.pacc + (size_t)h * p.smax * p.headDim)[d4];
-                o.x = a.x / den; o.y = a.y / den; o.z = a.z / den; o.w = a.w / den;
-            } else {
-                float M = pm[0];
-                for (int s = 1; s < nsplit; s++) M = fmaxf(M, pm[s]);
-                float den = 0.f;
-                float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
-                for (int s = 0; s < nsplit; s++) {
-                    float w = expf(pm[s] - M);
-                    den += w * pl[s];
-                    float4 a = reinterpret_cast<const float4*>(p.pacc + ((size_t)h * p.smax + s) * p.headDim)[d4];
-                    num.x += w * a.x; num.y += w * a.y; num.z += w * a.z; num.w += w * a.w;
-                }
-                o.x = num.x / den; o.y = num.y / den; o.z = num.z / den; o.w = num.w / den;
-            }
             a4[act_slot4<CH>(i, nch)] = o;
         }
     }
@@ -330,8 +313,8 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
                     if (EPI == EPI_QKV && rr.seg < 2 && lane == 0) {
                         int half = p.headDim >> 1;
                         int j = (g - p.segGroup0[rr.seg]) % half;
-                        rCs[slot] = p.cosTab[(size_t)pos * half + j];
-                        rSn[slot] = p.sinTab[(size_t)pos * half + j];
+                        rCs[slot] = p.cosRow[j];
+                        rSn[slot] = p.sinRow[j];
                     }
                 }
             }
@@ -502,7 +485,6 @@ static hipError_t launch_wf(int pro, int epi, MvParams& p, const MvConfig& c, hi
     if (pro == PRO_PLAIN && epi == EPI_STORE) return launch_pe<WF, PRO_PLAIN, EPI_STORE>(p, c, s);
     if (WF == WF_Q4RAW) return hipErrorInvalidValue;             // raw GGUF rows: per-op entry point only
     if (pro == PRO_RMS && epi == EPI_QKV) return launch_pe<WF == WF_Q4RAW ? WF_Q4P : WF, PRO_RMS, EPI_QKV>(p, c, s);
-    if (pro == PRO_ATTN && epi == EPI_RESID) return launch_pe<WF == WF_Q4RAW ? WF_Q4P : WF, PRO_ATTN, EPI_RESID>(p, c, s);
     if (pro == PRO_RMS && epi == EPI_SWIGLU) return launch_pe<WF == WF_Q4RAW ? WF_Q4P : WF, PRO_RMS, EPI_SWIGLU>(p, c, s);
     if (pro == PRO_PLAIN && epi == EPI_RESID) return launch_pe<WF == WF_Q4RAW ? WF_Q4P : WF, PRO_PLAIN, EPI_RESID>(p, c, s);
     if (pro == PRO_RMS && epi == EPI_ARGMAX) return launch_pe<WF == WF_Q4RAW ? WF_Q4P : WF, PRO_RMS, EPI_ARGMAX>(p, c, s);
@@ -579,20 +561,32 @@ hipError_t launch_matvec_generic_q8(const float* act, const void* w, const float
 // One workgroup = one KV head (all its GQA query heads, so K/V rows are read
 // once) x one split of the positions.  q arrives rotated and the K/V rows of
 // the current position are already in the caches (the QKV matvec's epilogue
-// did both).  Online softmax over 256-position tiles; scores: one lane per
-// position with the whole K row in registers; P.V: one lane per float4 of the
-// head, V rows prefetched while the scores are being computed.
+// did both).  The split geometry is fixed per context, so the first tile's
+// K/V rows are requested before the position is known (rows past the end are
+// clamped and masked): the kernel's critical path is one memory latency.
+// Online softmax over 256-position tiles; scores: one lane per position with
+// the K row in registers; P.V: one lane per float4 of the head.
+// With several splits the last workgroup of a column to finish combines the
+// partials, so the output is always the final [dim] vector.
 // ---------------------------------------------------------------------------
+__device__ __forceinline__ float ld_agent(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <int HD, int GMAX>
 __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     constexpr int LPR = HD / 4;        // lanes per V row
     constexpr int TG = WG / LPR;       // position groups in the P.V phase
-    constexpr int VU = 4;              // V rows in flight per thread
+    constexpr int VU = HD == 64 ? 16 : 8;   // V rows in flight per thread (HD 64: a whole tile)
     constexpr int KQ = 16;             // K float4s held in registers at a time
     __shared__ float4 q_s4[GMAX * HD / 4];
     __shared__ float sc[GMAX][WG];
     __shared__ float wred[2][GMAX][4];
     __shared__ float4 accbuf[TG][GMAX][LPR];
+    __shared__ int lastFlag;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -605,50 +599,52 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     const int split = blockIdx.y;
     const int kvOff = kvh * HD;
     const int tg = tid / LPR, dl = tid % LPR;
+    const int t0 = p.splitLen > 0 ? split * p.splitLen : 0;
+    const int lastRow = p.rowLimit - 1;
+    const size_t vStride = (size_t)p.kvDim / 4;
+    const float4* Vbase = reinterpret_cast<const float4*>(p.Vc + kvOff) + dl;
 
-    // q does not depend on the position: issue it first
-    float4 qv = make_float4(0.f, 0.f, 0.f, 0.f);
+    // ---- everything that does not need the position goes out first ----
+    float4 qv = make_float4(0.f, 0.f, 0.f, 0.f);                    // heads past gn stay zero
     if (tid < gn * (HD / 4)) qv = reinterpret_cast<const float4*>(p.q + (size_t)h0 * HD)[tid];
+    float4 kreg[KQ];
+    {
+        const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)min(t0 + tid, lastRow) * p.kvDim + kvOff);
+#pragma unroll
+        for (int d4 = 0; d4 < KQ; d4++) kreg[d4] = krow[d4];
+    }
+    float4 vreg[VU];
+#pragma unroll
+    for (int u = 0; u < VU; u++) vreg[u] = Vbase[(size_t)min(t0 + tg + u * TG, lastRow) * vStride];
 
     const int pos = p.state ? p.state->pos : p.posImm;
     const int len = pos + 1;
-    int splitLen, nsplit;
-    if (p.direct) { splitLen = len; nsplit = 1; }
-    else {
-        splitLen = attn_split_len(len, p.smax, p.minSplit);
-        nsplit = (len + splitLen - 1) / splitLen;
-    }
-    if (split >= nsplit) return;
-    const int t0 = split * splitLen;
-    const int t1 = min(len, t0 + splitLen);
+    if (t0 >= len) return;                                 // this split holds no position yet
+    const int nsplit = p.splitLen > 0 ? (len + p.splitLen - 1) / p.splitLen : 1;
+    const int t1 = p.splitLen > 0 ? min(len, t0 + p.splitLen) : len;
 
-    if (tid < gn * (HD / 4)) q_s4[tid] = qv;
+    if (tid < GMAX * (HD / 4)) q_s4[tid] = qv;
+    __syncthreads();
 
+    // Every loop below runs over all GMAX heads without a guard (straight-line code the
+    // scheduler can interleave); heads past gn work on zeros and are dropped at the end.
     const float scale = 1.0f / sqrtf((float)HD);     // mongoose.cu:867 rsqrtf(headDim)
     float m[GMAX], l[GMAX];
     float4 acc[GMAX];
 #pragma unroll
     for (int g = 0; g < GMAX; g++) { m[g] = -INFINITY; l[g] = 0.f; acc[g] = make_float4(0.f, 0.f, 0.f, 0.f); }
 
-    const float4* Vbase = reinterpret_cast<const float4*>(p.Vc + kvOff) + dl;
-    const size_t vStride = (size_t)p.kvDim / 4;
-
     for (int tile = t0; tile < t1; tile += WG) {
         const int t = tile + tid;
         const bool active = t < t1;
         const int tileLen = min(WG, t1 - tile);
-        // K row of this lane's position and the first V rows of this thread: all loads go out together
-        const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)(active ? t : tile) * p.kvDim + kvOff);
-        float4 kreg[KQ];
+        const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)min(t, lastRow) * p.kvDim + kvOff);
+        if (tile != t0) {
 #pragma unroll
-        for (int d4 = 0; d4 < KQ; d4++) kreg[d4] = krow[d4];
-        float4 vreg[VU];
+            for (int d4 = 0; d4 < KQ; d4++) kreg[d4] = krow[d4];
 #pragma unroll
-        for (int u = 0; u < VU; u++) {
-            int tt = tg + u * TG;
-            vreg[u] = Vbase[(size_t)(tile + (tt < tileLen ? tt : 0)) * vStride];
+            for (int u = 0; u < VU; u++) vreg[u] = Vbase[(size_t)min(tile + tg + u * TG, lastRow) * vStride];
         }
-        if (tile == t0) __syncthreads();              // q_s4 staged
         float s[GMAX];
 #pragma unroll
         for (int g = 0; g < GMAX; g++) s[g] = 0.f;
@@ -662,13 +658,11 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
             for (int d4 = 0; d4 < KQ; d4++) {
 #pragma unroll
                 for (int g = 0; g < GMAX; g++) {
-                    if (g < gn) {
-                        float4 q4 = q_s4[g * (HD / 4) + part + d4];
-                        s[g] = fmaf(q4.x, kreg[d4].x, s[g]);
-                        s[g] = fmaf(q4.y, kreg[d4].y, s[g]);
-                        s[g] = fmaf(q4.z, kreg[d4].z, s[g]);
-                        s[g] = fmaf(q4.w, kreg[d4].w, s[g]);
-                    }
+                    float4 q4 = q_s4[g * (HD / 4) + part + d4];
+                    s[g] = fmaf(q4.x, kreg[d4].x, s[g]);
+                    s[g] = fmaf(q4.y, kreg[d4].y, s[g]);
+                    s[g] = fmaf(q4.z, kreg[d4].z, s[g]);
+                    s[g] = fmaf(q4.w, kreg[d4].w, s[g]);
                 }
             }
         }
@@ -677,43 +671,34 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
             sv[g] = active ? s[g] * scale : -INFINITY;
-            if (g < gn) {
-                float wm = wave_max(sv[g]);
-                if (lane == 0) wred[0][g][wave] = wm;
-            }
+            float wm = wave_max(sv[g]);
+            if (lane == 0) wred[0][g][wave] = wm;
         }
         __syncthreads();
         float corr[GMAX];
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
-            if (g < gn) {
-                float tmax = fmaxf(fmaxf(wred[0][g][0], wred[0][g][1]), fmaxf(wred[0][g][2], wred[0][g][3]));
-                float mNew = fmaxf(m[g], tmax);
-                corr[g] = expf(m[g] - mNew);               // first tile: exp(-inf) = 0
-                float pv = active ? expf(sv[g] - mNew) : 0.f;
-                sc[g][tid] = pv;
-                float ws = wave_sum(pv);
-                if (lane == 0) wred[1][g][wave] = ws;
-                m[g] = mNew;
-            }
+            float tmax = fmaxf(fmaxf(wred[0][g][0], wred[0][g][1]), fmaxf(wred[0][g][2], wred[0][g][3]));
+            float mNew = fmaxf(m[g], tmax);
+            corr[g] = expf(m[g] - mNew);                   // first tile: exp(-inf) = 0
+            float pv = active ? expf(sv[g] - mNew) : 0.f;
+            sc[g][tid] = pv;
+            float ws = wave_sum(pv);
+            if (lane == 0) wred[1][g][wave] = ws;
+            m[g] = mNew;
         }
         __syncthreads();
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
-            if (g < gn) {
-                float tsum = (wred[1][g][0] + wred[1][g][1]) + (wred[1][g][2] + wred[1][g][3]);
-                l[g] = l[g] * corr[g] + tsum;
-                acc[g].x *= corr[g]; acc[g].y *= corr[g]; acc[g].z *= corr[g]; acc[g].w *= corr[g];
-            }
+            float tsum = (wred[1][g][0] + wred[1][g][1]) + (wred[1][g][2] + wred[1][g][3]);
+            l[g] = l[g] * corr[g] + tsum;
+            acc[g].x *= corr[g]; acc[g].y *= corr[g]; acc[g].z *= corr[g]; acc[g].w *= corr[g];
         }
         // P.V
         for (int k0 = 0; k0 * TG < tileLen; k0 += VU) {
             if (k0 > 0) {
 #pragma unroll
-                for (int u = 0; u < VU; u++) {
-                    int tt = tg + (k0 + u) * TG;
-                    vreg[u] = Vbase[(size_t)(tile + (tt < tileLen ? tt : 0)) * vStride];
-                }
+                for (int u = 0; u < VU; u++) vreg[u] = Vbase[(size_t)min(tile + tg + (k0 + u) * TG, lastRow) * vStride];
             }
 #pragma unroll
             for (int u = 0; u < VU; u++) {
@@ -721,13 +706,11 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
                 if (tt < tileLen) {
 #pragma unroll
                     for (int g = 0; g < GMAX; g++) {
-                        if (g < gn) {
-                            float w = sc[g][tt];
-                            acc[g].x = fmaf(w, vreg[u].x, acc[g].x);
-                            acc[g].y = fmaf(w, vreg[u].y, acc[g].y);
-                            acc[g].z = fmaf(w, vreg[u].z, acc[g].z);
-                            acc[g].w = fmaf(w, vreg[u].w, acc[g].w);
-                        }
+                        float w = sc[g][tt];
+                        acc[g].x = fmaf(w, vreg[u].x, acc[g].x);
+                        acc[g].y = fmaf(w, vreg[u].y, acc[g].y);
+                        acc[g].z = fmaf(w, vreg[u].z, acc[g].z);
+                        acc[g].w = fmaf(w, vreg[u].w, acc[g].w);
                     }
                 }
             }
@@ -736,7 +719,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     }
 
 #pragma unroll
-    for (int g = 0; g < GMAX; g++) if (g < gn) accbuf[tg][g][dl] = acc[g];
+    for (int g = 0; g < GMAX; g++) accbuf[tg][g][dl] = acc[g];
     __syncthreads();
     for (int i = tid; i < gn * LPR; i += WG) {
         int g = i / LPR, d4 = i % LPR;
@@ -751,26 +734,64 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
         for (int k = 1; k < GMAX; k++) if (g == k) { lg = l[k]; mg_ = m[k]; }
         int h = h0 + g;
-        if (p.direct) {
+        if (nsplit == 1) {
             float4 o;
             o.x = r.x / lg; o.y = r.y / lg; o.z = r.z / lg; o.w = r.w / lg;
             reinterpret_cast<float4*>(p.out + (size_t)h * HD)[d4] = o;
         } else {
-            reinterpret_cast<float4*>(p.pacc + ((size_t)h * p.smax + split) * HD)[d4] = r;
+            float* pa = p.pacc + ((size_t)h * p.smax + split) * HD + d4 * 4;
+            st_agent(pa, r.x); st_agent(pa + 1, r.y); st_agent(pa + 2, r.z); st_agent(pa + 3, r.w);
             if (d4 == 0) {
-                p.pm[(size_t)h * p.smax + split] = mg_;
-                p.pl[(size_t)h * p.smax + split] = lg;
+                st_agent(p.pm + (size_t)h * p.smax + split, mg_);
+                st_agent(p.pl + (size_t)h * p.smax + split, lg);
             }
         }
     }
+    if (nsplit == 1) return;
+
+    // ---- several splits: the last workgroup of this column combines ----
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        int old = __hip_atomic_fetch_add(p.counters + blockIdx.x, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        lastFlag = (old == nsplit - 1);
+    }
+    __syncthreads();
+    if (!lastFlag) return;
+    __threadfence();
+    for (int i = tid; i < gn * HD; i += WG) {
+        int g = i / HD, d = i % HD;
+        int h = h0 + g;
+        const float* pm = p.pm + (size_t)h * p.smax;
+        const float* pl = p.pl + (size_t)h * p.smax;
+        float M = ld_agent(pm);
+        for (int s = 1; s < nsplit; s++) M = fmaxf(M, ld_agent(pm + s));
+        float den = 0.f, num = 0.f;
+        for (int s = 0; s < nsplit; s++) {
+            float w = expf(ld_agent(pm + s) - M);
+            den += w * ld_agent(pl + s);
+            num += w * ld_agent(p.pacc + ((size_t)h * p.smax + s) * HD + d);
+        }
+        p.out[(size_t)h * HD + d] = num / den;
+    }
+    if (tid == 0) __hip_atomic_store(p.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Query heads handled per workgroup.  Long contexts: the whole GQA group (K/V
+// rows are fetched from HBM once).  Short contexts are latency-bound and the
+// K/V rows of a layer sit in L2, so the group is spread over more workgroups.
+static int attention_gmax(int G, int heads) {
+    int want = heads > 0 ? heads : G;
+    if (want > G) want = G;
+    return want >= 8 ? 8 : (want > 2 ? (want > 4 ? 8 : 4) : (want == 2 ? 2 : 1));
 }
 
 template <int HD>
-static hipError_t launch_attn_hd(const AttnParams& p, int maxSplits, hipStream_t s) {
+static hipError_t launch_attn_hd(const AttnParams& p, hipStream_t s) {
     int G = p.nHeads / p.nKVHeads;
-    int gmax = G >= 8 ? 8 : (G > 2 ? (G > 4 ? 8 : 4) : (G == 2 ? 2 : 1));
+    int gmax = attention_gmax(G, p.headsPerWG);
     int nChunks = (G + gmax - 1) / gmax;
-    dim3 grid(p.nKVHeads * nChunks, maxSplits);
+    dim3 grid(p.nKVHeads * nChunks, p.smax);
     switch (gmax) {
     case 1: hipLaunchKernelGGL((attn_decode_kernel<HD, 1>), grid, dim3(WG), 0, s, p); break;
     case 2: hipLaunchKernelGGL((attn_decode_kernel<HD, 2>), grid, dim3(WG), 0, s, p); break;
@@ -780,11 +801,18 @@ static hipError_t launch_attn_hd(const AttnParams& p, int maxSplits, hipStream_t
     return hipGetLastError();
 }
 
+// Columns of workgroups an attention launch uses (size of the counter array).
+int attention_columns(int nHeads, int nKVHeads, int headsPerWG) {
+    int G = nHeads / nKVHeads;
+    int gmax = attention_gmax(G, headsPerWG);
+    return nKVHeads * ((G + gmax - 1) / gmax);
+}
+
 hipError_t launch_attention(const AttnParams& p, hipStream_t s) {
-    if (p.nKVHeads <= 0 || p.nHeads % p.nKVHeads != 0) return hipErrorInvalidValue;
-    int splits = p.direct ? 1 : p.smax;
-    if (p.headDim == 64) return launch_attn_hd<64>(p, splits, s);
-    if (p.headDim == 128) return launch_attn_hd<128>(p, splits, s);
+    if (p.nKVHeads <= 0 || p.nHeads % p.nKVHeads != 0 || p.rowLimit <= 0 || p.smax < 1) return hipErrorInvalidValue;
+    if (p.smax > 1 && (p.splitLen <= 0 || p.splitLen % WG != 0 || !p.counters || !p.pm || !p.pl || !p.pacc)) return hipErrorInvalidValue;
+    if (p.headDim == 64) return launch_attn_hd<64>(p, s);
+    if (p.headDim == 128) return launch_attn_hd<128>(p, s);
     return hipErrorInvalidValue;
 }
 
@@ -980,10 +1008,23 @@ hipError_t launch_embed_token(int kind, const void* table, const float* scales, 
     return hipGetLastError();
 }
 
+// cos/sin row of position `pos` -> rope.cur (cos then sin), by the whole workgroup
+__device__ __forceinline__ void copy_rope_row(const RopeCur& rope, int pos) {
+    if (!rope.cur) return;
+    if (pos >= rope.maxSeq) pos = rope.maxSeq - 1;
+    for (int j = threadIdx.x; j < rope.half; j += blockDim.x) {
+        rope.cur[j] = rope.cosTab[(size_t)pos * rope.half + j];
+        rope.cur[rope.half + j] = rope.sinTab[(size_t)pos * rope.half + j];
+    }
+}
+
 __global__ __launch_bounds__(WG) void argmax_finish_kernel(const float* pv, const int* pi, int nparts, StepState* state,
-                                                           const int* prompt, int* history, int historyCap, int vocab) {
+                                                           const int* prompt, int* history, int historyCap, int vocab,
+                                                           RopeCur rope) {
     __shared__ float bv[WG];
     __shared__ int bi[WG];
+    const int np = state->pos + 1;
+    copy_rope_row(rope, np);
     float v = -INFINITY;
     int idx = INT_MAX;
     for (int i = threadIdx.x; i < nparts; i += WG) {
@@ -1002,7 +1043,6 @@ __global__ __launch_bounds__(WG) void argmax_finish_kernel(const float* pv, cons
     if (threadIdx.x == 0) {
         int tok = bi[0];
         if (tok < 0 || tok >= vocab) tok = 0;
-        int np = state->pos + 1;
         int next = tok;
         if (prompt && np < state->nPrompt) next = prompt[np];
         int cnt = state->count;
@@ -1013,26 +1053,30 @@ __global__ __launch_bounds__(WG) void argmax_finish_kernel(const float* pv, cons
     }
 }
 hipError_t launch_argmax_finish(const float* pv, const int* pi, int nparts, StepState* state, const int* prompt,
-                                int* history, int historyCap, int vocab, hipStream_t s) {
-    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(WG), 0, s, pv, pi, nparts, state, prompt, history, historyCap, vocab);
+                                int* history, int historyCap, int vocab, RopeCur rope, hipStream_t s) {
+    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(WG), 0, s, pv, pi, nparts, state, prompt, history, historyCap, vocab, rope);
     return hipGetLastError();
 }
 
-__global__ void set_state_kernel(StepState* state, int pos, int token, int count, int nPrompt) {
-    state->pos = pos; state->token = token; state->count = count; state->nPrompt = nPrompt;
+__global__ void set_state_kernel(StepState* state, int pos, int token, int count, int nPrompt, RopeCur rope) {
+    copy_rope_row(rope, pos);
+    if (threadIdx.x == 0) { state->pos = pos; state->token = token; state->count = count; state->nPrompt = nPrompt; }
 }
-hipError_t launch_set_state(StepState* state, int pos, int token, int count, int nPrompt, hipStream_t s) {
-    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, s, state, pos, token, count, nPrompt);
+hipError_t launch_set_state(StepState* state, int pos, int token, int count, int nPrompt, RopeCur rope, hipStream_t s) {
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, s, state, pos, token, count, nPrompt, rope);
     return hipGetLastError();
 }
 
-__global__ void advance_prompt_kernel(StepState* state, const int* prompt) {
+__global__ void advance_prompt_kernel(StepState* state, const int* prompt, RopeCur rope) {
     int np = state->pos + 1;
-    state->pos = np;
-    if (np < state->nPrompt) state->token = prompt[np];
+    copy_rope_row(rope, np);
+    if (threadIdx.x == 0) {
+        state->pos = np;
+        if (np < state->nPrompt) state->token = prompt[np];
+    }
 }
-hipError_t launch_advance_prompt(StepState* state, const int* prompt, hipStream_t s) {
-    hipLaunchKernelGGL(advance_prompt_kernel, dim3(1), dim3(1), 0, s, state, prompt);
+hipError_t launch_advance_prompt(StepState* state, const int* prompt, RopeCur rope, hipStream_t s) {
+    hipLaunchKernelGGL(advance_prompt_kernel, dim3(1), dim3(64), 0, s, state, prompt, rope);
     return hipGetLastError();
 }
 
@@ -1041,7 +1085,7 @@ hipError_t launch_advance_prompt(StepState* state, const int* prompt, hipStream_
 // lane; always exits.
 __global__ void gate_kernel(const volatile int* flag, long long limitTicks) {
     const long long t0 = wall_clock64();
-    while (*flag == 0) {
+    while (__hip_atomic_load(const_cast<const int*>(flag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == 0) {
         if (wall_clock64() - t0 > limitTicks) break;
         __builtin_amdgcn_s_sleep(32);
     }
