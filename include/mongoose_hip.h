@@ -206,6 +206,14 @@ int mg_timed_decode(mg_ctx* ctx, int token, int pos, int steps, int useGraph, fl
  * (+argmax partials), 7 argmax finish}; classLaunches[8] = launches per token. */
 int mg_profile_decode(mg_ctx* ctx, int token, int pos, int steps, float* classMs, int* classLaunches);
 
+/* Measurement helper: mean microseconds of one dequantizing matvec launch at
+ * shape [N, K] (wf 0 = Q8 per-row scale, 1 = Q4_0 split layout), over `iters`
+ * launches that rotate through `copies` weight buffers (choose copies so that
+ * copies * bytes exceeds the on-chip caches and every launch streams from
+ * HBM).  nr (rows per wave group), ks (1 or 4: waves sharing a row group) and
+ * grid = 0 use the library's own configuration. */
+int mg_bench_matvec(int wf, int N, int K, int nr, int ks, int grid, int copies, int iters, float* avgUs);
+
 /* Bytes of weights, scales and norm gains one token reads (the figure the
  * bandwidth roofline is computed from), and the KV bytes read at position pos. */
 uint64_t mg_weight_bytes_per_token(const mg_ctx* ctx);

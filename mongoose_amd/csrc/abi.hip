@@ -7,6 +7,7 @@
 #include <atomic>
 #include <cstdio>
 #include <cstring>
+#include <vector>
 
 namespace {
 std::atomic<int> g_lastErr{0};
@@ -144,6 +145,57 @@ void mongoose_zero(void* ptr, size_t bytes, void* stream) {
     note(mg::launch_fill_zero(ptr, bytes, S(stream)));
 }
 void mongoose_sync(void* stream) { note(hipStreamSynchronize(S(stream))); }
+
+// Measurement helper: average duration of the Q8 / Q4_0 matvec at one shape,
+// launched `iters` times over `copies` separate weight buffers in rotation (so
+// that with copies * bytes larger than the caches every launch streams from
+// HBM).  nr/ks/grid = 0 picks the library's own configuration.
+int mg_bench_matvec(int wf, int N, int K, int nr, int ks, int grid, int copies, int iters, float* avgUs) {
+    if ((wf != mg::WF_Q8 && wf != mg::WF_Q4P) || N <= 0 || K <= 0 || K % 32 || copies < 1 || iters < 1 || !avgUs) return MG_E_ARG;
+    size_t wbytes = wf == mg::WF_Q8 ? (size_t)N * K : (size_t)N * (K / 32) * 18;
+    std::vector<void*> w(copies, nullptr);
+    void* slab = nullptr;
+    float *scales = nullptr, *act = nullptr, *out = nullptr;
+    hipStream_t st = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int rc = MG_OK;
+    auto ok = [&](hipError_t e) { if (e != hipSuccess) { rc = MG_E_HIP; (void)hipGetLastError(); } return e == hipSuccess; };
+    do {
+        if (!ok(hipStreamCreateWithFlags(&st, hipStreamNonBlocking))) break;
+        if (!ok(hipEventCreate(&e0)) || !ok(hipEventCreate(&e1))) break;
+        // one slab for all copies (as the context's weight arena is laid out), 256-byte aligned slices
+        size_t slice = (wbytes + 255) & ~(size_t)255;
+        if (!ok(hipMalloc(&slab, slice * copies)) || !ok(hipMemset(slab, 0x11, slice * copies))) break;
+        for (int c = 0; c < copies; c++) w[c] = static_cast<char*>(slab) + slice * c;
+        if (!ok(hipMalloc((void**)&scales, (size_t)N * 4)) || !ok(hipMalloc((void**)&act, (size_t)K * 4)) ||
+            !ok(hipMalloc((void**)&out, (size_t)N * 4))) break;
+        if (!ok(hipMemset(scales, 0, (size_t)N * 4)) || !ok(hipMemset(act, 0, (size_t)K * 4))) break;
+        mg::MvConfig cfg{nr, ks ? ks : 1, grid};
+        auto launch = [&](int c) {
+            mg::MvParams p{};
+            p.seg[0] = mg::MvSeg{w[c], scales, nullptr, out, N};
+            p.nseg = 1; p.K = K; p.act = act;
+            mg::MvConfig use = cfg;
+            return mg::launch_matvec(wf, mg::EPI_STORE, mg::PRO_PLAIN, p, nr > 0 ? &use : nullptr, st);
+        };
+        for (int c = 0; c < copies && rc == MG_OK; c++) ok(launch(c));
+        if (rc != MG_OK || !ok(hipStreamSynchronize(st))) break;
+        if (!ok(hipEventRecord(e0, st))) break;
+        for (int i = 0; i < iters && rc == MG_OK; i++) ok(launch(i % copies));
+        if (rc != MG_OK || !ok(hipEventRecord(e1, st)) || !ok(hipEventSynchronize(e1))) break;
+        float ms = 0.f;
+        if (!ok(hipEventElapsedTime(&ms, e0, e1))) break;
+        *avgUs = ms * 1000.0f / (float)iters;
+    } while (0);
+    if (slab) (void)hipFree(slab);
+    if (scales) (void)hipFree(scales);
+    if (act) (void)hipFree(act);
+    if (out) (void)hipFree(out);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (st) (void)hipStreamDestroy(st);
+    return rc;
+}
 
 int mongoose_check(void) {
     hipError_t e = hipGetLastError();

@@ -20,6 +20,17 @@ struct DevMat {
     size_t bytes = 0;       // bytes a token reads from this matrix (weights + scales)
 };
 
+inline size_t alignUp256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// One device allocation handed out in 256-byte aligned pieces.
+struct Slab {
+    char* base = nullptr;
+    size_t size = 0, used = 0;
+    int init(size_t bytes);
+    void* take(size_t bytes);
+    void release();
+};
+
 struct LayerWeights {
     float* norm1 = nullptr;
     float* norm2 = nullptr;
@@ -86,15 +97,19 @@ private:
     HIPFusedInference() = default;
     bool built = false;
     int invalidateGraphs();
-    int uploadMat(DevMat& m, int rows, int cols, const int8_t* q, const float* scales);
-    int uploadMatQ4(DevMat& m, int rows, int cols, const uint8_t* raw, size_t nbytes);
-    int setVec(float*& dst, const float* data, size_t n, size_t expect);
+    int uploadMat(int idx, DevMat& m, int rows, int cols, const int8_t* q, const float* scales);
+    int uploadMatQ4(int idx, DevMat& m, int rows, int cols, const uint8_t* raw, size_t nbytes);
+    int setVec(int idx, float*& dst, const float* data, size_t n, size_t expect);
+    int slotAddr(int idx, char** out);
+    Slab scratch, headSlab;
+    std::vector<Slab> layerSlabs, kvSlabs;
+    size_t slotOff[12] = {0};
+    size_t layerSlabBytes = 0;
     DevMat* matSlot(int idx, int* rows, int* cols);
     int enqueueLayerFused(const LayerWeights& L, int layer, const StepState* st, int posImm);
     int enqueueLayerPerOp(const LayerWeights& L, int layer, int pos);
     int enqueueEmbed();
     int enqueueToken(bool withHead);      // embed -> layers -> final(+argmax) / advance, all from device state
-    int freeMat(DevMat& m);
 
     // scratch (cuda_fused_infer.go:56-69, :626)
     float *normed = nullptr, *Q = nullptr, *K = nullptr, *V = nullptr, *attnOut = nullptr, *proj = nullptr;

@@ -62,6 +62,25 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
     f->ffnDim = ffnDim; f->vocabSize = vocabSize; f->nLayers = nLayers; f->maxSeq = maxSeq;
     f->ropeTheta = ropeTheta; f->eps = eps;
     f->layers.resize(nLayers);
+    f->layerSlabs.resize(nLayers);
+    {
+        // slot offsets inside a layer slab, each slot sized for its largest format (Q8: bytes + row scales)
+        size_t off = 0;
+        for (int w = 0; w < 12; w++) {
+            size_t rows = 0, cols = 0;
+            switch (w) {
+            case 1: case 7: rows = dim; cols = dim; break;
+            case 2: case 3: rows = kvDim; cols = dim; break;
+            case 9: case 10: rows = ffnDim; cols = dim; break;
+            case 11: rows = dim; cols = ffnDim; break;
+            case 5: case 6: rows = kvDim; break;
+            default: rows = dim; break;
+            }
+            f->slotOff[w] = off;
+            off += cols ? alignUp256(rows * cols) + alignUp256(rows * 4) : alignUp256(rows * 4);
+        }
+        f->layerSlabBytes = off;
+    }
     f->kCache.assign(nLayers, nullptr);
     f->vCache.assign(nLayers, nullptr);
 
@@ -73,13 +92,36 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
     if (hipStreamCreateWithFlags(&f->stream, hipStreamNonBlocking) != hipSuccess) return fail("stream create failed");
     if (hipEventCreate(&f->ev0) != hipSuccess || hipEventCreate(&f->ev1) != hipSuccess) return fail("event create failed");
 
-    bool ok = devAlloc(f->hidden[0], dim, true) == 0 && devAlloc(f->hidden[1], dim, true) == 0 &&
-              devAlloc(f->logits, vocabSize, true) == 0 && devAlloc(f->normed, dim, true) == 0 &&
-              devAlloc(f->Q, dim, true) == 0 && devAlloc(f->K, kvDim, true) == 0 && devAlloc(f->V, kvDim, true) == 0 &&
-              devAlloc(f->attnOut, dim, true) == 0 && devAlloc(f->proj, dim, true) == 0 &&
-              devAlloc(f->normed2, dim, true) == 0 && devAlloc(f->gatePre, ffnDim, true) == 0 &&
-              devAlloc(f->upOut, ffnDim, true) == 0 && devAlloc(f->ffnMid, ffnDim, true) == 0;
-    if (!ok) return fail("scratch alloc failed");
+    // Every device buffer of the context comes out of a few large slabs (one for the scratch
+    // and tables, one per layer of weights, one for the head, one per KV range): large
+    // contiguous mappings keep the address-translation cost of a cold weight read low, which
+    // is a measurable part of a small matvec's latency.
+    const int half0 = headDim / 2;
+    f->splitLen = 256 * ((maxSeq + 256 * 32 - 1) / (256 * 32));
+    f->smax = (maxSeq + f->splitLen - 1) / f->splitLen;
+    f->attnHeadsPerWG = maxSeq <= 1024 ? 1 : 0;
+    f->amaxParts = 4096;
+    {
+        size_t floats = (size_t)7 * dim + 2 * (size_t)kvDim + 3 * (size_t)ffnDim + vocabSize +
+                        2 * (size_t)maxSeq * half0 + (size_t)nHeads * f->smax * (headDim + 2) + headDim + f->amaxParts;
+        size_t ints = (size_t)f->amaxParts + 2 * ((size_t)maxSeq + 1) + 64 + attention_columns(nHeads, nKVHeads, 1);
+        size_t bytes = (floats + ints) * 4 + 64 * 256;
+        if (f->scratch.init(bytes) != 0) return fail("scratch alloc failed");
+        if (hipMemset(f->scratch.base, 0, bytes) != hipSuccess) return fail("scratch clear failed");
+    }
+    auto takeF = [&](float*& p, size_t n) { p = static_cast<float*>(f->scratch.take(n * 4)); return p != nullptr; };
+    auto takeI = [&](int*& p, size_t n) { p = static_cast<int*>(f->scratch.take(n * 4)); return p != nullptr; };
+    bool ok = takeF(f->hidden[0], dim) && takeF(f->hidden[1], dim) && takeF(f->logits, vocabSize) && takeF(f->normed, dim) &&
+              takeF(f->Q, dim) && takeF(f->K, kvDim) && takeF(f->V, kvDim) && takeF(f->attnOut, dim) && takeF(f->proj, dim) &&
+              takeF(f->normed2, dim) && takeF(f->gatePre, ffnDim) && takeF(f->upOut, ffnDim) && takeF(f->ffnMid, ffnDim) &&
+              takeF(f->cosTab, (size_t)maxSeq * half0) && takeF(f->sinTab, (size_t)maxSeq * half0) &&
+              takeF(f->pm, (size_t)nHeads * f->smax) && takeF(f->pl, (size_t)nHeads * f->smax) &&
+              takeF(f->pacc, (size_t)nHeads * f->smax * headDim) && takeF(f->ropeCur, headDim) &&
+              takeF(f->amaxVal, f->amaxParts) && takeI(f->amaxIdx, f->amaxParts) &&
+              takeI(f->attnCounters, attention_columns(nHeads, nKVHeads, 1)) &&
+              takeI(f->dHistory, (size_t)maxSeq + 1) && takeI(f->dPrompt, (size_t)maxSeq + 1);
+    if (ok) { f->dState = static_cast<StepState*>(f->scratch.take(sizeof(StepState))); ok = f->dState != nullptr; }
+    if (!ok) return fail("scratch slab too small");
 
     // RoPE tables, cuda_fused_infer.go:181-192: angle in double, stored as float.
     const int half = headDim / 2;
@@ -93,24 +135,9 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
             sinD[(size_t)pos * half + j] = (float)std::sin(angle);
         }
     }
-    if (devAlloc(f->cosTab, cosD.size(), false) != 0 || devAlloc(f->sinTab, sinD.size(), false) != 0) return fail("rope alloc");
     if (hipMemcpy(f->cosTab, cosD.data(), cosD.size() * 4, hipMemcpyHostToDevice) != hipSuccess ||
         hipMemcpy(f->sinTab, sinD.data(), sinD.size() * 4, hipMemcpyHostToDevice) != hipSuccess) return fail("rope upload");
 
-    // split-KV geometry, fixed for the context: splits of a multiple of 256 positions, at most 32 of them
-    f->splitLen = 256 * ((maxSeq + 256 * 32 - 1) / (256 * 32));
-    f->smax = (maxSeq + f->splitLen - 1) / f->splitLen;
-    // short contexts: latency-bound, spread the GQA group over workgroups; long: read K/V once per group
-    f->attnHeadsPerWG = maxSeq <= 1024 ? 2 : 0;
-    if (devAlloc(f->pm, (size_t)nHeads * f->smax, true) != 0 || devAlloc(f->pl, (size_t)nHeads * f->smax, true) != 0 ||
-        devAlloc(f->pacc, (size_t)nHeads * f->smax * headDim, true) != 0 ||
-        devAlloc(f->attnCounters, (size_t)attention_columns(nHeads, nKVHeads, 1), true) != 0 ||
-        devAlloc(f->ropeCur, (size_t)headDim, true) != 0) return fail("attention partial alloc");
-
-    f->amaxParts = 2048;
-    if (devAlloc(f->amaxVal, f->amaxParts, true) != 0 || devAlloc(f->amaxIdx, f->amaxParts, true) != 0 ||
-        devAlloc(f->dState, 1, true) != 0 || devAlloc(f->dHistory, (size_t)maxSeq + 1, true) != 0 ||
-        devAlloc(f->dPrompt, (size_t)maxSeq + 1, true) != 0) return fail("state alloc");
     void* hp = nullptr;
     if (hipHostMalloc(&hp, sizeof(StepState), hipHostMallocDefault) != hipSuccess) return fail("pinned alloc");
     f->hState = static_cast<StepState*>(hp);
@@ -124,31 +151,47 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
     return f;
 }
 
-int HIPFusedInference::freeMat(DevMat& m) {
-    if (m.w) (void)hipFree(m.w);
-    if (m.scales) (void)hipFree(m.scales);
-    m = DevMat();
+int Slab::init(size_t bytes) {
+    release();
+    void* v = nullptr;
+    HIPCHK(hipMalloc(&v, bytes ? bytes : 256));
+    base = static_cast<char*>(v); size = bytes; used = 0;
+    return MG_OK;
+}
+void* Slab::take(size_t bytes) {
+    size_t off = alignUp256(used);
+    if (!base || off + bytes > size) return nullptr;
+    used = off + bytes;
+    return base + off;
+}
+void Slab::release() {
+    if (base) (void)hipFree(base);
+    base = nullptr; size = used = 0;
+}
+
+// Device address of a weight slot (allocating the layer's / head's slab on first use).
+int HIPFusedInference::slotAddr(int idx, char** out) {
+    if (idx < nLayers * 12) {
+        Slab& sl = layerSlabs[idx / 12];
+        if (!sl.base) { int rc = sl.init(layerSlabBytes); if (rc) return rc; }
+        *out = sl.base + slotOff[idx % 12];
+        return MG_OK;
+    }
+    if (!headSlab.base) {
+        int rc = headSlab.init(alignUp256((size_t)dim * 4) + alignUp256((size_t)vocabSize * dim) + alignUp256((size_t)vocabSize * 4));
+        if (rc) return rc;
+    }
+    *out = headSlab.base + (idx == nLayers * 12 ? 0 : alignUp256((size_t)dim * 4));
     return MG_OK;
 }
 
 HIPFusedInference::~HIPFusedInference() {
     if (stream) (void)hipStreamSynchronize(stream);
     invalidateGraphs();
-    for (auto& L : layers) {
-        for (float* p : {L.norm1, L.norm2, L.bq, L.bk, L.bv}) if (p) (void)hipFree(p);
-        for (DevMat* m : {&L.wq, &L.wk, &L.wv, &L.wo, &L.gate, &L.up, &L.down}) freeMat(*m);
-    }
-    freeMat(lmHead);
-    for (float* p : kCache) if (p) (void)hipFree(p);
-    for (float* p : vCache) if (p) (void)hipFree(p);
-    for (float* p : {hidden[0], hidden[1], logits, finalNorm, normed, Q, K, V, attnOut, proj, normed2, gatePre, upOut,
-                     ffnMid, cosTab, sinTab, pm, pl, pacc, amaxVal}) if (p) (void)hipFree(p);
-    if (amaxIdx) (void)hipFree(amaxIdx);
-    if (attnCounters) (void)hipFree(attnCounters);
-    if (ropeCur) (void)hipFree(ropeCur);
-    if (dState) (void)hipFree(dState);
-    if (dHistory) (void)hipFree(dHistory);
-    if (dPrompt) (void)hipFree(dPrompt);
+    scratch.release();
+    headSlab.release();
+    for (auto& sl : layerSlabs) sl.release();
+    for (auto& sl : kvSlabs) sl.release();
     if (embedTable) (void)hipFree(embedTable);
     if (hState) (void)hipHostFree(hState);
     if (hGate) (void)hipHostFree(hGate);
@@ -187,44 +230,47 @@ DevMat* HIPFusedInference::matSlot(int idx, int* rows, int* cols) {
     return nullptr;
 }
 
-int HIPFusedInference::setVec(float*& dst, const float* data, size_t n, size_t expect) {
+int HIPFusedInference::setVec(int idx, float*& dst, const float* data, size_t n, size_t expect) {
     ARGCHK(n == expect, "SetWeight: wrong element count for a norm/bias slot");
-    if (!dst) { int rc = devAlloc(dst, expect, false); if (rc) return rc; }
+    char* addr = nullptr;
+    int rc = slotAddr(idx, &addr);
+    if (rc) return rc;
     HIPCHK(hipStreamSynchronize(stream));
-    HIPCHK(hipMemcpy(dst, data, expect * sizeof(float), hipMemcpyHostToDevice));
+    HIPCHK(hipMemcpy(addr, data, expect * sizeof(float), hipMemcpyHostToDevice));
+    dst = reinterpret_cast<float*>(addr);
     return MG_OK;
 }
 
-int HIPFusedInference::uploadMat(DevMat& m, int rows, int cols, const int8_t* q, const float* scales) {
+int HIPFusedInference::uploadMat(int idx, DevMat& m, int rows, int cols, const int8_t* q, const float* scales) {
     HIPCHK(hipStreamSynchronize(stream));
     invalidateGraphs();
-    freeMat(m);
-    void* w = nullptr;
-    HIPCHK(hipMalloc(&w, (size_t)rows * cols));
-    m.w = w;
-    HIPCHK(hipMemcpy(m.w, q, (size_t)rows * cols, hipMemcpyHostToDevice));
-    int rc = devAlloc(m.scales, rows, false);
+    char* addr = nullptr;
+    int rc = slotAddr(idx, &addr);
     if (rc) return rc;
-    HIPCHK(hipMemcpy(m.scales, scales, (size_t)rows * 4, hipMemcpyHostToDevice));
+    m = DevMat();
+    HIPCHK(hipMemcpy(addr, q, (size_t)rows * cols, hipMemcpyHostToDevice));
+    char* sc = addr + alignUp256((size_t)rows * cols);
+    HIPCHK(hipMemcpy(sc, scales, (size_t)rows * 4, hipMemcpyHostToDevice));
+    m.w = addr; m.scales = reinterpret_cast<float*>(sc);
     m.kind = WF_Q8; m.rows = rows; m.cols = cols;
     m.bytes = (size_t)rows * cols + (size_t)rows * 4;
     return MG_OK;
 }
 
-int HIPFusedInference::uploadMatQ4(DevMat& m, int rows, int cols, const uint8_t* raw, size_t nbytes) {
+int HIPFusedInference::uploadMatQ4(int idx, DevMat& m, int rows, int cols, const uint8_t* raw, size_t nbytes) {
     ARGCHK(cols % 32 == 0, "SetWeightQ4_0: cols must be a multiple of 32");
     size_t expect = (size_t)rows * (cols / 32) * 18;          // cuda_q4_0.go:16-19
     ARGCHK(nbytes == expect, "SetWeightQ4_0: byte count is not rows*(cols/32)*18");
     HIPCHK(hipStreamSynchronize(stream));
     invalidateGraphs();
-    freeMat(m);
+    char* addr = nullptr;
+    int rc = slotAddr(idx, &addr);
+    if (rc) return rc;
+    m = DevMat();
     std::vector<uint8_t> planar(expect);
     repack_q4_0_host(raw, rows, cols, planar.data());
-    void* w = nullptr;
-    HIPCHK(hipMalloc(&w, expect));
-    m.w = w;
-    HIPCHK(hipMemcpy(m.w, planar.data(), expect, hipMemcpyHostToDevice));
-    m.kind = WF_Q4P; m.rows = rows; m.cols = cols; m.bytes = expect;
+    HIPCHK(hipMemcpy(addr, planar.data(), expect, hipMemcpyHostToDevice));
+    m.w = addr; m.kind = WF_Q4P; m.rows = rows; m.cols = cols; m.bytes = expect;
     return MG_OK;
 }
 
@@ -238,16 +284,16 @@ int HIPFusedInference::SetWeight(int idx, const float* data, size_t n) {
         std::vector<int8_t> q((size_t)rows * cols);
         std::vector<float> sc(rows);
         mg_quantize_q8(data, rows, cols, quantRounding, q.data(), sc.data());
-        return uploadMat(*m, rows, cols, q.data(), sc.data());
+        return uploadMat(idx, *m, rows, cols, q.data(), sc.data());
     }
-    if (idx == nLayers * 12) return setVec(finalNorm, data, n, dim);
+    if (idx == nLayers * 12) return setVec(idx, finalNorm, data, n, dim);
     LayerWeights& L = layers[idx / 12];
     switch (idx % 12) {
-    case 0: return setVec(L.norm1, data, n, dim);
-    case 8: return setVec(L.norm2, data, n, dim);
-    case 4: invalidateGraphs(); return setVec(L.bq, data, n, dim);
-    case 5: invalidateGraphs(); return setVec(L.bk, data, n, kvDim);
-    case 6: invalidateGraphs(); return setVec(L.bv, data, n, kvDim);
+    case 0: return setVec(idx, L.norm1, data, n, dim);
+    case 8: return setVec(idx, L.norm2, data, n, dim);
+    case 4: invalidateGraphs(); return setVec(idx, L.bq, data, n, dim);
+    case 5: invalidateGraphs(); return setVec(idx, L.bk, data, n, kvDim);
+    case 6: invalidateGraphs(); return setVec(idx, L.bv, data, n, kvDim);
     }
     set_error("SetWeight: unreachable slot");
     return MG_E_ARG;
@@ -258,7 +304,7 @@ int HIPFusedInference::SetWeightQ8(int idx, const int8_t* q, const float* scales
     int rows = 0, cols = 0;
     DevMat* m = matSlot(idx, &rows, &cols);
     ARGCHK(m && q && scales, "SetWeightQ8: not a matrix slot or NULL data");
-    return uploadMat(*m, rows, cols, q, scales);
+    return uploadMat(idx, *m, rows, cols, q, scales);
 }
 
 int HIPFusedInference::SetWeightQ4_0(int idx, const uint8_t* q4Data, size_t nbytes) {
@@ -268,7 +314,7 @@ int HIPFusedInference::SetWeightQ4_0(int idx, const uint8_t* q4Data, size_t nbyt
     // cuda_fused_infer_q4.go:52,66,78: norm, bias and final-norm slots are not Q4 and are ignored
     if (!m) return (idx >= 0 && idx < NumWeights()) ? MG_OK : MG_E_ARG;
     ARGCHK(q4Data != nullptr, "SetWeightQ4_0: NULL data");
-    return uploadMatQ4(*m, rows, cols, q4Data, nbytes);
+    return uploadMatQ4(idx, *m, rows, cols, q4Data, nbytes);
 }
 
 int HIPFusedInference::SetEmbeddingF16(const uint16_t* table) {
@@ -300,14 +346,20 @@ int HIPFusedInference::SetEmbeddingF32(const float* table) {
 int HIPFusedInference::SetLayerRange(int layerStart, int layerEnd) {
     if (!built) return MG_E_NOT_BUILT;
     ARGCHK(layerStart >= 0 && layerStart <= layerEnd, "SetLayerRange: bad range");
+    int need = 0;
+    for (int l = layerStart; l < layerEnd && l < nLayers; l++) if (!kCache[l]) need++;
+    if (need == 0) return MG_OK;
+    invalidateGraphs();
+    const size_t per = alignUp256((size_t)maxSeq * kvDim * 4);
+    kvSlabs.emplace_back();
+    Slab& sl = kvSlabs.back();
+    int rc = sl.init(per * 2 * need);
+    if (rc) { kvSlabs.pop_back(); return rc; }
+    HIPCHK(hipMemset(sl.base, 0, sl.size));
     for (int l = layerStart; l < layerEnd && l < nLayers; l++) {
-        if (!kCache[l]) {
-            invalidateGraphs();
-            int rc = devAlloc(kCache[l], (size_t)maxSeq * kvDim, true);
-            if (rc) return rc;
-            rc = devAlloc(vCache[l], (size_t)maxSeq * kvDim, true);
-            if (rc) return rc;
-        }
+        if (kCache[l]) continue;
+        kCache[l] = static_cast<float*>(sl.take(per));
+        vCache[l] = static_cast<float*>(sl.take(per));
     }
     return MG_OK;
 }

@@ -433,24 +433,25 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     }
 }
 
+// Launch shape from measurements on MI355X (cold weights, all benchmark shapes):
+// two rows per wave group is the best default, four for very tall matrices
+// (lm_head), and the K split over the workgroup only pays for long rows with
+// too few of them to give every CU a wave otherwise.
 MvConfig pick_config(int wf, int epi, int totalRows, int K) {
     const int CH = wf == WF_Q8 ? 16 : 32;
     const int nch = K / CH;
     MvConfig c;
-    c.ks = 1;
-    // Long rows and few of them: split K over the workgroup.
-    if (nch > 128 && totalRows <= 8192) c.ks = 4;
+    c.ks = (nch > 128 && totalRows < 2048) ? 4 : 1;
     if (epi == EPI_QKV) {
         c.nr = 2;
     } else if (epi == EPI_SWIGLU) {
         // totalRows counts gate rows; each group carries gate and up rows
-        c.nr = totalRows >= 8192 ? 4 : 2;
+        c.nr = totalRows >= 32768 ? 4 : 2;
     } else if (c.ks == 4) {
-        c.nr = totalRows >= 4096 ? 2 : 1;
+        c.nr = 4;
     } else {
-        c.nr = totalRows >= 16384 ? 4 : (totalRows >= 4096 ? 2 : 1);
+        c.nr = totalRows >= 65536 ? 4 : 2;
     }
-    if (epi == EPI_RESID && c.nr > 2) c.nr = 2;
     c.grid = 0;   // filled by the launcher from the group count
     return c;
 }
@@ -471,8 +472,6 @@ static hipError_t launch_pe(MvParams& p, const MvConfig& c, hipStream_t s) {
         MV_CASE(2, 1) MV_CASE(2, 4)
     } else if (EPI == EPI_SWIGLU) {
         MV_CASE(2, 1) MV_CASE(2, 4) MV_CASE(4, 1) MV_CASE(4, 4)
-    } else if (EPI == EPI_RESID) {
-        MV_CASE(1, 1) MV_CASE(1, 4) MV_CASE(2, 1) MV_CASE(2, 4)
     } else {
         MV_CASE(1, 1) MV_CASE(1, 4) MV_CASE(2, 1) MV_CASE(2, 4) MV_CASE(4, 1) MV_CASE(4, 4)
     }
@@ -522,7 +521,7 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
     }
     if (p.ngroups == 0) return hipSuccess;
     int wgs = c.ks == 1 ? (p.ngroups + 3) / 4 : p.ngroups;
-    int cap = 2048;
+    int cap = epi == EPI_ARGMAX ? 1024 : 4096;      // one argmax partial per workgroup
     if (c.grid <= 0 || c.grid > wgs) c.grid = wgs < cap ? wgs : cap;
     if (cfgInOut) *cfgInOut = c;
     if (wf == WF_Q8) return launch_wf<WF_Q8>(pro, epi, p, c, s);
