@@ -26,6 +26,15 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
 
+# HBM bytes per launch of the lm_head kernel from rocprofv3 --pmc runs of this script
+# (FETCH_SIZE then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
+# reads for a 256 MiB device copy in the same run (FETCH_SIZE reads 131091.6 KiB for the
+# 262144 KiB copied -> x1.9997; WRITE_SIZE reads 262144.0 -> x1.0).  Counts are a property
+# of kernel and shape, so they are recorded here; profiles/ holds the run they come from.
+PMC_TRAFFIC_BYTES = {
+    "qwen2.5-0.5b": int((67167.6 * (262144.0 / 131091.6) + 660.2 * 1.0) * 1024),
+}
+
 
 def slot_shape(s, kv, idx):
     nL = s.nLayers
@@ -145,6 +154,8 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds of CPU baseline work (0 = skip)")
     ap.add_argument("--profile-steps", type=int, default=20)
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--pmc-copy", action="store_true",
+                    help="also run three 256 MiB device copies (a kernel of known traffic, to scale rocprofv3 --pmc counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
@@ -188,6 +199,10 @@ def main():
     assert rc == 0, E.last_error()
     cls_ms = [float(x) for x in cls_ms]
     cls_n = [int(x) for x in cls_n]
+    # the dominant kernel once more with events around it alone (less event overhead in its interval)
+    rc, lm_only, _ = f.ProfileDecode(int(first[0]), W, args.profile_steps, classMask=1 << 6)
+    assert rc == 0, E.last_error()
+    lm_only_ms = float(lm_only[6])
 
     def mat(n, k):
         return n * k + 4 * n if s.fmt == "q8" else n * (k // 32) * 18
@@ -217,12 +232,21 @@ def main():
     assert f.WeightBytesPerToken() == wbytes
     step_bytes = wbytes + configs.kv_bytes_at(s, p_mid)
     lm_bytes = cls_bytes[6]
-    lm_s = float(cls_ms[6]) * 1e-3
+    lm_s = lm_only_ms * 1e-3
     roofline = {"bound": "hbm", "kernel": "matvec lm_head (final norm + Q8 matvec + argmax partials)",
                 "achieved": round(lm_bytes / lm_s / 1e9, 1) if lm_s > 0 else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(lm_bytes / lm_s / 1e9 / HBM_PEAK_GBS, 4) if lm_s > 0 else None,
                 "bytes_per_launch": int(lm_bytes), "avg_launch_us": round(lm_s * 1e6, 2),
-                "launches_timed": int(args.profile_steps), "traffic": None}
+                "launches_timed": int(args.profile_steps), "traffic": PMC_TRAFFIC_BYTES.get(s.name)}
+
+    if args.pmc_copy:
+        n = 256 << 20
+        a, b = eng.UploadRawBytes(np.zeros(n, np.uint8)), eng.UploadRawBytes(np.zeros(n, np.uint8))
+        for _ in range(3):
+            E.KCopy(b, a, n)
+        E.KSync()
+        a.Release()
+        b.Release()
 
     cpu = None
     if args.cpu_budget > 0:

@@ -203,8 +203,11 @@ int mg_timed_decode(mg_ctx* ctx, int token, int pos, int steps, int useGraph, fl
  * waits for the host.  classMs[8] = mean milliseconds per launch
  * of class {0 embedding gather, 1 norm+QKV(+bias), 2 RoPE+KV write+attention,
  * 3 Wo+residual, 4 norm+gate/up+SiLU*mul, 5 down+residual, 6 final norm+lm_head
- * (+argmax partials), 7 argmax finish}; classLaunches[8] = launches per token. */
-int mg_profile_decode(mg_ctx* ctx, int token, int pos, int steps, float* classMs, int* classLaunches);
+ * (+argmax partials), 7 argmax finish}; classLaunches[8] = launches per token.
+ * classMask selects the classes to bracket (bit c = class c, 0 = all): every
+ * event costs the stream a few microseconds, so one class alone is measured
+ * closest to its kernel time. */
+int mg_profile_decode(mg_ctx* ctx, int token, int pos, int steps, unsigned classMask, float* classMs, int* classLaunches);
 
 /* Measurement helper: mean microseconds of one dequantizing matvec launch at
  * shape [N, K] (wf 0 = Q8 per-row scale, 1 = Q4_0 split layout), over `iters`

@@ -69,7 +69,7 @@ public:
     int GraphLaunch(int token, int pos, int* nextToken);                          // cuda_graph.go:663
     int GraphValidate(int token, int pos, float* maxAbsDiff);                     // cuda_graph.go:554
     int TimedDecode(int token, int pos, int steps, bool useGraph, float* elapsedMs);
-    int ProfileDecode(int token, int pos, int steps, float* classMs, int* classLaunches);
+    int ProfileDecode(int token, int pos, int steps, unsigned classMask, float* classMs, int* classLaunches);
     uint64_t WeightBytesPerToken() const;
     uint64_t KVBytesAt(int pos) const { return (uint64_t)2 * nLayers * (uint64_t)(pos + 1) * kvDim * 4; }
 
@@ -141,6 +141,8 @@ private:
     std::vector<hipEvent_t> profEvents;
     std::vector<int> profClass;       // class of the launch that follows event i
     bool profiling = false;
+    unsigned profMask = 0xffu;
+    int profLast = -1;
     int mark(int cls);
 };
 

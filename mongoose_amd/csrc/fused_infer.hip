@@ -392,6 +392,12 @@ uint64_t HIPFusedInference::WeightBytesPerToken() const {
 // of class `cls` (the previous launch's end).  No-op otherwise.
 int HIPFusedInference::mark(int cls) {
     if (!profiling) return MG_OK;
+    // an event opens the interval of a wanted class and closes the interval of the one before it
+    const bool opens = cls >= 0 && cls < 8 && ((profMask >> cls) & 1);
+    const bool closes = profLast >= 0 && profLast < 8 && ((profMask >> profLast) & 1);
+    profLast = cls;
+    if (!opens && !closes) return MG_OK;
+    if (!opens) cls = 8;                      // interval that follows is not measured
     hipEvent_t e = nullptr;
     HIPCHK(hipEventCreate(&e));
     profEvents.push_back(e);
@@ -778,7 +784,7 @@ int HIPFusedInference::TimedDecode(int token, int pos, int steps, bool useGraph,
 // classMs[c] = mean milliseconds from the end of the previous launch to the
 // end of a launch of class c (0 embed, 1 norm+QKV, 2 attention, 3 Wo,
 // 4 gate/up, 5 down, 6 lm_head, 7 argmax finish); classLaunches[c] = launches per token.
-int HIPFusedInference::ProfileDecode(int token, int pos, int steps, float* classMs, int* classLaunches) {
+int HIPFusedInference::ProfileDecode(int token, int pos, int steps, unsigned classMask, float* classMs, int* classLaunches) {
     if (!built) return MG_E_NOT_BUILT;
     ARGCHK(steps >= 1 && steps <= 64 && pos >= 0 && pos + steps <= maxSeq && token >= 0 && token < vocabSize &&
            classMs && classLaunches, "ProfileDecode: bad arguments (1 <= steps <= 64)");
@@ -792,6 +798,8 @@ int HIPFusedInference::ProfileDecode(int token, int pos, int steps, float* class
     HIPCHK(launch_set_state(dState, pos, token, 0, 0, ropeRef(), stream));
     HIPCHK(launch_gate(gate, 100LL * 1000 * 500, stream));   // at most 0.5 s
     profiling = true;
+    profMask = classMask ? classMask : 0xffu;
+    profLast = -1;
     for (int i = 0; i < steps && rc == 0; i++) {
         rc = enqueueToken(true);
         if (rc == 0) rc = mark(8);
@@ -879,8 +887,8 @@ int mg_graph_validate(mg_ctx* c, int token, int pos, float* md) { CTX(c); return
 int mg_timed_decode(mg_ctx* c, int token, int pos, int steps, int useGraph, float* ms) {
     CTX(c); return f->TimedDecode(token, pos, steps, useGraph != 0, ms);
 }
-int mg_profile_decode(mg_ctx* c, int token, int pos, int steps, float* classMs, int* classLaunches) {
-    CTX(c); return f->ProfileDecode(token, pos, steps, classMs, classLaunches);
+int mg_profile_decode(mg_ctx* c, int token, int pos, int steps, unsigned classMask, float* classMs, int* classLaunches) {
+    CTX(c); return f->ProfileDecode(token, pos, steps, classMask, classMs, classLaunches);
 }
 uint64_t mg_weight_bytes_per_token(const mg_ctx* c) { return c && c->f ? c->f->WeightBytesPerToken() : 0; }
 uint64_t mg_kv_bytes_at(const mg_ctx* c, int pos) { return c && c->f ? c->f->KVBytesAt(pos) : 0; }

@@ -353,10 +353,10 @@ class HIPFusedInference:
         rc = lib.mg_timed_decode(self._h, token, pos, steps, 1 if useGraph else 0, ctypes.byref(ms))
         return rc, ms.value
 
-    def ProfileDecode(self, token, pos, steps):
+    def ProfileDecode(self, token, pos, steps, classMask=0):
         ms = np.zeros(8, dtype=np.float32)
         n = np.zeros(8, dtype=np.int32)
-        rc = lib.mg_profile_decode(self._h, token, pos, steps, _fp(ms), _ip(n))
+        rc = lib.mg_profile_decode(self._h, token, pos, steps, classMask, _fp(ms), _ip(n))
         return rc, ms, n
 
     def WeightBytesPerToken(self):

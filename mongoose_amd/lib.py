@@ -86,7 +86,7 @@ _sig("mg_graph_capture", c_int, c_void_p)
 _sig("mg_graph_launch", c_int, c_void_p, c_int, c_int, _i)
 _sig("mg_graph_validate", c_int, c_void_p, c_int, c_int, _f)
 _sig("mg_timed_decode", c_int, c_void_p, c_int, c_int, c_int, c_int, _f)
-_sig("mg_profile_decode", c_int, c_void_p, c_int, c_int, c_int, _f, _i)
+_sig("mg_profile_decode", c_int, c_void_p, c_int, c_int, c_int, ctypes.c_uint, _f, _i)
 _sig("mg_bench_matvec", c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _f)
 _sig("mg_weight_bytes_per_token", c_uint64, c_void_p)
 _sig("mg_kv_bytes_at", c_uint64, c_void_p, c_int)
