@@ -154,6 +154,8 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds of CPU baseline work (0 = skip)")
     ap.add_argument("--profile-steps", type=int, default=20)
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--context", type=int, default=0,
+                    help="start the timed decode at this position (KV rows between the prompt and it are zeros): long-context timing")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run three 256 MiB device copies (a kernel of known traffic, to scale rocprofv3 --pmc counters)")
     args = ap.parse_args()
@@ -172,7 +174,8 @@ def main():
         print("bench.py: no HIP device", file=sys.stderr)
         sys.exit(1)
     K, W = args.steps, max(args.warmup, 1)
-    maxSeq = W + K + args.profile_steps + 8
+    P0 = max(args.context, W)                      # position of the first timed step
+    maxSeq = P0 + K + args.profile_steps + 8
     t_load = time.perf_counter()
     f = load_model(E, np, s, args.seed, maxSeq, eng)
     t_load = time.perf_counter() - t_load
@@ -183,7 +186,7 @@ def main():
     rc, first = f.Generate(prompt, 1, useGraph=use_graph)
     assert rc == 0, E.last_error()
     # timed region: K decode steps at positions W .. W+K-1, token and position stay on the device
-    rc, ms = f.TimedDecode(int(first[0]), W, K, useGraph=use_graph)
+    rc, ms = f.TimedDecode(int(first[0]), P0, K, useGraph=use_graph)
     assert rc == 0, E.last_error()
     toks_per_s = K / (ms / 1e3)
     ms_per_step = ms / K
@@ -195,21 +198,22 @@ def main():
 
     # per-launch-class timing inside a replayed token
     kv = configs.kv_dim(s)
-    rc, cls_ms, cls_n = f.ProfileDecode(int(first[0]), W, args.profile_steps)
+    rc, cls_ms, cls_n = f.ProfileDecode(int(first[0]), P0 + K, args.profile_steps)
     assert rc == 0, E.last_error()
     cls_ms = [float(x) for x in cls_ms]
     cls_n = [int(x) for x in cls_n]
     # the dominant kernel once more with events around it alone (less event overhead in its interval)
-    rc, lm_only, _ = f.ProfileDecode(int(first[0]), W, args.profile_steps, classMask=1 << 6)
+    rc, lm_only, _ = f.ProfileDecode(int(first[0]), P0 + K, args.profile_steps, classMask=1 << 6)
     assert rc == 0, E.last_error()
     lm_only_ms = float(lm_only[6])
 
     def mat(n, k):
         return n * k + 4 * n if s.fmt == "q8" else n * (k // 32) * 18
-    p_mid = W + K // 2
+    p_mid = P0 + K // 2
+    p_prof = P0 + K + args.profile_steps // 2
     cls_bytes = {
         1: mat(s.dim, s.dim) + 2 * mat(kv, s.dim) + 4 * s.dim,
-        2: 2 * (p_mid + 1) * kv * 4,
+        2: 2 * (p_prof + 1) * kv * 4,
         3: mat(s.dim, s.dim),
         4: 2 * mat(s.ffnDim, s.dim) + 4 * s.dim,
         5: mat(s.dim, s.ffnDim),

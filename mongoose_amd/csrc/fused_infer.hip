@@ -97,7 +97,8 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
     // contiguous mappings keep the address-translation cost of a cold weight read low, which
     // is a measurable part of a small matvec's latency.
     const int half0 = headDim / 2;
-    f->splitLen = 256 * ((maxSeq + 256 * 32 - 1) / (256 * 32));
+    const int attnTile = headDim == 128 ? 128 : 256;      // positions per attention tile
+    f->splitLen = attnTile * ((maxSeq + attnTile * 32 - 1) / (attnTile * 32));
     f->smax = (maxSeq + f->splitLen - 1) / f->splitLen;
     f->attnHeadsPerWG = maxSeq <= 1024 ? 1 : 0;
     f->amaxParts = 4096;

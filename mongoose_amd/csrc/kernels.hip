@@ -63,31 +63,37 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 }
 
 // ---------------------------------------------------------------------------
-// Activation vector in LDS.  A lane that owns weight chunk c (CH consecutive
-// weights) needs activations [c*CH, c*CH+CH).  Stored linearly, neighbouring
-// lanes would read float4s CH*4 bytes apart and collide on LDS banks, so the
-// vector is stored as CH/4 planes: plane p holds, for every chunk c, the float4
-// a[c*CH+4p .. +3] at float4 index p*nch + c.  Lane reads are then 16 bytes
-// apart: conflict free.
+// Activation vector in LDS.  A lane owns a weight chunk of 16 weights: 16
+// consecutive int8 (Q8), or half a Q4_0 block = 8 bytes whose low nibbles are
+// elements 8h..8h+7 of the block and whose high nibbles are elements
+// 16+8h..16+8h+7.  Stored linearly, neighbouring lanes would read float4s 64
+// bytes apart and collide on LDS banks, so the vector is stored as 4 planes:
+// plane p holds, for every chunk c, one float4 of the chunk's activations at
+// float4 index p*nch + c.  Lane reads are then 16 bytes apart: conflict free.
 // ---------------------------------------------------------------------------
-template <int CH>
+template <int WF>
 __device__ __forceinline__ int act_slot4(int k4, int nch) {   // k4 = k/4 -> float4 index
-    constexpr int P = CH / 4;
-    int c = k4 / P, p = k4 % P;
-    return p * nch + c;
+    if (WF == WF_Q8) {
+        return (k4 & 3) * nch + (k4 >> 2);
+    } else {
+        // k4 = 8*block + r4; r4: 0,1 lo-half0  2,3 lo-half1  4,5 hi-half0  6,7 hi-half1
+        int blk = k4 >> 3, r4 = k4 & 7;
+        int hi = r4 >> 2, h = (r4 >> 1) & 1, q = r4 & 1;
+        return (hi * 2 + q) * nch + blk * 2 + h;
+    }
 }
 
 // All global loads of a prologue are issued before anything waits on them; the
 // caller has already issued its first weight loads, so the activation latency
 // and the weight latency overlap instead of adding up.
-template <int CH, int PRO>
+template <int WF, int PRO>
 __device__ __forceinline__ void stage_activation(const MvParams& p, float4* a4, float* red) {
     const int K4 = p.K >> 2;
-    const int nch = p.K / CH;
+    const int nch = p.K / 16;
     const int tid = threadIdx.x;
     if (PRO == PRO_PLAIN) {
         const float4* x4 = reinterpret_cast<const float4*>(p.act);
-        for (int i = tid; i < K4; i += WG) a4[act_slot4<CH>(i, nch)] = x4[i];
+        for (int i = tid; i < K4; i += WG) a4[act_slot4<WF>(i, nch)] = x4[i];
     } else if (PRO == PRO_RMS) {
         // mongoose.cu:145-174 / cpu.go:36-47: x * (1/sqrt(mean(x^2)+eps)) * g
         constexpr int XR = 4;                       // float4s kept in registers per thread (K <= 4096)
@@ -116,13 +122,13 @@ __device__ __forceinline__ void stage_activation(const MvParams& p, float4* a4, 
                 float4 o;
                 o.x = xv[r].x * rs * gv[r].x; o.y = xv[r].y * rs * gv[r].y;
                 o.z = xv[r].z * rs * gv[r].z; o.w = xv[r].w * rs * gv[r].w;
-                a4[act_slot4<CH>(i, nch)] = o;
+                a4[act_slot4<WF>(i, nch)] = o;
             }
         }
         for (int i = tid + XR * WG; i < K4; i += WG) {
             float4 v = x4[i], g = g4[i], o;
             o.x = v.x * rs * g.x; o.y = v.y * rs * g.y; o.z = v.z * rs * g.z; o.w = v.w * rs * g.w;
-            a4[act_slot4<CH>(i, nch)] = o;
+            a4[act_slot4<WF>(i, nch)] = o;
         }
     }
 }
@@ -137,81 +143,89 @@ __device__ __forceinline__ float dot4_i8(int w, float4 a, float acc) {
     acc = fmaf((float)(w >> 24), a.w, acc);
     return acc;
 }
-// sum over 4 bytes of a * (nibble - 8); n holds one nibble per byte (0..15)
+// sum over 4 bytes of a * nibble; n holds one nibble per byte (0..15).  The -8
+// offset of Q4_0 is applied once per chunk from the sum of its activations.
+template <int B>
+__device__ __forceinline__ float cvt_ubyte(unsigned n) {
+    // v_cvt_f32_ubyteN straight from the masked dword: one convert per weight; written out
+    // because the compiler otherwise re-derives every nibble with its own bit-field extract
+    float f;
+    if (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(n));
+    else if (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(n));
+    else if (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(n));
+    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(n));
+    return f;
+}
 __device__ __forceinline__ float dot4_nib(unsigned n, float4 a, float acc) {
-    acc = fmaf((float)(n & 0xff) - 8.0f, a.x, acc);
-    acc = fmaf((float)((n >> 8) & 0xff) - 8.0f, a.y, acc);
-    acc = fmaf((float)((n >> 16) & 0xff) - 8.0f, a.z, acc);
-    acc = fmaf((float)(n >> 24) - 8.0f, a.w, acc);
+    acc = fmaf(cvt_ubyte<0>(n), a.x, acc);
+    acc = fmaf(cvt_ubyte<1>(n), a.y, acc);
+    acc = fmaf(cvt_ubyte<2>(n), a.z, acc);
+    acc = fmaf(cvt_ubyte<3>(n), a.w, acc);
     return acc;
 }
 __device__ __forceinline__ float half_bits_to_float(unsigned short h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
 
+// av[0..3]: the chunk's activations (4 float4), asum: their sum (Q4 only).
 template <int WF> struct Fmt;
 template <> struct Fmt<WF_Q8> {
-    static constexpr int CH = 16;
     struct Row { const int4* w; };
     __device__ static Row row(const MvSeg& s, int r, int K) {
         return Row{reinterpret_cast<const int4*>(static_cast<const char*>(s.w) + (size_t)r * K)};
     }
     struct Chunk { int4 w; };
     __device__ static Chunk load(const Row& r, int c) { return Chunk{r.w[c]}; }
-    __device__ static float dot(const Chunk& ck, const float4* a4, int nch, int c, float acc) {
-        acc = dot4_i8(ck.w.x, a4[c], acc);
-        acc = dot4_i8(ck.w.y, a4[nch + c], acc);
-        acc = dot4_i8(ck.w.z, a4[2 * nch + c], acc);
-        acc = dot4_i8(ck.w.w, a4[3 * nch + c], acc);
+    __device__ static float dot(const Chunk& ck, const float4 (&av)[4], float, float acc) {
+        acc = dot4_i8(ck.w.x, av[0], acc);
+        acc = dot4_i8(ck.w.y, av[1], acc);
+        acc = dot4_i8(ck.w.z, av[2], acc);
+        acc = dot4_i8(ck.w.w, av[3], acc);
         return acc;
     }
 };
-// Q4_0: per block s = sum_i act_i*(nib_i-8), then acc += s * f32(d)
-// (kernels/infer.metal:63-75); element order: low nibble of byte j = element
-// j, high nibble = element j+16 (kernels/q4_simd.metal:6-19, GGML).
-__device__ __forceinline__ float dot_q4_block(int4 w, float d, const float4* a4, int nch, int c, float acc) {
-    float s = 0.f;
+// Q4_0 half block: s = sum_i act_i*nib_i - 8*sum_i act_i, then acc += s * f32(d)
+// (block form kernels/infer.metal:63-75; the -8 folded as kernels/q4_simd.metal:6-19
+// does).  Element order: low nibble of byte j = element j, high nibble = element
+// j+16 of the block (GGML).
+__device__ __forceinline__ float dot_q4_half(int2 w, float d, const float4 (&av)[4], float asum, float acc) {
+    float s = -8.0f * asum;
     unsigned q;
-    q = (unsigned)w.x; s = dot4_nib(q & 0x0f0f0f0fu, a4[c], s);           s = dot4_nib((q >> 4) & 0x0f0f0f0fu, a4[4 * nch + c], s);
-    q = (unsigned)w.y; s = dot4_nib(q & 0x0f0f0f0fu, a4[nch + c], s);     s = dot4_nib((q >> 4) & 0x0f0f0f0fu, a4[5 * nch + c], s);
-    q = (unsigned)w.z; s = dot4_nib(q & 0x0f0f0f0fu, a4[2 * nch + c], s); s = dot4_nib((q >> 4) & 0x0f0f0f0fu, a4[6 * nch + c], s);
-    q = (unsigned)w.w; s = dot4_nib(q & 0x0f0f0f0fu, a4[3 * nch + c], s); s = dot4_nib((q >> 4) & 0x0f0f0f0fu, a4[7 * nch + c], s);
+    q = (unsigned)w.x; s = dot4_nib(q & 0x0f0f0f0fu, av[0], s); s = dot4_nib((q >> 4) & 0x0f0f0f0fu, av[2], s);
+    q = (unsigned)w.y; s = dot4_nib(q & 0x0f0f0f0fu, av[1], s); s = dot4_nib((q >> 4) & 0x0f0f0f0fu, av[3], s);
     return fmaf(s, d, acc);
 }
 template <> struct Fmt<WF_Q4P> {
-    static constexpr int CH = 32;
-    struct Row { const int4* qs; const unsigned short* d; };
+    struct Row { const int2* qs; const unsigned short* d; };
     __device__ static Row row(const MvSeg& s, int r, int K) {
         const char* base = static_cast<const char*>(s.w);
         const char* dplane = base + (size_t)s.rows * (K >> 1);
-        return Row{reinterpret_cast<const int4*>(base + (size_t)r * (K >> 1)),
+        return Row{reinterpret_cast<const int2*>(base + (size_t)r * (K >> 1)),
                    reinterpret_cast<const unsigned short*>(dplane) + (size_t)r * (K >> 5)};
     }
-    struct Chunk { int4 w; unsigned short d; };
-    __device__ static Chunk load(const Row& r, int c) { return Chunk{r.qs[c], r.d[c]}; }
-    __device__ static float dot(const Chunk& ck, const float4* a4, int nch, int c, float acc) {
-        return dot_q4_block(ck.w, half_bits_to_float(ck.d), a4, nch, c, acc);
+    struct Chunk { int2 w; unsigned short d; };
+    __device__ static Chunk load(const Row& r, int c) { return Chunk{r.qs[c], r.d[c >> 1]}; }
+    __device__ static float dot(const Chunk& ck, const float4 (&av)[4], float asum, float acc) {
+        return dot_q4_half(ck.w, half_bits_to_float(ck.d), av, asum, acc);
     }
 };
 template <> struct Fmt<WF_Q4RAW> {
-    static constexpr int CH = 32;
     struct Row { const unsigned short* b; };   // 18-byte blocks, 2-byte aligned
     __device__ static Row row(const MvSeg& s, int r, int K) {
         return Row{reinterpret_cast<const unsigned short*>(static_cast<const char*>(s.w) + (size_t)r * (K >> 5) * 18)};
     }
-    struct Chunk { int4 w; unsigned short d; };
+    struct Chunk { int2 w; unsigned short d; };
     __device__ static Chunk load(const Row& r, int c) {
-        const unsigned short* b = r.b + (size_t)c * 9;
+        const unsigned short* b = r.b + (size_t)(c >> 1) * 9;
+        const unsigned short* h = b + 1 + (c & 1) * 4;
         Chunk ck;
         ck.d = b[0];
-        ck.w.x = (int)((unsigned)b[1] | ((unsigned)b[2] << 16));
-        ck.w.y = (int)((unsigned)b[3] | ((unsigned)b[4] << 16));
-        ck.w.z = (int)((unsigned)b[5] | ((unsigned)b[6] << 16));
-        ck.w.w = (int)((unsigned)b[7] | ((unsigned)b[8] << 16));
+        ck.w.x = (int)((unsigned)h[0] | ((unsigned)h[1] << 16));
+        ck.w.y = (int)((unsigned)h[2] | ((unsigned)h[3] << 16));
         return ck;
     }
-    __device__ static float dot(const Chunk& ck, const float4* a4, int nch, int c, float acc) {
-        return dot_q4_block(ck.w, half_bits_to_float(ck.d), a4, nch, c, acc);
+    __device__ static float dot(const Chunk& ck, const float4 (&av)[4], float asum, float acc) {
+        return dot_q4_half(ck.w, half_bits_to_float(ck.d), av, asum, acc);
     }
 };
 
@@ -266,7 +280,6 @@ __device__ __forceinline__ RowRef resolve_row(const MvParams& p, int g, int i) {
 template <int WF, int NR, int KS, int PRO, int EPI>
 __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     using F = Fmt<WF>;
-    constexpr int CH = F::CH;
     constexpr int LPG = KS == 1 ? 64 : WG;           // lanes per group
     constexpr int D = NR >= 4 ? 2 : 4;               // items in flight per wave
     extern __shared__ float4 a4[];
@@ -278,7 +291,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lig = KS == 1 ? lane : (int)threadIdx.x;       // lane within the group
-    const int nch = p.K / CH;
+    const int nch = p.K / 16;
     const int iters = (nch + LPG - 1) / LPG;
     const int gStart = KS == 1 ? blockIdx.x * 4 + wave : blockIdx.x;
     const int gStep = KS == 1 ? gridDim.x * 4 : gridDim.x;
@@ -325,7 +338,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
 #pragma unroll
     for (int s = 0; s < D; s++) issue(s, s);
 
-    stage_activation<CH, PRO>(p, a4, red);
+    stage_activation<WF, PRO>(p, a4, red);
     __syncthreads();
 
     float myBestV = -INFINITY;
@@ -344,8 +357,20 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
                 const int it = item % iters;
                 const int c = lig + it * LPG;
                 if (c < nch) {
+                    float4 av[4];
 #pragma unroll
-                    for (int i = 0; i < NR; i++) acc[i] = F::dot(ring[s][i], a4, nch, c, acc[i]);
+                    for (int pl = 0; pl < 4; pl++) av[pl] = a4[pl * nch + c];
+                    float asum = 0.f;
+                    if (WF != WF_Q8) {
+                        float4 t;
+                        t.x = (av[0].x + av[1].x) + (av[2].x + av[3].x);
+                        t.y = (av[0].y + av[1].y) + (av[2].y + av[3].y);
+                        t.z = (av[0].z + av[1].z) + (av[2].z + av[3].z);
+                        t.w = (av[0].w + av[1].w) + (av[2].w + av[3].w);
+                        asum = (t.x + t.y) + (t.z + t.w);
+                    }
+#pragma unroll
+                    for (int i = 0; i < NR; i++) acc[i] = F::dot(ring[s][i], av, asum, acc[i]);
                 }
                 // operands arrive with the group's first item and are held until its last
                 if (it == 0) { sc = rSc[s]; bi = rBi[s]; re = rRe[s]; cs = rCs[s]; sn = rSn[s]; }
@@ -438,8 +463,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
 // (lm_head), and the K split over the workgroup only pays for long rows with
 // too few of them to give every CU a wave otherwise.
 MvConfig pick_config(int wf, int epi, int totalRows, int K) {
-    const int CH = wf == WF_Q8 ? 16 : 32;
-    const int nch = K / CH;
+    const int nch = K / 16;
     MvConfig c;
     c.ks = (nch > 128 && totalRows < 2048) ? 4 : 1;
     if (epi == EPI_QKV) {
@@ -577,18 +601,21 @@ __device__ __forceinline__ void st_agent(float* p, float v) {
 
 template <int HD, int GMAX>
 __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
+    constexpr int LPP = HD / 64;       // lanes per position in the score phase (64 dims each)
+    constexpr int TILE = WG / LPP;     // positions per tile
     constexpr int LPR = HD / 4;        // lanes per V row
     constexpr int TG = WG / LPR;       // position groups in the P.V phase
-    constexpr int VU = HD == 64 ? 16 : 8;   // V rows in flight per thread (HD 64: a whole tile)
-    constexpr int KQ = 16;             // K float4s held in registers at a time
+    constexpr int VU = TILE / TG;      // V rows per thread and tile, all in flight (16)
+    constexpr int KQ = 16;             // K float4s per lane (64 dims)
     __shared__ float4 q_s4[GMAX * HD / 4];
-    __shared__ float sc[GMAX][WG];
+    __shared__ float sc[GMAX][TILE];
     __shared__ float wred[2][GMAX][4];
     __shared__ float4 accbuf[TG][GMAX][LPR];
     __shared__ int lastFlag;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
+    const int sub = tid % LPP, pIdx = tid / LPP;
     const int G = p.nHeads / p.nKVHeads;
     const int nChunks = (G + GMAX - 1) / GMAX;
     const int kvh = blockIdx.x / nChunks;
@@ -608,7 +635,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     if (tid < gn * (HD / 4)) qv = reinterpret_cast<const float4*>(p.q + (size_t)h0 * HD)[tid];
     float4 kreg[KQ];
     {
-        const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)min(t0 + tid, lastRow) * p.kvDim + kvOff);
+        const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)min(t0 + pIdx, lastRow) * p.kvDim + kvOff) + sub * KQ;
 #pragma unroll
         for (int d4 = 0; d4 < KQ; d4++) kreg[d4] = krow[d4];
     }
@@ -633,12 +660,12 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
     for (int g = 0; g < GMAX; g++) { m[g] = -INFINITY; l[g] = 0.f; acc[g] = make_float4(0.f, 0.f, 0.f, 0.f); }
 
-    for (int tile = t0; tile < t1; tile += WG) {
-        const int t = tile + tid;
+    for (int tile = t0; tile < t1; tile += TILE) {
+        const int t = tile + pIdx;
         const bool active = t < t1;
-        const int tileLen = min(WG, t1 - tile);
-        const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)min(t, lastRow) * p.kvDim + kvOff);
+        const int tileLen = min(TILE, t1 - tile);
         if (tile != t0) {
+            const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)min(t, lastRow) * p.kvDim + kvOff) + sub * KQ;
 #pragma unroll
             for (int d4 = 0; d4 < KQ; d4++) kreg[d4] = krow[d4];
 #pragma unroll
@@ -648,22 +675,19 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
         for (int g = 0; g < GMAX; g++) s[g] = 0.f;
 #pragma unroll
-        for (int part = 0; part < HD / 4; part += KQ) {
-            if (part > 0) {
+        for (int d4 = 0; d4 < KQ; d4++) {
 #pragma unroll
-                for (int d4 = 0; d4 < KQ; d4++) kreg[d4] = krow[part + d4];
+            for (int g = 0; g < GMAX; g++) {
+                float4 q4 = q_s4[g * (HD / 4) + sub * KQ + d4];
+                s[g] = fmaf(q4.x, kreg[d4].x, s[g]);
+                s[g] = fmaf(q4.y, kreg[d4].y, s[g]);
+                s[g] = fmaf(q4.z, kreg[d4].z, s[g]);
+                s[g] = fmaf(q4.w, kreg[d4].w, s[g]);
             }
+        }
+        if (LPP == 2) {
 #pragma unroll
-            for (int d4 = 0; d4 < KQ; d4++) {
-#pragma unroll
-                for (int g = 0; g < GMAX; g++) {
-                    float4 q4 = q_s4[g * (HD / 4) + part + d4];
-                    s[g] = fmaf(q4.x, kreg[d4].x, s[g]);
-                    s[g] = fmaf(q4.y, kreg[d4].y, s[g]);
-                    s[g] = fmaf(q4.z, kreg[d4].z, s[g]);
-                    s[g] = fmaf(q4.w, kreg[d4].w, s[g]);
-                }
-            }
+            for (int g = 0; g < GMAX; g++) s[g] += dpp_f<0xB1>(s[g]);      // the other half of the row
         }
         // tile maxima of all heads with one barrier, then the sums with another
         float sv[GMAX];
@@ -681,8 +705,8 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
             float mNew = fmaxf(m[g], tmax);
             corr[g] = expf(m[g] - mNew);                   // first tile: exp(-inf) = 0
             float pv = active ? expf(sv[g] - mNew) : 0.f;
-            sc[g][tid] = pv;
-            float ws = wave_sum(pv);
+            sc[g][pIdx] = pv;
+            float ws = wave_sum(sub == 0 ? pv : 0.f);
             if (lane == 0) wred[1][g][wave] = ws;
             m[g] = mNew;
         }
@@ -693,24 +717,18 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
             l[g] = l[g] * corr[g] + tsum;
             acc[g].x *= corr[g]; acc[g].y *= corr[g]; acc[g].z *= corr[g]; acc[g].w *= corr[g];
         }
-        // P.V
-        for (int k0 = 0; k0 * TG < tileLen; k0 += VU) {
-            if (k0 > 0) {
+        // P.V: this thread's VU rows of the tile are already in registers
 #pragma unroll
-                for (int u = 0; u < VU; u++) vreg[u] = Vbase[(size_t)min(tile + tg + (k0 + u) * TG, lastRow) * vStride];
-            }
+        for (int u = 0; u < VU; u++) {
+            int tt = tg + u * TG;
+            if (tt < tileLen) {
 #pragma unroll
-            for (int u = 0; u < VU; u++) {
-                int tt = tg + (k0 + u) * TG;
-                if (tt < tileLen) {
-#pragma unroll
-                    for (int g = 0; g < GMAX; g++) {
-                        float w = sc[g][tt];
-                        acc[g].x = fmaf(w, vreg[u].x, acc[g].x);
-                        acc[g].y = fmaf(w, vreg[u].y, acc[g].y);
-                        acc[g].z = fmaf(w, vreg[u].z, acc[g].z);
-                        acc[g].w = fmaf(w, vreg[u].w, acc[g].w);
-                    }
+                for (int g = 0; g < GMAX; g++) {
+                    float w = sc[g][tt];
+                    acc[g].x = fmaf(w, vreg[u].x, acc[g].x);
+                    acc[g].y = fmaf(w, vreg[u].y, acc[g].y);
+                    acc[g].z = fmaf(w, vreg[u].z, acc[g].z);
+                    acc[g].w = fmaf(w, vreg[u].w, acc[g].w);
                 }
             }
         }
@@ -749,29 +767,40 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     if (nsplit == 1) return;
 
     // ---- several splits: the last workgroup of this column combines ----
-    __threadfence();
+    // The partials were stored write-through at agent scope, so "release" is just waiting
+    // for those stores to be acknowledged; a full release fence would also write back the
+    // whole L2 from every workgroup, which serialises them.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
-        int old = __hip_atomic_fetch_add(p.counters + blockIdx.x, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        int old = __hip_atomic_fetch_add(p.counters + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         lastFlag = (old == nsplit - 1);
     }
     __syncthreads();
     if (!lastFlag) return;
-    __threadfence();
-    for (int i = tid; i < gn * HD; i += WG) {
-        int g = i / HD, d = i % HD;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");     // drop cached copies of the other workgroups' partials
+    for (int i = tid; i < gn * LPR; i += WG) {
+        int g = i / LPR, d4 = i % LPR;
         int h = h0 + g;
         const float* pm = p.pm + (size_t)h * p.smax;
         const float* pl = p.pl + (size_t)h * p.smax;
-        float M = ld_agent(pm);
-        for (int s = 1; s < nsplit; s++) M = fmaxf(M, ld_agent(pm + s));
-        float den = 0.f, num = 0.f;
+        const float4* pa = reinterpret_cast<const float4*>(p.pacc + (size_t)h * p.smax * HD) + d4;
+        float M = -INFINITY;
+#pragma unroll 8
+        for (int s = 0; s < nsplit; s++) M = fmaxf(M, pm[s]);
+        float den = 0.f;
+        float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 8
         for (int s = 0; s < nsplit; s++) {
-            float w = expf(ld_agent(pm + s) - M);
-            den += w * ld_agent(pl + s);
-            num += w * ld_agent(p.pacc + ((size_t)h * p.smax + s) * HD + d);
+            float w = expf(pm[s] - M);
+            float4 a = pa[(size_t)s * LPR];
+            den = fmaf(w, pl[s], den);
+            num.x = fmaf(w, a.x, num.x); num.y = fmaf(w, a.y, num.y);
+            num.z = fmaf(w, a.z, num.z); num.w = fmaf(w, a.w, num.w);
         }
-        p.out[(size_t)h * HD + d] = num / den;
+        float4 o;
+        o.x = num.x / den; o.y = num.y / den; o.z = num.z / den; o.w = num.w / den;
+        reinterpret_cast<float4*>(p.out + (size_t)h * HD)[d4] = o;
     }
     if (tid == 0) __hip_atomic_store(p.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -809,7 +838,8 @@ int attention_columns(int nHeads, int nKVHeads, int headsPerWG) {
 
 hipError_t launch_attention(const AttnParams& p, hipStream_t s) {
     if (p.nKVHeads <= 0 || p.nHeads % p.nKVHeads != 0 || p.rowLimit <= 0 || p.smax < 1) return hipErrorInvalidValue;
-    if (p.smax > 1 && (p.splitLen <= 0 || p.splitLen % WG != 0 || !p.counters || !p.pm || !p.pl || !p.pacc)) return hipErrorInvalidValue;
+    const int tile = p.headDim == 128 ? WG / 2 : WG;
+    if (p.smax > 1 && (p.splitLen <= 0 || p.splitLen % tile != 0 || !p.counters || !p.pm || !p.pl || !p.pacc)) return hipErrorInvalidValue;
     if (p.headDim == 64) return launch_attn_hd<64>(p, s);
     if (p.headDim == 128) return launch_attn_hd<128>(p, s);
     return hipErrorInvalidValue;
