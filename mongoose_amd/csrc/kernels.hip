@@ -87,50 +87,34 @@ __device__ __forceinline__ int act_slot4(int k4, int nch) {   // k4 = k/4 -> flo
 // caller has already issued its first weight loads, so the activation latency
 // and the weight latency overlap instead of adding up.
 template <int WF, int PRO>
-__device__ __forceinline__ void stage_activation(const MvParams& p, float4* a4, float* red) {
+__device__ __forceinline__ float stage_activation(const MvParams& p, float4* a4, float* red) {
     const int K4 = p.K >> 2;
     const int nch = p.K / 16;
     const int tid = threadIdx.x;
     if (PRO == PRO_PLAIN) {
         const float4* x4 = reinterpret_cast<const float4*>(p.act);
         for (int i = tid; i < K4; i += WG) a4[act_slot4<WF>(i, nch)] = x4[i];
-    } else if (PRO == PRO_RMS) {
-        // mongoose.cu:145-174 / cpu.go:36-47: x * (1/sqrt(mean(x^2)+eps)) * g
-        constexpr int XR = 4;                       // float4s kept in registers per thread (K <= 4096)
-        const float4* x4 = reinterpret_cast<const float4*>(p.act);
-        const float4* g4 = reinterpret_cast<const float4*>(p.gain);
-        float4 xv[XR], gv[XR];
-#pragma unroll
-        for (int r = 0; r < XR; r++) {
-            int i = tid + r * WG;
-            if (i < K4) { xv[r] = x4[i]; gv[r] = g4[i]; }
-            else { xv[r] = make_float4(0.f, 0.f, 0.f, 0.f); gv[r] = xv[r]; }
-        }
-        float ss = 0.f;
-#pragma unroll
-        for (int r = 0; r < XR; r++) ss += xv[r].x * xv[r].x + xv[r].y * xv[r].y + xv[r].z * xv[r].z + xv[r].w * xv[r].w;
-        for (int i = tid + XR * WG; i < K4; i += WG) {
-            float4 v = x4[i];
-            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-        }
-        float tot = block_sum(ss, red);
-        float rs = 1.0f / sqrtf(tot / (float)p.K + p.eps);
-#pragma unroll
-        for (int r = 0; r < XR; r++) {
-            int i = tid + r * WG;
-            if (i < K4) {
-                float4 o;
-                o.x = xv[r].x * rs * gv[r].x; o.y = xv[r].y * rs * gv[r].y;
-                o.z = xv[r].z * rs * gv[r].z; o.w = xv[r].w * rs * gv[r].w;
-                a4[act_slot4<WF>(i, nch)] = o;
-            }
-        }
-        for (int i = tid + XR * WG; i < K4; i += WG) {
-            float4 v = x4[i], g = g4[i], o;
-            o.x = v.x * rs * g.x; o.y = v.y * rs * g.y; o.z = v.z * rs * g.z; o.w = v.w * rs * g.w;
-            a4[act_slot4<WF>(i, nch)] = o;
-        }
+        __syncthreads();
+        return 1.0f;
     }
+    // RMSNorm (mongoose.cu:145-174 / cpu.go:36-47): x * (1/sqrt(mean(x^2)+eps)) * g.  The vector
+    // staged is x*g; the common factor 1/rms is returned and applied to each finished row, so
+    // nothing waits for the sum of squares before the weights can be consumed: one barrier
+    // covers both the staged vector and the partial sums.
+    const float4* x4 = reinterpret_cast<const float4*>(p.act);
+    const float4* g4 = reinterpret_cast<const float4*>(p.gain);
+    float ss = 0.f;
+    for (int i = tid; i < K4; i += WG) {
+        float4 v = x4[i], g = g4[i], o;
+        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        o.x = v.x * g.x; o.y = v.y * g.y; o.z = v.z * g.z; o.w = v.w * g.w;
+        a4[act_slot4<WF>(i, nch)] = o;
+    }
+    ss = wave_sum(ss);
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    __syncthreads();
+    float tot = (red[0] + red[1]) + (red[2] + red[3]);
+    return 1.0f / sqrtf(tot / (float)p.K + p.eps);
 }
 
 // ---------------------------------------------------------------------------
@@ -338,8 +322,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
 #pragma unroll
     for (int s = 0; s < D; s++) issue(s, s);
 
-    stage_activation<WF, PRO>(p, a4, red);
-    __syncthreads();
+    const float rs = stage_activation<WF, PRO>(p, a4, red);
 
     float myBestV = -INFINITY;
     int myBestI = INT_MAX;
@@ -399,6 +382,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
                             if (p.div127) sc = sc / 127.0f;      // mongoose.cu:1561
                             v *= sc;
                         }
+                        if (PRO == PRO_RMS) v *= rs;
                         v += bi;
                         RowRef rr = resolve_row<NR, EPI>(p, g, lane < NR ? lane : 0);
                         if (EPI == EPI_SWIGLU) {
