@@ -105,6 +105,15 @@ void mongoose_dequant_int8_to_fp32(const void* w_int8, const float* scales, floa
 void mongoose_dequant_q8_rowscale(const void* w_int8, const float* scales, float* out, int rows, int cols, void* stream);
 void mongoose_dequant_q4_0(const void* w_q4_0, float* out, int rows, int cols, void* stream);
 /* kernels.go:24-26, mongoose.cu:356-368. */
+/* out[T,N] (+)= act[T,K] . w[N,K]^T * scales[n] (+ bias[n]) on the matrix cores:
+ * the multi-row form of mongoose_q8_matvec_rowscale, used by the batched
+ * prefill.  The reference's nearest op is its dequantize-then-cuBLAS route
+ * (mongoose_dequant_int8_to_fp32, mongoose.cu:1489, followed by MatMul,
+ * cuda.go:230); here the int8 weights are read directly.  workspace: device
+ * memory of at least 2 * roundup256(T*K*2) bytes for the two bf16 planes of
+ * the split activations.  K a multiple of 32; w and workspace 16-byte aligned. */
+void mongoose_q8_gemm(const float* act, const void* w, const float* scales, const float* bias, float* out, int T, int N,
+                      int K, int accumulate, void* workspace, size_t workspaceBytes, void* stream);
 void mongoose_copy(void* dst, const void* src, size_t bytes, void* stream);
 void mongoose_zero(void* ptr, size_t bytes, void* stream);
 void mongoose_sync(void* stream);
@@ -208,6 +217,23 @@ int mg_timed_decode(mg_ctx* ctx, int token, int pos, int steps, int useGraph, fl
  * event costs the stream a few microseconds, so one class alone is measured
  * closest to its kernel time. */
 int mg_profile_decode(mg_ctx* ctx, int token, int pos, int steps, unsigned classMask, float* classMs, int* classLaunches);
+
+/* Batched prefill -- the multi-token counterpart of the decode step, for the
+ * prompt.  The reference has no batched prompt path: a caller feeds the prompt
+ * through PartialStep one position at a time (cuda_fused_infer.go:392), and it has
+ * GEMM-shaped launches only on its training path (cuda.go:230 MatMul via cuBLAS);
+ * here the seven projections of a layer over nTokens rows are MFMA GEMMs that
+ * read the int8 weights exactly (int8 is exact in bf16) against activations
+ * split into two bf16 terms, so the result stays within ~1e-5 of the
+ * token-by-token path.  Q8 weights only (MG_E_UNSUPPORTED otherwise).
+ * Positions pos0 .. pos0+nTokens-1 of the KV caches are written; the last
+ * position goes through final norm, lm_head and argmax: *nextToken, logitsOut
+ * [vocab] (both optional), and the device step state is left at pos0+nTokens
+ * with that token, so mg_generate-style graph replays can follow.  elapsedMs
+ * (optional) is the device time of the whole call measured with events. */
+int mg_prefill(mg_ctx* ctx, const int* tokens, int nTokens, int pos0, int* nextToken, float* logitsOut, float* elapsedMs);
+/* mg_generate with the prompt run through mg_prefill (nDecode >= 1). */
+int mg_generate_prefill(mg_ctx* ctx, const int* prompt, int nPrompt, int nDecode, int* outTokens);
 
 /* Measurement helper: mean microseconds of one dequantizing matvec launch at
  * shape [N, K] (wf 0 = Q8 per-row scale, 1 = Q4_0 split layout), over `iters`

@@ -3,6 +3,7 @@
 // reference's symbol names and argument order (kernels.go:12-72).
 #include "../../include/mongoose_hip.h"
 #include "kernels.h"
+#include "prefill.h"
 
 #include <atomic>
 #include <cstdio>
@@ -137,6 +138,16 @@ void mongoose_dequant_q8_rowscale(const void* w, const float* scales, float* out
 }
 void mongoose_dequant_q4_0(const void* w, float* out, int rows, int cols, void* stream) {
     note(mg::launch_dequant_q4_0(w, out, rows, cols, S(stream)));
+}
+void mongoose_q8_gemm(const float* act, const void* w, const float* scales, const float* bias, float* out, int T, int N,
+                      int K, int accumulate, void* workspace, size_t workspaceBytes, void* stream) {
+    const size_t plane = ((size_t)T * K * 2 + 255) & ~(size_t)255;
+    if (T < 0 || N < 0 || K <= 0 || K % 32 != 0 || !workspace || workspaceBytes < 2 * plane ||
+        ((uintptr_t)workspace & 15) || ((uintptr_t)w & 15)) { note(hipErrorInvalidValue); return; }
+    void* hi = workspace;
+    void* lo = static_cast<char*>(workspace) + plane;
+    note(mg::launch_split_rows(act, nullptr, 0.f, T, K, hi, lo, S(stream)));
+    note(mg::launch_gemm_q8(hi, lo, w, scales, bias, out, T, N, K, accumulate, S(stream)));
 }
 void mongoose_copy(void* dst, const void* src, size_t bytes, void* stream) {
     if (bytes) note(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, S(stream)));

@@ -70,6 +70,11 @@ public:
     int GraphValidate(int token, int pos, float* maxAbsDiff);                     // cuda_graph.go:554
     int TimedDecode(int token, int pos, int steps, bool useGraph, float* elapsedMs);
     int ProfileDecode(int token, int pos, int steps, unsigned classMask, float* classMs, int* classLaunches);
+    // Batched prefill of nTokens positions starting at pos0 (Q8 weights): fills the KV caches,
+    // leaves the last position's hidden state, logits and greedy token, and the device step
+    // state ready for the decode that follows.
+    int Prefill(const int* tokens, int nTokens, int pos0, int* nextToken, float* logitsOut, float* elapsedMs);
+    int GeneratePrefill(const int* prompt, int nPrompt, int nDecode, int* outTokens);
     uint64_t WeightBytesPerToken() const;
     uint64_t KVBytesAt(int pos) const { return (uint64_t)2 * nLayers * (uint64_t)(pos + 1) * kvDim * 4; }
 
@@ -101,7 +106,12 @@ private:
     int uploadMatQ4(int idx, DevMat& m, int rows, int cols, const uint8_t* raw, size_t nbytes);
     int setVec(int idx, float*& dst, const float* data, size_t n, size_t expect);
     int slotAddr(int idx, char** out);
-    Slab scratch, headSlab;
+    Slab scratch, headSlab, prefillSlab;
+    int prefillCap = 0;             // rows the prefill buffers hold
+    int* pfTokens = nullptr;
+    float *pfX = nullptr, *pfQ = nullptr, *pfK = nullptr, *pfV = nullptr, *pfAttn = nullptr, *pfGate = nullptr, *pfUp = nullptr;
+    void *pfHi = nullptr, *pfLo = nullptr;
+    int ensurePrefill(int rows);
     std::vector<Slab> layerSlabs, kvSlabs;
     size_t slotOff[12] = {0};
     size_t layerSlabBytes = 0;

@@ -3,6 +3,7 @@
 #include "fused_infer.h"
 #include "../../include/mongoose_hip.h"
 #include "host_util.h"
+#include "prefill.h"
 
 #include <cmath>
 #include <cstdio>
@@ -191,6 +192,7 @@ HIPFusedInference::~HIPFusedInference() {
     invalidateGraphs();
     scratch.release();
     headSlab.release();
+    prefillSlab.release();
     for (auto& sl : layerSlabs) sl.release();
     for (auto& sl : kvSlabs) sl.release();
     if (embedTable) (void)hipFree(embedTable);
@@ -827,6 +829,113 @@ int HIPFusedInference::ProfileDecode(int token, int pos, int steps, unsigned cla
     return MG_OK;
 }
 
+// ---------------------------------------------------------------------------
+// Batched prefill (Q8): the layer of the decode step applied to T rows at
+// once, the seven projections as MFMA GEMMs.
+// ---------------------------------------------------------------------------
+int HIPFusedInference::ensurePrefill(int rows) {
+    if (rows <= prefillCap) return MG_OK;
+    HIPCHK(hipStreamSynchronize(stream));
+    prefillSlab.release();
+    prefillCap = 0;
+    const size_t T = ((size_t)rows + 127) / 128 * 128;
+    const size_t wide = (size_t)(ffnDim > dim ? ffnDim : dim);
+    size_t bytes = alignUp256(T * 4) + 3 * alignUp256(T * dim * 4) + 2 * alignUp256(T * kvDim * 4) +
+                   2 * alignUp256(T * ffnDim * 4) + 2 * alignUp256(T * wide * 2) + 16 * 256;
+    int rc = prefillSlab.init(bytes);
+    if (rc) return rc;
+    pfTokens = static_cast<int*>(prefillSlab.take(T * 4));
+    pfX = static_cast<float*>(prefillSlab.take(T * dim * 4));
+    pfQ = static_cast<float*>(prefillSlab.take(T * dim * 4));
+    pfAttn = static_cast<float*>(prefillSlab.take(T * dim * 4));
+    pfK = static_cast<float*>(prefillSlab.take(T * kvDim * 4));
+    pfV = static_cast<float*>(prefillSlab.take(T * kvDim * 4));
+    pfGate = static_cast<float*>(prefillSlab.take(T * ffnDim * 4));
+    pfUp = static_cast<float*>(prefillSlab.take(T * ffnDim * 4));
+    pfHi = prefillSlab.take(T * wide * 2);
+    pfLo = prefillSlab.take(T * wide * 2);
+    if (!pfTokens || !pfX || !pfQ || !pfAttn || !pfK || !pfV || !pfGate || !pfUp || !pfHi || !pfLo) {
+        set_error("prefill slab too small");
+        return MG_E_STATE;
+    }
+    prefillCap = (int)T;
+    return MG_OK;
+}
+
+int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* nextToken, float* logitsOut, float* elapsedMs) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(tokens && nTokens >= 1 && pos0 >= 0 && pos0 + nTokens <= maxSeq, "Prefill: bad token count or position");
+    for (int i = 0; i < nTokens; i++) ARGCHK(tokens[i] >= 0 && tokens[i] < vocabSize, "Prefill: token out of range");
+    int rc = checkReady(this);
+    if (rc) return rc;
+    for (const auto& L : layers) {
+        const DevMat* ms[7] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.gate, &L.up, &L.down};
+        for (const DevMat* m : ms)
+            if (m->kind != WF_Q8) { set_error("Prefill: the GEMM path takes Q8 weights only"); return MG_E_UNSUPPORTED; }
+    }
+    rc = ensurePrefill(nTokens);
+    if (rc) return rc;
+    const int T = nTokens;
+    HIPCHK(hipStreamSynchronize(stream));
+    HIPCHK(hipMemcpy(pfTokens, tokens, sizeof(int) * (size_t)T, hipMemcpyHostToDevice));
+    HIPCHK(hipEventRecord(ev0, stream));
+    if (embedKind == 1 || embedKind == 2) {
+        HIPCHK(launch_embed_rows(embedKind, embedTable, nullptr, pfTokens, pfX, T, dim, vocabSize, stream));
+    } else {
+        if (lmHead.kind != WF_Q8) { set_error("Prefill: tied embedding needs a Q8 lm_head"); return MG_E_UNSUPPORTED; }
+        HIPCHK(launch_embed_rows(0, lmHead.w, lmHead.scales, pfTokens, pfX, T, dim, vocabSize, stream));
+    }
+    for (int l = 0; l < nLayers; l++) {
+        const LayerWeights& L = layers[l];
+        HIPCHK(launch_split_rows(pfX, L.norm1, eps, T, dim, pfHi, pfLo, stream));
+        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.wq.w, L.wq.scales, L.bq, pfQ, T, dim, dim, 0, stream));
+        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.wk.w, L.wk.scales, L.bk, pfK, T, kvDim, dim, 0, stream));
+        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.wv.w, L.wv.scales, L.bv, pfV, T, kvDim, dim, 0, stream));
+        HIPCHK(launch_rope_store_rows(pfQ, pfK, pfV, kCache[l], vCache[l], cosTab, sinTab, pos0, T, dim, kvDim, headDim, stream));
+        AttnParams a{};
+        a.q = pfQ; a.Kc = kCache[l]; a.Vc = vCache[l]; a.posImm = pos0; a.rowLimit = maxSeq;
+        a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
+        a.smax = 1; a.splitLen = 0; a.headsPerWG = 0; a.out = pfAttn;
+        a.batch = T; a.qStride = dim; a.outStride = dim;
+        HIPCHK(launch_attention(a, stream));
+        HIPCHK(launch_split_rows(pfAttn, nullptr, eps, T, dim, pfHi, pfLo, stream));
+        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.wo.w, L.wo.scales, nullptr, pfX, T, dim, dim, 1, stream));
+        HIPCHK(launch_split_rows(pfX, L.norm2, eps, T, dim, pfHi, pfLo, stream));
+        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.gate.w, L.gate.scales, nullptr, pfGate, T, ffnDim, dim, 0, stream));
+        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.up.w, L.up.scales, nullptr, pfUp, T, ffnDim, dim, 0, stream));
+        HIPCHK(launch_swiglu_split(pfGate, pfUp, (size_t)T * ffnDim, pfHi, pfLo, stream));
+        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.down.w, L.down.scales, nullptr, pfX, T, dim, ffnDim, 1, stream));
+    }
+    // the last position continues on the decode path: final norm, lm_head, greedy token, state -> pos0 + T
+    HIPCHK(hipMemcpyAsync(hidden[hiddenIdx], pfX + (size_t)(T - 1) * dim, (size_t)dim * 4, hipMemcpyDeviceToDevice, stream));
+    HIPCHK(launch_set_state(dState, pos0 + T - 1, tokens[T - 1], 0, 0, ropeRef(), stream));
+    rc = enqueueFinal(true);
+    if (rc) return rc;
+    HIPCHK(hipEventRecord(ev1, stream));
+    HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int), hipMemcpyDeviceToHost, stream));
+    HIPCHK(hipStreamSynchronize(stream));
+    if (nextToken) *nextToken = hTokens[0];
+    if (logitsOut) HIPCHK(hipMemcpy(logitsOut, logits, (size_t)vocabSize * 4, hipMemcpyDeviceToHost));
+    if (elapsedMs) HIPCHK(hipEventElapsedTime(elapsedMs, ev0, ev1));
+    return MG_OK;
+}
+
+// Prompt through the GEMM path, then nDecode - 1 graph replays from the device state it left.
+int HIPFusedInference::GeneratePrefill(const int* prompt, int nPrompt, int nDecode, int* outTokens) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(prompt && nPrompt >= 1 && nDecode >= 1 && outTokens, "GeneratePrefill: bad arguments");
+    ARGCHK(nPrompt + nDecode <= maxSeq + 1, "GeneratePrefill: prompt + decode exceeds maxSeq");
+    int rc = GraphCapture();
+    if (rc) return rc;
+    rc = Prefill(prompt, nPrompt, 0, nullptr, nullptr, nullptr);
+    if (rc) return rc;
+    for (int i = 1; i < nDecode; i++) HIPCHK(hipGraphLaunch(execFull, stream));
+    HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int) * (size_t)nDecode, hipMemcpyDeviceToHost, stream));
+    HIPCHK(hipStreamSynchronize(stream));
+    for (int i = 0; i < nDecode; i++) outTokens[i] = hTokens[i];
+    return MG_OK;
+}
+
 }  // namespace mg
 
 // ---------------------------------------------------------------------------
@@ -890,6 +999,12 @@ int mg_timed_decode(mg_ctx* c, int token, int pos, int steps, int useGraph, floa
 }
 int mg_profile_decode(mg_ctx* c, int token, int pos, int steps, unsigned classMask, float* classMs, int* classLaunches) {
     CTX(c); return f->ProfileDecode(token, pos, steps, classMask, classMs, classLaunches);
+}
+int mg_prefill(mg_ctx* c, const int* tokens, int nTokens, int pos0, int* next, float* logitsOut, float* ms) {
+    CTX(c); return f->Prefill(tokens, nTokens, pos0, next, logitsOut, ms);
+}
+int mg_generate_prefill(mg_ctx* c, const int* prompt, int nPrompt, int nDecode, int* out) {
+    CTX(c); return f->GeneratePrefill(prompt, nPrompt, nDecode, out);
 }
 uint64_t mg_weight_bytes_per_token(const mg_ctx* c) { return c && c->f ? c->f->WeightBytesPerToken() : 0; }
 uint64_t mg_kv_bytes_at(const mg_ctx* c, int pos) { return c && c->f ? c->f->KVBytesAt(pos) : 0; }

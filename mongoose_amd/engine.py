@@ -359,6 +359,22 @@ class HIPFusedInference:
         rc = lib.mg_profile_decode(self._h, token, pos, steps, classMask, _fp(ms), _ip(n))
         return rc, ms, n
 
+    def Prefill(self, tokens, pos0=0, wantLogits=False):
+        """Batched prefill of `tokens` at positions pos0.. ; returns (rc, nextToken, logits or None, device ms)."""
+        toks = np.ascontiguousarray(tokens, dtype=np.int32)
+        nxt = ctypes.c_int(-1)
+        ms = ctypes.c_float(0.0)
+        logits = np.zeros(self.vocabSize, dtype=np.float32) if wantLogits else None
+        rc = lib.mg_prefill(self._h, _ip(toks), len(toks), pos0, ctypes.byref(nxt),
+                            _fp(logits) if wantLogits else None, ctypes.byref(ms))
+        return rc, nxt.value, logits, ms.value
+
+    def GeneratePrefill(self, prompt, nDecode):
+        p = np.ascontiguousarray(prompt, dtype=np.int32)
+        out = np.zeros(max(nDecode, 1), dtype=np.int32)
+        rc = lib.mg_generate_prefill(self._h, _ip(p), len(p), nDecode, _ip(out))
+        return rc, out[:nDecode]
+
     def WeightBytesPerToken(self):
         return lib.mg_weight_bytes_per_token(self._h)
 
@@ -407,3 +423,9 @@ class HIPStreamInfer:
         h = _as_f32(embHidden)
         return lib.mg_stream_forward_token(self._h, pos, _fp(h), nLayers, arr,
                                            sizes.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), _fp(logitsOut))
+
+
+def KQ8Gemm(act, w, scales, bias, out, T, N, K, accumulate, workspace, workspaceBytes):
+    """Multi-row form of KQ8MatvecRowScale on the matrix cores (out[T,N] (+)= act[T,K] . w[N,K]^T * scales + bias)."""
+    lib.mongoose_q8_gemm(_p(act), _p(w), _p(scales), _p(bias) if bias is not None else None, _p(out), T, N, K,
+                         1 if accumulate else 0, _p(workspace), workspaceBytes, None)

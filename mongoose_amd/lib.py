@@ -58,6 +58,7 @@ _sig("mongoose_embed_gather", None, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_dequant_int8_to_fp32", None, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_dequant_q8_rowscale", None, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_dequant_q4_0", None, _p, _p, c_int, c_int, _p)
+_sig("mongoose_q8_gemm", None, _p, _p, _p, _p, _p, c_int, c_int, c_int, c_int, _p, c_size_t, _p)
 _sig("mongoose_copy", None, _p, _p, c_size_t, _p)
 _sig("mongoose_zero", None, _p, c_size_t, _p)
 _sig("mongoose_sync", None, _p)
@@ -87,6 +88,8 @@ _sig("mg_graph_launch", c_int, c_void_p, c_int, c_int, _i)
 _sig("mg_graph_validate", c_int, c_void_p, c_int, c_int, _f)
 _sig("mg_timed_decode", c_int, c_void_p, c_int, c_int, c_int, c_int, _f)
 _sig("mg_profile_decode", c_int, c_void_p, c_int, c_int, c_int, ctypes.c_uint, _f, _i)
+_sig("mg_prefill", c_int, c_void_p, _i, c_int, c_int, _i, _f, _f)
+_sig("mg_generate_prefill", c_int, c_void_p, _i, c_int, c_int, _i)
 _sig("mg_bench_matvec", c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _f)
 _sig("mg_weight_bytes_per_token", c_uint64, c_void_p)
 _sig("mg_kv_bytes_at", c_uint64, c_void_p, c_int)

@@ -1,0 +1,156 @@
+"""Batched prefill (MFMA GEMM path) against the token-by-token decode step.
+
+The reference has no batched prompt path: its semantics for a prompt are the
+decode step applied position by position, which is what the oracle does here.
+Bars: last-position logits within 1e-3 relative of the oracle (float path and
+double shadow), greedy tokens identical, and the decode that continues from
+the prefilled KV caches identical to the all-decode run (which checks every
+cache row the prefill wrote).  The GEMM itself is compared with a float64
+product at 2e-5 of the largest output (int8 weights are exact in bf16; the
+two-term bf16 split of an activation leaves 2^-16 relative)."""
+import numpy as np
+import pytest
+
+from mongoose_amd import configs
+from mongoose_amd import engine as E
+from oracle import binding as ob
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+rng = np.random.default_rng(77)
+
+
+def _up(eng, a):
+    return eng.UploadRawBytes(np.ascontiguousarray(a))
+
+
+@pytest.mark.parametrize("T,N,K,acc,bias", [
+    (1, 128, 32, False, False), (5, 100, 64, False, True), (130, 300, 896, True, False),
+    (128, 128, 4864, False, False), (257, 1376, 512, True, True), (512, 1024, 4096, False, False),
+])
+def test_q8_gemm_against_float64(hip, T, N, K, acc, bias):
+    print(f"q8 gemm T={T} N={N} K={K} acc={acc} bias={bias}", flush=True)
+    w = E.synth_normal(9, T * 7 + N, 0.02, (N, K))
+    q, s = ob.quantize_q8(w)
+    a = rng.standard_normal((T, K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32) if bias else None
+    y0 = rng.standard_normal((T, N)).astype(np.float32)
+    plane = (T * K * 2 + 255) // 256 * 256
+    dq, ds, da, dy = _up(hip, q), _up(hip, s), _up(hip, a), _up(hip, y0)
+    db = _up(hip, b) if bias else None
+    ws = hip.UploadRawBytes(np.zeros(2 * plane, np.uint8))
+    E.KQ8Gemm(da, dq, ds, db, dy, T, N, K, acc, ws, 2 * plane)
+    E.KSync()
+    assert E.HIPCheck() == 0
+    got = hip.DownloadRawBytes(dy, T * N * 4).view(np.float32).reshape(T, N)
+    ref = (a.astype(np.float64) @ q.astype(np.float64).T) * s.astype(np.float64)[None, :]
+    if bias:
+        ref = ref + b.astype(np.float64)[None, :]
+    if acc:
+        ref = ref + y0.astype(np.float64)
+    assert H.rel_err(got, ref) < 2e-5
+    # row 0 is also what the decode matvec gives for the same activation
+    if not acc and not bias:
+        mv = ob.q8_matvec(a[0], q, s, shadow=True, threads=4)
+        assert H.rel_err(got[0], mv) < 2e-5
+    for t in (dq, ds, da, dy, ws) + ((db,) if bias else ()):
+        t.Release()
+
+
+def test_q8_gemm_rejects_bad_arguments(hip):
+    t = hip.Zeros([64])
+    E.KQ8Gemm(t, t, t, None, t, 1, 1, 31, False, t, 256)      # K not a multiple of 32
+    E.KSync()
+    assert E.HIPCheck() != 0
+    E.KQ8Gemm(t, t, t, None, t, 1, 1, 32, False, t, 16)       # workspace too small
+    E.KSync()
+    assert E.HIPCheck() != 0
+    assert E.HIPCheck() == 0                                    # the error is reported once
+    t.Release()
+
+
+def _oracle_prompt_logits(m, prompt, shadow):
+    m.orc.reset_kv()
+    logits = None
+    for pos, tok in enumerate(prompt):
+        _, logits, _ = m.orc.decode_token(int(tok), pos, shadow=shadow, want_layers=False)
+    return logits.copy()
+
+
+def _prefill_case(hip, s, seed, nPrompt, nDecode, maxSeq):
+    m = H.Model(s, seed=seed, maxSeq=maxSeq, eng=hip, threads=8)
+    prompt = m.prompt(nPrompt)
+    lg32 = _oracle_prompt_logits(m, prompt, False)
+    lg64 = _oracle_prompt_logits(m, prompt, True)
+    assert m.hip.ResetKV() == 0
+    rc, nxt, logits, ms = m.hip.Prefill(prompt, 0, wantLogits=True)
+    assert rc == 0, E.last_error()
+    assert ms > 0
+    assert H.rel_err(logits, lg64) < 1e-3 and H.rel_err(logits, lg32) < 1e-3
+    assert nxt == int(np.argmax(lg32)) == int(np.argmax(lg64))
+    # the token-by-token GPU path gives the same logits to well inside the bar
+    assert m.hip.ResetKV() == 0
+    lg_dec = np.empty(s.vocab, np.float32)
+    for pos, tok in enumerate(prompt):
+        rc, _ = m.hip.DecodeToken(int(tok), pos, lg_dec if pos == len(prompt) - 1 else None)
+        assert rc == 0, E.last_error()
+    assert H.rel_err(logits, lg_dec) < 1e-4
+    # decode continues from the prefilled caches exactly as from decoded ones
+    toks_ref, _ = H.oracle_generate(m, prompt, nDecode)
+    assert m.hip.ResetKV() == 0
+    rc, toks_dec = m.hip.Generate(prompt, nDecode, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert m.hip.ResetKV() == 0
+    rc, toks_pf = m.hip.GeneratePrefill(prompt, nDecode)
+    assert rc == 0, E.last_error()
+    assert toks_pf.tolist() == toks_dec.tolist() == toks_ref.tolist()
+    return m, prompt, logits
+
+
+def test_prefill_toy_matches_decode(hip):
+    m, prompt, logits = _prefill_case(hip, configs.TOY, seed=1, nPrompt=37, nDecode=24, maxSeq=72)
+    # chunked: 20 positions, then the remaining 17 starting at pos0 = 20
+    assert m.hip.ResetKV() == 0
+    rc, _, _, _ = m.hip.Prefill(prompt[:20], 0)
+    assert rc == 0, E.last_error()
+    rc, nxt2, logits2, _ = m.hip.Prefill(prompt[20:], 20, wantLogits=True)
+    assert rc == 0, E.last_error()
+    assert H.rel_err(logits2, logits) < 1e-5
+    # a single-token prefill is a decode step
+    assert m.hip.ResetKV() == 0
+    rc, n1, l1, _ = m.hip.Prefill(prompt[:1], 0, wantLogits=True)
+    assert rc == 0, E.last_error()
+    assert m.hip.ResetKV() == 0
+    l2 = np.empty(m.s.vocab, np.float32)
+    rc, n2 = m.hip.DecodeToken(int(prompt[0]), 0, l2)
+    assert rc == 0 and n1 == n2 and H.rel_err(l1, l2) < 1e-5
+    m.close()
+
+
+def test_prefill_qwen_shape_with_bias(hip):
+    """Qwen2.5-0.5B shape (GQA 14/2, head 64, QKV bias), 3 layers, 200-token prompt (two row tiles)."""
+    s = H.with_layers(configs.QWEN, 3)
+    m, _, _ = _prefill_case(hip, s, seed=3, nPrompt=200, nDecode=8, maxSeq=256)
+    m.close()
+
+
+def test_prefill_llama3_shape_one_layer(hip):
+    """Llama-3-8B shape (head 128, GQA 32/8), 1 layer, 160-token prompt."""
+    s = H.with_layers(configs.LLAMA3_8B, 1)
+    m, _, _ = _prefill_case(hip, s, seed=4, nPrompt=160, nDecode=4, maxSeq=192)
+    m.close()
+
+
+def test_prefill_errors(hip):
+    s = H.with_layers(configs.TOY, 1)
+    m = H.Model(s, seed=2, maxSeq=32, eng=hip, oracle=False)
+    assert m.hip.Prefill(np.zeros(33, np.int32), 0)[0] == -2          # longer than maxSeq
+    assert m.hip.Prefill(np.zeros(4, np.int32), 30)[0] == -2          # runs past maxSeq
+    assert m.hip.Prefill(np.array([s.vocab], np.int32), 0)[0] == -2   # token out of range
+    assert m.hip.Prefill(np.zeros(4, np.int32), 0)[0] == 0
+    m.close()
+    sq = H.with_layers(configs.QWEN_Q4, 1)
+    mq = H.Model(sq, seed=2, maxSeq=32, eng=hip, oracle=False)
+    assert mq.hip.Prefill(np.zeros(4, np.int32), 0)[0] == -5          # Q4_0 weights: unsupported
+    assert "Q8" in E.last_error()
+    mq.close()
