@@ -158,6 +158,8 @@ def main():
                     help="start the timed decode at this position (KV rows between the prompt and it are zeros): long-context timing")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run three 256 MiB device copies (a kernel of known traffic, to scale rocprofv3 --pmc counters)")
+    ap.add_argument("--prefill", type=int, default=0,
+                    help="also time a batched prefill of this many prompt tokens (Q8 configurations; extra 'prefill' object)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
@@ -175,7 +177,7 @@ def main():
         sys.exit(1)
     K, W = args.steps, max(args.warmup, 1)
     P0 = max(args.context, W)                      # position of the first timed step
-    maxSeq = P0 + K + args.profile_steps + 8
+    maxSeq = max(P0 + K + args.profile_steps + 8, args.prefill)
     t_load = time.perf_counter()
     f = load_model(E, np, s, args.seed, maxSeq, eng)
     t_load = time.perf_counter() - t_load
@@ -252,6 +254,25 @@ def main():
         a.Release()
         b.Release()
 
+    prefill = None
+    if args.prefill > 0 and s.fmt == "q8":
+        ptoks = E.synth_tokens(args.seed, 20_000_003, s.vocab, args.prefill)
+        times = []
+        for _ in range(4):                              # first call allocates the row buffers
+            assert f.ResetKV() == 0
+            rc, _, _, pms = f.Prefill(ptoks, 0)
+            assert rc == 0, E.last_error()
+            times.append(pms)
+        pms = min(times[1:])
+        macs = sum((mat(n, k) - 4 * n) for n, k in
+                   [(s.dim, s.dim), (kv, s.dim), (kv, s.dim), (s.dim, s.dim), (s.ffnDim, s.dim), (s.ffnDim, s.dim),
+                    (s.dim, s.ffnDim)]) * s.nLayers
+        flops = 2.0 * macs * args.prefill
+        prefill = {"tokens": args.prefill, "ms": round(pms, 3), "tok_per_s": round(args.prefill / (pms * 1e-3), 1),
+                   "model_TFLOPs": round(flops / (pms * 1e-3) / 1e12, 2),
+                   "mfma_TFLOPs_issued": round(2 * flops / (pms * 1e-3) / 1e12, 2),
+                   "note": "model flops = 2*T*weights of the layer projections; each is issued twice (bf16 hi and lo activation terms)"}
+
     cpu = None
     if args.cpu_budget > 0:
         cpu = cpu_baseline(E, np, s, args.seed, prompt, toks, args.cpu_budget)
@@ -268,7 +289,7 @@ def main():
                    "kv_heads": s.nKVHeads, "ffn": s.ffnDim, "vocab": s.vocab, "graph_replay": use_graph},
         "step_bytes": int(step_bytes), "step_GBps": round(step_bytes * toks_per_s / 1e9, 1),
         "step_roofline_frac": round(step_bytes * toks_per_s / 1e9 / HBM_PEAK_GBS, 4),
-        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
+        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu, "prefill": prefill,
         "load_s": round(t_load, 1), "device": eng.Name(),
     }
     f.Close()

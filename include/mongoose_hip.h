@@ -110,8 +110,9 @@ void mongoose_dequant_q4_0(const void* w_q4_0, float* out, int rows, int cols, v
  * prefill.  The reference's nearest op is its dequantize-then-cuBLAS route
  * (mongoose_dequant_int8_to_fp32, mongoose.cu:1489, followed by MatMul,
  * cuda.go:230); here the int8 weights are read directly.  workspace: device
- * memory of at least 2 * roundup256(T*K*2) bytes for the two bf16 planes of
- * the split activations.  K a multiple of 32; w and workspace 16-byte aligned. */
+ * memory of at least 4 * roundup(T,128) * roundup(K,64) bytes for the two bf16
+ * planes of the split activations.  K a multiple of 32; w and workspace
+ * 16-byte aligned. */
 void mongoose_q8_gemm(const float* act, const void* w, const float* scales, const float* bias, float* out, int T, int N,
                       int K, int accumulate, void* workspace, size_t workspaceBytes, void* stream);
 void mongoose_copy(void* dst, const void* src, size_t bytes, void* stream);

@@ -141,13 +141,18 @@ void mongoose_dequant_q4_0(const void* w, float* out, int rows, int cols, void* 
 }
 void mongoose_q8_gemm(const float* act, const void* w, const float* scales, const float* bias, float* out, int T, int N,
                       int K, int accumulate, void* workspace, size_t workspaceBytes, void* stream) {
-    const size_t plane = ((size_t)T * K * 2 + 255) & ~(size_t)255;
+    const size_t plane = mg::split_plane_elems(T, K > 0 ? K : 64) * 2;     // a multiple of 16 KB
     if (T < 0 || N < 0 || K <= 0 || K % 32 != 0 || !workspace || workspaceBytes < 2 * plane ||
         ((uintptr_t)workspace & 15) || ((uintptr_t)w & 15)) { note(hipErrorInvalidValue); return; }
     void* hi = workspace;
     void* lo = static_cast<char*>(workspace) + plane;
     note(mg::launch_split_rows(act, nullptr, 0.f, T, K, hi, lo, S(stream)));
-    note(mg::launch_gemm_q8(hi, lo, w, scales, bias, out, T, N, K, accumulate, S(stream)));
+    if (T == 0 || N == 0) return;
+    mg::GemmParams g{};
+    g.seg[0] = mg::GemmSeg{static_cast<const signed char*>(w), scales, bias, out, N, 0};
+    g.nseg = 1; g.T = T; g.K = K;
+    g.Ahi = static_cast<const unsigned short*>(hi); g.Alo = static_cast<const unsigned short*>(lo);
+    note(mg::launch_gemm_q8(g, accumulate, S(stream)));
 }
 void mongoose_copy(void* dst, const void* src, size_t bytes, void* stream) {
     if (bytes) note(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, S(stream)));

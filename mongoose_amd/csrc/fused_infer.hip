@@ -839,9 +839,9 @@ int HIPFusedInference::ensurePrefill(int rows) {
     prefillSlab.release();
     prefillCap = 0;
     const size_t T = ((size_t)rows + 127) / 128 * 128;
-    const size_t wide = (size_t)(ffnDim > dim ? ffnDim : dim);
+    const size_t plane = split_plane_elems((int)T, ffnDim > dim ? ffnDim : dim) * 2;
     size_t bytes = alignUp256(T * 4) + 3 * alignUp256(T * dim * 4) + 2 * alignUp256(T * kvDim * 4) +
-                   2 * alignUp256(T * ffnDim * 4) + 2 * alignUp256(T * wide * 2) + 16 * 256;
+                   2 * alignUp256(T * ffnDim * 4) + 2 * alignUp256(plane) + 16 * 256;
     int rc = prefillSlab.init(bytes);
     if (rc) return rc;
     pfTokens = static_cast<int*>(prefillSlab.take(T * 4));
@@ -852,8 +852,8 @@ int HIPFusedInference::ensurePrefill(int rows) {
     pfV = static_cast<float*>(prefillSlab.take(T * kvDim * 4));
     pfGate = static_cast<float*>(prefillSlab.take(T * ffnDim * 4));
     pfUp = static_cast<float*>(prefillSlab.take(T * ffnDim * 4));
-    pfHi = prefillSlab.take(T * wide * 2);
-    pfLo = prefillSlab.take(T * wide * 2);
+    pfHi = prefillSlab.take(plane);
+    pfLo = prefillSlab.take(plane);
     if (!pfTokens || !pfX || !pfQ || !pfAttn || !pfK || !pfV || !pfGate || !pfUp || !pfHi || !pfLo) {
         set_error("prefill slab too small");
         return MG_E_STATE;
@@ -887,10 +887,15 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
     }
     for (int l = 0; l < nLayers; l++) {
         const LayerWeights& L = layers[l];
+        auto seg = [](const DevMat& m, const float* bias, float* y) {
+            return GemmSeg{static_cast<const signed char*>(m.w), m.scales, bias, y, m.rows, 0};
+        };
+        GemmParams g{};
+        g.T = T; g.Ahi = static_cast<const unsigned short*>(pfHi); g.Alo = static_cast<const unsigned short*>(pfLo);
         HIPCHK(launch_split_rows(pfX, L.norm1, eps, T, dim, pfHi, pfLo, stream));
-        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.wq.w, L.wq.scales, L.bq, pfQ, T, dim, dim, 0, stream));
-        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.wk.w, L.wk.scales, L.bk, pfK, T, kvDim, dim, 0, stream));
-        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.wv.w, L.wv.scales, L.bv, pfV, T, kvDim, dim, 0, stream));
+        g.K = dim; g.nseg = 3;
+        g.seg[0] = seg(L.wq, L.bq, pfQ); g.seg[1] = seg(L.wk, L.bk, pfK); g.seg[2] = seg(L.wv, L.bv, pfV);
+        HIPCHK(launch_gemm_q8(g, 0, stream));
         HIPCHK(launch_rope_store_rows(pfQ, pfK, pfV, kCache[l], vCache[l], cosTab, sinTab, pos0, T, dim, kvDim, headDim, stream));
         AttnParams a{};
         a.q = pfQ; a.Kc = kCache[l]; a.Vc = vCache[l]; a.posImm = pos0; a.rowLimit = maxSeq;
@@ -899,12 +904,14 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
         a.batch = T; a.qStride = dim; a.outStride = dim;
         HIPCHK(launch_attention(a, stream));
         HIPCHK(launch_split_rows(pfAttn, nullptr, eps, T, dim, pfHi, pfLo, stream));
-        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.wo.w, L.wo.scales, nullptr, pfX, T, dim, dim, 1, stream));
+        g.K = dim; g.nseg = 1; g.seg[0] = seg(L.wo, nullptr, pfX);
+        HIPCHK(launch_gemm_q8(g, 1, stream));
         HIPCHK(launch_split_rows(pfX, L.norm2, eps, T, dim, pfHi, pfLo, stream));
-        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.gate.w, L.gate.scales, nullptr, pfGate, T, ffnDim, dim, 0, stream));
-        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.up.w, L.up.scales, nullptr, pfUp, T, ffnDim, dim, 0, stream));
-        HIPCHK(launch_swiglu_split(pfGate, pfUp, (size_t)T * ffnDim, pfHi, pfLo, stream));
-        HIPCHK(launch_gemm_q8(pfHi, pfLo, L.down.w, L.down.scales, nullptr, pfX, T, dim, ffnDim, 1, stream));
+        g.K = dim; g.nseg = 2; g.seg[0] = seg(L.gate, nullptr, pfGate); g.seg[1] = seg(L.up, nullptr, pfUp);
+        HIPCHK(launch_gemm_q8(g, 0, stream));
+        HIPCHK(launch_swiglu_split(pfGate, pfUp, T, ffnDim, pfHi, pfLo, stream));
+        g.K = ffnDim; g.nseg = 1; g.seg[0] = seg(L.down, nullptr, pfX);
+        HIPCHK(launch_gemm_q8(g, 1, stream));
     }
     // the last position continues on the decode path: final norm, lm_head, greedy token, state -> pos0 + T
     HIPCHK(hipMemcpyAsync(hidden[hiddenIdx], pfX + (size_t)(T - 1) * dim, (size_t)dim * 4, hipMemcpyDeviceToDevice, stream));

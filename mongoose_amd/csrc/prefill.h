@@ -5,18 +5,30 @@
 
 namespace mg {
 
-// Rows of `in` [T,K] (RMS-normalised with `gain` when it is not NULL) split into two bf16 planes, a = hi + lo.
+// Elements of one bf16 plane of split activations for T rows of K (blocks of 128 rows x 64 k).
+inline size_t split_plane_elems(int T, int K) { return (size_t)((T + 127) / 128) * 128 * (size_t)((K + 63) / 64) * 64; }
+// Rows of `in` [T,K] (RMS-normalised with `gain` when it is not NULL) split into two bf16 planes, a = hi + lo,
+// stored block by block in the order the GEMM reads them.
 hipError_t launch_split_rows(const float* in, const float* gain, float eps, int T, int K, void* hi, void* lo, hipStream_t s);
-// silu(gate) * up over n elements, written as the hi/lo split.
-hipError_t launch_swiglu_split(const float* gate, const float* up, size_t n, void* hi, void* lo, hipStream_t s);
+// silu(gate) * up over [T,K], written as the hi/lo split.
+hipError_t launch_swiglu_split(const float* gate, const float* up, int T, int K, void* hi, void* lo, hipStream_t s);
 // RoPE on q rows in place; rotated k rows and v rows stored into cache rows pos0 .. pos0+T-1.
 hipError_t launch_rope_store_rows(float* q, const float* k, const float* v, float* Kc, float* Vc, const float* cosTab,
                                   const float* sinTab, int pos0, int T, int dim, int kvDim, int headDim, hipStream_t s);
 // Embedding rows of T tokens: kind 0 = Q8 row * scale, 1 = fp16 table, 2 = fp32 table.
 hipError_t launch_embed_rows(int kind, const void* table, const float* scales, const int* tokens, float* x, int T, int dim,
                              int vocab, hipStream_t s);
-// Y[T,N] (+)= (Ahi + Alo)[T,K] . W[N,K]^T * scales[n] (+ bias[n]); K a multiple of 32.
-hipError_t launch_gemm_q8(const void* Ahi, const void* Alo, const void* W, const float* scales, const float* bias, float* Y,
-                          int T, int N, int K, int residual, hipStream_t s);
+// One launch: for each of up to three weight matrices, Y[T,N] (+)= (Ahi + Alo)[T,K] . W[N,K]^T * scales[n] (+ bias[n]).
+// K a multiple of 32; W, Ahi, Alo 16-byte aligned; Ahi/Alo in the blocked layout of launch_split_rows.
+struct GemmSeg { const signed char* W; const float* scales; const float* bias; float* Y; int N; int tile0; };
+struct GemmParams {
+    GemmSeg seg[3];
+    int nseg;
+    const unsigned short* Ahi;
+    const unsigned short* Alo;
+    int T, K;
+    int nTiles;       // filled by the launcher
+};
+hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s);
 
 }  // namespace mg

@@ -37,6 +37,14 @@ __device__ __forceinline__ float block_sum256(float v, float* red) {
     return t;
 }
 
+// The split activations are stored in the order the GEMM walks them: blocks of
+// 128 rows x 64 k (16 KB per plane), block (t/128, k/64) at ((t/128)*ceil(K/64) + k/64) * 8192
+// elements, so one K step of a workgroup is one contiguous read.
+__device__ __forceinline__ size_t tiled_index(int t, int k, int K) {
+    const int ksteps = (K + 63) >> 6;
+    return ((size_t)(t >> 7) * ksteps + (k >> 6)) * 8192 + (size_t)(t & 127) * 64 + (k & 63);
+}
+
 // Row-wise: optional RMSNorm (x * 1/sqrt(mean(x^2)+eps) * g, the decode step's
 // order of operations), then the hi/lo bf16 split.  One workgroup per row.
 __global__ __launch_bounds__(PWG) void split_rows_kernel(const float* in, const float* gain, float eps, int K,
@@ -53,8 +61,9 @@ __global__ __launch_bounds__(PWG) void split_rows_kernel(const float* in, const 
     for (int i = threadIdx.x; i < K; i += PWG) {
         float a = gain ? x[i] * rs * gain[i] : x[i];
         unsigned short h = f32_to_bf16_rne(a);
-        hi[(size_t)blockIdx.x * K + i] = h;
-        lo[(size_t)blockIdx.x * K + i] = f32_to_bf16_rne(a - bf16_to_f32(h));
+        const size_t o = tiled_index(blockIdx.x, i, K);
+        hi[o] = h;
+        lo[o] = f32_to_bf16_rne(a - bf16_to_f32(h));
     }
 }
 hipError_t launch_split_rows(const float* in, const float* gain, float eps, int T, int K, void* hi, void* lo, hipStream_t s) {
@@ -65,18 +74,20 @@ hipError_t launch_split_rows(const float* in, const float* gain, float eps, int 
 }
 
 // SiLU(gate)*up (mongoose.cu:949-956) over [T, n], written as the hi/lo split the down GEMM reads.
-__global__ void swiglu_split_kernel(const float* gate, const float* up, size_t n, unsigned short* hi, unsigned short* lo) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    float g = gate[i];
-    float a = g * (1.0f / (1.0f + expf(-g))) * up[i];
+__global__ void swiglu_split_kernel(const float* gate, const float* up, int K, unsigned short* hi, unsigned short* lo) {
+    const int t = blockIdx.y;
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= K) return;
+    float g = gate[(size_t)t * K + k];
+    float a = g * (1.0f / (1.0f + expf(-g))) * up[(size_t)t * K + k];
     unsigned short h = f32_to_bf16_rne(a);
-    hi[i] = h;
-    lo[i] = f32_to_bf16_rne(a - bf16_to_f32(h));
+    const size_t o = tiled_index(t, k, K);
+    hi[o] = h;
+    lo[o] = f32_to_bf16_rne(a - bf16_to_f32(h));
 }
-hipError_t launch_swiglu_split(const float* gate, const float* up, size_t n, void* hi, void* lo, hipStream_t s) {
-    if (n == 0) return hipSuccess;
-    hipLaunchKernelGGL(swiglu_split_kernel, dim3((unsigned)((n + PWG - 1) / PWG)), dim3(PWG), 0, s, gate, up, n,
+hipError_t launch_swiglu_split(const float* gate, const float* up, int T, int K, void* hi, void* lo, hipStream_t s) {
+    if (T <= 0 || K <= 0) return hipSuccess;
+    hipLaunchKernelGGL(swiglu_split_kernel, dim3((unsigned)((K + PWG - 1) / PWG), (unsigned)T), dim3(PWG), 0, s, gate, up, K,
                        static_cast<unsigned short*>(hi), static_cast<unsigned short*>(lo));
     return hipGetLastError();
 }
@@ -133,105 +144,137 @@ hipError_t launch_embed_rows(int kind, const void* table, const float* scales, c
 }
 
 // ---------------------------------------------------------------------------
-// GEMM on v_mfma_f32_32x32x8_bf16_1k.  Workgroup tile 128 (T) x 128 (N), K in
-// steps of 32; four waves as 2x2, each 64x64 = 2x2 MFMA blocks, hi and lo
-// activations against the same weight fragment.  Fragment layouts (lane l):
-//   A: row l%32, k = 4*(l/32)..+3        B: col l%32, k = 4*(l/32)..+3
+// GEMM on v_mfma_f32_32x32x16_bf16.  Workgroup tile BM (T) x 128 (N), K in
+// steps of 64; four waves as 2x2, each (BM/2)x64 = (BM/64)x2 MFMA blocks, the
+// hi and the lo activation term against the same weight fragment.  Fragment
+// layouts (lane l):
+//   A: row l%32, k = 8*(l/32)..+7        B: col l%32, k = 8*(l/32)..+7
 //   C: col l%32, rows 8*(i/4) + 4*(l/32) + i%4 for i = 0..15
+// Up to three weight matrices (q/k/v, gate/up) share one launch.  Workgroups
+// that share a weight tile are placed on one XCD (ids congruent mod 8), so the
+// tile comes into that XCD's L2 once.
 // ---------------------------------------------------------------------------
-constexpr int BM = 128, BN = 128, BK = 32;
-constexpr int A_STRIDE = 40;   // bf16 per LDS row (80 bytes: 16-byte aligned, spreads banks)
-constexpr int B_STRIDE = 48;   // bytes per LDS row of int8 weights
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+constexpr int BN = 128, BK = 64;
+constexpr int A_STRIDE = BK + 8;    // bf16 per LDS row (144 bytes)
+constexpr int B_STRIDE = BK + 16;   // bytes per LDS row of int8 weights (80)
 
-template <int EPI>   // 0: Y = acc*scale (+bias)   1: Y += acc*scale (residual in place)
-__global__ __launch_bounds__(PWG) void gemm_q8_bf16x2_kernel(const unsigned short* Ahi, const unsigned short* Alo,
-                                                            const signed char* W, const float* scales, const float* bias,
-                                                            float* Y, int T, int N, int K) {
+__device__ __forceinline__ unsigned pack_bf16_exact(float lo, float hi) {
+    // both floats hold small integers: their low 16 bits are zero, truncation is exact
+    return (__builtin_bit_cast(unsigned, lo) >> 16) | (__builtin_bit_cast(unsigned, hi) & 0xffff0000u);
+}
+
+template <int BM, int EPI>   // EPI 0: Y = acc*scale (+bias)   1: Y += acc*scale (residual in place)
+__global__ __launch_bounds__(PWG) void gemm_q8_bf16x2_kernel(GemmParams p) {
+    constexpr int MI = BM / 64;                  // 32-row MFMA blocks per wave
+    constexpr int AR = BM / 32;                  // 16-byte segments per thread and A plane (BM*8 segments / 256)
     __shared__ __attribute__((aligned(16))) unsigned short sAh[BM * A_STRIDE];
     __shared__ __attribute__((aligned(16))) unsigned short sAl[BM * A_STRIDE];
     __shared__ __attribute__((aligned(16))) signed char sB[BN * B_STRIDE];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int numM = (p.T + BM - 1) / BM;
+    const int L = blockIdx.x;
+    const int grp = L / (8 * numM), rem = L % (8 * numM);
+    const int nTile = grp * 8 + (rem & 7), mTile = rem >> 3;
+    if (nTile >= p.nTiles) return;
+    int sgi = 0;
+    if (p.nseg > 1 && nTile >= p.seg[1].tile0) sgi = 1;
+    if (p.nseg > 2 && nTile >= p.seg[2].tile0) sgi = 2;
+    const GemmSeg sg = p.seg[sgi];
+    const int N = sg.N, K = p.K, T = p.T;
+    const int m0 = mTile * BM, n0 = (nTile - sg.tile0) * BN;
 
-    // global -> LDS assignment: A: row = tid/4 + 64*r, 16-byte segment tid%4 ; B: row = tid/2, segment tid%2
-    const int aRow = tid >> 2, aSeg = tid & 3;
-    const int bRow = tid >> 1, bSeg = tid & 1;
-    const int bRowG = min(n0 + bRow, N - 1);
-
-    float16_t acc[2][2];
+    // global -> LDS: A row = tid/8 + 32*r, segment tid%8 (8 bf16) ; B row = tid/4 + 64*r, segment tid%4 (16 int8)
+    const int aRow = tid >> 3, aSeg = tid & 7;
+    const int bRow = tid >> 2, bSeg = tid & 3;
+    const unsigned short* aHiP[AR]; const unsigned short* aLoP[AR];
+    const int ksteps = (K + BK - 1) / BK;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int r = 0; r < AR; r++) {         // rows past T exist in the padded planes; their results are dropped
+        const int row = m0 + aRow + 32 * r;
+        const size_t o = (size_t)(row >> 7) * ksteps * 8192 + (size_t)(row & 127) * 64 + aSeg * 8;
+        aHiP[r] = p.Ahi + o;
+        aLoP[r] = p.Alo + o;
+    }
+    const signed char* bP[2];
+#pragma unroll
+    for (int r = 0; r < 2; r++) bP[r] = sg.W + (size_t)min(n0 + bRow + 64 * r, N - 1) * K + bSeg * 16;
+
+    float16_t acc[MI][2];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-    int4 gAh[2], gAl[2], gB;
-    auto gload = [&](int k0) {
+    int4 gAh[AR], gAl[AR], gB[2];
+    const int4 zero4 = make_int4(0, 0, 0, 0);
+    auto gload = [&](int k0) {       // K is a multiple of 32: a last half step reads zeros past the end
+        const bool okA = k0 + aSeg * 8 < K, okB = k0 + bSeg * 16 < K;
 #pragma unroll
-        for (int r = 0; r < 2; r++) {
-            int row = min(m0 + aRow + 64 * r, T - 1);
-            gAh[r] = *reinterpret_cast<const int4*>(Ahi + (size_t)row * K + k0 + aSeg * 8);
-            gAl[r] = *reinterpret_cast<const int4*>(Alo + (size_t)row * K + k0 + aSeg * 8);
+        for (int r = 0; r < AR; r++) {
+            gAh[r] = okA ? *reinterpret_cast<const int4*>(aHiP[r] + (size_t)k0 * 128) : zero4;   // 8192 elements per K step
+            gAl[r] = okA ? *reinterpret_cast<const int4*>(aLoP[r] + (size_t)k0 * 128) : zero4;
         }
-        gB = *reinterpret_cast<const int4*>(W + (size_t)bRowG * K + k0 + bSeg * 16);
+#pragma unroll
+        for (int r = 0; r < 2; r++) gB[r] = okB ? *reinterpret_cast<const int4*>(bP[r] + k0) : zero4;
     };
     gload(0);
     for (int k0 = 0; k0 < K; k0 += BK) {
-        __syncthreads();                       // previous step's fragments are consumed
+        __syncthreads();                       // the previous step's fragments are consumed
 #pragma unroll
-        for (int r = 0; r < 2; r++) {
-            *reinterpret_cast<int4*>(&sAh[(aRow + 64 * r) * A_STRIDE + aSeg * 8]) = gAh[r];
-            *reinterpret_cast<int4*>(&sAl[(aRow + 64 * r) * A_STRIDE + aSeg * 8]) = gAl[r];
+        for (int r = 0; r < AR; r++) {
+            *reinterpret_cast<int4*>(&sAh[(aRow + 32 * r) * A_STRIDE + aSeg * 8]) = gAh[r];
+            *reinterpret_cast<int4*>(&sAl[(aRow + 32 * r) * A_STRIDE + aSeg * 8]) = gAl[r];
         }
-        *reinterpret_cast<int4*>(&sB[bRow * B_STRIDE + bSeg * 16]) = gB;
+#pragma unroll
+        for (int r = 0; r < 2; r++) *reinterpret_cast<int4*>(&sB[(bRow + 64 * r) * B_STRIDE + bSeg * 16]) = gB[r];
         __syncthreads();
         if (k0 + BK < K) gload(k0 + BK);       // next tile in flight while this one is multiplied
 #pragma unroll
-        for (int ks = 0; ks < BK / 8; ks++) {
-            const int kk = ks * 8 + 4 * (lane >> 5);
-            short4_t b[2];
+        for (int ks = 0; ks < BK / 16; ks++) {
+            const int kk = ks * 16 + 8 * (lane >> 5);
+            bf16x8_t b[2];
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                int w = *reinterpret_cast<const int*>(&sB[(wn * 64 + j * 32 + (lane & 31)) * B_STRIDE + kk]);
-                // int8 -> float -> bf16: exact, the float's low 16 bits are zero
-                unsigned f0 = __builtin_bit_cast(unsigned, (float)(int)(signed char)(w & 0xff));
-                unsigned f1 = __builtin_bit_cast(unsigned, (float)(int)(signed char)((w >> 8) & 0xff));
-                unsigned f2 = __builtin_bit_cast(unsigned, (float)(int)(signed char)((w >> 16) & 0xff));
-                unsigned f3 = __builtin_bit_cast(unsigned, (float)(w >> 24));
-                b[j][0] = (short)(f0 >> 16); b[j][1] = (short)(f1 >> 16);
-                b[j][2] = (short)(f2 >> 16); b[j][3] = (short)(f3 >> 16);
+                int2 w = *reinterpret_cast<const int2*>(&sB[(wn * 64 + j * 32 + (lane & 31)) * B_STRIDE + kk]);
+                uint4 u;
+                u.x = pack_bf16_exact((float)(signed char)(w.x), (float)(signed char)(w.x >> 8));
+                u.y = pack_bf16_exact((float)(signed char)(w.x >> 16), (float)(w.x >> 24));
+                u.z = pack_bf16_exact((float)(signed char)(w.y), (float)(signed char)(w.y >> 8));
+                u.w = pack_bf16_exact((float)(signed char)(w.y >> 16), (float)(w.y >> 24));
+                b[j] = __builtin_bit_cast(bf16x8_t, u);
             }
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const int arow = (wm * 64 + i * 32 + (lane & 31)) * A_STRIDE + kk;
-                short4_t ah = *reinterpret_cast<const short4_t*>(&sAh[arow]);
-                short4_t al = *reinterpret_cast<const short4_t*>(&sAl[arow]);
+            for (int i = 0; i < MI; i++) {
+                const int arow = (wm * (BM / 2) + i * 32 + (lane & 31)) * A_STRIDE + kk;
+                bf16x8_t ah = *reinterpret_cast<const bf16x8_t*>(&sAh[arow]);
+                bf16x8_t al = *reinterpret_cast<const bf16x8_t*>(&sAl[arow]);
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(ah, b[j], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(al, b[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, b[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, b[j], acc[i][j], 0, 0, 0);
                 }
             }
         }
     }
-    // epilogue
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const int n = n0 + wn * 64 + j * 32 + (lane & 31);
         if (n >= N) continue;
-        const float sc = scales[n];
-        const float bi = bias ? bias[n] : 0.f;
+        const float sc = sg.scales[n];
+        const float bi = sg.bias ? sg.bias[n] : 0.f;
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < MI; i++) {
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-                const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                 if (m < T) {
                     float v = acc[i][j][e] * sc + bi;
-                    float* dst = Y + (size_t)m * N + n;
+                    float* dst = sg.Y + (size_t)m * N + n;
                     if (EPI == 1) v = *dst + v;
                     *dst = v;
                 }
@@ -240,17 +283,28 @@ __global__ __launch_bounds__(PWG) void gemm_q8_bf16x2_kernel(const unsigned shor
     }
 }
 
-hipError_t launch_gemm_q8(const void* Ahi, const void* Alo, const void* W, const float* scales, const float* bias, float* Y,
-                          int T, int N, int K, int residual, hipStream_t s) {
-    if (T <= 0 || N <= 0) return hipSuccess;
-    if (K % BK != 0) return hipErrorInvalidValue;
-    dim3 grid((N + BN - 1) / BN, (T + BM - 1) / BM);
-    if (residual)
-        hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<1>), grid, dim3(PWG), 0, s, static_cast<const unsigned short*>(Ahi),
-                           static_cast<const unsigned short*>(Alo), static_cast<const signed char*>(W), scales, bias, Y, T, N, K);
-    else
-        hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<0>), grid, dim3(PWG), 0, s, static_cast<const unsigned short*>(Ahi),
-                           static_cast<const unsigned short*>(Alo), static_cast<const signed char*>(W), scales, bias, Y, T, N, K);
+hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s) {
+    if (p.T <= 0 || p.nseg < 1 || p.nseg > 3) return p.T <= 0 ? hipSuccess : hipErrorInvalidValue;
+    if (p.K <= 0 || p.K % 32 != 0) return hipErrorInvalidValue;
+    int tiles = 0;
+    for (int i = 0; i < p.nseg; i++) {
+        if (p.seg[i].N <= 0) return hipErrorInvalidValue;
+        p.seg[i].tile0 = tiles;
+        tiles += (p.seg[i].N + BN - 1) / BN;
+    }
+    p.nTiles = tiles;
+    // 128-row tiles once they fill the chip, 64-row tiles below that
+    const int numM128 = (p.T + 127) / 128;
+    const bool big = (long long)numM128 * tiles >= 512;
+    const int numM = big ? numM128 : (p.T + 63) / 64;
+    dim3 grid((unsigned)(((tiles + 7) / 8) * 8 * numM));
+    if (big) {
+        if (residual) hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<128, 1>), grid, dim3(PWG), 0, s, p);
+        else hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<128, 0>), grid, dim3(PWG), 0, s, p);
+    } else {
+        if (residual) hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<64, 1>), grid, dim3(PWG), 0, s, p);
+        else hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<64, 0>), grid, dim3(PWG), 0, s, p);
+    }
     return hipGetLastError();
 }
 

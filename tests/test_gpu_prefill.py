@@ -35,7 +35,7 @@ def test_q8_gemm_against_float64(hip, T, N, K, acc, bias):
     a = rng.standard_normal((T, K)).astype(np.float32)
     b = rng.standard_normal(N).astype(np.float32) if bias else None
     y0 = rng.standard_normal((T, N)).astype(np.float32)
-    plane = (T * K * 2 + 255) // 256 * 256
+    plane = 2 * ((T + 127) // 128 * 128) * ((K + 63) // 64 * 64)
     dq, ds, da, dy = _up(hip, q), _up(hip, s), _up(hip, a), _up(hip, y0)
     db = _up(hip, b) if bias else None
     ws = hip.UploadRawBytes(np.zeros(2 * plane, np.uint8))
