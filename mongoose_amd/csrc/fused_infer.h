@@ -111,6 +111,7 @@ private:
     int* pfTokens = nullptr;
     float *pfX = nullptr, *pfQ = nullptr, *pfK = nullptr, *pfV = nullptr, *pfAttn = nullptr, *pfGate = nullptr, *pfUp = nullptr;
     void *pfHi = nullptr, *pfLo = nullptr;
+    float* pfPartial = nullptr;
     int ensurePrefill(int rows);
     std::vector<Slab> layerSlabs, kvSlabs;
     size_t slotOff[12] = {0};

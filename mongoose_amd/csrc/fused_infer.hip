@@ -841,7 +841,7 @@ int HIPFusedInference::ensurePrefill(int rows) {
     const size_t T = ((size_t)rows + 127) / 128 * 128;
     const size_t plane = split_plane_elems((int)T, ffnDim > dim ? ffnDim : dim) * 2;
     size_t bytes = alignUp256(T * 4) + 3 * alignUp256(T * dim * 4) + 2 * alignUp256(T * kvDim * 4) +
-                   2 * alignUp256(T * ffnDim * 4) + 2 * alignUp256(plane) + 16 * 256;
+                   2 * alignUp256(T * ffnDim * 4) + 2 * alignUp256(plane) + alignUp256(gemm_partial_floats() * 4) + 16 * 256;
     int rc = prefillSlab.init(bytes);
     if (rc) return rc;
     pfTokens = static_cast<int*>(prefillSlab.take(T * 4));
@@ -854,7 +854,8 @@ int HIPFusedInference::ensurePrefill(int rows) {
     pfUp = static_cast<float*>(prefillSlab.take(T * ffnDim * 4));
     pfHi = prefillSlab.take(plane);
     pfLo = prefillSlab.take(plane);
-    if (!pfTokens || !pfX || !pfQ || !pfAttn || !pfK || !pfV || !pfGate || !pfUp || !pfHi || !pfLo) {
+    pfPartial = static_cast<float*>(prefillSlab.take(gemm_partial_floats() * 4));
+    if (!pfTokens || !pfX || !pfQ || !pfAttn || !pfK || !pfV || !pfGate || !pfUp || !pfHi || !pfLo || !pfPartial) {
         set_error("prefill slab too small");
         return MG_E_STATE;
     }
@@ -892,17 +893,13 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
         };
         GemmParams g{};
         g.T = T; g.Ahi = static_cast<const unsigned short*>(pfHi); g.Alo = static_cast<const unsigned short*>(pfLo);
+        g.partial = pfPartial;
         HIPCHK(launch_split_rows(pfX, L.norm1, eps, T, dim, pfHi, pfLo, stream));
         g.K = dim; g.nseg = 3;
         g.seg[0] = seg(L.wq, L.bq, pfQ); g.seg[1] = seg(L.wk, L.bk, pfK); g.seg[2] = seg(L.wv, L.bv, pfV);
         HIPCHK(launch_gemm_q8(g, 0, stream));
         HIPCHK(launch_rope_store_rows(pfQ, pfK, pfV, kCache[l], vCache[l], cosTab, sinTab, pos0, T, dim, kvDim, headDim, stream));
-        AttnParams a{};
-        a.q = pfQ; a.Kc = kCache[l]; a.Vc = vCache[l]; a.posImm = pos0; a.rowLimit = maxSeq;
-        a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
-        a.smax = 1; a.splitLen = 0; a.headsPerWG = 0; a.out = pfAttn;
-        a.batch = T; a.qStride = dim; a.outStride = dim;
-        HIPCHK(launch_attention(a, stream));
+        HIPCHK(launch_prefill_attention(pfQ, kCache[l], vCache[l], pfAttn, T, pos0, maxSeq, dim, kvDim, nHeads, nKVHeads, headDim, stream));
         HIPCHK(launch_split_rows(pfAttn, nullptr, eps, T, dim, pfHi, pfLo, stream));
         g.K = dim; g.nseg = 1; g.seg[0] = seg(L.wo, nullptr, pfX);
         HIPCHK(launch_gemm_q8(g, 1, stream));

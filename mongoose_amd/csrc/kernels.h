@@ -91,10 +91,6 @@ struct AttnParams {
     int* counters;        // one per workgroup column, zero between launches (smax > 1)
     int headsPerWG;       // query heads of a GQA group per workgroup (0 = the whole group, up to 8)
     float* out;           // [dim]
-    // Batched form for prefill: query b (blockIdx.z) sits at position posImm + b, reads
-    // q + b*qStride and writes out + b*outStride.  Needs state == NULL and smax == 1.
-    int batch = 1;
-    int qStride = 0, outStride = 0;
 };
 hipError_t launch_attention(const AttnParams& p, hipStream_t s);
 int attention_columns(int nHeads, int nKVHeads, int headsPerWG);

@@ -616,9 +616,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 
     // ---- everything that does not need the position goes out first ----
     float4 qv = make_float4(0.f, 0.f, 0.f, 0.f);                    // heads past gn stay zero
-    const float* qIn = p.q + (size_t)blockIdx.z * p.qStride;
-    float* outB = p.out + (size_t)blockIdx.z * p.outStride;
-    if (tid < gn * (HD / 4)) qv = reinterpret_cast<const float4*>(qIn + (size_t)h0 * HD)[tid];
+    if (tid < gn * (HD / 4)) qv = reinterpret_cast<const float4*>(p.q + (size_t)h0 * HD)[tid];
     float4 kreg[KQ];
     {
         const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)min(t0 + pIdx, lastRow) * p.kvDim + kvOff) + sub * KQ;
@@ -629,7 +627,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
     for (int u = 0; u < VU; u++) vreg[u] = Vbase[(size_t)min(t0 + tg + u * TG, lastRow) * vStride];
 
-    const int pos = p.state ? p.state->pos : p.posImm + (int)blockIdx.z;
+    const int pos = p.state ? p.state->pos : p.posImm;
     const int len = pos + 1;
     if (t0 >= len) return;                                 // this split holds no position yet
     const int nsplit = p.splitLen > 0 ? (len + p.splitLen - 1) / p.splitLen : 1;
@@ -740,7 +738,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
         if (nsplit == 1) {
             float4 o;
             o.x = r.x / lg; o.y = r.y / lg; o.z = r.z / lg; o.w = r.w / lg;
-            reinterpret_cast<float4*>(outB + (size_t)h * HD)[d4] = o;
+            reinterpret_cast<float4*>(p.out + (size_t)h * HD)[d4] = o;
         } else {
             float* pa = p.pacc + ((size_t)h * p.smax + split) * HD + d4 * 4;
             st_agent(pa, r.x); st_agent(pa + 1, r.y); st_agent(pa + 2, r.z); st_agent(pa + 3, r.w);
@@ -786,7 +784,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
         }
         float4 o;
         o.x = num.x / den; o.y = num.y / den; o.z = num.z / den; o.w = num.w / den;
-        reinterpret_cast<float4*>(outB + (size_t)h * HD)[d4] = o;
+        reinterpret_cast<float4*>(p.out + (size_t)h * HD)[d4] = o;
     }
     if (tid == 0) __hip_atomic_store(p.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -805,7 +803,7 @@ static hipError_t launch_attn_hd(const AttnParams& p, hipStream_t s) {
     int G = p.nHeads / p.nKVHeads;
     int gmax = attention_gmax(G, p.headsPerWG);
     int nChunks = (G + gmax - 1) / gmax;
-    dim3 grid(p.nKVHeads * nChunks, p.smax, p.batch);
+    dim3 grid(p.nKVHeads * nChunks, p.smax);
     switch (gmax) {
     case 1: hipLaunchKernelGGL((attn_decode_kernel<HD, 1>), grid, dim3(WG), 0, s, p); break;
     case 2: hipLaunchKernelGGL((attn_decode_kernel<HD, 2>), grid, dim3(WG), 0, s, p); break;
@@ -824,7 +822,6 @@ int attention_columns(int nHeads, int nKVHeads, int headsPerWG) {
 
 hipError_t launch_attention(const AttnParams& p, hipStream_t s) {
     if (p.nKVHeads <= 0 || p.nHeads % p.nKVHeads != 0 || p.rowLimit <= 0 || p.smax < 1) return hipErrorInvalidValue;
-    if (p.batch < 1 || p.batch > 65535 || (p.batch > 1 && (p.state || p.smax != 1 || p.posImm + p.batch > p.rowLimit))) return hipErrorInvalidValue;
     const int tile = p.headDim == 128 ? WG / 2 : WG;
     if (p.smax > 1 && (p.splitLen <= 0 || p.splitLen % tile != 0 || !p.counters || !p.pm || !p.pl || !p.pacc)) return hipErrorInvalidValue;
     if (p.headDim == 64) return launch_attn_hd<64>(p, s);

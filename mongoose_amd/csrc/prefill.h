@@ -15,6 +15,9 @@ hipError_t launch_swiglu_split(const float* gate, const float* up, int T, int K,
 // RoPE on q rows in place; rotated k rows and v rows stored into cache rows pos0 .. pos0+T-1.
 hipError_t launch_rope_store_rows(float* q, const float* k, const float* v, float* Kc, float* Vc, const float* cosTab,
                                   const float* sinTab, int pos0, int T, int dim, int kvDim, int headDim, hipStream_t s);
+// Causal attention of T query rows [T,dim] (rotated) at positions pos0.. over cache rows [0, pos0+T); out [T,dim].
+hipError_t launch_prefill_attention(const float* q, const float* Kc, const float* Vc, float* out, int T, int pos0, int rowLimit,
+                                    int dim, int kvDim, int nHeads, int nKVHeads, int headDim, hipStream_t s);
 // Embedding rows of T tokens: kind 0 = Q8 row * scale, 1 = fp16 table, 2 = fp32 table.
 hipError_t launch_embed_rows(int kind, const void* table, const float* scales, const int* tokens, float* x, int T, int dim,
                              int vocab, hipStream_t s);
@@ -27,8 +30,11 @@ struct GemmParams {
     const unsigned short* Ahi;
     const unsigned short* Alo;
     int T, K;
-    int nTiles;       // filled by the launcher
+    float* partial;   // workspace of gemm_partial_floats() floats for K-split partial sums (NULL: never split K)
+    // filled by the launcher
+    int nTiles, splitK, stepsPerSplit, ldPartial;
 };
+size_t gemm_partial_floats();
 hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s);
 
 }  // namespace mg

@@ -144,10 +144,145 @@ hipError_t launch_embed_rows(int kind, const void* table, const float* scales, c
 }
 
 // ---------------------------------------------------------------------------
-// GEMM on v_mfma_f32_32x32x16_bf16.  Workgroup tile BM (T) x 128 (N), K in
-// steps of 64; four waves as 2x2, each (BM/2)x64 = (BM/64)x2 MFMA blocks, the
-// hi and the lo activation term against the same weight fragment.  Fragment
-// layouts (lane l):
+// Causal attention over T query rows (mongoose.cu:251-353 for a training
+// sequence; here against the KV caches, query t at position pos0 + t).
+// One workgroup = 32 queries of one head; its four waves take the 32-position
+// KV tiles in turn (tile w, w+4, ...) with their own running max / sum /
+// output and are combined at the end, so the longest serial chain is a quarter
+// of the causal range.  Both products run on the fp32 matrix instruction
+// v_mfma_f32_32x32x2_f32 (exact fp32 products, fp32 accumulation), arranged
+// transposed so that a lane owns one query:
+//   S^T[kpos][q] = K . Q^T    A = K tile from LDS, B = Q rows held in registers
+//   O^T[d][q]    = V^T . P^T  A = V rows straight from the cache, B = the S^T accumulator itself
+// (C layout: lane l holds column l%32, rows 8*(i/4) + 4*(l/32) + i%4; as a B
+// operand step s wants row k = l/32 of its pair, so step s pairs exactly the
+// rows register s holds in the two lane halves.)
+// ---------------------------------------------------------------------------
+template <int HD>
+__global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const float* Kc, const float* Vc, float* out, int T,
+                                                          int pos0, int dim, int kvDim, int nHeads, int nKVHeads) {
+    constexpr int KS = HD + 4;                 // LDS row stride of the K tile (floats)
+    constexpr int DB = HD / 32;                // 32-wide blocks of the head dimension
+    __shared__ __attribute__((aligned(16))) float lds[4][32 * KS];
+    __shared__ float wm[4][32], wl[4][32];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int q0 = blockIdx.x * 32, head = blockIdx.y;
+    const int kvh = head / (nHeads / nKVHeads);
+    const int myq = q0 + col;                           // this lane's query row
+    const int qpos = pos0 + min(myq, T - 1);            // its position (clamped rows are never stored)
+    const float scale = 1.0f / sqrtf((float)HD);
+
+    // Q^T operand: lane holds Q[myq][2*s + half], s = 0 .. HD/2-1
+    float qreg[HD / 2];
+    {
+        const float* qr = q + (size_t)min(myq, T - 1) * dim + (size_t)head * HD + half;
+#pragma unroll
+        for (int s = 0; s < HD / 2; s++) qreg[s] = qr[2 * s];
+    }
+    float16_t o[DB];
+#pragma unroll
+    for (int b = 0; b < DB; b++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) o[b][e] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    const int lastPos = pos0 + min(q0 + 31, T - 1);     // furthest position any query of the block sees
+    const int nTiles = lastPos / 32 + 1;
+    float* kt = lds[wave];
+    for (int tile = wave; tile < nTiles; tile += 4) {
+        const int t0 = tile * 32;
+        // K tile -> this wave's LDS (rows past lastPos are clamped; they are masked below)
+#pragma unroll
+        for (int i = 0; i < 32 * HD / 4 / 64; i++) {
+            const int idx = i * 64 + lane, r = idx / (HD / 4), c4 = idx % (HD / 4);
+            const float4 v = *reinterpret_cast<const float4*>(Kc + (size_t)min(t0 + r, lastPos) * kvDim + (size_t)kvh * HD + c4 * 4);
+            *reinterpret_cast<float4*>(&kt[r * KS + c4 * 4]) = v;
+        }
+        __builtin_amdgcn_s_waitcnt(0);                   // wave-private buffer: the wave's own stores have landed
+        __builtin_amdgcn_wave_barrier();
+        float16_t sT;
+#pragma unroll
+        for (int e = 0; e < 16; e++) sT[e] = 0.f;
+#pragma unroll
+        for (int s = 0; s < HD / 2; s++)
+            sT = __builtin_amdgcn_mfma_f32_32x32x2f32(kt[col * KS + 2 * s + half], qreg[s], sT, 0, 0, 0);
+        // causal mask, online softmax for this lane's query over the tile's 32 positions
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const int kpos = t0 + 8 * (e >> 2) + 4 * half + (e & 3);
+            sT[e] = kpos <= qpos ? sT[e] * scale : -INFINITY;
+            tmax = fmaxf(tmax, sT[e]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float mNew = fmaxf(m, tmax);
+        const float corr = m == -INFINITY ? 0.f : expf(m - mNew);
+        float psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const float pv = sT[e] == -INFINITY ? 0.f : expf(sT[e] - mNew);
+            sT[e] = pv;
+            psum += pv;
+        }
+        psum += __shfl_xor(psum, 32, 64);
+        l = l * corr + psum;
+        m = mNew;
+#pragma unroll
+        for (int b = 0; b < DB; b++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) o[b][e] *= corr;
+        // O^T += V^T . P^T : step s takes positions 8*(s/4) + 4*half + s%4, which is what sT[s] holds
+#pragma unroll
+        for (int s = 0; s < 16; s++) {
+            const int kpos = min(t0 + 8 * (s >> 2) + 4 * half + (s & 3), lastPos);
+            const float* vr = Vc + (size_t)kpos * kvDim + (size_t)kvh * HD + col;
+#pragma unroll
+            for (int b = 0; b < DB; b++)
+                o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[32 * b], sT[s], o[b], 0, 0, 0);
+        }
+        __builtin_amdgcn_wave_barrier();                 // the K tile is overwritten next
+    }
+    // ---- combine the four waves: O^T partials through the (now free) tile buffers ----
+    // layout in kt: [d][q] with row stride 33
+    static_assert(HD * 33 <= 32 * KS, "tile buffer too small for the partial output");
+#pragma unroll
+    for (int b = 0; b < DB; b++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) kt[(32 * b + 8 * (e >> 2) + 4 * half + (e & 3)) * 33 + col] = o[b][e];
+    if (half == 0) { wm[wave][col] = m; wl[wave][col] = l; }
+    __syncthreads();
+    for (int i = tid; i < 32 * HD; i += 256) {
+        const int qq = i / HD, d = i % HD;
+        if (q0 + qq >= T) continue;
+        const float M = fmaxf(fmaxf(wm[0][qq], wm[1][qq]), fmaxf(wm[2][qq], wm[3][qq]));
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float wgt = wm[w][qq] == -INFINITY ? 0.f : expf(wm[w][qq] - M);
+            num = fmaf(wgt, lds[w][d * 33 + qq], num);
+            den = fmaf(wgt, wl[w][qq], den);
+        }
+        out[(size_t)(q0 + qq) * dim + (size_t)head * HD + d] = num / den;
+    }
+}
+
+hipError_t launch_prefill_attention(const float* q, const float* Kc, const float* Vc, float* out, int T, int pos0, int rowLimit,
+                                    int dim, int kvDim, int nHeads, int nKVHeads, int headDim, hipStream_t s) {
+    if (T <= 0) return hipSuccess;
+    if (nKVHeads <= 0 || nHeads % nKVHeads != 0 || pos0 < 0 || pos0 + T > rowLimit || dim != nHeads * headDim ||
+        kvDim != nKVHeads * headDim) return hipErrorInvalidValue;
+    dim3 grid((unsigned)((T + 31) / 32), (unsigned)nHeads);
+    if (headDim == 64) hipLaunchKernelGGL(prefill_attn_kernel<64>, grid, dim3(256), 0, s, q, Kc, Vc, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
+    else if (headDim == 128) hipLaunchKernelGGL(prefill_attn_kernel<128>, grid, dim3(256), 0, s, q, Kc, Vc, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// GEMM on v_mfma_f32_32x32x16_bf16, K in steps of 64; each wave owns 32-row x
+// 32-column MFMA blocks and issues the hi and the lo activation term against
+// the same weight fragment.  Fragment layouts (lane l):
 //   A: row l%32, k = 8*(l/32)..+7        B: col l%32, k = 8*(l/32)..+7
 //   C: col l%32, rows 8*(i/4) + 4*(l/32) + i%4 for i = 0..15
 // Up to three weight matrices (q/k/v, gate/up) share one launch.  Workgroups
@@ -155,7 +290,7 @@ hipError_t launch_embed_rows(int kind, const void* table, const float* scales, c
 // tile comes into that XCD's L2 once.
 // ---------------------------------------------------------------------------
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-constexpr int BN = 128, BK = 64;
+constexpr int BK = 64;
 constexpr int A_STRIDE = BK + 8;    // bf16 per LDS row (144 bytes)
 constexpr int B_STRIDE = BK + 16;   // bytes per LDS row of int8 weights (80)
 
@@ -164,16 +299,24 @@ __device__ __forceinline__ unsigned pack_bf16_exact(float lo, float hi) {
     return (__builtin_bit_cast(unsigned, lo) >> 16) | (__builtin_bit_cast(unsigned, hi) & 0xffff0000u);
 }
 
-template <int BM, int EPI>   // EPI 0: Y = acc*scale (+bias)   1: Y += acc*scale (residual in place)
-__global__ __launch_bounds__(PWG) void gemm_q8_bf16x2_kernel(GemmParams p) {
-    constexpr int MI = BM / 64;                  // 32-row MFMA blocks per wave
-    constexpr int AR = BM / 32;                  // 16-byte segments per thread and A plane (BM*8 segments / 256)
+// Workgroup tile BM x BN with NT threads: NT/64 waves as (NT/64)/(BN/64) x (BN/64), each wave
+// (BM/WM) x 64.  The L2-to-CU traffic per flop falls with the tile size (A costs 4 bytes an
+// element, W one), and it is that traffic which bounds the kernel: 256 x 256 tiles with 1024
+// threads where the problem is large enough, 64/128 x 128 with 256 threads for short prompts.
+// MODE 0: Y = acc*scale (+bias)   1: Y += acc*scale   2: raw partial sums of one K split into p.partial
+template <int BM, int BN, int NT, int MODE>
+__global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
+    constexpr int WN = BN / 64, WM = (NT / 64) / WN;
+    constexpr int MI = BM / WM / 32;             // 32-row MFMA blocks per wave
+    constexpr int AR = BM * 8 / NT;              // 16-byte segments per thread and A plane
+    constexpr int BR = BN * 4 / NT;              // 16-byte segments per thread of W
+    static_assert(MI >= 1 && AR >= 1 && BR >= 1, "tile too small for the thread count");
     __shared__ __attribute__((aligned(16))) unsigned short sAh[BM * A_STRIDE];
     __shared__ __attribute__((aligned(16))) unsigned short sAl[BM * A_STRIDE];
     __shared__ __attribute__((aligned(16))) signed char sB[BN * B_STRIDE];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int numM = (p.T + BM - 1) / BM;
     const int L = blockIdx.x;
     const int grp = L / (8 * numM), rem = L % (8 * numM);
@@ -185,22 +328,25 @@ __global__ __launch_bounds__(PWG) void gemm_q8_bf16x2_kernel(GemmParams p) {
     const GemmSeg sg = p.seg[sgi];
     const int N = sg.N, K = p.K, T = p.T;
     const int m0 = mTile * BM, n0 = (nTile - sg.tile0) * BN;
+    const int ksteps = (K + BK - 1) / BK;
+    const int stepBeg = MODE == 2 ? blockIdx.y * p.stepsPerSplit : 0;
+    const int stepEnd = MODE == 2 ? min(ksteps, stepBeg + p.stepsPerSplit) : ksteps;
 
-    // global -> LDS: A row = tid/8 + 32*r, segment tid%8 (8 bf16) ; B row = tid/4 + 64*r, segment tid%4 (16 int8)
+    // global -> LDS: A row = tid/8 (+NT/8 per pass), segment tid%8 (8 bf16) ; W row = tid/4 (+NT/4), segment tid%4 (16 int8)
     const int aRow = tid >> 3, aSeg = tid & 7;
     const int bRow = tid >> 2, bSeg = tid & 3;
     const unsigned short* aHiP[AR]; const unsigned short* aLoP[AR];
-    const int ksteps = (K + BK - 1) / BK;
+    const int planeRows = ((T + 127) >> 7) << 7;     // the planes are padded to whole 128-row blocks, not to BM
 #pragma unroll
-    for (int r = 0; r < AR; r++) {         // rows past T exist in the padded planes; their results are dropped
-        const int row = m0 + aRow + 32 * r;
+    for (int r = 0; r < AR; r++) {         // rows in [T, planeRows) exist in the planes; their results are dropped
+        const int row = min(m0 + aRow + (NT / 8) * r, planeRows - 1);
         const size_t o = (size_t)(row >> 7) * ksteps * 8192 + (size_t)(row & 127) * 64 + aSeg * 8;
         aHiP[r] = p.Ahi + o;
         aLoP[r] = p.Alo + o;
     }
-    const signed char* bP[2];
+    const signed char* bP[BR];
 #pragma unroll
-    for (int r = 0; r < 2; r++) bP[r] = sg.W + (size_t)min(n0 + bRow + 64 * r, N - 1) * K + bSeg * 16;
+    for (int r = 0; r < BR; r++) bP[r] = sg.W + (size_t)min(n0 + bRow + (NT / 4) * r, N - 1) * K + bSeg * 16;
 
     float16_t acc[MI][2];
 #pragma unroll
@@ -210,7 +356,7 @@ __global__ __launch_bounds__(PWG) void gemm_q8_bf16x2_kernel(GemmParams p) {
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-    int4 gAh[AR], gAl[AR], gB[2];
+    int4 gAh[AR], gAl[AR], gB[BR];
     const int4 zero4 = make_int4(0, 0, 0, 0);
     auto gload = [&](int k0) {       // K is a multiple of 32: a last half step reads zeros past the end
         const bool okA = k0 + aSeg * 8 < K, okB = k0 + bSeg * 16 < K;
@@ -220,20 +366,20 @@ __global__ __launch_bounds__(PWG) void gemm_q8_bf16x2_kernel(GemmParams p) {
             gAl[r] = okA ? *reinterpret_cast<const int4*>(aLoP[r] + (size_t)k0 * 128) : zero4;
         }
 #pragma unroll
-        for (int r = 0; r < 2; r++) gB[r] = okB ? *reinterpret_cast<const int4*>(bP[r] + k0) : zero4;
+        for (int r = 0; r < BR; r++) gB[r] = okB ? *reinterpret_cast<const int4*>(bP[r] + k0) : zero4;
     };
-    gload(0);
-    for (int k0 = 0; k0 < K; k0 += BK) {
+    if (stepBeg < stepEnd) gload(stepBeg * BK);
+    for (int step = stepBeg; step < stepEnd; step++) {
         __syncthreads();                       // the previous step's fragments are consumed
 #pragma unroll
         for (int r = 0; r < AR; r++) {
-            *reinterpret_cast<int4*>(&sAh[(aRow + 32 * r) * A_STRIDE + aSeg * 8]) = gAh[r];
-            *reinterpret_cast<int4*>(&sAl[(aRow + 32 * r) * A_STRIDE + aSeg * 8]) = gAl[r];
+            *reinterpret_cast<int4*>(&sAh[(aRow + (NT / 8) * r) * A_STRIDE + aSeg * 8]) = gAh[r];
+            *reinterpret_cast<int4*>(&sAl[(aRow + (NT / 8) * r) * A_STRIDE + aSeg * 8]) = gAl[r];
         }
 #pragma unroll
-        for (int r = 0; r < 2; r++) *reinterpret_cast<int4*>(&sB[(bRow + 64 * r) * B_STRIDE + bSeg * 16]) = gB[r];
+        for (int r = 0; r < BR; r++) *reinterpret_cast<int4*>(&sB[(bRow + (NT / 4) * r) * B_STRIDE + bSeg * 16]) = gB[r];
         __syncthreads();
-        if (k0 + BK < K) gload(k0 + BK);       // next tile in flight while this one is multiplied
+        if (step + 1 < stepEnd) gload((step + 1) * BK);       // next tile in flight while this one is multiplied
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ks++) {
             const int kk = ks * 16 + 8 * (lane >> 5);
@@ -250,7 +396,7 @@ __global__ __launch_bounds__(PWG) void gemm_q8_bf16x2_kernel(GemmParams p) {
             }
 #pragma unroll
             for (int i = 0; i < MI; i++) {
-                const int arow = (wm * (BM / 2) + i * 32 + (lane & 31)) * A_STRIDE + kk;
+                const int arow = (wm * (BM / WM) + i * 32 + (lane & 31)) * A_STRIDE + kk;
                 bf16x8_t ah = *reinterpret_cast<const bf16x8_t*>(&sAh[arow]);
                 bf16x8_t al = *reinterpret_cast<const bf16x8_t*>(&sAl[arow]);
 #pragma unroll
@@ -263,7 +409,20 @@ __global__ __launch_bounds__(PWG) void gemm_q8_bf16x2_kernel(GemmParams p) {
     }
 #pragma unroll
     for (int j = 0; j < 2; j++) {
-        const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+        const int nl = wn * 64 + j * 32 + (lane & 31);
+        const int n = n0 + nl;
+        if (MODE == 2) {
+            // partial[split][m][column in the concatenated, tile-padded column space]
+            float* dst = p.partial + ((size_t)blockIdx.y * T) * p.ldPartial + (size_t)nTile * BN + nl;
+#pragma unroll
+            for (int i = 0; i < MI; i++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int m = m0 + wm * (BM / WM) + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                    if (m < T) dst[(size_t)m * p.ldPartial] = acc[i][j][e];
+                }
+            continue;
+        }
         if (n >= N) continue;
         const float sc = sg.scales[n];
         const float bi = sg.bias ? sg.bias[n] : 0.f;
@@ -271,11 +430,11 @@ __global__ __launch_bounds__(PWG) void gemm_q8_bf16x2_kernel(GemmParams p) {
         for (int i = 0; i < MI; i++) {
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-                const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                const int m = m0 + wm * (BM / WM) + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                 if (m < T) {
                     float v = acc[i][j][e] * sc + bi;
                     float* dst = sg.Y + (size_t)m * N + n;
-                    if (EPI == 1) v = *dst + v;
+                    if (MODE == 1) v = *dst + v;
                     *dst = v;
                 }
             }
@@ -283,28 +442,79 @@ __global__ __launch_bounds__(PWG) void gemm_q8_bf16x2_kernel(GemmParams p) {
     }
 }
 
+// Sum of the K splits in split order (so the result does not depend on which workgroup
+// finished first), then scale, bias and the optional residual.
+__global__ __launch_bounds__(PWG) void gemm_reduce_kernel(GemmParams p, int BN, int residual) {
+    const int c = blockIdx.x * PWG + threadIdx.x;      // column in the padded column space
+    const int m = blockIdx.y;
+    if (c >= p.ldPartial) return;
+    const int tile = c / BN;
+    int sgi = 0;
+    if (p.nseg > 1 && tile >= p.seg[1].tile0) sgi = 1;
+    if (p.nseg > 2 && tile >= p.seg[2].tile0) sgi = 2;
+    const GemmSeg sg = p.seg[sgi];
+    const int n = c - sg.tile0 * BN;
+    if (n >= sg.N) return;
+    const float* src = p.partial + (size_t)m * p.ldPartial + c;
+    float v = 0.f;
+    for (int s = 0; s < p.splitK; s++) v += src[(size_t)s * p.T * p.ldPartial];
+    v = v * sg.scales[n] + (sg.bias ? sg.bias[n] : 0.f);
+    float* dst = sg.Y + (size_t)m * sg.N + n;
+    if (residual) v = *dst + v;
+    *dst = v;
+}
+
+size_t gemm_partial_floats() { return (size_t)320 * 256 * 256; }
+
 hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s) {
     if (p.T <= 0 || p.nseg < 1 || p.nseg > 3) return p.T <= 0 ? hipSuccess : hipErrorInvalidValue;
     if (p.K <= 0 || p.K % 32 != 0) return hipErrorInvalidValue;
-    int tiles = 0;
-    for (int i = 0; i < p.nseg; i++) {
-        if (p.seg[i].N <= 0) return hipErrorInvalidValue;
-        p.seg[i].tile0 = tiles;
-        tiles += (p.seg[i].N + BN - 1) / BN;
+    for (int i = 0; i < p.nseg; i++) if (p.seg[i].N <= 0) return hipErrorInvalidValue;
+    auto count = [&](int bn) {
+        int tiles = 0;
+        for (int i = 0; i < p.nseg; i++) { p.seg[i].tile0 = tiles; tiles += (p.seg[i].N + bn - 1) / bn; }
+        p.nTiles = tiles;
+        return tiles;
+    };
+    const int ksteps = (p.K + BK - 1) / BK;
+    p.splitK = 1; p.stepsPerSplit = ksteps;
+    if (p.T > 128) {
+        // 256 x 256 tiles; K is split until about one workgroup per CU exists (each split keeps >= 8 steps).
+        // Worth it when the tiles alone nearly fill the chip or K can be split; otherwise the small tiles
+        // below give more workgroups (short K, narrow N: latency-bound either way).
+        const int tiles = count(256);
+        const int numM = (p.T + 255) / 256;
+        const int wgs = tiles * numM;
+        int S = 1;
+        if (p.partial && wgs < 160) {
+            S = (224 + wgs / 2) / wgs;
+            if (S > ksteps / 8) S = ksteps / 8;
+            if (S < 1) S = 1;
+            while (S > 1 && (size_t)S * p.T * tiles * 256 > gemm_partial_floats()) S--;
+        }
+        if (wgs >= 96 || S >= 2) {
+            dim3 grid((unsigned)(((tiles + 7) / 8) * 8 * numM), 1);
+            if (S > 1) {
+                p.stepsPerSplit = (ksteps + S - 1) / S;
+                S = (ksteps + p.stepsPerSplit - 1) / p.stepsPerSplit;
+                grid.y = (unsigned)S;
+                p.splitK = S; p.ldPartial = tiles * 256;
+                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<256, 256, 1024, 2>), grid, dim3(1024), 0, s, p);
+                hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((p.ldPartial + PWG - 1) / PWG), (unsigned)p.T), dim3(PWG),
+                                   0, s, p, 256, residual);
+            } else if (residual) {
+                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<256, 256, 1024, 1>), grid, dim3(1024), 0, s, p);
+            } else {
+                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<256, 256, 1024, 0>), grid, dim3(1024), 0, s, p);
+            }
+            return hipGetLastError();
+        }
     }
-    p.nTiles = tiles;
-    // 128-row tiles once they fill the chip, 64-row tiles below that
-    const int numM128 = (p.T + 127) / 128;
-    const bool big = (long long)numM128 * tiles >= 512;
-    const int numM = big ? numM128 : (p.T + 63) / 64;
+    const int tiles = count(128);
+    const int numM = (p.T + 63) / 64;
     dim3 grid((unsigned)(((tiles + 7) / 8) * 8 * numM));
-    if (big) {
-        if (residual) hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<128, 1>), grid, dim3(PWG), 0, s, p);
-        else hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<128, 0>), grid, dim3(PWG), 0, s, p);
-    } else {
-        if (residual) hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<64, 1>), grid, dim3(PWG), 0, s, p);
-        else hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<64, 0>), grid, dim3(PWG), 0, s, p);
-    }
+    if (residual) hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<64, 128, 256, 1>), grid, dim3(PWG), 0, s, p);
+    else hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<64, 128, 256, 0>), grid, dim3(PWG), 0, s, p);
     return hipGetLastError();
 }
 
