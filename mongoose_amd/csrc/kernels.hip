@@ -243,9 +243,10 @@ __device__ __forceinline__ RowRef resolve_row(const MvParams& p, int g, int i) {
         int gi = g - p.segGroup0[s];
         r.seg = s;
         if (s < 2) {
-            int half = p.headDim >> 1;
-            int head = gi / half, j = gi % half;
-            r.row = head * p.headDim + j + (i ? half : 0);
+            // headDim is a power of two (checked by the launcher): gi = head * half + j
+            const int half = p.headDim >> 1;
+            const int j = gi & (half - 1);
+            r.row = ((gi - j) << 1) + j + (i ? half : 0);
         } else {
             r.row = gi * 2 + i;
         }
@@ -288,10 +289,14 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     typename F::Chunk ring[D][NR];
     float rSc[D], rBi[D], rRe[D], rCs[D], rSn[D];            // epilogue operands of the lane's row
 
+    // (group, chunk iteration) of the next item to issue and of the next item to consume:
+    // advanced step by step, no division in the loop
+    int gI = gStart, itI = 0, gC = gStart, itC = 0;
     auto issue = [&](int slot, int item) {
         if (item >= nItems) return;
-        const int g = gStart + (item / iters) * gStep;
-        const int it = item % iters;
+        const int g = gI;
+        const int it = itI;
+        if (++itI == iters) { itI = 0; gI += gStep; }
         const int c = lig + it * LPG;
 #pragma unroll
         for (int i = 0; i < NR; i++) {
@@ -308,8 +313,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
                     if (sg.bias) rBi[slot] = sg.bias[rr.row];
                     if (EPI == EPI_RESID) rRe[slot] = p.resid[rr.row];
                     if (EPI == EPI_QKV && rr.seg < 2 && lane == 0) {
-                        int half = p.headDim >> 1;
-                        int j = (g - p.segGroup0[rr.seg]) % half;
+                        const int j = (g - p.segGroup0[rr.seg]) & ((p.headDim >> 1) - 1);
                         rCs[slot] = p.cosRow[j];
                         rSn[slot] = p.sinRow[j];
                     }
@@ -336,8 +340,9 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
         for (int s = 0; s < D; s++) {
             const int item = base + s;
             if (item < nItems) {
-                const int g = gStart + (item / iters) * gStep;
-                const int it = item % iters;
+                const int g = gC;
+                const int it = itC;
+                if (++itC == iters) { itC = 0; gC += gStep; }
                 const int c = lig + it * LPG;
                 if (c < nch) {
                     float4 av[4];
@@ -513,7 +518,8 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
         p.segGroup0[0] = 0; p.segGroup0[1] = p.ngroups; p.segGroup0[2] = p.ngroups;
     } else if (epi == EPI_QKV) {
         // q and k rows pair up inside a head, so both need whole heads; v rows pair up consecutively
-        if (p.nseg != 3 || p.headDim <= 0 || p.seg[0].rows % p.headDim || p.seg[1].rows % p.headDim || p.seg[2].rows % 2)
+        if (p.nseg != 3 || p.headDim < 2 || (p.headDim & (p.headDim - 1)) || p.seg[0].rows % p.headDim ||
+            p.seg[1].rows % p.headDim || p.seg[2].rows % 2)
             return hipErrorInvalidValue;
         c.nr = 2;
         int g = 0;
