@@ -89,7 +89,7 @@ struct AttnParams {
     int smax;             // number of splits launched
     float* pm; float* pl; float* pacc;   // partials [nHeads, smax(, headDim)] when smax > 1
     int* counters;        // one per workgroup column, zero between launches (smax > 1)
-    int headsPerWG;       // query heads of a GQA group per workgroup (0 = the whole group, up to 8)
+    int headsPerWG;       // query heads of a GQA group per workgroup (0 = the whole group, in chunks of up to 4)
     float* out;           // [dim]
 };
 hipError_t launch_attention(const AttnParams& p, hipStream_t s);

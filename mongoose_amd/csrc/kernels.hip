@@ -571,14 +571,21 @@ hipError_t launch_matvec_generic_q8(const float* act, const void* w, const float
 
 // ---------------------------------------------------------------------------
 // Decode attention (mongoose.cu:856-933), split over the KV range.
-// One workgroup = one KV head (all its GQA query heads, so K/V rows are read
-// once) x one split of the positions.  q arrives rotated and the K/V rows of
-// the current position are already in the caches (the QKV matvec's epilogue
-// did both).  The split geometry is fixed per context, so the first tile's
-// K/V rows are requested before the position is known (rows past the end are
-// clamped and masked): the kernel's critical path is one memory latency.
-// Online softmax over 256-position tiles; scores: one lane per position with
-// the K row in registers; P.V: one lane per float4 of the head.
+// One workgroup = one KV head x up to GMAX of its GQA query heads (K/V rows are
+// read once for all of them) x one split of the positions.  q arrives rotated
+// and the K/V rows of the current position are already in the caches (the QKV
+// matvec's epilogue did both).  The split geometry is fixed per context, so the
+// first tile's K and V rows are requested before the position is known (rows
+// past the end are clamped and masked): the critical path is one memory latency.
+//
+// K and V use the same register layout: a row of the head is spread over LPR =
+// HD/4 lanes (one float4 each, so a wave's load covers whole rows: coalesced),
+// and a thread holds VU = 16 rows of the tile, tg + u*TG.  A score is the
+// lane's 4-term partial product reduced over the row's lanes by DPP; every lane
+// of a row ends up with the score, which is exactly where P.V needs it -- the
+// probabilities never leave registers.  Per tile there is one barrier (the
+// tile maximum across waves); the running sum and the output stay per-thread
+// partials over the thread's own rows and are reduced once at the end.
 // With several splits the last workgroup of a column to finish combines the
 // partials, so the output is always the final [dim] vector.
 // ---------------------------------------------------------------------------
@@ -588,24 +595,44 @@ __device__ __forceinline__ float ld_agent(const float* p) {
 __device__ __forceinline__ void st_agent(float* p, float v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// Sum over the LPR lanes that hold one row (16: one DPP row; 32: two).  Every step adds a lane's
+// value to its mirror partner's (quad_perm, then row_half_mirror = 0x141, row_mirror = 0x140), so
+// both partners compute the same commutative sum: all lanes of the row end with the same bits,
+// which keeps exp(score - max) identical across the lanes that apply it.
+template <int LPR>
+__device__ __forceinline__ float row_sum(float v) {
+    v += dpp_f<0xB1>(v);
+    v += dpp_f<0x4E>(v);
+    v += dpp_f<0x141>(v);
+    v += dpp_f<0x140>(v);
+    if (LPR == 32) v += __shfl_xor(v, 16, 64);
+    return v;
+}
+// combine a per-thread value over the row groups (tg) that share a wave
+template <int LPR>
+__device__ __forceinline__ float tg_max(float v) {
+    if (LPR == 16) v = fmaxf(v, __shfl_xor(v, 16, 64));
+    return fmaxf(v, __shfl_xor(v, 32, 64));
+}
+template <int LPR>
+__device__ __forceinline__ float tg_sum(float v) {
+    if (LPR == 16) v += __shfl_xor(v, 16, 64);
+    return v + __shfl_xor(v, 32, 64);
+}
 
 template <int HD, int GMAX>
 __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
-    constexpr int LPP = HD / 64;       // lanes per position in the score phase (64 dims each)
-    constexpr int TILE = WG / LPP;     // positions per tile
-    constexpr int LPR = HD / 4;        // lanes per V row
-    constexpr int TG = WG / LPR;       // position groups in the P.V phase
-    constexpr int VU = TILE / TG;      // V rows per thread and tile, all in flight (16)
-    constexpr int KQ = 16;             // K float4s per lane (64 dims)
-    __shared__ float4 q_s4[GMAX * HD / 4];
-    __shared__ float sc[GMAX][TILE];
+    constexpr int LPR = HD / 4;        // lanes per K/V row
+    constexpr int TG = WG / LPR;       // rows in flight per load step
+    constexpr int VU = 16;             // rows per thread and tile
+    constexpr int TILE = TG * VU;      // positions per tile (256 for head size 64, 128 for 128)
     __shared__ float wred[2][GMAX][4];
-    __shared__ float4 accbuf[TG][GMAX][LPR];
+    __shared__ float4 accbuf[4][GMAX][LPR];
+    __shared__ float lbuf[4][GMAX];
     __shared__ int lastFlag;
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int sub = tid % LPP, pIdx = tid / LPP;
+    const int wave = tid >> 6;
     const int G = p.nHeads / p.nKVHeads;
     const int nChunks = (G + GMAX - 1) / GMAX;
     const int kvh = blockIdx.x / nChunks;
@@ -617,21 +644,22 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     const int tg = tid / LPR, dl = tid % LPR;
     const int t0 = p.splitLen > 0 ? split * p.splitLen : 0;
     const int lastRow = p.rowLimit - 1;
-    const size_t vStride = (size_t)p.kvDim / 4;
+    const size_t rowStride = (size_t)p.kvDim / 4;
+    const float4* Kbase = reinterpret_cast<const float4*>(p.Kc + kvOff) + dl;
     const float4* Vbase = reinterpret_cast<const float4*>(p.Vc + kvOff) + dl;
 
     // ---- everything that does not need the position goes out first ----
-    float4 qv = make_float4(0.f, 0.f, 0.f, 0.f);                    // heads past gn stay zero
-    if (tid < gn * (HD / 4)) qv = reinterpret_cast<const float4*>(p.q + (size_t)h0 * HD)[tid];
-    float4 kreg[KQ];
-    {
-        const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)min(t0 + pIdx, lastRow) * p.kvDim + kvOff) + sub * KQ;
+    float4 q4[GMAX];
 #pragma unroll
-        for (int d4 = 0; d4 < KQ; d4++) kreg[d4] = krow[d4];
+    for (int g = 0; g < GMAX; g++) {           // heads past gn work on zeros and are dropped at the end
+        q4[g] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (g < gn) q4[g] = reinterpret_cast<const float4*>(p.q + (size_t)(h0 + g) * HD)[dl];
     }
-    float4 vreg[VU];
+    float4 kreg[VU], vreg[VU];
 #pragma unroll
-    for (int u = 0; u < VU; u++) vreg[u] = Vbase[(size_t)min(t0 + tg + u * TG, lastRow) * vStride];
+    for (int u = 0; u < VU; u++) kreg[u] = Kbase[(size_t)min(t0 + tg + u * TG, lastRow) * rowStride];
+#pragma unroll
+    for (int u = 0; u < VU; u++) vreg[u] = Vbase[(size_t)min(t0 + tg + u * TG, lastRow) * rowStride];
 
     const int pos = p.state ? p.state->pos : p.posImm;
     const int len = pos + 1;
@@ -639,107 +667,86 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     const int nsplit = p.splitLen > 0 ? (len + p.splitLen - 1) / p.splitLen : 1;
     const int t1 = p.splitLen > 0 ? min(len, t0 + p.splitLen) : len;
 
-    if (tid < GMAX * (HD / 4)) q_s4[tid] = qv;
-    __syncthreads();
-
-    // Every loop below runs over all GMAX heads without a guard (straight-line code the
-    // scheduler can interleave); heads past gn work on zeros and are dropped at the end.
     const float scale = 1.0f / sqrtf((float)HD);     // mongoose.cu:867 rsqrtf(headDim)
-    float m[GMAX], l[GMAX];
+    float m[GMAX], l[GMAX];                           // m: workgroup-wide running max; l, acc: this thread's rows only
     float4 acc[GMAX];
 #pragma unroll
     for (int g = 0; g < GMAX; g++) { m[g] = -INFINITY; l[g] = 0.f; acc[g] = make_float4(0.f, 0.f, 0.f, 0.f); }
 
+    int par = 0;
     for (int tile = t0; tile < t1; tile += TILE) {
-        const int t = tile + pIdx;
-        const bool active = t < t1;
-        const int tileLen = min(TILE, t1 - tile);
         if (tile != t0) {
-            const float4* krow = reinterpret_cast<const float4*>(p.Kc + (size_t)min(t, lastRow) * p.kvDim + kvOff) + sub * KQ;
 #pragma unroll
-            for (int d4 = 0; d4 < KQ; d4++) kreg[d4] = krow[d4];
+            for (int u = 0; u < VU; u++) kreg[u] = Kbase[(size_t)min(tile + tg + u * TG, lastRow) * rowStride];
 #pragma unroll
-            for (int u = 0; u < VU; u++) vreg[u] = Vbase[(size_t)min(tile + tg + u * TG, lastRow) * vStride];
+            for (int u = 0; u < VU; u++) vreg[u] = Vbase[(size_t)min(tile + tg + u * TG, lastRow) * rowStride];
         }
-        float s[GMAX];
-#pragma unroll
-        for (int g = 0; g < GMAX; g++) s[g] = 0.f;
-#pragma unroll
-        for (int d4 = 0; d4 < KQ; d4++) {
-#pragma unroll
-            for (int g = 0; g < GMAX; g++) {
-                float4 q4 = q_s4[g * (HD / 4) + sub * KQ + d4];
-                s[g] = fmaf(q4.x, kreg[d4].x, s[g]);
-                s[g] = fmaf(q4.y, kreg[d4].y, s[g]);
-                s[g] = fmaf(q4.z, kreg[d4].z, s[g]);
-                s[g] = fmaf(q4.w, kreg[d4].w, s[g]);
-            }
-        }
-        if (LPP == 2) {
-#pragma unroll
-            for (int g = 0; g < GMAX; g++) s[g] += dpp_f<0xB1>(s[g]);      // the other half of the row
-        }
-        // tile maxima of all heads with one barrier, then the sums with another
-        float sv[GMAX];
+        float sc[GMAX][VU];
+        float tmax[GMAX];
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
-            sv[g] = active ? s[g] * scale : -INFINITY;
-            float wm = wave_max(sv[g]);
-            if (lane == 0) wred[0][g][wave] = wm;
+            tmax[g] = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < VU; u++) {
+                float d = q4[g].x * kreg[u].x;
+                d = fmaf(q4[g].y, kreg[u].y, d);
+                d = fmaf(q4[g].z, kreg[u].z, d);
+                d = fmaf(q4[g].w, kreg[u].w, d);
+                d = row_sum<LPR>(d);
+                sc[g][u] = (tile + tg + u * TG < t1) ? d * scale : -INFINITY;
+                tmax[g] = fmaxf(tmax[g], sc[g][u]);
+            }
+            tmax[g] = tg_max<LPR>(tmax[g]);
+            if ((tid & 63) == 0) wred[par][g][wave] = tmax[g];
         }
         __syncthreads();
-        float corr[GMAX];
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
-            float tmax = fmaxf(fmaxf(wred[0][g][0], wred[0][g][1]), fmaxf(wred[0][g][2], wred[0][g][3]));
-            float mNew = fmaxf(m[g], tmax);
-            corr[g] = expf(m[g] - mNew);                   // first tile: exp(-inf) = 0
-            float pv = active ? expf(sv[g] - mNew) : 0.f;
-            sc[g][pIdx] = pv;
-            float ws = wave_sum(sub == 0 ? pv : 0.f);
-            if (lane == 0) wred[1][g][wave] = ws;
+            const float tm = fmaxf(fmaxf(wred[par][g][0], wred[par][g][1]), fmaxf(wred[par][g][2], wred[par][g][3]));
+            const float mNew = fmaxf(m[g], tm);            // finite: every tile holds at least one valid position
+            const float corr = expf(m[g] - mNew);          // first tile: exp(-inf) = 0
             m[g] = mNew;
-        }
-        __syncthreads();
+            float ps = 0.f;
+            float4 a = acc[g];
+            a.x *= corr; a.y *= corr; a.z *= corr; a.w *= corr;
 #pragma unroll
-        for (int g = 0; g < GMAX; g++) {
-            float tsum = (wred[1][g][0] + wred[1][g][1]) + (wred[1][g][2] + wred[1][g][3]);
-            l[g] = l[g] * corr[g] + tsum;
-            acc[g].x *= corr[g]; acc[g].y *= corr[g]; acc[g].z *= corr[g]; acc[g].w *= corr[g];
-        }
-        // P.V: this thread's VU rows of the tile are already in registers
-#pragma unroll
-        for (int u = 0; u < VU; u++) {
-            int tt = tg + u * TG;
-            if (tt < tileLen) {
-#pragma unroll
-                for (int g = 0; g < GMAX; g++) {
-                    float w = sc[g][tt];
-                    acc[g].x = fmaf(w, vreg[u].x, acc[g].x);
-                    acc[g].y = fmaf(w, vreg[u].y, acc[g].y);
-                    acc[g].z = fmaf(w, vreg[u].z, acc[g].z);
-                    acc[g].w = fmaf(w, vreg[u].w, acc[g].w);
-                }
+            for (int u = 0; u < VU; u++) {
+                const float pv = expf(sc[g][u] - mNew);    // masked rows: exp(-inf) = 0
+                ps += pv;
+                a.x = fmaf(pv, vreg[u].x, a.x);
+                a.y = fmaf(pv, vreg[u].y, a.y);
+                a.z = fmaf(pv, vreg[u].z, a.z);
+                a.w = fmaf(pv, vreg[u].w, a.w);
             }
+            acc[g] = a;
+            l[g] = l[g] * corr + ps;
         }
-        __syncthreads();                               // sc and wred are reused by the next tile
+        par ^= 1;                                          // the next tile's maxima go to the other buffer
     }
 
+    // ---- reduce the per-thread partials over the row groups: in the wave, then across waves ----
 #pragma unroll
-    for (int g = 0; g < GMAX; g++) accbuf[tg][g][dl] = acc[g];
+    for (int g = 0; g < GMAX; g++) {
+        acc[g].x = tg_sum<LPR>(acc[g].x); acc[g].y = tg_sum<LPR>(acc[g].y);
+        acc[g].z = tg_sum<LPR>(acc[g].z); acc[g].w = tg_sum<LPR>(acc[g].w);
+        l[g] = tg_sum<LPR>(l[g]);
+        if ((tid & 63) < LPR) accbuf[wave][g][dl] = acc[g];
+        if ((tid & 63) == 0) lbuf[wave][g] = l[g];
+    }
     __syncthreads();
     for (int i = tid; i < gn * LPR; i += WG) {
         int g = i / LPR, d4 = i % LPR;
         float4 r = accbuf[0][g][d4];
 #pragma unroll
-        for (int k = 1; k < TG; k++) {
+        for (int k = 1; k < 4; k++) {
             float4 a = accbuf[k][g][d4];
             r.x += a.x; r.y += a.y; r.z += a.z; r.w += a.w;
         }
-        // m[], l[] are replicated in every thread; pick g's with a select chain
-        float lg = l[0], mg_ = m[0];
+        // lbuf holds lane 0's column of each wave: every row's probability exactly once
+        const float lg = (lbuf[0][g] + lbuf[1][g]) + (lbuf[2][g] + lbuf[3][g]);
+        float mg_ = m[0];
 #pragma unroll
-        for (int k = 1; k < GMAX; k++) if (g == k) { lg = l[k]; mg_ = m[k]; }
+        for (int k = 1; k < GMAX; k++) if (g == k) mg_ = m[k];
         int h = h0 + g;
         if (nsplit == 1) {
             float4 o;
@@ -801,7 +808,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 static int attention_gmax(int G, int heads) {
     int want = heads > 0 ? heads : G;
     if (want > G) want = G;
-    return want >= 8 ? 8 : (want > 2 ? (want > 4 ? 8 : 4) : (want == 2 ? 2 : 1));
+    return want >= 3 ? 4 : (want == 2 ? 2 : 1);      // scores of GMAX heads x 16 rows live in registers: at most 4
 }
 
 template <int HD>
@@ -813,8 +820,7 @@ static hipError_t launch_attn_hd(const AttnParams& p, hipStream_t s) {
     switch (gmax) {
     case 1: hipLaunchKernelGGL((attn_decode_kernel<HD, 1>), grid, dim3(WG), 0, s, p); break;
     case 2: hipLaunchKernelGGL((attn_decode_kernel<HD, 2>), grid, dim3(WG), 0, s, p); break;
-    case 4: hipLaunchKernelGGL((attn_decode_kernel<HD, 4>), grid, dim3(WG), 0, s, p); break;
-    default: hipLaunchKernelGGL((attn_decode_kernel<HD, 8>), grid, dim3(WG), 0, s, p); break;
+    default: hipLaunchKernelGGL((attn_decode_kernel<HD, 4>), grid, dim3(WG), 0, s, p); break;
     }
     return hipGetLastError();
 }
