@@ -99,7 +99,7 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
     // is a measurable part of a small matvec's latency.
     const int half0 = headDim / 2;
     const int attnTile = headDim == 128 ? 128 : 256;      // positions per attention tile
-    f->splitLen = attnTile * ((maxSeq + attnTile * 32 - 1) / (attnTile * 32));
+    f->splitLen = attnTile * ((maxSeq + attnTile * 64 - 1) / (attnTile * 64));      // at most 64 splits
     f->smax = (maxSeq + f->splitLen - 1) / f->splitLen;
     f->attnHeadsPerWG = maxSeq <= 1024 ? 1 : 0;
     f->amaxParts = 4096;

@@ -578,10 +578,10 @@ hipError_t launch_matvec_generic_q8(const float* act, const void* w, const float
 // first tile's K and V rows are requested before the position is known (rows
 // past the end are clamped and masked): the critical path is one memory latency.
 //
-// K and V use the same register layout: a row of the head is spread over LPR =
-// HD/4 lanes (one float4 each, so a wave's load covers whole rows: coalesced),
-// and a thread holds VU = 16 rows of the tile, tg + u*TG.  A score is the
-// lane's 4-term partial product reduced over the row's lanes by DPP; every lane
+// K and V use the same register layout: a row of the head is spread over 16
+// lanes (one DPP row; HD/64 float4s each, lanes 16 bytes apart: coalesced), and
+// a thread holds the tile's rows tg + u*16.  A score is the lane's partial
+// product reduced over the row's lanes by DPP; every lane
 // of a row ends up with the score, which is exactly where P.V needs it -- the
 // probabilities never leave registers.  Per tile there is one barrier (the
 // tile maximum across waves); the running sum and the output stay per-thread
@@ -595,39 +595,36 @@ __device__ __forceinline__ float ld_agent(const float* p) {
 __device__ __forceinline__ void st_agent(float* p, float v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// Sum over the LPR lanes that hold one row (16: one DPP row; 32: two).  Every step adds a lane's
-// value to its mirror partner's (quad_perm, then row_half_mirror = 0x141, row_mirror = 0x140), so
-// both partners compute the same commutative sum: all lanes of the row end with the same bits,
-// which keeps exp(score - max) identical across the lanes that apply it.
-template <int LPR>
-__device__ __forceinline__ float row_sum(float v) {
+// Sum over the 16 lanes (one DPP row) that hold a K/V row.  Every step adds a lane's value to its
+// mirror partner's (quad_perm, then row_half_mirror = 0x141, row_mirror = 0x140), so both partners
+// compute the same commutative sum: all lanes of the row end with the same bits, which keeps
+// exp(score - max) identical across the lanes that apply it.
+__device__ __forceinline__ float row_sum16(float v) {
     v += dpp_f<0xB1>(v);
     v += dpp_f<0x4E>(v);
     v += dpp_f<0x141>(v);
     v += dpp_f<0x140>(v);
-    if (LPR == 32) v += __shfl_xor(v, 16, 64);
     return v;
 }
-// combine a per-thread value over the row groups (tg) that share a wave
-template <int LPR>
+// combine a per-thread value over the four row groups (tg) that share a wave
 __device__ __forceinline__ float tg_max(float v) {
-    if (LPR == 16) v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
     return fmaxf(v, __shfl_xor(v, 32, 64));
 }
-template <int LPR>
 __device__ __forceinline__ float tg_sum(float v) {
-    if (LPR == 16) v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 16, 64);
     return v + __shfl_xor(v, 32, 64);
 }
 
 template <int HD, int GMAX>
 __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
-    constexpr int LPR = HD / 4;        // lanes per K/V row
-    constexpr int TG = WG / LPR;       // rows in flight per load step
-    constexpr int VU = 16;             // rows per thread and tile
+    constexpr int LPR = 16;            // lanes per K/V row: one DPP row
+    constexpr int NF = HD / 64;        // float4s of a row per lane (float4 index j*16 + dl)
+    constexpr int TG = WG / LPR;       // rows in flight per load step (16)
+    constexpr int VU = 16 / NF;        // rows per thread and tile
     constexpr int TILE = TG * VU;      // positions per tile (256 for head size 64, 128 for 128)
     __shared__ float wred[2][GMAX][4];
-    __shared__ float4 accbuf[4][GMAX][LPR];
+    __shared__ float4 accbuf[4][GMAX][HD / 4];
     __shared__ float lbuf[4][GMAX];
     __shared__ int lastFlag;
 
@@ -649,17 +646,23 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     const float4* Vbase = reinterpret_cast<const float4*>(p.Vc + kvOff) + dl;
 
     // ---- everything that does not need the position goes out first ----
-    float4 q4[GMAX];
+    float4 q4[GMAX][NF];
 #pragma unroll
-    for (int g = 0; g < GMAX; g++) {           // heads past gn work on zeros and are dropped at the end
-        q4[g] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (g < gn) q4[g] = reinterpret_cast<const float4*>(p.q + (size_t)(h0 + g) * HD)[dl];
-    }
-    float4 kreg[VU], vreg[VU];
+    for (int g = 0; g < GMAX; g++)             // heads past gn work on zeros and are dropped at the end
 #pragma unroll
-    for (int u = 0; u < VU; u++) kreg[u] = Kbase[(size_t)min(t0 + tg + u * TG, lastRow) * rowStride];
+        for (int j = 0; j < NF; j++) {
+            q4[g][j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (g < gn) q4[g][j] = reinterpret_cast<const float4*>(p.q + (size_t)(h0 + g) * HD)[j * 16 + dl];
+        }
+    float4 kreg[VU][NF], vreg[VU][NF];
 #pragma unroll
-    for (int u = 0; u < VU; u++) vreg[u] = Vbase[(size_t)min(t0 + tg + u * TG, lastRow) * rowStride];
+    for (int u = 0; u < VU; u++)
+#pragma unroll
+        for (int j = 0; j < NF; j++) kreg[u][j] = Kbase[(size_t)min(t0 + tg + u * TG, lastRow) * rowStride + j * 16];
+#pragma unroll
+    for (int u = 0; u < VU; u++)
+#pragma unroll
+        for (int j = 0; j < NF; j++) vreg[u][j] = Vbase[(size_t)min(t0 + tg + u * TG, lastRow) * rowStride + j * 16];
 
     const int pos = p.state ? p.state->pos : p.posImm;
     const int len = pos + 1;
@@ -669,35 +672,46 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 
     const float scale = 1.0f / sqrtf((float)HD);     // mongoose.cu:867 rsqrtf(headDim)
     float m[GMAX], l[GMAX];                           // m: workgroup-wide running max; l, acc: this thread's rows only
-    float4 acc[GMAX];
+    float4 acc[GMAX][NF];
 #pragma unroll
-    for (int g = 0; g < GMAX; g++) { m[g] = -INFINITY; l[g] = 0.f; acc[g] = make_float4(0.f, 0.f, 0.f, 0.f); }
+    for (int g = 0; g < GMAX; g++) {
+        m[g] = -INFINITY; l[g] = 0.f;
+#pragma unroll
+        for (int j = 0; j < NF; j++) acc[g][j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
 
     int par = 0;
     for (int tile = t0; tile < t1; tile += TILE) {
         if (tile != t0) {
 #pragma unroll
-            for (int u = 0; u < VU; u++) kreg[u] = Kbase[(size_t)min(tile + tg + u * TG, lastRow) * rowStride];
+            for (int u = 0; u < VU; u++)
 #pragma unroll
-            for (int u = 0; u < VU; u++) vreg[u] = Vbase[(size_t)min(tile + tg + u * TG, lastRow) * rowStride];
+                for (int j = 0; j < NF; j++) kreg[u][j] = Kbase[(size_t)min(tile + tg + u * TG, lastRow) * rowStride + j * 16];
+#pragma unroll
+            for (int u = 0; u < VU; u++)
+#pragma unroll
+                for (int j = 0; j < NF; j++) vreg[u][j] = Vbase[(size_t)min(tile + tg + u * TG, lastRow) * rowStride + j * 16];
         }
         float sc[GMAX][VU];
-        float tmax[GMAX];
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
-            tmax[g] = -INFINITY;
+            float tmax = -INFINITY;
 #pragma unroll
             for (int u = 0; u < VU; u++) {
-                float d = q4[g].x * kreg[u].x;
-                d = fmaf(q4[g].y, kreg[u].y, d);
-                d = fmaf(q4[g].z, kreg[u].z, d);
-                d = fmaf(q4[g].w, kreg[u].w, d);
-                d = row_sum<LPR>(d);
+                float d = 0.f;
+#pragma unroll
+                for (int j = 0; j < NF; j++) {
+                    d = fmaf(q4[g][j].x, kreg[u][j].x, d);
+                    d = fmaf(q4[g][j].y, kreg[u][j].y, d);
+                    d = fmaf(q4[g][j].z, kreg[u][j].z, d);
+                    d = fmaf(q4[g][j].w, kreg[u][j].w, d);
+                }
+                d = row_sum16(d);
                 sc[g][u] = (tile + tg + u * TG < t1) ? d * scale : -INFINITY;
-                tmax[g] = fmaxf(tmax[g], sc[g][u]);
+                tmax = fmaxf(tmax, sc[g][u]);
             }
-            tmax[g] = tg_max<LPR>(tmax[g]);
-            if ((tid & 63) == 0) wred[par][g][wave] = tmax[g];
+            tmax = tg_max(tmax);
+            if ((tid & 63) == 0) wred[par][g][wave] = tmax;
         }
         __syncthreads();
 #pragma unroll
@@ -707,18 +721,20 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
             const float corr = expf(m[g] - mNew);          // first tile: exp(-inf) = 0
             m[g] = mNew;
             float ps = 0.f;
-            float4 a = acc[g];
-            a.x *= corr; a.y *= corr; a.z *= corr; a.w *= corr;
+#pragma unroll
+            for (int j = 0; j < NF; j++) { acc[g][j].x *= corr; acc[g][j].y *= corr; acc[g][j].z *= corr; acc[g][j].w *= corr; }
 #pragma unroll
             for (int u = 0; u < VU; u++) {
                 const float pv = expf(sc[g][u] - mNew);    // masked rows: exp(-inf) = 0
                 ps += pv;
-                a.x = fmaf(pv, vreg[u].x, a.x);
-                a.y = fmaf(pv, vreg[u].y, a.y);
-                a.z = fmaf(pv, vreg[u].z, a.z);
-                a.w = fmaf(pv, vreg[u].w, a.w);
+#pragma unroll
+                for (int j = 0; j < NF; j++) {
+                    acc[g][j].x = fmaf(pv, vreg[u][j].x, acc[g][j].x);
+                    acc[g][j].y = fmaf(pv, vreg[u][j].y, acc[g][j].y);
+                    acc[g][j].z = fmaf(pv, vreg[u][j].z, acc[g][j].z);
+                    acc[g][j].w = fmaf(pv, vreg[u][j].w, acc[g][j].w);
+                }
             }
-            acc[g] = a;
             l[g] = l[g] * corr + ps;
         }
         par ^= 1;                                          // the next tile's maxima go to the other buffer
@@ -727,15 +743,19 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     // ---- reduce the per-thread partials over the row groups: in the wave, then across waves ----
 #pragma unroll
     for (int g = 0; g < GMAX; g++) {
-        acc[g].x = tg_sum<LPR>(acc[g].x); acc[g].y = tg_sum<LPR>(acc[g].y);
-        acc[g].z = tg_sum<LPR>(acc[g].z); acc[g].w = tg_sum<LPR>(acc[g].w);
-        l[g] = tg_sum<LPR>(l[g]);
-        if ((tid & 63) < LPR) accbuf[wave][g][dl] = acc[g];
+#pragma unroll
+        for (int j = 0; j < NF; j++) {
+            acc[g][j].x = tg_sum(acc[g][j].x); acc[g][j].y = tg_sum(acc[g][j].y);
+            acc[g][j].z = tg_sum(acc[g][j].z); acc[g][j].w = tg_sum(acc[g][j].w);
+            if ((tid & 63) < LPR) accbuf[wave][g][j * 16 + dl] = acc[g][j];
+        }
+        l[g] = tg_sum(l[g]);
         if ((tid & 63) == 0) lbuf[wave][g] = l[g];
     }
     __syncthreads();
-    for (int i = tid; i < gn * LPR; i += WG) {
-        int g = i / LPR, d4 = i % LPR;
+    constexpr int F4 = HD / 4;                             // float4s of a head
+    for (int i = tid; i < gn * F4; i += WG) {
+        int g = i / F4, d4 = i % F4;
         float4 r = accbuf[0][g][d4];
 #pragma unroll
         for (int k = 1; k < 4; k++) {
@@ -776,8 +796,8 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     __syncthreads();
     if (!lastFlag) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");     // drop cached copies of the other workgroups' partials
-    for (int i = tid; i < gn * LPR; i += WG) {
-        int g = i / LPR, d4 = i % LPR;
+    for (int i = tid; i < gn * F4; i += WG) {
+        int g = i / F4, d4 = i % F4;
         int h = h0 + g;
         const float* pm = p.pm + (size_t)h * p.smax;
         const float* pl = p.pl + (size_t)h * p.smax;
@@ -790,7 +810,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll 8
         for (int s = 0; s < nsplit; s++) {
             float w = expf(pm[s] - M);
-            float4 a = pa[(size_t)s * LPR];
+            float4 a = pa[(size_t)s * F4];
             den = fmaf(w, pl[s], den);
             num.x = fmaf(w, a.x, num.x); num.y = fmaf(w, a.y, num.y);
             num.z = fmaf(w, a.z, num.z); num.w = fmaf(w, a.w, num.w);
