@@ -159,7 +159,7 @@ def main():
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run three 256 MiB device copies (a kernel of known traffic, to scale rocprofv3 --pmc counters)")
     ap.add_argument("--prefill", type=int, default=0,
-                    help="also time a batched prefill of this many prompt tokens (Q8 configurations; extra 'prefill' object)")
+                    help="also time a batched prefill of this many prompt tokens (extra 'prefill' object)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
@@ -255,7 +255,7 @@ def main():
         b.Release()
 
     prefill = None
-    if args.prefill > 0 and s.fmt == "q8":
+    if args.prefill > 0:
         ptoks = E.synth_tokens(args.seed, 20_000_003, s.vocab, args.prefill)
         times = []
         for _ in range(4):                              # first call allocates the row buffers
@@ -264,7 +264,7 @@ def main():
             assert rc == 0, E.last_error()
             times.append(pms)
         pms = min(times[1:])
-        macs = sum((mat(n, k) - 4 * n) for n, k in
+        macs = sum(n * k for n, k in
                    [(s.dim, s.dim), (kv, s.dim), (kv, s.dim), (s.dim, s.dim), (s.ffnDim, s.dim), (s.ffnDim, s.dim),
                     (s.dim, s.ffnDim)]) * s.nLayers
         flops = 2.0 * macs * args.prefill

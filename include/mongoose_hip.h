@@ -226,7 +226,9 @@ int mg_profile_decode(mg_ctx* ctx, int token, int pos, int steps, unsigned class
  * here the seven projections of a layer over nTokens rows are MFMA GEMMs that
  * read the int8 weights exactly (int8 is exact in bf16) against activations
  * split into two bf16 terms, so the result stays within ~1e-5 of the
- * token-by-token path.  Q8 weights only (MG_E_UNSUPPORTED otherwise).
+ * token-by-token path.  Q4_0 weights are multiplied block by block (nibble - 8
+ * is exact in bf16; the fp16 block scale is applied in fp32).  q/k/v, and
+ * gate/up, of a layer must share one format (MG_E_UNSUPPORTED otherwise).
  * Positions pos0 .. pos0+nTokens-1 of the KV caches are written; the last
  * position goes through final norm, lm_head and argmax: *nextToken, logitsOut
  * [vocab] (both optional), and the device step state is left at pos0+nTokens

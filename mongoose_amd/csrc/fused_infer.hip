@@ -870,9 +870,11 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
     int rc = checkReady(this);
     if (rc) return rc;
     for (const auto& L : layers) {
-        const DevMat* ms[7] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.gate, &L.up, &L.down};
-        for (const DevMat* m : ms)
-            if (m->kind != WF_Q8) { set_error("Prefill: the GEMM path takes Q8 weights only"); return MG_E_UNSUPPORTED; }
+        // q/k/v and gate/up share a launch: one weight format each
+        if (L.wq.kind != L.wk.kind || L.wk.kind != L.wv.kind || L.gate.kind != L.up.kind) {
+            set_error("Prefill: q/k/v (and gate/up) of a layer must share one weight format");
+            return MG_E_UNSUPPORTED;
+        }
     }
     rc = ensurePrefill(nTokens);
     if (rc) return rc;
@@ -883,8 +885,7 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
     if (embedKind == 1 || embedKind == 2) {
         HIPCHK(launch_embed_rows(embedKind, embedTable, nullptr, pfTokens, pfX, T, dim, vocabSize, stream));
     } else {
-        if (lmHead.kind != WF_Q8) { set_error("Prefill: tied embedding needs a Q8 lm_head"); return MG_E_UNSUPPORTED; }
-        HIPCHK(launch_embed_rows(0, lmHead.w, lmHead.scales, pfTokens, pfX, T, dim, vocabSize, stream));
+        HIPCHK(launch_embed_rows(lmHead.kind == WF_Q8 ? 0 : 3, lmHead.w, lmHead.scales, pfTokens, pfX, T, dim, vocabSize, stream));
     }
     for (int l = 0; l < nLayers; l++) {
         const LayerWeights& L = layers[l];
@@ -895,19 +896,19 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
         g.T = T; g.Ahi = static_cast<const unsigned short*>(pfHi); g.Alo = static_cast<const unsigned short*>(pfLo);
         g.partial = pfPartial;
         HIPCHK(launch_split_rows(pfX, L.norm1, eps, T, dim, pfHi, pfLo, stream));
-        g.K = dim; g.nseg = 3;
+        g.K = dim; g.nseg = 3; g.q4 = L.wq.kind == WF_Q4P;
         g.seg[0] = seg(L.wq, L.bq, pfQ); g.seg[1] = seg(L.wk, L.bk, pfK); g.seg[2] = seg(L.wv, L.bv, pfV);
         HIPCHK(launch_gemm_q8(g, 0, stream));
         HIPCHK(launch_rope_store_rows(pfQ, pfK, pfV, kCache[l], vCache[l], cosTab, sinTab, pos0, T, dim, kvDim, headDim, stream));
         HIPCHK(launch_prefill_attention(pfQ, kCache[l], vCache[l], pfAttn, T, pos0, maxSeq, dim, kvDim, nHeads, nKVHeads, headDim, stream));
         HIPCHK(launch_split_rows(pfAttn, nullptr, eps, T, dim, pfHi, pfLo, stream));
-        g.K = dim; g.nseg = 1; g.seg[0] = seg(L.wo, nullptr, pfX);
+        g.K = dim; g.nseg = 1; g.q4 = L.wo.kind == WF_Q4P; g.seg[0] = seg(L.wo, nullptr, pfX);
         HIPCHK(launch_gemm_q8(g, 1, stream));
         HIPCHK(launch_split_rows(pfX, L.norm2, eps, T, dim, pfHi, pfLo, stream));
-        g.K = dim; g.nseg = 2; g.seg[0] = seg(L.gate, nullptr, pfGate); g.seg[1] = seg(L.up, nullptr, pfUp);
+        g.K = dim; g.nseg = 2; g.q4 = L.gate.kind == WF_Q4P; g.seg[0] = seg(L.gate, nullptr, pfGate); g.seg[1] = seg(L.up, nullptr, pfUp);
         HIPCHK(launch_gemm_q8(g, 0, stream));
         HIPCHK(launch_swiglu_split(pfGate, pfUp, T, ffnDim, pfHi, pfLo, stream));
-        g.K = ffnDim; g.nseg = 1; g.seg[0] = seg(L.down, nullptr, pfX);
+        g.K = ffnDim; g.nseg = 1; g.q4 = L.down.kind == WF_Q4P; g.seg[0] = seg(L.down, nullptr, pfX);
         HIPCHK(launch_gemm_q8(g, 1, stream));
     }
     // the last position continues on the decode path: final norm, lm_head, greedy token, state -> pos0 + T

@@ -18,10 +18,12 @@ hipError_t launch_rope_store_rows(float* q, const float* k, const float* v, floa
 // Causal attention of T query rows [T,dim] (rotated) at positions pos0.. over cache rows [0, pos0+T); out [T,dim].
 hipError_t launch_prefill_attention(const float* q, const float* Kc, const float* Vc, float* out, int T, int pos0, int rowLimit,
                                     int dim, int kvDim, int nHeads, int nKVHeads, int headDim, hipStream_t s);
-// Embedding rows of T tokens: kind 0 = Q8 row * scale, 1 = fp16 table, 2 = fp32 table.
+// Embedding rows of T tokens: kind 0 = Q8 row * scale, 1 = fp16 table, 2 = fp32 table, 3 = Q4_0 split-layout row.
 hipError_t launch_embed_rows(int kind, const void* table, const float* scales, const int* tokens, float* x, int T, int dim,
                              int vocab, hipStream_t s);
 // One launch: for each of up to three weight matrices, Y[T,N] (+)= (Ahi + Alo)[T,K] . W[N,K]^T * scales[n] (+ bias[n]).
+// q4 = 0: W int8 [N,K] with float scales[N].  q4 = 1: W is Q4_0 in the split layout (16-byte nibble groups
+// [N, K/32], then fp16 d [N, K/32]), scales NULL.
 // K a multiple of 32; W, Ahi, Alo 16-byte aligned; Ahi/Alo in the blocked layout of launch_split_rows.
 struct GemmSeg { const signed char* W; const float* scales; const float* bias; float* Y; int N; int tile0; };
 struct GemmParams {
@@ -30,6 +32,7 @@ struct GemmParams {
     const unsigned short* Ahi;
     const unsigned short* Alo;
     int T, K;
+    int q4;
     float* partial;   // workspace of gemm_partial_floats() floats for K-split partial sums (NULL: never split K)
     // filled by the launcher
     int nTiles, splitK, stepsPerSplit, ldPartial;

@@ -125,7 +125,8 @@ hipError_t launch_rope_store_rows(float* q, const float* k, const float* v, floa
     return hipGetLastError();
 }
 
-// Embedding rows of T tokens from the tied Q8 table (kind 0) or an fp16 (1) / fp32 (2) table.
+// Embedding rows of T tokens from the tied Q8 table (kind 0), an fp16 (1) / fp32 (2) table, or the
+// tied Q4_0 table in the split layout (3).
 __global__ void embed_rows_kernel(int kind, const void* table, const float* scales, const int* tokens, float* x, int dim, int vocab) {
     int tok = tokens[blockIdx.x];
     tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
@@ -133,7 +134,15 @@ __global__ void embed_rows_kernel(int kind, const void* table, const float* scal
     for (int i = threadIdx.x; i < dim; i += blockDim.x) {
         if (kind == 0) o[i] = (float)static_cast<const signed char*>(table)[(size_t)tok * dim + i] * scales[tok];
         else if (kind == 1) o[i] = (float)__builtin_bit_cast(_Float16, static_cast<const unsigned short*>(table)[(size_t)tok * dim + i]);
-        else o[i] = static_cast<const float*>(table)[(size_t)tok * dim + i];
+        else if (kind == 2) o[i] = static_cast<const float*>(table)[(size_t)tok * dim + i];
+        else {
+            const unsigned char* base = static_cast<const unsigned char*>(table);
+            const int nb = dim >> 5, b = i >> 5, e = i & 31;
+            const unsigned char byte = base[((size_t)tok * nb + b) * 16 + (e & 15)];
+            const int nib = e < 16 ? (byte & 15) : (byte >> 4);
+            const unsigned short dh = reinterpret_cast<const unsigned short*>(base + (size_t)vocab * (dim >> 1))[(size_t)tok * nb + b];
+            o[i] = (float)(nib - 8) * (float)__builtin_bit_cast(_Float16, dh);
+        }
     }
 }
 hipError_t launch_embed_rows(int kind, const void* table, const float* scales, const int* tokens, float* x, int T, int dim,
@@ -304,16 +313,27 @@ __device__ __forceinline__ unsigned pack_bf16_exact(float lo, float hi) {
 // element, W one), and it is that traffic which bounds the kernel: 256 x 256 tiles with 1024
 // threads where the problem is large enough, 64/128 x 128 with 256 threads for short prompts.
 // MODE 0: Y = acc*scale (+bias)   1: Y += acc*scale   2: raw partial sums of one K split into p.partial
-template <int BM, int BN, int NT, int MODE>
+//
+// Q4 = 1 reads Q4_0 weights in the split layout (16-byte nibble groups [N, K/32], then fp16 d
+// [N, K/32]).  nibble - 8 is exact in bf16; the block scale cannot be folded into a bf16 weight
+// without loss, so each 32-k block is multiplied into a scratch accumulator (two MFMA steps, hi and
+// lo) and added to the running sums as d * scratch: 16 FMAs per MFMA block and Q4_0 block.  Element
+// order in a block (GGML): low nibble of byte j = element j, high nibble = element j + 16, so the 8
+// consecutive elements a fragment needs are the low or the high nibbles of 8 consecutive bytes.
+template <int Q4, int BM, int BN, int NT, int MODE>
 __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
     constexpr int WN = BN / 64, WM = (NT / 64) / WN;
     constexpr int MI = BM / WM / 32;             // 32-row MFMA blocks per wave
     constexpr int AR = BM * 8 / NT;              // 16-byte segments per thread and A plane
-    constexpr int BR = BN * 4 / NT;              // 16-byte segments per thread of W
-    static_assert(MI >= 1 && AR >= 1 && BR >= 1, "tile too small for the thread count");
+    constexpr int WSEG = Q4 ? 2 : 4;             // 16-byte segments of W per row and K step
+    constexpr int BR = BN * WSEG / NT > 0 ? BN * WSEG / NT : 1;
+    constexpr int WSTRIDE = Q4 ? 48 : B_STRIDE;  // bytes per LDS row of W
+    static_assert(MI >= 1 && AR >= 1, "tile too small for the thread count");
+    static_assert(BN * WSEG % NT == 0 || BN * WSEG < NT, "W segments do not divide over the threads");
     __shared__ __attribute__((aligned(16))) unsigned short sAh[BM * A_STRIDE];
     __shared__ __attribute__((aligned(16))) unsigned short sAl[BM * A_STRIDE];
-    __shared__ __attribute__((aligned(16))) signed char sB[BN * B_STRIDE];
+    __shared__ __attribute__((aligned(16))) signed char sB[BN * WSTRIDE];
+    __shared__ float sD[Q4 ? BN * 2 : 1];         // Q4_0: the step's two block scales of every row
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
@@ -334,7 +354,8 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
 
     // global -> LDS: A row = tid/8 (+NT/8 per pass), segment tid%8 (8 bf16) ; W row = tid/4 (+NT/4), segment tid%4 (16 int8)
     const int aRow = tid >> 3, aSeg = tid & 7;
-    const int bRow = tid >> 2, bSeg = tid & 3;
+    const int bRow = Q4 ? tid >> 1 : tid >> 2, bSeg = Q4 ? tid & 1 : tid & 3;
+    const bool bActive = bRow < BN;                  // Q4_0 with more threads than segments: the rest only load A
     const unsigned short* aHiP[AR]; const unsigned short* aLoP[AR];
     const int planeRows = ((T + 127) >> 7) << 7;     // the planes are padded to whole 128-row blocks, not to BM
 #pragma unroll
@@ -346,7 +367,14 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
     }
     const signed char* bP[BR];
 #pragma unroll
-    for (int r = 0; r < BR; r++) bP[r] = sg.W + (size_t)min(n0 + bRow + (NT / 4) * r, N - 1) * K + bSeg * 16;
+    for (int r = 0; r < BR; r++) {
+        const int row = min(n0 + bRow + (NT / WSEG) * r, N - 1);
+        bP[r] = Q4 ? sg.W + ((size_t)row * (K >> 5) + bSeg) * 16 : sg.W + (size_t)row * K + bSeg * 16;
+    }
+    // Q4_0: thread t < BN also fetches row t's two block scales of the step
+    const unsigned short* dP = nullptr;
+    if (Q4 && tid < BN)
+        dP = reinterpret_cast<const unsigned short*>(sg.W + (size_t)N * (K >> 1)) + (size_t)min(n0 + tid, N - 1) * (K >> 5);
 
     float16_t acc[MI][2];
 #pragma unroll
@@ -357,16 +385,22 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
     int4 gAh[AR], gAl[AR], gB[BR];
+    unsigned short gD[2] = {0, 0};
     const int4 zero4 = make_int4(0, 0, 0, 0);
     auto gload = [&](int k0) {       // K is a multiple of 32: a last half step reads zeros past the end
-        const bool okA = k0 + aSeg * 8 < K, okB = k0 + bSeg * 16 < K;
+        const bool okA = k0 + aSeg * 8 < K;
+        const bool okB = bActive && (Q4 ? k0 + bSeg * 32 < K : k0 + bSeg * 16 < K);
 #pragma unroll
         for (int r = 0; r < AR; r++) {
             gAh[r] = okA ? *reinterpret_cast<const int4*>(aHiP[r] + (size_t)k0 * 128) : zero4;   // 8192 elements per K step
             gAl[r] = okA ? *reinterpret_cast<const int4*>(aLoP[r] + (size_t)k0 * 128) : zero4;
         }
 #pragma unroll
-        for (int r = 0; r < BR; r++) gB[r] = okB ? *reinterpret_cast<const int4*>(bP[r] + k0) : zero4;
+        for (int r = 0; r < BR; r++) gB[r] = okB ? *reinterpret_cast<const int4*>(bP[r] + (Q4 ? k0 >> 1 : k0)) : zero4;
+        if (Q4 && dP) {
+            gD[0] = dP[k0 >> 5];
+            gD[1] = k0 + 32 < K ? dP[(k0 >> 5) + 1] : (unsigned short)0;
+        }
     };
     if (stepBeg < stepEnd) gload(stepBeg * BK);
     for (int step = stepBeg; step < stepEnd; step++) {
@@ -377,9 +411,56 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
             *reinterpret_cast<int4*>(&sAl[(aRow + (NT / 8) * r) * A_STRIDE + aSeg * 8]) = gAl[r];
         }
 #pragma unroll
-        for (int r = 0; r < BR; r++) *reinterpret_cast<int4*>(&sB[(bRow + (NT / 4) * r) * B_STRIDE + bSeg * 16]) = gB[r];
+        for (int r = 0; r < BR; r++)
+            if (bActive) *reinterpret_cast<int4*>(&sB[(bRow + (NT / WSEG) * r) * WSTRIDE + bSeg * 16]) = gB[r];
+        if (Q4 && tid < BN) {
+            sD[tid * 2] = (float)__builtin_bit_cast(_Float16, gD[0]);
+            sD[tid * 2 + 1] = (float)__builtin_bit_cast(_Float16, gD[1]);
+        }
         __syncthreads();
         if (step + 1 < stepEnd) gload((step + 1) * BK);       // next tile in flight while this one is multiplied
+        if (Q4) {
+            float16_t zero16;
+#pragma unroll
+            for (int e = 0; e < 16; e++) zero16[e] = 0.f;
+#pragma unroll
+            for (int bl = 0; bl < 2; bl++) {               // the step's two Q4_0 blocks
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int nrow = wn * 64 + j * 32 + (lane & 31);
+                    const float d = sD[nrow * 2 + bl];
+                    // this lane's 8 elements of each 16-k half: e = 16*h2 + 8*(lane/32) -> bytes (e & 8).., nibble e >= 16
+                    bf16x8_t b[2];
+#pragma unroll
+                    for (int h2 = 0; h2 < 2; h2++) {
+                        const int e0 = 16 * h2 + 8 * (lane >> 5);
+                        const int2 w = *reinterpret_cast<const int2*>(&sB[nrow * WSTRIDE + bl * 16 + (e0 & 8)]);
+                        const unsigned sh = h2 ? 4u : 0u;   // elements 16..31 are the high nibbles
+                        const unsigned n0v = ((unsigned)w.x >> sh) & 0x0f0f0f0fu, n1v = ((unsigned)w.y >> sh) & 0x0f0f0f0fu;
+                        uint4 u;
+                        u.x = pack_bf16_exact((float)(n0v & 0xff) - 8.0f, (float)((n0v >> 8) & 0xff) - 8.0f);
+                        u.y = pack_bf16_exact((float)((n0v >> 16) & 0xff) - 8.0f, (float)(n0v >> 24) - 8.0f);
+                        u.z = pack_bf16_exact((float)(n1v & 0xff) - 8.0f, (float)((n1v >> 8) & 0xff) - 8.0f);
+                        u.w = pack_bf16_exact((float)((n1v >> 16) & 0xff) - 8.0f, (float)(n1v >> 24) - 8.0f);
+                        b[h2] = __builtin_bit_cast(bf16x8_t, u);
+                    }
+#pragma unroll
+                    for (int i = 0; i < MI; i++) {
+                        float16_t t = zero16;
+#pragma unroll
+                        for (int h2 = 0; h2 < 2; h2++) {
+                            const int arow = (wm * (BM / WM) + i * 32 + (lane & 31)) * A_STRIDE + bl * 32 + h2 * 16 + 8 * (lane >> 5);
+                            bf16x8_t ah = *reinterpret_cast<const bf16x8_t*>(&sAh[arow]);
+                            bf16x8_t al = *reinterpret_cast<const bf16x8_t*>(&sAl[arow]);
+                            t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, b[h2], t, 0, 0, 0);
+                            t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, b[h2], t, 0, 0, 0);
+                        }
+#pragma unroll
+                        for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf(d, t[e], acc[i][j][e]);
+                    }
+                }
+            }
+        } else {
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ks++) {
             const int kk = ks * 16 + 8 * (lane >> 5);
@@ -406,6 +487,7 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
                 }
             }
         }
+        }
     }
 #pragma unroll
     for (int j = 0; j < 2; j++) {
@@ -424,7 +506,7 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
             continue;
         }
         if (n >= N) continue;
-        const float sc = sg.scales[n];
+        const float sc = Q4 ? 1.0f : sg.scales[n];
         const float bi = sg.bias ? sg.bias[n] : 0.f;
 #pragma unroll
         for (int i = 0; i < MI; i++) {
@@ -458,7 +540,7 @@ __global__ __launch_bounds__(PWG) void gemm_reduce_kernel(GemmParams p, int BN, 
     const float* src = p.partial + (size_t)m * p.ldPartial + c;
     float v = 0.f;
     for (int s = 0; s < p.splitK; s++) v += src[(size_t)s * p.T * p.ldPartial];
-    v = v * sg.scales[n] + (sg.bias ? sg.bias[n] : 0.f);
+    v = v * (sg.scales ? sg.scales[n] : 1.0f) + (sg.bias ? sg.bias[n] : 0.f);
     float* dst = sg.Y + (size_t)m * sg.N + n;
     if (residual) v = *dst + v;
     *dst = v;
@@ -466,24 +548,25 @@ __global__ __launch_bounds__(PWG) void gemm_reduce_kernel(GemmParams p, int BN, 
 
 size_t gemm_partial_floats() { return (size_t)320 * 256 * 256; }
 
-hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s) {
-    if (p.T <= 0 || p.nseg < 1 || p.nseg > 3) return p.T <= 0 ? hipSuccess : hipErrorInvalidValue;
-    if (p.K <= 0 || p.K % 32 != 0) return hipErrorInvalidValue;
-    for (int i = 0; i < p.nseg; i++) if (p.seg[i].N <= 0) return hipErrorInvalidValue;
+template <int Q4>
+static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
     auto count = [&](int bn) {
         int tiles = 0;
         for (int i = 0; i < p.nseg; i++) { p.seg[i].tile0 = tiles; tiles += (p.seg[i].N + bn - 1) / bn; }
         p.nTiles = tiles;
         return tiles;
     };
+    // the large configuration: Q8 256 x 256 with 1024 threads; Q4_0 128 x 256 with 512 (it needs the
+    // scratch accumulator and more fragment registers than 1024 threads leave)
+    constexpr int BMB = Q4 ? 128 : 256, NTB = Q4 ? 512 : 1024;
     const int ksteps = (p.K + BK - 1) / BK;
     p.splitK = 1; p.stepsPerSplit = ksteps;
     if (p.T > 128) {
-        // 256 x 256 tiles; K is split until about one workgroup per CU exists (each split keeps >= 8 steps).
-        // Worth it when the tiles alone nearly fill the chip or K can be split; otherwise the small tiles
-        // below give more workgroups (short K, narrow N: latency-bound either way).
+        // K is split until about one workgroup per CU exists (each split keeps >= 8 steps).  Worth it
+        // when the tiles alone nearly fill the chip or K can be split; otherwise the small tiles below
+        // give more workgroups (short K, narrow N: latency-bound either way).
         const int tiles = count(256);
-        const int numM = (p.T + 255) / 256;
+        const int numM = (p.T + BMB - 1) / BMB;
         const int wgs = tiles * numM;
         int S = 1;
         if (p.partial && wgs < 160) {
@@ -499,13 +582,13 @@ hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s) {
                 S = (ksteps + p.stepsPerSplit - 1) / p.stepsPerSplit;
                 grid.y = (unsigned)S;
                 p.splitK = S; p.ldPartial = tiles * 256;
-                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<256, 256, 1024, 2>), grid, dim3(1024), 0, s, p);
+                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 2>), grid, dim3(NTB), 0, s, p);
                 hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((p.ldPartial + PWG - 1) / PWG), (unsigned)p.T), dim3(PWG),
                                    0, s, p, 256, residual);
             } else if (residual) {
-                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<256, 256, 1024, 1>), grid, dim3(1024), 0, s, p);
+                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 1>), grid, dim3(NTB), 0, s, p);
             } else {
-                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<256, 256, 1024, 0>), grid, dim3(1024), 0, s, p);
+                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 0>), grid, dim3(NTB), 0, s, p);
             }
             return hipGetLastError();
         }
@@ -513,9 +596,16 @@ hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s) {
     const int tiles = count(128);
     const int numM = (p.T + 63) / 64;
     dim3 grid((unsigned)(((tiles + 7) / 8) * 8 * numM));
-    if (residual) hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<64, 128, 256, 1>), grid, dim3(PWG), 0, s, p);
-    else hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<64, 128, 256, 0>), grid, dim3(PWG), 0, s, p);
+    if (residual) hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 1>), grid, dim3(PWG), 0, s, p);
+    else hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 0>), grid, dim3(PWG), 0, s, p);
     return hipGetLastError();
+}
+
+hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s) {
+    if (p.T <= 0 || p.nseg < 1 || p.nseg > 3) return p.T <= 0 ? hipSuccess : hipErrorInvalidValue;
+    if (p.K <= 0 || p.K % 32 != 0) return hipErrorInvalidValue;
+    for (int i = 0; i < p.nseg; i++) if (p.seg[i].N <= 0) return hipErrorInvalidValue;
+    return p.q4 ? launch_gemm_fmt<1>(p, residual, s) : launch_gemm_fmt<0>(p, residual, s);
 }
 
 }  // namespace mg

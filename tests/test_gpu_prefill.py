@@ -149,8 +149,17 @@ def test_prefill_errors(hip):
     assert m.hip.Prefill(np.array([s.vocab], np.int32), 0)[0] == -2   # token out of range
     assert m.hip.Prefill(np.zeros(4, np.int32), 0)[0] == 0
     m.close()
-    sq = H.with_layers(configs.QWEN_Q4, 1)
-    mq = H.Model(sq, seed=2, maxSeq=32, eng=hip, oracle=False)
-    assert mq.hip.Prefill(np.zeros(4, np.int32), 0)[0] == -5          # Q4_0 weights: unsupported
-    assert "Q8" in E.last_error()
-    mq.close()
+
+
+def test_prefill_qwen_q4_0_shape(hip):
+    """Qwen shape with GGUF Q4_0 weights and an fp16 embedding table, 2 layers, 150-token prompt (large-tile path)."""
+    s = H.with_layers(configs.QWEN_Q4, 2)
+    m, _, _ = _prefill_case(hip, s, seed=5, nPrompt=150, nDecode=6, maxSeq=192)
+    m.close()
+
+
+def test_prefill_q4_0_short_prompt_and_k_tail(hip):
+    """Toy shape in Q4_0 (ffn 1376: a K of 43 blocks, odd, so the last K step is half empty), 40-token prompt (small tiles)."""
+    s = configs.TOY._replace(fmt="q4_0", name="toy-q4")
+    m, _, _ = _prefill_case(hip, s, seed=6, nPrompt=40, nDecode=6, maxSeq=64)
+    m.close()
