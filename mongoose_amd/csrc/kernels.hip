@@ -93,7 +93,27 @@ __device__ __forceinline__ float stage_activation(const MvParams& p, float4* a4,
     const int tid = threadIdx.x;
     if (PRO == PRO_PLAIN) {
         const float4* x4 = reinterpret_cast<const float4*>(p.act);
-        for (int i = tid; i < K4; i += WG) a4[act_slot4<WF>(i, nch)] = x4[i];
+        if (K4 <= 4 * WG) {
+            for (int i = tid; i < K4; i += WG) a4[act_slot4<WF>(i, nch)] = x4[i];
+        } else {
+            // Long vectors (down projection, K = 14336): every load of a batch is issued before the
+            // first LDS store, so a batch costs one memory round trip; a load-store loop pays one per
+            // few iterations.
+            constexpr int B = 16;
+            for (int base = 0; base < K4; base += B * WG) {
+                float4 v[B];
+#pragma unroll
+                for (int u = 0; u < B; u++) {
+                    v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (base + u * WG < K4) v[u] = x4[min(base + u * WG + tid, K4 - 1)];   // uniform test
+                }
+#pragma unroll
+                for (int u = 0; u < B; u++) {
+                    const int i = base + u * WG + tid;
+                    if (i < K4) a4[act_slot4<WF>(i, nch)] = v[u];
+                }
+            }
+        }
         __syncthreads();
         return 1.0f;
     }
