@@ -555,8 +555,13 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
     }
     if (p.ngroups == 0) return hipSuccess;
     int wgs = c.ks == 1 ? (p.ngroups + 3) / 4 : p.ngroups;
-    int cap = epi == EPI_ARGMAX ? 1024 : 4096;      // one argmax partial per workgroup
-    if (c.grid <= 0 || c.grid > wgs) c.grid = wgs < cap ? wgs : cap;
+    int cap = epi == EPI_ARGMAX ? 1024 : 2048;      // one argmax partial per workgroup
+    if (c.grid <= 0 || c.grid > wgs) {
+        // every workgroup stages the activation vector: beyond the cap each takes several groups,
+        // the same number each (an uneven last round leaves most of the chip idle)
+        const int rounds = (wgs + cap - 1) / cap;
+        c.grid = epi == EPI_ARGMAX ? (wgs < cap ? wgs : cap) : (wgs + rounds - 1) / rounds;
+    }
     if (cfgInOut) *cfgInOut = c;
     if (wf == WF_Q8) return launch_wf<WF_Q8>(pro, epi, p, c, s);
     if (wf == WF_Q4P) return launch_wf<WF_Q4P>(pro, epi, p, c, s);
