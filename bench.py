@@ -62,7 +62,7 @@ def slots(s):
         yield idx
 
 
-def load_model(E, np, s, seed, maxSeq, eng, oracle=None, oracle_layers=None):
+def load_model(E, np, s, seed, maxSeq, eng, oracle=None, oracle_layers=None, kv_f16=False):
     """Build the GPU context through the library's own loader (SetWeight quantizes on the host);
     optionally mirror the same quantized bytes into the CPU oracle."""
     from mongoose_amd import configs
@@ -71,6 +71,8 @@ def load_model(E, np, s, seed, maxSeq, eng, oracle=None, oracle_layers=None):
                                maxSeq, s.theta, s.eps)
     if f is None:
         raise RuntimeError("NewHIPFusedInference failed: " + E.last_error())
+    if kv_f16 and f.SetKVFormat(1) != 0:
+        raise RuntimeError(E.last_error())
     if f.SetLayerRange(0, s.nLayers) != 0:
         raise RuntimeError(E.last_error())
     for idx in slots(s):
@@ -101,7 +103,7 @@ def load_model(E, np, s, seed, maxSeq, eng, oracle=None, oracle_layers=None):
     return f
 
 
-def cpu_baseline(E, np, s, seed, prompt, first_tokens, budget_s):
+def cpu_baseline(E, np, s, seed, prompt, first_tokens, budget_s, kv_f16=False):
     """The CPU oracle (restatement of the Go CPU engine's arithmetic, single
     thread like cpu.go) on the same model and the same positions, for a bounded
     number of tokens."""
@@ -112,6 +114,8 @@ def cpu_baseline(E, np, s, seed, prompt, first_tokens, budget_s):
     sample = 4
     orc = ob.Oracle(s.dim, kv, s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab, s.nLayers, nP + 64,
                     s.theta, s.eps, threads=1)
+    if kv_f16:
+        orc.set_kv_f16(True)
     for idx in slots(s):
         rows, cols = slot_shape(s, kv, idx)
         data = gen_slot(E, np, s, kv, seed, idx)
@@ -158,6 +162,8 @@ def main():
                     help="start the timed decode at this position (KV rows between the prompt and it are zeros): long-context timing")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run three 256 MiB device copies (a kernel of known traffic, to scale rocprofv3 --pmc counters)")
+    ap.add_argument("--kv", choices=["f32", "f16"], default="f32",
+                    help="KV cache row format (f32 is the reference's; f16 is this backend's option, not the headline configuration)")
     ap.add_argument("--prefill", type=int, default=0,
                     help="also time a batched prefill of this many prompt tokens (extra 'prefill' object)")
     args = ap.parse_args()
@@ -179,7 +185,8 @@ def main():
     P0 = max(args.context, W)                      # position of the first timed step
     maxSeq = max(P0 + K + args.profile_steps + 8, args.prefill)
     t_load = time.perf_counter()
-    f = load_model(E, np, s, args.seed, maxSeq, eng)
+    kv_f16 = args.kv == "f16"
+    f = load_model(E, np, s, args.seed, maxSeq, eng, kv_f16=kv_f16)
     t_load = time.perf_counter() - t_load
     prompt = E.synth_tokens(args.seed, 20_000_003, s.vocab, W)
     use_graph = not args.no_graph
@@ -215,7 +222,7 @@ def main():
     p_prof = P0 + K + args.profile_steps // 2
     cls_bytes = {
         1: mat(s.dim, s.dim) + 2 * mat(kv, s.dim) + 4 * s.dim,
-        2: 2 * (p_prof + 1) * kv * 4,
+        2: 2 * (p_prof + 1) * kv * (2 if kv_f16 else 4),
         3: mat(s.dim, s.dim),
         4: 2 * mat(s.ffnDim, s.dim) + 4 * s.dim,
         5: mat(s.dim, s.ffnDim),
@@ -236,7 +243,7 @@ def main():
 
     wbytes = configs.weight_bytes_per_token(s)
     assert f.WeightBytesPerToken() == wbytes
-    step_bytes = wbytes + configs.kv_bytes_at(s, p_mid)
+    step_bytes = wbytes + configs.kv_bytes_at(s, p_mid) // (2 if kv_f16 else 1)
     lm_bytes = cls_bytes[6]
     lm_s = lm_only_ms * 1e-3
     roofline = {"bound": "hbm", "kernel": "matvec lm_head (final norm + Q8 matvec + argmax partials)",
@@ -275,7 +282,7 @@ def main():
 
     cpu = None
     if args.cpu_budget > 0:
-        cpu = cpu_baseline(E, np, s, args.seed, prompt, toks, args.cpu_budget)
+        cpu = cpu_baseline(E, np, s, args.seed, prompt, toks, args.cpu_budget, kv_f16=kv_f16)
 
     out = {
         "metric": "Q8 decode tok/s (bs=1, Qwen2.5-0.5B shape) + matvec HBM GB/s % of peak" if s.name == "qwen2.5-0.5b"
@@ -285,7 +292,7 @@ def main():
         "dtype": "f32", "weight_dtype": "int8 per-row scale" if s.fmt == "q8" else "q4_0 (fp16 block scale)",
         "data": "synthetic",
         "config": {"workload": f"{s.name} random-init {s.fmt.upper()} greedy decode, {W}-token prompt, {K} decode tokens, "
-                               f"batch 1, fp32 KV cache", "layers": s.nLayers, "hidden": s.dim, "heads": s.nHeads,
+                               f"batch 1, {'fp16' if kv_f16 else 'fp32'} KV cache", "layers": s.nLayers, "hidden": s.dim, "heads": s.nHeads,
                    "kv_heads": s.nKVHeads, "ffn": s.ffnDim, "vocab": s.vocab, "graph_replay": use_graph},
         "step_bytes": int(step_bytes), "step_GBps": round(step_bytes * toks_per_s / 1e9, 1),
         "step_roofline_frac": round(step_bytes * toks_per_s / 1e9 / HBM_PEAK_GBS, 4),

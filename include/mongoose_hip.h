@@ -163,6 +163,14 @@ int mg_set_embedding_f32(mg_ctx* ctx, const float* table /* [vocab, dim] */);
  * ResetKV :530-537. */
 int mg_set_layer_range(mg_ctx* ctx, int layerStart, int layerEnd);
 int mg_reset_kv(mg_ctx* ctx);
+/* KV cache row format: 0 = fp32 (the reference's layout, cuda_fused_infer.go:546),
+ * 1 = fp16 rows (rounded to nearest even when a row is written; scores, softmax
+ * and P.V stay fp32).  The reference only declares hooks for compressed caches
+ * (kernels.go:71-72, no kernel source), so fp16 is this backend's own first step
+ * in that direction: half the attention bytes at long context.  Must be called
+ * before mg_set_layer_range (MG_E_STATE afterwards).  The per-op launches
+ * (mongoose_kv_cache_write, mongoose_decode_attention) keep fp32 caches. */
+int mg_set_kv_format(mg_ctx* ctx, int format);
 
 /* PartialStep :392-452 / PartialStepQ4 cuda_fused_infer_q4.go:92.  hiddenIn
  * [dim] host floats, or NULL for the ...Continue forms (:456, q4:272) that keep

@@ -76,7 +76,9 @@ public:
     int Prefill(const int* tokens, int nTokens, int pos0, int* nextToken, float* logitsOut, float* elapsedMs);
     int GeneratePrefill(const int* prompt, int nPrompt, int nDecode, int* outTokens);
     uint64_t WeightBytesPerToken() const;
-    uint64_t KVBytesAt(int pos) const { return (uint64_t)2 * nLayers * (uint64_t)(pos + 1) * kvDim * 4; }
+    uint64_t KVBytesAt(int pos) const { return (uint64_t)2 * nLayers * (uint64_t)(pos + 1) * kvDim * (kvHalf ? 2 : 4); }
+    int SetKVFormat(int fmt);                 // 0: fp32 rows (the reference's layout), 1: fp16 rows
+    int kvHalf = 0;
 
     int quantRounding = 0;
     int execMode = 1;

@@ -353,7 +353,7 @@ int HIPFusedInference::SetLayerRange(int layerStart, int layerEnd) {
     for (int l = layerStart; l < layerEnd && l < nLayers; l++) if (!kCache[l]) need++;
     if (need == 0) return MG_OK;
     invalidateGraphs();
-    const size_t per = alignUp256((size_t)maxSeq * kvDim * 4);
+    const size_t per = alignUp256((size_t)maxSeq * kvDim * (kvHalf ? 2 : 4));
     kvSlabs.emplace_back();
     Slab& sl = kvSlabs.back();
     int rc = sl.init(per * 2 * need);
@@ -367,14 +367,26 @@ int HIPFusedInference::SetLayerRange(int layerStart, int layerEnd) {
     return MG_OK;
 }
 
+// KV rows in fp16 halve the attention's bytes (the step toward the compressed caches the reference
+// only declares hooks for, kernels.go:71-72).  The choice fixes the allocation, so it comes first.
+int HIPFusedInference::SetKVFormat(int fmt) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(fmt == 0 || fmt == 1, "SetKVFormat: 0 (fp32) or 1 (fp16)");
+    if (fmt == kvHalf) return MG_OK;
+    if (!kvSlabs.empty()) { set_error("SetKVFormat: call before SetLayerRange (the caches are already allocated)"); return MG_E_STATE; }
+    invalidateGraphs();
+    kvHalf = fmt;
+    return MG_OK;
+}
+
 // cuda_fused_infer.go:530-537 uploads zeros over K only; V is cleared as well
 // here (a fresh sequence never reads V rows it has not written).
 int HIPFusedInference::ResetKV() {
     if (!built) return MG_E_NOT_BUILT;
     HIPCHK(hipStreamSynchronize(stream));
     for (int l = 0; l < nLayers; l++) {
-        if (kCache[l]) HIPCHK(hipMemset(kCache[l], 0, (size_t)maxSeq * kvDim * 4));
-        if (vCache[l]) HIPCHK(hipMemset(vCache[l], 0, (size_t)maxSeq * kvDim * 4));
+        if (kCache[l]) HIPCHK(hipMemset(kCache[l], 0, (size_t)maxSeq * kvDim * (kvHalf ? 2 : 4)));
+        if (vCache[l]) HIPCHK(hipMemset(vCache[l], 0, (size_t)maxSeq * kvDim * (kvHalf ? 2 : 4)));
     }
     return MG_OK;
 }
@@ -439,9 +451,15 @@ int HIPFusedInference::enqueueLayerPerOp(const LayerWeights& L, int layer, int p
     const float* sinRow = sinTab + (size_t)pos * half;
     HIPCHK(launch_rope(Q, cosRow, sinRow, 1, dim, headDim, nHeads, stream));
     HIPCHK(launch_rope(K, cosRow, sinRow, 1, kvDim, headDim, nKVHeads, stream));
-    HIPCHK(launch_kv_cache_write(kCache[layer], K, pos, kvDim, stream));
-    HIPCHK(launch_kv_cache_write(vCache[layer], V, pos, kvDim, stream));
+    if (kvHalf) {
+        HIPCHK(launch_kv_cache_write_f16(kCache[layer], K, pos, kvDim, stream));
+        HIPCHK(launch_kv_cache_write_f16(vCache[layer], V, pos, kvDim, stream));
+    } else {
+        HIPCHK(launch_kv_cache_write(kCache[layer], K, pos, kvDim, stream));
+        HIPCHK(launch_kv_cache_write(vCache[layer], V, pos, kvDim, stream));
+    }
     AttnParams a{};
+    a.kvHalf = kvHalf;
     a.q = Q; a.Kc = kCache[layer]; a.Vc = vCache[layer]; a.posImm = pos; a.rowLimit = maxSeq;
     a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
     a.out = attnOut; a.smax = 1; a.splitLen = 0;
@@ -469,7 +487,7 @@ int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const
         p.seg[1] = MvSeg{L.wk.w, L.wk.scales, L.bk, kCache[layer], kvDim};
         p.seg[2] = MvSeg{L.wv.w, L.wv.scales, L.bv, vCache[layer], kvDim};
         p.nseg = 3;
-        p.headDim = headDim; p.kvDim = kvDim;
+        p.headDim = headDim; p.kvDim = kvDim; p.kvHalf = kvHalf;
         p.state = st; p.posImm = posImm;
         const int half = headDim / 2;
         p.cosRow = st ? ropeCur : cosTab + (size_t)posImm * half;
@@ -479,6 +497,7 @@ int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const
     if (mark(2)) return MG_E_HIP;
     {
         AttnParams a{};
+        a.kvHalf = kvHalf;
         a.q = Q; a.Kc = kCache[layer]; a.Vc = vCache[layer];
         a.state = st; a.posImm = posImm; a.rowLimit = maxSeq;
         a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
@@ -899,8 +918,8 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
         g.K = dim; g.nseg = 3; g.q4 = L.wq.kind == WF_Q4P;
         g.seg[0] = seg(L.wq, L.bq, pfQ); g.seg[1] = seg(L.wk, L.bk, pfK); g.seg[2] = seg(L.wv, L.bv, pfV);
         HIPCHK(launch_gemm_q8(g, 0, stream));
-        HIPCHK(launch_rope_store_rows(pfQ, pfK, pfV, kCache[l], vCache[l], cosTab, sinTab, pos0, T, dim, kvDim, headDim, stream));
-        HIPCHK(launch_prefill_attention(pfQ, kCache[l], vCache[l], pfAttn, T, pos0, maxSeq, dim, kvDim, nHeads, nKVHeads, headDim, stream));
+        HIPCHK(launch_rope_store_rows(pfQ, pfK, pfV, kCache[l], vCache[l], kvHalf, cosTab, sinTab, pos0, T, dim, kvDim, headDim, stream));
+        HIPCHK(launch_prefill_attention(pfQ, kCache[l], vCache[l], kvHalf, pfAttn, T, pos0, maxSeq, dim, kvDim, nHeads, nKVHeads, headDim, stream));
         HIPCHK(launch_split_rows(pfAttn, nullptr, eps, T, dim, pfHi, pfLo, stream));
         g.K = dim; g.nseg = 1; g.q4 = L.wo.kind == WF_Q4P; g.seg[0] = seg(L.wo, nullptr, pfX);
         HIPCHK(launch_gemm_q8(g, 1, stream));
@@ -979,6 +998,7 @@ int mg_set_embedding_f16(mg_ctx* c, const uint16_t* t) { CTX(c); return f->SetEm
 int mg_set_embedding_f32(mg_ctx* c, const float* t) { CTX(c); return f->SetEmbeddingF32(t); }
 int mg_set_layer_range(mg_ctx* c, int a, int b) { CTX(c); return f->SetLayerRange(a, b); }
 int mg_reset_kv(mg_ctx* c) { CTX(c); return f->ResetKV(); }
+int mg_set_kv_format(mg_ctx* c, int fmt) { CTX(c); return f->SetKVFormat(fmt); }
 int mg_partial_step(mg_ctx* c, const float* hiddenIn, int pos, int l0, int l1, float* hiddenOut, float* logitsOut) {
     CTX(c); return f->PartialStep(hiddenIn, pos, l0, l1, hiddenOut, logitsOut);
 }

@@ -62,6 +62,7 @@ struct MvParams {
     const float* cosRow;
     const float* sinRow;
     int headDim, kvDim;
+    int kvHalf;           // EPI_QKV: the caches hold fp16 (seg1/seg2.out point at them all the same)
     // epilogue
     const float* resid;
     int div127;           // Q8: multiply by scales[r]/127 instead of scales[r]
@@ -91,6 +92,7 @@ struct AttnParams {
     int* counters;        // one per workgroup column, zero between launches (smax > 1)
     int headsPerWG;       // query heads of a GQA group per workgroup (0 = the whole group, in chunks of up to 4)
     float* out;           // [dim]
+    int kvHalf;           // Kc / Vc hold fp16 instead of fp32 (same [row, kvDim] indexing)
 };
 hipError_t launch_attention(const AttnParams& p, hipStream_t s);
 int attention_columns(int nHeads, int nKVHeads, int headsPerWG);
@@ -98,6 +100,7 @@ int attention_columns(int nHeads, int nKVHeads, int headsPerWG);
 hipError_t launch_rmsnorm_out(const float* in, float* out, const float* w, int seqLen, int dim, float eps, hipStream_t s);
 hipError_t launch_rope(float* x, const float* cosTab, const float* sinTab, int seqLen, int dim, int headDim, int nHeads, hipStream_t s);
 hipError_t launch_kv_cache_write(float* cache, const float* src, int pos, int kvDim, hipStream_t s);
+hipError_t launch_kv_cache_write_f16(void* cache, const float* src, int pos, int kvDim, hipStream_t s);
 hipError_t launch_silu_gate_mul(const float* gate, const float* up, float* out, int n, hipStream_t s);
 hipError_t launch_add_inplace(float* a, const float* b, int n, hipStream_t s);
 hipError_t launch_embed_gather_f32(float* out, const float* embed, const int* tokens, int seqLen, int dim, hipStream_t s);

@@ -421,14 +421,24 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
                             float v1 = __shfl(v, 1, 64);
                             if (lane == 0 && rr.valid) {
                                 const MvSeg& sg = p.seg[rr.seg];
-                                float* dst = rr.seg == 0 ? sg.out : sg.out + (size_t)pos * p.kvDim;
+                                float o0, o1;
+                                int i1;
                                 if (rr.seg < 2) {                               // mongoose.cu:991-1006
-                                    int half = p.headDim >> 1;
-                                    dst[rr.row] = v * cs - v1 * sn;
-                                    dst[rr.row + half] = v * sn + v1 * cs;
+                                    o0 = v * cs - v1 * sn;
+                                    o1 = v * sn + v1 * cs;
+                                    i1 = rr.row + (p.headDim >> 1);
                                 } else {                                        // mongoose.cu:1644-1647
-                                    dst[rr.row] = v;
-                                    if (rr.row + 1 < sg.rows) dst[rr.row + 1] = v1;
+                                    o0 = v; o1 = v1;
+                                    i1 = rr.row + 1 < sg.rows ? rr.row + 1 : rr.row;
+                                }
+                                if (rr.seg > 0 && p.kvHalf) {                   // fp16 cache rows
+                                    _Float16* dst = reinterpret_cast<_Float16*>(sg.out) + (size_t)pos * p.kvDim;
+                                    dst[i1] = (_Float16)o1;
+                                    dst[rr.row] = (_Float16)o0;
+                                } else {
+                                    float* dst = rr.seg == 0 ? sg.out : sg.out + (size_t)pos * p.kvDim;
+                                    dst[i1] = o1;
+                                    dst[rr.row] = o0;
                                 }
                             }
                         } else if (lane < NR && rr.valid) {
@@ -641,7 +651,16 @@ __device__ __forceinline__ float tg_sum(float v) {
     return v + __shfl_xor(v, 32, 64);
 }
 
-template <int HD, int GMAX>
+// One float4 of a cache row: fp32 rows are read as they are, fp16 rows as 8 bytes and widened.
+template <bool KVH>
+__device__ __forceinline__ float4 ld_kv4(const void* base, size_t idx4) {
+    if (!KVH) return static_cast<const float4*>(base)[idx4];
+    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+    const half4_t h = static_cast<const half4_t*>(base)[idx4];
+    return make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
+}
+
+template <int HD, int GMAX, bool KVH>
 __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     constexpr int LPR = 16;            // lanes per K/V row: one DPP row
     constexpr int NF = HD / 64;        // float4s of a row per lane (float4 index j*16 + dl)
@@ -667,8 +686,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     const int t0 = p.splitLen > 0 ? split * p.splitLen : 0;
     const int lastRow = p.rowLimit - 1;
     const size_t rowStride = (size_t)p.kvDim / 4;
-    const float4* Kbase = reinterpret_cast<const float4*>(p.Kc + kvOff) + dl;
-    const float4* Vbase = reinterpret_cast<const float4*>(p.Vc + kvOff) + dl;
+    const size_t colOff = (size_t)kvOff / 4 + dl;      // float4 index of this lane's first piece inside a row
 
     // ---- everything that does not need the position goes out first ----
     float4 q4[GMAX][NF];
@@ -683,11 +701,11 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
     for (int u = 0; u < VU; u++)
 #pragma unroll
-        for (int j = 0; j < NF; j++) kreg[u][j] = Kbase[(size_t)min(t0 + tg + u * TG, lastRow) * rowStride + j * 16];
+        for (int j = 0; j < NF; j++) kreg[u][j] = ld_kv4<KVH>(p.Kc, (size_t)min(t0 + tg + u * TG, lastRow) * rowStride + colOff + j * 16);
 #pragma unroll
     for (int u = 0; u < VU; u++)
 #pragma unroll
-        for (int j = 0; j < NF; j++) vreg[u][j] = Vbase[(size_t)min(t0 + tg + u * TG, lastRow) * rowStride + j * 16];
+        for (int j = 0; j < NF; j++) vreg[u][j] = ld_kv4<KVH>(p.Vc, (size_t)min(t0 + tg + u * TG, lastRow) * rowStride + colOff + j * 16);
 
     const int pos = p.state ? p.state->pos : p.posImm;
     const int len = pos + 1;
@@ -711,11 +729,11 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
             for (int u = 0; u < VU; u++)
 #pragma unroll
-                for (int j = 0; j < NF; j++) kreg[u][j] = Kbase[(size_t)min(tile + tg + u * TG, lastRow) * rowStride + j * 16];
+                for (int j = 0; j < NF; j++) kreg[u][j] = ld_kv4<KVH>(p.Kc, (size_t)min(tile + tg + u * TG, lastRow) * rowStride + colOff + j * 16);
 #pragma unroll
             for (int u = 0; u < VU; u++)
 #pragma unroll
-                for (int j = 0; j < NF; j++) vreg[u][j] = Vbase[(size_t)min(tile + tg + u * TG, lastRow) * rowStride + j * 16];
+                for (int j = 0; j < NF; j++) vreg[u][j] = ld_kv4<KVH>(p.Vc, (size_t)min(tile + tg + u * TG, lastRow) * rowStride + colOff + j * 16);
         }
         float sc[GMAX][VU];
 #pragma unroll
@@ -827,18 +845,34 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
         const float* pm = p.pm + (size_t)h * p.smax;
         const float* pl = p.pl + (size_t)h * p.smax;
         const float4* pa = reinterpret_cast<const float4*>(p.pacc + (size_t)h * p.smax * HD) + d4;
-        float M = -INFINITY;
-#pragma unroll 8
-        for (int s = 0; s < nsplit; s++) M = fmaxf(M, pm[s]);
-        float den = 0.f;
+        // Splits are merged 16 at a time: all 48 loads of a batch are issued before the first is
+        // used (one memory round trip a batch), then folded in with the running-maximum rescale.
+        float M = -INFINITY, den = 0.f;
         float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll 8
-        for (int s = 0; s < nsplit; s++) {
-            float w = expf(pm[s] - M);
-            float4 a = pa[(size_t)s * F4];
-            den = fmaf(w, pl[s], den);
-            num.x = fmaf(w, a.x, num.x); num.y = fmaf(w, a.y, num.y);
-            num.z = fmaf(w, a.z, num.z); num.w = fmaf(w, a.w, num.w);
+        for (int s0 = 0; s0 < nsplit; s0 += 16) {
+            float pmv[16], plv[16];
+            float4 pav[16];
+#pragma unroll
+            for (int u = 0; u < 16; u++) {
+                const int sidx = min(s0 + u, nsplit - 1);           // clamped, unconditional: stays in registers
+                pmv[u] = pm[sidx]; plv[u] = pl[sidx]; pav[u] = pa[(size_t)sidx * F4];
+            }
+            float bm = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < 16; u++) if (s0 + u < nsplit) bm = fmaxf(bm, pmv[u]);
+            const float Mn = fmaxf(M, bm);
+            const float c = expf(M - Mn);                           // first batch: exp(-inf) = 0
+            den *= c; num.x *= c; num.y *= c; num.z *= c; num.w *= c;
+            M = Mn;
+#pragma unroll
+            for (int u = 0; u < 16; u++) {
+                if (s0 + u < nsplit) {
+                    const float w = expf(pmv[u] - M);
+                    den = fmaf(w, plv[u], den);
+                    num.x = fmaf(w, pav[u].x, num.x); num.y = fmaf(w, pav[u].y, num.y);
+                    num.z = fmaf(w, pav[u].z, num.z); num.w = fmaf(w, pav[u].w, num.w);
+                }
+            }
         }
         float4 o;
         o.x = num.x / den; o.y = num.y / den; o.z = num.z / den; o.w = num.w / den;
@@ -856,16 +890,16 @@ static int attention_gmax(int G, int heads) {
     return want >= 3 ? 4 : (want == 2 ? 2 : 1);      // scores of GMAX heads x 16 rows live in registers: at most 4
 }
 
-template <int HD>
+template <int HD, bool KVH>
 static hipError_t launch_attn_hd(const AttnParams& p, hipStream_t s) {
     int G = p.nHeads / p.nKVHeads;
     int gmax = attention_gmax(G, p.headsPerWG);
     int nChunks = (G + gmax - 1) / gmax;
     dim3 grid(p.nKVHeads * nChunks, p.smax);
     switch (gmax) {
-    case 1: hipLaunchKernelGGL((attn_decode_kernel<HD, 1>), grid, dim3(WG), 0, s, p); break;
-    case 2: hipLaunchKernelGGL((attn_decode_kernel<HD, 2>), grid, dim3(WG), 0, s, p); break;
-    default: hipLaunchKernelGGL((attn_decode_kernel<HD, 4>), grid, dim3(WG), 0, s, p); break;
+    case 1: hipLaunchKernelGGL((attn_decode_kernel<HD, 1, KVH>), grid, dim3(WG), 0, s, p); break;
+    case 2: hipLaunchKernelGGL((attn_decode_kernel<HD, 2, KVH>), grid, dim3(WG), 0, s, p); break;
+    default: hipLaunchKernelGGL((attn_decode_kernel<HD, 4, KVH>), grid, dim3(WG), 0, s, p); break;
     }
     return hipGetLastError();
 }
@@ -881,8 +915,8 @@ hipError_t launch_attention(const AttnParams& p, hipStream_t s) {
     if (p.nKVHeads <= 0 || p.nHeads % p.nKVHeads != 0 || p.rowLimit <= 0 || p.smax < 1) return hipErrorInvalidValue;
     const int tile = p.headDim == 128 ? WG / 2 : WG;
     if (p.smax > 1 && (p.splitLen <= 0 || p.splitLen % tile != 0 || !p.counters || !p.pm || !p.pl || !p.pacc)) return hipErrorInvalidValue;
-    if (p.headDim == 64) return launch_attn_hd<64>(p, s);
-    if (p.headDim == 128) return launch_attn_hd<128>(p, s);
+    if (p.headDim == 64) return p.kvHalf ? launch_attn_hd<64, true>(p, s) : launch_attn_hd<64, false>(p, s);
+    if (p.headDim == 128) return p.kvHalf ? launch_attn_hd<128, true>(p, s) : launch_attn_hd<128, false>(p, s);
     return hipErrorInvalidValue;
 }
 
@@ -932,6 +966,14 @@ __global__ void kv_cache_write_kernel(float* cache, const float* src, int pos, i
 }
 hipError_t launch_kv_cache_write(float* cache, const float* src, int pos, int kvDim, hipStream_t s) {
     hipLaunchKernelGGL(kv_cache_write_kernel, dim3((kvDim + WG - 1) / WG), dim3(WG), 0, s, cache, src, pos, kvDim);
+    return hipGetLastError();
+}
+__global__ void kv_cache_write_f16_kernel(_Float16* cache, const float* src, int pos, int kvDim) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < kvDim) cache[(size_t)pos * kvDim + i] = (_Float16)src[i];
+}
+hipError_t launch_kv_cache_write_f16(void* cache, const float* src, int pos, int kvDim, hipStream_t s) {
+    hipLaunchKernelGGL(kv_cache_write_f16_kernel, dim3((kvDim + WG - 1) / WG), dim3(WG), 0, s, static_cast<_Float16*>(cache), src, pos, kvDim);
     return hipGetLastError();
 }
 

@@ -94,7 +94,8 @@ hipError_t launch_swiglu_split(const float* gate, const float* up, int T, int K,
 
 // RoPE (mongoose.cu:991-1006) on the q and k rows of T positions and the K/V
 // rows stored into the caches (mongoose.cu:1644-1647).  One workgroup per row.
-__global__ void rope_store_rows_kernel(float* q, const float* k, const float* v, float* Kc, float* Vc,
+template <typename KVT>
+__global__ void rope_store_rows_kernel(float* q, const float* k, const float* v, KVT* Kc, KVT* Vc,
                                        const float* cosTab, const float* sinTab, int pos0, int dim, int kvDim, int headDim) {
     const int t = blockIdx.x, pos = pos0 + t, half = headDim / 2;
     const float* c = cosTab + (size_t)pos * half;
@@ -108,20 +109,25 @@ __global__ void rope_store_rows_kernel(float* q, const float* k, const float* v,
     }
     const float* kr = k + (size_t)t * kvDim;
     const float* vr = v + (size_t)t * kvDim;
-    float* kd = Kc + (size_t)pos * kvDim;
-    float* vd = Vc + (size_t)pos * kvDim;
+    KVT* kd = Kc + (size_t)pos * kvDim;
+    KVT* vd = Vc + (size_t)pos * kvDim;
     for (int i = threadIdx.x; i < kvDim / 2; i += blockDim.x) {
         int h = i / half, j = i % half;
         float x0 = kr[h * headDim + j], x1 = kr[h * headDim + half + j];
-        kd[h * headDim + j] = x0 * c[j] - x1 * s[j];
-        kd[h * headDim + half + j] = x0 * s[j] + x1 * c[j];
+        kd[h * headDim + j] = (KVT)(x0 * c[j] - x1 * s[j]);
+        kd[h * headDim + half + j] = (KVT)(x0 * s[j] + x1 * c[j]);
     }
-    for (int i = threadIdx.x; i < kvDim; i += blockDim.x) vd[i] = vr[i];
+    for (int i = threadIdx.x; i < kvDim; i += blockDim.x) vd[i] = (KVT)vr[i];
 }
-hipError_t launch_rope_store_rows(float* q, const float* k, const float* v, float* Kc, float* Vc, const float* cosTab,
+hipError_t launch_rope_store_rows(float* q, const float* k, const float* v, void* Kc, void* Vc, int kvHalf, const float* cosTab,
                                   const float* sinTab, int pos0, int T, int dim, int kvDim, int headDim, hipStream_t s) {
     if (T <= 0) return hipSuccess;
-    hipLaunchKernelGGL(rope_store_rows_kernel, dim3(T), dim3(PWG), 0, s, q, k, v, Kc, Vc, cosTab, sinTab, pos0, dim, kvDim, headDim);
+    if (kvHalf)
+        hipLaunchKernelGGL(rope_store_rows_kernel<_Float16>, dim3(T), dim3(PWG), 0, s, q, k, v, static_cast<_Float16*>(Kc),
+                           static_cast<_Float16*>(Vc), cosTab, sinTab, pos0, dim, kvDim, headDim);
+    else
+        hipLaunchKernelGGL(rope_store_rows_kernel<float>, dim3(T), dim3(PWG), 0, s, q, k, v, static_cast<float*>(Kc),
+                           static_cast<float*>(Vc), cosTab, sinTab, pos0, dim, kvDim, headDim);
     return hipGetLastError();
 }
 
@@ -167,8 +173,8 @@ hipError_t launch_embed_rows(int kind, const void* table, const float* scales, c
 // operand step s wants row k = l/32 of its pair, so step s pairs exactly the
 // rows register s holds in the two lane halves.)
 // ---------------------------------------------------------------------------
-template <int HD>
-__global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const float* Kc, const float* Vc, float* out, int T,
+template <int HD, typename KVT>
+__global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const KVT* Kc, const KVT* Vc, float* out, int T,
                                                           int pos0, int dim, int kvDim, int nHeads, int nKVHeads) {
     constexpr int KS = HD + 4;                 // LDS row stride of the K tile (floats)
     constexpr int DB = HD / 32;                // 32-wide blocks of the head dimension
@@ -205,8 +211,9 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const
 #pragma unroll
         for (int i = 0; i < 32 * HD / 4 / 64; i++) {
             const int idx = i * 64 + lane, r = idx / (HD / 4), c4 = idx % (HD / 4);
-            const float4 v = *reinterpret_cast<const float4*>(Kc + (size_t)min(t0 + r, lastPos) * kvDim + (size_t)kvh * HD + c4 * 4);
-            *reinterpret_cast<float4*>(&kt[r * KS + c4 * 4]) = v;
+            typedef KVT kv4_t __attribute__((ext_vector_type(4)));
+            const kv4_t kv = *reinterpret_cast<const kv4_t*>(Kc + (size_t)min(t0 + r, lastPos) * kvDim + (size_t)kvh * HD + c4 * 4);
+            *reinterpret_cast<float4*>(&kt[r * KS + c4 * 4]) = make_float4((float)kv[0], (float)kv[1], (float)kv[2], (float)kv[3]);
         }
         __builtin_amdgcn_s_waitcnt(0);                   // wave-private buffer: the wave's own stores have landed
         __builtin_amdgcn_wave_barrier();
@@ -245,10 +252,10 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const
 #pragma unroll
         for (int s = 0; s < 16; s++) {
             const int kpos = min(t0 + 8 * (s >> 2) + 4 * half + (s & 3), lastPos);
-            const float* vr = Vc + (size_t)kpos * kvDim + (size_t)kvh * HD + col;
+            const KVT* vr = Vc + (size_t)kpos * kvDim + (size_t)kvh * HD + col;
 #pragma unroll
             for (int b = 0; b < DB; b++)
-                o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[32 * b], sT[s], o[b], 0, 0, 0);
+                o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32((float)vr[32 * b], sT[s], o[b], 0, 0, 0);
         }
         __builtin_amdgcn_wave_barrier();                 // the K tile is overwritten next
     }
@@ -276,15 +283,21 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const
     }
 }
 
-hipError_t launch_prefill_attention(const float* q, const float* Kc, const float* Vc, float* out, int T, int pos0, int rowLimit,
-                                    int dim, int kvDim, int nHeads, int nKVHeads, int headDim, hipStream_t s) {
+hipError_t launch_prefill_attention(const float* q, const void* Kc, const void* Vc, int kvHalf, float* out, int T, int pos0,
+                                    int rowLimit, int dim, int kvDim, int nHeads, int nKVHeads, int headDim, hipStream_t s) {
     if (T <= 0) return hipSuccess;
     if (nKVHeads <= 0 || nHeads % nKVHeads != 0 || pos0 < 0 || pos0 + T > rowLimit || dim != nHeads * headDim ||
-        kvDim != nKVHeads * headDim) return hipErrorInvalidValue;
+        kvDim != nKVHeads * headDim || (headDim != 64 && headDim != 128)) return hipErrorInvalidValue;
     dim3 grid((unsigned)((T + 31) / 32), (unsigned)nHeads);
-    if (headDim == 64) hipLaunchKernelGGL(prefill_attn_kernel<64>, grid, dim3(256), 0, s, q, Kc, Vc, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
-    else if (headDim == 128) hipLaunchKernelGGL(prefill_attn_kernel<128>, grid, dim3(256), 0, s, q, Kc, Vc, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
-    else return hipErrorInvalidValue;
+    const float* kf = static_cast<const float*>(Kc); const float* vf = static_cast<const float*>(Vc);
+    const _Float16* kh = static_cast<const _Float16*>(Kc); const _Float16* vh = static_cast<const _Float16*>(Vc);
+    if (headDim == 64) {
+        if (kvHalf) hipLaunchKernelGGL((prefill_attn_kernel<64, _Float16>), grid, dim3(256), 0, s, q, kh, vh, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
+        else hipLaunchKernelGGL((prefill_attn_kernel<64, float>), grid, dim3(256), 0, s, q, kf, vf, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
+    } else {
+        if (kvHalf) hipLaunchKernelGGL((prefill_attn_kernel<128, _Float16>), grid, dim3(256), 0, s, q, kh, vh, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
+        else hipLaunchKernelGGL((prefill_attn_kernel<128, float>), grid, dim3(256), 0, s, q, kf, vf, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
+    }
     return hipGetLastError();
 }
 

@@ -298,6 +298,10 @@ class HIPFusedInference:
     def SetLayerRange(self, layerStart, layerEnd):
         return lib.mg_set_layer_range(self._h, layerStart, layerEnd)
 
+    def SetKVFormat(self, fmt):
+        """0 = fp32 KV rows, 1 = fp16; before SetLayerRange."""
+        return lib.mg_set_kv_format(self._h, fmt)
+
     def ResetKV(self):
         return lib.mg_reset_kv(self._h)
 

@@ -77,6 +77,7 @@ _sig("mg_set_embedding_f16", c_int, c_void_p, POINTER(c_uint16))
 _sig("mg_set_embedding_f32", c_int, c_void_p, _f)
 _sig("mg_set_layer_range", c_int, c_void_p, c_int, c_int)
 _sig("mg_reset_kv", c_int, c_void_p)
+_sig("mg_set_kv_format", c_int, c_void_p, c_int)
 _sig("mg_partial_step", c_int, c_void_p, _f, c_int, c_int, c_int, _f, _f)
 _sig("mg_step_layer_resident", c_int, c_void_p, c_int, c_int, _f, _f, _f, _f)
 _sig("mg_export_hidden", c_int, c_void_p, _f)

@@ -55,6 +55,7 @@ _sig("orc_set_q4_0", c_int, c_void_p, c_int, POINTER(c_uint8))
 _sig("orc_set_embed_f16", None, c_void_p, POINTER(c_uint16))
 _sig("orc_set_embed_f32", None, c_void_p, _f)
 _sig("orc_reset_kv", None, c_void_p)
+_sig("orc_set_kv_f16", None, c_void_p, c_int)
 _sig("orc_embed", c_int, c_void_p, c_int, _f)
 _sig("orc_argmax", c_int, _f, c_int)
 for pfx, real in (("orc32", _f), ("orc64", _d)):
@@ -222,6 +223,9 @@ class Oracle:
 
     def reset_kv(self):
         lib.orc_reset_kv(self.h)
+
+    def set_kv_f16(self, on):
+        lib.orc_set_kv_f16(self.h, 1 if on else 0)
 
     def embed(self, tok):
         out = np.empty(self.dim, np.float32)

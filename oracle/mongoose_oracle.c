@@ -33,6 +33,8 @@
  *                        identity, norm preservation, relative-position property,
  *                        seqLen 1 -> out == V, uniform keys -> mean of V) and by an
  *                        independent numpy restatement.
+ *   orc_set_kv_f16       option without a reference counterpart: K/V rows pass through the
+ *                        pinned fp16 conversions when written (models an fp16 KV cache)
  *   embedding gather, argmax   no reference function (the reference's caller does
  *                        both on the host); textbook semantics, lowest index on ties.
  *
@@ -283,6 +285,7 @@ typedef struct {
     float *cosT, *sinT;       /* [maxSeq, headDim/2] */
     float *kc32, *vc32;       /* [nLayers, maxSeq, kvDim] float caches */
     double *kc64, *vc64;      /* double shadow caches */
+    int kv_f16;               /* K/V rows rounded to fp16 (RNE) when written: models an fp16 KV cache */
     int threads;
 } orc_ctx;
 
@@ -393,6 +396,11 @@ ORC_API void orc_set_embed_f32(orc_ctx* c, const float* table) {
 /* cuda_fused_infer.go:530-537 zeroes K only; both are zeroed here because a
  * fresh sequence never reads rows beyond pos and V rows are always written
  * before they are read, so the two are indistinguishable in outputs. */
+/* fp16 KV rows (no reference counterpart: the reference's caches are fp32 and it only declares hooks
+ * for compressed ones, kernels.go:71-72).  The rounding is the pinned orc_f32_to_f16; everything
+ * around it is the unchanged step, so the option is pinned by those two. */
+ORC_API void orc_set_kv_f16(orc_ctx* c, int on) { c->kv_f16 = on ? 1 : 0; }
+
 ORC_API void orc_reset_kv(orc_ctx* c) {
     size_t kvn = (size_t)c->nLayers * c->maxSeq * c->kvDim;
     memset(c->kc32, 0, kvn * sizeof(float));

@@ -49,17 +49,21 @@ def with_layers(s, n):
 class Model:
     """Oracle and/or HIP context holding the same synthetic model."""
 
-    def __init__(self, s, seed, maxSeq, eng=None, oracle=True, threads=8, fmt=None, keep_dequant=False):
+    def __init__(self, s, seed, maxSeq, eng=None, oracle=True, threads=8, fmt=None, keep_dequant=False, kv_f16=False):
         self.s, self.seed, self.maxSeq = s, seed, maxSeq
         fmt = fmt or s.fmt
         kv = configs.kv_dim(s)
         self.orc = ob.Oracle(s.dim, kv, s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab, s.nLayers, maxSeq,
                              s.theta, s.eps, threads=threads) if oracle else None
+        if kv_f16 and self.orc:
+            self.orc.set_kv_f16(True)
         self.hip = None
         if eng is not None:
             self.hip = E.NewHIPFusedInference(eng, s.dim, kv, s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab,
                                               s.nLayers, maxSeq, s.theta, s.eps)
             assert self.hip is not None, E.last_error()
+            if kv_f16:
+                assert self.hip.SetKVFormat(1) == 0, E.last_error()
             assert self.hip.SetLayerRange(0, s.nLayers) == 0, E.last_error()
         self.dequant = {} if keep_dequant else None
         self.vecs = {}

@@ -68,7 +68,8 @@ def rope_tables(maxSeq, headDim, theta):
 class NpModel:
     """Decode step in float64 over dequantized float32 weights."""
 
-    def __init__(self, shape_args, weights, vecs, maxSeq):
+    def __init__(self, shape_args, weights, vecs, maxSeq, kv_f16=False):
+        self.kv_f16 = kv_f16       # K/V rows stored as float16 (numpy's own rounding)
         (self.dim, self.kvDim, self.headDim, self.nHeads, self.nKVHeads, self.ffnDim, self.vocab,
          self.nLayers, self.theta, self.eps) = shape_args
         self.W = {k: np.asarray(v, np.float64) for k, v in weights.items()}     # idx -> dequantized [N,K]
@@ -105,6 +106,9 @@ class NpModel:
                 v = v + self.V[b + 6]
             q = self.rope(q, pos, self.nHeads)
             k = self.rope(k, pos, self.nKVHeads)
+            if self.kv_f16:
+                k = k.astype(np.float32).astype(np.float16).astype(np.float64)
+                v = v.astype(np.float32).astype(np.float16).astype(np.float64)
             self.Kc[l, pos] = k
             self.Vc[l, pos] = v
             out = np.zeros(self.dim)

@@ -77,8 +77,8 @@ def _oracle_prompt_logits(m, prompt, shadow):
     return logits.copy()
 
 
-def _prefill_case(hip, s, seed, nPrompt, nDecode, maxSeq):
-    m = H.Model(s, seed=seed, maxSeq=maxSeq, eng=hip, threads=8)
+def _prefill_case(hip, s, seed, nPrompt, nDecode, maxSeq, kv_f16=False):
+    m = H.Model(s, seed=seed, maxSeq=maxSeq, eng=hip, threads=8, kv_f16=kv_f16)
     prompt = m.prompt(nPrompt)
     lg32 = _oracle_prompt_logits(m, prompt, False)
     lg64 = _oracle_prompt_logits(m, prompt, True)
@@ -138,6 +138,15 @@ def test_prefill_llama3_shape_one_layer(hip):
     """Llama-3-8B shape (head 128, GQA 32/8), 1 layer, 160-token prompt."""
     s = H.with_layers(configs.LLAMA3_8B, 1)
     m, _, _ = _prefill_case(hip, s, seed=4, nPrompt=160, nDecode=4, maxSeq=192)
+    m.close()
+
+
+def test_prefill_fp16_kv(hip):
+    """Prefill writing fp16 KV rows (head sizes 64 and 128) against the oracle with the same rounding."""
+    m, _, _ = _prefill_case(hip, H.with_layers(configs.QWEN, 2), seed=7, nPrompt=70, nDecode=6, maxSeq=96, kv_f16=True)
+    m.close()
+    s = configs.Shape("l3-mini", 2, 512, 4, 1, 128, 1024, 512, 1e-5, 5e5, False, True, "q8")
+    m, _, _ = _prefill_case(hip, s, seed=8, nPrompt=45, nDecode=6, maxSeq=64, kv_f16=True)
     m.close()
 
 

@@ -10,10 +10,10 @@ from tests import helpers as H
 from tests import np_reference as npr
 
 
-def _np_model(m, maxSeq):
+def _np_model(m, maxSeq, kv_f16=False):
     s = m.s
     args = (s.dim, configs.kv_dim(s), s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab, s.nLayers, s.theta, s.eps)
-    return npr.NpModel(args, m.dequant, m.vecs, maxSeq)
+    return npr.NpModel(args, m.dequant, m.vecs, maxSeq, kv_f16=kv_f16)
 
 
 MINI = configs.Shape("mini", 2, 128, 4, 2, 32, 160, 96, 1e-5, 1e4, True, True, "q8")
@@ -40,6 +40,27 @@ def test_step_matches_numpy_restatement(shape):
         assert H.rel_err(logits64, logits) < 1e-6, pos
         assert H.rel_err(hout64, x) < 1e-6
     m.close()
+
+
+def test_fp16_kv_option_matches_numpy_float16_rows():
+    """K/V rows rounded to fp16 when written: the oracle's conversion against numpy.float16 inside the
+    independent model; and the option changes the result (it is not a no-op)."""
+    maxSeq = 10
+    m = H.Model(MINI, seed=13, maxSeq=maxSeq, eng=None, oracle=True, threads=1, keep_dequant=True, kv_f16=True)
+    plain = H.Model(MINI, seed=13, maxSeq=maxSeq, eng=None, oracle=True, threads=1)
+    ref = _np_model(m, maxSeq, kv_f16=True)
+    prompt = m.prompt(maxSeq)
+    differs = False
+    for pos in range(maxSeq):
+        h = m.orc.embed(prompt[pos])
+        hout64, logits64, _ = m.orc.step(h, pos, shadow=True)
+        x, logits, _ = ref.step(h, pos)
+        assert H.rel_err(logits64, logits) < 1e-6 and H.rel_err(hout64, x) < 1e-6, pos
+        _, logits_plain, _ = plain.orc.step(h, pos, shadow=True)
+        differs = differs or H.rel_err(logits64, logits_plain) > 1e-6
+    assert differs
+    m.close()
+    plain.close()
 
 
 def test_float_step_tracks_double_shadow():
