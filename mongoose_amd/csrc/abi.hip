@@ -52,7 +52,10 @@ int tw_hip_device_info(char* name, size_t nameLen, uint64_t* totalMem) {
     int dev = 0;
     hipDeviceProp_t prop;
     if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) { (void)hipGetLastError(); return -1; }
-    if (name && nameLen) { std::strncpy(name, prop.name, nameLen - 1); name[nameLen - 1] = 0; }
+    if (name && nameLen) {          // some driver stacks leave the marketing name empty: fall back to the ISA name
+        std::strncpy(name, prop.name[0] ? prop.name : prop.gcnArchName, nameLen - 1);
+        name[nameLen - 1] = 0;
+    }
     if (totalMem) *totalMem = (uint64_t)prop.totalGlobalMem;
     return 0;
 }
