@@ -608,9 +608,30 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
     }
     const int tiles = count(128);
     const int numM = (p.T + 63) / 64;
-    dim3 grid((unsigned)(((tiles + 7) / 8) * 8 * numM));
-    if (residual) hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 1>), grid, dim3(PWG), 0, s, p);
-    else hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 0>), grid, dim3(PWG), 0, s, p);
+    dim3 grid((unsigned)(((tiles + 7) / 8) * 8 * numM), 1);
+    // These shapes are bound by the memory latency of each K step (one workgroup per CU or fewer, one
+    // step of lookahead), so K is split as well, down to 4 steps a piece, until a few workgroups share
+    // every CU and cover each other's waits.
+    const int wgs = tiles * numM;
+    int S = 1;
+    if (p.partial && wgs < 512 && ksteps >= 8) {
+        S = (768 + wgs - 1) / wgs;
+        if (S > ksteps / 4) S = ksteps / 4;
+        while (S > 1 && (size_t)S * p.T * tiles * 128 > gemm_partial_floats()) S--;
+    }
+    if (S > 1) {
+        p.stepsPerSplit = (ksteps + S - 1) / S;
+        S = (ksteps + p.stepsPerSplit - 1) / p.stepsPerSplit;
+        grid.y = (unsigned)S;
+        p.splitK = S; p.ldPartial = tiles * 128;
+        hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 2>), grid, dim3(PWG), 0, s, p);
+        hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((p.ldPartial + PWG - 1) / PWG), (unsigned)p.T), dim3(PWG), 0, s,
+                           p, 128, residual);
+    } else if (residual) {
+        hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 1>), grid, dim3(PWG), 0, s, p);
+    } else {
+        hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 0>), grid, dim3(PWG), 0, s, p);
+    }
     return hipGetLastError();
 }
 
