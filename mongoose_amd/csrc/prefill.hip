@@ -537,6 +537,166 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// The large Q8 tile (256 x 256, 1024 threads) fed by direct global -> LDS loads
+// (global_load_lds_dwordx4: no register staging, no LDS store instructions)
+// through a three-stage LDS ring with K steps of 32: a stage's loads are issued
+// two steps before it is multiplied, one barrier per step.  A wave's load
+// lands as 1 KB of consecutive 16-byte slots, so the layout is made on the
+// global side: slot s of wave w holds, for A, row 16w + s/4 and piece
+// (s%4) ^ ((row>>1)&3) of the row's 64 bytes; for W (waves 0-7), row 32w + s/2
+// and piece (s%2) ^ ((row>>2)&1) of its 32 bytes.  The XOR makes every
+// fragment read (8 lanes = 128 bytes) touch all LDS banks once.  A W piece is
+// 16 consecutive k of one lane half: its low 8 bytes feed the first MFMA step,
+// its high 8 bytes the second, and the A pieces are picked to match.
+// 917 TF issued against 717 for the register-staged tile on the gate/up shape.
+// ---------------------------------------------------------------------------
+constexpr int RK = 32, RS = 3;
+constexpr int RING_STAGE_BYTES = 256 * 64 * 2 + 256 * 32;      // A hi + A lo + W
+
+__device__ __forceinline__ bf16x8_t cvt8_i8_bf16(int lo, int hi) {
+    uint4 u;
+    u.x = pack_bf16_exact((float)(signed char)(lo), (float)(signed char)(lo >> 8));
+    u.y = pack_bf16_exact((float)(signed char)(lo >> 16), (float)(lo >> 24));
+    u.z = pack_bf16_exact((float)(signed char)(hi), (float)(signed char)(hi >> 8));
+    u.w = pack_bf16_exact((float)(signed char)(hi >> 16), (float)(hi >> 24));
+    return __builtin_bit_cast(bf16x8_t, u);
+}
+
+template <int MODE>
+__global__ __launch_bounds__(1024) void gemm_q8_ring_kernel(GemmParams p) {
+    constexpr int BM = 256, BN = 256;
+    extern __shared__ __attribute__((aligned(16))) unsigned char ring[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 2, wn = wave & 3;             // 4 x 4 waves, each 64 x 64
+    const int numM = (p.T + BM - 1) / BM;
+    const int L = blockIdx.x;
+    const int grp = L / (8 * numM), rem = L % (8 * numM);
+    const int nTile = grp * 8 + (rem & 7), mTile = rem >> 3;
+    if (nTile >= p.nTiles) return;
+    GemmSeg sg = p.seg[0];
+    if (p.nseg > 1 && nTile >= p.seg[1].tile0) sg = p.seg[1];
+    if (p.nseg > 2 && nTile >= p.seg[2].tile0) sg = p.seg[2];
+    const int N = sg.N, K = p.K, T = p.T;
+    const int m0 = mTile * BM, n0 = (nTile - sg.tile0) * BN;
+    const int ksteps = K / RK;                            // K is a multiple of 32
+    const int ks64 = (K + 63) / 64;                       // the split planes are blocked in 64-k steps
+    const int stepBeg = MODE == 2 ? blockIdx.y * p.stepsPerSplit * 2 : 0;
+    const int stepEnd = MODE == 2 ? min(ksteps, stepBeg + p.stepsPerSplit * 2) : ksteps;
+    const int planeRows = ((T + 127) >> 7) << 7;
+
+    const int aRowL = 16 * wave + (lane >> 2);
+    const int aSeg = (lane & 3) ^ ((aRowL >> 1) & 3);
+    const int aRowG = min(m0 + aRowL, planeRows - 1);
+    const size_t aOff = (size_t)(aRowG >> 7) * ks64 * 8192 + (size_t)(aRowG & 127) * 64 + aSeg * 8;
+    const unsigned short* aH = p.Ahi + aOff;
+    const unsigned short* aL = p.Alo + aOff;
+    const int bRowL = 32 * (wave & 7) + (lane >> 1);
+    const int bSeg = (lane & 1) ^ ((bRowL >> 2) & 1);
+    const signed char* bG = sg.W + (size_t)min(n0 + bRowL, N - 1) * K + bSeg * 16;
+    const bool bWave = wave < 8;
+
+    auto issue = [&](int step, int stage) __attribute__((always_inline)) {
+        const int st = min(step, ksteps - 1);            // past the end: a harmless reload that keeps the counters uniform
+        unsigned char* base = ring + stage * RING_STAGE_BYTES;
+        const size_t ko = (size_t)(st >> 1) * 8192 + (st & 1) * 32;
+        __builtin_amdgcn_global_load_lds(aH + ko, reinterpret_cast<int4*>(base + wave * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(aL + ko, reinterpret_cast<int4*>(base + BM * 64 + wave * 1024), 16, 0, 0);
+        if (bWave) __builtin_amdgcn_global_load_lds(bG + (size_t)st * RK, reinterpret_cast<int4*>(base + BM * 128 + wave * 1024), 16, 0, 0);
+    };
+
+    float16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+    issue(stepBeg, 0);
+    issue(stepBeg + 1, 1);
+    int stage = 0;
+    for (int step = stepBeg; step < stepEnd; step++) {
+        // this step's stage has landed; the next stage's loads may still be in flight
+        if (bWave) asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        __syncthreads();
+        int nst = stage + 2; if (nst >= RS) nst -= RS;
+        issue(step + 2, nst);                            // refills the stage every wave finished reading before this barrier
+        const unsigned char* base = ring + stage * RING_STAGE_BYTES;
+        const int half = lane >> 5;
+        bf16x8_t b[2][2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int row = wn * 64 + j * 32 + (lane & 31);
+            const int4 w = *reinterpret_cast<const int4*>(base + BM * 128 + (row * 2 + (half ^ ((row >> 2) & 1))) * 16);
+            b[j][0] = cvt8_i8_bf16(w.x, w.y);
+            b[j][1] = cvt8_i8_bf16(w.z, w.w);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int row = wm * 64 + i * 32 + (lane & 31);
+#pragma unroll
+            for (int ksub = 0; ksub < 2; ksub++) {
+                const int slot = row * 4 + ((2 * half + ksub) ^ ((row >> 1) & 3));
+                const bf16x8_t ah = *reinterpret_cast<const bf16x8_t*>(base + slot * 16);
+                const bf16x8_t al = *reinterpret_cast<const bf16x8_t*>(base + BM * 64 + slot * 16);
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, b[j][ksub], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, b[j][ksub], acc[i][j], 0, 0, 0);
+                }
+            }
+        }
+        stage = stage + 1 == RS ? 0 : stage + 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the trailing reloads must not outlive the workgroup's LDS
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int nl = wn * 64 + j * 32 + (lane & 31);
+        const int n = n0 + nl;
+        if (MODE == 2) {
+            float* dst = p.partial + ((size_t)blockIdx.y * T) * p.ldPartial + (size_t)nTile * BN + nl;
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                    if (m < T) dst[(size_t)m * p.ldPartial] = acc[i][j][e];
+                }
+            continue;
+        }
+        if (n >= N) continue;
+        const float sc = sg.scales[n];
+        const float bi = sg.bias ? sg.bias[n] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                if (m < T) {
+                    float v = acc[i][j][e] * sc + bi;
+                    float* dst = sg.Y + (size_t)m * N + n;
+                    if (MODE == 1) v = *dst + v;
+                    *dst = v;
+                }
+            }
+    }
+}
+
+template <int MODE>
+static hipError_t launch_ring(const GemmParams& p, dim3 grid, hipStream_t s) {
+    constexpr int bytes = RS * RING_STAGE_BYTES;          // 120 KB of the CU's 160 KB
+    static bool raised = false;                            // the default cap on dynamic LDS is 64 KB
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q8_ring_kernel<MODE>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    hipLaunchKernelGGL((gemm_q8_ring_kernel<MODE>), grid, dim3(1024), bytes, s, p);
+    return hipGetLastError();
+}
+
 // Sum of the K splits in split order (so the result does not depend on which workgroup
 // finished first), then scale, bias and the optional residual.
 __global__ __launch_bounds__(PWG) void gemm_reduce_kernel(GemmParams p, int BN, int residual) {
@@ -595,9 +755,16 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
                 S = (ksteps + p.stepsPerSplit - 1) / p.stepsPerSplit;
                 grid.y = (unsigned)S;
                 p.splitK = S; p.ldPartial = tiles * 256;
-                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 2>), grid, dim3(NTB), 0, s, p);
+                if (Q4) {
+                    hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 2>), grid, dim3(NTB), 0, s, p);
+                } else {
+                    hipError_t e = launch_ring<2>(p, grid, s);
+                    if (e != hipSuccess) return e;
+                }
                 hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((p.ldPartial + PWG - 1) / PWG), (unsigned)p.T), dim3(PWG),
                                    0, s, p, 256, residual);
+            } else if (!Q4) {
+                return residual ? launch_ring<1>(p, grid, s) : launch_ring<0>(p, grid, s);
             } else if (residual) {
                 hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 1>), grid, dim3(NTB), 0, s, p);
             } else {
