@@ -27,6 +27,8 @@ def _up(eng, a):
 @pytest.mark.parametrize("T,N,K,acc,bias", [
     (1, 128, 32, False, False), (5, 100, 64, False, True), (130, 300, 896, True, False),
     (128, 128, 4864, False, False), (257, 1376, 512, True, True), (512, 1024, 4096, False, False),
+    # enough 256 x 256 tiles for the direct-to-LDS ring kernel: accumulate form, bias form, odd count of 32-wide K steps
+    (512, 12288, 64, True, False), (300, 12800, 96, False, True),
 ])
 def test_q8_gemm_against_float64(hip, T, N, K, acc, bias):
     print(f"q8 gemm T={T} N={N} K={K} acc={acc} bias={bias}", flush=True)
