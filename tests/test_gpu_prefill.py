@@ -152,6 +152,32 @@ def test_prefill_fp16_kv(hip):
     m.close()
 
 
+def test_prefill_buffer_growth_and_sequence_end(hip):
+    """Row buffers grow with the prompt (small call first), and a prompt may run to the last position."""
+    s = H.with_layers(configs.TOY, 2)
+    maxSeq = 200
+    m = H.Model(s, seed=12, maxSeq=maxSeq, eng=hip, threads=8)
+    prompt = m.prompt(maxSeq)
+    rc, n_small, _, _ = m.hip.Prefill(prompt[:5], 0)                  # allocates for 128 rows
+    assert rc == 0, E.last_error()
+    assert m.hip.ResetKV() == 0
+    rc, nxt, logits, _ = m.hip.Prefill(prompt, 0, wantLogits=True)    # 200 rows: buffers are re-made; ends at maxSeq - 1
+    assert rc == 0, E.last_error()
+    lg64 = _oracle_prompt_logits(m, prompt, True)
+    assert H.rel_err(logits, lg64) < 1e-3 and nxt == int(np.argmax(lg64))
+    # the position after the last one does not exist
+    assert m.hip.Prefill(prompt[:1], maxSeq)[0] == -2
+    # prompt + decode may fill the sequence exactly: maxSeq - 3 prompt positions, 4 tokens (the last needs no cache row)
+    assert m.hip.ResetKV() == 0
+    rc, toks = m.hip.GeneratePrefill(prompt[:maxSeq - 3], 4)
+    assert rc == 0, E.last_error()
+    assert m.hip.ResetKV() == 0
+    rc, toks_dec = m.hip.Generate(prompt[:maxSeq - 3], 4, useGraph=True)
+    assert rc == 0 and toks.tolist() == toks_dec.tolist()
+    assert m.hip.GeneratePrefill(prompt[:maxSeq - 3], 5)[0] == -2
+    m.close()
+
+
 def test_prefill_errors(hip):
     s = H.with_layers(configs.TOY, 1)
     m = H.Model(s, seed=2, maxSeq=32, eng=hip, oracle=False)
