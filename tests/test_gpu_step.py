@@ -318,3 +318,38 @@ def test_fp16_kv_cache_long_context_head128(hip):
     assert rc == 0, E.last_error()
     assert toks.tolist() == toks_ref.tolist()
     m.close()
+
+
+def test_qwen_full_workload_paths_agree(hip):
+    """The benchmark's own workload at full size (Qwen2.5-0.5B shape, 24 layers, 16-token prompt, 200 greedy
+    tokens): graph replay, eager fused launches, the reference-order per-op launches and the prompt
+    through the batched prefill all give the same 200 tokens (a size-independent property: the paths
+    differ only in summation order), and the first tokens are the oracle's."""
+    s = configs.QWEN
+    m = H.Model(s, seed=20250, maxSeq=224, eng=hip, threads=8)
+    prompt = m.prompt(16)
+    rc, toks_graph = m.hip.Generate(prompt, 200, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert m.hip.ResetKV() == 0
+    rc, toks_eager = m.hip.Generate(prompt, 200, useGraph=False)
+    assert rc == 0, E.last_error()
+    assert m.hip.SetExecMode(0) == 0
+    assert m.hip.ResetKV() == 0
+    rc, toks_perop = m.hip.Generate(prompt, 200, useGraph=False)
+    assert rc == 0, E.last_error()
+    assert m.hip.SetExecMode(1) == 0
+    assert m.hip.ResetKV() == 0
+    rc, toks_prefill = m.hip.GeneratePrefill(prompt, 200)
+    assert rc == 0, E.last_error()
+    assert toks_graph.tolist() == toks_eager.tolist()
+    # different summation orders may part ways at a near-tie somewhere in 200 tokens; the common prefix must be long
+    def common(a, b):
+        n = 0
+        while n < len(a) and a[n] == b[n]:
+            n += 1
+        return n
+    assert common(toks_graph, toks_perop) >= 32, common(toks_graph, toks_perop)
+    assert common(toks_graph, toks_prefill) >= 32, common(toks_graph, toks_prefill)
+    toks_ref, _ = H.oracle_generate(m, prompt, 6)
+    assert toks_graph[:6].tolist() == toks_ref.tolist()
+    m.close()
