@@ -477,6 +477,96 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     }
 }
 
+// Tall matrix of short rows (lm_head of a small model: K <= 1024, so one wave pass covers a row):
+// a lane meets the same 16 activations in every row, so they are read from LDS once and stay in
+// registers, and the loop is nothing but "four row loads, four dots, four reductions".  No ring:
+// the loads of the eight waves a SIMD holds overlap each other.  Arithmetic and order are
+// matvec_kernel's, so the two give the same bits.
+template <int EPI>
+__global__ __launch_bounds__(WG) void matvec_rows_q8_kernel(MvParams p) {
+    constexpr int NR = 4;
+    extern __shared__ float4 a4[];
+    __shared__ float red[4];
+    __shared__ float bestV[4];
+    __shared__ int bestI[4];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nch = p.K / 16;
+    const int nrows = p.seg[0].rows;
+    const char* __restrict__ w = static_cast<const char*>(p.seg[0].w);
+    const float* __restrict__ scales = static_cast<const float*>(p.seg[0].aux);
+    float* __restrict__ out = p.seg[0].out;
+    const bool live = lane < nch;
+    const int gStep = gridDim.x * 4;
+
+    int g = blockIdx.x * 4 + wave;
+    int4 v[NR];
+    float scl = 0.f;
+    auto fetch = [&](int gg) {
+#pragma unroll
+        for (int i = 0; i < NR; i++) {
+            const int r = gg * NR + i;
+            v[i] = make_int4(0, 0, 0, 0);
+            if (r < nrows && live) v[i] = *reinterpret_cast<const int4*>(w + (size_t)r * p.K + lane * 16);
+        }
+        scl = 0.f;
+        if (lane < NR && gg * NR + lane < nrows) scl = scales[gg * NR + lane];
+    };
+    if (g * NR < nrows) fetch(g);                    // the first rows go out before the vector is staged
+
+    const float rs = stage_activation<WF_Q8, PRO_RMS>(p, a4, red);
+    float4 av[4];
+#pragma unroll
+    for (int pl = 0; pl < 4; pl++) av[pl] = live ? a4[pl * nch + lane] : make_float4(0.f, 0.f, 0.f, 0.f);
+
+    float myBestV = -INFINITY;
+    int myBestI = INT_MAX;
+    for (; g * NR < nrows; g += gStep) {
+        float acc[NR];
+#pragma unroll
+        for (int i = 0; i < NR; i++) {
+            float a = 0.f;
+            a = dot4_i8(v[i].x, av[0], a); a = dot4_i8(v[i].y, av[1], a);
+            a = dot4_i8(v[i].z, av[2], a); a = dot4_i8(v[i].w, av[3], a);
+            acc[i] = a;
+        }
+        const float sc = scl;
+        const int gNext = g + gStep;
+        if (gNext * NR < nrows) fetch(gNext);
+#pragma unroll
+        for (int i = 0; i < NR; i++) acc[i] = wave_sum(acc[i]);
+        float val = acc[0];
+#pragma unroll
+        for (int i = 1; i < NR; i++) if (lane == i) val = acc[i];
+        const int r = g * NR + lane;
+        if (lane < NR && r < nrows) {
+            val *= sc;
+            val *= rs;
+            out[r] = val;
+            if (EPI == EPI_ARGMAX) {
+                if (val > myBestV || (val == myBestV && r < myBestI)) { myBestV = val; myBestI = r; }
+            }
+        }
+    }
+    if (EPI == EPI_ARGMAX) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            float ov = __shfl_xor(myBestV, o, 64);
+            int oi = __shfl_xor(myBestI, o, 64);
+            if (ov > myBestV || (ov == myBestV && oi < myBestI)) { myBestV = ov; myBestI = oi; }
+        }
+        if (lane == 0) { bestV[wave] = myBestV; bestI[wave] = myBestI; }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float bv = bestV[0]; int bi = bestI[0];
+            for (int k = 1; k < 4; k++)
+                if (bestV[k] > bv || (bestV[k] == bv && bestI[k] < bi)) { bv = bestV[k]; bi = bestI[k]; }
+            p.amaxVal[blockIdx.x] = bv;
+            p.amaxIdx[blockIdx.x] = bi;
+        }
+    }
+}
+
 // Launch shape from measurements on MI355X (cold weights, all benchmark shapes):
 // two rows per wave group is the best default, four for very tall matrices
 // (lm_head), and the K split over the workgroup only pays for long rows with
@@ -571,6 +661,15 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
         // the same number each (an uneven last round leaves most of the chip idle)
         const int rounds = (wgs + cap - 1) / cap;
         c.grid = epi == EPI_ARGMAX ? (wgs < cap ? wgs : cap) : (wgs + rounds - 1) / rounds;
+    }
+    if (wf == WF_Q8 && pro == PRO_RMS && epi == EPI_ARGMAX && p.nseg == 1 && !p.seg[0].bias && !p.div127 &&
+        p.K / 16 <= 64 && c.ks == 1 && !(cfgInOut && cfgInOut->nr > 0)) {
+        c.nr = 4;
+        wgs = ((p.seg[0].rows + 3) / 4 + 3) / 4;
+        c.grid = wgs < cap ? wgs : cap;
+        if (cfgInOut) *cfgInOut = c;
+        hipLaunchKernelGGL((matvec_rows_q8_kernel<EPI_ARGMAX>), dim3(c.grid), dim3(WG), (size_t)p.K * sizeof(float), s, p);
+        return hipGetLastError();
     }
     if (cfgInOut) *cfgInOut = c;
     if (wf == WF_Q8) return launch_wf<WF_Q8>(pro, epi, p, c, s);
