@@ -477,14 +477,13 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     }
 }
 
-// Tall matrix of short rows (lm_head of a small model: K <= 1024, so one wave pass covers a row):
-// a lane meets the same 16 activations in every row, so they are read from LDS once and stay in
+// Tall matrix of short rows (lm_head of a small model: K <= 1024*CH, so CH wave passes cover a row):
+// a lane meets the same 16*CH activations in every row, so they are read from LDS once and stay in
 // registers, and the loop is nothing but "four row loads, four dots, four reductions".  No ring:
-// the loads of the eight waves a SIMD holds overlap each other.  Arithmetic and order are
+// the loads of the waves a SIMD holds overlap each other.  Arithmetic and order are
 // matvec_kernel's, so the two give the same bits.
-template <int EPI>
+template <int EPI, int CH, int NR>
 __global__ __launch_bounds__(WG) void matvec_rows_q8_kernel(MvParams p) {
-    constexpr int NR = 4;
     extern __shared__ float4 a4[];
     __shared__ float red[4];
     __shared__ float bestV[4];
@@ -496,18 +495,20 @@ __global__ __launch_bounds__(WG) void matvec_rows_q8_kernel(MvParams p) {
     const char* __restrict__ w = static_cast<const char*>(p.seg[0].w);
     const float* __restrict__ scales = static_cast<const float*>(p.seg[0].aux);
     float* __restrict__ out = p.seg[0].out;
-    const bool live = lane < nch;
     const int gStep = gridDim.x * 4;
 
     int g = blockIdx.x * 4 + wave;
-    int4 v[NR];
+    int4 v[NR * CH];
     float scl = 0.f;
     auto fetch = [&](int gg) {
 #pragma unroll
         for (int i = 0; i < NR; i++) {
             const int r = gg * NR + i;
-            v[i] = make_int4(0, 0, 0, 0);
-            if (r < nrows && live) v[i] = *reinterpret_cast<const int4*>(w + (size_t)r * p.K + lane * 16);
+#pragma unroll
+            for (int ch = 0; ch < CH; ch++) {
+                v[i * CH + ch] = make_int4(0, 0, 0, 0);
+                if (r < nrows && lane + ch * 64 < nch) v[i * CH + ch] = *reinterpret_cast<const int4*>(w + (size_t)r * p.K + (lane + ch * 64) * 16);
+            }
         }
         scl = 0.f;
         if (lane < NR && gg * NR + lane < nrows) scl = scales[gg * NR + lane];
@@ -515,9 +516,11 @@ __global__ __launch_bounds__(WG) void matvec_rows_q8_kernel(MvParams p) {
     if (g * NR < nrows) fetch(g);                    // the first rows go out before the vector is staged
 
     const float rs = stage_activation<WF_Q8, PRO_RMS>(p, a4, red);
-    float4 av[4];
+    float4 av[CH * 4];
 #pragma unroll
-    for (int pl = 0; pl < 4; pl++) av[pl] = live ? a4[pl * nch + lane] : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int ch = 0; ch < CH; ch++)
+#pragma unroll
+        for (int pl = 0; pl < 4; pl++) av[ch * 4 + pl] = lane + ch * 64 < nch ? a4[pl * nch + lane + ch * 64] : make_float4(0.f, 0.f, 0.f, 0.f);
 
     float myBestV = -INFINITY;
     int myBestI = INT_MAX;
@@ -526,9 +529,13 @@ __global__ __launch_bounds__(WG) void matvec_rows_q8_kernel(MvParams p) {
 #pragma unroll
         for (int i = 0; i < NR; i++) {
             float a = 0.f;
-            a = dot4_i8(v[i].x, av[0], a); a = dot4_i8(v[i].y, av[1], a);
-            a = dot4_i8(v[i].z, av[2], a); a = dot4_i8(v[i].w, av[3], a);
+#pragma unroll
+            for (int ch = 0; ch < CH; ch++) {
+                a = dot4_i8(v[i * CH + ch].x, av[ch * 4], a); a = dot4_i8(v[i * CH + ch].y, av[ch * 4 + 1], a);
+                a = dot4_i8(v[i * CH + ch].z, av[ch * 4 + 2], a); a = dot4_i8(v[i * CH + ch].w, av[ch * 4 + 3], a);
+            }
             acc[i] = a;
+            if (CH > 1) asm volatile("" : "+v"(acc[i]));    // finished here, not sunk below the next loads
         }
         const float sc = scl;
         const int gNext = g + gStep;
@@ -541,6 +548,111 @@ __global__ __launch_bounds__(WG) void matvec_rows_q8_kernel(MvParams p) {
         const int r = g * NR + lane;
         if (lane < NR && r < nrows) {
             val *= sc;
+            val *= rs;
+            out[r] = val;
+            if (EPI == EPI_ARGMAX) {
+                if (val > myBestV || (val == myBestV && r < myBestI)) { myBestV = val; myBestI = r; }
+            }
+        }
+    }
+    if (EPI == EPI_ARGMAX) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            float ov = __shfl_xor(myBestV, o, 64);
+            int oi = __shfl_xor(myBestI, o, 64);
+            if (ov > myBestV || (ov == myBestV && oi < myBestI)) { myBestV = ov; myBestI = oi; }
+        }
+        if (lane == 0) { bestV[wave] = myBestV; bestI[wave] = myBestI; }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float bv = bestV[0]; int bi = bestI[0];
+            for (int k = 1; k < 4; k++)
+                if (bestV[k] > bv || (bestV[k] == bv && bestI[k] < bi)) { bv = bestV[k]; bi = bestI[k]; }
+            p.amaxVal[blockIdx.x] = bv;
+            p.amaxIdx[blockIdx.x] = bi;
+        }
+    }
+}
+
+// The same for Q4_0 rows in the split layout (K <= 1024): a lane owns one whole block (16 bytes of
+// nibbles + its fp16 d), so a row takes K/32 <= 32 lanes and each half of the wave streams its own
+// row; the lane's 32 activations and the two -8*sum terms stay in registers.
+template <int EPI>
+__global__ __launch_bounds__(WG) void matvec_rows_q4_kernel(MvParams p) {
+    constexpr int NR = 4;                            // row pairs per step
+    extern __shared__ float4 a4[];
+    __shared__ float red[4];
+    __shared__ float bestV[4];
+    __shared__ int bestI[4];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int half = lane >> 5, bl = lane & 31;
+    const int nblk = p.K / 32;
+    const int nch = p.K / 16;
+    const int nrows = p.seg[0].rows;
+    const char* __restrict__ qs = static_cast<const char*>(p.seg[0].w);
+    const unsigned short* __restrict__ dpl = reinterpret_cast<const unsigned short*>(qs + (size_t)nrows * (p.K >> 1));
+    float* __restrict__ out = p.seg[0].out;
+    const bool live = bl < nblk;
+    const int gStep = gridDim.x * 4;
+
+    int g = blockIdx.x * 4 + wave;
+    int4 v[NR];
+    unsigned short dh[NR];
+    auto fetch = [&](int gg) {
+#pragma unroll
+        for (int i = 0; i < NR; i++) {
+            const int r = (gg * NR + i) * 2 + half;
+            v[i] = make_int4(0, 0, 0, 0);
+            dh[i] = 0;
+            if (r < nrows && live) {
+                v[i] = *reinterpret_cast<const int4*>(qs + (size_t)r * (p.K >> 1) + bl * 16);
+                dh[i] = dpl[(size_t)r * nblk + bl];
+            }
+        }
+    };
+    if (g * NR * 2 < nrows) fetch(g);
+
+    const float rs = stage_activation<WF_Q4P, PRO_RMS>(p, a4, red);
+    // half block h of the lane's block: low nibbles meet lo[h][0..1], high nibbles hi[h][0..1]
+    float4 avh[2][4];
+    float asum[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int pl = 0; pl < 4; pl++) avh[h][pl] = live ? a4[pl * nch + bl * 2 + h] : make_float4(0.f, 0.f, 0.f, 0.f);
+        float4 t;
+        t.x = (avh[h][0].x + avh[h][1].x) + (avh[h][2].x + avh[h][3].x);
+        t.y = (avh[h][0].y + avh[h][1].y) + (avh[h][2].y + avh[h][3].y);
+        t.z = (avh[h][0].z + avh[h][1].z) + (avh[h][2].z + avh[h][3].z);
+        t.w = (avh[h][0].w + avh[h][1].w) + (avh[h][2].w + avh[h][3].w);
+        asum[h] = (t.x + t.y) + (t.z + t.w);
+    }
+
+    float myBestV = -INFINITY;
+    int myBestI = INT_MAX;
+#pragma nounroll
+    for (; g * NR * 2 < nrows; g += gStep) {
+        float acc[NR];
+#pragma unroll
+        for (int i = 0; i < NR; i++) {
+            const float d = half_bits_to_float(dh[i]);
+            float a = dot_q4_half(make_int2(v[i].x, v[i].y), d, avh[0], asum[0], 0.f);
+            acc[i] = dot_q4_half(make_int2(v[i].z, v[i].w), d, avh[1], asum[1], a);
+            asm volatile("" : "+v"(acc[i]));            // the row's sum is finished here, not sunk below the next loads
+        }
+        const int gNext = g + gStep;
+        if (gNext * NR * 2 < nrows) fetch(gNext);
+        float val = 0.f;
+#pragma unroll
+        for (int i = 0; i < NR; i++) {
+            float a = acc[i];                        // sum over the 32 lanes of this half
+            a += dpp_f<0xB1>(a); a += dpp_f<0x4E>(a); a += dpp_f<0x124>(a); a += dpp_f<0x128>(a);
+            a += __shfl_xor(a, 16, 64);
+            if (bl == i) val = a;
+        }
+        const int r = (g * NR + bl) * 2 + half;
+        if (bl < NR && r < nrows) {
             val *= rs;
             out[r] = val;
             if (EPI == EPI_ARGMAX) {
@@ -663,12 +775,23 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
         c.grid = epi == EPI_ARGMAX ? (wgs < cap ? wgs : cap) : (wgs + rounds - 1) / rounds;
     }
     if (wf == WF_Q8 && pro == PRO_RMS && epi == EPI_ARGMAX && p.nseg == 1 && !p.seg[0].bias && !p.div127 &&
-        p.K / 16 <= 64 && c.ks == 1 && !(cfgInOut && cfgInOut->nr > 0)) {
+        p.K / 16 <= 128 && c.ks == 1 && !(cfgInOut && cfgInOut->nr > 0)) {
         c.nr = 4;
         wgs = ((p.seg[0].rows + 3) / 4 + 3) / 4;
         c.grid = wgs < cap ? wgs : cap;
         if (cfgInOut) *cfgInOut = c;
-        hipLaunchKernelGGL((matvec_rows_q8_kernel<EPI_ARGMAX>), dim3(c.grid), dim3(WG), (size_t)p.K * sizeof(float), s, p);
+        const size_t lds = (size_t)p.K * sizeof(float);
+        if (p.K / 16 <= 64) hipLaunchKernelGGL((matvec_rows_q8_kernel<EPI_ARGMAX, 1, 4>), dim3(c.grid), dim3(WG), lds, s, p);
+        else hipLaunchKernelGGL((matvec_rows_q8_kernel<EPI_ARGMAX, 2, 4>), dim3(c.grid), dim3(WG), lds, s, p);
+        return hipGetLastError();
+    }
+    if (wf == WF_Q4P && pro == PRO_RMS && epi == EPI_ARGMAX && p.nseg == 1 && !p.seg[0].bias &&
+        p.K / 32 <= 32 && c.ks == 1 && !(cfgInOut && cfgInOut->nr > 0)) {
+        c.nr = 8;
+        wgs = ((p.seg[0].rows + 7) / 8 + 3) / 4;
+        c.grid = wgs < cap ? wgs : cap;
+        if (cfgInOut) *cfgInOut = c;
+        hipLaunchKernelGGL((matvec_rows_q4_kernel<EPI_ARGMAX>), dim3(c.grid), dim3(WG), (size_t)p.K * sizeof(float), s, p);
         return hipGetLastError();
     }
     if (cfgInOut) *cfgInOut = c;

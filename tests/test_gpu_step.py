@@ -353,3 +353,21 @@ def test_qwen_full_workload_paths_agree(hip):
     toks_ref, _ = H.oracle_generate(m, prompt, 6)
     assert toks_graph[:6].tolist() == toks_ref.tolist()
     m.close()
+
+
+@pytest.mark.parametrize("fmt,dim,heads,kvHeads,vocab", [
+    ("q8", 192, 3, 1, 1003),       # one chunk pass, 12 of 64 lanes live, vocab not a multiple of the row step
+    ("q8", 1024, 16, 4, 1001),     # one chunk pass, all lanes live
+    ("q8", 1536, 24, 4, 1003),     # two chunk passes, the second half empty
+    ("q8", 2048, 32, 4, 509),      # two full passes, fewer rows than one grid round
+    ("q4_0", 192, 3, 3, 1003),     # 6 of 32 block lanes live, odd row count (last pair ragged)
+    ("q4_0", 1024, 16, 2, 1001),   # all 32 block lanes live
+])
+def test_lm_head_short_row_kernels_ragged_shapes(hip, fmt, dim, heads, kvHeads, vocab):
+    """The lm_head kernels for rows of at most 2048 (Q8) / 1024 (Q4_0) weights on shapes that leave
+    lanes, chunk passes and the last row step partly empty: logits and greedy tokens against the oracle."""
+    s = configs.Shape(f"ragged-{fmt}-{dim}", 1, dim, heads, kvHeads, 64, 256, vocab, 1e-5, 1e4, False, fmt == "q8", fmt)
+    m = H.Model(s, seed=31, maxSeq=12, eng=hip, threads=4)
+    prompt = m.prompt(3)
+    _compare_sequence(m, prompt, 4, check_positions=[0, 2, 5])
+    m.close()
