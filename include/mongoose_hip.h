@@ -187,6 +187,26 @@ int mg_step_layer_resident(mg_ctx* ctx, int layer, int pos, const float* hiddenI
 /* ExportHidden :235-239. */
 int mg_export_hidden(mg_ctx* ctx, float* out /* [dim] */);
 
+/* L3 bridge and mailbox, cuda_fused_infer.go:118-131 and :556-737: every context owns a pinned host
+ * buffer ([0:4] mailbox counter, [64:] hidden state) for handing a pipeline stage's output to the
+ * host while the compute stream runs on.  mg_partial_step with both outputs NULL only queues the
+ * stage's launches; then either
+ *   mg_queue_hidden_to_l3 (QueueHiddenToL3 :688: the copy stream waits for the launches queued so
+ *   far and copies the hidden state into the bridge), mg_wait_l3 (WaitL3 :709: waits for that copy
+ *   only) and mg_get_l3_hidden (GetL3Hidden :725: host pointer to the dim floats), or
+ *   mg_signal_mailbox (SignalMailbox :558: a kernel behind the stage's last launch moves the
+ *   counter) and mg_wait_mailbox (WaitMailbox :575: the host polls the counter; here with a
+ *   timeout in milliseconds, MG_E_HIP when it expires, MG_E_STATE when no signal is outstanding).
+ * mg_swap_hidden_buffer (SwapHiddenBuffer :737) alternates the device hidden buffer, mg_hidden_idx
+ * (HiddenIdx :603) returns which of the two is current. */
+int mg_queue_hidden_to_l3(mg_ctx* ctx);
+int mg_wait_l3(mg_ctx* ctx);
+const float* mg_get_l3_hidden(mg_ctx* ctx);
+int mg_signal_mailbox(mg_ctx* ctx);
+int mg_wait_mailbox(mg_ctx* ctx, int timeoutMs);
+int mg_swap_hidden_buffer(mg_ctx* ctx);
+int mg_hidden_idx(mg_ctx* ctx);
+
 /* Execution mode of the layer loop: 0 = one launch per reference op, in the
  * reference's order (cuda_fused_infer.go:417-443, 17 launches a layer);
  * 1 = fused launches (default).  Both give the same results to rounding. */

@@ -77,6 +77,15 @@ public:
     int GeneratePrefill(const int* prompt, int nPrompt, int nDecode, int* outTokens);
     uint64_t WeightBytesPerToken() const;
     uint64_t KVBytesAt(int pos) const { return (uint64_t)2 * nLayers * (uint64_t)(pos + 1) * kvDim * (kvHalf ? 2 : 4); }
+    // L3 bridge (cuda_fused_infer.go:118-131, :556-737): a pinned host buffer, [0:4] mailbox counter,
+    // [64:] hidden state, for handing a pipeline stage's output to the host without a device sync.
+    int QueueHiddenToL3();                    // :688  copy stream waits for compute, then D2H into the bridge
+    int WaitL3();                             // :709  waits for the copy stream only
+    const float* GetL3Hidden() const;         // :725  host view of the bridge's hidden state
+    int SignalMailbox();                      // :558  kernel behind the stage's last launch bumps the counter
+    int WaitMailbox(int timeoutMs);           // :575  host polls the counter
+    int SwapHiddenBuffer();                   // :737
+    bool HasL3() const { return l3 != nullptr; }
     int SetKVFormat(int fmt);                 // 0: fp32 rows (the reference's layout), 1: fp16 rows
     int kvHalf = 0;
 
@@ -150,6 +159,11 @@ private:
     hipGraph_t graphFull = nullptr, graphPrompt = nullptr;
     hipGraphExec_t execFull = nullptr, execPrompt = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    // L3 bridge
+    char* l3 = nullptr;               // pinned: [0:4] mailbox counter, [64:64+dim*4] hidden
+    hipStream_t copyStream = nullptr;
+    hipEvent_t computeDone = nullptr;
+    unsigned mailboxSignaled = 0, mailboxExpected = 1;
     // instrumented run: an event between every two launches of a token
     std::vector<hipEvent_t> profEvents;
     std::vector<int> profClass;       // class of the launch that follows event i

@@ -5,6 +5,7 @@
 #include "host_util.h"
 #include "prefill.h"
 
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -92,6 +93,13 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
     };
     if (hipStreamCreateWithFlags(&f->stream, hipStreamNonBlocking) != hipSuccess) return fail("stream create failed");
     if (hipEventCreate(&f->ev0) != hipSuccess || hipEventCreate(&f->ev1) != hipSuccess) return fail("event create failed");
+    // L3 bridge: 64-byte mailbox line + the hidden state, pinned (cuda_fused_infer.go:204-217)
+    if (hipHostMalloc(reinterpret_cast<void**>(&f->l3), 64 + (size_t)dim * 4, hipHostMallocDefault) != hipSuccess)
+        return fail("L3 bridge allocation failed");
+    std::memset(f->l3, 0, 64 + (size_t)dim * 4);
+    if (hipStreamCreateWithFlags(&f->copyStream, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&f->computeDone, hipEventDisableTiming) != hipSuccess)
+        return fail("L3 copy stream create failed");
 
     // Every device buffer of the context comes out of a few large slabs (one for the scratch
     // and tables, one per layer of weights, one for the head, one per KV range): large
@@ -200,6 +208,9 @@ HIPFusedInference::~HIPFusedInference() {
     if (hGate) (void)hipHostFree(hGate);
     if (hTokens) (void)hipHostFree(hTokens);
     for (hipEvent_t e : profEvents) (void)hipEventDestroy(e);
+    if (copyStream) { (void)hipStreamSynchronize(copyStream); (void)hipStreamDestroy(copyStream); }
+    if (computeDone) (void)hipEventDestroy(computeDone);
+    if (l3) (void)hipHostFree(l3);
     if (ev0) (void)hipEventDestroy(ev0);
     if (ev1) (void)hipEventDestroy(ev1);
     if (stream) (void)hipStreamDestroy(stream);
@@ -586,8 +597,56 @@ int HIPFusedInference::PartialStep(const float* hiddenIn, int pos, int layerStar
         HIPCHK(hipStreamSynchronize(stream));
         HIPCHK(hipMemcpy(hiddenOut, h, (size_t)dim * 4, hipMemcpyDeviceToHost));
     }
-    HIPCHK(hipStreamSynchronize(stream));
+    return MG_OK;      // nothing read back: the launches stay queued (the reference does not sync here either)
+}
+
+// ---- L3 bridge and mailbox (cuda_fused_infer.go:556-737) ----
+int HIPFusedInference::QueueHiddenToL3() {
+    if (!built) return MG_E_NOT_BUILT;
+    HIPCHK(hipEventRecord(computeDone, stream));
+    HIPCHK(hipStreamWaitEvent(copyStream, computeDone, 0));
+    HIPCHK(hipMemcpyAsync(l3 + 64, hidden[hiddenIdx], (size_t)dim * 4, hipMemcpyDeviceToHost, copyStream));
     return MG_OK;
+}
+
+int HIPFusedInference::WaitL3() {
+    if (!built) return MG_E_NOT_BUILT;
+    HIPCHK(hipStreamSynchronize(copyStream));
+    return MG_OK;
+}
+
+const float* HIPFusedInference::GetL3Hidden() const {
+    return l3 ? reinterpret_cast<const float*>(l3 + 64) : nullptr;
+}
+
+int HIPFusedInference::SignalMailbox() {
+    if (!built) return MG_E_NOT_BUILT;
+    mailboxSignaled++;
+    HIPCHK(launch_signal_mailbox(reinterpret_cast<unsigned*>(l3), mailboxSignaled, stream));
+    return MG_OK;
+}
+
+int HIPFusedInference::WaitMailbox(int timeoutMs) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(timeoutMs > 0, "WaitMailbox: timeout must be positive");
+    if (mailboxSignaled < mailboxExpected) { set_error("WaitMailbox: no signal queued for this stage"); return MG_E_STATE; }
+    volatile unsigned* counter = reinterpret_cast<volatile unsigned*>(l3);
+    const auto t0 = std::chrono::steady_clock::now();
+    while (*counter < mailboxExpected) {
+        if (std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(timeoutMs)) {
+            set_error("WaitMailbox: timed out");
+            return MG_E_HIP;
+        }
+    }
+    mailboxExpected++;
+    return MG_OK;
+}
+
+int HIPFusedInference::SwapHiddenBuffer() {
+    if (!built) return MG_E_NOT_BUILT;
+    HIPCHK(hipStreamSynchronize(stream));
+    hiddenIdx = 1 - hiddenIdx;
+    return invalidateGraphs();                // captured launches point at the other buffer
 }
 
 int HIPFusedInference::StepLayerResident(int layer, int pos, const float* hiddenIn, float* preOut, float* postOut,
@@ -1006,6 +1065,13 @@ int mg_step_layer_resident(mg_ctx* c, int layer, int pos, const float* hiddenIn,
     CTX(c); return f->StepLayerResident(layer, pos, hiddenIn, preOut, postOut, logitsOut);
 }
 int mg_export_hidden(mg_ctx* c, float* out) { CTX(c); return f->ExportHidden(out); }
+int mg_queue_hidden_to_l3(mg_ctx* c) { CTX(c); return f->QueueHiddenToL3(); }
+int mg_wait_l3(mg_ctx* c) { CTX(c); return f->WaitL3(); }
+const float* mg_get_l3_hidden(mg_ctx* c) { return c && c->f ? c->f->GetL3Hidden() : nullptr; }
+int mg_signal_mailbox(mg_ctx* c) { CTX(c); return f->SignalMailbox(); }
+int mg_wait_mailbox(mg_ctx* c, int timeoutMs) { CTX(c); return f->WaitMailbox(timeoutMs); }
+int mg_swap_hidden_buffer(mg_ctx* c) { CTX(c); return f->SwapHiddenBuffer(); }
+int mg_hidden_idx(mg_ctx* c) { CTX(c); return f->hiddenIdx; }
 int mg_set_exec_mode(mg_ctx* c, int mode) {
     CTX(c);
     if (mode != 0 && mode != 1) { mg::set_error("exec mode must be 0 or 1"); return MG_E_ARG; }

@@ -126,6 +126,10 @@ hipError_t launch_set_state(StepState* state, int pos, int token, int count, int
 // Advance state without an lm_head (prompt positions): pos++, token = prompt[pos].
 hipError_t launch_advance_prompt(StepState* state, const int* prompt, RopeCur rope, hipStream_t s);
 
+// Pipeline-stage mailbox (SignalMailbox, cuda_fused_infer.go:558): stores `value` into a counter in
+// host-visible memory once everything queued before it on the stream has finished.
+hipError_t launch_signal_mailbox(unsigned* counter, unsigned value, hipStream_t s);
+
 // Stream gate for timing runs: waits for *flag != 0 (host-pinned) or limitTicks of the 100 MHz wall clock.
 hipError_t launch_gate(const int* flag, long long limitTicks, hipStream_t s);
 

@@ -1417,6 +1417,17 @@ hipError_t launch_advance_prompt(StepState* state, const int* prompt, RopeCur ro
 // Holds the stream until the host sets *flag (or the tick limit passes), so
 // that the host can queue a whole batch of launches ahead of the GPU.  One
 // lane; always exits.
+__global__ void signal_mailbox_kernel(unsigned* counter, unsigned value) {
+    // the stream orders this kernel behind the stage's launches; the fence makes their writes
+    // visible to the host before the counter moves
+    __atomic_thread_fence(__ATOMIC_SEQ_CST);
+    __hip_atomic_store(counter, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+hipError_t launch_signal_mailbox(unsigned* counter, unsigned value, hipStream_t s) {
+    hipLaunchKernelGGL(signal_mailbox_kernel, dim3(1), dim3(1), 0, s, counter, value);
+    return hipGetLastError();
+}
+
 __global__ void gate_kernel(const volatile int* flag, long long limitTicks) {
     const long long t0 = wall_clock64();
     while (__hip_atomic_load(const_cast<const int*>(flag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == 0) {

@@ -308,6 +308,33 @@ class HIPFusedInference:
     def SetExecMode(self, mode):
         return lib.mg_set_exec_mode(self._h, mode)
 
+    # L3 bridge and mailbox (cuda_fused_infer.go:556-737)
+    def QueueHiddenToL3(self):
+        return lib.mg_queue_hidden_to_l3(self._h)
+
+    def WaitL3(self):
+        return lib.mg_wait_l3(self._h)
+
+    def GetL3Hidden(self):
+        """Host view (no copy) of the bridge's hidden state; valid after QueueHiddenToL3 + WaitL3."""
+        p = lib.mg_get_l3_hidden(self._h)
+        return np.ctypeslib.as_array(p, shape=(self.dim,)) if p else None
+
+    def HasL3(self):
+        return bool(lib.mg_get_l3_hidden(self._h))
+
+    def SignalMailbox(self):
+        return lib.mg_signal_mailbox(self._h)
+
+    def WaitMailbox(self, timeoutMs=2000):
+        return lib.mg_wait_mailbox(self._h, timeoutMs)
+
+    def SwapHiddenBuffer(self):
+        return lib.mg_swap_hidden_buffer(self._h)
+
+    def HiddenIdx(self):
+        return lib.mg_hidden_idx(self._h)
+
     def PartialStep(self, hiddenIn, pos, layerStart, layerEnd, hiddenOut, logitsOut):
         h = _as_f32(hiddenIn) if hiddenIn is not None else None
         return lib.mg_partial_step(self._h, _fp(h), pos, layerStart, layerEnd, _fp(hiddenOut), _fp(logitsOut))

@@ -82,6 +82,13 @@ _sig("mg_partial_step", c_int, c_void_p, _f, c_int, c_int, c_int, _f, _f)
 _sig("mg_step_layer_resident", c_int, c_void_p, c_int, c_int, _f, _f, _f, _f)
 _sig("mg_export_hidden", c_int, c_void_p, _f)
 _sig("mg_set_exec_mode", c_int, c_void_p, c_int)
+_sig("mg_queue_hidden_to_l3", c_int, c_void_p)
+_sig("mg_wait_l3", c_int, c_void_p)
+_sig("mg_get_l3_hidden", _f, c_void_p)
+_sig("mg_signal_mailbox", c_int, c_void_p)
+_sig("mg_wait_mailbox", c_int, c_void_p, c_int)
+_sig("mg_swap_hidden_buffer", c_int, c_void_p)
+_sig("mg_hidden_idx", c_int, c_void_p)
 _sig("mg_decode_token", c_int, c_void_p, c_int, c_int, _i, _f)
 _sig("mg_generate", c_int, c_void_p, _i, c_int, c_int, _i, c_int)
 _sig("mg_graph_capture", c_int, c_void_p)

@@ -371,3 +371,45 @@ def test_lm_head_short_row_kernels_ragged_shapes(hip, fmt, dim, heads, kvHeads, 
     prompt = m.prompt(3)
     _compare_sequence(m, prompt, 4, check_positions=[0, 2, 5])
     m.close()
+
+
+def test_layer_range_pipeline_with_l3_bridge_and_mailbox(hip):
+    """Two contexts as pipeline stages (layers 0-1 and 2-3 of the toy model, PartialStep's layer
+    ranges): stage A's hidden state reaches the host through the L3 bridge (copy stream) and its
+    completion through the mailbox, stage B continues from it.  Logits equal the one-context run
+    bit for bit (same kernels on the same values) and match the oracle."""
+    s = configs.TOY
+    whole = H.Model(s, seed=41, maxSeq=8, eng=hip, threads=4)
+    a = H.Model(s, seed=41, maxSeq=8, eng=hip, oracle=False)
+    b = H.Model(s, seed=41, maxSeq=8, eng=hip, oracle=False)
+    assert a.hip.HasL3() and a.hip.HiddenIdx() == 0
+    prompt = whole.prompt(5)
+    whole.orc.reset_kv()
+    for pos in range(5):
+        h = whole.orc.embed(prompt[pos])
+        ref = np.empty(s.vocab, np.float32)
+        assert whole.hip.PartialStep(h, pos, 0, 4, None, ref) == 0, E.last_error()
+        # stage A: queue layers 0-1, then the hand-off
+        assert a.hip.PartialStep(h, pos, 0, 2, None, None) == 0, E.last_error()
+        assert a.hip.QueueHiddenToL3() == 0 and a.hip.SignalMailbox() == 0
+        assert a.hip.WaitMailbox(2000) == 0, E.last_error()      # stage A's launches are done
+        assert a.hip.WaitL3() == 0
+        mid = a.hip.GetL3Hidden().copy()
+        assert np.array_equal(mid, a.hip.ExportHidden())
+        # stage B: layers 2-3 and the head
+        got = np.empty(s.vocab, np.float32)
+        assert b.hip.PartialStep(mid, pos, 2, 4, None, got) == 0, E.last_error()
+        assert np.array_equal(got, ref), pos
+        _, lg, _ = whole.orc.step(h, pos, shadow=True, want_logits=True)
+        assert H.rel_err(got, lg) < LOGIT_TOL
+    # no signal outstanding: the wait refuses instead of spinning
+    assert a.hip.WaitMailbox(50) != 0 and "no signal" in E.last_error()
+    assert a.hip.WaitMailbox(0) != 0
+    # the second hidden buffer works the same
+    assert a.hip.SwapHiddenBuffer() == 0 and a.hip.HiddenIdx() == 1
+    h = whole.orc.embed(prompt[0])
+    assert a.hip.PartialStep(h, 5, 0, 2, None, None) == 0
+    assert a.hip.QueueHiddenToL3() == 0 and a.hip.WaitL3() == 0
+    assert np.array_equal(a.hip.GetL3Hidden(), a.hip.ExportHidden())
+    for m in (whole, a, b):
+        m.close()
