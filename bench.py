@@ -28,11 +28,11 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the lm_head kernel from rocprofv3 --pmc runs of this script
 # (FETCH_SIZE then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
-# reads for a 256 MiB device copy in the same run (FETCH_SIZE reads 131091.6 KiB for the
-# 262144 KiB copied -> x1.9997; WRITE_SIZE reads 262144.0 -> x1.0).  Counts are a property
+# reads for a 256 MiB device copy in the same run (FETCH_SIZE reads 131106.2 KiB for the
+# 262144 KiB copied -> x1.9995; WRITE_SIZE reads 262144.0 -> x1.0).  Counts are a property
 # of kernel and shape, so they are recorded here; profiles/ holds the run they come from.
 PMC_TRAFFIC_BYTES = {
-    "qwen2.5-0.5b": int((67167.6 * (262144.0 / 131091.6) + 660.2 * 1.0) * 1024),
+    "qwen2.5-0.5b": int((67136.6 * (262144.0 / 131106.2) + 661.7 * 1.0) * 1024),
 }
 
 
