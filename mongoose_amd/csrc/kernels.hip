@@ -919,15 +919,16 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
             q4[g][j] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (g < gn) q4[g][j] = reinterpret_cast<const float4*>(p.q + (size_t)(h0 + g) * HD)[j * 16 + dl];
         }
+    // K and V rows alternate in issue order, lowest rows first: the load unit works through them in
+    // that order, and a short context only waits for the rows it has (the rest is never looked at).
     float4 kreg[VU][NF], vreg[VU][NF];
 #pragma unroll
-    for (int u = 0; u < VU; u++)
+    for (int u = 0; u < VU; u++) {
 #pragma unroll
         for (int j = 0; j < NF; j++) kreg[u][j] = ld_kv4<KVH>(p.Kc, (size_t)min(t0 + tg + u * TG, lastRow) * rowStride + colOff + j * 16);
 #pragma unroll
-    for (int u = 0; u < VU; u++)
-#pragma unroll
         for (int j = 0; j < NF; j++) vreg[u][j] = ld_kv4<KVH>(p.Vc, (size_t)min(t0 + tg + u * TG, lastRow) * rowStride + colOff + j * 16);
+    }
 
     const int pos = p.state ? p.state->pos : p.posImm;
     const int len = pos + 1;
@@ -949,20 +950,22 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     for (int tile = t0; tile < t1; tile += TILE) {
         if (tile != t0) {
 #pragma unroll
-            for (int u = 0; u < VU; u++)
+            for (int u = 0; u < VU; u++) {
 #pragma unroll
                 for (int j = 0; j < NF; j++) kreg[u][j] = ld_kv4<KVH>(p.Kc, (size_t)min(tile + tg + u * TG, lastRow) * rowStride + colOff + j * 16);
 #pragma unroll
-            for (int u = 0; u < VU; u++)
-#pragma unroll
                 for (int j = 0; j < NF; j++) vreg[u][j] = ld_kv4<KVH>(p.Vc, (size_t)min(tile + tg + u * TG, lastRow) * rowStride + colOff + j * 16);
+            }
         }
+        const int live = t1 - tile;                        // positions of this tile that exist (uniform)
         float sc[GMAX][VU];
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
             float tmax = -INFINITY;
 #pragma unroll
             for (int u = 0; u < VU; u++) {
+                sc[g][u] = -INFINITY;
+                if (u * TG >= live) continue;              // whole row step past the end: its loads are not waited for
                 float d = 0.f;
 #pragma unroll
                 for (int j = 0; j < NF; j++) {
@@ -990,6 +993,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
             for (int j = 0; j < NF; j++) { acc[g][j].x *= corr; acc[g][j].y *= corr; acc[g][j].z *= corr; acc[g][j].w *= corr; }
 #pragma unroll
             for (int u = 0; u < VU; u++) {
+                if (u * TG >= live) continue;
                 const float pv = expf(sc[g][u] - mNew);    // masked rows: exp(-inf) = 0
                 ps += pv;
 #pragma unroll
