@@ -346,7 +346,25 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
 #pragma unroll
     for (int s = 0; s < D; s++) issue(s, s);
 
-    const float rs = stage_activation<WF, PRO>(p, a4, red);
+    // K split over the workgroup and at most two chunk rounds: a thread only ever meets its own one or
+    // two chunks of the vector, so it reads them straight into registers -- no LDS copy, no barrier,
+    // and no more bytes than staging reads.  (With KS == 1 every wave would read the whole vector
+    // itself, four times the requests: measured slower.)
+    constexpr bool CAN_DIRECT = KS == 4 && PRO == PRO_PLAIN && WF == WF_Q8;
+    const bool direct = CAN_DIRECT && iters <= 2;
+    float4 avr[2][4];
+    float rs = 1.0f;
+    if (direct) {
+        const float4* x4 = reinterpret_cast<const float4*>(p.act);
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int c = min(lig + it * LPG, nch - 1);
+#pragma unroll
+            for (int pl = 0; pl < 4; pl++) avr[it][pl] = x4[c * 4 + pl];
+        }
+    } else {
+        rs = stage_activation<WF, PRO>(p, a4, red);
+    }
 
     float myBestV = -INFINITY;
     int myBestI = INT_MAX;
@@ -366,8 +384,13 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
                 const int c = lig + it * LPG;
                 if (c < nch) {
                     float4 av[4];
+                    if (CAN_DIRECT && direct) {
 #pragma unroll
-                    for (int pl = 0; pl < 4; pl++) av[pl] = a4[pl * nch + c];
+                        for (int pl = 0; pl < 4; pl++) av[pl] = it == 0 ? avr[0][pl] : avr[1][pl];
+                    } else {
+#pragma unroll
+                        for (int pl = 0; pl < 4; pl++) av[pl] = a4[pl * nch + c];
+                    }
                     float asum = 0.f;
                     if (WF != WF_Q8) {
                         float4 t;
@@ -680,8 +703,8 @@ __global__ __launch_bounds__(WG) void matvec_rows_q4_kernel(MvParams p) {
 }
 
 // Launch shape from measurements on MI355X (cold weights, all benchmark shapes):
-// two rows per wave group is the best default, four for very tall matrices
-// (lm_head), and the K split over the workgroup only pays for long rows with
+// two rows per wave group is the best default, one for matrices of at most 1024 rows,
+// four for very tall ones (lm_head), and the K split over the workgroup only pays for long rows with
 // too few of them to give every CU a wave otherwise.
 MvConfig pick_config(int wf, int epi, int totalRows, int K) {
     const int nch = K / 16;
@@ -695,7 +718,8 @@ MvConfig pick_config(int wf, int epi, int totalRows, int K) {
     } else if (c.ks == 4) {
         c.nr = 4;
     } else {
-        c.nr = totalRows >= 65536 ? 4 : 2;
+        // few rows (Wo of a small model): one row a wave spreads them over twice the workgroups
+        c.nr = totalRows >= 65536 ? 4 : (totalRows <= 1024 ? 1 : 2);
     }
     c.grid = 0;   // filled by the launcher from the group count
     return c;
