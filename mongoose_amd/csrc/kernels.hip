@@ -350,7 +350,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     // two chunks of the vector, so it reads them straight into registers -- no LDS copy, no barrier,
     // and no more bytes than staging reads.  (With KS == 1 every wave would read the whole vector
     // itself, four times the requests: measured slower.)
-    constexpr bool CAN_DIRECT = KS == 4 && PRO == PRO_PLAIN && WF == WF_Q8;
+    constexpr bool CAN_DIRECT = KS == 4 && PRO == PRO_PLAIN;
     const bool direct = CAN_DIRECT && iters <= 2;
     float4 avr[2][4];
     float rs = 1.0f;
@@ -359,8 +359,16 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
 #pragma unroll
         for (int it = 0; it < 2; it++) {
             const int c = min(lig + it * LPG, nch - 1);
+            if (WF == WF_Q8) {
 #pragma unroll
-            for (int pl = 0; pl < 4; pl++) avr[it][pl] = x4[c * 4 + pl];
+                for (int pl = 0; pl < 4; pl++) avr[it][pl] = x4[c * 4 + pl];
+            } else {
+                // half block h of block blk: planes 0,1 meet its low nibbles (elements 8h..8h+7),
+                // planes 2,3 its high nibbles (16+8h..16+8h+7), as act_slot4 lays them out
+                const int base = (c >> 1) * 8 + (c & 1) * 2;
+                avr[it][0] = x4[base]; avr[it][1] = x4[base + 1];
+                avr[it][2] = x4[base + 4]; avr[it][3] = x4[base + 5];
+            }
         }
     } else {
         rs = stage_activation<WF, PRO>(p, a4, red);
