@@ -166,6 +166,9 @@ def main():
                     help="KV cache row format (f32 is the reference's; f16 is this backend's option, not the headline configuration)")
     ap.add_argument("--prefill", type=int, default=0,
                     help="also time a batched prefill of this many prompt tokens (extra 'prefill' object)")
+    ap.add_argument("--stream", type=int, default=0,
+                    help="also time this many tokens through the weight-streaming front end (Q4_0 configurations: "
+                         "every layer's weights cross PCIe per token; extra 'stream' object)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
@@ -183,7 +186,7 @@ def main():
         sys.exit(1)
     K, W = args.steps, max(args.warmup, 1)
     P0 = max(args.context, W)                      # position of the first timed step
-    maxSeq = max(P0 + K + args.profile_steps + 8, args.prefill)
+    maxSeq = max(P0 + K + args.profile_steps + 8, args.prefill, args.stream + 2)
     t_load = time.perf_counter()
     kv_f16 = args.kv == "f16"
     f = load_model(E, np, s, args.seed, maxSeq, eng, kv_f16=kv_f16)
@@ -280,6 +283,43 @@ def main():
                    "mfma_TFLOPs_issued": round(2 * flops / (pms * 1e-3) / 1e12, 2),
                    "note": "model flops = 2*T*weights of the layer projections; each is issued twice (bf16 hi and lo activation terms)"}
 
+    stream = None
+    if args.stream > 0:
+        if s.fmt != "q4_0":
+            print("bench.py: --stream needs a Q4_0 configuration (the streaming front end takes GGUF block_q4_0 layers)",
+                  file=sys.stderr)
+            sys.exit(2)
+        st = f.StreamBuild()
+        assert st is not None, E.last_error()
+        ptrs, sizes = [], []
+        for l in range(s.nLayers):
+            for w in range(12):
+                idx = l * 12 + w
+                rows, cols = slot_shape(s, kv, idx)
+                if cols == 1:
+                    ptrs.append(gen_slot(E, np, s, kv, args.seed, idx) if (w not in (4, 5, 6) or s.bias) else None)
+                else:
+                    blk = E.quantize_q4_0(gen_slot(E, np, s, kv, args.seed, idx))
+                    ptrs.append(blk)
+                    sizes.append(blk.size)
+        layer_bytes = sum(a.nbytes for a in ptrs if a is not None)
+        assert f.ResetKV() == 0
+        h0 = np.zeros(s.dim, np.float32)
+        h0[:] = E.synth_normal(args.seed, 30_000_001, 0.02, (s.dim,))
+        logits = np.empty(s.vocab, np.float32)
+        for pos in range(2):                               # warm the staging buffers
+            assert st.StreamForwardToken(pos, h0, s.nLayers, ptrs, sizes, logits) == 0, E.last_error()
+        t0 = time.perf_counter()
+        for i in range(args.stream):
+            assert st.StreamForwardToken(2 + i, h0, s.nLayers, ptrs, sizes, logits) == 0, E.last_error()
+        el = time.perf_counter() - t0
+        st.Close()
+        stream = {"tokens": args.stream, "ms_per_token": round(el / args.stream * 1e3, 3),
+                  "tok_per_s": round(args.stream / el, 1), "host_to_device_bytes_per_token": int(layer_bytes),
+                  "host_to_device_GBps": round(layer_bytes * args.stream / el / 1e9, 2),
+                  "note": "host wall clock; every token stages all layers from pageable host memory through two pinned "
+                          "buffers into two device sets (copy of layer l+1 overlaps compute of layer l); logits read back each token"}
+
     cpu = None
     if args.cpu_budget > 0:
         cpu = cpu_baseline(E, np, s, args.seed, prompt, toks, args.cpu_budget, kv_f16=kv_f16)
@@ -296,7 +336,7 @@ def main():
                    "kv_heads": s.nKVHeads, "ffn": s.ffnDim, "vocab": s.vocab, "graph_replay": use_graph},
         "step_bytes": int(step_bytes), "step_GBps": round(step_bytes * toks_per_s / 1e9, 1),
         "step_roofline_frac": round(step_bytes * toks_per_s / 1e9 / HBM_PEAK_GBS, 4),
-        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu, "prefill": prefill,
+        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu, "prefill": prefill, "stream": stream,
         "load_s": round(t_load, 1), "device": eng.Name(),
     }
     f.Close()

@@ -7,44 +7,119 @@
 #include "host_util.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
+#include <condition_variable>
 #include <cstring>
+#include <memory>
+#include <mutex>
 #include <thread>
 #include <vector>
 
 namespace mg {
 
+// A fixed set of worker threads shared by every host-side loop of the library (starting threads per
+// loop costs more than the per-layer staging loops themselves).  One parallel region at a time; the
+// calling thread takes jobs too.  Jobs must not start a region themselves.
+class WorkPool {
+    // Each parallel region has its own state object: a worker that wakes late holds the region it was
+    // woken for, finds its job counter exhausted and never touches a later region's function.
+    struct Region {
+        const std::function<void(size_t)>* fn;
+        size_t total;
+        std::atomic<size_t> next{0};
+        std::atomic<size_t> remaining;
+    };
+
+public:
+    static WorkPool& get() {
+        static WorkPool* pool = new WorkPool();      // lives until the process ends
+        return *pool;
+    }
+    void run(size_t njobs, const std::function<void(size_t)>& fn) {
+        if (njobs == 0) return;
+        if (njobs == 1 || nWorkers == 0) {
+            for (size_t j = 0; j < njobs; j++) fn(j);
+            return;
+        }
+        std::lock_guard<std::mutex> region(regionMutex);
+        auto r = std::make_shared<Region>();
+        r->fn = &fn; r->total = njobs; r->remaining.store(njobs);
+        {
+            std::lock_guard<std::mutex> lk(m);
+            current = r;
+            generation++;
+        }
+        wake.notify_all();
+        work(*r);
+        std::unique_lock<std::mutex> lk(m);
+        done.wait(lk, [&] { return r->remaining.load() == 0; });
+    }
+
+private:
+    WorkPool() {
+        unsigned hw = std::thread::hardware_concurrency();
+        if (hw == 0) hw = 1;
+        if (hw > 16) hw = 16;
+        nWorkers = hw - 1;
+        for (unsigned t = 0; t < nWorkers; t++) std::thread([this] { loop(); }).detach();
+    }
+    void work(Region& r) {
+        for (;;) {
+            const size_t j = r.next.fetch_add(1);
+            if (j >= r.total) break;
+            (*r.fn)(j);
+            if (r.remaining.fetch_sub(1) == 1) {
+                std::lock_guard<std::mutex> lk(m);
+                done.notify_all();
+            }
+        }
+    }
+    void loop() {
+        unsigned long seen = 0;
+        for (;;) {
+            std::shared_ptr<Region> r;
+            {
+                std::unique_lock<std::mutex> lk(m);
+                wake.wait(lk, [&] { return generation != seen; });
+                seen = generation;
+                r = current;
+            }
+            if (r) work(*r);
+        }
+    }
+    unsigned nWorkers = 0;
+    std::mutex regionMutex, m;
+    std::condition_variable wake, done;
+    std::shared_ptr<Region> current;
+    unsigned long generation = 0;
+};
+
+void parallel_jobs(size_t njobs, const std::function<void(size_t)>& fn) { WorkPool::get().run(njobs, fn); }
+
 void parallel_for(size_t n, size_t grain, const std::function<void(size_t, size_t)>& fn) {
     if (n == 0) return;
-    unsigned hw = std::thread::hardware_concurrency();
-    if (hw == 0) hw = 1;
-    if (hw > 16) hw = 16;
-    size_t chunks = (n + grain - 1) / grain;
-    size_t nt = std::min<size_t>(hw, chunks);
-    if (nt <= 1) { fn(0, n); return; }
-    std::vector<std::thread> th;
-    size_t per = (chunks + nt - 1) / nt * grain;
-    for (size_t t = 0; t < nt; t++) {
-        size_t a = t * per, b = std::min(n, a + per);
-        if (a >= b) break;
-        th.emplace_back([=, &fn] { fn(a, b); });
-    }
-    for (auto& x : th) x.join();
+    if (grain == 0) grain = 1;
+    const size_t chunks = (n + grain - 1) / grain;
+    if (chunks <= 1) { fn(0, n); return; }
+    parallel_jobs(chunks, [&](size_t c) { fn(c * grain, std::min(n, (c + 1) * grain)); });
 }
 
 // Split layout read by the fast Q4_0 kernel: all 16-byte nibble groups of the
 // matrix (row-major), then all fp16 block scales.  Same bytes as GGUF, only
 // regrouped so that both are reachable with aligned loads.
-void repack_q4_0_host(const uint8_t* raw, int rows, int cols, uint8_t* planar) {
-    size_t nb = (size_t)rows * (cols / 32);
+void repack_q4_0_blocks(const uint8_t* raw, size_t nb, size_t b0, size_t b1, uint8_t* planar) {
     uint8_t* qs = planar;
     uint8_t* d = planar + nb * 16;
-    parallel_for(nb, 1 << 14, [&](size_t a, size_t b) {
-        for (size_t i = a; i < b; i++) {
-            std::memcpy(qs + i * 16, raw + i * 18 + 2, 16);
-            std::memcpy(d + i * 2, raw + i * 18, 2);
-        }
-    });
+    for (size_t i = b0; i < b1; i++) {
+        std::memcpy(qs + i * 16, raw + i * 18 + 2, 16);
+        std::memcpy(d + i * 2, raw + i * 18, 2);
+    }
+}
+
+void repack_q4_0_host(const uint8_t* raw, int rows, int cols, uint8_t* planar) {
+    const size_t nb = (size_t)rows * (cols / 32);
+    parallel_for(nb, 1 << 13, [&](size_t a, size_t b) { repack_q4_0_blocks(raw, nb, a, b, planar); });
 }
 
 }  // namespace mg

@@ -15,7 +15,9 @@
 #include "../../include/mongoose_hip.h"
 #include "host_util.h"
 
+#include <algorithm>
 #include <cstring>
+#include <vector>
 
 namespace mg {
 
@@ -107,18 +109,29 @@ public:
         return MG_OK;
     }
 
-    // stageLayerToPinned, cuda_fused_stream.go:200-247 (NULL bias -> zeros).
+    // stageLayerToPinned, cuda_fused_stream.go:200-247 (NULL bias -> zeros).  The seven matrices are cut
+    // into pieces of 8192 blocks and regrouped by all worker threads in one parallel region.
     int stage(int set, const void* const* ptrs, const int32_t* sizes) {
         static const int matIdx[7] = {1, 2, 3, 7, 9, 10, 11};        // order of layerSizes[i*7+m] (:571-598)
+        constexpr size_t PIECE = 8192;
         char* dst = pinned[set];
+        struct Job { const uint8_t* src; uint8_t* out; size_t nb, b0, b1; };
+        std::vector<Job> jobs;
         for (int m = 0; m < 7; m++) {
             int k = matIdx[m];
             if (!ptrs[k]) { set_error("StreamForwardToken: NULL matrix pointer"); return MG_E_ARG; }
             if ((size_t)sizes[m] != nbytes[k]) { set_error("StreamForwardToken: layerSizes entry is not rows*(cols/32)*18"); return MG_E_ARG; }
             int r, c;
             matShape(k, &r, &c);
-            repack_q4_0_host(static_cast<const uint8_t*>(ptrs[k]), r, c, reinterpret_cast<uint8_t*>(dst + off[k]));
+            const size_t nb = (size_t)r * (c / 32);
+            for (size_t b0 = 0; b0 < nb; b0 += PIECE)
+                jobs.push_back(Job{static_cast<const uint8_t*>(ptrs[k]), reinterpret_cast<uint8_t*>(dst + off[k]), nb, b0,
+                                   std::min(nb, b0 + PIECE)});
         }
+        parallel_jobs(jobs.size(), [&](size_t j) {
+            const Job& jb = jobs[j];
+            repack_q4_0_blocks(jb.src, jb.nb, jb.b0, jb.b1, jb.out);
+        });
         for (int k : {0, 8}) {
             if (!ptrs[k]) { set_error("StreamForwardToken: NULL norm pointer"); return MG_E_ARG; }
             std::memcpy(dst + off[k], ptrs[k], nbytes[k]);
