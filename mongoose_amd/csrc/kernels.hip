@@ -1097,34 +1097,41 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     __syncthreads();
     if (!lastFlag) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");     // drop cached copies of the other workgroups' partials
-    for (int i = tid; i < gn * F4; i += WG) {
-        int g = i / F4, d4 = i % F4;
-        int h = h0 + g;
+    // The workgroup's threads form NG groups of IT = GMAX*F4 items (head, float4 of the head); group q
+    // merges the splits q, q+NG, ... 16 at a time -- all 48 loads of a batch are issued before the first
+    // is used, one memory round trip a batch, and up to 16*NG splits need only one -- and the NG results
+    // of an item are folded through LDS with the same running-maximum rescale.
+    constexpr int IT = GMAX * F4;
+    constexpr int NG = WG / IT;
+    __shared__ float4 cnum[WG];
+    __shared__ float cM[WG], cden[WG];
+    {
+        const int q = tid / IT, i = tid % IT;
+        const int g = i / F4, d4 = i % F4;
+        const int h = h0 + min(g, gn - 1);                           // heads past gn repeat the last one, dropped below
         const float* pm = p.pm + (size_t)h * p.smax;
         const float* pl = p.pl + (size_t)h * p.smax;
         const float4* pa = reinterpret_cast<const float4*>(p.pacc + (size_t)h * p.smax * HD) + d4;
-        // Splits are merged 16 at a time: all 48 loads of a batch are issued before the first is
-        // used (one memory round trip a batch), then folded in with the running-maximum rescale.
         float M = -INFINITY, den = 0.f;
         float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int s0 = 0; s0 < nsplit; s0 += 16) {
+        for (int s0 = q; s0 < nsplit; s0 += 16 * NG) {
             float pmv[16], plv[16];
             float4 pav[16];
 #pragma unroll
             for (int u = 0; u < 16; u++) {
-                const int sidx = min(s0 + u, nsplit - 1);           // clamped, unconditional: stays in registers
+                const int sidx = min(s0 + u * NG, nsplit - 1);      // clamped, unconditional: stays in registers
                 pmv[u] = pm[sidx]; plv[u] = pl[sidx]; pav[u] = pa[(size_t)sidx * F4];
             }
             float bm = -INFINITY;
 #pragma unroll
-            for (int u = 0; u < 16; u++) if (s0 + u < nsplit) bm = fmaxf(bm, pmv[u]);
+            for (int u = 0; u < 16; u++) if (s0 + u * NG < nsplit) bm = fmaxf(bm, pmv[u]);
             const float Mn = fmaxf(M, bm);
             const float c = expf(M - Mn);                           // first batch: exp(-inf) = 0
             den *= c; num.x *= c; num.y *= c; num.z *= c; num.w *= c;
             M = Mn;
 #pragma unroll
             for (int u = 0; u < 16; u++) {
-                if (s0 + u < nsplit) {
+                if (s0 + u * NG < nsplit) {
                     const float w = expf(pmv[u] - M);
                     den = fmaf(w, plv[u], den);
                     num.x = fmaf(w, pav[u].x, num.x); num.y = fmaf(w, pav[u].y, num.y);
@@ -1132,9 +1139,25 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
                 }
             }
         }
-        float4 o;
-        o.x = num.x / den; o.y = num.y / den; o.z = num.z / den; o.w = num.w / den;
-        reinterpret_cast<float4*>(p.out + (size_t)h * HD)[d4] = o;
+        cM[tid] = M; cden[tid] = den; cnum[tid] = num;              // a group without splits leaves (-inf, 0, 0)
+        __syncthreads();
+        if (q == 0 && g < gn) {
+            float Mt = cM[i];
+#pragma unroll
+            for (int k = 1; k < NG; k++) Mt = fmaxf(Mt, cM[k * IT + i]);
+            float dt = 0.f;
+            float4 nt = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int k = 0; k < NG; k++) {
+                const float w = expf(cM[k * IT + i] - Mt);           // empty group: exp(-inf) = 0
+                const float4 a = cnum[k * IT + i];
+                dt = fmaf(w, cden[k * IT + i], dt);
+                nt.x = fmaf(w, a.x, nt.x); nt.y = fmaf(w, a.y, nt.y); nt.z = fmaf(w, a.z, nt.z); nt.w = fmaf(w, a.w, nt.w);
+            }
+            float4 o;
+            o.x = nt.x / dt; o.y = nt.y / dt; o.z = nt.z / dt; o.w = nt.w / dt;
+            reinterpret_cast<float4*>(p.out + (size_t)h * HD)[d4] = o;
+        }
     }
     if (tid == 0) __hip_atomic_store(p.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
