@@ -717,7 +717,7 @@ __global__ __launch_bounds__(WG) void matvec_rows_q4_kernel(MvParams p) {
 MvConfig pick_config(int wf, int epi, int totalRows, int K) {
     const int nch = K / 16;
     MvConfig c;
-    c.ks = (nch > 128 && totalRows < 2048) ? 4 : 1;
+    c.ks = (nch > 128 && totalRows <= 2048) ? 4 : 1;
     if (epi == EPI_QKV) {
         c.nr = 2;
     } else if (epi == EPI_SWIGLU) {
