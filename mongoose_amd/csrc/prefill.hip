@@ -358,7 +358,9 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
     int sgi = 0;
     if (p.nseg > 1 && nTile >= p.seg[1].tile0) sgi = 1;
     if (p.nseg > 2 && nTile >= p.seg[2].tile0) sgi = 2;
-    const GemmSeg sg = p.seg[sgi];
+    GemmSeg sg = p.seg[0];                       // selected by value: indexing the argument array by a
+    if (sgi == 1) sg = p.seg[1];                 // run-time index would copy it into scratch memory
+    if (sgi == 2) sg = p.seg[2];
     const int N = sg.N, K = p.K, T = p.T;
     const int m0 = mTile * BM, n0 = (nTile - sg.tile0) * BN;
     const int ksteps = (K + BK - 1) / BK;
@@ -399,23 +401,34 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
 
     int4 gAh[AR], gAl[AR], gB[BR];
     unsigned short gD[2] = {0, 0};
-    const int4 zero4 = make_int4(0, 0, 0, 0);
-    auto gload = [&](int k0) {       // K is a multiple of 32: a last half step reads zeros past the end
-        const bool okA = k0 + aSeg * 8 < K;
-        const bool okB = bActive && (Q4 ? k0 + bSeg * 32 < K : k0 + bSeg * 16 < K);
-#pragma unroll
-        for (int r = 0; r < AR; r++) {
-            gAh[r] = okA ? *reinterpret_cast<const int4*>(aHiP[r] + (size_t)k0 * 128) : zero4;   // 8192 elements per K step
-            gAl[r] = okA ? *reinterpret_cast<const int4*>(aLoP[r] + (size_t)k0 * 128) : zero4;
-        }
-#pragma unroll
-        for (int r = 0; r < BR; r++) gB[r] = okB ? *reinterpret_cast<const int4*>(bP[r] + (Q4 ? k0 >> 1 : k0)) : zero4;
-        if (Q4 && dP) {
-            gD[0] = dP[k0 >> 5];
-            gD[1] = k0 + 32 < K ? dP[(k0 >> 5) + 1] : (unsigned short)0;
-        }
-    };
-    if (stepBeg < stepEnd) gload(stepBeg * BK);
+    // K is a multiple of 32: a last half step reads zeros past the end.  The load itself is never
+    // conditional (`ok ? *p : zero` made the compiler select between p and the address of a private
+    // zero, i.e. a flat load that is waited for at once and staged through scratch memory): a
+    // segment past the end re-reads the step's first segment and is zeroed afterwards.
+    // (A macro rather than a lambda: with the staging arrays captured by reference the compiler kept
+    // them in scratch memory in some instantiations.)
+#define MG_GEMM_GLOAD(K0)                                                                                   \
+    do {                                                                                                    \
+        const int k0_ = (K0);                                                                               \
+        const bool okA_ = k0_ + aSeg * 8 < K;                                                               \
+        const bool okB_ = bActive && (Q4 ? k0_ + bSeg * 32 < K : k0_ + bSeg * 16 < K);                      \
+        const int aBack_ = okA_ ? 0 : aSeg * 8;      /* elements back to segment 0 of the step */           \
+        const int bBack_ = okB_ ? 0 : bSeg * 16;     /* bytes back to segment 0 of the step */              \
+        _Pragma("unroll") for (int r = 0; r < AR; r++) {                                                    \
+            gAh[r] = *reinterpret_cast<const int4*>(aHiP[r] + (size_t)k0_ * 128 - aBack_);                  \
+            gAl[r] = *reinterpret_cast<const int4*>(aLoP[r] + (size_t)k0_ * 128 - aBack_);                  \
+            if (!okA_) { gAh[r] = make_int4(0, 0, 0, 0); gAl[r] = make_int4(0, 0, 0, 0); }                  \
+        }                                                                                                   \
+        _Pragma("unroll") for (int r = 0; r < BR; r++) {                                                    \
+            gB[r] = *reinterpret_cast<const int4*>(bP[r] + (Q4 ? k0_ >> 1 : k0_) - bBack_);                 \
+            if (!okB_) gB[r] = make_int4(0, 0, 0, 0);                                                       \
+        }                                                                                                   \
+        if (Q4 && dP) {                                                                                     \
+            gD[0] = dP[k0_ >> 5];                                                                           \
+            gD[1] = k0_ + 32 < K ? dP[(k0_ >> 5) + 1] : (unsigned short)0;                                  \
+        }                                                                                                   \
+    } while (0)
+    if (stepBeg < stepEnd) MG_GEMM_GLOAD(stepBeg * BK);
     for (int step = stepBeg; step < stepEnd; step++) {
         __syncthreads();                       // the previous step's fragments are consumed
 #pragma unroll
@@ -431,7 +444,7 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
             sD[tid * 2 + 1] = (float)__builtin_bit_cast(_Float16, gD[1]);
         }
         __syncthreads();
-        if (step + 1 < stepEnd) gload((step + 1) * BK);       // next tile in flight while this one is multiplied
+        if (step + 1 < stepEnd) MG_GEMM_GLOAD((step + 1) * BK);       // next tile in flight while this one is multiplied
         if (Q4) {
             float16_t zero16;
 #pragma unroll
@@ -516,21 +529,20 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
                     const int m = m0 + wm * (BM / WM) + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                     if (m < T) dst[(size_t)m * p.ldPartial] = acc[i][j][e];
                 }
-            continue;
-        }
-        if (n >= N) continue;
-        const float sc = Q4 ? 1.0f : sg.scales[n];
-        const float bi = sg.bias ? sg.bias[n] : 0.f;
+        } else if (n < N) {      // no `continue` in this loop: it must unroll, or acc is indexed at run time (scratch)
+            const float sc = Q4 ? 1.0f : sg.scales[n];
+            const float bi = sg.bias ? sg.bias[n] : 0.f;
 #pragma unroll
-        for (int i = 0; i < MI; i++) {
+            for (int i = 0; i < MI; i++) {
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int m = m0 + wm * (BM / WM) + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                if (m < T) {
-                    float v = acc[i][j][e] * sc + bi;
-                    float* dst = sg.Y + (size_t)m * N + n;
-                    if (MODE == 1) v = *dst + v;
-                    *dst = v;
+                for (int e = 0; e < 16; e++) {
+                    const int m = m0 + wm * (BM / WM) + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                    if (m < T) {
+                        float v = acc[i][j][e] * sc + bi;
+                        float* dst = sg.Y + (size_t)m * N + n;
+                        if (MODE == 1) v = *dst + v;
+                        *dst = v;
+                    }
                 }
             }
         }
@@ -707,7 +719,9 @@ __global__ __launch_bounds__(PWG) void gemm_reduce_kernel(GemmParams p, int BN, 
     int sgi = 0;
     if (p.nseg > 1 && tile >= p.seg[1].tile0) sgi = 1;
     if (p.nseg > 2 && tile >= p.seg[2].tile0) sgi = 2;
-    const GemmSeg sg = p.seg[sgi];
+    GemmSeg sg = p.seg[0];
+    if (sgi == 1) sg = p.seg[1];
+    if (sgi == 2) sg = p.seg[2];
     const int n = c - sg.tile0 * BN;
     if (n >= sg.N) return;
     const float* src = p.partial + (size_t)m * p.ldPartial + c;
