@@ -304,7 +304,13 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     const int nItems = myGroups * iters;
 
     int pos = 0;
-    if (EPI == EPI_QKV) pos = p.state ? p.state->pos : p.posImm;
+    if (EPI == EPI_QKV) {
+        // not `state ? state->pos : posImm`: that selects between a global address and the kernel-argument
+        // address, i.e. a flat load, and the kernel's first scalar/LDS wait then sits behind it.  A vector
+        // load issued ahead of the weights instead: it is back before they are, and nothing waits for it alone.
+        pos = p.posImm;
+        if (p.state) pos = __hip_atomic_load(&p.state->pos, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 
     typename F::Chunk ring[D][NR];
     float rSc[D], rBi[D], rRe[D], rCs[D], rSn[D];            // epilogue operands of the lane's row
@@ -962,7 +968,7 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
         for (int j = 0; j < NF; j++) vreg[u][j] = ld_kv4<KVH>(p.Vc, (size_t)min(t0 + tg + u * TG, lastRow) * rowStride + colOff + j * 16);
     }
 
-    const int pos = p.state ? p.state->pos : p.posImm;
+    const int pos = p.state ? p.state->pos : p.posImm;     // compiles to a branch and a scalar load (checked)
     const int len = pos + 1;
     if (t0 >= len) return;                                 // this split holds no position yet
     const int nsplit = p.splitLen > 0 ? (len + p.splitLen - 1) / p.splitLen : 1;
