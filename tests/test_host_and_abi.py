@@ -83,3 +83,28 @@ def test_context_requires_device_or_fails_cleanly():
     else:
         assert f is not None and f.NumWeights() == 14
         f.Close()
+
+
+def test_host_worker_pool_is_safe_under_concurrent_callers():
+    """The library's host loops share one set of worker threads, one parallel region at a time.
+    Several Python threads (ctypes drops the GIL) quantizing matrices of very different sizes at
+    once must each get exactly what a lone caller gets."""
+    import threading
+    mats = [(rng.standard_normal((r, 256)) * 0.02).astype(np.float32) for r in (1, 3, 17, 64, 300, 1000)]
+    want = [(E.quantize_q8(m, 0), E.quantize_q4_0(m)) for m in mats]
+    bad = []
+
+    def worker(seed):
+        for it in range(60):
+            i = (seed + it) % len(mats)
+            q, s = E.quantize_q8(mats[i], 0)
+            b = E.quantize_q4_0(mats[i])
+            if not (np.array_equal(q, want[i][0][0]) and np.array_equal(s, want[i][0][1]) and np.array_equal(b, want[i][1])):
+                bad.append((seed, it))
+
+    ths = [threading.Thread(target=worker, args=(k,)) for k in range(6)]
+    for t in ths:
+        t.start()
+    for t in ths:
+        t.join()
+    assert not bad, bad[:5]
