@@ -966,6 +966,7 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
     } else {
         HIPCHK(launch_embed_rows(lmHead.kind == WF_Q8 ? 0 : 3, lmHead.w, lmHead.scales, pfTokens, pfX, T, dim, vocabSize, stream));
     }
+    bool normSplitDone = false;
     for (int l = 0; l < nLayers; l++) {
         const LayerWeights& L = layers[l];
         auto seg = [](const DevMat& m, const float* bias, float* y) {
@@ -974,7 +975,8 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
         GemmParams g{};
         g.T = T; g.Ahi = static_cast<const unsigned short*>(pfHi); g.Alo = static_cast<const unsigned short*>(pfLo);
         g.partial = pfPartial;
-        HIPCHK(launch_split_rows(pfX, L.norm1, eps, T, dim, pfHi, pfLo, stream));
+        // (the previous layer's down projection may already have written this split)
+        if (!normSplitDone) HIPCHK(launch_split_rows(pfX, L.norm1, eps, T, dim, pfHi, pfLo, stream));
         g.K = dim; g.nseg = 3; g.q4 = L.wq.kind == WF_Q4P;
         g.seg[0] = seg(L.wq, L.bq, pfQ); g.seg[1] = seg(L.wk, L.bk, pfK); g.seg[2] = seg(L.wv, L.bv, pfV);
         HIPCHK(launch_gemm_q8(g, 0, stream));
@@ -982,13 +984,22 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
         HIPCHK(launch_prefill_attention(pfQ, kCache[l], vCache[l], kvHalf, pfAttn, T, pos0, maxSeq, dim, kvDim, nHeads, nKVHeads, headDim, stream));
         HIPCHK(launch_split_rows(pfAttn, nullptr, eps, T, dim, pfHi, pfLo, stream));
         g.K = dim; g.nseg = 1; g.q4 = L.wo.kind == WF_Q4P; g.seg[0] = seg(L.wo, nullptr, pfX);
+        // where K is split, the kernel that sums the splits also writes norm2's split of the new rows
+        g.nextGain = L.norm2; g.nextEps = eps;
+        g.nextHi = static_cast<unsigned short*>(pfHi); g.nextLo = static_cast<unsigned short*>(pfLo);
         HIPCHK(launch_gemm_q8(g, 1, stream));
-        HIPCHK(launch_split_rows(pfX, L.norm2, eps, T, dim, pfHi, pfLo, stream));
+        if (!g.wroteNext) HIPCHK(launch_split_rows(pfX, L.norm2, eps, T, dim, pfHi, pfLo, stream));
+        g.nextGain = nullptr; g.nextHi = nullptr; g.nextLo = nullptr;
         g.K = dim; g.nseg = 2; g.q4 = L.gate.kind == WF_Q4P; g.seg[0] = seg(L.gate, nullptr, pfGate); g.seg[1] = seg(L.up, nullptr, pfUp);
         HIPCHK(launch_gemm_q8(g, 0, stream));
         HIPCHK(launch_swiglu_split(pfGate, pfUp, T, ffnDim, pfHi, pfLo, stream));
         g.K = ffnDim; g.nseg = 1; g.q4 = L.down.kind == WF_Q4P; g.seg[0] = seg(L.down, nullptr, pfX);
+        if (l + 1 < nLayers) {                  // ... and here the next layer's norm1 split
+            g.nextGain = layers[l + 1].norm1; g.nextEps = eps;
+            g.nextHi = static_cast<unsigned short*>(pfHi); g.nextLo = static_cast<unsigned short*>(pfLo);
+        }
         HIPCHK(launch_gemm_q8(g, 1, stream));
+        normSplitDone = g.wroteNext != 0;
     }
     // the last position continues on the decode path: final norm, lm_head, greedy token, state -> pos0 + T
     HIPCHK(hipMemcpyAsync(hidden[hiddenIdx], pfX + (size_t)(T - 1) * dim, (size_t)dim * 4, hipMemcpyDeviceToDevice, stream));

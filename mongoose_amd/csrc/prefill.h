@@ -34,8 +34,16 @@ struct GemmParams {
     int T, K;
     int q4;
     float* partial;   // workspace of gemm_partial_floats() floats for K-split partial sums (NULL: never split K)
+    // Optional (one matrix, residual form): when K was split, the kernel that sums the splits into Y also
+    // writes the hi/lo split of the finished rows, RMS-normalised with nextGain (NULL: plain), for the
+    // projection that follows -- into nextHi/nextLo, in launch_split_rows's layout for K = N.
+    const float* nextGain;
+    float nextEps;
+    unsigned short* nextHi;
+    unsigned short* nextLo;
     // filled by the launcher
     int nTiles, splitK, stepsPerSplit, ldPartial;
+    int wroteNext;    // 1: nextHi/nextLo were written; 0: the caller still has to split Y's rows itself
 };
 size_t gemm_partial_floats();
 hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s);

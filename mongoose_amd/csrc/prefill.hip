@@ -733,6 +733,83 @@ __global__ __launch_bounds__(PWG) void gemm_reduce_kernel(GemmParams p, int BN, 
     *dst = v;
 }
 
+// The same for one matrix in residual form, one workgroup per row, with the row kept in registers:
+// x = Y + scale * (sum of the splits) + bias is stored, and the next projection's (RMSNorm +) hi/lo
+// split of x is written straight away (split_rows_kernel's arithmetic, term by term).  N <= 16384.
+__global__ __launch_bounds__(PWG) void gemm_reduce_norm_split_kernel(GemmParams p) {
+    constexpr int MAXV = 16;                            // float4 per thread
+    __shared__ float red[4];
+    const int m = blockIdx.x;
+    const GemmSeg sg = p.seg[0];
+    const int N = sg.N;
+    const size_t plane = (size_t)p.T * p.ldPartial;
+    const float4* src = reinterpret_cast<const float4*>(p.partial + (size_t)m * p.ldPartial);
+    float4* y4 = reinterpret_cast<float4*>(sg.Y + (size_t)m * N);
+    float4 x[MAXV];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXV; i++) {
+        const int c4 = threadIdx.x + i * PWG;
+        if (c4 * 4 >= N) continue;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        int s = 0;
+        for (; s + 4 <= p.splitK; s += 4) {             // four loads in flight, added in split order
+            const float4 a = src[(size_t)s * plane / 4 + c4], b = src[(size_t)(s + 1) * plane / 4 + c4];
+            const float4 c = src[(size_t)(s + 2) * plane / 4 + c4], d = src[(size_t)(s + 3) * plane / 4 + c4];
+            v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
+            v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+            v.x += c.x; v.y += c.y; v.z += c.z; v.w += c.w;
+            v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+        }
+        for (; s < p.splitK; s++) {
+            const float4 a = src[(size_t)s * plane / 4 + c4];
+            v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
+        }
+        float4 sc = make_float4(1.f, 1.f, 1.f, 1.f), bi = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (sg.scales) sc = reinterpret_cast<const float4*>(sg.scales)[c4];
+        if (sg.bias) bi = reinterpret_cast<const float4*>(sg.bias)[c4];
+        const float4 r = y4[c4];
+        v.x = r.x + (v.x * sc.x + bi.x); v.y = r.y + (v.y * sc.y + bi.y);
+        v.z = r.z + (v.z * sc.z + bi.z); v.w = r.w + (v.w * sc.w + bi.w);
+        y4[c4] = v;
+        x[i] = v;
+        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    float rs = 1.0f;
+    if (p.nextGain) rs = 1.0f / sqrtf(block_sum256(ss, red) / (float)N + p.nextEps);
+#pragma unroll
+    for (int i = 0; i < MAXV; i++) {
+        const int c4 = threadIdx.x + i * PWG;
+        if (c4 * 4 >= N) continue;
+        float a[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
+        if (p.nextGain) {
+            const float4 g = reinterpret_cast<const float4*>(p.nextGain)[c4];
+            a[0] = a[0] * rs * g.x; a[1] = a[1] * rs * g.y; a[2] = a[2] * rs * g.z; a[3] = a[3] * rs * g.w;
+        }
+        unsigned short h[4], l[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            h[e] = f32_to_bf16_rne(a[e]);
+            l[e] = f32_to_bf16_rne(a[e] - bf16_to_f32(h[e]));
+        }
+        const size_t o = tiled_index(m, c4 * 4, N);      // four consecutive k stay inside one 64-k block
+        *reinterpret_cast<uint2*>(p.nextHi + o) = make_uint2((unsigned)h[0] | ((unsigned)h[1] << 16), (unsigned)h[2] | ((unsigned)h[3] << 16));
+        *reinterpret_cast<uint2*>(p.nextLo + o) = make_uint2((unsigned)l[0] | ((unsigned)l[1] << 16), (unsigned)l[2] | ((unsigned)l[3] << 16));
+    }
+}
+
+// Sums the splits (and, where the caller asked for it and the shape allows, writes the next split).
+static void launch_reduce(GemmParams& p, int BN, int residual, hipStream_t s) {
+    const int N = p.seg[0].N;
+    if (p.nseg == 1 && residual && p.nextHi && p.nextLo && N % 4 == 0 && N <= 16 * 4 * PWG) {
+        hipLaunchKernelGGL(gemm_reduce_norm_split_kernel, dim3((unsigned)p.T), dim3(PWG), 0, s, p);
+        p.wroteNext = 1;
+        return;
+    }
+    hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((p.ldPartial + PWG - 1) / PWG), (unsigned)p.T), dim3(PWG), 0, s, p, BN,
+                       residual);
+}
+
 size_t gemm_partial_floats() { return (size_t)320 * 256 * 256; }
 
 template <int Q4>
@@ -775,8 +852,7 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
                     hipError_t e = launch_ring<2>(p, grid, s);
                     if (e != hipSuccess) return e;
                 }
-                hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((p.ldPartial + PWG - 1) / PWG), (unsigned)p.T), dim3(PWG),
-                                   0, s, p, 256, residual);
+                launch_reduce(p, 256, residual, s);
             } else if (!Q4) {
                 return residual ? launch_ring<1>(p, grid, s) : launch_ring<0>(p, grid, s);
             } else if (residual) {
@@ -806,8 +882,7 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
         grid.y = (unsigned)S;
         p.splitK = S; p.ldPartial = tiles * 128;
         hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 2>), grid, dim3(PWG), 0, s, p);
-        hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((p.ldPartial + PWG - 1) / PWG), (unsigned)p.T), dim3(PWG), 0, s,
-                           p, 128, residual);
+        launch_reduce(p, 128, residual, s);
     } else if (residual) {
         hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 1>), grid, dim3(PWG), 0, s, p);
     } else {
@@ -820,6 +895,7 @@ hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s) {
     if (p.T <= 0 || p.nseg < 1 || p.nseg > 3) return p.T <= 0 ? hipSuccess : hipErrorInvalidValue;
     if (p.K <= 0 || p.K % 32 != 0) return hipErrorInvalidValue;
     for (int i = 0; i < p.nseg; i++) if (p.seg[i].N <= 0) return hipErrorInvalidValue;
+    p.wroteNext = 0;
     return p.q4 ? launch_gemm_fmt<1>(p, residual, s) : launch_gemm_fmt<0>(p, residual, s);
 }
 
