@@ -120,7 +120,7 @@ private:
     Slab scratch, headSlab, prefillSlab;
     int prefillCap = 0;             // rows the prefill buffers hold
     int* pfTokens = nullptr;
-    float *pfX = nullptr, *pfQ = nullptr, *pfK = nullptr, *pfV = nullptr, *pfAttn = nullptr, *pfGate = nullptr, *pfUp = nullptr;
+    float *pfX = nullptr, *pfQ = nullptr, *pfK = nullptr, *pfV = nullptr, *pfGate = nullptr, *pfUp = nullptr;
     void *pfHi = nullptr, *pfLo = nullptr;
     float* pfPartial = nullptr;
     int ensurePrefill(int rows);

@@ -919,14 +919,13 @@ int HIPFusedInference::ensurePrefill(int rows) {
     prefillCap = 0;
     const size_t T = ((size_t)rows + 127) / 128 * 128;
     const size_t plane = split_plane_elems((int)T, ffnDim > dim ? ffnDim : dim) * 2;
-    size_t bytes = alignUp256(T * 4) + 3 * alignUp256(T * dim * 4) + 2 * alignUp256(T * kvDim * 4) +
+    size_t bytes = alignUp256(T * 4) + 2 * alignUp256(T * dim * 4) + 2 * alignUp256(T * kvDim * 4) +
                    2 * alignUp256(T * ffnDim * 4) + 2 * alignUp256(plane) + alignUp256(gemm_partial_floats() * 4) + 16 * 256;
     int rc = prefillSlab.init(bytes);
     if (rc) return rc;
     pfTokens = static_cast<int*>(prefillSlab.take(T * 4));
     pfX = static_cast<float*>(prefillSlab.take(T * dim * 4));
     pfQ = static_cast<float*>(prefillSlab.take(T * dim * 4));
-    pfAttn = static_cast<float*>(prefillSlab.take(T * dim * 4));
     pfK = static_cast<float*>(prefillSlab.take(T * kvDim * 4));
     pfV = static_cast<float*>(prefillSlab.take(T * kvDim * 4));
     pfGate = static_cast<float*>(prefillSlab.take(T * ffnDim * 4));
@@ -934,7 +933,7 @@ int HIPFusedInference::ensurePrefill(int rows) {
     pfHi = prefillSlab.take(plane);
     pfLo = prefillSlab.take(plane);
     pfPartial = static_cast<float*>(prefillSlab.take(gemm_partial_floats() * 4));
-    if (!pfTokens || !pfX || !pfQ || !pfAttn || !pfK || !pfV || !pfGate || !pfUp || !pfHi || !pfLo || !pfPartial) {
+    if (!pfTokens || !pfX || !pfQ || !pfK || !pfV || !pfGate || !pfUp || !pfHi || !pfLo || !pfPartial) {
         set_error("prefill slab too small");
         return MG_E_STATE;
     }
@@ -981,8 +980,9 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
         g.seg[0] = seg(L.wq, L.bq, pfQ); g.seg[1] = seg(L.wk, L.bk, pfK); g.seg[2] = seg(L.wv, L.bv, pfV);
         HIPCHK(launch_gemm_q8(g, 0, stream));
         HIPCHK(launch_rope_store_rows(pfQ, pfK, pfV, kCache[l], vCache[l], kvHalf, cosTab, sinTab, pos0, T, dim, kvDim, headDim, stream));
-        HIPCHK(launch_prefill_attention(pfQ, kCache[l], vCache[l], kvHalf, pfAttn, T, pos0, maxSeq, dim, kvDim, nHeads, nKVHeads, headDim, stream));
-        HIPCHK(launch_split_rows(pfAttn, nullptr, eps, T, dim, pfHi, pfLo, stream));
+        // the attention writes its rows as the hi/lo split the output projection reads
+        HIPCHK(launch_prefill_attention(pfQ, kCache[l], vCache[l], kvHalf, nullptr, pfHi, pfLo, T, pos0, maxSeq, dim, kvDim, nHeads,
+                                        nKVHeads, headDim, stream));
         g.K = dim; g.nseg = 1; g.q4 = L.wo.kind == WF_Q4P; g.seg[0] = seg(L.wo, nullptr, pfX);
         // where K is split, the kernel that sums the splits also writes norm2's split of the new rows
         g.nextGain = L.norm2; g.nextEps = eps;

@@ -174,7 +174,8 @@ hipError_t launch_embed_rows(int kind, const void* table, const float* scales, c
 // rows register s holds in the two lane halves.)
 // ---------------------------------------------------------------------------
 template <int HD, typename KVT>
-__global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const KVT* Kc, const KVT* Vc, float* out, int T,
+__global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const KVT* Kc, const KVT* Vc, float* out,
+                                                          unsigned short* hi, unsigned short* lo, int T,
                                                           int pos0, int dim, int kvDim, int nHeads, int nKVHeads) {
     constexpr int KS = HD + 4;                 // LDS row stride of the K tile (floats)
     constexpr int DB = HD / 32;                // 32-wide blocks of the head dimension
@@ -279,24 +280,35 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const
             num = fmaf(wgt, lds[w][d * 33 + qq], num);
             den = fmaf(wgt, wl[w][qq], den);
         }
-        out[(size_t)(q0 + qq) * dim + (size_t)head * HD + d] = num / den;
+        const float v = num / den;
+        if (out) out[(size_t)(q0 + qq) * dim + (size_t)head * HD + d] = v;
+        if (hi) {            // the output projection's hi/lo split, written here instead of by a pass of its own
+            const unsigned short h = f32_to_bf16_rne(v);
+            const size_t o2 = tiled_index(q0 + qq, head * HD + d, dim);
+            hi[o2] = h;
+            lo[o2] = f32_to_bf16_rne(v - bf16_to_f32(h));
+        }
     }
 }
 
-hipError_t launch_prefill_attention(const float* q, const void* Kc, const void* Vc, int kvHalf, float* out, int T, int pos0,
-                                    int rowLimit, int dim, int kvDim, int nHeads, int nKVHeads, int headDim, hipStream_t s) {
+hipError_t launch_prefill_attention(const float* q, const void* Kc, const void* Vc, int kvHalf, float* out, void* splitHi,
+                                    void* splitLo, int T, int pos0, int rowLimit, int dim, int kvDim, int nHeads, int nKVHeads,
+                                    int headDim, hipStream_t s) {
     if (T <= 0) return hipSuccess;
+    if ((!out && !splitHi) || (splitHi == nullptr) != (splitLo == nullptr)) return hipErrorInvalidValue;
+    unsigned short* hi = static_cast<unsigned short*>(splitHi);
+    unsigned short* lo = static_cast<unsigned short*>(splitLo);
     if (nKVHeads <= 0 || nHeads % nKVHeads != 0 || pos0 < 0 || pos0 + T > rowLimit || dim != nHeads * headDim ||
         kvDim != nKVHeads * headDim || (headDim != 64 && headDim != 128)) return hipErrorInvalidValue;
     dim3 grid((unsigned)((T + 31) / 32), (unsigned)nHeads);
     const float* kf = static_cast<const float*>(Kc); const float* vf = static_cast<const float*>(Vc);
     const _Float16* kh = static_cast<const _Float16*>(Kc); const _Float16* vh = static_cast<const _Float16*>(Vc);
     if (headDim == 64) {
-        if (kvHalf) hipLaunchKernelGGL((prefill_attn_kernel<64, _Float16>), grid, dim3(256), 0, s, q, kh, vh, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
-        else hipLaunchKernelGGL((prefill_attn_kernel<64, float>), grid, dim3(256), 0, s, q, kf, vf, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
+        if (kvHalf) hipLaunchKernelGGL((prefill_attn_kernel<64, _Float16>), grid, dim3(256), 0, s, q, kh, vh, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
+        else hipLaunchKernelGGL((prefill_attn_kernel<64, float>), grid, dim3(256), 0, s, q, kf, vf, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
     } else {
-        if (kvHalf) hipLaunchKernelGGL((prefill_attn_kernel<128, _Float16>), grid, dim3(256), 0, s, q, kh, vh, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
-        else hipLaunchKernelGGL((prefill_attn_kernel<128, float>), grid, dim3(256), 0, s, q, kf, vf, out, T, pos0, dim, kvDim, nHeads, nKVHeads);
+        if (kvHalf) hipLaunchKernelGGL((prefill_attn_kernel<128, _Float16>), grid, dim3(256), 0, s, q, kh, vh, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
+        else hipLaunchKernelGGL((prefill_attn_kernel<128, float>), grid, dim3(256), 0, s, q, kf, vf, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
     }
     return hipGetLastError();
 }
