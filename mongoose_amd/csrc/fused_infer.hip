@@ -978,8 +978,13 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
         if (!normSplitDone) HIPCHK(launch_split_rows(pfX, L.norm1, eps, T, dim, pfHi, pfLo, stream));
         g.K = dim; g.nseg = 3; g.q4 = L.wq.kind == WF_Q4P;
         g.seg[0] = seg(L.wq, L.bq, pfQ); g.seg[1] = seg(L.wk, L.bk, pfK); g.seg[2] = seg(L.wv, L.bv, pfV);
+        // where K is split, the kernel that sums the splits also rotates q/k and stores the K/V rows
+        g.ropeKc = kCache[l]; g.ropeVc = vCache[l]; g.ropeCos = cosTab; g.ropeSin = sinTab;
+        g.ropePos0 = pos0; g.ropeHeadDim = headDim; g.ropeKvHalf = kvHalf;
         HIPCHK(launch_gemm_q8(g, 0, stream));
-        HIPCHK(launch_rope_store_rows(pfQ, pfK, pfV, kCache[l], vCache[l], kvHalf, cosTab, sinTab, pos0, T, dim, kvDim, headDim, stream));
+        if (!g.wroteRope)
+            HIPCHK(launch_rope_store_rows(pfQ, pfK, pfV, kCache[l], vCache[l], kvHalf, cosTab, sinTab, pos0, T, dim, kvDim, headDim, stream));
+        g.ropeKc = nullptr; g.ropeVc = nullptr;
         // the attention writes its rows as the hi/lo split the output projection reads
         HIPCHK(launch_prefill_attention(pfQ, kCache[l], vCache[l], kvHalf, nullptr, pfHi, pfLo, T, pos0, maxSeq, dim, kvDim, nHeads,
                                         nKVHeads, headDim, stream));

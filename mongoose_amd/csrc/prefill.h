@@ -43,9 +43,19 @@ struct GemmParams {
     float nextEps;
     unsigned short* nextHi;
     unsigned short* nextLo;
+    // Optional (q | k | v in one launch, plain form): when K was split, the kernel that sums the splits
+    // also applies RoPE to the q and k rows and stores the k / v rows into the caches at pos0 + row
+    // (what launch_rope_store_rows does); seg[0].Y still receives the rotated q rows, seg[1].Y / seg[2].Y
+    // are not written then.
+    void* ropeKc;
+    void* ropeVc;
+    const float* ropeCos;
+    const float* ropeSin;
+    int ropePos0, ropeHeadDim, ropeKvHalf;
     // filled by the launcher
     int nTiles, splitK, stepsPerSplit, ldPartial;
     int wroteNext;    // 1: nextHi/nextLo were written; 0: the caller still has to split Y's rows itself
+    int wroteRope;    // 1: q rows rotated and K/V rows stored; 0: the caller still has to call launch_rope_store_rows
 };
 size_t gemm_partial_floats();
 hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s);

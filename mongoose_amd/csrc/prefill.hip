@@ -810,13 +810,79 @@ __global__ __launch_bounds__(PWG) void gemm_reduce_norm_split_kernel(GemmParams 
     }
 }
 
-// Sums the splits (and, where the caller asked for it and the shape allows, writes the next split).
+// q | k | v: the row's sums go to LDS (scale and bias applied), then RoPE on q and k
+// (mongoose.cu:991-1006) and the K/V rows into the caches (mongoose.cu:1644-1647), as
+// rope_store_rows_kernel does them.  One workgroup per row; dynamic LDS = (dim + 2*kvDim) floats.
+template <typename KVT>
+__global__ __launch_bounds__(PWG) void gemm_reduce_qkv_rope_kernel(GemmParams p, int BN) {
+    extern __shared__ float row[];
+    const int m = blockIdx.x;
+    const int dim = p.seg[0].N, kvDim = p.seg[1].N;
+    const size_t plane = (size_t)p.T * p.ldPartial / 4;
+    const float4* src = reinterpret_cast<const float4*>(p.partial + (size_t)m * p.ldPartial);
+    for (int c4 = threadIdx.x; c4 * 4 < p.ldPartial; c4 += PWG) {
+        const int tile = c4 * 4 / BN;
+        int sgi = 0;
+        if (tile >= p.seg[1].tile0) sgi = 1;
+        if (tile >= p.seg[2].tile0) sgi = 2;
+        GemmSeg sg = p.seg[0];
+        if (sgi == 1) sg = p.seg[1];
+        if (sgi == 2) sg = p.seg[2];
+        const int n = c4 * 4 - sg.tile0 * BN;
+        if (n >= sg.N) continue;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int s = 0; s < p.splitK; s++) {
+            const float4 a = src[(size_t)s * plane + c4];
+            v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
+        }
+        float4 sc = make_float4(1.f, 1.f, 1.f, 1.f), bi = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (sg.scales) sc = *reinterpret_cast<const float4*>(sg.scales + n);
+        if (sg.bias) bi = *reinterpret_cast<const float4*>(sg.bias + n);
+        v.x = v.x * sc.x + bi.x; v.y = v.y * sc.y + bi.y; v.z = v.z * sc.z + bi.z; v.w = v.w * sc.w + bi.w;
+        const int base = sgi == 0 ? 0 : (sgi == 1 ? dim : dim + kvDim);
+        *reinterpret_cast<float4*>(&row[base + n]) = v;
+    }
+    __syncthreads();
+    const int headDim = p.ropeHeadDim, half = headDim / 2, pos = p.ropePos0 + m;
+    const float* c = p.ropeCos + (size_t)pos * half;
+    const float* s = p.ropeSin + (size_t)pos * half;
+    float* qr = p.seg[0].Y + (size_t)m * dim;
+    for (int i = threadIdx.x; i < dim / 2; i += PWG) {
+        const int h = i / half, j = i % half;
+        const float x0 = row[h * headDim + j], x1 = row[h * headDim + half + j];
+        qr[h * headDim + j] = x0 * c[j] - x1 * s[j];
+        qr[h * headDim + half + j] = x0 * s[j] + x1 * c[j];
+    }
+    KVT* kd = static_cast<KVT*>(p.ropeKc) + (size_t)pos * kvDim;
+    KVT* vd = static_cast<KVT*>(p.ropeVc) + (size_t)pos * kvDim;
+    const float* kr = row + dim;
+    const float* vr = row + dim + kvDim;
+    for (int i = threadIdx.x; i < kvDim / 2; i += PWG) {
+        const int h = i / half, j = i % half;
+        const float x0 = kr[h * headDim + j], x1 = kr[h * headDim + half + j];
+        kd[h * headDim + j] = (KVT)(x0 * c[j] - x1 * s[j]);
+        kd[h * headDim + half + j] = (KVT)(x0 * s[j] + x1 * c[j]);
+    }
+    for (int i = threadIdx.x; i < kvDim; i += PWG) vd[i] = (KVT)vr[i];
+}
+
+// Sums the splits (and, where the caller asked for it and the shape allows, does the row-wise step that follows).
 static void launch_reduce(GemmParams& p, int BN, int residual, hipStream_t s) {
     const int N = p.seg[0].N;
     if (p.nseg == 1 && residual && p.nextHi && p.nextLo && N % 4 == 0 && N <= 16 * 4 * PWG) {
         hipLaunchKernelGGL(gemm_reduce_norm_split_kernel, dim3((unsigned)p.T), dim3(PWG), 0, s, p);
         p.wroteNext = 1;
         return;
+    }
+    if (p.nseg == 3 && !residual && p.ropeKc && p.ropeVc && p.seg[1].N == p.seg[2].N && p.seg[0].N % 4 == 0 &&
+        p.seg[1].N % 4 == 0 && p.ropeHeadDim > 0 && p.seg[0].N % p.ropeHeadDim == 0 && p.seg[1].N % p.ropeHeadDim == 0) {
+        const size_t lds = (size_t)(p.seg[0].N + 2 * p.seg[1].N) * sizeof(float);
+        if (lds <= 48 * 1024) {
+            if (p.ropeKvHalf) hipLaunchKernelGGL(gemm_reduce_qkv_rope_kernel<_Float16>, dim3((unsigned)p.T), dim3(PWG), lds, s, p, BN);
+            else hipLaunchKernelGGL(gemm_reduce_qkv_rope_kernel<float>, dim3((unsigned)p.T), dim3(PWG), lds, s, p, BN);
+            p.wroteRope = 1;
+            return;
+        }
     }
     hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((p.ldPartial + PWG - 1) / PWG), (unsigned)p.T), dim3(PWG), 0, s, p, BN,
                        residual);
@@ -908,6 +974,7 @@ hipError_t launch_gemm_q8(GemmParams& p, int residual, hipStream_t s) {
     if (p.K <= 0 || p.K % 32 != 0) return hipErrorInvalidValue;
     for (int i = 0; i < p.nseg; i++) if (p.seg[i].N <= 0) return hipErrorInvalidValue;
     p.wroteNext = 0;
+    p.wroteRope = 0;
     return p.q4 ? launch_gemm_fmt<1>(p, residual, s) : launch_gemm_fmt<0>(p, residual, s);
 }
 
