@@ -121,7 +121,7 @@ private:
     int prefillCap = 0;             // rows the prefill buffers hold
     int* pfTokens = nullptr;
     float *pfX = nullptr, *pfQ = nullptr, *pfK = nullptr, *pfV = nullptr, *pfGate = nullptr, *pfUp = nullptr;
-    void *pfHi = nullptr, *pfLo = nullptr;
+    void *pfHi = nullptr, *pfLo = nullptr, *pfHi2 = nullptr, *pfLo2 = nullptr;
     float* pfPartial = nullptr;
     int ensurePrefill(int rows);
     std::vector<Slab> layerSlabs, kvSlabs;

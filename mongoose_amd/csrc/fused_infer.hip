@@ -920,7 +920,7 @@ int HIPFusedInference::ensurePrefill(int rows) {
     const size_t T = ((size_t)rows + 127) / 128 * 128;
     const size_t plane = split_plane_elems((int)T, ffnDim > dim ? ffnDim : dim) * 2;
     size_t bytes = alignUp256(T * 4) + 2 * alignUp256(T * dim * 4) + 2 * alignUp256(T * kvDim * 4) +
-                   2 * alignUp256(T * ffnDim * 4) + 2 * alignUp256(plane) + alignUp256(gemm_partial_floats() * 4) + 16 * 256;
+                   2 * alignUp256(T * ffnDim * 4) + 4 * alignUp256(plane) + alignUp256(gemm_partial_floats() * 4) + 16 * 256;
     int rc = prefillSlab.init(bytes);
     if (rc) return rc;
     pfTokens = static_cast<int*>(prefillSlab.take(T * 4));
@@ -932,8 +932,10 @@ int HIPFusedInference::ensurePrefill(int rows) {
     pfUp = static_cast<float*>(prefillSlab.take(T * ffnDim * 4));
     pfHi = prefillSlab.take(plane);
     pfLo = prefillSlab.take(plane);
+    pfHi2 = prefillSlab.take(plane);      // second pair: written by the gate|up GEMM's own epilogue while it still reads the first
+    pfLo2 = prefillSlab.take(plane);
     pfPartial = static_cast<float*>(prefillSlab.take(gemm_partial_floats() * 4));
-    if (!pfTokens || !pfX || !pfQ || !pfK || !pfV || !pfGate || !pfUp || !pfHi || !pfLo || !pfPartial) {
+    if (!pfTokens || !pfX || !pfQ || !pfK || !pfV || !pfGate || !pfUp || !pfHi || !pfLo || !pfHi2 || !pfLo2 || !pfPartial) {
         set_error("prefill slab too small");
         return MG_E_STATE;
     }
@@ -996,8 +998,13 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
         if (!g.wroteNext) HIPCHK(launch_split_rows(pfX, L.norm2, eps, T, dim, pfHi, pfLo, stream));
         g.nextGain = nullptr; g.nextHi = nullptr; g.nextLo = nullptr;
         g.K = dim; g.nseg = 2; g.q4 = L.gate.kind == WF_Q4P; g.seg[0] = seg(L.gate, nullptr, pfGate); g.seg[1] = seg(L.up, nullptr, pfUp);
+        // silu(gate) * up and its hi/lo split come out of the GEMM's epilogue or of the kernel that sums its K splits
+        // (into the second pair of planes: the GEMM is still reading the first)
+        g.nextSwiglu = 1; g.nextHi = static_cast<unsigned short*>(pfHi2); g.nextLo = static_cast<unsigned short*>(pfLo2);
         HIPCHK(launch_gemm_q8(g, 0, stream));
-        HIPCHK(launch_swiglu_split(pfGate, pfUp, T, ffnDim, pfHi, pfLo, stream));
+        if (!g.wroteNext) HIPCHK(launch_swiglu_split(pfGate, pfUp, T, ffnDim, pfHi2, pfLo2, stream));
+        g.nextSwiglu = 0; g.nextHi = nullptr; g.nextLo = nullptr;
+        g.Ahi = static_cast<const unsigned short*>(pfHi2); g.Alo = static_cast<const unsigned short*>(pfLo2);
         g.K = ffnDim; g.nseg = 1; g.q4 = L.down.kind == WF_Q4P; g.seg[0] = seg(L.down, nullptr, pfX);
         if (l + 1 < nLayers) {                  // ... and here the next layer's norm1 split
             g.nextGain = layers[l + 1].norm1; g.nextEps = eps;
@@ -1005,6 +1012,7 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
         }
         HIPCHK(launch_gemm_q8(g, 1, stream));
         normSplitDone = g.wroteNext != 0;
+        g.Ahi = static_cast<const unsigned short*>(pfHi); g.Alo = static_cast<const unsigned short*>(pfLo);
     }
     // the last position continues on the decode path: final norm, lm_head, greedy token, state -> pos0 + T
     HIPCHK(hipMemcpyAsync(hidden[hiddenIdx], pfX + (size_t)(T - 1) * dim, (size_t)dim * 4, hipMemcpyDeviceToDevice, stream));

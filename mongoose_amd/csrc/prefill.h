@@ -52,6 +52,10 @@ struct GemmParams {
     const float* ropeCos;
     const float* ropeSin;
     int ropePos0, ropeHeadDim, ropeKvHalf;
+    // Optional (gate | up in one launch, plain form): nextSwiglu != 0 asks for silu(gate) * up
+    // (mongoose.cu:949-956) written as the hi/lo split for K = N into nextHi/nextLo (what launch_swiglu_split
+    // does); seg[0].Y / seg[1].Y are not written when the launcher could do that (wroteNext = 1).
+    int nextSwiglu;
     // filled by the launcher
     int nTiles, splitK, stepsPerSplit, ldPartial;
     int wroteNext;    // 1: nextHi/nextLo were written; 0: the caller still has to split Y's rows itself

@@ -599,10 +599,15 @@ __global__ __launch_bounds__(1024) void gemm_q8_ring_kernel(GemmParams p) {
     const int nTile = grp * 8 + (rem & 7), mTile = rem >> 3;
     if (nTile >= p.nTiles) return;
     GemmSeg sg = p.seg[0];
-    if (p.nseg > 1 && nTile >= p.seg[1].tile0) sg = p.seg[1];
-    if (p.nseg > 2 && nTile >= p.seg[2].tile0) sg = p.seg[2];
+    if (MODE != 3) {
+        if (p.nseg > 1 && nTile >= p.seg[1].tile0) sg = p.seg[1];
+        if (p.nseg > 2 && nTile >= p.seg[2].tile0) sg = p.seg[2];
+    }
     const int N = sg.N, K = p.K, T = p.T;
-    const int m0 = mTile * BM, n0 = (nTile - sg.tile0) * BN;
+    // MODE 3 (gate | up -> silu(gate) * up): a tile is 128 columns of the output; its 256 weight rows
+    // alternate in blocks of 32 between the gate and the up matrix, so a wave's two 32-column MFMA
+    // blocks are the gate and the up values of the same 32 columns and the product needs no exchange.
+    const int m0 = mTile * BM, n0 = MODE == 3 ? nTile * 128 : (nTile - sg.tile0) * BN;
     const int ksteps = K / RK;                            // K is a multiple of 32
     const int ks64 = (K + 63) / 64;                       // the split planes are blocked in 64-k steps
     const int stepBeg = MODE == 2 ? blockIdx.y * p.stepsPerSplit * 2 : 0;
@@ -618,6 +623,11 @@ __global__ __launch_bounds__(1024) void gemm_q8_ring_kernel(GemmParams p) {
     const int bRowL = 32 * (wave & 7) + (lane >> 1);
     const int bSeg = (lane & 1) ^ ((bRowL >> 2) & 1);
     const signed char* bG = sg.W + (size_t)min(n0 + bRowL, N - 1) * K + bSeg * 16;
+    if (MODE == 3) {
+        const int blk = wave & 7;                         // this wave's 32 rows: block blk of the tile
+        const int wrow = min(n0 + (blk >> 1) * 32 + (bRowL & 31), N - 1);
+        bG = ((blk & 1) ? p.seg[1].W : p.seg[0].W) + (size_t)wrow * K + bSeg * 16;
+    }
     const bool bWave = wave < 8;
 
     auto issue = [&](int step, int stage) __attribute__((always_inline)) {
@@ -674,6 +684,28 @@ __global__ __launch_bounds__(1024) void gemm_q8_ring_kernel(GemmParams p) {
         stage = stage + 1 == RS ? 0 : stage + 1;
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the trailing reloads must not outlive the workgroup's LDS
+    if (MODE == 3) {
+        const int n = n0 + wn * 32 + (lane & 31);
+        if (n < N) {
+            const float scg = p.seg[0].scales[n], scu = p.seg[1].scales[n];
+            const float big = p.seg[0].bias ? p.seg[0].bias[n] : 0.f, biu = p.seg[1].bias ? p.seg[1].bias[n] : 0.f;
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                    if (m < T) {
+                        const float g = acc[i][0][e] * scg + big, u = acc[i][1][e] * scu + biu;
+                        const float a = g * (1.0f / (1.0f + expf(-g))) * u;        // mongoose.cu:949-956
+                        const unsigned short h = f32_to_bf16_rne(a);
+                        const size_t o = tiled_index(m, n, N);
+                        p.nextHi[o] = h;
+                        p.nextLo[o] = f32_to_bf16_rne(a - bf16_to_f32(h));
+                    }
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const int nl = wn * 64 + j * 32 + (lane & 31);
@@ -866,6 +898,32 @@ __global__ __launch_bounds__(PWG) void gemm_reduce_qkv_rope_kernel(GemmParams p,
     for (int i = threadIdx.x; i < kvDim; i += PWG) vd[i] = (KVT)vr[i];
 }
 
+// gate | up: sums of the splits, scale/bias, silu(gate) * up, hi/lo split.  Grid (columns / 256, rows).
+__global__ __launch_bounds__(PWG) void gemm_reduce_swiglu_split_kernel(GemmParams p, int BN) {
+    const int n = blockIdx.x * PWG + threadIdx.x;
+    const int m = blockIdx.y;
+    const int N = p.seg[0].N;
+    if (n >= N) return;
+    const size_t plane = (size_t)p.T * p.ldPartial;
+    const float* sg_ = p.partial + (size_t)m * p.ldPartial + n;
+    const float* su_ = sg_ + (size_t)p.seg[1].tile0 * BN;
+    float g = 0.f, u = 0.f;
+    int s = 0;
+    for (; s + 2 <= p.splitK; s += 2) {
+        const float g0 = sg_[(size_t)s * plane], g1 = sg_[(size_t)(s + 1) * plane];
+        const float u0 = su_[(size_t)s * plane], u1 = su_[(size_t)(s + 1) * plane];
+        g += g0; g += g1; u += u0; u += u1;
+    }
+    for (; s < p.splitK; s++) { g += sg_[(size_t)s * plane]; u += su_[(size_t)s * plane]; }
+    g = g * (p.seg[0].scales ? p.seg[0].scales[n] : 1.0f) + (p.seg[0].bias ? p.seg[0].bias[n] : 0.f);
+    u = u * (p.seg[1].scales ? p.seg[1].scales[n] : 1.0f) + (p.seg[1].bias ? p.seg[1].bias[n] : 0.f);
+    const float a = g * (1.0f / (1.0f + expf(-g))) * u;
+    const unsigned short h = f32_to_bf16_rne(a);
+    const size_t o = tiled_index(m, n, N);
+    p.nextHi[o] = h;
+    p.nextLo[o] = f32_to_bf16_rne(a - bf16_to_f32(h));
+}
+
 // Sums the splits (and, where the caller asked for it and the shape allows, does the row-wise step that follows).
 static void launch_reduce(GemmParams& p, int BN, int residual, hipStream_t s) {
     const int N = p.seg[0].N;
@@ -883,6 +941,12 @@ static void launch_reduce(GemmParams& p, int BN, int residual, hipStream_t s) {
             p.wroteRope = 1;
             return;
         }
+    }
+    if (p.nseg == 2 && !residual && p.nextSwiglu && p.nextHi && p.nextLo && p.seg[0].N == p.seg[1].N) {
+        hipLaunchKernelGGL(gemm_reduce_swiglu_split_kernel, dim3((unsigned)((p.seg[0].N + PWG - 1) / PWG), (unsigned)p.T), dim3(PWG), 0,
+                           s, p, BN);
+        p.wroteNext = 1;
+        return;
     }
     hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((p.ldPartial + PWG - 1) / PWG), (unsigned)p.T), dim3(PWG), 0, s, p, BN,
                        residual);
@@ -903,6 +967,19 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
     constexpr int BMB = Q4 ? 128 : 256, NTB = Q4 ? 512 : 1024;
     const int ksteps = (p.K + BK - 1) / BK;
     p.splitK = 1; p.stepsPerSplit = ksteps;
+    if (!Q4 && p.T > 128 && p.nseg == 2 && !residual && p.nextSwiglu && p.nextHi && p.nextLo && p.seg[0].N == p.seg[1].N) {
+        // gate | up with enough 128-column tiles to fill the chip without splitting K: the GEMM's own
+        // epilogue forms silu(gate) * up and writes its hi/lo split
+        const int tiles = (p.seg[0].N + 127) / 128;
+        const int numM = (p.T + 255) / 256;
+        if (tiles * numM >= 160) {
+            p.nTiles = tiles;
+            dim3 grid((unsigned)(((tiles + 7) / 8) * 8 * numM), 1);
+            hipError_t e = launch_ring<3>(p, grid, s);
+            if (e == hipSuccess) p.wroteNext = 1;
+            return e;
+        }
+    }
     if (p.T > 128) {
         // K is split until about one workgroup per CU exists (each split keeps >= 8 steps).  Worth it
         // when the tiles alone nearly fill the chip or K can be split; otherwise the small tiles below

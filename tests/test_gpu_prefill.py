@@ -143,6 +143,16 @@ def test_prefill_llama3_shape_one_layer(hip):
     m.close()
 
 
+def test_prefill_llama3_shape_two_row_tiles(hip):
+    """Llama-3-8B layer shape with a 300-token prompt (vocab cut to 8192 so the oracle stays fast): two
+    256-row tiles, which is where the gate|up GEMM has enough tiles to run unsplit and forms
+    silu(gate)*up in its own epilogue, while q|k|v, Wo and down split K and finish in the
+    row-wise kernels (RoPE + cache rows; residual + next norm + split)."""
+    s = H.with_layers(configs.LLAMA3_8B, 1)._replace(vocab=8192)
+    m, _, _ = _prefill_case(hip, s, seed=14, nPrompt=300, nDecode=2, maxSeq=320)
+    m.close()
+
+
 def test_prefill_fp16_kv(hip):
     """Prefill writing fp16 KV rows (head sizes 64 and 128) against the oracle with the same rounding."""
     m, _, _ = _prefill_case(hip, H.with_layers(configs.QWEN, 2), seed=7, nPrompt=70, nDecode=6, maxSeq=96, kv_f16=True)
