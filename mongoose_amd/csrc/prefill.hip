@@ -994,7 +994,9 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
             if (S < 1) S = 1;
             while (S > 1 && (size_t)S * p.T * tiles * 256 > gemm_partial_floats()) S--;
         }
-        if (wgs >= 96 || S >= 2) {
+        // ... and only if that launch then has a workgroup for (nearly) every CU: a down projection of a
+        // small model (N = 896: 8 tiles, 9 splits) is better off on the small tiles, which split K further
+        if ((wgs >= 96 || S >= 2) && wgs * S >= 200) {
             dim3 grid((unsigned)(((tiles + 7) / 8) * 8 * numM), 1);
             if (S > 1) {
                 p.stepsPerSplit = (ksteps + S - 1) / S;
