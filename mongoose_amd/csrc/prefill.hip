@@ -368,13 +368,21 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
     const int nTile = grp * 8 + (rem & 7), mTile = rem >> 3;
     if (nTile >= p.nTiles) return;
     int sgi = 0;
-    if (p.nseg > 1 && nTile >= p.seg[1].tile0) sgi = 1;
-    if (p.nseg > 2 && nTile >= p.seg[2].tile0) sgi = 2;
+    if (MODE != 3) {
+        if (p.nseg > 1 && nTile >= p.seg[1].tile0) sgi = 1;
+        if (p.nseg > 2 && nTile >= p.seg[2].tile0) sgi = 2;
+    }
     GemmSeg sg = p.seg[0];                       // selected by value: indexing the argument array by a
     if (sgi == 1) sg = p.seg[1];                 // run-time index would copy it into scratch memory
     if (sgi == 2) sg = p.seg[2];
     const int N = sg.N, K = p.K, T = p.T;
-    const int m0 = mTile * BM, n0 = (nTile - sg.tile0) * BN;
+    // MODE 3 (gate | up -> silu(gate) * up): a tile is BN/2 columns of the output; its BN weight rows
+    // alternate in blocks of 32 between the gate and the up matrix, so a wave's two 32-column MFMA
+    // blocks are the gate and the up values of the same 32 columns.
+    const int m0 = mTile * BM, n0 = MODE == 3 ? nTile * (BN / 2) : (nTile - sg.tile0) * BN;
+    // weight row (and matrix) behind local row lr of the tile
+    auto wrow = [&](int lr) { return MODE == 3 ? n0 + (lr >> 6) * 32 + (lr & 31) : n0 + lr; };
+    auto wmat = [&](int lr) { return MODE == 3 && ((lr >> 5) & 1) ? p.seg[1].W : sg.W; };
     const int ksteps = (K + BK - 1) / BK;
     const int stepBeg = MODE == 2 ? blockIdx.y * p.stepsPerSplit : 0;
     const int stepEnd = MODE == 2 ? min(ksteps, stepBeg + p.stepsPerSplit) : ksteps;
@@ -395,13 +403,15 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
     const signed char* bP[BR];
 #pragma unroll
     for (int r = 0; r < BR; r++) {
-        const int row = min(n0 + bRow + (NT / WSEG) * r, N - 1);
-        bP[r] = Q4 ? sg.W + ((size_t)row * (K >> 5) + bSeg) * 16 : sg.W + (size_t)row * K + bSeg * 16;
+        const int lr = bRow + (NT / WSEG) * r;
+        const int row = min(wrow(lr), N - 1);
+        const signed char* Wm = wmat(lr);
+        bP[r] = Q4 ? Wm + ((size_t)row * (K >> 5) + bSeg) * 16 : Wm + (size_t)row * K + bSeg * 16;
     }
     // Q4_0: thread t < BN also fetches row t's two block scales of the step
     const unsigned short* dP = nullptr;
     if (Q4 && tid < BN)
-        dP = reinterpret_cast<const unsigned short*>(sg.W + (size_t)N * (K >> 1)) + (size_t)min(n0 + tid, N - 1) * (K >> 5);
+        dP = reinterpret_cast<const unsigned short*>(wmat(tid) + (size_t)N * (K >> 1)) + (size_t)min(wrow(tid), N - 1) * (K >> 5);
 
     float16_t acc[MI][2];
 #pragma unroll
@@ -526,6 +536,28 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
             }
         }
         }
+    }
+    if (MODE == 3) {
+        const int n = n0 + wn * 32 + (lane & 31);
+        if (n < N) {
+            const float scg = Q4 ? 1.0f : p.seg[0].scales[n], scu = Q4 ? 1.0f : p.seg[1].scales[n];
+            const float big = p.seg[0].bias ? p.seg[0].bias[n] : 0.f, biu = p.seg[1].bias ? p.seg[1].bias[n] : 0.f;
+#pragma unroll
+            for (int i = 0; i < MI; i++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int m = m0 + wm * (BM / WM) + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                    if (m < T) {
+                        const float g = acc[i][0][e] * scg + big, u = acc[i][1][e] * scu + biu;
+                        const float a = g * (1.0f / (1.0f + expf(-g))) * u;        // mongoose.cu:949-956
+                        const unsigned short h = f32_to_bf16_rne(a);
+                        const size_t o = tiled_index(m, n, N);
+                        p.nextHi[o] = h;
+                        p.nextLo[o] = f32_to_bf16_rne(a - bf16_to_f32(h));
+                    }
+                }
+        }
+        return;
     }
 #pragma unroll
     for (int j = 0; j < 2; j++) {
@@ -1042,6 +1074,12 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
         launch_reduce(p, 128, residual, s);
     } else if (residual) {
         hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 1>), grid, dim3(PWG), 0, s, p);
+    } else if (p.nseg == 2 && p.nextSwiglu && p.nextHi && p.nextLo && p.seg[0].N == p.seg[1].N) {
+        // gate | up, K not split: silu(gate) * up and its hi/lo split in the GEMM's own epilogue
+        p.nTiles = (p.seg[0].N + 63) / 64;
+        dim3 g3((unsigned)(((p.nTiles + 7) / 8) * 8 * numM), 1);
+        hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 3>), g3, dim3(PWG), 0, s, p);
+        p.wroteNext = 1;
     } else {
         hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 64, 128, 256, 0>), grid, dim3(PWG), 0, s, p);
     }
