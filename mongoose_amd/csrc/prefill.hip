@@ -1052,6 +1052,29 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
             return hipGetLastError();
         }
     }
+    if constexpr (Q4 != 0) {
+        // Q4_0 in between: the 128 x 256 tiles, K not split, where they give at least a workgroup for
+        // every other CU (gate | up of a small model): half the L2-to-CU bytes per flop of the small tile.
+        // (For Q8 the small tiles measured faster at this size.)
+        if (p.T > 128) {
+            const bool swiglu = p.nseg == 2 && !residual && p.nextSwiglu && p.nextHi && p.nextLo && p.seg[0].N == p.seg[1].N;
+            const int tilesM = swiglu ? (p.seg[0].N + 127) / 128 : count(256);
+            const int numM = (p.T + 127) / 128;
+            if (tilesM * numM >= 128) {
+                p.nTiles = tilesM;
+                dim3 grid((unsigned)(((tilesM + 7) / 8) * 8 * numM), 1);
+                if (swiglu) {
+                    hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 128, 256, 512, 3>), grid, dim3(512), 0, s, p);
+                    p.wroteNext = 1;
+                } else if (residual) {
+                    hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 128, 256, 512, 1>), grid, dim3(512), 0, s, p);
+                } else {
+                    hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, 128, 256, 512, 0>), grid, dim3(512), 0, s, p);
+                }
+                return hipGetLastError();
+            }
+        }
+    }
     const int tiles = count(128);
     const int numM = (p.T + 63) / 64;
     dim3 grid((unsigned)(((tiles + 7) / 8) * 8 * numM), 1);
