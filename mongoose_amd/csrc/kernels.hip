@@ -282,7 +282,7 @@ __device__ __forceinline__ RowRef resolve_row(const MvParams& p, int g, int i) {
     return r;
 }
 
-template <int WF, int NR, int KS, int PRO, int EPI>
+template <int WF, int NR, int KS, int PRO, int EPI, bool EARLY = false>
 __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     using F = Fmt<WF>;
     constexpr int LPG = KS == 1 ? 64 : WG;           // lanes per group
@@ -348,7 +348,30 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
         }
     };
 
-    // first loads go out before the activation vector is staged
+    // Vectors of 1025..4096 elements (two to four float4 per thread): all of a thread's pieces of the
+    // vector (and of the norm gain) are requested in one batch, ahead of the first weights, and held in
+    // registers -- one memory round trip; the load-then-store loop of stage_activation pays one per
+    // piece.  (A single piece gains nothing from this and costs registers: measured slower at K = 896.)
+    constexpr int SB = 4;                             // float4 per thread held across the weight issue
+    const int K4 = p.K >> 2;
+    constexpr bool early = EARLY;                     // chosen by the launcher: KS == 1 and WG < K/4 <= SB*WG
+    float4 sx[SB], sgn[SB];
+    if (early) {
+        const float4* x4 = reinterpret_cast<const float4*>(p.act);
+        const float4* g4 = reinterpret_cast<const float4*>(p.gain);
+#pragma unroll
+        for (int u = 0; u < SB; u++) {
+            sx[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            sgn[u] = sx[u];
+            if (u * WG < K4) {                                        // uniform: whole rounds past the end issue nothing
+                const int i = min((int)threadIdx.x + u * WG, K4 - 1);
+                sx[u] = x4[i];
+                if (PRO == PRO_RMS) sgn[u] = g4[i];
+            }
+        }
+    }
+
+    // first weight loads go out before the activation vector is staged
 #pragma unroll
     for (int s = 0; s < D; s++) issue(s, s);
 
@@ -376,6 +399,27 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
                 avr[it][2] = x4[base + 4]; avr[it][3] = x4[base + 5];
             }
         }
+    } else if (early) {
+        // stage_activation's arithmetic on the registers loaded above
+        float ss = 0.f;
+#pragma unroll
+        for (int u = 0; u < SB; u++) {
+            const int i = threadIdx.x + u * WG;
+            if (i < K4) {
+                float4 v = sx[u];
+                if (PRO == PRO_RMS) {
+                    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                    v.x *= sgn[u].x; v.y *= sgn[u].y; v.z *= sgn[u].z; v.w *= sgn[u].w;
+                }
+                a4[act_slot4<WF>(i, nch)] = v;
+            }
+        }
+        if (PRO == PRO_RMS) {
+            ss = wave_sum(ss);
+            if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+        }
+        __syncthreads();
+        if (PRO == PRO_RMS) rs = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)p.K + p.eps);
     } else {
         rs = stage_activation<WF, PRO>(p, a4, red);
     }
@@ -742,6 +786,14 @@ MvConfig pick_config(int wf, int epi, int totalRows, int K) {
 template <int WF, int NR, int KS, int PRO, int EPI>
 static hipError_t launch_t(MvParams& p, int grid, hipStream_t s) {
     size_t lds = (size_t)p.K * sizeof(float);
+    const int K4 = p.K >> 2;
+    // only for the launch shapes the decode step itself picks: NR 2, fused epilogues
+    if constexpr (KS == 1 && NR == 2 && WF != WF_Q4RAW && (EPI == EPI_QKV || EPI == EPI_SWIGLU || EPI == EPI_RESID)) {
+        if (K4 > WG && K4 <= 4 * WG) {                // a variant of its own: the batch costs registers the short vectors need not pay
+            hipLaunchKernelGGL((matvec_kernel<WF, NR, KS, PRO, EPI, true>), dim3(grid), dim3(WG), lds, s, p);
+            return hipGetLastError();
+        }
+    }
     hipLaunchKernelGGL((matvec_kernel<WF, NR, KS, PRO, EPI>), dim3(grid), dim3(WG), lds, s, p);
     return hipGetLastError();
 }
