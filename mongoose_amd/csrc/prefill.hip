@@ -895,7 +895,16 @@ __global__ __launch_bounds__(PWG) void gemm_reduce_qkv_rope_kernel(GemmParams p,
         const int n = c4 * 4 - sg.tile0 * BN;
         if (n >= sg.N) continue;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int s = 0; s < p.splitK; s++) {
+        int s = 0;
+        for (; s + 4 <= p.splitK; s += 4) {             // four loads in flight, added in split order
+            const float4 a = src[(size_t)s * plane + c4], b = src[(size_t)(s + 1) * plane + c4];
+            const float4 c = src[(size_t)(s + 2) * plane + c4], d = src[(size_t)(s + 3) * plane + c4];
+            v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
+            v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+            v.x += c.x; v.y += c.y; v.z += c.z; v.w += c.w;
+            v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+        }
+        for (; s < p.splitK; s++) {
             const float4 a = src[(size_t)s * plane + c4];
             v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
         }
