@@ -1044,21 +1044,22 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
                 S = (ksteps + p.stepsPerSplit - 1) / p.stepsPerSplit;
                 grid.y = (unsigned)S;
                 p.splitK = S; p.ldPartial = tiles * 256;
-                if (Q4) {
+                if constexpr (Q4 != 0) {
                     hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 2>), grid, dim3(NTB), 0, s, p);
                 } else {
                     hipError_t e = launch_ring<2>(p, grid, s);
                     if (e != hipSuccess) return e;
                 }
                 launch_reduce(p, 256, residual, s);
-            } else if (!Q4) {
-                return residual ? launch_ring<1>(p, grid, s) : launch_ring<0>(p, grid, s);
-            } else if (residual) {
-                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 1>), grid, dim3(NTB), 0, s, p);
-            } else {
-                hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 0>), grid, dim3(NTB), 0, s, p);
+                return hipGetLastError();
             }
-            return hipGetLastError();
+            if constexpr (Q4 != 0) {
+                if (residual) hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 1>), grid, dim3(NTB), 0, s, p);
+                else hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 0>), grid, dim3(NTB), 0, s, p);
+                return hipGetLastError();
+            } else {
+                return residual ? launch_ring<1>(p, grid, s) : launch_ring<0>(p, grid, s);
+            }
         }
     }
     if constexpr (Q4 != 0) {
