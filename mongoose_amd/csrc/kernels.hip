@@ -972,16 +972,17 @@ __device__ __forceinline__ float4 ld_kv4(const void* base, size_t idx4) {
     return make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
 }
 
-template <int HD, int GMAX, bool KVH>
-__global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
+template <int HD, int GMAX, bool KVH, int AWG = WG>
+__global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
+    constexpr int NWV = AWG / 64;      // waves: 4, or more for the one-head workgroups of short contexts (fewer rows per thread)
     constexpr int LPR = 16;            // lanes per K/V row: one DPP row
     constexpr int NF = HD / 64;        // float4s of a row per lane (float4 index j*16 + dl)
-    constexpr int TG = WG / LPR;       // rows in flight per load step (16)
-    constexpr int VU = 16 / NF;        // rows per thread and tile
+    constexpr int TG = AWG / LPR;      // rows in flight per load step (16 or 32)
+    constexpr int VU = 16 / NF / (AWG / WG);   // rows per thread and tile
     constexpr int TILE = TG * VU;      // positions per tile (256 for head size 64, 128 for 128)
-    __shared__ float wred[2][GMAX][4];
-    __shared__ float4 accbuf[4][GMAX][HD / 4];
-    __shared__ float lbuf[4][GMAX];
+    __shared__ float wred[2][GMAX][NWV];
+    __shared__ float4 accbuf[NWV][GMAX][HD / 4];
+    __shared__ float lbuf[NWV][GMAX];
     __shared__ int lastFlag;
 
     const int tid = threadIdx.x;
@@ -1074,7 +1075,10 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
         __syncthreads();
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
-            const float tm = fmaxf(fmaxf(wred[par][g][0], wred[par][g][1]), fmaxf(wred[par][g][2], wred[par][g][3]));
+            float tm = fmaxf(fmaxf(wred[par][g][0], wred[par][g][1]), fmaxf(wred[par][g][2], wred[par][g][3]));
+#pragma unroll
+            for (int w = 4; w < NWV; w += 4)
+                tm = fmaxf(tm, fmaxf(fmaxf(wred[par][g][w], wred[par][g][w + 1]), fmaxf(wred[par][g][w + 2], wred[par][g][w + 3])));
             const float mNew = fmaxf(m[g], tm);            // finite: every tile holds at least one valid position
             const float corr = expf(m[g] - mNew);          // first tile: exp(-inf) = 0
             m[g] = mNew;
@@ -1113,16 +1117,18 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     }
     __syncthreads();
     constexpr int F4 = HD / 4;                             // float4s of a head
-    for (int i = tid; i < gn * F4; i += WG) {
+    for (int i = tid; i < gn * F4; i += AWG) {
         int g = i / F4, d4 = i % F4;
         float4 r = accbuf[0][g][d4];
 #pragma unroll
-        for (int k = 1; k < 4; k++) {
+        for (int k = 1; k < NWV; k++) {
             float4 a = accbuf[k][g][d4];
             r.x += a.x; r.y += a.y; r.z += a.z; r.w += a.w;
         }
         // lbuf holds lane 0's column of each wave: every row's probability exactly once
-        const float lg = (lbuf[0][g] + lbuf[1][g]) + (lbuf[2][g] + lbuf[3][g]);
+        float lg = (lbuf[0][g] + lbuf[1][g]) + (lbuf[2][g] + lbuf[3][g]);
+#pragma unroll
+        for (int w = 4; w < NWV; w += 4) lg += (lbuf[w][g] + lbuf[w + 1][g]) + (lbuf[w + 2][g] + lbuf[w + 3][g]);
         float mg_ = m[0];
 #pragma unroll
         for (int k = 1; k < GMAX; k++) if (g == k) mg_ = m[k];
@@ -1160,9 +1166,9 @@ __global__ __launch_bounds__(WG) void attn_decode_kernel(AttnParams p) {
     // is used, one memory round trip a batch, and up to 16*NG splits need only one -- and the NG results
     // of an item are folded through LDS with the same running-maximum rescale.
     constexpr int IT = GMAX * F4;
-    constexpr int NG = WG / IT;
-    __shared__ float4 cnum[WG];
-    __shared__ float cM[WG], cden[WG];
+    constexpr int NG = AWG / IT;
+    __shared__ float4 cnum[AWG];
+    __shared__ float cM[AWG], cden[AWG];
     {
         const int q = tid / IT, i = tid % IT;
         const int g = i / F4, d4 = i % F4;
@@ -1236,7 +1242,7 @@ static hipError_t launch_attn_hd(const AttnParams& p, hipStream_t s) {
     int nChunks = (G + gmax - 1) / gmax;
     dim3 grid(p.nKVHeads * nChunks, p.smax);
     switch (gmax) {
-    case 1: hipLaunchKernelGGL((attn_decode_kernel<HD, 1, KVH>), grid, dim3(WG), 0, s, p); break;
+    case 1: hipLaunchKernelGGL((attn_decode_kernel<HD, 1, KVH, 2 * WG>), grid, dim3(2 * WG), 0, s, p); break;
     case 2: hipLaunchKernelGGL((attn_decode_kernel<HD, 2, KVH>), grid, dim3(WG), 0, s, p); break;
     default: hipLaunchKernelGGL((attn_decode_kernel<HD, 4, KVH>), grid, dim3(WG), 0, s, p); break;
     }
