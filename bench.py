@@ -158,6 +158,8 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds of CPU baseline work (0 = skip)")
     ap.add_argument("--profile-steps", type=int, default=20)
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--exec-mode", type=int, default=1, choices=[1, 2],
+                    help="1 = fused launches (default); 2 = the same without the L2 prefetch by the attention launch's idle workgroups")
     ap.add_argument("--context", type=int, default=0,
                     help="start the timed decode at this position (KV rows between the prompt and it are zeros): long-context timing")
     ap.add_argument("--pmc-copy", action="store_true",
@@ -190,6 +192,8 @@ def main():
     t_load = time.perf_counter()
     kv_f16 = args.kv == "f16"
     f = load_model(E, np, s, args.seed, maxSeq, eng, kv_f16=kv_f16)
+    if args.exec_mode != 1 and f.SetExecMode(args.exec_mode) != 0:
+        raise SystemExit("bench.py: " + E.last_error())
     t_load = time.perf_counter() - t_load
     prompt = E.synth_tokens(args.seed, 20_000_003, s.vocab, W)
     use_graph = not args.no_graph

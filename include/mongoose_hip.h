@@ -209,7 +209,9 @@ int mg_hidden_idx(mg_ctx* ctx);
 
 /* Execution mode of the layer loop: 0 = one launch per reference op, in the
  * reference's order (cuda_fused_infer.go:417-443, 17 launches a layer);
- * 1 = fused launches (default).  Both give the same results to rounding. */
+ * 1 = fused launches (default); 2 = fused launches whose attention launch does not
+ * also fetch the following matrices into L2 with its idle workgroups (for a GPU
+ * shared with other work).  All give the same results to rounding. */
 int mg_set_exec_mode(mg_ctx* ctx, int mode);
 
 /* Whole token on the device: embedding gather -> layers -> final norm ->

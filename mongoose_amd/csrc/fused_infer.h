@@ -90,7 +90,8 @@ public:
     int kvHalf = 0;
 
     int quantRounding = 0;
-    int execMode = 1;
+    int execMode = 1;       // 0: one launch per reference op; 1: fused launches; 2: fused, attention launches without the L2 prefetch helpers
+    void SetExecMode(int mode) { if (mode != execMode) invalidateGraphs(); execMode = mode; }
 
     // shape
     int dim, kvDim, headDim, nHeads, nKVHeads, ffnDim, vocabSize, nLayers, maxSeq;
@@ -129,6 +130,11 @@ private:
     size_t layerSlabBytes = 0;
     DevMat* matSlot(int idx, int* rows, int* cols);
     int enqueueLayerFused(const LayerWeights& L, int layer, const StepState* st, int posImm);
+    MvParams qkvParams(const LayerWeights& L, int layer, const StepState* st, int posImm) const;
+    MvParams woParams(const LayerWeights& L) const;
+    MvParams gateUpParams(const LayerWeights& L) const;
+    MvParams downParams(const LayerWeights& L) const;
+    void planPrefetch(int layer, PfJob& job) const;
     int enqueueLayerPerOp(const LayerWeights& L, int layer, int pos);
     int enqueueEmbed();
     int enqueueToken(bool withHead);      // embed -> layers -> final(+argmax) / advance, all from device state

@@ -489,21 +489,74 @@ int HIPFusedInference::enqueueLayerPerOp(const LayerWeights& L, int layer, int p
 
 // Five launches a layer: [norm1 + QKV + bias + RoPE + KV-cache write] [attention]
 // [Wo + residual] [norm2 + gate/up + SiLU*mul] [down + residual].
-int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const StepState* st, int posImm) {
+// Operands of the four matvec launches of a layer (what is launched and what the prefetch plan describes).
+MvParams HIPFusedInference::qkvParams(const LayerWeights& L, int layer, const StepState* st, int posImm) const {
+    MvParams p{};
+    p.K = dim; p.act = hidden[hiddenIdx]; p.gain = L.norm1; p.eps = eps;
+    p.seg[0] = MvSeg{L.wq.w, L.wq.scales, L.bq, Q, dim};
+    p.seg[1] = MvSeg{L.wk.w, L.wk.scales, L.bk, kCache[layer], kvDim};
+    p.seg[2] = MvSeg{L.wv.w, L.wv.scales, L.bv, vCache[layer], kvDim};
+    p.nseg = 3;
+    p.headDim = headDim; p.kvDim = kvDim; p.kvHalf = kvHalf;
+    p.state = st; p.posImm = posImm;
+    const int half = headDim / 2;
+    p.cosRow = st ? ropeCur : cosTab + (size_t)posImm * half;
+    p.sinRow = st ? ropeCur + half : sinTab + (size_t)posImm * half;
+    return p;
+}
+MvParams HIPFusedInference::woParams(const LayerWeights& L) const {
+    MvParams p{};
     float* h = hidden[hiddenIdx];
+    p.seg[0] = MvSeg{L.wo.w, L.wo.scales, nullptr, h, dim};
+    p.nseg = 1; p.K = dim; p.act = attnOut; p.resid = h;
+    return p;
+}
+MvParams HIPFusedInference::gateUpParams(const LayerWeights& L) const {
+    MvParams p{};
+    p.seg[0] = MvSeg{L.gate.w, L.gate.scales, nullptr, ffnMid, ffnDim};
+    p.seg[1] = MvSeg{L.up.w, L.up.scales, nullptr, nullptr, ffnDim};
+    p.nseg = 2; p.K = dim; p.act = hidden[hiddenIdx]; p.gain = L.norm2; p.eps = eps;
+    return p;
+}
+MvParams HIPFusedInference::downParams(const LayerWeights& L) const {
+    MvParams p{};
+    float* h = hidden[hiddenIdx];
+    p.seg[0] = MvSeg{L.down.w, L.down.scales, nullptr, h, dim};
+    p.nseg = 1; p.K = ffnDim; p.act = ffnMid; p.resid = h;
+    return p;
+}
+
+// What the idle part of layer `layer`'s attention launch fetches into L2: the next layer's q|k|v and Wo
+// (this layer's Wo is the very next launch: too late) and this layer's gate|up.  The down projection
+// is left out: fetching it too makes the attention launch wait for its helpers longer than the
+// down launch gains.  Only for a model whose layer fits the L2s several times over; a larger one
+// would evict what was fetched before it is used, and streams its weights at HBM speed anyway.
+void HIPFusedInference::planPrefetch(int layer, PfJob& job) const {
+    job = PfJob{};
+    if (execMode != 1) return;
+    const LayerWeights& L = layers[layer];
+    if (L.wq.bytes + L.wk.bytes + L.wv.bytes + L.wo.bytes + L.gate.bytes + L.up.bytes + L.down.bytes > ((size_t)20 << 20)) return;
+    PfJob j{};
+    if (layer + 1 < nLayers) {
+        const LayerWeights& N = layers[layer + 1];
+        const bool uniform = N.wq.kind == N.wk.kind && N.wk.kind == N.wv.kind && N.gate.kind == N.up.kind;
+        if (layerComplete(N) && uniform && kCache[layer + 1]) {
+            PfJob k = j;
+            if (plan_matvec_prefetch(N.wq.kind, EPI_QKV, PRO_RMS, qkvParams(N, layer + 1, nullptr, 0), k) &&
+                plan_matvec_prefetch(N.wo.kind, EPI_RESID, PRO_PLAIN, woParams(N), k))
+                j = k;
+        }
+    }
+    plan_matvec_prefetch(L.gate.kind, EPI_SWIGLU, PRO_RMS, gateUpParams(L), j);
+    if (j.nregion == 0) return;
+    j.helperWaves = 960;          // measured: 120 workgroups of eight waves; twice as many disturb the attention workgroups more
+    job = j;
+}
+
+int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const StepState* st, int posImm) {
     if (mark(1)) return MG_E_HIP;
     {
-        MvParams p{};
-        p.K = dim; p.act = h; p.gain = L.norm1; p.eps = eps;
-        p.seg[0] = MvSeg{L.wq.w, L.wq.scales, L.bq, Q, dim};
-        p.seg[1] = MvSeg{L.wk.w, L.wk.scales, L.bk, kCache[layer], kvDim};
-        p.seg[2] = MvSeg{L.wv.w, L.wv.scales, L.bv, vCache[layer], kvDim};
-        p.nseg = 3;
-        p.headDim = headDim; p.kvDim = kvDim; p.kvHalf = kvHalf;
-        p.state = st; p.posImm = posImm;
-        const int half = headDim / 2;
-        p.cosRow = st ? ropeCur : cosTab + (size_t)posImm * half;
-        p.sinRow = st ? ropeCur + half : sinTab + (size_t)posImm * half;
+        MvParams p = qkvParams(L, layer, st, posImm);
         HIPCHK(launch_matvec(L.wq.kind, EPI_QKV, PRO_RMS, p, nullptr, stream));
     }
     if (mark(2)) return MG_E_HIP;
@@ -515,28 +568,22 @@ int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const
         a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
         a.smax = smax; a.splitLen = splitLen; a.headsPerWG = attnHeadsPerWG;
         a.pm = pm; a.pl = pl; a.pacc = pacc; a.counters = attnCounters; a.out = attnOut;
+        planPrefetch(layer, a.pf);
         HIPCHK(launch_attention(a, stream));
     }
     if (mark(3)) return MG_E_HIP;
     {
-        MvParams p{};
-        p.seg[0] = MvSeg{L.wo.w, L.wo.scales, nullptr, h, dim};
-        p.nseg = 1; p.K = dim; p.act = attnOut; p.resid = h;
+        MvParams p = woParams(L);
         HIPCHK(launch_matvec(L.wo.kind, EPI_RESID, PRO_PLAIN, p, nullptr, stream));
     }
     if (mark(4)) return MG_E_HIP;
     {
-        MvParams p{};
-        p.seg[0] = MvSeg{L.gate.w, L.gate.scales, nullptr, ffnMid, ffnDim};
-        p.seg[1] = MvSeg{L.up.w, L.up.scales, nullptr, nullptr, ffnDim};
-        p.nseg = 2; p.K = dim; p.act = h; p.gain = L.norm2; p.eps = eps;
+        MvParams p = gateUpParams(L);
         HIPCHK(launch_matvec(L.gate.kind, EPI_SWIGLU, PRO_RMS, p, nullptr, stream));
     }
     if (mark(5)) return MG_E_HIP;
     {
-        MvParams p{};
-        p.seg[0] = MvSeg{L.down.w, L.down.scales, nullptr, h, dim};
-        p.nseg = 1; p.K = ffnDim; p.act = ffnMid; p.resid = h;
+        MvParams p = downParams(L);
         HIPCHK(launch_matvec(L.down.kind, EPI_RESID, PRO_PLAIN, p, nullptr, stream));
     }
     return MG_OK;
@@ -1099,8 +1146,8 @@ int mg_swap_hidden_buffer(mg_ctx* c) { CTX(c); return f->SwapHiddenBuffer(); }
 int mg_hidden_idx(mg_ctx* c) { CTX(c); return f->hiddenIdx; }
 int mg_set_exec_mode(mg_ctx* c, int mode) {
     CTX(c);
-    if (mode != 0 && mode != 1) { mg::set_error("exec mode must be 0 or 1"); return MG_E_ARG; }
-    f->execMode = mode;
+    if (mode < 0 || mode > 2) { mg::set_error("exec mode must be 0, 1 or 2"); return MG_E_ARG; }
+    f->SetExecMode(mode);
     return MG_OK;
 }
 int mg_decode_token(mg_ctx* c, int token, int pos, int* next, float* logitsOut) { CTX(c); return f->DecodeToken(token, pos, next, logitsOut); }

@@ -78,6 +78,26 @@ MvConfig pick_config(int wf, int epi, int totalRows, int K);
 // grid size, is written back.
 hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInOut, hipStream_t s);
 
+// What later launches of the step will read, for workgroups that have nothing else to do: the decode
+// attention of a small model keeps a handful of CUs busy, the rest of its launch pulls the next
+// matrices into L2.  Workgroup i of a launch runs on XCD i & 7 and every XCD has an L2 of its own, so
+// weights are described in runs: run r of a region (bytes [r * runBytes, (r + 1) * runBytes)) will be
+// read by a workgroup on XCD (xoff + r) & 7 and is fetched by a helper on that XCD.  A region with
+// xoff < 0 (scales, gains, biases) is read by every workgroup and fetched on every XCD.
+struct PfRegion { const char* base; unsigned bytes; unsigned runBytes; int xoff; int nruns; };
+constexpr int PF_MAX_REGIONS = 28;
+struct PfJob {
+    PfRegion region[PF_MAX_REGIONS];
+    int nregion;
+    int helperWaves;      // waves to spread the job over (0: no helpers); the launcher turns it into
+    int rows;             // rows of helper workgroups appended to the attention grid,
+    int wgsPerXcd;        // helper workgroups that take part on each XCD, and
+    int waveStart[PF_MAX_REGIONS + 1];   // region r is fetched by waves waveStart[r] .. waveStart[r+1]-1 of an XCD's helper waves
+};
+// Appends what launch_matvec(wf, epi, ..., p) will read; false (job unchanged) when that launch does not
+// keep rows on fixed XCDs (several rounds of workgroups, formats without a fast kernel) or the job is full.
+bool plan_matvec_prefetch(int wf, int epi, int pro, const MvParams& p, PfJob& job);
+
 struct AttnParams {
     const float* q;       // [dim], rotated
     const float* Kc;      // [rowLimit, kvDim], row pos already written
@@ -93,6 +113,7 @@ struct AttnParams {
     int headsPerWG;       // query heads of a GQA group per workgroup (0 = the whole group, in chunks of up to 4)
     float* out;           // [dim]
     int kvHalf;           // Kc / Vc hold fp16 instead of fp32 (same [row, kvDim] indexing)
+    PfJob pf;             // pf.rows > 0: grid rows smax .. smax + pf.rows - 1 are prefetch helpers
 };
 hipError_t launch_attention(const AttnParams& p, hipStream_t s);
 int attention_columns(int nHeads, int nKVHeads, int headsPerWG);

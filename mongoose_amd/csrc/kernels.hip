@@ -825,12 +825,14 @@ static hipError_t launch_wf(int pro, int epi, MvParams& p, const MvConfig& c, hi
     return hipErrorInvalidValue;
 }
 
-hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInOut, hipStream_t s) {
+// Row grouping and grid of a launch: fills p.ngroups / p.segGroup0 and c (what launch_matvec runs with,
+// the short-row lm_head kernels aside).
+static hipError_t resolve_matvec(int wf, int epi, MvParams& p, const MvConfig* cfgInOut, MvConfig& c) {
     const int CH = wf == WF_Q8 ? 16 : 32;
     if (p.K <= 0 || p.K % CH != 0 || (size_t)p.K * 4 > 64 * 1024) return hipErrorInvalidValue;
     int total = 0;
     for (int i = 0; i < p.nseg; i++) total += p.seg[i].rows;
-    MvConfig c = (cfgInOut && cfgInOut->nr > 0) ? *cfgInOut
+    c = (cfgInOut && cfgInOut->nr > 0) ? *cfgInOut
                                                 : pick_config(wf, epi, epi == EPI_SWIGLU ? p.seg[0].rows : total, p.K);
     if (epi == EPI_SWIGLU) {
         if (p.nseg != 2 || p.seg[0].rows != p.seg[1].rows) return hipErrorInvalidValue;
@@ -856,14 +858,24 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
         p.ngroups = g;
     }
     if (p.ngroups == 0) return hipSuccess;
-    int wgs = c.ks == 1 ? (p.ngroups + 3) / 4 : p.ngroups;
-    int cap = epi == EPI_ARGMAX ? 1024 : 2048;      // one argmax partial per workgroup
+    const int wgs = c.ks == 1 ? (p.ngroups + 3) / 4 : p.ngroups;
+    const int cap = epi == EPI_ARGMAX ? 1024 : 2048;      // one argmax partial per workgroup
     if (c.grid <= 0 || c.grid > wgs) {
         // every workgroup stages the activation vector: beyond the cap each takes several groups,
         // the same number each (an uneven last round leaves most of the chip idle)
         const int rounds = (wgs + cap - 1) / cap;
         c.grid = epi == EPI_ARGMAX ? (wgs < cap ? wgs : cap) : (wgs + rounds - 1) / rounds;
     }
+    return hipSuccess;
+}
+
+hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInOut, hipStream_t s) {
+    MvConfig c{0, 0, 0};
+    hipError_t e = resolve_matvec(wf, epi, p, cfgInOut, c);
+    if (e != hipSuccess) return e;
+    if (p.ngroups == 0) return hipSuccess;
+    int wgs;
+    const int cap = epi == EPI_ARGMAX ? 1024 : 2048;
     if (wf == WF_Q8 && pro == PRO_RMS && epi == EPI_ARGMAX && p.nseg == 1 && !p.seg[0].bias && !p.div127 &&
         p.K / 16 <= 128 && c.ks == 1 && !(cfgInOut && cfgInOut->nr > 0)) {
         c.nr = 4;
@@ -888,6 +900,56 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
     if (wf == WF_Q8) return launch_wf<WF_Q8>(pro, epi, p, c, s);
     if (wf == WF_Q4P) return launch_wf<WF_Q4P>(pro, epi, p, c, s);
     return launch_wf<WF_Q4RAW>(pro, epi, p, c, s);
+}
+
+bool plan_matvec_prefetch(int wf, int epi, int pro, const MvParams& pin, PfJob& job) {
+    if (wf != WF_Q8 && wf != WF_Q4P) return false;
+    MvParams p = pin;
+    MvConfig c{0, 0, 0};
+    if (resolve_matvec(wf, epi, p, nullptr, c) != hipSuccess || p.ngroups == 0) return false;
+    const int wgs = c.ks == 1 ? (p.ngroups + 3) / 4 : p.ngroups;
+    if (c.grid != wgs) return false;                 // several rounds: a row's workgroup index is not its run index
+    PfJob j = job;
+    auto region = [&](const void* base, size_t bytes, size_t runBytes, int xoff) {
+        if (j.nregion >= PF_MAX_REGIONS || bytes == 0 || bytes >= (1ull << 31)) return false;
+        j.region[j.nregion++] = PfRegion{static_cast<const char*>(base), (unsigned)bytes, (unsigned)runBytes, xoff & 7,
+                                         (int)((bytes + runBytes - 1) / runBytes)};
+        return true;
+    };
+    auto flat = [&](const void* base, size_t bytes) {
+        if (!base || bytes == 0) return true;
+        if (j.nregion >= PF_MAX_REGIONS || bytes >= (1ull << 31)) return false;
+        j.region[j.nregion++] = PfRegion{static_cast<const char*>(base), (unsigned)bytes, 1024u, -1, (int)((bytes + 1023) / 1024)};
+        return true;
+    };
+    for (int i = 0; i < p.nseg; i++) {
+        // rows of one workgroup are consecutive (q/k: two such pieces half a head apart, whose run
+        // indices differ by a multiple of 8 once a head has 64 rows or more)
+        int run, xoff;
+        const int perWG = c.ks == 1 ? 4 : 1;         // row groups a workgroup takes
+        if (epi == EPI_SWIGLU) {
+            run = perWG * (c.nr / 2); xoff = 0;
+        } else if (epi == EPI_QKV) {
+            if (c.ks != 1 || p.headDim < 64 || (p.segGroup0[i] & 3)) return false;
+            run = i < 2 ? 4 : 8; xoff = p.segGroup0[i] >> 2;
+        } else {
+            if (c.ks == 1 && (p.segGroup0[i] & 3)) return false;
+            run = perWG * c.nr; xoff = c.ks == 1 ? p.segGroup0[i] >> 2 : p.segGroup0[i];
+        }
+        const size_t rows = p.seg[i].rows;
+        const char* w = static_cast<const char*>(p.seg[i].w);
+        if (wf == WF_Q8) {
+            if (!region(w, rows * p.K, (size_t)run * p.K, xoff) || !flat(p.seg[i].aux, rows * 4)) return false;
+        } else {
+            if (!region(w, rows * (p.K / 2), (size_t)run * (p.K / 2), xoff) ||
+                !region(w + rows * (p.K / 2), rows * (p.K / 16), (size_t)run * (p.K / 16), xoff))
+                return false;
+        }
+        if (!flat(p.seg[i].bias, rows * 4)) return false;
+    }
+    if (pro == PRO_RMS && !flat(p.gain, (size_t)p.K * 4)) return false;
+    job = j;
+    return true;
 }
 
 // Any K, any alignment: one wave per row, byte loads.  Only used by the
@@ -972,8 +1034,48 @@ __device__ __forceinline__ float4 ld_kv4(const void* base, size_t idx4) {
     return make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
 }
 
+// A helper workgroup of the attention launch (grid rows past the splits): its waves fetch their share
+// of one region each into this XCD's L2.  Two scalar loads (the wave table, one region) come before
+// the first fetch; the loads all land in one register that nothing reads, and none is waited for
+// before the last one is out.
+typedef int pf_v4i __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void prefetch_helper(const PfJob& job, int firstFlat, int nWaves) {
+    const int lane = threadIdx.x & 63;
+    const int flatId = blockIdx.x + blockIdx.y * gridDim.x;      // dispatch order: XCD = flatId & 7
+    const int x = flatId & 7;
+    const int first = firstFlat + ((x - firstFlat) & 7);         // first helper on this XCD
+    const int rank = (flatId - first) >> 3;                      // this workgroup among the XCD's helpers
+    if (rank >= job.wgsPerXcd) return;
+    const int hw = rank * nWaves + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    int r = 0;
+#pragma unroll
+    for (int i = 1; i < PF_MAX_REGIONS; i++)
+        if (i < job.nregion && hw >= job.waveStart[i]) r = i;
+    const int lw = hw - job.waveStart[r];
+    const int nw = job.waveStart[r + 1] - job.waveStart[r];
+    if (lw >= nw) return;
+    const PfRegion R = job.region[r];
+    const unsigned end = (R.bytes + 15u) & ~15u;
+    const int nruns = R.nruns;
+    const int q0 = R.xoff < 0 ? 0 : (x - R.xoff) & 7;
+    const int qs = R.xoff < 0 ? 1 : 8;                           // runs q0, q0 + qs, ...
+    pf_v4i sink = {0, 0, 0, 0};
+    for (int q = q0 + qs * lw; q < nruns; q += qs * nw) {
+        const unsigned b0 = (unsigned)q * R.runBytes;
+        unsigned b1 = b0 + R.runBytes;
+        b1 = b1 < end ? (b1 + 15u) & ~15u : end;
+        for (unsigned o = (b0 & ~15u) + lane * 16; o < b1; o += 1024)
+            asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(sink) : "v"(R.base + o) : "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(sink) : : "memory");
+}
+
 template <int HD, int GMAX, bool KVH, int AWG = WG>
 __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
+    if (blockIdx.y >= p.smax) {                          // uniform: a whole workgroup is either a helper or not
+        prefetch_helper(p.pf, p.smax * gridDim.x, AWG / 64);
+        return;
+    }
     constexpr int NWV = AWG / 64;      // waves: 4, or more for the one-head workgroups of short contexts (fewer rows per thread)
     constexpr int LPR = 16;            // lanes per K/V row: one DPP row
     constexpr int NF = HD / 64;        // float4s of a row per lane (float4 index j*16 + dl)
@@ -1236,11 +1338,40 @@ static int attention_gmax(int G, int heads) {
 }
 
 template <int HD, bool KVH>
-static hipError_t launch_attn_hd(const AttnParams& p, hipStream_t s) {
+static hipError_t launch_attn_hd(const AttnParams& pin, hipStream_t s) {
+    AttnParams p = pin;
     int G = p.nHeads / p.nKVHeads;
     int gmax = attention_gmax(G, p.headsPerWG);
     int nChunks = (G + gmax - 1) / gmax;
-    dim3 grid(p.nKVHeads * nChunks, p.smax);
+    const int cols = p.nKVHeads * nChunks;
+    const int wavesPerWG = gmax == 1 ? 8 : 4;
+    p.pf.rows = 0;
+    if (p.pf.helperWaves > 0 && p.pf.nregion > 0) {
+        // helper workgroups: the same number on every XCD (a few of the last grid row stay idle); the
+        // XCD's helper waves are shared out over the regions by the bytes an XCD fetches of each
+        const int rows = (p.pf.helperWaves + wavesPerWG * cols - 1) / (wavesPerWG * cols);
+        const int perXcd = rows * cols / 8;
+        const int W = perXcd * wavesPerWG;
+        if (W >= p.pf.nregion) {
+            double share[PF_MAX_REGIONS], total = 0.0;
+            for (int i = 0; i < p.pf.nregion; i++) {
+                share[i] = p.pf.region[i].xoff < 0 ? (double)p.pf.region[i].bytes : p.pf.region[i].bytes / 8.0;
+                total += share[i];
+            }
+            int spare = W - p.pf.nregion, at = 0;        // one wave each, the rest by share
+            double acc = 0.0;
+            for (int i = 0; i < p.pf.nregion; i++) {
+                p.pf.waveStart[i] = at;
+                const int before = (int)(acc / total * spare + 0.5);
+                acc += share[i];
+                at += 1 + (int)(acc / total * spare + 0.5) - before;
+            }
+            p.pf.waveStart[p.pf.nregion] = at;
+            p.pf.rows = rows;
+            p.pf.wgsPerXcd = perXcd;
+        }
+    }
+    dim3 grid(cols, p.smax + p.pf.rows);
     switch (gmax) {
     case 1: hipLaunchKernelGGL((attn_decode_kernel<HD, 1, KVH, 2 * WG>), grid, dim3(2 * WG), 0, s, p); break;
     case 2: hipLaunchKernelGGL((attn_decode_kernel<HD, 2, KVH>), grid, dim3(WG), 0, s, p); break;

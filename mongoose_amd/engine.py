@@ -306,6 +306,7 @@ class HIPFusedInference:
         return lib.mg_reset_kv(self._h)
 
     def SetExecMode(self, mode):
+        """0 = one launch per reference op, 1 = fused launches (default), 2 = fused without the L2 prefetch helpers."""
         return lib.mg_set_exec_mode(self._h, mode)
 
     # L3 bridge and mailbox (cuda_fused_infer.go:556-737)

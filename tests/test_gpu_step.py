@@ -373,6 +373,41 @@ def test_lm_head_short_row_kernels_ragged_shapes(hip, fmt, dim, heads, kvHeads, 
     m.close()
 
 
+@pytest.mark.parametrize("fmt,maxSeq", [("q8", 40), ("q8", 600), ("q4_0", 40)])
+def test_attention_prefetch_helpers_change_nothing(hip, fmt, maxSeq):
+    """Exec mode 1 appends helper workgroups to every attention launch of a small model (they pull the
+    next matrices into L2); mode 2 launches attention alone.  The helpers only read, so logits are
+    identical bit for bit -- with one KV split (maxSeq 40) and with several, where the helper rows of
+    the grid come after the split rows (maxSeq 600: three splits), Q8 and Q4_0 weights (the Q4_0 job
+    has two regions per matrix, and its fp16 scale plane is fetched in runs that are not multiples of 16 bytes)."""
+    s = H.with_layers(configs.QWEN if fmt == "q8" else configs.QWEN_Q4, 3)._replace(vocab=2000 if fmt == "q8" else 2016)
+    m = H.Model(s, seed=23, maxSeq=maxSeq, eng=hip, threads=8)
+    n = 6 if maxSeq < 100 else 300
+    prompt = m.prompt(n)
+    outs = {}
+    for mode in (1, 2):
+        assert m.hip.SetExecMode(mode) == 0
+        assert m.hip.ResetKV() == 0
+        logits = np.empty(s.vocab, np.float32)
+        res = []
+        for pos in range(n):
+            last = pos >= n - 3
+            rc, nxt = m.hip.DecodeToken(int(prompt[pos]), pos, logits if last else None)
+            assert rc == 0, E.last_error()
+            if last:
+                res.append((nxt, logits.copy()))
+        outs[mode] = res
+    for (n1, l1), (n2, l2) in zip(outs[1], outs[2]):
+        assert n1 == n2 and np.array_equal(l1, l2)
+    # and the graph replay (mode 1) gives the oracle's tokens
+    assert m.hip.SetExecMode(1) == 0
+    assert m.hip.ResetKV() == 0
+    toks_ref, _ = H.oracle_generate(m, prompt[:5], 6)
+    rc, toks = m.hip.Generate(prompt[:5], 6, useGraph=True)
+    assert rc == 0 and toks.tolist() == toks_ref.tolist()
+    m.close()
+
+
 def test_layer_range_pipeline_with_l3_bridge_and_mailbox(hip):
     """Two contexts as pipeline stages (layers 0-1 and 2-3 of the toy model, PartialStep's layer
     ranges): stage A's hidden state reaches the host through the L3 bridge (copy stream) and its
