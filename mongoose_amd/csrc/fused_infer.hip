@@ -526,30 +526,51 @@ MvParams HIPFusedInference::downParams(const LayerWeights& L) const {
     return p;
 }
 
-// What the idle part of layer `layer`'s attention launch fetches into L2: the next layer's q|k|v and Wo
-// (this layer's Wo is the very next launch: too late) and this layer's gate|up.  The down projection
-// is left out: fetching it too makes the attention launch wait for its helpers longer than the
-// down launch gains.  Only for a model whose layer fits the L2s several times over; a larger one
-// would evict what was fetched before it is used, and streams its weights at HBM speed anyway.
+// What the idle part of layer `layer`'s attention launch fetches into L2: the launches that follow it,
+// in their order -- Wo, gate|up, down, the next layer's q|k|v and Wo -- as long as the helpers can
+// have it in before the attention itself is done (a budget in bytes) and the lines will still be
+// there when they are wanted (what flows through the L2s in between stays under their size).  A
+// layer small enough for its successor's Wo to stay gets that one instead of its own (which came
+// with the launch before): it need not be in by the end of this launch.
 void HIPFusedInference::planPrefetch(int layer, PfJob& job) const {
     job = PfJob{};
     if (execMode != 1) return;
+    const size_t budget = (size_t)12 << 20;       // measured: 10.6 MB make the attention launch 0.3 us longer, 15 MB 3 us
+    const size_t l2 = (size_t)24 << 20;           // of 8 x 4 MB
     const LayerWeights& L = layers[layer];
-    if (L.wq.bytes + L.wk.bytes + L.wv.bytes + L.wo.bytes + L.gate.bytes + L.up.bytes + L.down.bytes > ((size_t)20 << 20)) return;
-    PfJob j{};
+    const LayerWeights* N = nullptr;
     if (layer + 1 < nLayers) {
-        const LayerWeights& N = layers[layer + 1];
-        const bool uniform = N.wq.kind == N.wk.kind && N.wk.kind == N.wv.kind && N.gate.kind == N.up.kind;
-        if (layerComplete(N) && uniform && kCache[layer + 1]) {
-            PfJob k = j;
-            if (plan_matvec_prefetch(N.wq.kind, EPI_QKV, PRO_RMS, qkvParams(N, layer + 1, nullptr, 0), k) &&
-                plan_matvec_prefetch(N.wo.kind, EPI_RESID, PRO_PLAIN, woParams(N), k))
-                j = k;
-        }
+        const LayerWeights& C = layers[layer + 1];
+        const bool uniform = C.wq.kind == C.wk.kind && C.wk.kind == C.wv.kind && C.gate.kind == C.up.kind;
+        if (layerComplete(C) && uniform && kCache[layer + 1]) N = &C;
     }
-    plan_matvec_prefetch(L.gate.kind, EPI_SWIGLU, PRO_RMS, gateUpParams(L), j);
+    const size_t nextQkv = N ? N->wq.bytes + N->wk.bytes + N->wv.bytes : 0;
+    const bool nextWoStays = N && L.wo.bytes + L.gate.bytes + L.up.bytes + L.down.bytes + nextQkv + N->wo.bytes <= l2;
+    // the regions wanted last are listed first: they go to the helper workgroups that start first
+    // (measured: 0.3 % of the step against the other order)
+    PfJob late{}, soon{};
+    size_t taken = 0, flowed = 0;
+    auto considerFor = [&](PfJob& j, size_t bytes, auto&& plan) {
+        if (taken + bytes <= budget && flowed + bytes <= l2) {
+            PfJob k = j;
+            if (late.nregion + soon.nregion + (k.nregion - j.nregion) <= PF_MAX_REGIONS && plan(k)) { j = k; taken += bytes; }
+        }
+        flowed += bytes;
+    };
+    auto consider = [&](size_t bytes, auto&& plan) { considerFor(soon, bytes, plan); };
+    if (nextWoStays) flowed += L.wo.bytes;
+    else consider(L.wo.bytes, [&](PfJob& k) { return plan_matvec_prefetch(L.wo.kind, EPI_RESID, PRO_PLAIN, woParams(L), k); });
+    consider(L.gate.bytes + L.up.bytes, [&](PfJob& k) { return plan_matvec_prefetch(L.gate.kind, EPI_SWIGLU, PRO_RMS, gateUpParams(L), k); });
+    consider(L.down.bytes, [&](PfJob& k) { return plan_matvec_prefetch(L.down.kind, EPI_RESID, PRO_PLAIN, downParams(L), k); });
+    if (N) {
+        considerFor(late, nextQkv, [&](PfJob& k) { return plan_matvec_prefetch(N->wq.kind, EPI_QKV, PRO_RMS, qkvParams(*N, layer + 1, nullptr, 0), k); });
+        if (nextWoStays)
+            considerFor(late, N->wo.bytes, [&](PfJob& k) { return plan_matvec_prefetch(N->wo.kind, EPI_RESID, PRO_PLAIN, woParams(*N), k); });
+    }
+    PfJob j = late;
+    for (int i = 0; i < soon.nregion && j.nregion < PF_MAX_REGIONS; i++) j.region[j.nregion++] = soon.region[i];
     if (j.nregion == 0) return;
-    j.helperWaves = 960;          // measured: 120 workgroups of eight waves; twice as many disturb the attention workgroups more
+    j.helperWaves = 960;          // measured: half as many are too slow, twice as many disturb the attention workgroups
     job = j;
 }
 
