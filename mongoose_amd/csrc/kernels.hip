@@ -1348,14 +1348,16 @@ static hipError_t launch_attn_hd(const AttnParams& pin, hipStream_t s) {
     p.pf.rows = 0;
     if (p.pf.helperWaves > 0 && p.pf.nregion > 0) {
         // helper workgroups: the same number on every XCD (a few of the last grid row stay idle); the
-        // XCD's helper waves are shared out over the regions by the bytes an XCD fetches of each
+        // XCD's helper waves are shared out over the regions by the loads an XCD issues for each
         const int rows = (p.pf.helperWaves + wavesPerWG * cols - 1) / (wavesPerWG * cols);
         const int perXcd = rows * cols / 8;
         const int W = perXcd * wavesPerWG;
         if (W >= p.pf.nregion) {
             double share[PF_MAX_REGIONS], total = 0.0;
             for (int i = 0; i < p.pf.nregion; i++) {
-                share[i] = p.pf.region[i].xoff < 0 ? (double)p.pf.region[i].bytes : p.pf.region[i].bytes / 8.0;
+                // in load instructions (1 KB a wave): a region of short runs needs as many as one of long runs
+                const PfRegion& R = p.pf.region[i];
+                share[i] = (double)((R.runBytes + 1023) / 1024) * (R.xoff < 0 ? R.nruns : (R.nruns + 7) / 8);
                 total += share[i];
             }
             int spare = W - p.pf.nregion, at = 0;        // one wave each, the rest by share
