@@ -530,8 +530,10 @@ MvParams HIPFusedInference::downParams(const LayerWeights& L) const {
 // in their order -- Wo, gate|up, down, the next layer's q|k|v and Wo -- as long as the helpers can
 // have it in before the attention itself is done (a budget in bytes) and the lines will still be
 // there when they are wanted (what flows through the L2s in between stays under their size).  A
-// layer small enough for its successor's Wo to stay gets that one instead of its own (which came
-// with the launch before): it need not be in by the end of this launch.
+// launch too large for what is left of the budget is taken in part -- the rows its first
+// workgroups read, which fills the idle start of that launch -- and ends the list.  A layer small
+// enough for its successor's Wo to stay gets that one instead of its own (which came with the
+// launch before): it need not be in by the end of this launch.
 void HIPFusedInference::planPrefetch(int layer, PfJob& job) const {
     job = PfJob{};
     if (execMode != 1) return;
@@ -550,22 +552,27 @@ void HIPFusedInference::planPrefetch(int layer, PfJob& job) const {
     // (measured: 0.3 % of the step against the other order)
     PfJob late{}, soon{};
     size_t taken = 0, flowed = 0;
-    auto considerFor = [&](PfJob& j, size_t bytes, auto&& plan) {
-        if (taken + bytes <= budget && flowed + bytes <= l2) {
+    bool open = true;                              // nothing after a launch that was taken in part or not at all
+    const size_t minPart = (size_t)4 << 20;       // a launch that does not fit is taken in part (its first rows) if that much room is left
+    auto considerFor = [&](PfJob& j, size_t bytes, bool needWhole, auto&& plan) {
+        const size_t room = budget > taken ? budget - taken : 0;
+        if (open && flowed + (bytes < room ? bytes : room) <= l2 && (bytes <= room || (!needWhole && room >= minPart))) {
             PfJob k = j;
-            if (late.nregion + soon.nregion + (k.nregion - j.nregion) <= PF_MAX_REGIONS && plan(k)) { j = k; taken += bytes; }
+            const size_t got = plan(k, bytes <= room ? (size_t)0 : room);
+            if (got && late.nregion + soon.nregion + (k.nregion - j.nregion) <= PF_MAX_REGIONS) { j = k; taken += got; }
+            if (bytes > room) open = false;
         }
         flowed += bytes;
     };
-    auto consider = [&](size_t bytes, auto&& plan) { considerFor(soon, bytes, plan); };
     if (nextWoStays) flowed += L.wo.bytes;
-    else consider(L.wo.bytes, [&](PfJob& k) { return plan_matvec_prefetch(L.wo.kind, EPI_RESID, PRO_PLAIN, woParams(L), k); });
-    consider(L.gate.bytes + L.up.bytes, [&](PfJob& k) { return plan_matvec_prefetch(L.gate.kind, EPI_SWIGLU, PRO_RMS, gateUpParams(L), k); });
-    consider(L.down.bytes, [&](PfJob& k) { return plan_matvec_prefetch(L.down.kind, EPI_RESID, PRO_PLAIN, downParams(L), k); });
+    else considerFor(soon, L.wo.bytes, false, [&](PfJob& k, size_t lim) { return plan_matvec_prefetch(L.wo.kind, EPI_RESID, PRO_PLAIN, woParams(L), k, lim); });
+    considerFor(soon, L.gate.bytes + L.up.bytes, false,
+                [&](PfJob& k, size_t lim) { return plan_matvec_prefetch(L.gate.kind, EPI_SWIGLU, PRO_RMS, gateUpParams(L), k, lim); });
+    considerFor(soon, L.down.bytes, true, [&](PfJob& k, size_t lim) { return plan_matvec_prefetch(L.down.kind, EPI_RESID, PRO_PLAIN, downParams(L), k, lim); });
     if (N) {
-        considerFor(late, nextQkv, [&](PfJob& k) { return plan_matvec_prefetch(N->wq.kind, EPI_QKV, PRO_RMS, qkvParams(*N, layer + 1, nullptr, 0), k); });
+        considerFor(late, nextQkv, true, [&](PfJob& k, size_t lim) { return plan_matvec_prefetch(N->wq.kind, EPI_QKV, PRO_RMS, qkvParams(*N, layer + 1, nullptr, 0), k, lim); });
         if (nextWoStays)
-            considerFor(late, N->wo.bytes, [&](PfJob& k) { return plan_matvec_prefetch(N->wo.kind, EPI_RESID, PRO_PLAIN, woParams(*N), k); });
+            considerFor(late, N->wo.bytes, true, [&](PfJob& k, size_t lim) { return plan_matvec_prefetch(N->wo.kind, EPI_RESID, PRO_PLAIN, woParams(*N), k, lim); });
     }
     PfJob j = late;
     for (int i = 0; i < soon.nregion && j.nregion < PF_MAX_REGIONS; i++) j.region[j.nregion++] = soon.region[i];

@@ -84,7 +84,7 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
 // weights are described in runs: run r of a region (bytes [r * runBytes, (r + 1) * runBytes)) will be
 // read by a workgroup on XCD (xoff + r) & 7 and is fetched by a helper on that XCD.  A region with
 // xoff < 0 (scales, gains, biases) is read by every workgroup and fetched on every XCD.
-struct PfRegion { const char* base; unsigned bytes; unsigned runBytes; int xoff; int nruns; };
+struct PfRegion { const char* base; unsigned bytes; unsigned runBytes; int xoff; int nruns; int splitLog2; };   // 2^splitLog2 waves share a run (set by the launcher)
 constexpr int PF_MAX_REGIONS = 28;
 struct PfJob {
     PfRegion region[PF_MAX_REGIONS];
@@ -94,9 +94,11 @@ struct PfJob {
     int wgsPerXcd;        // helper workgroups that take part on each XCD, and
     int waveStart[PF_MAX_REGIONS + 1];   // region r is fetched by waves waveStart[r] .. waveStart[r+1]-1 of an XCD's helper waves
 };
-// Appends what launch_matvec(wf, epi, ..., p) will read; false (job unchanged) when that launch does not
-// keep rows on fixed XCDs (several rounds of workgroups, formats without a fast kernel) or the job is full.
-bool plan_matvec_prefetch(int wf, int epi, int pro, const MvParams& p, PfJob& job);
+// Appends what launch_matvec(wf, epi, ..., p) will read and returns its weight bytes; 0 (job unchanged)
+// when that launch does not keep rows on fixed XCDs (rounds of workgroups that are not a multiple of 8,
+// formats without a fast kernel) or the job is full.  limitBytes > 0 and below the launch's bytes: only
+// the first rows of each matrix, as many as fit (not for the q|k|v launch).
+size_t plan_matvec_prefetch(int wf, int epi, int pro, const MvParams& p, PfJob& job, size_t limitBytes = 0);
 
 struct AttnParams {
     const float* q;       // [dim], rotated

@@ -902,24 +902,32 @@ hipError_t launch_matvec(int wf, int epi, int pro, MvParams& p, MvConfig* cfgInO
     return launch_wf<WF_Q4RAW>(pro, epi, p, c, s);
 }
 
-bool plan_matvec_prefetch(int wf, int epi, int pro, const MvParams& pin, PfJob& job) {
-    if (wf != WF_Q8 && wf != WF_Q4P) return false;
+size_t plan_matvec_prefetch(int wf, int epi, int pro, const MvParams& pin, PfJob& job, size_t limitBytes) {
+    if (wf != WF_Q8 && wf != WF_Q4P) return 0;
     MvParams p = pin;
     MvConfig c{0, 0, 0};
-    if (resolve_matvec(wf, epi, p, nullptr, c) != hipSuccess || p.ngroups == 0) return false;
+    if (resolve_matvec(wf, epi, p, nullptr, c) != hipSuccess || p.ngroups == 0) return 0;
     const int wgs = c.ks == 1 ? (p.ngroups + 3) / 4 : p.ngroups;
-    if (c.grid != wgs) return false;                 // several rounds: a row's workgroup index is not its run index
+    // several rounds of workgroups: workgroup b also takes groups b + grid, b + 2 grid, ..., which are
+    // runs of its XCD only when grid is a multiple of 8
+    if (c.grid != wgs && (c.grid & 7)) return 0;
+    const size_t rowBytes = wf == WF_Q8 ? (size_t)p.K : (size_t)p.K / 2 + p.K / 16;
+    size_t total = 0;
+    for (int i = 0; i < p.nseg; i++) total += (size_t)p.seg[i].rows * rowBytes;
+    const bool partial = limitBytes > 0 && limitBytes < total;
+    if (partial && epi == EPI_QKV) return 0;         // q, k and v rows do not come in one order
+    size_t takenBytes = 0;
     PfJob j = job;
     auto region = [&](const void* base, size_t bytes, size_t runBytes, int xoff) {
         if (j.nregion >= PF_MAX_REGIONS || bytes == 0 || bytes >= (1ull << 31)) return false;
         j.region[j.nregion++] = PfRegion{static_cast<const char*>(base), (unsigned)bytes, (unsigned)runBytes, xoff & 7,
-                                         (int)((bytes + runBytes - 1) / runBytes)};
+                                         (int)((bytes + runBytes - 1) / runBytes), 0};
         return true;
     };
     auto flat = [&](const void* base, size_t bytes) {
         if (!base || bytes == 0) return true;
         if (j.nregion >= PF_MAX_REGIONS || bytes >= (1ull << 31)) return false;
-        j.region[j.nregion++] = PfRegion{static_cast<const char*>(base), (unsigned)bytes, 1024u, -1, (int)((bytes + 1023) / 1024)};
+        j.region[j.nregion++] = PfRegion{static_cast<const char*>(base), (unsigned)bytes, 1024u, -1, (int)((bytes + 1023) / 1024), 0};
         return true;
     };
     for (int i = 0; i < p.nseg; i++) {
@@ -930,26 +938,35 @@ bool plan_matvec_prefetch(int wf, int epi, int pro, const MvParams& pin, PfJob& 
         if (epi == EPI_SWIGLU) {
             run = perWG * (c.nr / 2); xoff = 0;
         } else if (epi == EPI_QKV) {
-            if (c.ks != 1 || p.headDim < 64 || (p.segGroup0[i] & 3)) return false;
+            if (c.ks != 1 || p.headDim < 64 || (p.segGroup0[i] & 3)) return 0;
             run = i < 2 ? 4 : 8; xoff = p.segGroup0[i] >> 2;
         } else {
-            if (c.ks == 1 && (p.segGroup0[i] & 3)) return false;
+            if (c.ks == 1 && (p.segGroup0[i] & 3)) return 0;
             run = perWG * c.nr; xoff = c.ks == 1 ? p.segGroup0[i] >> 2 : p.segGroup0[i];
         }
-        const size_t rows = p.seg[i].rows;
+        const size_t allRows = p.seg[i].rows;
+        size_t rows = allRows;
+        if (partial) {
+            // the first rows of every segment (the workgroups that start first), whole sets of 8 runs
+            const size_t set = (size_t)run * 8;
+            rows = limitBytes / p.nseg / rowBytes / set * set;
+            if (rows == 0) return 0;
+            if (rows > allRows) rows = allRows;
+        }
         const char* w = static_cast<const char*>(p.seg[i].w);
         if (wf == WF_Q8) {
-            if (!region(w, rows * p.K, (size_t)run * p.K, xoff) || !flat(p.seg[i].aux, rows * 4)) return false;
+            if (!region(w, rows * p.K, (size_t)run * p.K, xoff) || !flat(p.seg[i].aux, rows * 4)) return 0;
         } else {
             if (!region(w, rows * (p.K / 2), (size_t)run * (p.K / 2), xoff) ||
-                !region(w + rows * (p.K / 2), rows * (p.K / 16), (size_t)run * (p.K / 16), xoff))
-                return false;
+                !region(w + allRows * (p.K / 2), rows * (p.K / 16), (size_t)run * (p.K / 16), xoff))
+                return 0;
         }
-        if (!flat(p.seg[i].bias, rows * 4)) return false;
+        if (!flat(p.seg[i].bias, rows * 4)) return 0;
+        takenBytes += rows * rowBytes;
     }
-    if (pro == PRO_RMS && !flat(p.gain, (size_t)p.K * 4)) return false;
+    if (pro == PRO_RMS && !flat(p.gain, (size_t)p.K * 4)) return 0;
     job = j;
-    return true;
+    return takenBytes;
 }
 
 // Any K, any alignment: one wave per row, byte loads.  Only used by the
@@ -1059,12 +1076,17 @@ __device__ __forceinline__ void prefetch_helper(const PfJob& job, int firstFlat,
     const int nruns = R.nruns;
     const int q0 = R.xoff < 0 ? 0 : (x - R.xoff) & 7;
     const int qs = R.xoff < 0 ? 1 : 8;                           // runs q0, q0 + qs, ...
+    // long runs are shared by 2^splitLog2 waves (every wave gets about the same number of loads)
+    const int sub = lw & ((1 << R.splitLog2) - 1);
+    const int grp = lw >> R.splitLog2;
+    const int ngrp = nw >> R.splitLog2;
+    if (grp >= ngrp) return;
     pf_v4i sink = {0, 0, 0, 0};
-    for (int q = q0 + qs * lw; q < nruns; q += qs * nw) {
+    for (int q = q0 + qs * grp; q < nruns; q += qs * ngrp) {
         const unsigned b0 = (unsigned)q * R.runBytes;
         unsigned b1 = b0 + R.runBytes;
         b1 = b1 < end ? (b1 + 15u) & ~15u : end;
-        for (unsigned o = (b0 & ~15u) + lane * 16; o < b1; o += 1024)
+        for (unsigned o = (b0 & ~15u) + (unsigned)sub * 1024 + lane * 16; o < b1; o += 1024u << R.splitLog2)
             asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(sink) : "v"(R.base + o) : "memory");
     }
     asm volatile("s_waitcnt vmcnt(0)" : "+v"(sink) : : "memory");
@@ -1369,6 +1391,15 @@ static hipError_t launch_attn_hd(const AttnParams& pin, hipStream_t s) {
                 at += 1 + (int)(acc / total * spare + 0.5) - before;
             }
             p.pf.waveStart[p.pf.nregion] = at;
+            for (int i = 0; i < p.pf.nregion; i++) {
+                PfRegion& R = p.pf.region[i];
+                const int nw = p.pf.waveStart[i + 1] - p.pf.waveStart[i];
+                const int runsHere = R.xoff < 0 ? R.nruns : (R.nruns + 7) / 8;
+                const int pieces = (int)((R.runBytes + 1023) / 1024);
+                int s2 = 0;
+                while ((nw >> s2) > runsHere && (2 << s2) <= pieces) s2++;
+                R.splitLog2 = s2;
+            }
             p.pf.rows = rows;
             p.pf.wgsPerXcd = perXcd;
         }
