@@ -110,7 +110,11 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
     const int attnTile = headDim == 128 ? 128 : 256;      // positions per attention tile
     f->splitLen = attnTile * ((maxSeq + attnTile * 64 - 1) / (attnTile * 64));      // at most 64 splits
     f->smax = (maxSeq + f->splitLen - 1) / f->splitLen;
-    f->attnHeadsPerWG = maxSeq <= 1024 ? 1 : 0;
+    // query heads of a GQA group per attention workgroup: one while the K/V rows of a layer sit in L2
+    // anyway, two up to 8k positions (four heads a workgroup measured 20 us against 16 us at 2k-4k
+    // positions of the 0.5B and 1.1B shapes, no difference at Llama-3-8B's), the whole group beyond,
+    // where every extra pass over the rows is HBM traffic
+    f->attnHeadsPerWG = maxSeq <= 1024 ? 1 : (maxSeq <= 8192 ? 2 : 0);
     f->amaxParts = 4096;
     {
         size_t floats = (size_t)7 * dim + 2 * (size_t)kvDim + 3 * (size_t)ffnDim + vocabSize +
