@@ -282,11 +282,14 @@ __device__ __forceinline__ RowRef resolve_row(const MvParams& p, int g, int i) {
     return r;
 }
 
-template <int WF, int NR, int KS, int PRO, int EPI, bool EARLY = false>
+template <int WF, int NR, int KS, int PRO, int EPI, bool EARLY = false, bool ONCE = false>
 __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     using F = Fmt<WF>;
     constexpr int LPG = KS == 1 ? 64 : WG;           // lanes per group
-    constexpr int D = NR >= 4 ? 2 : 4;               // items in flight per wave
+    // items in flight per wave; ONCE: the launcher knows that no wave has more than one item (short
+    // rows, one round of workgroups), and the ring with its unrolled slots shrinks to one: a quarter of
+    // the code for a launch that runs every instruction once
+    constexpr int D = ONCE ? 1 : (NR >= 4 ? 2 : 4);
     extern __shared__ float4 a4[];
     __shared__ float red[4];
     __shared__ float part[4][NR];
@@ -793,6 +796,14 @@ static hipError_t launch_t(MvParams& p, int grid, hipStream_t s) {
     if constexpr (KS == 1 && NR == 2 && WF != WF_Q4RAW && (EPI == EPI_QKV || EPI == EPI_SWIGLU || EPI == EPI_RESID)) {
         if (K4 > WG && K4 <= 4 * WG) {                // a variant of its own: the batch costs registers the short vectors need not pay
             hipLaunchKernelGGL((matvec_kernel<WF, NR, KS, PRO, EPI, true>), dim3(grid), dim3(WG), lds, s, p);
+            return hipGetLastError();
+        }
+    }
+    if constexpr (KS == 1 && WF != WF_Q4RAW && (EPI == EPI_QKV || EPI == EPI_SWIGLU || EPI == EPI_RESID) &&
+                  (NR <= 2 || EPI == EPI_SWIGLU)) {
+        const int chunk = WF == WF_Q8 ? 16 : 32;
+        if (p.K / chunk <= 64 && p.ngroups <= grid * 4) {        // one chunk pass a row, one group a wave
+            hipLaunchKernelGGL((matvec_kernel<WF, NR, KS, PRO, EPI, false, true>), dim3(grid), dim3(WG), lds, s, p);
             return hipGetLastError();
         }
     }
