@@ -289,7 +289,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     // items in flight per wave; ONCE: the launcher knows that no wave has more than one item (short
     // rows, one round of workgroups), and the ring with its unrolled slots shrinks to one: a quarter of
     // the code for a launch that runs every instruction once
-    constexpr int D = ONCE ? 1 : (NR >= 4 ? 2 : 4);
+    constexpr int D = (ONCE && KS == 1) ? 1 : (NR >= 4 ? 2 : 4);
     extern __shared__ float4 a4[];
     __shared__ float red[4];
     __shared__ float part[4][NR];
@@ -383,7 +383,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     // and no more bytes than staging reads.  (With KS == 1 every wave would read the whole vector
     // itself, four times the requests: measured slower.)
     constexpr bool CAN_DIRECT = KS == 4 && PRO == PRO_PLAIN;
-    const bool direct = CAN_DIRECT && iters <= 2;
+    const bool direct = CAN_DIRECT && (ONCE || iters <= 2);      // ONCE with KS == 4: the launcher has checked iters <= 2
     float4 avr[2][4];
     float rs = 1.0f;
     if (direct) {
@@ -801,8 +801,13 @@ static hipError_t launch_t(MvParams& p, int grid, hipStream_t s) {
     }
     if constexpr (KS == 1 && WF != WF_Q4RAW && (EPI == EPI_QKV || EPI == EPI_SWIGLU || EPI == EPI_RESID) &&
                   (NR <= 2 || EPI == EPI_SWIGLU)) {
-        const int chunk = WF == WF_Q8 ? 16 : 32;
-        if (p.K / chunk <= 64 && p.ngroups <= grid * 4) {        // one chunk pass a row, one group a wave
+        if (p.K / 16 <= 64 && p.ngroups <= grid * 4) {           // one chunk pass a row (16 weights a lane), one group a wave
+            hipLaunchKernelGGL((matvec_kernel<WF, NR, KS, PRO, EPI, false, true>), dim3(grid), dim3(WG), lds, s, p);
+            return hipGetLastError();
+        }
+    }
+    if constexpr (KS == 4 && NR == 4 && WF != WF_Q4RAW && PRO == PRO_PLAIN && EPI == EPI_RESID) {
+        if (p.K / 16 <= 2 * WG) {                                // registers hold the thread's one or two chunks: no staging path
             hipLaunchKernelGGL((matvec_kernel<WF, NR, KS, PRO, EPI, false, true>), dim3(grid), dim3(WG), lds, s, p);
             return hipGetLastError();
         }
