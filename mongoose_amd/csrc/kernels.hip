@@ -808,7 +808,7 @@ static hipError_t launch_t(MvParams& p, int grid, hipStream_t s) {
     }
     if constexpr (KS == 4 && NR == 4 && WF != WF_Q4RAW && PRO == PRO_PLAIN && EPI == EPI_RESID) {
         if (p.K / 16 <= 2 * WG) {                                // registers hold the thread's one or two chunks: no staging path
-            hipLaunchKernelGGL((matvec_kernel<WF, NR, KS, PRO, EPI, false, true>), dim3(grid), dim3(WG), lds, s, p);
+            hipLaunchKernelGGL((matvec_kernel<WF, NR, KS, PRO, EPI, false, true>), dim3(grid), dim3(WG), 0, s, p);   // nothing is staged in LDS
             return hipGetLastError();
         }
     }
