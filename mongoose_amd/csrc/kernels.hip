@@ -1110,6 +1110,11 @@ __device__ __forceinline__ void prefetch_helper(const PfJob& job, int firstFlat,
     asm volatile("s_waitcnt vmcnt(0)" : "+v"(sink) : : "memory");
 }
 
+// exp(x) for x <= 0 as one multiply and the hardware's 2^x (1 ulp; the product x * log2(e) adds
+// |x| * 2^-24 relative, 2e-6 at x = -20): the library's expf is a dozen instructions, and a thread
+// of the decode attention, at one or two waves a SIMD, pays the latency of every one of them.
+__device__ __forceinline__ float exp_neg(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+
 template <int HD, int GMAX, bool KVH, int AWG = WG>
 __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
     if (blockIdx.y >= p.smax) {                          // uniform: a whole workgroup is either a helper or not
@@ -1222,7 +1227,7 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
             for (int w = 4; w < NWV; w += 4)
                 tm = fmaxf(tm, fmaxf(fmaxf(wred[par][g][w], wred[par][g][w + 1]), fmaxf(wred[par][g][w + 2], wred[par][g][w + 3])));
             const float mNew = fmaxf(m[g], tm);            // finite: every tile holds at least one valid position
-            const float corr = expf(m[g] - mNew);          // first tile: exp(-inf) = 0
+            const float corr = exp_neg(m[g] - mNew);       // first tile: exp(-inf) = 0
             m[g] = mNew;
             float ps = 0.f;
 #pragma unroll
@@ -1230,7 +1235,7 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
             for (int u = 0; u < VU; u++) {
                 if (u * TG >= live) continue;
-                const float pv = expf(sc[g][u] - mNew);    // masked rows: exp(-inf) = 0
+                const float pv = exp_neg(sc[g][u] - mNew); // masked rows: exp(-inf) = 0
                 ps += pv;
 #pragma unroll
                 for (int j = 0; j < NF; j++) {
