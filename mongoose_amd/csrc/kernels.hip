@@ -25,23 +25,45 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_f(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
 }
+// Exchange between the four rows of 16 lanes, in the VALU instead of through the LDS crossbar
+// (ds_bpermute): v_permlane16_swap exchanges the odd rows of its first operand with the even rows of
+// its second, v_permlane32_swap the upper half of the first with the lower half of the second.  With
+// the same value in both operands the two results are (own, partner) or (partner, own) in every lane:
+// their sum / maximum is v combined with the lane 16 (32) away, and since both operations are
+// commutative the bits are those of v op shfl_xor(v, 16 / 32).
+__device__ __forceinline__ void row_swap16(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void row_swap32(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float rows_sum(float v) {      // over lanes l, l^16, l^32, l^48
+    float a = v, b = v;
+    row_swap16(a, b);
+    a = a + b; b = a;
+    row_swap32(a, b);
+    return a + b;
+}
+__device__ __forceinline__ float rows_max(float v) {
+    float a = v, b = v;
+    row_swap16(a, b);
+    a = fmaxf(a, b); b = a;
+    row_swap32(a, b);
+    return fmaxf(a, b);
+}
 __device__ __forceinline__ float wave_sum(float v) {
     v += dpp_f<0xB1>(v);
     v += dpp_f<0x4E>(v);
     v += dpp_f<0x124>(v);
     v += dpp_f<0x128>(v);
-    v += __shfl_xor(v, 16, 64);
-    v += __shfl_xor(v, 32, 64);
-    return v;
+    return rows_sum(v);
 }
 __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, dpp_f<0xB1>(v));
     v = fmaxf(v, dpp_f<0x4E>(v));
     v = fmaxf(v, dpp_f<0x124>(v));
     v = fmaxf(v, dpp_f<0x128>(v));
-    v = fmaxf(v, __shfl_xor(v, 16, 64));
-    v = fmaxf(v, __shfl_xor(v, 32, 64));
-    return v;
+    return rows_max(v);
 }
 // Sum over the 256 threads of a workgroup; every thread gets the result.
 // red: 4 floats of LDS.  Two barriers, so red can be reused right after.
@@ -1051,14 +1073,8 @@ __device__ __forceinline__ float row_sum16(float v) {
     return v;
 }
 // combine a per-thread value over the four row groups (tg) that share a wave
-__device__ __forceinline__ float tg_max(float v) {
-    v = fmaxf(v, __shfl_xor(v, 16, 64));
-    return fmaxf(v, __shfl_xor(v, 32, 64));
-}
-__device__ __forceinline__ float tg_sum(float v) {
-    v += __shfl_xor(v, 16, 64);
-    return v + __shfl_xor(v, 32, 64);
-}
+__device__ __forceinline__ float tg_max(float v) { return rows_max(v); }
+__device__ __forceinline__ float tg_sum(float v) { return rows_sum(v); }
 
 // One float4 of a cache row: fp32 rows are read as they are, fp16 rows as 8 bytes and widened.
 template <bool KVH>
