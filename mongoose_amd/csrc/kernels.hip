@@ -51,6 +51,28 @@ __device__ __forceinline__ float rows_max(float v) {
     row_swap32(a, b);
     return fmaxf(a, b);
 }
+// Greatest value of the wave and, among equals, its lowest index, in every lane: the combination is
+// symmetric and idempotent, so it does not matter which of the two operands is the lane's own.
+__device__ __forceinline__ void argmax_pick(float& v, int& i, float ov, int oi) {
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true); }
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+    float va = v, vb = v;
+    float ia = __builtin_bit_cast(float, i), ib = ia;
+    row_swap32(va, vb); row_swap32(ia, ib);
+    v = va; i = __builtin_bit_cast(int, ia);
+    argmax_pick(v, i, vb, __builtin_bit_cast(int, ib));
+    va = v; vb = v; ia = __builtin_bit_cast(float, i); ib = ia;
+    row_swap16(va, vb); row_swap16(ia, ib);
+    v = va; i = __builtin_bit_cast(int, ia);
+    argmax_pick(v, i, vb, __builtin_bit_cast(int, ib));
+    argmax_pick(v, i, dpp_f<0x128>(v), dpp_i<0x128>(i));     // row_ror:8, row_ror:4, then the quad
+    argmax_pick(v, i, dpp_f<0x124>(v), dpp_i<0x124>(i));
+    argmax_pick(v, i, dpp_f<0x4E>(v), dpp_i<0x4E>(i));
+    argmax_pick(v, i, dpp_f<0xB1>(v), dpp_i<0xB1>(i));
+}
 __device__ __forceinline__ float wave_sum(float v) {
     v += dpp_f<0xB1>(v);
     v += dpp_f<0x4E>(v);
@@ -565,12 +587,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     }
 
     if (EPI == EPI_ARGMAX) {
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            float ov = __shfl_xor(myBestV, o, 64);
-            int oi = __shfl_xor(myBestI, o, 64);
-            if (ov > myBestV || (ov == myBestV && oi < myBestI)) { myBestV = ov; myBestI = oi; }
-        }
+        wave_argmax(myBestV, myBestI);
         if (lane == 0) { bestV[wave] = myBestV; bestI[wave] = myBestI; }
         __syncthreads();
         if (threadIdx.x == 0) {
@@ -662,12 +679,7 @@ __global__ __launch_bounds__(WG) void matvec_rows_q8_kernel(MvParams p) {
         }
     }
     if (EPI == EPI_ARGMAX) {
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            float ov = __shfl_xor(myBestV, o, 64);
-            int oi = __shfl_xor(myBestI, o, 64);
-            if (ov > myBestV || (ov == myBestV && oi < myBestI)) { myBestV = ov; myBestI = oi; }
-        }
+        wave_argmax(myBestV, myBestI);
         if (lane == 0) { bestV[wave] = myBestV; bestI[wave] = myBestI; }
         __syncthreads();
         if (threadIdx.x == 0) {
@@ -754,7 +766,7 @@ __global__ __launch_bounds__(WG) void matvec_rows_q4_kernel(MvParams p) {
         for (int i = 0; i < NR; i++) {
             float a = acc[i];                        // sum over the 32 lanes of this half
             a += dpp_f<0xB1>(a); a += dpp_f<0x4E>(a); a += dpp_f<0x124>(a); a += dpp_f<0x128>(a);
-            a += __shfl_xor(a, 16, 64);
+            { float b = a; row_swap16(a, b); a += b; }
             if (bl == i) val = a;
         }
         const int r = (g * NR + bl) * 2 + half;
@@ -767,12 +779,7 @@ __global__ __launch_bounds__(WG) void matvec_rows_q4_kernel(MvParams p) {
         }
     }
     if (EPI == EPI_ARGMAX) {
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            float ov = __shfl_xor(myBestV, o, 64);
-            int oi = __shfl_xor(myBestI, o, 64);
-            if (ov > myBestV || (ov == myBestV && oi < myBestI)) { myBestV = ov; myBestI = oi; }
-        }
+        wave_argmax(myBestV, myBestI);
         if (lane == 0) { bestV[wave] = myBestV; bestI[wave] = myBestI; }
         __syncthreads();
         if (threadIdx.x == 0) {
