@@ -540,13 +540,13 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
                         RowRef rr = resolve_row<NR, EPI>(p, g, lane < NR ? lane : 0);
                         if (EPI == EPI_SWIGLU) {
                             constexpr int H = NR / 2 > 0 ? NR / 2 : 1;
-                            float u = __shfl(v, lane + H, 64);
+                            const float u = dpp_f<0x100 + H>(v);               // row_shl:H -- lane l reads lane l + H (the up row)
                             if (lane < H && rr.valid) {
                                 float sig = 1.0f / (1.0f + expf(-v));          // mongoose.cu:949-956
                                 p.seg[0].out[rr.row] = v * sig * u;
                             }
                         } else if (EPI == EPI_QKV) {
-                            float v1 = __shfl(v, 1, 64);
+                            const float v1 = dpp_f<0x101>(v);                  // row_shl:1 -- lane 0 reads lane 1 (the pair's second row)
                             if (lane == 0 && rr.valid) {
                                 const MvSeg& sg = p.seg[rr.seg];
                                 float o0, o1;
