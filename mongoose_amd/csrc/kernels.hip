@@ -542,7 +542,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
                             constexpr int H = NR / 2 > 0 ? NR / 2 : 1;
                             const float u = dpp_f<0x100 + H>(v);               // row_shl:H -- lane l reads lane l + H (the up row)
                             if (lane < H && rr.valid) {
-                                float sig = 1.0f / (1.0f + expf(-v));          // mongoose.cu:949-956
+                                float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-v * 1.4426950408889634f));   // mongoose.cu:949-956
                                 p.seg[0].out[rr.row] = v * sig * u;
                             }
                         } else if (EPI == EPI_QKV) {
@@ -1305,7 +1305,8 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
         int h = h0 + g;
         if (nsplit == 1) {
             float4 o;
-            o.x = r.x / lg; o.y = r.y / lg; o.z = r.z / lg; o.w = r.w / lg;
+            const float il = __builtin_amdgcn_rcpf(lg);
+            o.x = r.x * il; o.y = r.y * il; o.z = r.z * il; o.w = r.w * il;
             reinterpret_cast<float4*>(p.out + (size_t)h * HD)[d4] = o;
         } else {
             float* pa = p.pacc + ((size_t)h * p.smax + split) * HD + d4 * 4;
