@@ -178,7 +178,7 @@ __device__ __forceinline__ float stage_activation(const MvParams& p, float4* a4,
     if ((tid & 63) == 0) red[tid >> 6] = ss;
     __syncthreads();
     float tot = (red[0] + red[1]) + (red[2] + red[3]);
-    return 1.0f / sqrtf(tot / (float)p.K + p.eps);
+    return __builtin_amdgcn_rsqf(tot * __builtin_amdgcn_rcpf((float)p.K) + p.eps);   // 1 ulp each; the reference's rsqrtf (mongoose.cu:170) is no closer
 }
 
 // ---------------------------------------------------------------------------
