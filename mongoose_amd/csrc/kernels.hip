@@ -1361,13 +1361,13 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
             for (int u = 0; u < 16; u++) if (s0 + u * NG < nsplit) bm = fmaxf(bm, pmv[u]);
             const float Mn = fmaxf(M, bm);
-            const float c = expf(M - Mn);                           // first batch: exp(-inf) = 0
+            const float c = exp_neg(M - Mn);                           // first batch: exp(-inf) = 0
             den *= c; num.x *= c; num.y *= c; num.z *= c; num.w *= c;
             M = Mn;
 #pragma unroll
             for (int u = 0; u < 16; u++) {
                 if (s0 + u * NG < nsplit) {
-                    const float w = expf(pmv[u] - M);
+                    const float w = exp_neg(pmv[u] - M);
                     den = fmaf(w, plv[u], den);
                     num.x = fmaf(w, pav[u].x, num.x); num.y = fmaf(w, pav[u].y, num.y);
                     num.z = fmaf(w, pav[u].z, num.z); num.w = fmaf(w, pav[u].w, num.w);
@@ -1384,7 +1384,7 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
             float4 nt = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
             for (int k = 0; k < NG; k++) {
-                const float w = expf(cM[k * IT + i] - Mt);           // empty group: exp(-inf) = 0
+                const float w = exp_neg(cM[k * IT + i] - Mt);           // empty group: exp(-inf) = 0
                 const float4 a = cnum[k * IT + i];
                 dt = fmaf(w, cden[k * IT + i], dt);
                 nt.x = fmaf(w, a.x, nt.x); nt.y = fmaf(w, a.y, nt.y); nt.z = fmaf(w, a.z, nt.z); nt.w = fmaf(w, a.w, nt.w);
