@@ -130,14 +130,17 @@ __device__ __forceinline__ int act_slot4(int k4, int nch) {   // k4 = k/4 -> flo
 // All global loads of a prologue are issued before anything waits on them; the
 // caller has already issued its first weight loads, so the activation latency
 // and the weight latency overlap instead of adding up.
-template <int WF, int PRO>
+// SHORT: the caller knows K <= 4 * WG (one float4 a thread at most): no loops, no long-vector path.
+template <int WF, int PRO, bool SHORT = false>
 __device__ __forceinline__ float stage_activation(const MvParams& p, float4* a4, float* red) {
     const int K4 = p.K >> 2;
     const int nch = p.K / 16;
     const int tid = threadIdx.x;
     if (PRO == PRO_PLAIN) {
         const float4* x4 = reinterpret_cast<const float4*>(p.act);
-        if (K4 <= 4 * WG) {
+        if (SHORT) {
+            if (tid < K4) a4[act_slot4<WF>(tid, nch)] = x4[tid];
+        } else if (K4 <= 4 * WG) {
             for (int i = tid; i < K4; i += WG) a4[act_slot4<WF>(i, nch)] = x4[i];
         } else {
             // Long vectors (down projection, K = 14336): every load of a batch is issued before the
@@ -168,7 +171,7 @@ __device__ __forceinline__ float stage_activation(const MvParams& p, float4* a4,
     const float4* x4 = reinterpret_cast<const float4*>(p.act);
     const float4* g4 = reinterpret_cast<const float4*>(p.gain);
     float ss = 0.f;
-    for (int i = tid; i < K4; i += WG) {
+    for (int i = tid; i < (SHORT ? min(K4, WG) : K4); i += WG) {      // SHORT: at most one pass
         float4 v = x4[i], g = g4[i], o;
         ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
         o.x = v.x * g.x; o.y = v.y * g.y; o.z = v.z * g.z; o.w = v.w * g.w;
@@ -347,7 +350,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     const int iters = (nch + LPG - 1) / LPG;
     const int gStart = KS == 1 ? blockIdx.x * 4 + wave : blockIdx.x;
     const int gStep = KS == 1 ? gridDim.x * 4 : gridDim.x;
-    const int myGroups = gStart < p.ngroups ? (p.ngroups - gStart + gStep - 1) / gStep : 0;
+    const int myGroups = gStart >= p.ngroups ? 0 : ((ONCE && KS == 1) ? 1 : (p.ngroups - gStart + gStep - 1) / gStep);
     const int nItems = myGroups * iters;
 
     int pos = 0;
@@ -468,7 +471,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
         __syncthreads();
         if (PRO == PRO_RMS) rs = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)p.K + p.eps);
     } else {
-        rs = stage_activation<WF, PRO>(p, a4, red);
+        rs = stage_activation<WF, PRO, ONCE && KS == 1>(p, a4, red);     // one-item launches have K <= 1024
     }
 
     float myBestV = -INFINITY;
