@@ -336,7 +336,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     // items in flight per wave; ONCE: the launcher knows that no wave has more than one item (short
     // rows, one round of workgroups), and the ring with its unrolled slots shrinks to one: a quarter of
     // the code for a launch that runs every instruction once
-    constexpr int D = (ONCE && KS == 1) ? 1 : (NR >= 4 ? 2 : 4);
+    constexpr int D = (ONCE && KS == 1) ? (EARLY ? 2 : 1) : (NR >= 4 ? 2 : 4);      // with EARLY (K of 1025..2048): two chunk passes
     extern __shared__ float4 a4[];
     __shared__ float red[4];
     __shared__ float part[4][NR];
@@ -471,7 +471,7 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
         __syncthreads();
         if (PRO == PRO_RMS) rs = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)p.K + p.eps);
     } else {
-        rs = stage_activation<WF, PRO, ONCE && KS == 1>(p, a4, red);     // one-item launches have K <= 1024
+        rs = stage_activation<WF, PRO, ONCE && KS == 1 && !EARLY>(p, a4, red);     // one-item launches have K <= 1024
     }
 
     float myBestV = -INFINITY;
@@ -827,6 +827,10 @@ static hipError_t launch_t(MvParams& p, int grid, hipStream_t s) {
     // only for the launch shapes the decode step itself picks: NR 2, fused epilogues
     if constexpr (KS == 1 && NR == 2 && WF != WF_Q4RAW && (EPI == EPI_QKV || EPI == EPI_SWIGLU || EPI == EPI_RESID)) {
         if (K4 > WG && K4 <= 4 * WG) {                // a variant of its own: the batch costs registers the short vectors need not pay
+            if (p.K / 16 <= 128 && p.ngroups <= grid * 4) {          // and one row group a wave in two chunk passes: two load slots, no ring
+                hipLaunchKernelGGL((matvec_kernel<WF, NR, KS, PRO, EPI, true, true>), dim3(grid), dim3(WG), lds, s, p);
+                return hipGetLastError();
+            }
             hipLaunchKernelGGL((matvec_kernel<WF, NR, KS, PRO, EPI, true>), dim3(grid), dim3(WG), lds, s, p);
             return hipGetLastError();
         }
