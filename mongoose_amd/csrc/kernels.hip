@@ -1696,8 +1696,8 @@ __device__ __forceinline__ void copy_rope_row(const RopeCur& rope, int pos) {
 __global__ __launch_bounds__(WG) void argmax_finish_kernel(const float* pv, const int* pi, int nparts, StepState* state,
                                                            const int* prompt, int* history, int historyCap, int vocab,
                                                            RopeCur rope) {
-    __shared__ float bv[WG];
-    __shared__ int bi[WG];
+    __shared__ float bv[WG / 64];
+    __shared__ int bi[WG / 64];
     const int np = state->pos + 1;
     copy_rope_row(rope, np);
     float v = -INFINITY;
@@ -1706,17 +1706,13 @@ __global__ __launch_bounds__(WG) void argmax_finish_kernel(const float* pv, cons
         float ov = pv[i]; int oi = pi[i];
         if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
     }
-    bv[threadIdx.x] = v; bi[threadIdx.x] = idx;
+    // inside the wave without LDS, then the four waves' results through it: one barrier instead of nine
+    wave_argmax(v, idx);
+    if ((threadIdx.x & 63) == 0) { bv[threadIdx.x >> 6] = v; bi[threadIdx.x >> 6] = idx; }
     __syncthreads();
-    for (int o = WG / 2; o > 0; o >>= 1) {
-        if ((int)threadIdx.x < o) {
-            float ov = bv[threadIdx.x + o]; int oi = bi[threadIdx.x + o];
-            if (ov > bv[threadIdx.x] || (ov == bv[threadIdx.x] && oi < bi[threadIdx.x])) { bv[threadIdx.x] = ov; bi[threadIdx.x] = oi; }
-        }
-        __syncthreads();
-    }
     if (threadIdx.x == 0) {
-        int tok = bi[0];
+        for (int w = 1; w < WG / 64; w++) argmax_pick(v, idx, bv[w], bi[w]);
+        int tok = idx;
         if (tok < 0 || tok >= vocab) tok = 0;
         int next = tok;
         if (prompt && np < state->nPrompt) next = prompt[np];
