@@ -184,7 +184,9 @@ int mg_partial_step(mg_ctx* ctx, const float* hiddenIn, int pos, int layerStart,
  * hiddenIn is uploaded when layer == 0; logitsOut as above. */
 int mg_step_layer_resident(mg_ctx* ctx, int layer, int pos, const float* hiddenIn,
                            float* preOut, float* postOut, float* logitsOut);
-/* ExportHidden :235-239. */
+/* ExportHidden :235-239.  The hidden state after mg_partial_step / mg_step_layer_resident /
+ * mg_decode_token.  After launches of the captured graph (mg_graph_launch, mg_generate with
+ * useGraph) the buffer already holds the next token's embedding instead. */
 int mg_export_hidden(mg_ctx* ctx, float* out /* [dim] */);
 
 /* L3 bridge and mailbox, cuda_fused_infer.go:118-131 and :556-737: every context owns a pinned host

@@ -135,6 +135,9 @@ private:
     MvParams gateUpParams(const LayerWeights& L) const;
     MvParams downParams(const LayerWeights& L) const;
     void planPrefetch(int layer, PfJob& job) const;
+    EmbedRef embedRef() const;
+    int primeGraph();
+    bool fuseEmbed = false;      // set while the graphs are captured
     int enqueueLayerPerOp(const LayerWeights& L, int layer, int pos);
     int enqueueEmbed();
     int enqueueToken(bool withHead);      // embed -> layers -> final(+argmax) / advance, all from device state

@@ -647,7 +647,7 @@ int HIPFusedInference::enqueueFinal(bool withArgmax) {
     if (mark(7)) return MG_E_HIP;
     if (withArgmax) {
         if (c.grid > amaxParts) { set_error("argmax partial buffer too small"); return MG_E_STATE; }
-        HIPCHK(launch_argmax_finish(amaxVal, amaxIdx, c.grid, dState, nullptr, dHistory, maxSeq + 1, vocabSize, ropeRef(), stream));
+        HIPCHK(launch_argmax_finish(amaxVal, amaxIdx, c.grid, dState, nullptr, dHistory, maxSeq + 1, vocabSize, ropeRef(), embedRef(), stream));
     }
     return MG_OK;
 }
@@ -781,15 +781,30 @@ int HIPFusedInference::enqueueEmbed() {
 }
 
 // One whole token from the device-resident state.
+// Inside the captured graphs the embedding of the next token is written by the kernel that chooses
+// it (argmax finish / prompt advance), one launch fewer a token: a graph then starts from a hidden
+// buffer that already holds its token's embedding, and whoever sets the state by hand before a
+// graph launch embeds once (primeGraph).  After graph launches the hidden buffer holds that next
+// embedding, not the last hidden state; launches outside the graphs keep the separate embed kernel.
+EmbedRef HIPFusedInference::embedRef() const {
+    EmbedRef e{};
+    if (!fuseEmbed) return e;
+    if (embedKind == 1 || embedKind == 2) { e.kind = embedKind; e.table = embedTable; }
+    else { e.kind = lmHead.kind == WF_Q8 ? 0 : 3; e.table = lmHead.w; e.scales = lmHead.scales; }
+    e.out = hidden[hiddenIdx]; e.dim = dim; e.vocab = vocabSize;
+    return e;
+}
+int HIPFusedInference::primeGraph() { return enqueueEmbed(); }
+
 int HIPFusedInference::enqueueToken(bool withHead) {
-    int rc = enqueueEmbed();
+    int rc = fuseEmbed ? MG_OK : enqueueEmbed();
     if (rc) return rc;
     for (int l = 0; l < nLayers; l++) {
         rc = enqueueLayer(layers[l], l, dState, 0);
         if (rc) return rc;
     }
     if (withHead) return enqueueFinal(true);
-    HIPCHK(launch_advance_prompt(dState, dPrompt, ropeRef(), stream));
+    HIPCHK(launch_advance_prompt(dState, dPrompt, ropeRef(), embedRef(), stream));
     return MG_OK;
 }
 
@@ -836,7 +851,9 @@ int HIPFusedInference::GraphCapture() {
     HIPCHK(hipStreamSynchronize(stream));
     for (int which = 0; which < 2; which++) {
         HIPCHK(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));
+        fuseEmbed = true;
         rc = enqueueToken(which == 0);
+        fuseEmbed = false;
         hipGraph_t g = nullptr;
         hipError_t e = hipStreamEndCapture(stream, &g);
         if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
@@ -854,6 +871,8 @@ int HIPFusedInference::GraphLaunch(int token, int pos, int* nextToken) {
     int rc = GraphCapture();
     if (rc) return rc;
     HIPCHK(launch_set_state(dState, pos, token, 0, 0, ropeRef(), stream));
+    rc = primeGraph();
+    if (rc) return rc;
     HIPCHK(hipGraphLaunch(execFull, stream));
     HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int), hipMemcpyDeviceToHost, stream));
     HIPCHK(hipStreamSynchronize(stream));
@@ -903,6 +922,7 @@ int HIPFusedInference::Generate(const int* prompt, int nPrompt, int nDecode, int
     HIPCHK(hipStreamSynchronize(stream));
     HIPCHK(hipMemcpy(dPrompt, prompt, sizeof(int) * (size_t)nPrompt, hipMemcpyHostToDevice));
     HIPCHK(launch_set_state(dState, 0, prompt[0], 0, nPrompt, ropeRef(), stream));
+    if (useGraph) { rc = primeGraph(); if (rc) return rc; }
     for (int i = 0; i < nPrompt - 1; i++) {
         if (useGraph) HIPCHK(hipGraphLaunch(execPrompt, stream));
         else { rc = enqueueToken(false); if (rc) return rc; }
@@ -924,6 +944,7 @@ int HIPFusedInference::TimedDecode(int token, int pos, int steps, bool useGraph,
     if (rc) return rc;
     if (useGraph) { rc = GraphCapture(); if (rc) return rc; }
     HIPCHK(launch_set_state(dState, pos, token, 0, 0, ropeRef(), stream));
+    if (useGraph) { rc = primeGraph(); if (rc) return rc; }
     HIPCHK(hipStreamSynchronize(stream));
     HIPCHK(hipEventRecord(ev0, stream));
     for (int i = 0; i < steps; i++) {
@@ -1116,6 +1137,7 @@ int HIPFusedInference::GeneratePrefill(const int* prompt, int nPrompt, int nDeco
     if (rc) return rc;
     rc = Prefill(prompt, nPrompt, 0, nullptr, nullptr, nullptr);
     if (rc) return rc;
+    if (nDecode > 1) { rc = primeGraph(); if (rc) return rc; }
     for (int i = 1; i < nDecode; i++) HIPCHK(hipGraphLaunch(execFull, stream));
     HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int) * (size_t)nDecode, hipMemcpyDeviceToHost, stream));
     HIPCHK(hipStreamSynchronize(stream));

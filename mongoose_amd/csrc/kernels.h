@@ -143,11 +143,14 @@ hipError_t launch_embed_token(int kind, const void* table, const float* scales, 
 // into rope.cur (cos then sin, headDim/2 each), so that the next token's
 // kernels read it without first waiting for the position.
 struct RopeCur { const float* cosTab; const float* sinTab; float* cur; int half; int maxSeq; };
+// Where the token-advancing kernels also leave the embedding row of the token they have just chosen
+// (out == NULL: they do not).  kind as in launch_embed_token.
+struct EmbedRef { int kind; const void* table; const float* scales; float* out; int dim; int vocab; };
 hipError_t launch_argmax_finish(const float* pv, const int* pi, int nparts, StepState* state,
-                                const int* prompt, int* history, int historyCap, int vocab, RopeCur rope, hipStream_t s);
+                                const int* prompt, int* history, int historyCap, int vocab, RopeCur rope, EmbedRef emb, hipStream_t s);
 hipError_t launch_set_state(StepState* state, int pos, int token, int count, int nPrompt, RopeCur rope, hipStream_t s);
 // Advance state without an lm_head (prompt positions): pos++, token = prompt[pos].
-hipError_t launch_advance_prompt(StepState* state, const int* prompt, RopeCur rope, hipStream_t s);
+hipError_t launch_advance_prompt(StepState* state, const int* prompt, RopeCur rope, EmbedRef emb, hipStream_t s);
 
 // Pipeline-stage mailbox (SignalMailbox, cuda_fused_infer.go:558): stores `value` into a counter in
 // host-visible memory once everything queued before it on the stream has finished.

@@ -1652,6 +1652,14 @@ hipError_t launch_fill_zero(void* ptr, size_t bytes, hipStream_t s) {
 // ---------------------------------------------------------------------------
 // Token-level stages that the reference leaves to its caller
 // ---------------------------------------------------------------------------
+__device__ __forceinline__ void embed_element(int kind, const void* table, const float* scales, int tok, float* x, int dim, int vocab, int i);
+// Row `tok` of the table into e.out, by the whole workgroup.
+__device__ __forceinline__ void embed_gather(const EmbedRef& e, int tok) {
+    if (!e.out) return;
+    if (tok < 0) tok = 0;
+    if (tok >= e.vocab) tok = e.vocab - 1;
+    for (int i = threadIdx.x; i < e.dim; i += blockDim.x) embed_element(e.kind, e.table, e.scales, tok, e.out, e.dim, e.vocab, i);
+}
 __global__ void embed_token_kernel(int kind, const void* table, const float* scales, const StepState* state,
                                    float* x, int dim, int vocab) {
     int tok = state->token;
@@ -1659,6 +1667,9 @@ __global__ void embed_token_kernel(int kind, const void* table, const float* sca
     if (tok >= vocab) tok = vocab - 1;
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= dim) return;
+    embed_element(kind, table, scales, tok, x, dim, vocab, i);
+}
+__device__ __forceinline__ void embed_element(int kind, const void* table, const float* scales, int tok, float* x, int dim, int vocab, int i) {
     if (kind == 0) {
         const signed char* q = static_cast<const signed char*>(table) + (size_t)tok * dim;
         x[i] = (float)q[i] * scales[tok];
@@ -1695,9 +1706,10 @@ __device__ __forceinline__ void copy_rope_row(const RopeCur& rope, int pos) {
 
 __global__ __launch_bounds__(WG) void argmax_finish_kernel(const float* pv, const int* pi, int nparts, StepState* state,
                                                            const int* prompt, int* history, int historyCap, int vocab,
-                                                           RopeCur rope) {
+                                                           RopeCur rope, EmbedRef emb) {
     __shared__ float bv[WG / 64];
     __shared__ int bi[WG / 64];
+    __shared__ int nextTok;
     const int np = state->pos + 1;
     copy_rope_row(rope, np);
     float v = -INFINITY;
@@ -1721,11 +1733,16 @@ __global__ __launch_bounds__(WG) void argmax_finish_kernel(const float* pv, cons
         state->count = cnt + 1;
         state->token = next;
         state->pos = np;
+        nextTok = next;
+    }
+    if (emb.out) {                                   // uniform: the next step's embedding, one launch saved
+        __syncthreads();
+        embed_gather(emb, nextTok);
     }
 }
 hipError_t launch_argmax_finish(const float* pv, const int* pi, int nparts, StepState* state, const int* prompt,
-                                int* history, int historyCap, int vocab, RopeCur rope, hipStream_t s) {
-    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(WG), 0, s, pv, pi, nparts, state, prompt, history, historyCap, vocab, rope);
+                                int* history, int historyCap, int vocab, RopeCur rope, EmbedRef emb, hipStream_t s) {
+    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(WG), 0, s, pv, pi, nparts, state, prompt, history, historyCap, vocab, rope, emb);
     return hipGetLastError();
 }
 
@@ -1738,16 +1755,19 @@ hipError_t launch_set_state(StepState* state, int pos, int token, int count, int
     return hipGetLastError();
 }
 
-__global__ void advance_prompt_kernel(StepState* state, const int* prompt, RopeCur rope) {
+__global__ void advance_prompt_kernel(StepState* state, const int* prompt, RopeCur rope, EmbedRef emb) {
     int np = state->pos + 1;
     copy_rope_row(rope, np);
+    const int tok = np < state->nPrompt ? prompt[np] : state->token;      // every thread reads the same words
+    if (emb.out) embed_gather(emb, tok);
+    __syncthreads();                                 // every wave has read the old position before it changes
     if (threadIdx.x == 0) {
         state->pos = np;
-        if (np < state->nPrompt) state->token = prompt[np];
+        state->token = tok;
     }
 }
-hipError_t launch_advance_prompt(StepState* state, const int* prompt, RopeCur rope, hipStream_t s) {
-    hipLaunchKernelGGL(advance_prompt_kernel, dim3(1), dim3(64), 0, s, state, prompt, rope);
+hipError_t launch_advance_prompt(StepState* state, const int* prompt, RopeCur rope, EmbedRef emb, hipStream_t s) {
+    hipLaunchKernelGGL(advance_prompt_kernel, dim3(1), dim3(emb.out ? WG : 64), 0, s, state, prompt, rope, emb);
     return hipGetLastError();
 }
 
