@@ -1063,9 +1063,10 @@ hipError_t launch_matvec_generic_q8(const float* act, const void* w, const float
 // a thread holds the tile's rows tg + u*16.  A score is the lane's partial
 // product reduced over the row's lanes by DPP; every lane
 // of a row ends up with the score, which is exactly where P.V needs it -- the
-// probabilities never leave registers.  Per tile there is one barrier (the
-// tile maximum across waves); the running sum and the output stay per-thread
-// partials over the thread's own rows and are reduced once at the end.
+// probabilities never leave registers.  A wave keeps its own running maximum
+// (no barrier per tile); the running sum and the output stay per-thread
+// partials over the thread's own rows and are reduced once at the end, where
+// the waves' partials are weighted by exp(wave maximum - workgroup maximum).
 // With several splits the last workgroup of a column to finish combines the
 // partials, so the output is always the final [dim] vector.
 // ---------------------------------------------------------------------------
@@ -1157,7 +1158,7 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
     constexpr int TG = AWG / LPR;      // rows in flight per load step (16 or 32)
     constexpr int VU = 16 / NF / (AWG / WG);   // rows per thread and tile
     constexpr int TILE = TG * VU;      // positions per tile (256 for head size 64, 128 for 128)
-    __shared__ float wred[2][GMAX][NWV];
+    __shared__ float wred[GMAX][NWV];                  // the waves' running maxima, for the final combination
     __shared__ float4 accbuf[NWV][GMAX][HD / 4];
     __shared__ float lbuf[NWV][GMAX];
     __shared__ int lastFlag;
@@ -1205,7 +1206,7 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
     const int t1 = p.splitLen > 0 ? min(len, t0 + p.splitLen) : len;
 
     const float scale = 1.0f / sqrtf((float)HD);     // mongoose.cu:867 rsqrtf(headDim)
-    float m[GMAX], l[GMAX];                           // m: workgroup-wide running max; l, acc: this thread's rows only
+    float m[GMAX], l[GMAX];                           // m: the wave's running max; l, acc: this thread's rows only
     float4 acc[GMAX][NF];
 #pragma unroll
     for (int g = 0; g < GMAX; g++) {
@@ -1214,7 +1215,6 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
         for (int j = 0; j < NF; j++) acc[g][j] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
 
-    int par = 0;
     for (int tile = t0; tile < t1; tile += TILE) {
         if (tile != t0) {
 #pragma unroll
@@ -1226,7 +1226,7 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
             }
         }
         const int live = t1 - tile;                        // positions of this tile that exist (uniform)
-        float sc[GMAX][VU];
+        float sc[GMAX][VU], tmaxg[GMAX];
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
             float tmax = -INFINITY;
@@ -1246,18 +1246,13 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
                 sc[g][u] = (tile + tg + u * TG < t1) ? d * scale : -INFINITY;
                 tmax = fmaxf(tmax, sc[g][u]);
             }
-            tmax = tg_max(tmax);
-            if ((tid & 63) == 0) wred[par][g][wave] = tmax;
+            tmaxg[g] = tg_max(tmax);                       // the wave's maximum: no other wave is asked
         }
-        __syncthreads();
 #pragma unroll
         for (int g = 0; g < GMAX; g++) {
-            float tm = fmaxf(fmaxf(wred[par][g][0], wred[par][g][1]), fmaxf(wred[par][g][2], wred[par][g][3]));
-#pragma unroll
-            for (int w = 4; w < NWV; w += 4)
-                tm = fmaxf(tm, fmaxf(fmaxf(wred[par][g][w], wred[par][g][w + 1]), fmaxf(wred[par][g][w + 2], wred[par][g][w + 3])));
-            const float mNew = fmaxf(m[g], tm);            // finite: every tile holds at least one valid position
-            const float corr = exp_neg(m[g] - mNew);       // first tile: exp(-inf) = 0
+            const float mNew = fmaxf(m[g], tmaxg[g]);
+            const float mRef = mNew == -INFINITY ? 0.f : mNew;     // a wave none of whose rows exist yet
+            const float corr = exp_neg(m[g] - mRef);       // first tile: exp(-inf) = 0
             m[g] = mNew;
             float ps = 0.f;
 #pragma unroll
@@ -1265,7 +1260,7 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
             for (int u = 0; u < VU; u++) {
                 if (u * TG >= live) continue;
-                const float pv = exp_neg(sc[g][u] - mNew); // masked rows: exp(-inf) = 0
+                const float pv = exp_neg(sc[g][u] - mRef); // masked rows: exp(-inf) = 0
                 ps += pv;
 #pragma unroll
                 for (int j = 0; j < NF; j++) {
@@ -1277,7 +1272,6 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
             }
             l[g] = l[g] * corr + ps;
         }
-        par ^= 1;                                          // the next tile's maxima go to the other buffer
     }
 
     // ---- reduce the per-thread partials over the row groups: in the wave, then across waves ----
@@ -1290,25 +1284,26 @@ __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {
             if ((tid & 63) < LPR) accbuf[wave][g][j * 16 + dl] = acc[g][j];
         }
         l[g] = tg_sum(l[g]);
-        if ((tid & 63) == 0) lbuf[wave][g] = l[g];
+        if ((tid & 63) == 0) { lbuf[wave][g] = l[g]; wred[g][wave] = m[g]; }
     }
     __syncthreads();
     constexpr int F4 = HD / 4;                             // float4s of a head
     for (int i = tid; i < gn * F4; i += AWG) {
         int g = i / F4, d4 = i % F4;
-        float4 r = accbuf[0][g][d4];
+        // every wave kept its own running maximum: the workgroup's is the greatest of them (finite, the
+        // split holds at least one position), and a wave's sums count with exp(its maximum - that)
+        float mg_ = wred[g][0];
 #pragma unroll
-        for (int k = 1; k < NWV; k++) {
-            float4 a = accbuf[k][g][d4];
-            r.x += a.x; r.y += a.y; r.z += a.z; r.w += a.w;
+        for (int k = 1; k < NWV; k++) mg_ = fmaxf(mg_, wred[g][k]);
+        float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+        float lg = 0.f;                                    // lbuf holds lane 0's column of each wave: every row's probability exactly once
+#pragma unroll
+        for (int k = 0; k < NWV; k++) {
+            const float w = exp_neg(wred[g][k] - mg_);     // a wave without rows: exp(-inf) = 0
+            const float4 a = accbuf[k][g][d4];
+            r.x = fmaf(w, a.x, r.x); r.y = fmaf(w, a.y, r.y); r.z = fmaf(w, a.z, r.z); r.w = fmaf(w, a.w, r.w);
+            lg = fmaf(w, lbuf[k][g], lg);
         }
-        // lbuf holds lane 0's column of each wave: every row's probability exactly once
-        float lg = (lbuf[0][g] + lbuf[1][g]) + (lbuf[2][g] + lbuf[3][g]);
-#pragma unroll
-        for (int w = 4; w < NWV; w += 4) lg += (lbuf[w][g] + lbuf[w + 1][g]) + (lbuf[w + 2][g] + lbuf[w + 3][g]);
-        float mg_ = m[0];
-#pragma unroll
-        for (int k = 1; k < GMAX; k++) if (g == k) mg_ = m[k];
         int h = h0 + g;
         if (nsplit == 1) {
             float4 o;
