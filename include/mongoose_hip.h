@@ -66,6 +66,14 @@ void mongoose_rmsnorm_out(const float* in, float* out, const float* w, int seqLe
  * parameter; the CUDA kernel hard-codes 1e-6). */
 void mongoose_rmsnorm_out_eps(const float* in, float* out, const float* w, int seqLen, int dim, float eps, void* stream);
 
+/* kernels.go:12, mongoose.cu:16-50.  In place: x = x * rsqrt(mean(x^2)+1e-6) * w, per row of [seqLen, dim]
+ * (what TRMSNorm binds, kernel_tensor.go:23-26). */
+void mongoose_rmsnorm(float* x, const float* w, int seqLen, int dim, void* stream);
+/* kernels.go:20, mongoose.cu:372-404.  out = rmsnorm(a + b, w), eps 1e-6; out may be a or b.
+ * The _eps form takes eps as an argument (as mongoose_rmsnorm_out_eps does). */
+void mongoose_fused_add_rmsnorm(const float* a, const float* b, float* out, const float* w, int seqLen, int dim, void* stream);
+void mongoose_fused_add_rmsnorm_eps(const float* a, const float* b, float* out, const float* w, int seqLen, int dim, float eps, void* stream);
+
 /* kernels.go:62, mongoose.cu:1556-1595.  out[r] = sum_k act[k]*w[r,k] * (scales[r]/127):
  * the reference kernel's convention, `scales` holding per-row absmax
  * (producer: mongoose_requant_fp32_to_int8, mongoose.cu:1501-1545). */
@@ -74,6 +82,11 @@ void mongoose_q8_matvec(const float* act, const void* w_int8, const float* scale
  * scales[r] = absmax/127 as quantizeQ8 stores them (cuda_fused_infer.go:373-374,
  * metal_impl_darwin.m:5533-5535).  This is what the mg_* context uses. */
 void mongoose_q8_matvec_rowscale(const float* act, const void* w_int8, const float* scales, float* out, int N, int K, void* stream);
+
+/* kernels.go:63, mongoose.cu:1598-1640.  Per-row-scale 4-bit weights (what TQ8Matvec binds for
+ * Q8Weight.Q4, kernel_tensor.go:34-40; not GGUF Q4_0): w_packed is [N, K/2] bytes, low nibble =
+ * element 2k, high nibble = element 2k+1, value (nib-8) * scales[r]/7.  K even. */
+void mongoose_q4_matvec(const float* act, const void* w_packed, const float* scales, float* out, int N, int K, void* stream);
 
 /* kernels.go:65.  w is raw GGUF block_q4_0 (18-byte blocks: fp16 d, 16 bytes of
  * nibbles; low nibble = element j, high nibble = element j+16; value (nib-8)*d),
@@ -288,7 +301,10 @@ uint64_t mg_kv_bytes_at(const mg_ctx* ctx, int pos);
 /* CUDAStreamInfer, cuda_fused_stream.go:98-726                         */
 /* ------------------------------------------------------------------ */
 typedef struct mg_stream mg_stream;
-/* StreamBuild :127-198: two device weight sets + two pinned staging buffers. */
+/* StreamBuild :127-198: two device weight sets + two pinned staging buffers.  The object uses the
+ * context's stream and scratch; destroy it before the context.  If the context goes first the
+ * object becomes inert: mg_stream_forward_token returns MG_E_STATE and mg_stream_destroy still
+ * releases its own buffers. */
 mg_stream* mg_stream_build(mg_ctx* ctx);
 void       mg_stream_destroy(mg_stream* s);
 /* StreamForwardToken :559-670.  layerPtrs[i*12+k] are host pointers to the

@@ -67,6 +67,23 @@ void mongoose_rmsnorm_out(const float* in, float* out, const float* w, int seqLe
     mongoose_rmsnorm_out_eps(in, out, w, seqLen, dim, 1e-6f, stream);     // mongoose.cu:170
 }
 
+// kernels.go:12, mongoose.cu:16-50: in place, eps 1e-6 (mongoose.cu:47).
+void mongoose_rmsnorm(float* x, const float* w, int seqLen, int dim, void* stream) {
+    note(mg::launch_rmsnorm_out(x, x, w, seqLen, dim, 1e-6f, S(stream)));     // every thread reads an element before it writes it
+}
+// kernels.go:20, mongoose.cu:372-404.
+void mongoose_fused_add_rmsnorm(const float* a, const float* b, float* out, const float* w, int seqLen, int dim, void* stream) {
+    note(mg::launch_fused_add_rmsnorm(a, b, out, w, seqLen, dim, 1e-6f, S(stream)));
+}
+void mongoose_fused_add_rmsnorm_eps(const float* a, const float* b, float* out, const float* w, int seqLen, int dim, float eps,
+                                    void* stream) {
+    note(mg::launch_fused_add_rmsnorm(a, b, out, w, seqLen, dim, eps, S(stream)));
+}
+// kernels.go:63, mongoose.cu:1598-1640.
+void mongoose_q4_matvec(const float* act, const void* w_packed, const float* scales, float* out, int N, int K, void* stream) {
+    note(mg::launch_q4_rowscale_matvec(act, w_packed, scales, out, N, K, S(stream)));
+}
+
 static void q8_matvec_any(const float* act, const void* w, const float* scales, float* out, int N, int K, int div127, void* stream) {
     if (N <= 0 || K <= 0) return;
     if (K % 16 == 0 && K * 4 <= 64 * 1024 && aligned16(w) && aligned16(act)) {

@@ -99,6 +99,9 @@ public:
     float eps;
 
     // used by the streaming front end
+    // Objects that keep a pointer to this context (stream front ends) register where they keep it; the
+    // destructor clears those pointers, so that destroying the context first leaves them inert.
+    std::vector<HIPFusedInference**> backrefs;
     hipStream_t stream = nullptr;
     std::vector<LayerWeights> layers;
     std::vector<float*> kCache, vCache;
@@ -134,7 +137,7 @@ private:
     MvParams woParams(const LayerWeights& L) const;
     MvParams gateUpParams(const LayerWeights& L) const;
     MvParams downParams(const LayerWeights& L) const;
-    void planPrefetch(int layer, PfJob& job) const;
+    void planPrefetch(const LayerWeights& L, const LayerWeights* next, int layer, PfJob& job) const;
     EmbedRef embedRef() const;
     int primeGraph();
     bool fuseEmbed = false;      // set while the graphs are captured
@@ -183,3 +186,6 @@ private:
 };
 
 }  // namespace mg
+
+// the opaque handle of the C ABI
+struct mg_ctx { mg::HIPFusedInference* f; };

@@ -122,7 +122,8 @@ HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int n
         size_t ints = (size_t)f->amaxParts + 2 * ((size_t)maxSeq + 1) + 64 + attention_columns(nHeads, nKVHeads, 1);
         size_t bytes = (floats + ints) * 4 + 64 * 256;
         if (f->scratch.init(bytes) != 0) return fail("scratch alloc failed");
-        if (hipMemset(f->scratch.base, 0, bytes) != hipSuccess) return fail("scratch clear failed");
+        if (hipMemsetAsync(f->scratch.base, 0, bytes, f->stream) != hipSuccess || hipStreamSynchronize(f->stream) != hipSuccess)
+            return fail("scratch clear failed");
     }
     auto takeF = [&](float*& p, size_t n) { p = static_cast<float*>(f->scratch.take(n * 4)); return p != nullptr; };
     auto takeI = [&](int*& p, size_t n) { p = static_cast<int*>(f->scratch.take(n * 4)); return p != nullptr; };
@@ -201,6 +202,7 @@ int HIPFusedInference::slotAddr(int idx, char** out) {
 }
 
 HIPFusedInference::~HIPFusedInference() {
+    for (HIPFusedInference** ref : backrefs) *ref = nullptr;
     if (stream) (void)hipStreamSynchronize(stream);
     invalidateGraphs();
     scratch.release();
@@ -374,7 +376,9 @@ int HIPFusedInference::SetLayerRange(int layerStart, int layerEnd) {
     Slab& sl = kvSlabs.back();
     int rc = sl.init(per * 2 * need);
     if (rc) { kvSlabs.pop_back(); return rc; }
-    HIPCHK(hipMemset(sl.base, 0, sl.size));
+    // on the stream the kernels run on (a non-blocking stream does not order itself behind the NULL stream)
+    HIPCHK(hipMemsetAsync(sl.base, 0, sl.size, stream));
+    HIPCHK(hipStreamSynchronize(stream));
     for (int l = layerStart; l < layerEnd && l < nLayers; l++) {
         if (kCache[l]) continue;
         kCache[l] = static_cast<float*>(sl.take(per));
@@ -399,11 +403,13 @@ int HIPFusedInference::SetKVFormat(int fmt) {
 // here (a fresh sequence never reads V rows it has not written).
 int HIPFusedInference::ResetKV() {
     if (!built) return MG_E_NOT_BUILT;
-    HIPCHK(hipStreamSynchronize(stream));
+    // on the context's own stream: it is non-blocking, so a fill on the NULL stream would not be ordered
+    // before the launches that follow; ResetKV is never part of a captured graph
     for (int l = 0; l < nLayers; l++) {
-        if (kCache[l]) HIPCHK(hipMemset(kCache[l], 0, (size_t)maxSeq * kvDim * (kvHalf ? 2 : 4)));
-        if (vCache[l]) HIPCHK(hipMemset(vCache[l], 0, (size_t)maxSeq * kvDim * (kvHalf ? 2 : 4)));
+        if (kCache[l]) HIPCHK(hipMemsetAsync(kCache[l], 0, (size_t)maxSeq * kvDim * (kvHalf ? 2 : 4), stream));
+        if (vCache[l]) HIPCHK(hipMemsetAsync(vCache[l], 0, (size_t)maxSeq * kvDim * (kvHalf ? 2 : 4), stream));
     }
+    HIPCHK(hipStreamSynchronize(stream));
     return MG_OK;
 }
 
@@ -538,15 +544,14 @@ MvParams HIPFusedInference::downParams(const LayerWeights& L) const {
 // workgroups read, which fills the idle start of that launch -- and ends the list.  A layer small
 // enough for its successor's Wo to stay gets that one instead of its own (which came with the
 // launch before): it need not be in by the end of this launch.
-void HIPFusedInference::planPrefetch(int layer, PfJob& job) const {
+void HIPFusedInference::planPrefetch(const LayerWeights& L, const LayerWeights* next, int layer, PfJob& job) const {
     job = PfJob{};
     if (execMode != 1) return;
     const size_t budget = (size_t)12 << 20;       // measured: 10.6 MB make the attention launch 0.3 us longer, 15 MB 3 us
     const size_t l2 = (size_t)24 << 20;           // of 8 x 4 MB
-    const LayerWeights& L = layers[layer];
     const LayerWeights* N = nullptr;
-    if (layer + 1 < nLayers) {
-        const LayerWeights& C = layers[layer + 1];
+    if (next && layer + 1 < nLayers) {
+        const LayerWeights& C = *next;
         const bool uniform = C.wq.kind == C.wk.kind && C.wk.kind == C.wv.kind && C.gate.kind == C.up.kind;
         if (layerComplete(C) && uniform && kCache[layer + 1]) N = &C;
     }
@@ -600,7 +605,10 @@ int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const
         a.kvDim = kvDim; a.nHeads = nHeads; a.nKVHeads = nKVHeads; a.headDim = headDim;
         a.smax = smax; a.splitLen = splitLen; a.headsPerWG = attnHeadsPerWG;
         a.pm = pm; a.pl = pl; a.pacc = pacc; a.counters = attnCounters; a.out = attnOut;
-        planPrefetch(layer, a.pf);
+        // the weights this launch was given (a streamed layer's device copy is not the resident slot), and the
+        // resident successor only when this layer is the resident one itself
+        const bool resident = &L == &layers[layer];
+        planPrefetch(L, resident && layer + 1 < nLayers ? &layers[layer + 1] : nullptr, layer, a.pf);
         HIPCHK(launch_attention(a, stream));
     }
     if (mark(3)) return MG_E_HIP;
@@ -1151,7 +1159,6 @@ int HIPFusedInference::GeneratePrefill(const int* prompt, int nPrompt, int nDeco
 // C entry points
 // ---------------------------------------------------------------------------
 using mg::HIPFusedInference;
-struct mg_ctx { HIPFusedInference* f; };
 
 extern "C" {
 

@@ -121,6 +121,8 @@ hipError_t launch_attention(const AttnParams& p, hipStream_t s);
 int attention_columns(int nHeads, int nKVHeads, int headsPerWG);
 
 hipError_t launch_rmsnorm_out(const float* in, float* out, const float* w, int seqLen, int dim, float eps, hipStream_t s);
+hipError_t launch_fused_add_rmsnorm(const float* a, const float* b, float* out, const float* w, int seqLen, int dim, float eps, hipStream_t s);
+hipError_t launch_q4_rowscale_matvec(const float* act, const void* w, const float* scales, float* out, int N, int K, hipStream_t s);
 hipError_t launch_rope(float* x, const float* cosTab, const float* sinTab, int seqLen, int dim, int headDim, int nHeads, hipStream_t s);
 hipError_t launch_kv_cache_write(float* cache, const float* src, int pos, int kvDim, hipStream_t s);
 hipError_t launch_kv_cache_write_f16(void* cache, const float* src, int pos, int kvDim, hipStream_t s);

@@ -1498,6 +1498,75 @@ hipError_t launch_rmsnorm_out(const float* in, float* out, const float* w, int s
     return hipGetLastError();
 }
 
+// mongoose.cu:372-404: out = rmsnorm(a + b, w).  The sum goes into out first and is scaled in place,
+// so out may be a or b.
+__global__ __launch_bounds__(WG) void fused_add_rmsnorm_kernel(const float* a, const float* b, float* out, const float* w,
+                                                               int dim, float eps) {
+    __shared__ float red[4];
+    const float* ar = a + (size_t)blockIdx.x * dim;
+    const float* br = b + (size_t)blockIdx.x * dim;
+    float* o = out + (size_t)blockIdx.x * dim;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < dim; i += WG) {
+        const float v = ar[i] + br[i];
+        o[i] = v;
+        ss += v * v;
+    }
+    float tot = block_sum(ss, red);
+    float rs = 1.0f / sqrtf(tot / (float)dim + eps);
+    for (int i = threadIdx.x; i < dim; i += WG) o[i] = o[i] * rs * w[i];      // a thread re-reads only what it wrote
+}
+hipError_t launch_fused_add_rmsnorm(const float* a, const float* b, float* out, const float* w, int seqLen, int dim, float eps,
+                                    hipStream_t s) {
+    if (seqLen <= 0) return hipSuccess;
+    hipLaunchKernelGGL(fused_add_rmsnorm_kernel, dim3(seqLen), dim3(WG), 0, s, a, b, out, w, dim, eps);
+    return hipGetLastError();
+}
+
+// mongoose.cu:1598-1630: per-row-scale 4-bit weights, two per byte in sequence (low nibble = element
+// 2k, high nibble = element 2k+1), value (nib - 8) * (scales[row] / 7).  One wave per row; a lane
+// takes four bytes (eight weights) at a time when rows are word-aligned, single bytes otherwise.
+__global__ __launch_bounds__(WG) void q4_rowscale_matvec_kernel(const float* act, const unsigned char* w, const float* scales,
+                                                                float* out, int N, int K, int words) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= N) return;
+    const int halfK = K / 2;
+    const unsigned char* wr = w + (size_t)row * halfK;
+    float sum = 0.f;
+    int k0 = 0;
+    if (words) {
+        const unsigned* w4 = reinterpret_cast<const unsigned*>(wr);
+        const int nw = halfK / 4;
+        for (int i = lane; i < nw; i += 64) {
+            const unsigned q = w4[i];
+            const float* a = act + (size_t)i * 8;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const unsigned byte = (q >> (8 * b)) & 0xffu;
+                sum = fmaf(a[2 * b], (float)((int)(byte & 0xfu) - 8), sum);
+                sum = fmaf(a[2 * b + 1], (float)((int)(byte >> 4) - 8), sum);
+            }
+        }
+        k0 = nw * 4;
+    }
+    for (int k = k0 + lane; k < halfK; k += 64) {
+        const unsigned byte = wr[k];
+        sum = fmaf(act[2 * k], (float)((int)(byte & 0xfu) - 8), sum);
+        sum = fmaf(act[2 * k + 1], (float)((int)(byte >> 4) - 8), sum);
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) out[row] = sum * (scales[row] / 7.0f);
+}
+hipError_t launch_q4_rowscale_matvec(const float* act, const void* w, const float* scales, float* out, int N, int K, hipStream_t s) {
+    if (N <= 0 || K <= 0) return hipSuccess;
+    if (K & 1) return hipErrorInvalidValue;
+    const int words = ((K / 2) % 4 == 0 && ((uintptr_t)w & 3) == 0) ? 1 : 0;
+    hipLaunchKernelGGL(q4_rowscale_matvec_kernel, dim3((N + 3) / 4), dim3(WG), 0, s, act, static_cast<const unsigned char*>(w),
+                       scales, out, N, K, words);
+    return hipGetLastError();
+}
+
 // mongoose.cu:991-1006
 __global__ void rope_kernel(float* x, const float* cosTab, const float* sinTab, int dim, int headDim, int nHeads) {
     int pos = blockIdx.x;
@@ -1633,7 +1702,18 @@ __global__ void fill_zero_kernel(unsigned* p, size_t nwords, unsigned char* tail
 }
 hipError_t launch_fill_zero(void* ptr, size_t bytes, hipStream_t s) {
     if (bytes == 0) return hipSuccess;
-    if (((uintptr_t)ptr & 3) != 0) return hipMemsetAsync(ptr, 0, bytes, s);
+    if (((uintptr_t)ptr & 3) != 0) {
+        // unaligned start: the bytes up to the next word boundary by the same kernel (a fill kernel, not a
+        // memset node, so that the call stays safe inside a captured graph), then the aligned rest
+        const size_t head = 4 - ((uintptr_t)ptr & 3);
+        const size_t n = head < bytes ? head : bytes;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(WG), 0, s, static_cast<unsigned*>(nullptr), (size_t)0,
+                           static_cast<unsigned char*>(ptr), (int)n);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess || n == bytes) return e;
+        ptr = static_cast<unsigned char*>(ptr) + n;
+        bytes -= n;
+    }
     size_t nwords = bytes / 4;
     int ntail = (int)(bytes % 4);
     size_t blocks = (nwords + WG - 1) / WG;

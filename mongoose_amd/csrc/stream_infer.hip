@@ -49,6 +49,10 @@ public:
     LayerWeights view[2];
 
     ~HIPStreamInfer() {
+        if (f) {                                   // still alive: no longer tell it about this object
+            auto& br = f->backrefs;
+            br.erase(std::remove(br.begin(), br.end(), &f), br.end());
+        }
         if (f && f->stream) (void)hipStreamSynchronize(f->stream);
         if (uploadStream) { (void)hipStreamSynchronize(uploadStream); (void)hipStreamDestroy(uploadStream); }
         for (int i = 0; i < 2; i++) {
@@ -146,6 +150,7 @@ public:
     // StreamForwardToken, cuda_fused_stream.go:559-670
     int forward(int pos, const float* embHidden, int nLayers, const void* const* layerPtrs, const int32_t* layerSizes,
                 float* logitsOut) {
+        if (!f) { set_error("StreamForwardToken: the context this object was built on has been destroyed"); return MG_E_STATE; }
         if (!embHidden || !layerPtrs || !layerSizes) { set_error("StreamForwardToken: NULL argument"); return MG_E_ARG; }
         if (nLayers < 1 || nLayers > f->nLayers || pos < 0 || pos >= f->maxSeq) { set_error("StreamForwardToken: bad nLayers or pos"); return MG_E_ARG; }
         for (int l = 0; l < nLayers; l++)
@@ -196,7 +201,6 @@ public:
 
 }  // namespace mg
 
-struct mg_ctx { mg::HIPFusedInference* f; };
 struct mg_stream { mg::HIPStreamInfer* s; };
 
 extern "C" {
@@ -206,6 +210,7 @@ mg_stream* mg_stream_build(mg_ctx* ctx) {
     if (ctx->f->dim % 32 || ctx->f->ffnDim % 32) { mg::set_error("mg_stream_build: Q4_0 needs dims % 32 == 0"); return nullptr; }
     auto* s = new mg::HIPStreamInfer();
     s->f = ctx->f;
+    ctx->f->backrefs.push_back(&s->f);
     if (s->build() != MG_OK) { delete s; return nullptr; }
     return new mg_stream{s};
 }

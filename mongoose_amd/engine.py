@@ -146,6 +146,25 @@ def KRMSNormOutEps(inp, out, w, seqLen, dim, eps):
     lib.mongoose_rmsnorm_out_eps(_p(inp), _p(out), _p(w), seqLen, dim, eps, None)
 
 
+def KRMSNorm(x, w, seqLen, dim):
+    """kernels.go:601: in place."""
+    lib.mongoose_rmsnorm(_p(x), _p(w), seqLen, dim, None)
+
+
+def KFusedAddRMSNorm(a, b, out, w, seqLen, dim):
+    """kernels.go:641: out = rmsnorm(a + b, w)."""
+    lib.mongoose_fused_add_rmsnorm(_p(a), _p(b), _p(out), _p(w), seqLen, dim, None)
+
+
+def KFusedAddRMSNormEps(a, b, out, w, seqLen, dim, eps):
+    lib.mongoose_fused_add_rmsnorm_eps(_p(a), _p(b), _p(out), _p(w), seqLen, dim, eps, None)
+
+
+def KQ4Matvec(act, w, scales, out, N, K):
+    """kernels.go:947: per-row-scale 4-bit weights (not GGUF Q4_0)."""
+    lib.mongoose_q4_matvec(_p(act), _p(w), _p(scales), _p(out), N, K, None)
+
+
 def KQ8Matvec(act, w, scales, out, N, K):
     lib.mongoose_q8_matvec(_p(act), _p(w), _p(scales), _p(out), N, K, None)
 
@@ -212,6 +231,75 @@ def KZero(ptr, nbytes):
 
 def KSync():
     lib.mongoose_sync(None)
+
+
+# ---- kernel_tensor.go:14-94: the tensor-typed helpers over the K* set ----
+class Q8Weight:
+    """kernel_tensor.go:14-21."""
+
+    def __init__(self, Data, Scales, Rows, Cols, Q4=False):
+        self.Data, self.Scales, self.Rows, self.Cols, self.Q4 = Data, Scales, Rows, Cols, Q4
+
+
+def TRMSNorm(x, weight, seqLen, dim):
+    KRMSNorm(x, weight, seqLen, dim)                          # kernel_tensor.go:23-26
+
+
+def TRMSNormOut(inp, out, weight, seqLen, dim):
+    KRMSNormOut(inp, out, weight, seqLen, dim)                # :28-31
+
+
+def TQ8Matvec(act, w, out):
+    """kernel_tensor.go:33-41: the 4-bit or the 8-bit kernel by w.Q4."""
+    if w.Q4:
+        KQ4Matvec(act, w.Data, w.Scales, out, w.Rows, w.Cols)
+    else:
+        KQ8Matvec(act, w.Data, w.Scales, out, w.Rows, w.Cols)
+
+
+def TRoPE(x, cos, sin, seqLen, dim, headDim, nHeads):
+    KRoPE(x, cos, sin, seqLen, dim, headDim, nHeads)          # :43-46
+
+
+def TDecodeAttention(q, kCache, vCache, out, cacheLen, dim, kvDim, numHeads, numKVHeads):
+    KDecodeAttention(q, kCache, vCache, out, cacheLen, dim, kvDim, numHeads, numKVHeads)   # :48-53
+
+
+def TSiLUGateMul(gate, up, out, n):
+    KSiLUGateMul(gate, up, out, n)                            # :55-58
+
+
+def TCopy(dst, src, nbytes):
+    KCopy(dst, src, nbytes)                                   # :60-63
+
+
+def TCopyAt(dst, dstByteOffset, src, nbytes):
+    KCopy(_p(dst) + dstByteOffset, src, nbytes)               # :65-69
+
+
+def TAddInPlace(a, b, n):
+    KAddInPlace(a, b, n)                                      # :71-74
+
+
+def TRoPEAt(x, cosTable, sinTable, byteOffset, seqLen, dim, headDim, nHeads):
+    """kernel_tensor.go:76-79: the table row of a position is passed as a byte offset."""
+    KRoPE(x, _p(cosTable) + byteOffset, _p(sinTable) + byteOffset, seqLen, dim, headDim, nHeads)
+
+
+def TDecodeAttentionKV(q, kCache, vCache, out, cacheLen, dim, kvDim, numHeads, numKVHeads):
+    KDecodeAttention(q, kCache, vCache, out, cacheLen, dim, kvDim, numHeads, numKVHeads)   # :81-85
+
+
+def TZero(t, nBytes):
+    KZero(t, nBytes)                                          # :92-95
+
+
+def PackInt8ToFloat32(q):
+    """kernel_tensor.go:97-106: int8 bytes viewed as float32 words (padded to a multiple of four)."""
+    b = np.ascontiguousarray(q, dtype=np.int8).view(np.uint8).ravel()
+    buf = np.zeros((b.size + 3) // 4 * 4, np.uint8)
+    buf[:b.size] = b
+    return buf.view(np.float32)
 
 
 def HIPCheck():

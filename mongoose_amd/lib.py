@@ -44,6 +44,10 @@ _sig("tw_hip_device_info", c_int, c_char_p, c_size_t, POINTER(c_uint64))
 _p = c_void_p
 _sig("mongoose_rmsnorm_out", None, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_rmsnorm_out_eps", None, _p, _p, _p, c_int, c_int, c_float, _p)
+_sig("mongoose_rmsnorm", None, _p, _p, c_int, c_int, _p)
+_sig("mongoose_fused_add_rmsnorm", None, _p, _p, _p, _p, c_int, c_int, _p)
+_sig("mongoose_fused_add_rmsnorm_eps", None, _p, _p, _p, _p, c_int, c_int, c_float, _p)
+_sig("mongoose_q4_matvec", None, _p, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_q8_matvec", None, _p, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_q8_matvec_rowscale", None, _p, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_q4_0_matvec", None, _p, _p, _p, c_int, c_int, _p)

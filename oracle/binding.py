@@ -65,6 +65,8 @@ for pfx, real in (("orc32", _f), ("orc64", _d)):
     _sig(pfx + "_rope", None, real, _f, _f, c_int, c_int)
     _sig(pfx + "_decode_attention", None, real, real, real, real, c_int, c_int, c_int, c_int, c_int, real)
     _sig(pfx + "_silu_gate_mul", None, real, real, real, c_int)
+    _sig(pfx + "_q4_matvec", None, real, POINTER(c_uint8), _f, real, c_int, c_int)
+    _sig(pfx + "_fused_add_rmsnorm", None, real, real, _f, c_int, c_float, real)
     _sig(pfx + "_step", c_int, c_void_p, _f, c_int, c_int, c_int, _f, _f, _f)
     _sig(pfx + "_decode_token", c_int, c_void_p, c_int, c_int, _f, _f)
 
@@ -183,6 +185,32 @@ def silu_gate_mul(g, u, shadow=False):
     out = np.empty_like(g)
     getattr(lib, pfx + "_silu_gate_mul")(p(g), p(u), p(out), g.size)
     return out
+
+
+def q4_matvec(act, packed, scales, N, K, shadow=False):
+    """Per-row-scale 4-bit matvec (mongoose_q4_matvec): packed [N, K/2] bytes, scales [N]."""
+    pfx, dt, p = _real(shadow)
+    act = np.ascontiguousarray(act, dt)
+    packed = np.ascontiguousarray(packed, np.uint8)
+    out = np.empty(N, dt)
+    getattr(lib, pfx + "_q4_matvec")(p(act), u8p(packed), fp(f32(scales)), p(out), N, K)
+    return out
+
+
+def fused_add_rmsnorm(a, b, g, eps, shadow=False):
+    pfx, dt, p = _real(shadow)
+    a = np.ascontiguousarray(a, dt)
+    b = np.ascontiguousarray(b, dt)
+    out = np.empty_like(a)
+    getattr(lib, pfx + "_fused_add_rmsnorm")(p(a), p(b), fp(f32(g)), a.size, eps, p(out))
+    return out
+
+
+def rmsnorm_inplace(x, g, eps):
+    """cpu.go:36-47 (CPU.RMSNorm), in place on a copy."""
+    x = np.array(x, dtype=np.float32, order="C")
+    lib.orc_rmsnorm(fp(x), fp(f32(g)), x.size, eps)
+    return x
 
 
 class Oracle:

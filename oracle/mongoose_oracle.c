@@ -35,6 +35,10 @@
  *                        independent numpy restatement.
  *   orc_set_kv_f16       option without a reference counterpart: K/V rows pass through the
  *                        pinned fp16 conversions when written (models an fp16 KV cache)
+ *   orcNN_q4_matvec      kernels/mongoose.cu:1598-1630 (per-row-scale 4-bit, sequential nibble
+ *                        pairs, (nib-8)*s/7); pinned by unit activations that pick single
+ *                        nibbles and by orc_matmul over the densely dequantized matrix
+ *   orcNN_fused_add_rmsnorm  kernels/mongoose.cu:372-404; pinned by orc_rmsnorm on a+b
  *   embedding gather, argmax   no reference function (the reference's caller does
  *                        both on the host); textbook semantics, lowest index on ties.
  *
@@ -46,6 +50,9 @@
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
 
 #define ORC_API __attribute__((visibility("default")))
 

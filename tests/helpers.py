@@ -136,3 +136,75 @@ def oracle_generate(m, prompt, nDecode, want=None, shadow=False):
             toks.append(nxt)
             tok = nxt
     return np.array(toks, np.int32), rec
+
+
+def first_divergence(a, b):
+    """Index of the first position where two token sequences differ, or None."""
+    n = min(len(a), len(b))
+    for i in range(n):
+        if int(a[i]) != int(b[i]):
+            return i
+    return None if len(a) == len(b) else n
+
+
+def assert_same_tokens_or_near_tie(m, prompt, toks, other, what, tol=1e-3):
+    """Two correct evaluation orders of the same model give the same greedy tokens unless two logits
+    are closer than the arithmetic can resolve.  Either the sequences are identical, or at their first
+    difference the oracle's (double-precision) logits of the two candidate tokens differ by less than
+    `tol` of the largest logit: the logit bar itself.  `toks` is the sequence the oracle is replayed on."""
+    i = first_divergence(toks, other)
+    if i is None:
+        return None
+    m.orc.reset_kv()
+    stream = list(prompt) + [int(t) for t in toks[:i]]
+    logits = None
+    for pos, tok in enumerate(stream):
+        _, logits, _ = m.orc.decode_token(int(tok), pos, shadow=True)
+    a, b = int(toks[i]), int(other[i])
+    gap = abs(float(logits[a]) - float(logits[b])) / float(np.abs(logits).max())
+    assert gap < tol, f"{what}: sequences part at token {i} ({a} vs {b}) and the oracle's logits differ by {gap:.2e}"
+    return i
+
+
+def load_fast(s, seed, maxSeq, eng, oracle=True, threads=16, kv_f16=False):
+    """A Model whose matrices are quantized by the library's parallel host quantizer (bit-identical to
+    the oracle's, checked on the CPU) and shared with the oracle: for the multi-gigabyte shapes."""
+    m = Model.__new__(Model)
+    m.s, m.seed, m.maxSeq = s, seed, maxSeq
+    kv = configs.kv_dim(s)
+    m.orc = ob.Oracle(s.dim, kv, s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab, s.nLayers, maxSeq,
+                      s.theta, s.eps, threads=threads) if oracle else None
+    if kv_f16 and m.orc:
+        m.orc.set_kv_f16(True)
+    m.hip = E.NewHIPFusedInference(eng, s.dim, kv, s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab, s.nLayers,
+                                   maxSeq, s.theta, s.eps)
+    assert m.hip is not None, E.last_error()
+    if kv_f16:
+        assert m.hip.SetKVFormat(1) == 0, E.last_error()
+    assert m.hip.SetLayerRange(0, s.nLayers) == 0, E.last_error()
+    m.dequant, m.vecs = None, {}
+    for idx in all_slots(s):
+        rows, cols = slot_shape(s, idx)
+        data = gen_slot(s, seed, idx)
+        if cols == 1:
+            m.vecs[idx] = data
+            if m.orc:
+                m.orc.set_f32(idx, data)
+            assert m.hip.SetWeight(idx, data) == 0, E.last_error()
+        elif s.fmt == "q8":
+            q, sc = E.quantize_q8(data, 0)
+            if m.orc:
+                m.orc.set_q8(idx, q, sc)
+            assert m.hip.SetWeightQ8(idx, q, sc) == 0, E.last_error()
+        else:
+            blocks = E.quantize_q4_0(data)
+            if m.orc:
+                m.orc.set_q4_0(idx, blocks)
+            assert m.hip.SetWeightQ4_0(idx, blocks) == 0, E.last_error()
+    if not s.tied:
+        emb = E.synth_normal(seed, 10_000_019, 0.02, (s.vocab, s.dim)).astype(np.float16)
+        m.embed16 = emb
+        if m.orc:
+            m.orc.set_embed_f16(emb)
+        assert m.hip.SetEmbeddingF16(emb) == 0, E.last_error()
+    return m

@@ -223,3 +223,69 @@ def test_elementwise_ops(hip):
     _check()
     z = hip.ToHost(dout)
     assert (z[:-1] == 0).all() and z[-1] == table[3, 63]
+
+
+# ---- the symbols the tensor-typed helpers bind (kernel_tensor.go:23-40) ----
+@pytest.mark.parametrize("N,K", [(896, 896), (128, 4864), (33, 70), (5, 2), (1000, 1376)])
+def test_q4_rowscale_matvec(hip, N, K):
+    """mongoose_q4_matvec (mongoose.cu:1598-1640): per-row-scale 4-bit, sequential nibble pairs, (nib-8)*s/7.
+    Shapes with word-aligned rows and without (K/2 not a multiple of 4), a single byte per row."""
+    packed = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    scales = rng.uniform(0.01, 0.3, N).astype(np.float32)
+    act = rng.standard_normal(K).astype(np.float32)
+    dw, ds, da = _up(hip, packed), _up(hip, scales), _up(hip, act)
+    dout = hip.Zeros([N])
+    E.TQ8Matvec(da, E.Q8Weight(dw, ds, N, K, Q4=True), dout)      # the route TQ8Matvec takes for Q4 weights
+    _check()
+    got = hip.ToHost(dout)
+    assert H.rel_err(got, ob.q4_matvec(act, packed, scales, N, K, shadow=True)) < 1e-5
+    assert H.rel_err(got, ob.q4_matvec(act, packed, scales, N, K)) < 1e-5
+    for t in (dw, ds, da, dout):
+        t.Release()
+
+
+@pytest.mark.parametrize("seqLen,dim", [(1, 896), (3, 512), (2, 4096), (1, 100)])
+def test_rmsnorm_in_place_and_fused_add(hip, seqLen, dim):
+    """mongoose_rmsnorm (mongoose.cu:16-50, in place) and mongoose_fused_add_rmsnorm (:372-404), eps 1e-6 as
+    the CUDA kernels hard-code; the _eps form against another eps; out aliasing an input."""
+    x = rng.standard_normal((seqLen, dim)).astype(np.float32)
+    y = rng.standard_normal((seqLen, dim)).astype(np.float32)
+    g = (1.0 + 0.1 * rng.standard_normal(dim)).astype(np.float32)
+    dx, dy, dg = _up(hip, x), _up(hip, y), _up(hip, g)
+    dout = hip.Zeros([seqLen * dim])
+    E.KFusedAddRMSNorm(dx, dy, dout, dg, seqLen, dim)
+    _check()
+    got = hip.ToHost(dout).reshape(seqLen, dim)
+    for r in range(seqLen):
+        assert H.rel_err(got[r], ob.fused_add_rmsnorm(x[r], y[r], g, 1e-6, shadow=True)) < 1e-6
+    E.KFusedAddRMSNormEps(dx, dy, dout, dg, seqLen, dim, 0.25)
+    _check()
+    got = hip.ToHost(dout).reshape(seqLen, dim)
+    for r in range(seqLen):
+        assert H.rel_err(got[r], ob.fused_add_rmsnorm(x[r], y[r], g, 0.25, shadow=True)) < 1e-6
+    E.KFusedAddRMSNorm(dx, dy, dy, dg, seqLen, dim)                # out aliases b
+    _check()
+    got = _down(hip, dy, np.float32, seqLen * dim).reshape(seqLen, dim)
+    for r in range(seqLen):
+        assert H.rel_err(got[r], ob.fused_add_rmsnorm(x[r], y[r], g, 1e-6, shadow=True)) < 1e-6
+    E.TRMSNorm(dx, dg, seqLen, dim)                                # in place
+    _check()
+    got = _down(hip, dx, np.float32, seqLen * dim).reshape(seqLen, dim)
+    for r in range(seqLen):
+        assert H.rel_err(got[r], ob.rmsnorm_out(x[r], g, 1e-6, shadow=True)) < 1e-6
+        assert H.rel_err(got[r], ob.rmsnorm_inplace(x[r], g, 1e-6)) < 1e-5     # the float path's serial sum of 4096 squares
+    for t in (dx, dy, dg, dout):
+        t.Release()
+
+
+def test_zero_fill_unaligned(hip):
+    """mongoose_zero on a range that starts and ends off a word boundary touches exactly its bytes."""
+    buf = np.full(64, 0xAB, np.uint8)
+    d = _up(hip, buf)
+    E.KZero(d.DevicePtr() + 3, 22)
+    _check()
+    got = hip.DownloadRawBytes(d, 64)
+    want = buf.copy()
+    want[3:25] = 0
+    assert np.array_equal(got, want)
+    d.Release()

@@ -270,3 +270,73 @@ def test_silu_gate_mul_closed_form():
 def test_argmax_lowest_index_on_ties():
     x = np.array([1, 5, 5, 2, 5], np.float32)
     assert ob.lib.orc_argmax(ob.fp(x), 5) == 1
+
+
+# ---- per-row-scale 4-bit matvec (mongoose_q4_matvec, kernels/mongoose.cu:1598-1630) ----
+def _dense_q4_rowscale(packed, scales, N, K):
+    """Element 2k = low nibble of byte k, element 2k+1 = high nibble; value (nib-8) * (s/7), in float."""
+    b = np.asarray(packed, np.uint8).reshape(N, K // 2)
+    s7 = (np.asarray(scales, np.float32) / np.float32(7.0)).astype(np.float32)
+    w = np.empty((N, K), np.float32)
+    w[:, 0::2] = ((b & 0x0F).astype(np.int32) - 8).astype(np.float32) * s7[:, None]
+    w[:, 1::2] = ((b >> 4).astype(np.int32) - 8).astype(np.float32) * s7[:, None]
+    return w
+
+
+def test_q4_rowscale_matvec_unit_activations_pick_single_nibbles():
+    """A unit activation at element e returns, for every row, exactly that element's dequantized
+    weight: pins which nibble is which element, the -8 offset and the /7."""
+    N, K = 3, 8
+    packed = np.array([[0x10, 0x32, 0x54, 0xF6], [0x8F, 0x08, 0x80, 0x77], [0xFF, 0x00, 0xA5, 0x5A]], np.uint8)
+    scales = np.array([7.0, 3.5, 0.25], np.float32)
+    for e in range(K):
+        act = np.zeros(K, np.float32)
+        act[e] = 1.0
+        got = ob.q4_matvec(act, packed, scales, N, K)
+        byte = packed[:, e // 2]
+        nib = (byte & 0x0F) if e % 2 == 0 else (byte >> 4)
+        want = (nib.astype(np.int32) - 8).astype(np.float32) * (scales / np.float32(7.0)).astype(np.float32)
+        assert (got == want).all(), e
+    # row 0 with scale 7: the weights are the integers nib - 8 themselves
+    act = np.ones(K, np.float32)
+    assert ob.q4_matvec(act, packed, scales, N, K)[0] == sum(n - 8 for n in (0, 1, 2, 3, 4, 5, 6, 15))
+
+
+def test_q4_rowscale_matvec_equals_matmul_over_dequantized_weights():
+    rng = np.random.default_rng(17)
+    N, K = 37, 96
+    packed = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    scales = rng.uniform(0.01, 0.2, N).astype(np.float32)
+    act = rng.standard_normal(K).astype(np.float32)
+    w = _dense_q4_rowscale(packed, scales, N, K)
+    got64 = ob.q4_matvec(act, packed, scales, N, K, shadow=True)
+    assert np.allclose(got64, w.astype(np.float64) @ act.astype(np.float64), rtol=1e-12, atol=1e-14)
+    got32 = ob.q4_matvec(act, packed, scales, N, K)
+    assert H_rel(got32, got64) < 1e-5
+    # a zero scale row gives zero; K = 2 is the smallest row
+    assert ob.q4_matvec(np.ones(2, np.float32), np.array([[0xF0]], np.uint8), np.array([0.0], np.float32), 1, 2)[0] == 0.0
+
+
+def H_rel(a, b):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    return float(np.abs(a - b).max() / np.abs(b).max())
+
+
+def test_fused_add_rmsnorm_is_rmsnorm_of_the_sum():
+    """kernels/mongoose.cu:372-404 against CPU.RMSNorm (cpu.go:36-47) applied to a + b."""
+    rng = np.random.default_rng(23)
+    n = 896
+    a = rng.standard_normal(n).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    g = (1.0 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    for eps in (1e-6, 1e-5, 0.5):
+        got = ob.fused_add_rmsnorm(a, b, g, eps)
+        want = ob.rmsnorm_inplace((a + b).astype(np.float32), g, eps)
+        assert (got == want).all()
+    # b = -a: the sum is zero and so is the output, whatever eps (> 0) is
+    assert (ob.fused_add_rmsnorm(a, -a, g, 1e-6) == 0).all()
+    # closed form in double
+    s = a.astype(np.float64) + b.astype(np.float64)
+    want64 = s / np.sqrt((s * s).mean() + 1e-6) * g
+    assert H_rel(ob.fused_add_rmsnorm(a, b, g, 1e-6, shadow=True), want64) < 1e-12

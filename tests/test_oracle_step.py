@@ -100,3 +100,132 @@ def test_threads_do_not_change_results():
     assert (a[0] == b[0]).all() and (a[1] == b[1]).all()
     m1.close()
     m4.close()
+
+
+# ---------------------------------------------------------------------------
+# Step-level checks that the mathematics fixes (independent of tests/np_reference.py)
+# ---------------------------------------------------------------------------
+def _oracle_from(shape, maxSeq, mats, vecs):
+    """Oracle with explicitly given fp32 matrices (quantized to Q8 here) and vectors."""
+    kv = configs.kv_dim(shape)
+    o = ob.Oracle(shape.dim, kv, shape.headDim, shape.nHeads, shape.nKVHeads, shape.ffnDim, shape.vocab,
+                  shape.nLayers, maxSeq, shape.theta, shape.eps, threads=1)
+    deq = {}
+    for idx, w in mats.items():
+        q, s = ob.quantize_q8(w, 0)
+        o.set_q8(idx, q, s)
+        deq[idx] = ob.dequant_q8(q, s)
+    for idx, v in vecs.items():
+        o.set_f32(idx, v)
+    return o, deq
+
+
+def _random_layer(shape, rng, l=0):
+    kv = configs.kv_dim(shape)
+    d, f = shape.dim, shape.ffnDim
+    n = lambda *sh: (rng.standard_normal(sh) * 0.1).astype(np.float32)
+    mats = {l * 12 + 1: n(d, d), l * 12 + 2: n(kv, d), l * 12 + 3: n(kv, d), l * 12 + 7: n(d, d),
+            l * 12 + 9: n(f, d), l * 12 + 10: n(f, d), l * 12 + 11: n(d, f)}
+    vecs = {l * 12 + 0: (1 + n(d)).astype(np.float32), l * 12 + 8: (1 + n(d)).astype(np.float32)}
+    return mats, vecs
+
+
+def test_zero_output_projections_leave_the_residual_stream_unchanged():
+    """x += Wo.attn and x += Wdown.ffn are the only writes to the residual stream
+    (cuda_fused_infer.go:434-435, 442-443): with both matrices zero a layer is the identity, bit for bit,
+    whatever the other weights are, at every position."""
+    shape = configs.Shape("id", 2, 64, 2, 1, 32, 96, 40, 1e-5, 1e4, True, True, "q8")
+    rng = np.random.default_rng(5)
+    mats, vecs = {}, {}
+    for l in range(shape.nLayers):
+        m, v = _random_layer(shape, rng, l)
+        m[l * 12 + 7][:] = 0
+        m[l * 12 + 11][:] = 0
+        v[l * 12 + 4] = rng.standard_normal(shape.dim).astype(np.float32)
+        mats.update(m)
+        vecs.update(v)
+    vecs[shape.nLayers * 12] = np.ones(shape.dim, np.float32)
+    mats[shape.nLayers * 12 + 1] = (rng.standard_normal((shape.vocab, shape.dim)) * 0.1).astype(np.float32)
+    o, _ = _oracle_from(shape, 6, mats, vecs)
+    for pos in range(6):
+        h = rng.standard_normal(shape.dim).astype(np.float32)
+        for shadow in (False, True):
+            out, _, layers = o.step(h, pos, shadow=shadow, want_layers=True)
+            assert (out == h).all() and (layers == h).all()
+    o.close()
+
+
+def test_bias_is_added_before_rope_closed_form():
+    """One head, Wq = Wk = 0: q and k are the biases alone, so with the bias added BEFORE the rotation
+    (cuda_fused_stream.go:319-321) the score of positions (P, t) is
+        [ sum_j (bq_j bk_j + bq_j' bk_j') cos((P-t) f_j) - (bq_j' bk_j - bq_j bk_j') sin((P-t) f_j) ] / sqrt(hd)
+    (j' = j + hd/2, f_j = theta^(-2j/hd)): a function of P - t only.  With the bias added after the
+    rotation every score would be bq.bk / sqrt(hd) and the softmax uniform.  Wo = identity and
+    Wdown = 0 expose the attention output as hidden_out - hidden_in."""
+    hd = 32
+    shape = configs.Shape("one-head", 1, hd, 1, 1, hd, 32, 16, 1e-5, 1e4, True, True, "q8")
+    rng = np.random.default_rng(11)
+    mats, vecs = _random_layer(shape, rng)
+    mats[1][:] = 0
+    mats[2][:] = 0
+    mats[7] = np.eye(hd, dtype=np.float32)
+    mats[11][:] = 0
+    bq = rng.standard_normal(hd).astype(np.float32)
+    bk = rng.standard_normal(hd).astype(np.float32)
+    bv = rng.standard_normal(hd).astype(np.float32)
+    vecs.update({4: bq, 5: bk, 6: bv, 12: np.ones(hd, np.float32)})
+    mats[13] = (rng.standard_normal((shape.vocab, hd)) * 0.1).astype(np.float32)
+    P = 7
+    o, deq = _oracle_from(shape, P + 1, mats, vecs)
+    hs = rng.standard_normal((P + 1, hd)).astype(np.float64)
+    outs = [o.step(hs[t].astype(np.float32), t, shadow=True)[0] for t in range(P + 1)]
+    hs = hs.astype(np.float32).astype(np.float64)
+    # value rows: v_t = Wv . rmsnorm(h_t, g1) + bv, in double from the dequantized matrix
+    g1 = vecs[0].astype(np.float64)
+    nrm = hs / np.sqrt((hs * hs).mean(axis=1, keepdims=True) + shape.eps) * g1
+    v = nrm @ deq[3].astype(np.float64).T + bv
+    half = hd // 2
+    f = shape.theta ** (-2.0 * np.arange(half) / hd)
+    q0, q1, k0, k1 = bq[:half].astype(np.float64), bq[half:].astype(np.float64), bk[:half].astype(np.float64), bk[half:].astype(np.float64)
+    wo = deq[7].astype(np.float64)
+    for pos in (0, 3, P):
+        t = np.arange(pos + 1)
+        ang = (pos - t)[:, None] * f[None, :]
+        s_before = ((q0 * k0 + q1 * k1) * np.cos(ang) - (q1 * k0 - q0 * k1) * np.sin(ang)).sum(axis=1) / np.sqrt(hd)
+        p = np.exp(s_before - s_before.max())
+        p /= p.sum()
+        want = hs[pos] + wo @ (p @ v[:pos + 1])
+        assert H.rel_err(outs[pos], want) < 2e-6, pos              # the cos/sin tables are stored as floats
+        if pos > 0:
+            uniform = hs[pos] + wo @ v[:pos + 1].mean(axis=0)       # what bias-after-rotation would give
+            assert H.rel_err(outs[pos], uniform) > 1e-3, pos
+    o.close()
+
+
+def test_no_logits_before_the_last_layer():
+    """cuda_fused_infer.go:446: the final norm and lm_head run only when layerEnd reaches nLayers."""
+    m = H.Model(MINI, seed=3, maxSeq=4, oracle=True, threads=1)
+    h = m.orc.embed(5)
+    for pfx in ("orc32", "orc64"):
+        logits = np.full(MINI.vocab, -123.0, np.float32)
+        hout = np.empty(MINI.dim, np.float32)
+        rc = getattr(ob.lib, pfx + "_step")(m.orc.h, ob.fp(h), 0, 0, MINI.nLayers - 1, ob.fp(hout), ob.fp(logits), None)
+        assert rc == 0 and (logits == -123.0).all()
+        rc = getattr(ob.lib, pfx + "_step")(m.orc.h, ob.fp(h), 0, 0, MINI.nLayers, ob.fp(hout), ob.fp(logits), None)
+        assert rc == 0 and not (logits == -123.0).any()
+    m.close()
+
+
+def test_threaded_attention_changes_nothing():
+    """Heads are shared out over the oracle's threads; each head's arithmetic is untouched."""
+    shape = MINI._replace(nHeads=4, nKVHeads=2)
+    a = H.Model(shape, seed=21, maxSeq=40, oracle=True, threads=1)
+    b = H.Model(shape, seed=21, maxSeq=40, oracle=True, threads=3)
+    prompt = a.prompt(40)
+    for pos in range(40):
+        h = a.orc.embed(prompt[pos])
+        for shadow in (False, True):
+            x, y = a.orc.step(h, pos, shadow=shadow), b.orc.step(h, pos, shadow=shadow)
+            assert (x[0] == y[0]).all() and (x[1] == y[1]).all()
+    a.close()
+    b.close()
