@@ -128,6 +128,21 @@ void mongoose_dequant_q4_0(const void* w_q4_0, float* out, int rows, int cols, v
  * 16-byte aligned. */
 void mongoose_q8_gemm(const float* act, const void* w, const float* scales, const float* bias, float* out, int T, int N,
                       int K, int accumulate, void* workspace, size_t workspaceBytes, void* stream);
+/* No counterpart in the reference.  mongoose_q8_gemm for callers that cannot allocate and have no
+ * workspace to hand over (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): the two bf16 planes of the split activations are written into a static device array
+ * of mg_q8_gemm_noalloc_max_bytes() = 8 MiB inside the library, so the call allocates nothing.
+ * Limit: 4 * roundup(T,128) * roundup(K,64) <= 8 MiB (e.g. 512 x 4096, 128 x 16384); larger shapes
+ * return MG_E_ARG with the sizes in mg_last_error().  Results are those of mongoose_q8_gemm bit
+ * for bit.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
+ * (different streams or threads) race; serialise them.  Nothing in the array has to start at zero
+ * (rows and k past the ends of the input are either not read or their results are dropped), so it
+ * is not cleared between calls.  The array's device address is looked up once per device, by
+ * tw_hip_init_device or by the first call on that device -- make one of the two before a capture
+ * begins.  Returns MG_OK, MG_E_ARG or MG_E_HIP. */
+int mg_q8_gemm_noalloc(const float* act, const void* w, const float* scales, const float* bias, float* out, int T, int N,
+                       int K, int accumulate, void* stream);
+size_t mg_q8_gemm_noalloc_max_bytes(void);
 void mongoose_copy(void* dst, const void* src, size_t bytes, void* stream);
 void mongoose_zero(void* ptr, size_t bytes, void* stream);
 void mongoose_sync(void* stream);

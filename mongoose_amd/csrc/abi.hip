@@ -4,14 +4,44 @@
 #include "../../include/mongoose_hip.h"
 #include "kernels.h"
 #include "prefill.h"
+#include "fused_infer.h"
 
 #include <atomic>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
+#include <string>
 #include <vector>
+
+// Scratch memory of mg_q8_gemm_noalloc: the two bf16 planes of the split activations live in this
+// array instead of a caller's workspace.  Every GPU the library runs on holds its own copy for the life
+// of the process.  In host code the name is only a handle: the device address is looked up once per
+// device (scratch_on_current_device) and that pointer is what kernels and copies are given.
+#define MG_NOALLOC_SCRATCH_BYTES (8u << 20)
+static __device__ __align__(256) unsigned char scratch[MG_NOALLOC_SCRATCH_BYTES];
 
 namespace {
 std::atomic<int> g_lastErr{0};
+constexpr int kMaxDevices = 64;
+std::mutex g_scratchMu;
+void* g_scratchPtr[kMaxDevices] = {};
+// Device address of `scratch` on the current device (looked up on the first call per device).
+hipError_t scratch_on_current_device(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lk(g_scratchMu);
+    if (!g_scratchPtr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!ptr) return hipErrorInvalidSymbol;
+        g_scratchPtr[dev] = ptr;
+    }
+    *out = g_scratchPtr[dev];
+    return hipSuccess;
+}
 inline void note(hipError_t e) {
     if (e != hipSuccess) g_lastErr.store((int)e);
 }
@@ -46,7 +76,12 @@ void tw_gpu_free_pinned(void* ptr) { if (ptr) note(hipHostFree(ptr)); }
 int tw_hip_init_device(int device) {
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess || device < 0 || device >= n) { (void)hipGetLastError(); return -1; }
-    return hipSetDevice(device) == hipSuccess ? 0 : -1;
+    if (hipSetDevice(device) != hipSuccess) { (void)hipGetLastError(); return -1; }
+    // set-up work that later calls must not have to do: the address of the no-allocation entry
+    // point's scratch array on this device
+    void* ptr = nullptr;
+    if (scratch_on_current_device(&ptr) != hipSuccess) { (void)hipGetLastError(); return -1; }
+    return 0;
 }
 int tw_hip_device_info(char* name, size_t nameLen, uint64_t* totalMem) {
     int dev = 0;
@@ -174,6 +209,48 @@ void mongoose_q8_gemm(const float* act, const void* w, const float* scales, cons
     g.Ahi = static_cast<const unsigned short*>(hi); g.Alo = static_cast<const unsigned short*>(lo);
     note(mg::launch_gemm_q8(g, accumulate, S(stream)));
 }
+// mongoose_q8_gemm with the split planes in the library's static scratch array: no allocation of any
+// kind on this path (no hipMalloc / hipFree, no workspace from the caller).
+int mg_q8_gemm_noalloc(const float* act, const void* w, const float* scales, const float* bias, float* out, int T, int N,
+                       int K, int accumulate, void* stream) {
+    if (T < 0 || N < 0 || K <= 0 || K % 32 != 0 || !act || !w || !scales || !out || ((uintptr_t)w & 15)) {
+        mg::set_error("mg_q8_gemm_noalloc: bad argument (K must be a positive multiple of 32, w 16-byte aligned)");
+        return MG_E_ARG;
+    }
+    const size_t plane = mg::split_plane_elems(T, K) * 2;
+    if (2 * plane > MG_NOALLOC_SCRATCH_BYTES) {
+        mg::set_error("mg_q8_gemm_noalloc: 4 * roundup(T,128) * roundup(K,64) = " + std::to_string(2 * plane) +
+                      " bytes of split activations exceed the static scratch of " + std::to_string(MG_NOALLOC_SCRATCH_BYTES) +
+                      " bytes; use mongoose_q8_gemm with a workspace");
+        return MG_E_ARG;
+    }
+    if (T == 0 || N == 0) return MG_OK;
+    void* base = nullptr;
+    hipError_t e = scratch_on_current_device(&base);
+    if (e != hipSuccess) {
+        mg::set_error(std::string("mg_q8_gemm_noalloc: scratch address lookup failed: ") + hipGetErrorString(e));
+        (void)hipGetLastError();
+        return MG_E_HIP;
+    }
+    void* hi = base;
+    void* lo = static_cast<char*>(base) + plane;
+    e = mg::launch_split_rows(act, nullptr, 0.f, T, K, hi, lo, S(stream));
+    if (e == hipSuccess) {
+        mg::GemmParams g{};
+        g.seg[0] = mg::GemmSeg{static_cast<const signed char*>(w), scales, bias, out, N, 0};
+        g.nseg = 1; g.T = T; g.K = K;
+        g.Ahi = static_cast<const unsigned short*>(hi); g.Alo = static_cast<const unsigned short*>(lo);
+        e = mg::launch_gemm_q8(g, accumulate, S(stream));
+    }
+    if (e != hipSuccess) {
+        mg::set_error(std::string("mg_q8_gemm_noalloc: launch failed: ") + hipGetErrorString(e));
+        (void)hipGetLastError();
+        return MG_E_HIP;
+    }
+    return MG_OK;
+}
+size_t mg_q8_gemm_noalloc_max_bytes(void) { return MG_NOALLOC_SCRATCH_BYTES; }
+
 void mongoose_copy(void* dst, const void* src, size_t bytes, void* stream) {
     if (bytes) note(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, S(stream)));
 }

@@ -545,6 +545,12 @@ class HIPStreamInfer:
                                            sizes.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), _fp(logitsOut))
 
 
+def KQ8GemmNoAlloc(act, w, scales, bias, out, T, N, K, accumulate):
+    """KQ8Gemm without a workspace: the split planes live in the library's static scratch array."""
+    return lib.mg_q8_gemm_noalloc(_p(act), _p(w), _p(scales), _p(bias) if bias is not None else None, _p(out), T, N, K,
+                                  1 if accumulate else 0, None)
+
+
 def KQ8Gemm(act, w, scales, bias, out, T, N, K, accumulate, workspace, workspaceBytes):
     """Multi-row form of KQ8MatvecRowScale on the matrix cores (out[T,N] (+)= act[T,K] . w[N,K]^T * scales + bias)."""
     lib.mongoose_q8_gemm(_p(act), _p(w), _p(scales), _p(bias) if bias is not None else None, _p(out), T, N, K,

@@ -63,6 +63,8 @@ _sig("mongoose_dequant_int8_to_fp32", None, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_dequant_q8_rowscale", None, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_dequant_q4_0", None, _p, _p, c_int, c_int, _p)
 _sig("mongoose_q8_gemm", None, _p, _p, _p, _p, _p, c_int, c_int, c_int, c_int, _p, c_size_t, _p)
+_sig("mg_q8_gemm_noalloc", c_int, _p, _p, _p, _p, _p, c_int, c_int, c_int, c_int, _p)
+_sig("mg_q8_gemm_noalloc_max_bytes", c_size_t)
 _sig("mongoose_copy", None, _p, _p, c_size_t, _p)
 _sig("mongoose_zero", None, _p, c_size_t, _p)
 _sig("mongoose_sync", None, _p)
