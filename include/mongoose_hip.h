@@ -239,9 +239,22 @@ int mg_hidden_idx(mg_ctx* ctx);
 
 /* Execution mode of the layer loop: 0 = one launch per reference op, in the
  * reference's order (cuda_fused_infer.go:417-443, 17 launches a layer);
- * 1 = fused launches (default); 2 = fused launches whose attention launch does not
+ * 1 = fused launches (five a layer); 2 = fused launches whose attention launch does not
  * also fetch the following matrices into L2 with its idle workgroups (for a GPU
- * shared with other work).  All give the same results to rounding. */
+ * shared with other work); 3 = all layers of a step in ONE persistent launch whose
+ * workgroups hand their vectors over through device memory, wherever the model allows it
+ * (Q8 weights, fp32 KV rows, heads of 64 or 128, the context within 256 (heads of 64) or
+ * 128 (heads of 128) positions per attention workgroup with nHeads x splits workgroups at
+ * most as many as the GPU has CUs; otherwise as mode 1).
+ * A new context is in automatic mode: as mode 3 where that launch is also the faster one --
+ * at least 8 layers of at most 64 MB of weights each, i.e. steps bound by the hand-over
+ * between dependent phases rather than by HBM (measured: 0.5B and 1.1B shapes 10-18 %
+ * faster, the 8B shape 26 % slower than mode 1) -- and as mode 1 elsewhere.  Setting a mode
+ * ends automatic mode.
+ * The persistent launch needs all its workgroups resident at once: on a GPU shared with
+ * other kernels its waits can run into their time limit; the call then returns MG_E_HIP,
+ * and the context continues with the fused launches.  All modes give the same results to
+ * rounding. */
 int mg_set_exec_mode(mg_ctx* ctx, int mode);
 
 /* Whole token on the device: embedding gather -> layers -> final norm ->
@@ -305,6 +318,33 @@ int mg_generate_prefill(mg_ctx* ctx, const int* prompt, int nPrompt, int nDecode
  * HBM).  nr (rows per wave group), ks (1 or 4: waves sharing a row group) and
  * grid = 0 use the library's own configuration. */
 int mg_bench_matvec(int wf, int N, int K, int nr, int ks, int grid, int copies, int iters, float* avgUs);
+
+/* Exec mode 3 hands vectors from phase to phase through an exchange area in device memory; this copies
+ * layer `layer`'s block as the last step left it (cap floats at most) and describes it: geo[11] =
+ * {floats per layer, offsets of q, current K row, current V row, attention partial accumulators
+ * [smax, dim], their maxima [smax, nHeads], their sums [smax, nHeads], hidden after the attention
+ * block, SwiGLU vector, layer output, smax}.  A float never written reads 0xFFFFFFFF.  For tests. */
+int mg_flow_exchange(mg_ctx* ctx, int layer, float* out, size_t cap, int* geo);
+
+/* 1 when a step over all layers goes through the persistent launch of exec mode 3 (mode, model and
+ * context as they are now), else 0. */
+int mg_flow_in_use(mg_ctx* ctx);
+
+/* Timing diagnostic of exec mode 3: with enable != 0 every persistent launch records, per layer and
+ * workgroup, when thread 0 passed each of 11 points (layer top; q|k|v input staged; q|k|v done; q, K, V
+ * rows in; attention done; attention merged; Wo done; gate|up input staged; gate|up done; down input
+ * staged; down done) in ticks of the 100 MHz wall clock.  out != NULL receives the last launch's ticks
+ * [layer][point][workgroup] (cap int64 at least layers x 11 x workgroups), dims[3] = {layers, 11,
+ * workgroups}.  enable == 0 stops and frees.  No counterpart in the reference; MG_E_STATE when the
+ * persistent launch is not in use for the model. */
+int mg_flow_trace(mg_ctx* ctx, int enable, long long* out, size_t cap, int* dims);
+
+/* Time limit of each wait inside the persistent launch, in ticks of the 100 MHz wall clock (default
+ * 5,000,000 = 50 ms).  A workgroup whose wait runs out stops waiting for the rest of the launch, the
+ * launch ends normally with an error flag set, the call that issued it returns MG_E_HIP and the
+ * context goes on with the fused launches.  A limit below zero makes every wait that is not satisfied
+ * at once give up: the way the tests reach that path.  No counterpart in the reference. */
+int mg_flow_set_wait_limit(mg_ctx* ctx, long long ticks);
 
 /* Bytes of weights, scales and norm gains one token reads (the figure the
  * bandwidth roofline is computed from), and the KV bytes read at position pos. */

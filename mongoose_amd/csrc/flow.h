@@ -1,0 +1,70 @@
+// flow.h -- the layers of a decode step as ONE persistent launch (flow.hip).
+//
+// A small model's token is ~120 dependent phases of a few microseconds each; as separate launches every
+// phase pays a kernel boundary and starts with cold registers.  Here one workgroup per CU stays resident
+// for all layers of the token and the phases hand their vectors over through a small exchange area in
+// device memory: a producer stores its floats write-through, a consumer polls the vector it needs until
+// no element is the "not written yet" pattern.  No barrier across the grid and no atomics: a phase costs
+// one store-to-load hand-over, and a wave requests its next weights before it starts to wait.
+#pragma once
+#include "kernels.h"
+
+namespace mg {
+
+// Per-layer operands, a table in device memory (Q8 weights: int8 rows + per-row float scales).
+struct FlowLayer {
+    const float* g1;
+    const float* g2;
+    const signed char* wq; const signed char* wk; const signed char* wv; const signed char* wo;
+    const signed char* gate; const signed char* up; const signed char* down;
+    const float* sq; const float* sk; const float* sv; const float* so;
+    const float* sgate; const float* sup; const float* sdown;
+    const float* bq; const float* bk; const float* bv;      // optional (NULL)
+    float* Kc; float* Vc;                                    // fp32 caches [maxSeq, kvDim]
+};
+
+// Exchange area: per layer one block of `stride` floats holding, at the offsets below, the rotated query,
+// the K and V rows of the current position, the attention partials of up to smax KV splits (accumulator,
+// maximum, sum), the hidden state after the attention block, the SwiGLU vector and the layer's output.
+// Every float is the pattern 0xFFFFFFFF until its producer has written it.
+constexpr int FLOW_MIN_TILE = 128;     // positions of the smallest attention tile (it doubles until the slots cover the context)
+struct FlowGeometry {
+    int stride;
+    int offQ, offKc, offVc, offPacc, offPm, offPl, offX1, offM, offX2;
+    int smax;
+};
+FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int headDim, int maxSeq, int grid);
+bool flow_context_fits(int headDim, int maxSeq, const FlowGeometry& g);
+
+// Trace slots of a layer, in program order: when thread 0 of a workgroup passed the point.
+constexpr int FLOW_TRACE_SLOTS = 11;
+#define FLOW_TRACE_NAMES "layer-top", "qkv-input-staged", "qkv-done", "q-k-v-rows-in", "attention-done", "attention-merged", \
+                         "wo-done", "gate-up-input-staged", "gate-up-done", "down-input-staged", "down-done"
+
+struct FlowParams {
+    const FlowLayer* layers;     // indexed by layer
+    int l0, l1;                  // layers [l0, l1)
+    int nLayersTotal;            // layers the table and the exchange area hold
+    int dim, kvDim, ffn, nHeads, nKVHeads, headDim, maxSeq;
+    float eps;
+    const StepState* state;      // position source (NULL -> posImm)
+    int posImm;
+    const float* cosRow;         // cos / sin row of the position [headDim/2]
+    const float* sinRow;
+    float* hidden;               // input of layer l0 and output of layer l1-1 [dim]
+    float* xchg;                 // exchange area, geo.stride floats per layer (indexed by layer)
+    FlowGeometry geo;
+    int* err;                    // set to 1 when a wait ran into its time limit
+    long long limitTicks;        // per wait, in ticks of the 100 MHz wall clock
+    long long* trace;            // optional (diagnostic): wall-clock ticks [layer][FLOW_TRACE_SLOTS][workgroup], see FLOW_TRACE_NAMES
+};
+
+// Workgroups the launch needs at least (one per query head and KV split) for this shape.
+int flow_min_grid(int nHeads, const FlowGeometry& g);
+bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads, int headDim);
+// grid workgroups of 256 threads, all of which must be resident at once (grid <= CUs x resident workgroups per CU).
+hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s);
+// Fills the blocks of layers [l0, l1) with the "not written yet" pattern.
+hipError_t launch_flow_reset(float* xchg, const FlowGeometry& g, int l0, int l1, hipStream_t s);
+
+}  // namespace mg

@@ -1,0 +1,669 @@
+// flow.hip -- all layers of a batch-1 decode step in one persistent launch (see flow.h).
+//
+// Arithmetic per phase is that of the separate launches (kernels.hip): RMSNorm folded into the staged
+// vector and the row epilogue, int8 rows against fp32 activations with fp32 accumulation, RoPE on (j, j+hd/2)
+// pairs, softmax with a running maximum, SiLU(g)*u, residual adds (cuda_fused_infer.go:414-444,
+// cuda_fused_stream.go:319-321, kernels/mongoose.cu:145-174, 856-933, 949-956, 991-1006, 1556-1585).
+//
+// Hand-over protocol.  Every vector that one phase produces and the next consumes lives in the exchange
+// area, one block per layer.  Before the launch every float there is XSENT (a NaN pattern no arithmetic
+// here produces: results equal to it are canonicalised on the way out).  Producers store at agent scope
+// (write-through, visible to the other XCDs' loads that bypass their L2); consumers load at agent scope
+// and repeat until nothing they need is XSENT.  A workgroup only ever waits for phases that precede its
+// own in the same fixed order, so with all workgroups resident every wait ends; every wait is bounded by
+// a time limit all the same, after which the workgroup stops waiting (results are then garbage and
+// *err is set, which the host checks).
+#include <cstddef>
+#include "flow.h"
+#include "device_util.h"
+
+namespace mg {
+
+constexpr unsigned XSENT = 0xFFFFFFFFu;
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bool unset(float v) { return __builtin_bit_cast(unsigned, v) == XSENT; }
+__device__ __forceinline__ float canon(float v) { return unset(v) ? __builtin_bit_cast(float, 0x7FC00000u) : v; }
+__device__ __forceinline__ bool ready4(f4 v) { return !(unset(v.x) || unset(v.y) || unset(v.z) || unset(v.w)); }
+
+struct Waiter {
+    long long limit;
+    int* err;
+    bool dead;
+    __device__ __forceinline__ void fail() {
+        dead = true;
+        __hip_atomic_store(err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+};
+
+// 16-byte agent-scope load (bypasses this XCD's L2) / store (write-through)
+__device__ __forceinline__ f4 ldx4(const f4* p) {
+    f4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ void stx4(f4* p, f4 v) {
+    v.x = canon(v.x); v.y = canon(v.y); v.z = canon(v.z); v.w = canon(v.w);
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void stx(float* p, float v) { st_agent(p, canon(v)); }
+
+__device__ __forceinline__ f4 poll4(const f4* p, Waiter& w) {
+    f4 v = ldx4(p);
+    if (ready4(v) || w.dead) return v;
+    const long long t0 = wall_clock64();
+    for (;;) {
+        v = ldx4(p);
+        if (ready4(v)) break;
+        if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
+    }
+    return v;
+}
+__device__ __forceinline__ float poll1(const float* p, Waiter& w) {
+    float v = ld_agent(p);
+    if (!unset(v) || w.dead) return v;
+    const long long t0 = wall_clock64();
+    for (;;) {
+        v = ld_agent(p);
+        if (!unset(v)) break;
+        if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
+    }
+    return v;
+}
+// The first n of five pieces with all their loads in flight at once: one memory round trip instead of n.
+// Loads and the wait for them are one asm statement each time -- with the wait in a statement of its own the
+// compiler is free to copy a destination register between the two, i.e. before the data has arrived.
+__device__ __forceinline__ void ldx4_n(const f4* const (&p)[5], f4 (&v)[5], int n) {
+    switch (n) {
+    case 1:
+        asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(v[0]) : "v"(p[0]) : "memory");
+        break;
+    case 2:
+        asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %3, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]) : "v"(p[0]), "v"(p[1]) : "memory");
+        break;
+    case 3:
+        asm volatile("global_load_dwordx4 %0, %3, off sc1\n\tglobal_load_dwordx4 %1, %4, off sc1\n\t"
+                     "global_load_dwordx4 %2, %5, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]) : "v"(p[0]), "v"(p[1]), "v"(p[2]) : "memory");
+        break;
+    case 4:
+        asm volatile("global_load_dwordx4 %0, %4, off sc1\n\tglobal_load_dwordx4 %1, %5, off sc1\n\t"
+                     "global_load_dwordx4 %2, %6, off sc1\n\tglobal_load_dwordx4 %3, %7, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]) : "memory");
+        break;
+    default:
+        asm volatile("global_load_dwordx4 %0, %5, off sc1\n\tglobal_load_dwordx4 %1, %6, off sc1\n\t"
+                     "global_load_dwordx4 %2, %7, off sc1\n\tglobal_load_dwordx4 %3, %8, off sc1\n\t"
+                     "global_load_dwordx4 %4, %9, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4])
+                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]) : "memory");
+        break;
+    }
+}
+// A layer's table entry, read one layer ahead: lane i loads word i, and the fields are picked out of the lanes into
+// scalar registers when the layer starts (the entry is in HBM and cold; read at the top of its layer it would
+// hold up every wave of the launch).
+__device__ __forceinline__ unsigned layer_words(const FlowLayer* t, int l, int lane) {
+    static_assert(sizeof(FlowLayer) <= 64 * 4, "one word a lane");
+    const unsigned* q = reinterpret_cast<const unsigned*>(t + l);
+    return q[lane < (int)(sizeof(FlowLayer) / 4) ? lane : 0];
+}
+template <class T>
+__device__ __forceinline__ T* lane_ptr(unsigned v, int word) {
+    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)v, word), hi = (unsigned)__builtin_amdgcn_readlane((int)v, word + 1);
+    return reinterpret_cast<T*>(((unsigned long long)hi << 32) | lo);
+}
+#define FL_PTR(T, field) lane_ptr<T>(v, (int)(offsetof(FlowLayer, field) / 4))
+__device__ __forceinline__ FlowLayer unpack_layer(unsigned v) {
+    FlowLayer L;
+    L.g1 = FL_PTR(const float, g1); L.g2 = FL_PTR(const float, g2);
+    L.wq = FL_PTR(const signed char, wq); L.wk = FL_PTR(const signed char, wk); L.wv = FL_PTR(const signed char, wv);
+    L.wo = FL_PTR(const signed char, wo); L.gate = FL_PTR(const signed char, gate); L.up = FL_PTR(const signed char, up);
+    L.down = FL_PTR(const signed char, down);
+    L.sq = FL_PTR(const float, sq); L.sk = FL_PTR(const float, sk); L.sv = FL_PTR(const float, sv); L.so = FL_PTR(const float, so);
+    L.sgate = FL_PTR(const float, sgate); L.sup = FL_PTR(const float, sup); L.sdown = FL_PTR(const float, sdown);
+    L.bq = FL_PTR(const float, bq); L.bk = FL_PTR(const float, bk); L.bv = FL_PTR(const float, bv);
+    L.Kc = FL_PTR(float, Kc); L.Vc = FL_PTR(float, Vc);
+    return L;
+}
+#undef FL_PTR
+
+constexpr int PB = 5;        // float4 pieces a thread polls at once
+// n uniform in the workgroup, 1..PB; pieces past n are left as they are
+__device__ __forceinline__ void poll_batch(const f4* const (&ptr)[PB], f4 (&v)[PB], int n, Waiter& w) {
+    long long t0 = 0;
+    bool timing = false;
+    for (;;) {
+        ldx4_n(ptr, v, n);
+        bool ok = true;
+#pragma unroll
+        for (int i = 0; i < PB; i++) ok = ok && (i >= n || ready4(v[i]));
+        if (ok || w.dead) break;
+        if (!timing) { timing = true; t0 = wall_clock64(); }
+        else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
+    }
+}
+
+// planar LDS layout of an activation vector for 16-weight chunks (as the matvec kernels use):
+// float4 k4 of the vector sits at (k4 & 3) * nch + (k4 >> 2); lane c reads a4[pl * nch + c], pl = 0..3
+__device__ __forceinline__ int slot4(int k4, int nch) { return (k4 & 3) * nch + (k4 >> 2); }
+__device__ __forceinline__ float4 tof4(f4 v) { return make_float4(v.x, v.y, v.z, v.w); }
+
+// x (optionally polled) -> LDS as x * gain; returns 1/rms.  Leaves with a barrier done.
+__device__ __forceinline__ float stage_rms(const float* x, bool polled, const float* gain, int K, float eps, float4* a4,
+                                           float* red, Waiter& w) {
+    const int K4 = K >> 2, nch = K >> 4, tid = threadIdx.x;
+    const f4* x4 = reinterpret_cast<const f4*>(x);
+    const float4* g4 = reinterpret_cast<const float4*>(gain);
+    __syncthreads();                                   // the previous phase's readers of a4 are done
+    float ss = 0.f;
+    for (int base = 0; base < K4; base += WG * PB) {
+        f4 v[PB];
+        float4 g[PB];
+        const f4* ptr[PB];
+#pragma unroll
+        for (int u = 0; u < PB; u++) {
+            const int i = min(base + u * WG + tid, K4 - 1);
+            ptr[u] = x4 + i;
+            g[u] = g4[i];
+        }
+        const int np = min(PB, (K4 - base + WG - 1) / WG);      // pieces of this round (uniform)
+#pragma unroll
+        for (int u = 0; u < PB; u++) v[u] = f4{0.f, 0.f, 0.f, 0.f};
+        if (polled) {
+            poll_batch(ptr, v, np, w);
+        } else {
+#pragma unroll
+            for (int u = 0; u < PB; u++) if (u < np) v[u] = *ptr[u];
+        }
+#pragma unroll
+        for (int u = 0; u < PB; u++) {
+            const int i = base + u * WG + tid;
+            if (i < K4) {
+                ss += v[u].x * v[u].x + v[u].y * v[u].y + v[u].z * v[u].z + v[u].w * v[u].w;
+                a4[slot4(i, nch)] = make_float4(v[u].x * g[u].x, v[u].y * g[u].y, v[u].z * g[u].z, v[u].w * g[u].w);
+            }
+        }
+    }
+    ss = wave_sum(ss);
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    __syncthreads();
+    const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+    return __builtin_amdgcn_rsqf(tot * __builtin_amdgcn_rcpf((float)K) + eps);
+}
+
+// polled x -> LDS.  Leaves with a barrier done.
+__device__ __forceinline__ void stage_plain(const float* x, int K, float4* a4, Waiter& w) {
+    const int K4 = K >> 2, nch = K >> 4, tid = threadIdx.x;
+    const f4* x4 = reinterpret_cast<const f4*>(x);
+    __syncthreads();
+    for (int base = 0; base < K4; base += WG * PB) {
+        f4 v[PB];
+        const f4* ptr[PB];
+#pragma unroll
+        for (int u = 0; u < PB; u++) { ptr[u] = x4 + min(base + u * WG + tid, K4 - 1); v[u] = f4{0.f, 0.f, 0.f, 0.f}; }
+        poll_batch(ptr, v, min(PB, (K4 - base + WG - 1) / WG), w);
+#pragma unroll
+        for (int u = 0; u < PB; u++) {
+            const int i = base + u * WG + tid;
+            if (i < K4) a4[slot4(i, nch)] = tof4(v[u]);
+        }
+    }
+    __syncthreads();
+}
+
+// chunks c0 + lane + i*64 of an int8 row (clamped inside the row: loads are unconditional)
+template <int CB>
+__device__ __forceinline__ void ld_row(const signed char* row, int nch, int lane, int c0, int4 (&wr)[CB]) {
+#pragma unroll
+    for (int i = 0; i < CB; i++) wr[i] = reinterpret_cast<const int4*>(row)[min(c0 + lane + i * 64, nch - 1)];
+}
+template <int NR, int CB>
+__device__ __forceinline__ void dot_rows(const int4 (&wr)[NR][CB], const float4* a4, int nch, int lane, int c0, float (&acc)[NR]) {
+#pragma unroll
+    for (int i = 0; i < CB; i++) {
+        const int c = c0 + lane + i * 64;
+        if (c < nch) {
+            const float4 a0 = a4[c], a1 = a4[nch + c], a2 = a4[2 * nch + c], a3 = a4[3 * nch + c];
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                float a = acc[r];
+                a = dot4_i8(wr[r][i].x, a0, a); a = dot4_i8(wr[r][i].y, a1, a);
+                a = dot4_i8(wr[r][i].z, a2, a); a = dot4_i8(wr[r][i].w, a3, a);
+                acc[r] = a;
+            }
+        }
+    }
+}
+// the rest of rows longer than the prefetched batch
+template <int NR, int CB>
+__device__ __forceinline__ void dot_rows_tail(const signed char* const (&rows)[NR], const float4* a4, int nch, int lane, float (&acc)[NR]) {
+    for (int c0 = CB * 64; c0 < nch; c0 += CB * 64) {
+        int4 wr[NR][CB];
+#pragma unroll
+        for (int r = 0; r < NR; r++) ld_row<CB>(rows[r], nch, lane, c0, wr[r]);
+        dot_rows<NR, CB>(wr, a4, nch, lane, c0, acc);
+    }
+}
+
+constexpr int CBD = 2;       // chunks a lane prefetches per row of K = dim (rows up to 2048 weights in one batch)
+constexpr int CBF = 6;       // ... per row of K = ffnDim (rows up to 6144 weights in one batch)
+constexpr int NIB = 6;       // gate/up items (a gate row and its up row) a wave holds in flight
+constexpr int NID = 2;       // down rows a wave holds in flight
+
+template <int HD>
+__global__ __launch_bounds__(WG) void flow_layers_kernel(FlowParams p) {
+    extern __shared__ float4 a4[];                     // the staged activation vector, max(dim, ffn) floats
+    __shared__ float red[4];
+    __shared__ float4 sqkv[3][HD / 4];                 // q of the head, K and V row of the current position
+    __shared__ float4 accbuf[4][HD / 4];
+    __shared__ float lbuf[4], wred[4];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int gw = blockIdx.x * 4 + wave;              // this wave among all waves of the launch
+    const int W = gridDim.x * 4;
+    const int dim = p.dim, kvDim = p.kvDim, ffn = p.ffn;
+    const int nchD = dim >> 4, nchF = ffn >> 4;
+    const FlowGeometry G = p.geo;
+    const int pos = p.state ? p.state->pos : p.posImm;
+    Waiter wt{p.limitTicks, p.err, false};
+
+    // attention geometry (decode attention of kernels.hip with one query head per workgroup, 256 threads)
+    // A thread group of 16 lanes holds a K/V row; a thread holds up to VU rows of its workgroup's tile.  The tile is
+    // FLOW_MIN_TILE positions and doubles until the partial slots cover the context: the fewer rows a thread has,
+    // the shorter the serial part of the phase (measured on the 0.5B shape at 100-200 positions: 128 beats 256
+    // by 5%, and beats 64 and 32, whose extra partials cost more to merge than the rows save).
+    constexpr int LPR = 16, NF = HD / 64, TG = WG / LPR, VU = 16 / NF;
+    const int half = HD >> 1;
+    int tile = FLOW_MIN_TILE;
+    while (pos / tile + 1 > G.smax && tile < TG * VU) tile <<= 1;
+    const int TILE = tile, VUe = tile / TG;
+
+    // timing trace (diagnostic): slot b of layer l, per workgroup, in ticks of the 100 MHz wall clock
+#define FLOW_TRACE(b) do { if (p.trace && tid == 0) \
+        p.trace[((size_t)(l - p.l0) * FLOW_TRACE_SLOTS + (b)) * gridDim.x + blockIdx.x] = wall_clock64(); } while (0)
+    unsigned lw = layer_words(p.layers, p.l0, lane);
+    for (int l = p.l0; l < p.l1; l++) {
+        const FlowLayer L = unpack_layer(lw);
+        if (l + 1 < p.l1) lw = layer_words(p.layers, l + 1, lane);
+        FLOW_TRACE(0);
+        float* X = p.xchg + (size_t)l * G.stride;
+        const bool first = l == p.l0;
+        const float* xin = first ? p.hidden : p.xchg + (size_t)(l - 1) * G.stride + G.offX2;
+
+        // ------------------------------------------------------------------ q | k | v
+        {
+            const int nq = dim >> 1, nk = kvDim >> 1, nI = nq + 2 * nk;       // RoPE pairs of q, of k; row pairs of v
+            if (blockIdx.x * 4 < nI) {
+                int it = gw;
+                int4 wr[2][CBD];
+                const signed char* rows[2] = {L.wq, L.wq};
+                int kind = 0, r0 = 0, r1 = 0;
+                float e0 = 0.f, e1 = 0.f;                // per-lane epilogue operands: lanes 0/1 scale and bias, lane 2 cos and sin
+                auto resolve = [&](int item) {
+                    const signed char* Wm; const float* sc; const float* bias;
+                    if (item < nq) { kind = 0; Wm = L.wq; sc = L.sq; bias = L.bq; const int j = item % half; r0 = (item - j) * 2 + j; r1 = r0 + half; }
+                    else if (item < nq + nk) { kind = 1; Wm = L.wk; sc = L.sk; bias = L.bk; const int i2 = item - nq; const int j = i2 % half; r0 = (i2 - j) * 2 + j; r1 = r0 + half; }
+                    else { kind = 2; Wm = L.wv; sc = L.sv; bias = L.bv; r0 = (item - nq - nk) * 2; r1 = r0 + 1; }
+                    rows[0] = Wm + (size_t)r0 * dim; rows[1] = Wm + (size_t)r1 * dim;
+                    ld_row<CBD>(rows[0], nchD, lane, 0, wr[0]);
+                    ld_row<CBD>(rows[1], nchD, lane, 0, wr[1]);
+                    e0 = 1.f; e1 = 0.f;
+                    if (lane < 2) {
+                        const int r = lane ? r1 : r0;
+                        e0 = sc[r];
+                        if (bias) e1 = bias[r];
+                    }
+                    if (lane == 2 && kind < 2) { const int j = r0 % half; e0 = p.cosRow[j]; e1 = p.sinRow[j]; }
+                };
+                if (it < nI) resolve(it);
+                const float rs = stage_rms(xin, !first, L.g1, dim, p.eps, a4, red, wt);
+                FLOW_TRACE(1);
+                for (; it < nI; it += W) {
+                    if (it != gw) resolve(it);
+                    float acc[2] = {0.f, 0.f};
+                    dot_rows<2, CBD>(wr, a4, nchD, lane, 0, acc);
+                    if (nchD > CBD * 64) dot_rows_tail<2, CBD>(rows, a4, nchD, lane, acc);
+                    acc[0] = wave_sum(acc[0]);
+                    acc[1] = wave_sum(acc[1]);
+                    float v = lane == 1 ? acc[1] : acc[0];
+                    v = v * e0;                                                  // row scale (lanes 0 and 1)
+                    v = v * rs;
+                    v = v + e1;
+                    const float v1 = dpp_f<0x101>(v);                            // lane 0 reads lane 1: the pair's second row
+                    const float cs = dpp_f<0x102>(e0), sn = dpp_f<0x102>(e1);    // lane 0 reads lane 2
+                    if (lane == 0) {
+                        float o0 = v, o1 = v1;
+                        if (kind < 2) { o0 = v * cs - v1 * sn; o1 = v * sn + v1 * cs; }      // mongoose.cu:991-1006
+                        if (kind == 0) {
+                            stx(X + G.offQ + r0, o0); stx(X + G.offQ + r1, o1);
+                        } else {                                                  // mongoose.cu:1644-1647, and the hand-over copy
+                            float* cache = (kind == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim;
+                            cache[r0] = o0; cache[r1] = o1;
+                            float* cur = X + (kind == 1 ? G.offKc : G.offVc);
+                            stx(cur + r0, o0); stx(cur + r1, o1);
+                        }
+                    }
+                }
+            }
+        }
+
+        FLOW_TRACE(2);
+        // ------------------------------------------------------------------ attention: one (head, KV split) per workgroup
+        {
+            const int nsplit = pos / TILE + 1;
+            const int split = blockIdx.x / p.nHeads, h = blockIdx.x % p.nHeads;
+            if (split < G.smax && split < nsplit) {
+                const int kvh = h / (p.nHeads / p.nKVHeads);
+                const int tg = tid / LPR, dl = tid % LPR;
+                const int t0 = split * TILE;
+                const int len = pos + 1;
+                const int t1 = min(len, t0 + TILE);
+                const int lastRow = p.maxSeq - 1;
+                const size_t rowStride = (size_t)kvDim / 4;
+                const size_t colOff = (size_t)(kvh * HD) / 4 + dl;
+                const float4* Kc4 = reinterpret_cast<const float4*>(L.Kc);
+                const float4* Vc4 = reinterpret_cast<const float4*>(L.Vc);
+                float4 kreg[VU][NF], vreg[VU][NF];
+#pragma unroll
+                for (int u = 0; u < VU; u++) {
+                    if (u >= VUe) continue;             // uniform
+                    const size_t ro = (size_t)min(t0 + tg + u * TG, lastRow) * rowStride + colOff;
+#pragma unroll
+                    for (int j = 0; j < NF; j++) kreg[u][j] = Kc4[ro + j * 16];
+#pragma unroll
+                    for (int j = 0; j < NF; j++) vreg[u][j] = Vc4[ro + j * 16];
+                }
+                __syncthreads();
+                if (tid < 3 * (HD / 4)) {
+                    const int which = tid / (HD / 4), i = tid % (HD / 4);
+                    const float* src = which == 0 ? X + G.offQ + h * HD : X + (which == 1 ? G.offKc : G.offVc) + kvh * HD;
+                    sqkv[which][i] = tof4(poll4(reinterpret_cast<const f4*>(src) + i, wt));
+                }
+                __syncthreads();
+                FLOW_TRACE(3);
+                float4 q4[NF];
+#pragma unroll
+                for (int j = 0; j < NF; j++) q4[j] = sqkv[0][j * 16 + dl];
+                const int live = t1 - t0;
+                const float scale = 1.0f / sqrtf((float)HD);
+                float sc[VU];
+                float tmax = -INFINITY;
+#pragma unroll
+                for (int u = 0; u < VU; u++) {
+                    sc[u] = -INFINITY;
+                    if (u * TG >= live) continue;
+                    const int row = t0 + tg + u * TG;
+                    if (row == pos) {                   // the current position's rows come from this launch, not from the cache
+#pragma unroll
+                        for (int j = 0; j < NF; j++) { kreg[u][j] = sqkv[1][j * 16 + dl]; vreg[u][j] = sqkv[2][j * 16 + dl]; }
+                    }
+                    float d = 0.f;
+#pragma unroll
+                    for (int j = 0; j < NF; j++) {
+                        d = fmaf(q4[j].x, kreg[u][j].x, d); d = fmaf(q4[j].y, kreg[u][j].y, d);
+                        d = fmaf(q4[j].z, kreg[u][j].z, d); d = fmaf(q4[j].w, kreg[u][j].w, d);
+                    }
+                    d = row_sum16(d);
+                    sc[u] = row < t1 ? d * scale : -INFINITY;
+                    tmax = fmaxf(tmax, sc[u]);
+                }
+                const float m = tg_max(tmax);               // the wave's maximum
+                const float mRef = m == -INFINITY ? 0.f : m;
+                float4 acc[NF];
+#pragma unroll
+                for (int j = 0; j < NF; j++) acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                float lsum = 0.f;
+#pragma unroll
+                for (int u = 0; u < VU; u++) {
+                    if (u * TG >= live) continue;
+                    const float pv = exp_neg(sc[u] - mRef);
+                    lsum += pv;
+#pragma unroll
+                    for (int j = 0; j < NF; j++) {
+                        acc[j].x = fmaf(pv, vreg[u][j].x, acc[j].x); acc[j].y = fmaf(pv, vreg[u][j].y, acc[j].y);
+                        acc[j].z = fmaf(pv, vreg[u][j].z, acc[j].z); acc[j].w = fmaf(pv, vreg[u][j].w, acc[j].w);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < NF; j++) {
+                    acc[j].x = tg_sum(acc[j].x); acc[j].y = tg_sum(acc[j].y); acc[j].z = tg_sum(acc[j].z); acc[j].w = tg_sum(acc[j].w);
+                    if (lane < LPR) accbuf[wave][j * 16 + dl] = acc[j];
+                }
+                lsum = tg_sum(lsum);
+                if (lane == 0) { lbuf[wave] = lsum; wred[wave] = m; }
+                __syncthreads();
+                if (tid < HD / 4) {
+                    const float mg_ = fmaxf(fmaxf(wred[0], wred[1]), fmaxf(wred[2], wred[3]));
+                    f4 r = {0.f, 0.f, 0.f, 0.f};
+                    float lg = 0.f;
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        const float wk = exp_neg(wred[k] - mg_);
+                        const float4 a = accbuf[k][tid];
+                        r.x = fmaf(wk, a.x, r.x); r.y = fmaf(wk, a.y, r.y); r.z = fmaf(wk, a.z, r.z); r.w = fmaf(wk, a.w, r.w);
+                        lg = fmaf(wk, lbuf[k], lg);
+                    }
+                    stx4(reinterpret_cast<f4*>(X + G.offPacc + (size_t)split * dim + h * HD) + tid, r);
+                    if (tid == 0) {
+                        stx(X + G.offPm + split * p.nHeads + h, mg_);
+                        stx(X + G.offPl + split * p.nHeads + h, lg);
+                    }
+                }
+            }
+        }
+
+        FLOW_TRACE(4);
+        // ------------------------------------------------------------------ Wo + residual
+        {
+            const int nI = dim;
+            if (blockIdx.x * 4 < nI) {
+                int it = gw;
+                int4 wr[1][CBD];
+                const signed char* rows[1] = {L.wo};
+                float e0 = 0.f, e1 = 0.f;
+                auto resolve = [&](int item) {
+                    rows[0] = L.wo + (size_t)item * dim;
+                    ld_row<CBD>(rows[0], nchD, lane, 0, wr[0]);
+                    if (lane == 0) {
+                        e0 = L.so[item];
+                        e1 = first ? xin[item] : poll1(xin + item, wt);         // there already if this workgroup staged it for q | k | v
+                    }
+                };
+                if (it < nI) resolve(it);
+                // stage the attention output: merge the KV splits' partials (running maximum, as the split-KV combine)
+                __syncthreads();
+                {
+                    const int nsplit = pos / TILE + 1;
+                    const int ns = nsplit < G.smax ? nsplit : G.smax;
+                    for (int i = tid; i < (dim >> 2); i += WG) {
+                        const int h = (i * 4) / HD;
+                        float M = -INFINITY, den = 0.f;
+                        f4 num = {0.f, 0.f, 0.f, 0.f};
+                        for (int s = 0; s < ns; s++) {
+                            const f4 a = poll4(reinterpret_cast<const f4*>(X + G.offPacc + (size_t)s * dim) + i, wt);
+                            const float ms = poll1(X + G.offPm + s * p.nHeads + h, wt);
+                            const float ls = poll1(X + G.offPl + s * p.nHeads + h, wt);
+                            const float Mn = fmaxf(M, ms);
+                            const float c = exp_neg(M - Mn);                    // first split: exp(-inf) = 0
+                            const float wgt = exp_neg(ms - Mn);
+                            den = den * c + wgt * ls;
+                            num.x = num.x * c + wgt * a.x; num.y = num.y * c + wgt * a.y;
+                            num.z = num.z * c + wgt * a.z; num.w = num.w * c + wgt * a.w;
+                            M = Mn;
+                        }
+                        const float il = __builtin_amdgcn_rcpf(den);
+                        a4[slot4(i, nchD)] = make_float4(num.x * il, num.y * il, num.z * il, num.w * il);
+                    }
+                }
+                __syncthreads();
+                FLOW_TRACE(5);
+                for (; it < nI; it += W) {
+                    if (it != gw) resolve(it);
+                    float acc[1] = {0.f};
+                    dot_rows<1, CBD>(wr, a4, nchD, lane, 0, acc);
+                    if (nchD > CBD * 64) dot_rows_tail<1, CBD>(rows, a4, nchD, lane, acc);
+                    const float v = wave_sum(acc[0]);
+                    if (lane == 0) stx(X + G.offX1 + it, e1 + v * e0);
+                }
+            }
+        }
+
+        FLOW_TRACE(6);
+        // ------------------------------------------------------------------ gate | up, SiLU(g) * u
+        {
+            const int nI = ffn;
+            if (blockIdx.x * 4 < nI) {
+                int4 wr[NIB][2][CBD];
+                float sg = 0.f, su = 0.f;
+                auto issue = [&](int it0) {
+#pragma unroll
+                    for (int k = 0; k < NIB; k++) {
+                        const int r = it0 + k * W;
+                        if (r < nI) {                                           // uniform in the wave
+                            ld_row<CBD>(L.gate + (size_t)r * dim, nchD, lane, 0, wr[k][0]);
+                            ld_row<CBD>(L.up + (size_t)r * dim, nchD, lane, 0, wr[k][1]);
+                        }
+                    }
+                    if (lane < NIB) { const int r = min(it0 + lane * W, nI - 1); sg = L.sgate[r]; su = L.sup[r]; }
+                };
+                if (gw < nI) issue(gw);
+                const float rs = stage_rms(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                FLOW_TRACE(7);
+                for (int it0 = gw; it0 < nI; it0 += NIB * W) {
+                    if (it0 != gw) issue(it0);
+                    float g = 0.f, u = 0.f;
+#pragma unroll
+                    for (int k = 0; k < NIB; k++) {
+                        float acc[2] = {0.f, 0.f};
+                        if (it0 + k * W < nI) {                                 // uniform in the wave
+                            dot_rows<2, CBD>(wr[k], a4, nchD, lane, 0, acc);
+                            if (nchD > CBD * 64) {
+                                const int r = it0 + k * W;
+                                const signed char* rows[2] = {L.gate + (size_t)r * dim, L.up + (size_t)r * dim};
+                                dot_rows_tail<2, CBD>(rows, a4, nchD, lane, acc);
+                            }
+                            acc[0] = wave_sum(acc[0]);
+                            acc[1] = wave_sum(acc[1]);
+                        }
+                        if (lane == k) { g = acc[0]; u = acc[1]; }
+                    }
+                    const int r = it0 + lane * W;
+                    if (lane < NIB && r < nI) {
+                        g = g * sg; g = g * rs;
+                        u = u * su; u = u * rs;
+                        const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f));   // mongoose.cu:949-956
+                        stx(X + G.offM + r, g * sig * u);
+                    }
+                }
+            }
+        }
+
+        FLOW_TRACE(8);
+        // ------------------------------------------------------------------ down + residual
+        {
+            const int nI = dim;
+            if (blockIdx.x * 4 < nI) {
+                int4 wr[NID][1][CBF];
+                float e0 = 0.f, e1 = 0.f;
+                auto issue = [&](int it0) {
+#pragma unroll
+                    for (int k = 0; k < NID; k++) {
+                        const int r = it0 + k * W;
+                        if (r < nI) ld_row<CBF>(L.down + (size_t)r * ffn, nchF, lane, 0, wr[k][0]);      // uniform in the wave
+                    }
+                    if (lane < NID) { const int r = min(it0 + lane * W, nI - 1); e0 = L.sdown[r]; e1 = poll1(X + G.offX1 + r, wt); }
+                };
+                if (gw < nI) issue(gw);
+                stage_plain(X + G.offM, ffn, a4, wt);
+                FLOW_TRACE(9);
+                for (int it0 = gw; it0 < nI; it0 += NID * W) {
+                    if (it0 != gw) issue(it0);
+                    float v = 0.f;
+#pragma unroll
+                    for (int k = 0; k < NID; k++) {
+                        float acc[1] = {0.f};
+                        if (it0 + k * W < nI) {
+                            dot_rows<1, CBF>(wr[k], a4, nchF, lane, 0, acc);
+                            if (nchF > CBF * 64) {
+                                const signed char* rows[1] = {L.down + (size_t)(it0 + k * W) * ffn};
+                                dot_rows_tail<1, CBF>(rows, a4, nchF, lane, acc);
+                            }
+                            acc[0] = wave_sum(acc[0]);
+                        }
+                        if (lane == k) v = acc[0];
+                    }
+                    const int r = it0 + lane * W;
+                    if (lane < NID && r < nI) {
+                        const float o = e1 + v * e0;
+                        stx(X + G.offX2 + r, o);
+                        if (l == p.l1 - 1) p.hidden[r] = o;
+                    }
+                }
+            }
+        }
+        FLOW_TRACE(10);
+    }
+}
+
+FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int headDim, int maxSeq, int grid) {
+    FlowGeometry g{};
+    // partial slots: one per FLOW_MIN_TILE positions, at most as many as the workgroups of the launch can serve
+    g.smax = (maxSeq + FLOW_MIN_TILE - 1) / FLOW_MIN_TILE;
+    if (nHeads > 0 && g.smax > grid / nHeads) g.smax = grid / nHeads;
+    if (g.smax < 1) g.smax = 1;
+    auto up64 = [](int v) { return (v + 63) & ~63; };
+    int o = 0;
+    g.offQ = o; o += up64(dim);
+    g.offKc = o; o += up64(kvDim);
+    g.offVc = o; o += up64(kvDim);
+    g.offPacc = o; o += up64(g.smax * dim);
+    g.offPm = o; o += up64(g.smax * nHeads);
+    g.offPl = o; o += up64(g.smax * nHeads);
+    g.offX1 = o; o += up64(dim);
+    g.offM = o; o += up64(ffn);
+    g.offX2 = o; o += up64(dim);
+    g.stride = o;
+    return g;
+}
+
+int flow_min_grid(int nHeads, const FlowGeometry& g) { return nHeads * g.smax; }
+// the largest tile (16 rows a thread for heads of 64, 8 for heads of 128) times the slots covers the context
+bool flow_context_fits(int headDim, int maxSeq, const FlowGeometry& g) { return (long long)(headDim == 128 ? 128 : 256) * g.smax >= maxSeq; }
+
+bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads, int headDim) {
+    if (headDim != 64 && headDim != 128) return false;
+    // the staged vector and the kernel's own 4 KB of LDS stay inside a 64 KB allocation
+    if (dim % 16 || ffn % 16 || kvDim % 16 || dim > 15360 || ffn > 15360) return false;
+    if (nKVHeads <= 0 || nHeads % nKVHeads || nHeads * headDim != dim || nKVHeads * headDim != kvDim) return false;
+    return true;
+}
+
+hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
+    if (!flow_shape_supported(p.dim, p.kvDim, p.ffn, p.nHeads, p.nKVHeads, p.headDim)) return hipErrorInvalidValue;
+    if (p.l0 < 0 || p.l1 <= p.l0 || p.l1 > p.nLayersTotal || grid < flow_min_grid(p.nHeads, p.geo) ||
+        !flow_context_fits(p.headDim, p.maxSeq, p.geo) || !p.layers || !p.xchg || !p.err || !p.hidden)
+        return hipErrorInvalidValue;
+    const size_t lds = (size_t)(p.dim > p.ffn ? p.dim : p.ffn) * sizeof(float);
+    if (p.headDim == 64) hipLaunchKernelGGL(flow_layers_kernel<64>, dim3(grid), dim3(WG), lds, s, p);
+    else hipLaunchKernelGGL(flow_layers_kernel<128>, dim3(grid), dim3(WG), lds, s, p);
+    return hipGetLastError();
+}
+
+__global__ void flow_reset_kernel(uint4* x, size_t n4) {
+    const uint4 sent = make_uint4(XSENT, XSENT, XSENT, XSENT);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) x[i] = sent;
+}
+hipError_t launch_flow_reset(float* xchg, const FlowGeometry& g, int l0, int l1, hipStream_t s) {
+    if (l1 <= l0) return hipSuccess;
+    const size_t n4 = (size_t)(l1 - l0) * g.stride / 4;
+    size_t blocks = (n4 + WG - 1) / WG;
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(flow_reset_kernel, dim3((unsigned)blocks), dim3(WG), 0, s,
+                       reinterpret_cast<uint4*>(xchg + (size_t)l0 * g.stride), n4);
+    return hipGetLastError();
+}
+
+}  // namespace mg

@@ -5,6 +5,7 @@
 // stand in for; the mg_* C functions are thin wrappers over them.
 #pragma once
 #include "kernels.h"
+#include "flow.h"
 
 #include <cstdint>
 #include <string>
@@ -90,8 +91,12 @@ public:
     int kvHalf = 0;
 
     int quantRounding = 0;
-    int execMode = 1;       // 0: one launch per reference op; 1: fused launches; 2: fused, attention launches without the L2 prefetch helpers
-    void SetExecMode(int mode) { if (mode != execMode) invalidateGraphs(); execMode = mode; }
+    // 0: one launch per reference op; 1: fused launches; 2: fused, attention launches without the L2 prefetch
+    // helpers; 3: all layers of a step in one persistent launch where the model allows it (else as 1).
+    // execAuto (until a mode is set): mode 3 only where that launch is also the faster one.
+    int execMode = 3;
+    bool execAuto = true;
+    void SetExecMode(int mode) { if (mode != execMode || execAuto) invalidateGraphs(); execMode = mode; execAuto = false; }
 
     // shape
     int dim, kvDim, headDim, nHeads, nKVHeads, ffnDim, vocabSize, nLayers, maxSeq;
@@ -143,6 +148,26 @@ private:
     bool fuseEmbed = false;      // set while the graphs are captured
     int enqueueLayerPerOp(const LayerWeights& L, int layer, int pos);
     int enqueueEmbed();
+    // persistent layer launch (flow.hip)
+public:
+    FlowGeometry flowGeo{};
+    float* flowXchg = nullptr;
+    long long* flowTrace = nullptr;
+    int FlowTrace(int enable, long long* out, size_t cap, int* dims);
+    bool FlowInUse() const { return flowEligible(0, nLayers); }
+    long long flowLimitTicks = 5000000;       // per wait of the persistent launch: 50 ms of the 100 MHz wall clock
+    void SetFlowWaitLimit(long long ticks) { invalidateGraphs(); flowLimitTicks = ticks; }
+private:
+    FlowLayer* dFlowLayers = nullptr;
+    int* dFlowErr = nullptr;
+    int* hFlowErr = nullptr;        // pinned
+    int flowGrid = 0;
+    bool flowTableDirty = true;
+    bool flowBroken = false;        // a wait ran into its limit once: the separate launches are used from then on
+    bool flowEligible(int l0, int l1) const;
+    int ensureFlow();
+    int enqueueLayersFlow(int l0, int l1, const StepState* st, int posImm, bool resetFirst);
+    int checkFlowError();
     int enqueueToken(bool withHead);      // embed -> layers -> final(+argmax) / advance, all from device state
 
     // scratch (cuda_fused_infer.go:56-69, :626)

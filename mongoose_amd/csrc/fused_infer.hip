@@ -211,6 +211,10 @@ HIPFusedInference::~HIPFusedInference() {
     for (auto& sl : layerSlabs) sl.release();
     for (auto& sl : kvSlabs) sl.release();
     if (embedTable) (void)hipFree(embedTable);
+    if (dFlowLayers) (void)hipFree(dFlowLayers);
+    if (flowXchg) (void)hipFree(flowXchg);
+    if (dFlowErr) (void)hipFree(dFlowErr);
+    if (hFlowErr) (void)hipHostFree(hFlowErr);
     if (hState) (void)hipHostFree(hState);
     if (hGate) (void)hipHostFree(hGate);
     if (hTokens) (void)hipHostFree(hTokens);
@@ -224,6 +228,7 @@ HIPFusedInference::~HIPFusedInference() {
 }
 
 int HIPFusedInference::invalidateGraphs() {
+    flowTableDirty = true;          // whatever invalidates the graphs may have moved a weight or a cache
     if (execFull) { (void)hipGraphExecDestroy(execFull); execFull = nullptr; }
     if (execPrompt) { (void)hipGraphExecDestroy(execPrompt); execPrompt = nullptr; }
     if (graphFull) { (void)hipGraphDestroy(graphFull); graphFull = nullptr; }
@@ -546,7 +551,7 @@ MvParams HIPFusedInference::downParams(const LayerWeights& L) const {
 // launch before): it need not be in by the end of this launch.
 void HIPFusedInference::planPrefetch(const LayerWeights& L, const LayerWeights* next, int layer, PfJob& job) const {
     job = PfJob{};
-    if (execMode != 1) return;
+    if (execMode != 1 && execMode != 3) return;
     const size_t budget = (size_t)12 << 20;       // measured: 10.6 MB make the attention launch 0.3 us longer, 15 MB 3 us
     const size_t l2 = (size_t)24 << 20;           // of 8 x 4 MB
     const LayerWeights* N = nullptr;
@@ -629,6 +634,143 @@ int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const
     return MG_OK;
 }
 
+// ---- all layers of a step in one persistent launch (flow.hip) ----
+bool HIPFusedInference::flowEligible(int l0, int l1) const {
+    if (execMode != 3 || flowBroken || kvHalf) return false;
+    if (!flow_shape_supported(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim)) return false;
+    if (execAuto) {
+        // Only where the step is bound by the hand-over between dependent phases, not by HBM: with hundreds of KB of
+        // weights per CU and layer the separate launches stream them faster than the persistent workgroups do.
+        const uint64_t layerBytes = (uint64_t)dim * dim * 2 + (uint64_t)kvDim * dim * 2 + (uint64_t)ffnDim * dim * 3;
+        if (nLayers < 8 || layerBytes > (64ull << 20)) return false;
+    }
+    if (l1 > nLayers) l1 = nLayers;
+    if (l0 < 0 || l0 >= l1) return false;
+    for (int l = l0; l < l1; l++) {
+        const LayerWeights& L = layers[l];
+        if (!layerComplete(L) || !kCache[l] || !vCache[l]) return false;
+        const DevMat* ms[7] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.gate, &L.up, &L.down};
+        for (const DevMat* m : ms) if (m->kind != WF_Q8) return false;
+    }
+    // one workgroup per CU, all resident at once; a (query head, KV split) per workgroup in the attention phase
+    int cus = flowGrid;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) { (void)hipGetLastError(); return false; }
+        cus = prop.multiProcessorCount;
+    }
+    const FlowGeometry g = flow_geometry(dim, kvDim, ffnDim, nHeads, headDim, maxSeq, cus);
+    return flow_min_grid(nHeads, g) <= cus && flow_context_fits(headDim, maxSeq, g);
+}
+
+int HIPFusedInference::ensureFlow() {
+    if (!dFlowLayers) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        HIPCHK(hipGetDevice(&dev));
+        HIPCHK(hipGetDeviceProperties(&prop, dev));
+        flowGrid = prop.multiProcessorCount;
+        flowGeo = flow_geometry(dim, kvDim, ffnDim, nHeads, headDim, maxSeq, flowGrid);
+        void* v = nullptr;
+        HIPCHK(hipMalloc(&v, sizeof(FlowLayer) * (size_t)nLayers));
+        dFlowLayers = static_cast<FlowLayer*>(v);
+        HIPCHK(hipMalloc(&v, sizeof(float) * (size_t)nLayers * flowGeo.stride));
+        flowXchg = static_cast<float*>(v);
+        HIPCHK(hipMalloc(&v, 256));
+        dFlowErr = static_cast<int*>(v);
+        HIPCHK(hipMemsetAsync(dFlowErr, 0, 256, stream));
+        HIPCHK(hipHostMalloc(&v, 64, hipHostMallocDefault));
+        hFlowErr = static_cast<int*>(v);
+        *hFlowErr = 0;
+        flowTableDirty = true;
+    }
+    if (flowTableDirty) {
+        std::vector<FlowLayer> t((size_t)nLayers);
+        for (int l = 0; l < nLayers; l++) {
+            const LayerWeights& L = layers[l];
+            FlowLayer& F = t[l];
+            F = FlowLayer{};
+            F.g1 = L.norm1; F.g2 = L.norm2;
+            auto w8 = [](const DevMat& m) { return static_cast<const signed char*>(m.w); };
+            F.wq = w8(L.wq); F.wk = w8(L.wk); F.wv = w8(L.wv); F.wo = w8(L.wo); F.gate = w8(L.gate); F.up = w8(L.up); F.down = w8(L.down);
+            F.sq = L.wq.scales; F.sk = L.wk.scales; F.sv = L.wv.scales; F.so = L.wo.scales;
+            F.sgate = L.gate.scales; F.sup = L.up.scales; F.sdown = L.down.scales;
+            F.bq = L.bq; F.bk = L.bk; F.bv = L.bv;
+            F.Kc = kCache[l]; F.Vc = vCache[l];
+        }
+        HIPCHK(hipStreamSynchronize(stream));
+        HIPCHK(hipMemcpy(dFlowLayers, t.data(), sizeof(FlowLayer) * (size_t)nLayers, hipMemcpyHostToDevice));
+        flowTableDirty = false;
+    }
+    return MG_OK;
+}
+
+// Diagnostic: per-workgroup timestamps of the persistent launch (flow.h: FLOW_TRACE_SLOTS per layer).  enable != 0
+// starts recording (graphs are re-captured with the trace pointer), out != NULL copies the last launch's ticks
+// [layer][slot][workgroup] (100 MHz wall clock), dims gets {layers, slots, workgroups}; enable == 0 stops.
+int HIPFusedInference::FlowTrace(int enable, long long* out, size_t cap, int* dims) {
+    if (!flowEligible(0, nLayers)) { set_error("flow trace: the persistent launch is not in use for this model (exec mode, weight kinds, shape)"); return MG_E_STATE; }
+    if (int rc = ensureFlow()) return rc;
+    const size_t n = (size_t)nLayers * FLOW_TRACE_SLOTS * (size_t)flowGrid;
+    HIPCHK(hipStreamSynchronize(stream));
+    if (dims) { dims[0] = nLayers; dims[1] = FLOW_TRACE_SLOTS; dims[2] = flowGrid; }
+    if (enable && !flowTrace) {
+        void* v = nullptr;
+        HIPCHK(hipMalloc(&v, sizeof(long long) * n));
+        flowTrace = static_cast<long long*>(v);
+        HIPCHK(hipMemset(v, 0, sizeof(long long) * n));
+        invalidateGraphs();
+    }
+    if (out && flowTrace) {
+        if (cap < n) { set_error("flow trace: buffer too small"); return MG_E_ARG; }
+        HIPCHK(hipMemcpy(out, flowTrace, sizeof(long long) * n, hipMemcpyDeviceToHost));
+    }
+    if (!enable && flowTrace) {
+        invalidateGraphs();
+        (void)hipFree(flowTrace);
+        flowTrace = nullptr;
+    }
+    return MG_OK;
+}
+
+int HIPFusedInference::enqueueLayersFlow(int l0, int l1, const StepState* st, int posImm, bool resetFirst) {
+    if (l1 > nLayers) l1 = nLayers;
+    FlowParams p{};
+    p.layers = dFlowLayers; p.l0 = l0; p.l1 = l1; p.nLayersTotal = nLayers;
+    p.dim = dim; p.kvDim = kvDim; p.ffn = ffnDim; p.nHeads = nHeads; p.nKVHeads = nKVHeads; p.headDim = headDim; p.maxSeq = maxSeq;
+    p.eps = eps;
+    p.state = st; p.posImm = posImm;
+    const int half = headDim / 2;
+    p.cosRow = st ? ropeCur : cosTab + (size_t)posImm * half;
+    p.sinRow = st ? ropeCur + half : sinTab + (size_t)posImm * half;
+    p.hidden = hidden[hiddenIdx];
+    p.xchg = flowXchg; p.geo = flowGeo;
+    p.err = dFlowErr;
+    p.limitTicks = flowLimitTicks;
+    p.trace = flowTrace;
+    if (resetFirst) HIPCHK(launch_flow_reset(flowXchg, flowGeo, l0, l1, stream));
+    if (mark(1)) return MG_E_HIP;
+    HIPCHK(launch_flow_layers(p, flowGrid, stream));
+    return MG_OK;
+}
+
+// After a synchronisation: did a wait of the persistent launch give up?  (Its workgroups were then not all
+// resident at once -- a GPU shared with other work, fewer CUs than reported.)  The step's results are not
+// valid; later steps use the separate launches.
+int HIPFusedInference::checkFlowError() {
+    if (!dFlowErr) return MG_OK;
+    HIPCHK(hipMemcpy(hFlowErr, dFlowErr, sizeof(int), hipMemcpyDeviceToHost));
+    if (*hFlowErr == 0) return MG_OK;
+    *hFlowErr = 0;
+    HIPCHK(hipMemset(dFlowErr, 0, sizeof(int)));
+    flowBroken = true;
+    invalidateGraphs();
+    set_error("persistent layer launch: a wait between phases ran into its time limit (workgroups not all resident at once?); "
+              "this step's results are invalid, later steps use the separate launches");
+    return MG_E_HIP;
+}
+
 int HIPFusedInference::enqueueLayer(const LayerWeights& L, int layer, const StepState* st, int posImm) {
     if (!kCache[layer] || !vCache[layer]) { set_error("layer has no KV cache: call SetLayerRange first"); return MG_E_STATE; }
     if (!layerComplete(L)) { set_error("layer weights incomplete"); return MG_E_STATE; }
@@ -649,6 +791,12 @@ int HIPFusedInference::enqueueFinal(bool withArgmax) {
     p.seg[0] = MvSeg{lmHead.w, lmHead.scales, nullptr, logits, vocabSize};
     p.nseg = 1; p.K = dim; p.act = hidden[hiddenIdx]; p.gain = finalNorm; p.eps = eps;
     p.amaxVal = amaxVal; p.amaxIdx = amaxIdx;
+    if (fuseEmbed && flowEligible(0, nLayers)) {
+        // inside the captured token: the lm_head launch also leaves the exchange area of the persistent
+        // layer launch in its "nothing written yet" state for the next token (one launch saved)
+        p.xreset = reinterpret_cast<unsigned*>(flowXchg);
+        p.xresetWords = (unsigned)((size_t)nLayers * flowGeo.stride);
+    }
     MvConfig c{0, 0, 0};
     if (mark(6)) return MG_E_HIP;
     HIPCHK(launch_matvec(lmHead.kind, EPI_ARGMAX, PRO_RMS, p, &c, stream));
@@ -670,20 +818,30 @@ int HIPFusedInference::PartialStep(const float* hiddenIn, int pos, int layerStar
         HIPCHK(hipStreamSynchronize(stream));
         HIPCHK(hipMemcpy(h, hiddenIn, (size_t)dim * 4, hipMemcpyHostToDevice));      // :395
     }
-    for (int l = layerStart; l < layerEnd && l < nLayers; l++) {
-        if (!layers[l].norm1) continue;                                               // :415
-        int rc = enqueueLayer(layers[l], l, nullptr, pos);
+    if (flowEligible(layerStart, layerEnd)) {
+        int rc = ensureFlow();
+        if (rc == 0) rc = enqueueLayersFlow(layerStart, layerEnd, nullptr, pos, true);
         if (rc) return rc;
+    } else {
+        for (int l = layerStart; l < layerEnd && l < nLayers; l++) {
+            if (!layers[l].norm1) continue;                                           // :415
+            int rc = enqueueLayer(layers[l], l, nullptr, pos);
+            if (rc) return rc;
+        }
     }
     if (layerEnd >= nLayers && logitsOut && finalNorm) {                              // :446
         int rc = enqueueFinal(false);
         if (rc) return rc;
         HIPCHK(hipStreamSynchronize(stream));
         HIPCHK(hipMemcpy(logitsOut, logits, (size_t)vocabSize * 4, hipMemcpyDeviceToHost));
+        rc = checkFlowError();
+        if (rc) return rc;
     }
     if (hiddenOut && layerEnd < nLayers) {                                            // :452
         HIPCHK(hipStreamSynchronize(stream));
         HIPCHK(hipMemcpy(hiddenOut, h, (size_t)dim * 4, hipMemcpyDeviceToHost));
+        int rc = checkFlowError();
+        if (rc) return rc;
     }
     return MG_OK;      // nothing read back: the launches stay queued (the reference does not sync here either)
 }
@@ -772,7 +930,7 @@ int HIPFusedInference::ExportHidden(float* out) {
     ARGCHK(out, "ExportHidden: NULL out");
     HIPCHK(hipStreamSynchronize(stream));
     HIPCHK(hipMemcpy(out, hidden[hiddenIdx], (size_t)dim * 4, hipMemcpyDeviceToHost));
-    return MG_OK;
+    return checkFlowError();
 }
 
 int HIPFusedInference::enqueueEmbed() {
@@ -802,17 +960,31 @@ EmbedRef HIPFusedInference::embedRef() const {
     e.out = hidden[hiddenIdx]; e.dim = dim; e.vocab = vocabSize;
     return e;
 }
-int HIPFusedInference::primeGraph() { return enqueueEmbed(); }
+int HIPFusedInference::primeGraph() {
+    int rc = enqueueEmbed();
+    if (rc) return rc;
+    // a captured token leaves the exchange area reset for its successor; the first one finds it so here
+    if (flowEligible(0, nLayers)) HIPCHK(launch_flow_reset(flowXchg, flowGeo, 0, nLayers, stream));
+    return MG_OK;
+}
 
 int HIPFusedInference::enqueueToken(bool withHead) {
     int rc = fuseEmbed ? MG_OK : enqueueEmbed();
     if (rc) return rc;
-    for (int l = 0; l < nLayers; l++) {
-        rc = enqueueLayer(layers[l], l, dState, 0);
+    const bool flow = flowEligible(0, nLayers);
+    if (flow) {
+        rc = ensureFlow();
+        if (rc == 0) rc = enqueueLayersFlow(0, nLayers, dState, 0, !fuseEmbed);
         if (rc) return rc;
+    } else {
+        for (int l = 0; l < nLayers; l++) {
+            rc = enqueueLayer(layers[l], l, dState, 0);
+            if (rc) return rc;
+        }
     }
     if (withHead) return enqueueFinal(true);
     HIPCHK(launch_advance_prompt(dState, dPrompt, ropeRef(), embedRef(), stream));
+    if (flow && fuseEmbed) HIPCHK(launch_flow_reset(flowXchg, flowGeo, 0, nLayers, stream));    // captured prompt step: no lm_head launch to do it
     return MG_OK;
 }
 
@@ -847,7 +1019,7 @@ int HIPFusedInference::DecodeToken(int token, int pos, int* nextToken, float* lo
     HIPCHK(hipStreamSynchronize(stream));
     if (nextToken) *nextToken = hTokens[0];
     if (logitsOut) HIPCHK(hipMemcpy(logitsOut, logits, (size_t)vocabSize * 4, hipMemcpyDeviceToHost));
-    return MG_OK;
+    return checkFlowError();
 }
 
 int HIPFusedInference::GraphCapture() {
@@ -856,6 +1028,7 @@ int HIPFusedInference::GraphCapture() {
     if (rc) return rc;
     if (execFull && execPrompt) return MG_OK;
     invalidateGraphs();
+    if (flowEligible(0, nLayers)) { rc = ensureFlow(); if (rc) return rc; }     // allocations and uploads come before the capture
     HIPCHK(hipStreamSynchronize(stream));
     for (int which = 0; which < 2; which++) {
         HIPCHK(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));
@@ -885,7 +1058,7 @@ int HIPFusedInference::GraphLaunch(int token, int pos, int* nextToken) {
     HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int), hipMemcpyDeviceToHost, stream));
     HIPCHK(hipStreamSynchronize(stream));
     if (nextToken) *nextToken = hTokens[0];
-    return MG_OK;
+    return checkFlowError();
 }
 
 int HIPFusedInference::GraphValidate(int token, int pos, float* maxAbsDiff) {
@@ -893,7 +1066,7 @@ int HIPFusedInference::GraphValidate(int token, int pos, float* maxAbsDiff) {
     std::vector<float> a(vocabSize), b(vocabSize);
     int t0 = -1, t1 = -1;
     int saved = execMode;
-    execMode = 1;
+    if (execMode == 0) execMode = 1;         // the per-op launches are not captured: compare the graph with the fused launches
     int rc = DecodeToken(token, pos, &t0, a.data());
     execMode = saved;
     if (rc) return rc;
@@ -942,7 +1115,7 @@ int HIPFusedInference::Generate(const int* prompt, int nPrompt, int nDecode, int
     if (nDecode > 0) HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int) * (size_t)nDecode, hipMemcpyDeviceToHost, stream));
     HIPCHK(hipStreamSynchronize(stream));
     for (int i = 0; i < nDecode; i++) outTokens[i] = hTokens[i];
-    return MG_OK;
+    return checkFlowError();
 }
 
 int HIPFusedInference::TimedDecode(int token, int pos, int steps, bool useGraph, float* elapsedMs) {
@@ -964,7 +1137,7 @@ int HIPFusedInference::TimedDecode(int token, int pos, int steps, bool useGraph,
     float ms = 0.f;
     HIPCHK(hipEventElapsedTime(&ms, ev0, ev1));
     if (elapsedMs) *elapsedMs = ms;
-    return MG_OK;
+    return checkFlowError();
 }
 
 // Per-launch-class durations inside a token.  Events cannot be read back from
@@ -1150,7 +1323,7 @@ int HIPFusedInference::GeneratePrefill(const int* prompt, int nPrompt, int nDeco
     HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int) * (size_t)nDecode, hipMemcpyDeviceToHost, stream));
     HIPCHK(hipStreamSynchronize(stream));
     for (int i = 0; i < nDecode; i++) outTokens[i] = hTokens[i];
-    return MG_OK;
+    return checkFlowError();
 }
 
 }  // namespace mg
@@ -1207,7 +1380,7 @@ int mg_swap_hidden_buffer(mg_ctx* c) { CTX(c); return f->SwapHiddenBuffer(); }
 int mg_hidden_idx(mg_ctx* c) { CTX(c); return f->hiddenIdx; }
 int mg_set_exec_mode(mg_ctx* c, int mode) {
     CTX(c);
-    if (mode < 0 || mode > 2) { mg::set_error("exec mode must be 0, 1 or 2"); return MG_E_ARG; }
+    if (mode < 0 || mode > 3) { mg::set_error("exec mode must be 0, 1, 2 or 3"); return MG_E_ARG; }
     f->SetExecMode(mode);
     return MG_OK;
 }
@@ -1229,6 +1402,37 @@ int mg_prefill(mg_ctx* c, const int* tokens, int nTokens, int pos0, int* next, f
 }
 int mg_generate_prefill(mg_ctx* c, const int* prompt, int nPrompt, int nDecode, int* out) {
     CTX(c); return f->GeneratePrefill(prompt, nPrompt, nDecode, out);
+}
+// Inspection of the persistent layer launch's exchange area after a step (for tests): copies layer `layer`'s
+// block into out (cap floats) and writes its geometry {stride, offQ, offKc, offVc, offPacc, offPm, offPl,
+// offX1, offM, offX2, smax} into geo[11].  MG_E_STATE when that launch has not been set up.
+int mg_flow_exchange(mg_ctx* c, int layer, float* out, size_t cap, int* geo) {
+    CTX(c);
+    if (!f->flowXchg || layer < 0 || layer >= f->nLayers) { mg::set_error("mg_flow_exchange: no exchange area (or bad layer)"); return MG_E_STATE; }
+    const mg::FlowGeometry& g = f->flowGeo;
+    if (geo) {
+        const int v[11] = {g.stride, g.offQ, g.offKc, g.offVc, g.offPacc, g.offPm, g.offPl, g.offX1, g.offM, g.offX2, g.smax};
+        for (int i = 0; i < 11; i++) geo[i] = v[i];
+    }
+    if (out) {
+        if (hipStreamSynchronize(f->stream) != hipSuccess) return MG_E_HIP;
+        const size_t n = cap < (size_t)g.stride ? cap : (size_t)g.stride;
+        if (hipMemcpy(out, f->flowXchg + (size_t)layer * g.stride, n * 4, hipMemcpyDeviceToHost) != hipSuccess) return MG_E_HIP;
+    }
+    return MG_OK;
+}
+int mg_flow_in_use(mg_ctx* c) {
+    if (!c || !c->f) return 0;
+    return c->f->FlowInUse() ? 1 : 0;
+}
+int mg_flow_set_wait_limit(mg_ctx* c, long long ticks) {
+    CTX(c);
+    f->SetFlowWaitLimit(ticks);
+    return MG_OK;
+}
+int mg_flow_trace(mg_ctx* c, int enable, long long* out, size_t cap, int* dims) {
+    CTX(c);
+    return f->FlowTrace(enable, out, cap, dims);
 }
 uint64_t mg_weight_bytes_per_token(const mg_ctx* c) { return c && c->f ? c->f->WeightBytesPerToken() : 0; }
 uint64_t mg_kv_bytes_at(const mg_ctx* c, int pos) { return c && c->f ? c->f->KVBytesAt(pos) : 0; }

@@ -68,6 +68,11 @@ struct MvParams {
     int div127;           // Q8: multiply by scales[r]/127 instead of scales[r]
     float* amaxVal;       // EPI_ARGMAX partials [gridDim.x]
     int* amaxIdx;
+    // EPI_ARGMAX, optional: xresetWords 32-bit words at xreset (a multiple of 4, 16-byte aligned) are filled
+    // with 0xFFFFFFFF by the launch's workgroups -- the exchange area of the persistent layer launch, which
+    // must read "nothing written yet" before the next token
+    unsigned* xreset;
+    unsigned xresetWords;
 };
 
 struct MvConfig { int nr; int ks; int grid; };

@@ -9,102 +9,9 @@
 // once in the epilogue; norm, bias, residual, SiLU*mul and argmax are folded
 // into its prologue/epilogue so a layer is five launches instead of seventeen.
 #include "kernels.h"
-#include <limits.h>
-#include <math.h>
+#include "device_util.h"
 
 namespace mg {
-
-constexpr int WG = 256;
-
-// ---------------------------------------------------------------------------
-// wave64 / workgroup reductions
-// ---------------------------------------------------------------------------
-// Lane exchange inside a row of 16 lanes through DPP (no LDS traffic):
-// quad_perm [1,0,3,2] = 0xB1, quad_perm [2,3,0,1] = 0x4E, row_ror:4 = 0x124, row_ror:8 = 0x128.
-template <int CTRL>
-__device__ __forceinline__ float dpp_f(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
-}
-// Exchange between the four rows of 16 lanes, in the VALU instead of through the LDS crossbar
-// (ds_bpermute): v_permlane16_swap exchanges the odd rows of its first operand with the even rows of
-// its second, v_permlane32_swap the upper half of the first with the lower half of the second.  With
-// the same value in both operands the two results are (own, partner) or (partner, own) in every lane:
-// their sum / maximum is v combined with the lane 16 (32) away, and since both operations are
-// commutative the bits are those of v op shfl_xor(v, 16 / 32).
-__device__ __forceinline__ void row_swap16(float& a, float& b) {
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-}
-__device__ __forceinline__ void row_swap32(float& a, float& b) {
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-}
-__device__ __forceinline__ float rows_sum(float v) {      // over lanes l, l^16, l^32, l^48
-    float a = v, b = v;
-    row_swap16(a, b);
-    a = a + b; b = a;
-    row_swap32(a, b);
-    return a + b;
-}
-__device__ __forceinline__ float rows_max(float v) {
-    float a = v, b = v;
-    row_swap16(a, b);
-    a = fmaxf(a, b); b = a;
-    row_swap32(a, b);
-    return fmaxf(a, b);
-}
-// Greatest value of the wave and, among equals, its lowest index, in every lane: the combination is
-// symmetric and idempotent, so it does not matter which of the two operands is the lane's own.
-__device__ __forceinline__ void argmax_pick(float& v, int& i, float ov, int oi) {
-    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
-}
-template <int CTRL>
-__device__ __forceinline__ int dpp_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true); }
-__device__ __forceinline__ void wave_argmax(float& v, int& i) {
-    float va = v, vb = v;
-    float ia = __builtin_bit_cast(float, i), ib = ia;
-    row_swap32(va, vb); row_swap32(ia, ib);
-    v = va; i = __builtin_bit_cast(int, ia);
-    argmax_pick(v, i, vb, __builtin_bit_cast(int, ib));
-    va = v; vb = v; ia = __builtin_bit_cast(float, i); ib = ia;
-    row_swap16(va, vb); row_swap16(ia, ib);
-    v = va; i = __builtin_bit_cast(int, ia);
-    argmax_pick(v, i, vb, __builtin_bit_cast(int, ib));
-    argmax_pick(v, i, dpp_f<0x128>(v), dpp_i<0x128>(i));     // row_ror:8, row_ror:4, then the quad
-    argmax_pick(v, i, dpp_f<0x124>(v), dpp_i<0x124>(i));
-    argmax_pick(v, i, dpp_f<0x4E>(v), dpp_i<0x4E>(i));
-    argmax_pick(v, i, dpp_f<0xB1>(v), dpp_i<0xB1>(i));
-}
-__device__ __forceinline__ float wave_sum(float v) {
-    v += dpp_f<0xB1>(v);
-    v += dpp_f<0x4E>(v);
-    v += dpp_f<0x124>(v);
-    v += dpp_f<0x128>(v);
-    return rows_sum(v);
-}
-__device__ __forceinline__ float wave_max(float v) {
-    v = fmaxf(v, dpp_f<0xB1>(v));
-    v = fmaxf(v, dpp_f<0x4E>(v));
-    v = fmaxf(v, dpp_f<0x124>(v));
-    v = fmaxf(v, dpp_f<0x128>(v));
-    return rows_max(v);
-}
-// Sum over the 256 threads of a workgroup; every thread gets the result.
-// red: 4 floats of LDS.  Two barriers, so red can be reused right after.
-__device__ __forceinline__ float block_sum(float v, float* red) {
-    v = wave_sum(v);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float t = (red[0] + red[1]) + (red[2] + red[3]);
-    __syncthreads();
-    return t;
-}
-__device__ __forceinline__ float block_max(float v, float* red) {
-    v = wave_max(v);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float t = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    __syncthreads();
-    return t;
-}
 
 // ---------------------------------------------------------------------------
 // Activation vector in LDS.  A lane owns a weight chunk of 16 weights: 16
@@ -184,40 +91,6 @@ __device__ __forceinline__ float stage_activation(const MvParams& p, float4* a4,
     return __builtin_amdgcn_rsqf(tot * __builtin_amdgcn_rcpf((float)p.K) + p.eps);   // 1 ulp each; the reference's rsqrtf (mongoose.cu:170) is no closer
 }
 
-// ---------------------------------------------------------------------------
-// Chunk dot products
-// ---------------------------------------------------------------------------
-__device__ __forceinline__ float dot4_i8(int w, float4 a, float acc) {
-    acc = fmaf((float)(int)(signed char)(w & 0xff), a.x, acc);
-    acc = fmaf((float)(int)(signed char)((w >> 8) & 0xff), a.y, acc);
-    acc = fmaf((float)(int)(signed char)((w >> 16) & 0xff), a.z, acc);
-    acc = fmaf((float)(w >> 24), a.w, acc);
-    return acc;
-}
-// sum over 4 bytes of a * nibble; n holds one nibble per byte (0..15).  The -8
-// offset of Q4_0 is applied once per chunk from the sum of its activations.
-template <int B>
-__device__ __forceinline__ float cvt_ubyte(unsigned n) {
-    // v_cvt_f32_ubyteN straight from the masked dword: one convert per weight; written out
-    // because the compiler otherwise re-derives every nibble with its own bit-field extract
-    float f;
-    if (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(n));
-    else if (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(n));
-    else if (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(n));
-    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(n));
-    return f;
-}
-__device__ __forceinline__ float dot4_nib(unsigned n, float4 a, float acc) {
-    acc = fmaf(cvt_ubyte<0>(n), a.x, acc);
-    acc = fmaf(cvt_ubyte<1>(n), a.y, acc);
-    acc = fmaf(cvt_ubyte<2>(n), a.z, acc);
-    acc = fmaf(cvt_ubyte<3>(n), a.w, acc);
-    return acc;
-}
-__device__ __forceinline__ float half_bits_to_float(unsigned short h) {
-    return (float)__builtin_bit_cast(_Float16, h);
-}
-
 // av[0..3]: the chunk's activations (4 float4), asum: their sum (Q4 only).
 template <int WF> struct Fmt;
 template <> struct Fmt<WF_Q8> {
@@ -294,6 +167,14 @@ template <> struct Fmt<WF_Q4RAW> {
 // ---------------------------------------------------------------------------
 struct RowRef { int seg; int row; bool valid; };
 
+// Every workgroup of the launch fills its share of [x, x + words) with 0xFFFFFFFF (16 bytes a store).
+__device__ __forceinline__ void fill_unset(unsigned* x, unsigned words) {
+    if (!x) return;
+    const unsigned n4 = words >> 2;
+    const uint4 v = make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu);
+    for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += gridDim.x * blockDim.x) reinterpret_cast<uint4*>(x)[i] = v;
+}
+
 template <int NR, int EPI>
 __device__ __forceinline__ RowRef resolve_row(const MvParams& p, int g, int i) {
     RowRef r;
@@ -352,6 +233,8 @@ __global__ __launch_bounds__(WG) void matvec_kernel(MvParams p) {
     const int gStep = KS == 1 ? gridDim.x * 4 : gridDim.x;
     const int myGroups = gStart >= p.ngroups ? 0 : ((ONCE && KS == 1) ? 1 : (p.ngroups - gStart + gStep - 1) / gStep);
     const int nItems = myGroups * iters;
+
+    if (EPI == EPI_ARGMAX) fill_unset(p.xreset, p.xresetWords);
 
     int pos = 0;
     if (EPI == EPI_QKV) {
@@ -640,6 +523,7 @@ __global__ __launch_bounds__(WG) void matvec_rows_q8_kernel(MvParams p) {
         if (lane < NR && gg * NR + lane < nrows) scl = scales[gg * NR + lane];
     };
     if (g * NR < nrows) fetch(g);                    // the first rows go out before the vector is staged
+    if (EPI == EPI_ARGMAX) fill_unset(p.xreset, p.xresetWords);
 
     const float rs = stage_activation<WF_Q8, PRO_RMS>(p, a4, red);
     float4 av[CH * 4];
@@ -733,6 +617,7 @@ __global__ __launch_bounds__(WG) void matvec_rows_q4_kernel(MvParams p) {
         }
     };
     if (g * NR * 2 < nrows) fetch(g);
+    if (EPI == EPI_ARGMAX) fill_unset(p.xreset, p.xresetWords);
 
     const float rs = stage_activation<WF_Q4P, PRO_RMS>(p, a4, red);
     // half block h of the lane's block: low nibbles meet lo[h][0..1], high nibbles hi[h][0..1]
@@ -1070,27 +955,6 @@ hipError_t launch_matvec_generic_q8(const float* act, const void* w, const float
 // With several splits the last workgroup of a column to finish combines the
 // partials, so the output is always the final [dim] vector.
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ float ld_agent(const float* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void st_agent(float* p, float v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// Sum over the 16 lanes (one DPP row) that hold a K/V row.  Every step adds a lane's value to its
-// mirror partner's (quad_perm, then row_half_mirror = 0x141, row_mirror = 0x140), so both partners
-// compute the same commutative sum: all lanes of the row end with the same bits, which keeps
-// exp(score - max) identical across the lanes that apply it.
-__device__ __forceinline__ float row_sum16(float v) {
-    v += dpp_f<0xB1>(v);
-    v += dpp_f<0x4E>(v);
-    v += dpp_f<0x141>(v);
-    v += dpp_f<0x140>(v);
-    return v;
-}
-// combine a per-thread value over the four row groups (tg) that share a wave
-__device__ __forceinline__ float tg_max(float v) { return rows_max(v); }
-__device__ __forceinline__ float tg_sum(float v) { return rows_sum(v); }
-
 // One float4 of a cache row: fp32 rows are read as they are, fp16 rows as 8 bytes and widened.
 template <bool KVH>
 __device__ __forceinline__ float4 ld_kv4(const void* base, size_t idx4) {
@@ -1140,11 +1004,6 @@ __device__ __forceinline__ void prefetch_helper(const PfJob& job, int firstFlat,
     }
     asm volatile("s_waitcnt vmcnt(0)" : "+v"(sink) : : "memory");
 }
-
-// exp(x) for x <= 0 as one multiply and the hardware's 2^x (1 ulp; the product x * log2(e) adds
-// |x| * 2^-24 relative, 2e-6 at x = -20): the library's expf is a dozen instructions, and a thread
-// of the decode attention, at one or two waves a SIMD, pays the latency of every one of them.
-__device__ __forceinline__ float exp_neg(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
 
 template <int HD, int GMAX, bool KVH, int AWG = WG>
 __global__ __launch_bounds__(AWG) void attn_decode_kernel(AttnParams p) {

@@ -394,7 +394,8 @@ class HIPFusedInference:
         return lib.mg_reset_kv(self._h)
 
     def SetExecMode(self, mode):
-        """0 = one launch per reference op, 1 = fused launches (default), 2 = fused without the L2 prefetch helpers."""
+        """0 = one launch per reference op, 1 = fused launches, 2 = fused without the L2 prefetch helpers,
+        3 (default) = all layers in one persistent launch where the model allows it."""
         return lib.mg_set_exec_mode(self._h, mode)
 
     # L3 bridge and mailbox (cuda_fused_infer.go:556-737)
@@ -494,6 +495,45 @@ class HIPFusedInference:
         out = np.zeros(max(nDecode, 1), dtype=np.int32)
         rc = lib.mg_generate_prefill(self._h, _ip(p), len(p), nDecode, _ip(out))
         return rc, out[:nDecode]
+
+    def FlowExchange(self, layer):
+        """The persistent layer launch's exchange block of `layer` after the last step, as a dict of named
+        vectors (tests); None when that launch is not in use."""
+        geo = np.zeros(11, dtype=np.int32)
+        if not self.FlowInUse() or lib.mg_flow_exchange(self._h, layer, None, 0, _ip(geo)) != 0:
+            return None
+        buf = np.empty(int(geo[0]), dtype=np.float32)
+        if lib.mg_flow_exchange(self._h, layer, _fp(buf), buf.size, _ip(geo)) != 0:
+            return None
+        stride, oq, okc, ovc, opa, opm, opl, ox1, om, ox2, smax = [int(x) for x in geo]
+        kv = self.kvDim
+        return {"q": buf[oq:oq + self.dim], "k": buf[okc:okc + kv], "v": buf[ovc:ovc + kv],
+                "pacc": buf[opa:opa + smax * self.dim].reshape(smax, self.dim),
+                "pm": buf[opm:opm + smax * self.nHeads].reshape(smax, self.nHeads),
+                "pl": buf[opl:opl + smax * self.nHeads].reshape(smax, self.nHeads),
+                "x1": buf[ox1:ox1 + self.dim], "m": buf[om:om + self.ffnDim], "x2": buf[ox2:ox2 + self.dim], "smax": smax}
+
+    FLOW_TRACE_POINTS = ("layer-top", "qkv-input-staged", "qkv-done", "q-k-v-rows-in", "attention-done", "attention-merged",
+                         "wo-done", "gate-up-input-staged", "gate-up-done", "down-input-staged", "down-done")
+
+    def FlowTrace(self, enable=True, read=False):
+        """Timing diagnostic of the persistent layer launch (mg_flow_trace).  enable starts / stops recording;
+        read=True returns the last launch's ticks (10 ns) as an int64 array [layer, point, workgroup]."""
+        dims = np.zeros(3, dtype=np.int32)
+        rc = lib.mg_flow_trace(self._h, 1 if enable else 0, None, 0, _ip(dims))
+        if rc != 0 or not read:
+            return rc, None
+        buf = np.zeros(int(dims[0]) * int(dims[1]) * int(dims[2]), dtype=np.int64)
+        rc = lib.mg_flow_trace(self._h, 1, buf.ctypes.data_as(ctypes.POINTER(ctypes.c_longlong)), buf.size, _ip(dims))
+        return rc, buf.reshape(int(dims[0]), int(dims[1]), int(dims[2]))
+
+    def FlowInUse(self):
+        """True when a step over all layers goes through the persistent layer launch."""
+        return lib.mg_flow_in_use(self._h) == 1
+
+    def SetFlowWaitLimit(self, ticks):
+        """Per-wait time limit of the persistent layer launch in 10 ns ticks (negative: give up at once)."""
+        return lib.mg_flow_set_wait_limit(self._h, int(ticks))
 
     def WeightBytesPerToken(self):
         return lib.mg_weight_bytes_per_token(self._h)

@@ -105,6 +105,10 @@ _sig("mg_profile_decode", c_int, c_void_p, c_int, c_int, c_int, ctypes.c_uint, _
 _sig("mg_prefill", c_int, c_void_p, _i, c_int, c_int, _i, _f, _f)
 _sig("mg_generate_prefill", c_int, c_void_p, _i, c_int, c_int, _i)
 _sig("mg_bench_matvec", c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _f)
+_sig("mg_flow_exchange", c_int, c_void_p, c_int, _f, c_size_t, _i)
+_sig("mg_flow_in_use", c_int, c_void_p)
+_sig("mg_flow_set_wait_limit", c_int, c_void_p, ctypes.c_longlong)
+_sig("mg_flow_trace", c_int, c_void_p, c_int, ctypes.POINTER(ctypes.c_longlong), c_size_t, _i)
 _sig("mg_weight_bytes_per_token", c_uint64, c_void_p)
 _sig("mg_kv_bytes_at", c_uint64, c_void_p, c_int)
 _sig("mg_stream_build", c_void_p, c_void_p)

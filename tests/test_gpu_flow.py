@@ -1,0 +1,203 @@
+"""The persistent layer launch (exec mode 3): all layers of a decode step in one launch whose workgroups hand
+their vectors over through an exchange area in device memory.
+
+* every vector a phase hands over (q, K row, V row, attention partials, hidden after the attention block, SwiGLU
+  vector, layer output), read back from the exchange area, against a float64 numpy evaluation of the layer
+  (cuda_fused_infer.go:414-444 order, kernels/mongoose.cu:145-174, 856-933, 949-956, 991-1006 arithmetic);
+* tokens through the launch == the oracle's, through graph replay and eager launches, and == the fused launches';
+* contexts that need several KV splits per head, and a context long enough that the attention tile doubles;
+* heads of 128 with grouped KV heads;
+* automatic mode picks the launch for a many-layer small model and not for a 4-layer one;
+* a wait that runs out: the launch still ends, the call reports it, the context continues with the fused launches.
+"""
+import numpy as np
+import pytest
+
+from mongoose_amd import configs
+from mongoose_amd import engine as E
+from oracle import binding as ob
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+MG_E_STATE = -4
+
+
+def _in_use(hipctx):
+    return hipctx.FlowInUse()
+
+
+def test_every_handed_over_vector_matches_numpy(hip):
+    s = H.with_layers(configs.TOY, 1)
+    m = H.Model(s, seed=1, maxSeq=72, eng=hip, threads=8, keep_dequant=True)
+    assert m.hip.SetExecMode(3) == 0
+    D = {k: v.astype(np.float64) for k, v in m.dequant.items()}
+    hd, half = s.headDim, s.headDim // 2
+    cosT, sinT = ob.rope_tables(72, hd, s.theta)
+
+    def rms(x, g):
+        x = x.astype(np.float64)
+        return x / np.sqrt((x * x).mean() + s.eps) * g
+
+    def rope(x, pos, nH):
+        x = x.reshape(nH, hd).copy()
+        c, sn = cosT[pos].astype(np.float64), sinT[pos].astype(np.float64)
+        a, b = x[:, :half].copy(), x[:, half:].copy()
+        x[:, :half] = a * c - b * sn
+        x[:, half:] = a * sn + b * c
+        return x.reshape(-1)
+
+    rng = np.random.default_rng(0)
+    Ks, Vs = [], []
+    G = s.nHeads // s.nKVHeads
+    for pos in range(5):
+        h = rng.standard_normal(s.dim).astype(np.float32)
+        assert m.hip.PartialStep(h, pos, 0, 1, None, None) == 0, E.last_error()
+        x = m.hip.FlowExchange(0)
+        assert x is not None, "the persistent launch is not in use"
+        n = rms(h, m.vecs[0])
+        q = rope(D[1] @ n, pos, s.nHeads)
+        k = rope(D[2] @ n, pos, s.nKVHeads)
+        v = D[3] @ n
+        Ks.append(k)
+        Vs.append(v)
+        assert H.rel_err(x["q"], q) < 1e-5 and H.rel_err(x["k"], k) < 1e-5 and H.rel_err(x["v"], v) < 1e-5
+        K = np.array(Ks).reshape(pos + 1, s.nKVHeads, hd)
+        V = np.array(Vs).reshape(pos + 1, s.nKVHeads, hd)
+        att = np.zeros(s.dim)
+        for hh in range(s.nHeads):
+            sc = (K[:, hh // G] @ q[hh * hd:(hh + 1) * hd]) / np.sqrt(hd)
+            p = np.exp(sc - sc.max())
+            att[hh * hd:(hh + 1) * hd] = (p / p.sum()) @ V[:, hh // G]
+        got = x["pacc"][0] / np.repeat(x["pl"][0], hd)           # one KV split at these positions
+        assert H.rel_err(got, att) < 1e-5
+        x1 = h.astype(np.float64) + D[7] @ att
+        assert H.rel_err(x["x1"], x1) < 1e-5
+        n2 = rms(x1, m.vecs[8])
+        g, u = D[9] @ n2, D[10] @ n2
+        mm = g / (1 + np.exp(-g)) * u
+        assert H.rel_err(x["m"], mm) < 1e-5
+        x2 = x1 + D[11] @ mm
+        assert H.rel_err(x["x2"], x2) < 1e-5
+        assert H.rel_err(m.hip.ExportHidden(), x2) < 1e-5
+    m.close()
+
+
+def test_tokens_match_oracle_and_fused_launches(hip):
+    s = configs.TOY
+    m = H.Model(s, seed=3, maxSeq=72, eng=hip, threads=8)
+    prompt = m.prompt(8)
+    ref, _ = H.oracle_generate(m, prompt, 64)
+    assert not _in_use(m.hip), "automatic mode takes the persistent launch for a 4-layer model"
+    out = {}
+    for mode in (1, 3):
+        assert m.hip.SetExecMode(mode) == 0
+        for graph in (True, False):
+            assert m.hip.ResetKV() == 0
+            rc, t = m.hip.Generate(prompt, 64, useGraph=graph)
+            assert rc == 0, E.last_error()
+            out[(mode, graph)] = t.tolist()
+        assert _in_use(m.hip) == (mode == 3)
+    assert out[(3, True)] == ref.tolist(), H.first_divergence(out[(3, True)], ref)
+    assert out[(3, False)] == ref.tolist()
+    assert out[(1, True)] == ref.tolist() and out[(1, False)] == ref.tolist()
+    # logits and hidden of a step through the launch against the oracle's
+    assert m.hip.SetExecMode(3) == 0
+    assert m.hip.ResetKV() == 0
+    m.orc.reset_kv()
+    stream = list(prompt) + list(ref)
+    logits = np.empty(s.vocab, np.float32)
+    for pos in range(12):
+        h = m.orc.embed(stream[pos])
+        hid, lg, _ = m.orc.step(h, pos, shadow=True)
+        assert m.hip.PartialStep(h, pos, 0, s.nLayers, None, logits) == 0, E.last_error()
+        assert H.rel_err(logits, lg) < 1e-4
+        assert H.rel_err(m.hip.ExportHidden(), hid) < 1e-4
+    m.close()
+
+
+def _modes_agree(m, prompt, nDecode, what):
+    out = {}
+    for mode in (1, 3):
+        assert m.hip.SetExecMode(mode) == 0
+        assert m.hip.ResetKV() == 0
+        rc, t = m.hip.GeneratePrefill(prompt, nDecode)
+        assert rc == 0, E.last_error()
+        out[mode] = t
+    assert _in_use(m.hip)
+    i = H.first_divergence(out[3], out[1])
+    assert i is None, f"{what}: persistent launch and fused launches part at token {i}"
+    return out[3]
+
+
+def test_kv_splits_and_tile_doubling_heads_of_64(hip):
+    """0.5B geometry (14 query heads on 2 KV heads, biases), 2 layers.  Up to 18 partial slots per head: positions
+    600..640 use 5-6 splits of 128 positions; from position 2304 the tile is 256."""
+    s = H.with_layers(configs.QWEN, 2)._replace(name="qwen-geom", vocab=2048)
+    m = H.Model(s, seed=11, maxSeq=2400, eng=hip, oracle=False)
+    print("flow: qwen geometry, positions 600..640", flush=True)
+    _modes_agree(m, m.prompt(600), 40, "5-6 splits")
+    print("flow: qwen geometry, positions 2290..2330 (tile doubles at 2304)", flush=True)
+    _modes_agree(m, m.prompt(2290), 40, "tile 128 -> 256")
+    m.close()
+
+
+def test_heads_of_128_grouped_kv(hip):
+    """Llama-3-8B attention geometry (32 query heads of 128 on 8 KV heads, dim 4096: rows of two chunks a lane), 2
+    layers, FFN and vocabulary cut: 8 partial slots, tile 128."""
+    s = H.with_layers(configs.LLAMA3_8B, 2)._replace(name="l3-geom", ffnDim=1024, vocab=1024, tied=True)
+    m = H.Model(s, seed=12, maxSeq=700, eng=hip, threads=16)
+    print("flow: llama-3 geometry, 6 + 6 against the oracle", flush=True)
+    prompt = m.prompt(6)
+    ref, _ = H.oracle_generate(m, prompt, 6)
+    assert m.hip.SetExecMode(3) == 0
+    rc, t = m.hip.Generate(prompt, 6, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert _in_use(m.hip)
+    assert t.tolist() == ref.tolist()
+    print("flow: llama-3 geometry, positions 300..330 (3 splits)", flush=True)
+    _modes_agree(m, m.prompt(300), 30, "heads of 128")
+    m.close()
+
+
+def test_automatic_mode_takes_the_launch_for_many_small_layers(hip):
+    s = H.with_layers(configs.TOY, 8)
+    m = H.Model(s, seed=5, maxSeq=40, eng=hip, threads=8)
+    prompt = m.prompt(4)
+    ref, _ = H.oracle_generate(m, prompt, 16)
+    rc, t = m.hip.Generate(prompt, 16, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert _in_use(m.hip), "8 small layers: automatic mode should use the persistent launch"
+    assert t.tolist() == ref.tolist()
+    rc, tr = m.hip.FlowTrace(True, read=False)
+    assert rc == 0, E.last_error()
+    rc, t2 = m.hip.Generate(prompt, 2, useGraph=False)
+    assert rc == 0
+    rc, tr = m.hip.FlowTrace(True, read=True)
+    assert rc == 0 and tr.shape[0] == 8 and tr.shape[1] == len(m.hip.FLOW_TRACE_POINTS)
+    # every workgroup passed the top of every layer, later in every later layer
+    tops = tr[:, 0, :]
+    assert (tops > 0).all() and (np.diff(tops.astype(np.int64), axis=0) > 0).all()
+    assert m.hip.FlowTrace(False)[0] == 0
+    # a context in another mode has no such launch to trace
+    assert m.hip.SetExecMode(1) == 0
+    assert m.hip.FlowTrace(True)[0] == MG_E_STATE
+    m.close()
+
+
+def test_a_wait_that_runs_out_is_reported_and_the_context_goes_on(hip):
+    s = configs.TOY
+    m = H.Model(s, seed=7, maxSeq=40, eng=hip, threads=8)
+    prompt = m.prompt(4)
+    ref, _ = H.oracle_generate(m, prompt, 12)
+    assert m.hip.SetExecMode(3) == 0
+    assert m.hip.SetFlowWaitLimit(-1) == 0          # every wait not satisfied at once gives up; all workgroups still exit
+    rc, _ = m.hip.Generate(prompt, 12, useGraph=False)
+    assert rc != 0 and "persistent" in E.last_error(), (rc, E.last_error())
+    assert not _in_use(m.hip)
+    assert m.hip.SetFlowWaitLimit(5_000_000) == 0
+    assert m.hip.ResetKV() == 0
+    rc, t = m.hip.Generate(prompt, 12, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert t.tolist() == ref.tolist()
+    m.close()
