@@ -10,9 +10,14 @@ steps are the W prompt positions; the K timed steps are the K decode positions
 after them.  Weights are synthetic (seeded N(0, 0.02), quantized on the host by
 the library's own loader) and resident in HBM before the timed region starts.
 
-Prints ONE JSON line with the throughput, the roofline of the dominant kernel
-(the lm_head matvec) measured inside the replayed token, a per-launch-class
-table, and the CPU oracle timed on this box's host cores as a baseline.
+Prints ONE JSON line: the throughput of the headline configuration, the roofline of
+the kernel that takes most of the step's time (HIP events around its launches inside
+the step), a per-launch table, the lm_head matvec's own bandwidth (the second half of
+the metric), the CPU oracle timed on this box's host cores as a baseline, and -- under
+"configs" -- the same measurements for the other benchmark configurations (toy,
+TinyLlama-1.1B shape, Qwen2.5-0.5B Q4_0, Llama-3-8B shape at a short context, at ~4k
+context and its 512-token batched prefill), each with its greedy tokens checked against
+the oracle on a bounded sample.
 """
 import argparse
 import json
@@ -26,14 +31,21 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
 
-# HBM bytes per launch of the lm_head kernel from rocprofv3 --pmc runs of this script
-# (FETCH_SIZE then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
-# reads for a 256 MiB device copy in the same run (FETCH_SIZE reads 131106.2 KiB for the
-# 262144 KiB copied -> x1.9995; WRITE_SIZE reads 262144.0 -> x1.0).  Counts are a property
-# of kernel and shape, so they are recorded here; profiles/ holds the run they come from.
+# HBM bytes per launch from rocprofv3 --pmc runs of this script (FETCH_SIZE then WRITE_SIZE,
+# KiB per dispatch), each scaled by what the same counter reads for a 256 MiB device copy in
+# the same run (FETCH_SIZE reads 131102.4 KiB for the 262144 KiB copied -> x1.9995; WRITE_SIZE
+# reads 262144.0 -> x1.0).  Counts are a property of kernel and shape, so they are recorded
+# here, keyed by (configuration, launch); profiles/ holds the runs they come from.  They are
+# NOT measured by the run that prints them: "traffic_source" in the output says so.
 PMC_TRAFFIC_BYTES = {
-    "qwen2.5-0.5b": int((67136.6 * (262144.0 / 131106.2) + 661.7 * 1.0) * 1024),
+    ("qwen2.5-0.5b", "lm_head"): int((67135.0 * (262144.0 / 131102.4) + 660.7 * 1.0) * 1024),
+    ("qwen2.5-0.5b", "flow"): int((190997.2 * (262144.0 / 131102.4) + 6004.0 * 1.0) * 1024),
 }
+PMC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script recorded in profiles/ (constants in bench.py, not measured by this run)"
+
+LAUNCH_NAMES = {0: "embed_gather", 1: "norm+qkv", 2: "rope+kvwrite+attention", 3: "wo+residual", 4: "norm+gate_up+swiglu",
+                5: "down+residual", 6: "norm+lm_head+argmax_partials", 7: "argmax_finish"}
+FLOW_NAME = "persistent layer launch (all layers: norm, q|k|v, RoPE, KV write, attention, Wo, gate|up, SwiGLU, down)"
 
 
 def slot_shape(s, kv, idx):
@@ -148,6 +160,147 @@ def cpu_baseline(E, np, s, seed, prompt, first_tokens, budget_s, kv_f16=False):
             "tokens_match_gpu": bool(match)}
 
 
+def oracle_for(ob, configs, s, maxSeq, threads):
+    kv = configs.kv_dim(s)
+    return ob.Oracle(s.dim, kv, s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab, s.nLayers, maxSeq, s.theta, s.eps,
+                     threads=threads)
+
+
+def launch_table(f, configs, s, first_tok, pos, steps, ms_per_step, kv_f16):
+    """Per-launch-class averages inside eager steps at positions pos.. (HIP events on the context's stream)."""
+    kv = configs.kv_dim(s)
+    rc, cls_ms, cls_n = f.ProfileDecode(first_tok, pos, steps)
+    assert rc == 0
+    flow = f.FlowInUse()
+
+    def mat(n, k):
+        return n * k + 4 * n if s.fmt == "q8" else n * (k // 32) * 18
+    p_prof = pos + steps // 2
+    kvb = 2 * (p_prof + 1) * kv * (2 if kv_f16 else 4)
+    layer_w = mat(s.dim, s.dim) * 2 + 2 * mat(kv, s.dim) + 2 * mat(s.ffnDim, s.dim) + mat(s.dim, s.ffnDim) + 8 * s.dim
+    cls_bytes = {
+        1: (layer_w + kvb) * s.nLayers if flow else mat(s.dim, s.dim) + 2 * mat(kv, s.dim) + 4 * s.dim,
+        2: kvb,
+        3: mat(s.dim, s.dim),
+        4: 2 * mat(s.ffnDim, s.dim) + 4 * s.dim,
+        5: mat(s.dim, s.ffnDim),
+        6: mat(s.vocab, s.dim) + 4 * s.dim,
+    }
+    rows = []
+    total = sum(float(cls_ms[c]) * int(cls_n[c]) for c in range(8))
+    for c in range(8):
+        n = int(cls_n[c])
+        if n == 0:
+            continue
+        ms = float(cls_ms[c])
+        # share of the eager step's launch time (events between launches; a replayed graph runs the same kernels closer together)
+        e = {"launch": FLOW_NAME if (flow and c == 1) else LAUNCH_NAMES[c], "cls": c, "per_token": n, "avg_us": round(ms * 1e3, 3),
+             "share_of_step": round(ms * n / total, 4) if total > 0 else None}
+        if c in cls_bytes and ms > 0:
+            e["bytes"] = int(cls_bytes[c])
+            e["GBps"] = round(cls_bytes[c] / (ms * 1e-3) / 1e9, 1)
+            e["frac_of_peak"] = round(e["GBps"] / HBM_PEAK_GBS, 4)
+        rows.append(e)
+    return rows
+
+
+def check_tokens(E, orc, prompt, toks, budget_s):
+    """Greedy tokens of the GPU against the oracle's on the same stream, as far as the budget goes."""
+    stream = list(prompt) + [int(t) for t in toks]
+    nP = len(prompt)
+    t0 = time.perf_counter()
+    checked, match = 0, True
+    for pos in range(len(stream) - 1):
+        nxt, _, _ = orc.decode_token(int(stream[pos]), pos)
+        if pos >= nP - 1:
+            checked += 1
+            if nxt != int(stream[pos + 1]):
+                match = False
+                break
+        if time.perf_counter() - t0 > budget_s and checked >= 2:
+            break
+    return {"tokens_match": bool(match), "tokens_checked": checked, "oracle_s": round(time.perf_counter() - t0, 1)}
+
+
+def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_graph=True, exec_mode=None, kv_f16=False,
+            prefill=0, oracle_threads=0, check_budget_s=8.0, want_mode1_table=True, keep=False):
+    """One configuration: load, warm up on the W prompt positions, time K decode steps at each start position of
+    `contexts` (0 = right after the prompt), per-launch table, optional batched prefill, optional token check."""
+    from oracle import binding as ob
+    P = [max(c, W) for c in contexts]
+    maxSeq = max(max(P) + K + profile_steps + 8, prefill + 8, W + 56)
+    orc = oracle_for(ob, configs, s, W + 72, oracle_threads) if oracle_threads else None
+    t_load = time.perf_counter()
+    f = load_model(E, np, s, seed, maxSeq, eng, oracle=orc, kv_f16=kv_f16)
+    if exec_mode is not None and f.SetExecMode(exec_mode) != 0:
+        raise SystemExit("bench.py: " + E.last_error())
+    t_load = time.perf_counter() - t_load
+    prompt = E.synth_tokens(seed, 20_000_003, s.vocab, W)
+    rc, first = f.Generate(prompt, 1, useGraph=use_graph)
+    assert rc == 0, E.last_error()
+    wbytes = configs.weight_bytes_per_token(s)
+    assert f.WeightBytesPerToken() == wbytes
+    flow = f.FlowInUse()
+    res = {"exec": ("persistent layer launch + lm_head + argmax" if flow else "fused launches (5 a layer)") +
+                   (", hipGraph replay" if use_graph else ", eager"),
+           "weight_bytes_per_token": int(wbytes), "load_s": round(t_load, 1), "runs": []}
+    for P0 in P:
+        rc, ms = f.TimedDecode(int(first[0]), P0, K, useGraph=use_graph)
+        assert rc == 0, E.last_error()
+        ms_step = ms / K
+        step_bytes = wbytes + configs.kv_bytes_at(s, P0 + K // 2) // (2 if kv_f16 else 1)
+        run = {"start_position": P0, "steps": K, "ms_per_step": round(ms_step, 5), "tok_per_s": round(K / (ms / 1e3), 1),
+               "step_bytes": int(step_bytes), "step_GBps": round(step_bytes / (ms_step * 1e-3) / 1e9, 1),
+               "step_roofline_frac": round(step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        table = launch_table(f, configs, s, int(first[0]), P0 + K, profile_steps, ms_step, kv_f16)
+        run["kernels"] = table
+        if flow and want_mode1_table:
+            assert f.SetExecMode(1) == 0
+            rc, ms1 = f.TimedDecode(int(first[0]), P0, K, useGraph=use_graph)
+            assert rc == 0, E.last_error()
+            run["fused_launches_ms_per_step"] = round(ms1 / K, 5)
+            run["kernels_fused_launches"] = launch_table(f, configs, s, int(first[0]), P0 + K, profile_steps, ms1 / K, kv_f16)
+            assert f.SetExecMode(3 if exec_mode is None else exec_mode) == 0
+            table = run["kernels_fused_launches"]
+        att = [e for e in table if e["cls"] == 2]
+        if att and "GBps" in att[0]:
+            run["attention_KV_GBps"] = att[0]["GBps"]
+        res["runs"].append(run)
+    if prefill > 0:
+        ptoks = E.synth_tokens(seed, 20_000_003, s.vocab, prefill)
+        times = []
+        for _ in range(4):                              # first call allocates the row buffers
+            assert f.ResetKV() == 0
+            rc, _, _, pms = f.Prefill(ptoks, 0)
+            assert rc == 0, E.last_error()
+            times.append(pms)
+        pms = min(times[1:])
+        kv = configs.kv_dim(s)
+        macs = sum(n * k for n, k in
+                   [(s.dim, s.dim), (kv, s.dim), (kv, s.dim), (s.dim, s.dim), (s.ffnDim, s.dim), (s.ffnDim, s.dim),
+                    (s.dim, s.ffnDim)]) * s.nLayers
+        flops = 2.0 * macs * prefill
+        res["prefill"] = {"tokens": prefill, "ms": round(pms, 3), "tok_per_s": round(prefill / (pms * 1e-3), 1),
+                          "model_TFLOPs": round(flops / (pms * 1e-3) / 1e12, 2),
+                          "mfma_TFLOPs_issued": round(2 * flops / (pms * 1e-3) / 1e12, 2),
+                          "mfma_frac_of_bf16_peak": round(2 * flops / (pms * 1e-3) / 1e12 / 2500.0, 4),
+                          "note": "model flops = 2*T*weights of the layer projections; each is issued twice (bf16 hi and lo activation terms)"}
+    toks = None
+    if orc is not None or keep:
+        # the token check runs on a 4-token prompt, so that the oracle's budget goes into decoded tokens
+        cprompt = prompt[:4] if orc is not None else prompt
+        assert f.ResetKV() == 0
+        rc, toks = f.Generate(cprompt, 48, useGraph=use_graph)
+        assert rc == 0, E.last_error()
+    if orc is not None:
+        res.update(check_tokens(E, orc, cprompt, toks, check_budget_s))
+        orc.close()
+    if keep:
+        return res, f, prompt, first, toks
+    f.Close()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -158,8 +311,9 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds of CPU baseline work (0 = skip)")
     ap.add_argument("--profile-steps", type=int, default=20)
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--exec-mode", type=int, default=1, choices=[1, 2],
-                    help="1 = fused launches (default); 2 = the same without the L2 prefetch by the attention launch's idle workgroups")
+    ap.add_argument("--exec-mode", type=int, default=-1, choices=[-1, 0, 1, 2, 3],
+                    help="-1 = the library's automatic choice (default); 1 = fused launches; 2 = the same without the L2 prefetch by "
+                         "the attention launch's idle workgroups; 3 = one persistent launch for all layers wherever the model allows it")
     ap.add_argument("--context", type=int, default=0,
                     help="start the timed decode at this position (KV rows between the prompt and it are zeros): long-context timing")
     ap.add_argument("--pmc-copy", action="store_true",
@@ -171,6 +325,10 @@ def main():
     ap.add_argument("--stream", type=int, default=0,
                     help="also time this many tokens through the weight-streaming front end (Q4_0 configurations: "
                          "every layer's weights cross PCIe per token; extra 'stream' object)")
+    ap.add_argument("--flow-trace", action="store_true",
+                    help="also record the persistent layer launch's per-workgroup timeline (extra 'flow_trace' object)")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="only the configuration named by --config (no 'configs' object with the other benchmark configurations)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
@@ -187,77 +345,57 @@ def main():
         print("bench.py: no HIP device", file=sys.stderr)
         sys.exit(1)
     K, W = args.steps, max(args.warmup, 1)
-    P0 = max(args.context, W)                      # position of the first timed step
-    maxSeq = max(P0 + K + args.profile_steps + 8, args.prefill, args.stream + 2)
-    t_load = time.perf_counter()
-    kv_f16 = args.kv == "f16"
-    f = load_model(E, np, s, args.seed, maxSeq, eng, kv_f16=kv_f16)
-    if args.exec_mode != 1 and f.SetExecMode(args.exec_mode) != 0:
-        raise SystemExit("bench.py: " + E.last_error())
-    t_load = time.perf_counter() - t_load
-    prompt = E.synth_tokens(args.seed, 20_000_003, s.vocab, W)
     use_graph = not args.no_graph
+    kv_f16 = args.kv == "f16"
+    mode = None if args.exec_mode < 0 else args.exec_mode
+    res, f, prompt, first, toks = measure(E, np, configs, eng, s, args.seed, W, K, [args.context], args.profile_steps,
+                                          use_graph=use_graph, exec_mode=mode, kv_f16=kv_f16, prefill=args.prefill,
+                                          oracle_threads=0, keep=True)
+    run = res["runs"][0]
+    P0 = run["start_position"]
+    ms_per_step = run["ms_per_step"]
+    toks_per_s = K / (ms_per_step * K / 1e3)
+    flow = f.FlowInUse()
 
-    # warmup = the W prompt positions (+ graph capture), then the first decoded token
-    rc, first = f.Generate(prompt, 1, useGraph=use_graph)
-    assert rc == 0, E.last_error()
-    # timed region: K decode steps at positions W .. W+K-1, token and position stay on the device
-    rc, ms = f.TimedDecode(int(first[0]), P0, K, useGraph=use_graph)
-    assert rc == 0, E.last_error()
-    toks_per_s = K / (ms / 1e3)
-    ms_per_step = ms / K
-
-    # the same K tokens again to read them back (for the CPU baseline's comparison)
-    assert f.ResetKV() == 0
-    rc, toks = f.Generate(prompt, min(K, 48), useGraph=use_graph)
+    # the launch that takes most of the step, and the lm_head matvec, once more with events around them alone
+    # (less event overhead inside their intervals)
+    table = run["kernels"]
+    dom = max(table, key=lambda e: e["avg_us"] * e["per_token"])
+    rc, only, _ = f.ProfileDecode(int(first[0]), P0 + K, args.profile_steps, classMask=(1 << dom["cls"]) | (1 << 6))
     assert rc == 0, E.last_error()
 
-    # per-launch-class timing inside a replayed token
-    kv = configs.kv_dim(s)
-    rc, cls_ms, cls_n = f.ProfileDecode(int(first[0]), P0 + K, args.profile_steps)
-    assert rc == 0, E.last_error()
-    cls_ms = [float(x) for x in cls_ms]
-    cls_n = [int(x) for x in cls_n]
-    # the dominant kernel once more with events around it alone (less event overhead in its interval)
-    rc, lm_only, _ = f.ProfileDecode(int(first[0]), P0 + K, args.profile_steps, classMask=1 << 6)
-    assert rc == 0, E.last_error()
-    lm_only_ms = float(lm_only[6])
+    def roof(entry, ms, key):
+        sec = ms * 1e-3
+        b = entry["bytes"]
+        return {"bound": "hbm", "kernel": entry["launch"], "achieved": round(b / sec / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(b / sec / 1e9 / HBM_PEAK_GBS, 4), "bytes_per_launch": int(b), "avg_launch_us": round(sec * 1e6, 2),
+                "launches_per_step": entry["per_token"], "share_of_step": entry["share_of_step"],
+                "launches_timed": int(args.profile_steps) * entry["per_token"],
+                "traffic": PMC_TRAFFIC_BYTES.get((s.name, key)),
+                "traffic_source": PMC_SOURCE if (s.name, key) in PMC_TRAFFIC_BYTES else None}
+    roofline = roof(dom, float(only[dom["cls"]]), "flow" if (flow and dom["cls"] == 1) else LAUNCH_NAMES[dom["cls"]])
+    lm = [e for e in table if e["cls"] == 6][0]
+    matvec = roof(lm, float(only[6]), "lm_head")
 
-    def mat(n, k):
-        return n * k + 4 * n if s.fmt == "q8" else n * (k // 32) * 18
-    p_mid = P0 + K // 2
-    p_prof = P0 + K + args.profile_steps // 2
-    cls_bytes = {
-        1: mat(s.dim, s.dim) + 2 * mat(kv, s.dim) + 4 * s.dim,
-        2: 2 * (p_prof + 1) * kv * (2 if kv_f16 else 4),
-        3: mat(s.dim, s.dim),
-        4: 2 * mat(s.ffnDim, s.dim) + 4 * s.dim,
-        5: mat(s.dim, s.ffnDim),
-        6: mat(s.vocab, s.dim) + 4 * s.dim,
-    }
-    names = {0: "embed_gather", 1: "norm+qkv", 2: "rope+kvwrite+attention", 3: "wo+residual", 4: "norm+gate_up+swiglu",
-             5: "down+residual", 6: "norm+lm_head+argmax_partials", 7: "argmax_finish"}
-    kernels = []
-    for c in range(8):
-        if cls_n[c] == 0:
-            continue
-        e = {"launch": names[c], "per_token": int(cls_n[c]), "avg_us": round(float(cls_ms[c]) * 1e3, 3)}
-        if c in cls_bytes and cls_ms[c] > 0:
-            e["bytes"] = int(cls_bytes[c])
-            e["GBps"] = round(cls_bytes[c] / (cls_ms[c] * 1e-3) / 1e9, 1)
-            e["frac_of_peak"] = round(e["GBps"] / HBM_PEAK_GBS, 4)
-        kernels.append(e)
-
-    wbytes = configs.weight_bytes_per_token(s)
-    assert f.WeightBytesPerToken() == wbytes
-    step_bytes = wbytes + configs.kv_bytes_at(s, p_mid) // (2 if kv_f16 else 1)
-    lm_bytes = cls_bytes[6]
-    lm_s = lm_only_ms * 1e-3
-    roofline = {"bound": "hbm", "kernel": "matvec lm_head (final norm + Q8 matvec + argmax partials)",
-                "achieved": round(lm_bytes / lm_s / 1e9, 1) if lm_s > 0 else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(lm_bytes / lm_s / 1e9 / HBM_PEAK_GBS, 4) if lm_s > 0 else None,
-                "bytes_per_launch": int(lm_bytes), "avg_launch_us": round(lm_s * 1e6, 2),
-                "launches_timed": int(args.profile_steps), "traffic": PMC_TRAFFIC_BYTES.get(s.name)}
+    flow_trace = None
+    if args.flow_trace and flow:
+        rc, _ = f.FlowTrace(True)
+        assert rc == 0, E.last_error()
+        rc, _ = f.TimedDecode(int(first[0]), P0 + K, 8, useGraph=use_graph)
+        assert rc == 0, E.last_error()
+        rc, tr = f.FlowTrace(True, read=True)
+        assert rc == 0, E.last_error()
+        f.FlowTrace(False)
+        L = s.nLayers // 2
+        base = float(np.median(tr[L, 0]))
+        pts = []
+        for b, name in enumerate(f.FLOW_TRACE_POINTS):
+            v = (tr[L, b][tr[L, b] > 0] - base) / 100.0
+            pts.append({"point": name, "workgroups": int(v.size), "min_us": round(float(v.min()), 2),
+                        "median_us": round(float(np.median(v)), 2), "max_us": round(float(v.max()), 2)})
+        flow_trace = {"position": P0 + K + 7, "layer": L, "zero": "median workgroup entering the layer",
+                      "points": pts, "layer_us": round((float(np.median(tr[L + 1, 0])) - base) / 100.0, 2),
+                      "all_layers_us": round((float(tr[-1, -1].max()) - float(np.median(tr[0, 0]))) / 100.0, 1)}
 
     if args.pmc_copy:
         n = 256 << 20
@@ -268,31 +406,13 @@ def main():
         a.Release()
         b.Release()
 
-    prefill = None
-    if args.prefill > 0:
-        ptoks = E.synth_tokens(args.seed, 20_000_003, s.vocab, args.prefill)
-        times = []
-        for _ in range(4):                              # first call allocates the row buffers
-            assert f.ResetKV() == 0
-            rc, _, _, pms = f.Prefill(ptoks, 0)
-            assert rc == 0, E.last_error()
-            times.append(pms)
-        pms = min(times[1:])
-        macs = sum(n * k for n, k in
-                   [(s.dim, s.dim), (kv, s.dim), (kv, s.dim), (s.dim, s.dim), (s.ffnDim, s.dim), (s.ffnDim, s.dim),
-                    (s.dim, s.ffnDim)]) * s.nLayers
-        flops = 2.0 * macs * args.prefill
-        prefill = {"tokens": args.prefill, "ms": round(pms, 3), "tok_per_s": round(args.prefill / (pms * 1e-3), 1),
-                   "model_TFLOPs": round(flops / (pms * 1e-3) / 1e12, 2),
-                   "mfma_TFLOPs_issued": round(2 * flops / (pms * 1e-3) / 1e12, 2),
-                   "note": "model flops = 2*T*weights of the layer projections; each is issued twice (bf16 hi and lo activation terms)"}
-
     stream = None
     if args.stream > 0:
         if s.fmt != "q4_0":
             print("bench.py: --stream needs a Q4_0 configuration (the streaming front end takes GGUF block_q4_0 layers)",
                   file=sys.stderr)
             sys.exit(2)
+        kv = configs.kv_dim(s)
         st = f.StreamBuild()
         assert st is not None, E.last_error()
         ptrs, sizes = [], []
@@ -323,10 +443,24 @@ def main():
                   "host_to_device_GBps": round(layer_bytes * args.stream / el / 1e9, 2),
                   "note": "host wall clock; every token stages all layers from pageable host memory through two pinned "
                           "buffers into two device sets (copy of layer l+1 overlaps compute of layer l); logits read back each token"}
+    f.Close()
 
     cpu = None
     if args.cpu_budget > 0:
         cpu = cpu_baseline(E, np, s, args.seed, prompt, toks, args.cpu_budget, kv_f16=kv_f16)
+
+    others = None
+    if not args.no_configs and args.config == "qwen2.5-0.5b":
+        others = {}
+        plan = [("toy", dict(K=200, contexts=[0], threads=8)),
+                ("tinyllama-1.1b", dict(K=50, contexts=[0], threads=16)),
+                ("qwen2.5-0.5b-q4_0", dict(K=200, contexts=[0], threads=16)),
+                ("llama-3-8b", dict(K=64, contexts=[0, 4000], threads=16, prefill=512))]
+        for name, o in plan:
+            print(f"bench.py: configuration {name}", file=sys.stderr, flush=True)
+            others[name] = measure(E, np, configs, eng, configs.BY_NAME[name], args.seed + 1, 16, o["K"], o["contexts"],
+                                   10, use_graph=True, prefill=o.get("prefill", 0), oracle_threads=o["threads"],
+                                   check_budget_s=10.0)
 
     out = {
         "metric": "Q8 decode tok/s (bs=1, Qwen2.5-0.5B shape) + matvec HBM GB/s % of peak" if s.name == "qwen2.5-0.5b"
@@ -335,15 +469,15 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "weight_dtype": "int8 per-row scale" if s.fmt == "q8" else "q4_0 (fp16 block scale)",
         "data": "synthetic",
-        "config": {"workload": f"{s.name} random-init {s.fmt.upper()} greedy decode, {W}-token prompt, {K} decode tokens, "
-                               f"batch 1, {'fp16' if kv_f16 else 'fp32'} KV cache", "layers": s.nLayers, "hidden": s.dim, "heads": s.nHeads,
-                   "kv_heads": s.nKVHeads, "ffn": s.ffnDim, "vocab": s.vocab, "graph_replay": use_graph},
-        "step_bytes": int(step_bytes), "step_GBps": round(step_bytes * toks_per_s / 1e9, 1),
-        "step_roofline_frac": round(step_bytes * toks_per_s / 1e9 / HBM_PEAK_GBS, 4),
-        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu, "prefill": prefill, "stream": stream,
-        "load_s": round(t_load, 1), "device": eng.Name(),
+        "config": {"workload": f"{s.name} shape, random-init {s.fmt.upper()} weights, greedy decode: {W}-token prompt, {K} decode "
+                               f"tokens from position {P0}, batch 1, {'fp16' if kv_f16 else 'fp32'} KV cache; {res['exec']}"},
+        "step_bytes": run["step_bytes"], "step_GBps": run["step_GBps"], "step_roofline_frac": run["step_roofline_frac"],
+        "roofline": roofline, "matvec": matvec, "kernels": run["kernels"],
+        "kernels_fused_launches": run.get("kernels_fused_launches"),
+        "fused_launches_ms_per_step": run.get("fused_launches_ms_per_step"),
+        "cpu_baseline": cpu, "prefill": res.get("prefill"), "stream": stream, "flow_trace": flow_trace, "configs": others,
+        "load_s": res["load_s"], "device": eng.Name(),
     }
-    f.Close()
     print(json.dumps(out))
 
 
