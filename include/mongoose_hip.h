@@ -266,13 +266,47 @@ int mg_decode_token(mg_ctx* ctx, int token, int pos, int* nextToken, float* logi
  * the position and the token stay in device memory between steps. */
 int mg_generate(mg_ctx* ctx, const int* prompt, int nPrompt, int nDecode, int* outTokens, int useGraph);
 
-/* CUDAGraph, cuda_graph.go:286-739.  Capture once; every launch advances the
- * device-resident position by one.  mg_graph_validate replays one step both
- * ways and returns the largest absolute logit difference (the reference's
- * criterion is < 1e-3, cuda_graph.go:590-597). */
+/* Whole-token graphs (embedding gather .. argmax), the form the decode loop replays: capture once;
+ * every launch advances the device-resident position by one.  mg_graph_validate replays one step both
+ * ways and returns the largest absolute logit difference (the reference's criterion is < 1e-3,
+ * cuda_graph.go:590-597).  No counterpart in the reference, whose graphs stop at the hidden state. */
 int mg_graph_capture(mg_ctx* ctx);
 int mg_graph_launch(mg_ctx* ctx, int token, int pos, int* nextToken);
 int mg_graph_validate(mg_ctx* ctx, int token, int pos, float* maxAbsDiff);
+
+/* CUDAGraph, cuda_graph.go:286-739: a captured graph over the layers [layerStart, layerEnd) that takes
+ * the current hidden buffer as input and leaves its output there.
+ *
+ * mg_layer_graph_capture  = (*CUDAFusedInference).CaptureGraph(GraphCaptureConfig{LayerStart, LayerEnd,
+ *     StreamCount, PipelineBreak}, pos), cuda_graph.go:315-498.  StreamCount 0 means 1 (:316); other
+ *     values than 1 and 2 and a PipelineBreak outside (LayerStart, LayerEnd) with StreamCount 2 return
+ *     NULL as there (:323, :396-400).  The reference's two-stream form runs stage B after stage A (an
+ *     event joins them), so its result is that of one stream; here both forms are one capture on the
+ *     context's stream.  pos is checked and otherwise unused: the kernels read the position from device
+ *     memory, so one capture serves every position.
+ * mg_layer_graph_launch   = (*CUDAGraph).Launch(pos), :663-669: writes the position, replays.
+ *     Asynchronous on the context's stream like the reference's; mg_read_hidden / mg_export_hidden wait.
+ * mg_layer_graph_update_and_launch = (*CUDAFusedInference).UpdateAndLaunch(g, pos), :673-714: returns 1
+ *     (true) or 0.  The reference re-captures and updates the executable graph because pos is baked
+ *     into its kernel arguments; here it is the same as a launch.
+ * A graph whose operands went stale (a weight or cache replaced, the exec mode or the hidden buffer
+ *     switched) is re-captured by its next launch.  Exec mode 0 (host-side positions) is not captured.
+ * mg_layer_graph_destroy  = (*CUDAGraph).Destroy(), :716-739; a graph may be destroyed after its context.
+ * mg_upload_hidden / mg_read_hidden = UploadHidden / ReadHidden, :650-658.
+ * mg_validate_graph_capture = ValidateGraphCapture(hiddenIn, layerStart, layerEnd), :554-598: resets the
+ *     KV cache, runs the range eagerly and through a fresh graph at position 0 on the same input, stores
+ *     the largest absolute difference in *maxDiff and returns 1 when it is below 1e-3 (the reference's
+ *     true), 0 when not, or a negative error code.  ValidateMultiStreamGraph (:603-647) is the same call.
+ * mg_has_graph_kernel = HasGraphKernel(), :281: always 1 (the kernels here all take a device position). */
+typedef struct mg_layer_graph mg_layer_graph;
+mg_layer_graph* mg_layer_graph_capture(mg_ctx* ctx, int layerStart, int layerEnd, int streamCount, int pipelineBreak, int pos);
+int mg_layer_graph_launch(mg_layer_graph* g, int pos);
+int mg_layer_graph_update_and_launch(mg_layer_graph* g, int pos);
+void mg_layer_graph_destroy(mg_layer_graph* g);
+int mg_upload_hidden(mg_ctx* ctx, const float* data /* [dim] */);
+int mg_read_hidden(mg_ctx* ctx, float* out /* [dim] */);
+int mg_validate_graph_capture(mg_ctx* ctx, const float* hiddenIn, int layerStart, int layerEnd, float* maxDiff);
+int mg_has_graph_kernel(void);
 
 /* Timed decode for measurement: runs `steps` graph (or eager) decode steps
  * starting at device state (token, pos), bracketed by events on the context's

@@ -154,6 +154,18 @@ public:
     float* flowXchg = nullptr;
     long long* flowTrace = nullptr;
     int FlowTrace(int enable, long long* out, size_t cap, int* dims);
+    // Graphs over a range of layers (cuda_graph.go:315-388, 663-714): hidden state in, hidden state out.
+    struct LayerGraph {
+        int l0 = 0, l1 = 0, hiddenIdx = 0;
+        unsigned generation = 0;
+        hipGraph_t g = nullptr;
+        hipGraphExec_t ex = nullptr;
+    };
+    int LayerGraphCapture(LayerGraph& lg);                 // (re)captures lg.l0 .. lg.l1 on the context's stream
+    int LayerGraphLaunch(LayerGraph& lg, int pos);         // sets the device position, replays; asynchronous
+    void LayerGraphDestroy(LayerGraph& lg);
+    int UploadHidden(const float* data);                   // cuda_graph.go:650
+    int ValidateGraphCapture(const float* hiddenIn, int layerStart, int layerEnd, float* maxDiff);   // :554-598
     bool FlowInUse() const { return flowEligible(0, nLayers); }
     long long flowLimitTicks = 5000000;       // per wait of the persistent launch: 50 ms of the 100 MHz wall clock
     void SetFlowWaitLimit(long long ticks) { invalidateGraphs(); flowLimitTicks = ticks; }
@@ -193,6 +205,7 @@ private:
     int* dHistory = nullptr;
     int* dPrompt = nullptr;
     int* hTokens = nullptr;         // pinned
+    unsigned graphGeneration = 0;     // bumped by whatever makes captured graphs stale (weights, caches, modes)
     hipGraph_t graphFull = nullptr, graphPrompt = nullptr;
     hipGraphExec_t execFull = nullptr, execPrompt = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -213,4 +226,8 @@ private:
 }  // namespace mg
 
 // the opaque handle of the C ABI
-struct mg_ctx { mg::HIPFusedInference* f; };
+struct mg_layer_graph;
+struct mg_ctx {
+    mg::HIPFusedInference* f;
+    std::vector<mg_layer_graph*> layerGraphs;      // live graph objects: they outlive the context as dead handles
+};

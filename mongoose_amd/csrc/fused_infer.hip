@@ -228,6 +228,7 @@ HIPFusedInference::~HIPFusedInference() {
 }
 
 int HIPFusedInference::invalidateGraphs() {
+    graphGeneration++;
     flowTableDirty = true;          // whatever invalidates the graphs may have moved a weight or a cache
     if (execFull) { (void)hipGraphExecDestroy(execFull); execFull = nullptr; }
     if (execPrompt) { (void)hipGraphExecDestroy(execPrompt); execPrompt = nullptr; }
@@ -1046,6 +1047,91 @@ int HIPFusedInference::GraphCapture() {
     return MG_OK;
 }
 
+// ---- graphs over a range of layers (cuda_graph.go:286-388, 554-598, 650-739) ----
+// The reference bakes pos into the kernel arguments and re-captures or updates the executable graph per token
+// (:673-714); here the position is read from device memory, so one capture serves every position.
+int HIPFusedInference::LayerGraphCapture(LayerGraph& lg) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(lg.l0 >= 0 && lg.l1 > lg.l0 && lg.l1 <= nLayers, "CaptureGraph: layer range outside the model");
+    for (int l = lg.l0; l < lg.l1; l++) {
+        if (!layerComplete(layers[l])) { set_error("CaptureGraph: layer weights incomplete"); return MG_E_STATE; }
+        if (!kCache[l]) { set_error("CaptureGraph: KV cache missing, call SetLayerRange first"); return MG_E_STATE; }
+    }
+    if (execMode == 0) { set_error("CaptureGraph: the per-op launches (exec mode 0) take their position from the host and are not captured"); return MG_E_STATE; }
+    LayerGraphDestroy(lg);
+    const bool flow = flowEligible(lg.l0, lg.l1);
+    if (flow) { int rc = ensureFlow(); if (rc) return rc; }          // allocations and uploads come before the capture
+    HIPCHK(hipStreamSynchronize(stream));
+    HIPCHK(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));
+    int rc = MG_OK;
+    if (flow) rc = enqueueLayersFlow(lg.l0, lg.l1, dState, 0, true);
+    else for (int l = lg.l0; l < lg.l1 && rc == MG_OK; l++) rc = enqueueLayer(layers[l], l, dState, 0);
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(stream, &g);
+    if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
+    HIPCHK(e);
+    hipGraphExec_t ex = nullptr;
+    e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) { (void)hipGraphDestroy(g); HIPCHK(e); }
+    lg.g = g; lg.ex = ex; lg.hiddenIdx = hiddenIdx; lg.generation = graphGeneration;
+    return MG_OK;
+}
+
+int HIPFusedInference::LayerGraphLaunch(LayerGraph& lg, int pos) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(pos >= 0 && pos < maxSeq, "graph Launch: pos out of range");
+    // a graph captured before a weight, a cache, the mode or the hidden buffer changed points at the old operands
+    if (!lg.ex || lg.generation != graphGeneration || lg.hiddenIdx != hiddenIdx) {
+        int rc = LayerGraphCapture(lg);
+        if (rc) return rc;
+    }
+    HIPCHK(launch_set_state(dState, pos, 0, 0, 0, ropeRef(), stream));
+    HIPCHK(hipGraphLaunch(lg.ex, stream));
+    return MG_OK;
+}
+
+void HIPFusedInference::LayerGraphDestroy(LayerGraph& lg) {
+    if (lg.ex) { (void)hipGraphExecDestroy(lg.ex); lg.ex = nullptr; }
+    if (lg.g) { (void)hipGraphDestroy(lg.g); lg.g = nullptr; }
+}
+
+int HIPFusedInference::UploadHidden(const float* data) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(data, "UploadHidden: NULL data");
+    HIPCHK(hipStreamSynchronize(stream));
+    HIPCHK(hipMemcpy(hidden[hiddenIdx], data, (size_t)dim * 4, hipMemcpyHostToDevice));
+    return MG_OK;
+}
+
+// cuda_graph.go:554-598: the eager path and the graph on the same input at position 0, largest difference below 1e-3.
+int HIPFusedInference::ValidateGraphCapture(const float* hiddenIn, int layerStart, int layerEnd, float* maxDiff) {
+    if (!built) return MG_E_NOT_BUILT;
+    ARGCHK(hiddenIn, "ValidateGraphCapture: NULL hiddenIn");
+    std::vector<float> ref((size_t)dim), got((size_t)dim);
+    int rc = ResetKV();
+    if (rc) return rc;
+    rc = PartialStep(hiddenIn, 0, layerStart, layerEnd, nullptr, nullptr);
+    if (rc == 0) rc = ExportHidden(ref.data());
+    if (rc) return rc;
+    rc = ResetKV();
+    if (rc) return rc;
+    LayerGraph lg;
+    lg.l0 = layerStart; lg.l1 = layerEnd < nLayers ? layerEnd : nLayers;
+    rc = LayerGraphCapture(lg);
+    if (rc == 0) rc = UploadHidden(hiddenIn);
+    if (rc == 0) rc = LayerGraphLaunch(lg, 0);
+    if (rc == 0) rc = ExportHidden(got.data());
+    LayerGraphDestroy(lg);
+    if (rc) return rc;
+    float md = 0.f;
+    for (int i = 0; i < dim; i++) {
+        const float d = std::fabs(ref[(size_t)i] - got[(size_t)i]);
+        if (!(d <= md)) md = d;                 // a NaN difference counts as the largest
+    }
+    if (maxDiff) *maxDiff = md;
+    return MG_OK;
+}
+
 int HIPFusedInference::GraphLaunch(int token, int pos, int* nextToken) {
     if (!built) return MG_E_NOT_BUILT;
     ARGCHK(pos >= 0 && pos < maxSeq && token >= 0 && token < vocabSize, "GraphLaunch: token or pos out of range");
@@ -1345,7 +1431,13 @@ mg_ctx* mg_create(int dim, int kvDim, int headDim, int nHeads, int nKVHeads, int
     if (!f) return nullptr;
     return new mg_ctx{f};
 }
-void mg_destroy(mg_ctx* c) { if (c) { delete c->f; delete c; } }
+struct mg_layer_graph { mg_ctx* c; mg::HIPFusedInference::LayerGraph lg; };
+void mg_destroy(mg_ctx* c) {
+    if (!c) return;
+    for (mg_layer_graph* g : c->layerGraphs) { if (c->f) c->f->LayerGraphDestroy(g->lg); g->c = nullptr; }
+    delete c->f;
+    delete c;
+}
 
 #define CTX(c) if (!(c) || !(c)->f) { mg::set_error("NULL context"); return MG_E_NOT_BUILT; } HIPFusedInference* f = (c)->f
 
@@ -1391,6 +1483,54 @@ int mg_generate(mg_ctx* c, const int* prompt, int nPrompt, int nDecode, int* out
 int mg_graph_capture(mg_ctx* c) { CTX(c); return f->GraphCapture(); }
 int mg_graph_launch(mg_ctx* c, int token, int pos, int* next) { CTX(c); return f->GraphLaunch(token, pos, next); }
 int mg_graph_validate(mg_ctx* c, int token, int pos, float* md) { CTX(c); return f->GraphValidate(token, pos, md); }
+mg_layer_graph* mg_layer_graph_capture(mg_ctx* c, int layerStart, int layerEnd, int streamCount, int pipelineBreak, int pos) {
+    if (!c || !c->f) { mg::set_error("NULL context"); return nullptr; }
+    if (streamCount == 0) streamCount = 1;                                   // cuda_graph.go:316
+    if (streamCount != 1 && streamCount != 2) { mg::set_error("CaptureGraph: unsupported StreamCount (use 1 or 2)"); return nullptr; }
+    if (streamCount == 2 && (pipelineBreak <= layerStart || pipelineBreak >= layerEnd)) {   // :396-400
+        mg::set_error("CaptureGraph: PipelineBreak must lie between LayerStart and LayerEnd");
+        return nullptr;
+    }
+    if (pos < 0 || pos >= c->f->maxSeq) { mg::set_error("CaptureGraph: pos out of range"); return nullptr; }
+    mg_layer_graph* g = new mg_layer_graph{c, {}};
+    g->lg.l0 = layerStart; g->lg.l1 = layerEnd;
+    if (c->f->LayerGraphCapture(g->lg) != MG_OK) { delete g; return nullptr; }
+    c->layerGraphs.push_back(g);
+    return g;
+}
+static bool live(mg_layer_graph* g) {
+    if (!g) { mg::set_error("NULL graph"); return false; }
+    if (!g->c) { mg::set_error("graph: its context was destroyed"); return false; }
+    return true;
+}
+int mg_layer_graph_launch(mg_layer_graph* g, int pos) {
+    if (!live(g)) return MG_E_STATE;
+    return g->c->f->LayerGraphLaunch(g->lg, pos);
+}
+int mg_layer_graph_update_and_launch(mg_layer_graph* g, int pos) {
+    if (!live(g)) return 0;
+    return g->c->f->LayerGraphLaunch(g->lg, pos) == MG_OK ? 1 : 0;
+}
+void mg_layer_graph_destroy(mg_layer_graph* g) {
+    if (!g) return;
+    if (g->c) {
+        g->c->f->LayerGraphDestroy(g->lg);
+        auto& v = g->c->layerGraphs;
+        for (size_t i = 0; i < v.size(); i++) if (v[i] == g) { v.erase(v.begin() + (long)i); break; }
+    }
+    delete g;
+}
+int mg_upload_hidden(mg_ctx* c, const float* data) { CTX(c); return f->UploadHidden(data); }
+int mg_read_hidden(mg_ctx* c, float* out) { CTX(c); return f->ExportHidden(out); }
+int mg_validate_graph_capture(mg_ctx* c, const float* hiddenIn, int layerStart, int layerEnd, float* maxDiff) {
+    CTX(c);
+    float md = 0.f;
+    int rc = f->ValidateGraphCapture(hiddenIn, layerStart, layerEnd, &md);
+    if (maxDiff) *maxDiff = md;
+    if (rc) return rc;
+    return md < 0.001f ? 1 : 0;
+}
+int mg_has_graph_kernel(void) { return 1; }
 int mg_timed_decode(mg_ctx* c, int token, int pos, int steps, int useGraph, float* ms) {
     CTX(c); return f->TimedDecode(token, pos, steps, useGraph != 0, ms);
 }

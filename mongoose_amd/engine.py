@@ -337,6 +337,37 @@ def synth_tokens(seed, idx, bound, n):
     return out
 
 
+class GraphCaptureConfig:
+    """cuda_graph.go:292-298."""
+
+    def __init__(self, LayerStart=0, LayerEnd=0, StreamCount=1, PipelineBreak=0):
+        self.LayerStart, self.LayerEnd, self.StreamCount, self.PipelineBreak = LayerStart, LayerEnd, StreamCount, PipelineBreak
+
+
+class HIPGraph:
+    """CUDAGraph, cuda_graph.go:300-310: a captured graph over a range of layers."""
+
+    def __init__(self, handle, cfg):
+        self._h, self.config = handle, cfg
+
+    def Launch(self, pos):
+        """cuda_graph.go:663: asynchronous; ReadHidden / ExportHidden wait for it."""
+        if not self._h:
+            return -1
+        return lib.mg_layer_graph_launch(self._h, pos)
+
+    def Destroy(self):
+        """cuda_graph.go:716."""
+        if self._h:
+            lib.mg_layer_graph_destroy(self._h)
+            self._h = None
+
+
+def HasGraphKernel():
+    """cuda_graph.go:281."""
+    return lib.mg_has_graph_kernel() != 0
+
+
 class HIPFusedInference:
     """Method set of CUDAFusedInference (cuda_fused_infer_stub.go:11-49)."""
 
@@ -468,6 +499,51 @@ class HIPFusedInference:
         md = ctypes.c_float(0)
         rc = lib.mg_graph_validate(self._h, token, pos, ctypes.byref(md))
         return rc, md.value
+
+    # ---- CUDAGraph mirror, cuda_graph.go:286-739 ----
+    def CaptureGraph(self, cfg, pos):
+        """(*CUDAFusedInference).CaptureGraph(cfg, pos), cuda_graph.go:315: a HIPGraph over cfg.LayerStart ..
+        cfg.LayerEnd, or None (error text in last_error())."""
+        h = lib.mg_layer_graph_capture(self._h, cfg.LayerStart, cfg.LayerEnd, cfg.StreamCount, cfg.PipelineBreak, pos)
+        return HIPGraph(h, cfg) if h else None
+
+    def UpdateAndLaunch(self, g, pos):
+        """cuda_graph.go:673: True when the graph was launched at pos."""
+        return bool(g._h) and lib.mg_layer_graph_update_and_launch(g._h, pos) == 1
+
+    def UploadHidden(self, data):
+        """cuda_graph.go:650."""
+        d = np.ascontiguousarray(data, dtype=np.float32)
+        assert d.size == self.dim
+        return lib.mg_upload_hidden(self._h, _fp(d))
+
+    def ReadHidden(self):
+        """cuda_graph.go:655: the current hidden buffer (waits for the stream)."""
+        out = np.empty(self.dim, dtype=np.float32)
+        return out if lib.mg_read_hidden(self._h, _fp(out)) == 0 else None
+
+    def ValidateGraphCapture(self, hiddenIn, layerStart, layerEnd):
+        """cuda_graph.go:554-598: eager and graph output of the range at position 0 differ by less than 1e-3.
+        Returns (ok, maxDiff)."""
+        d = np.ascontiguousarray(hiddenIn, dtype=np.float32)
+        md = ctypes.c_float(0)
+        rc = lib.mg_validate_graph_capture(self._h, _fp(d), layerStart, layerEnd, ctypes.byref(md))
+        return rc == 1, md.value
+
+    def ValidateMultiStreamGraph(self, hiddenIn, layerStart, layerEnd, pipelineBreak):
+        """cuda_graph.go:603-647.  The two-stream graph of the reference is sequential (stage B waits for stage A),
+        so this is ValidateGraphCapture with the break checked."""
+        if pipelineBreak <= layerStart or pipelineBreak >= layerEnd:
+            return False, float("nan")
+        return self.ValidateGraphCapture(hiddenIn, layerStart, layerEnd)
+
+    def TestMinimalCapture(self):
+        """cuda_graph.go:536: the graph API works on this runtime (a one-layer capture and replay)."""
+        g = self.CaptureGraph(GraphCaptureConfig(0, 1), 0)
+        if g is None:
+            return False
+        g.Destroy()
+        return True
 
     def TimedDecode(self, token, pos, steps, useGraph=True):
         ms = ctypes.c_float(0)

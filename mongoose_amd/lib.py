@@ -100,6 +100,14 @@ _sig("mg_generate", c_int, c_void_p, _i, c_int, c_int, _i, c_int)
 _sig("mg_graph_capture", c_int, c_void_p)
 _sig("mg_graph_launch", c_int, c_void_p, c_int, c_int, _i)
 _sig("mg_graph_validate", c_int, c_void_p, c_int, c_int, _f)
+_sig("mg_layer_graph_capture", c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int)
+_sig("mg_layer_graph_launch", c_int, c_void_p, c_int)
+_sig("mg_layer_graph_update_and_launch", c_int, c_void_p, c_int)
+_sig("mg_layer_graph_destroy", None, c_void_p)
+_sig("mg_upload_hidden", c_int, c_void_p, _f)
+_sig("mg_read_hidden", c_int, c_void_p, _f)
+_sig("mg_validate_graph_capture", c_int, c_void_p, _f, c_int, c_int, _f)
+_sig("mg_has_graph_kernel", c_int)
 _sig("mg_timed_decode", c_int, c_void_p, c_int, c_int, c_int, c_int, _f)
 _sig("mg_profile_decode", c_int, c_void_p, c_int, c_int, c_int, ctypes.c_uint, _f, _i)
 _sig("mg_prefill", c_int, c_void_p, _i, c_int, c_int, _i, _f, _f)
