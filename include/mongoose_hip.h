@@ -243,9 +243,8 @@ int mg_hidden_idx(mg_ctx* ctx);
  * also fetch the following matrices into L2 with its idle workgroups (for a GPU
  * shared with other work); 3 = all layers of a step in ONE persistent launch whose
  * workgroups hand their vectors over through device memory, wherever the model allows it
- * (Q8 weights, fp32 KV rows, heads of 64 or 128, the context within 256 (heads of 64) or
- * 128 (heads of 128) positions per attention workgroup with nHeads x splits workgroups at
- * most as many as the GPU has CUs; otherwise as mode 1).
+ * (Q8 weights, fp32 KV rows, heads of 64 or 128, a context of at most 128 x floor(CUs / nHeads)
+ * positions: one workgroup per query head and 128 positions; otherwise as mode 1).
  * A new context is in automatic mode: as mode 3 where that launch is also the faster one --
  * at least 8 layers of at most 64 MB of weights each, i.e. steps bound by the hand-over
  * between dependent phases rather than by HBM (measured: 0.5B and 1.1B shapes 10-18 %

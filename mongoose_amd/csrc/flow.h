@@ -27,14 +27,14 @@ struct FlowLayer {
 // the K and V rows of the current position, the attention partials of up to smax KV splits (accumulator,
 // maximum, sum), the hidden state after the attention block, the SwiGLU vector and the layer's output.
 // Every float is the pattern 0xFFFFFFFF until its producer has written it.
-constexpr int FLOW_MIN_TILE = 128;     // positions of the smallest attention tile (it doubles until the slots cover the context)
+constexpr int FLOW_TILE = 128;         // positions of an attention tile: one workgroup per (query head, tile)
 struct FlowGeometry {
     int stride;
     int offQ, offKc, offVc, offPacc, offPm, offPl, offX1, offM, offX2;
     int smax;
 };
 FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int headDim, int maxSeq, int grid);
-bool flow_context_fits(int headDim, int maxSeq, const FlowGeometry& g);
+bool flow_context_fits(int maxSeq, const FlowGeometry& g);
 
 // Trace slots of a layer, in program order: when thread 0 of a workgroup passed the point.
 constexpr int FLOW_TRACE_SLOTS = 11;
@@ -62,7 +62,7 @@ struct FlowParams {
 // Workgroups the launch needs at least (one per query head and KV split) for this shape.
 int flow_min_grid(int nHeads, const FlowGeometry& g);
 bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads, int headDim);
-// grid workgroups of 256 threads, all of which must be resident at once (grid <= CUs x resident workgroups per CU).
+// grid workgroups of 512 threads, all of which must be resident at once (grid <= CUs x resident workgroups per CU).
 hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s);
 // Fills the blocks of layers [l0, l1) with the "not written yet" pattern.
 hipError_t launch_flow_reset(float* xchg, const FlowGeometry& g, int l0, int l1, hipStream_t s);

@@ -20,6 +20,8 @@
 namespace mg {
 
 constexpr unsigned XSENT = 0xFFFFFFFFu;
+constexpr int FWAVES = 8;                 // waves of a workgroup (two a SIMD: a wave's instruction latencies are covered by its partner)
+constexpr int FWG = 64 * FWAVES;
 typedef float f4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ bool unset(float v) { return __builtin_bit_cast(unsigned, v) == XSENT; }
@@ -70,10 +72,10 @@ __device__ __forceinline__ float poll1(const float* p, Waiter& w) {
     }
     return v;
 }
-// The first n of five pieces with all their loads in flight at once: one memory round trip instead of n.
+// The first n of three pieces with all their loads in flight at once: one memory round trip instead of n.
 // Loads and the wait for them are one asm statement each time -- with the wait in a statement of its own the
 // compiler is free to copy a destination register between the two, i.e. before the data has arrived.
-__device__ __forceinline__ void ldx4_n(const f4* const (&p)[5], f4 (&v)[5], int n) {
+__device__ __forceinline__ void ldx4_n(const f4* const (&p)[3], f4 (&v)[3], int n) {
     switch (n) {
     case 1:
         asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(v[0]) : "v"(p[0]) : "memory");
@@ -82,23 +84,25 @@ __device__ __forceinline__ void ldx4_n(const f4* const (&p)[5], f4 (&v)[5], int 
         asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %3, off sc1\n\ts_waitcnt vmcnt(0)"
                      : "=&v"(v[0]), "=&v"(v[1]) : "v"(p[0]), "v"(p[1]) : "memory");
         break;
-    case 3:
+    default:
         asm volatile("global_load_dwordx4 %0, %3, off sc1\n\tglobal_load_dwordx4 %1, %4, off sc1\n\t"
                      "global_load_dwordx4 %2, %5, off sc1\n\ts_waitcnt vmcnt(0)"
                      : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]) : "v"(p[0]), "v"(p[1]), "v"(p[2]) : "memory");
         break;
-    case 4:
-        asm volatile("global_load_dwordx4 %0, %4, off sc1\n\tglobal_load_dwordx4 %1, %5, off sc1\n\t"
-                     "global_load_dwordx4 %2, %6, off sc1\n\tglobal_load_dwordx4 %3, %7, off sc1\n\ts_waitcnt vmcnt(0)"
-                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]) : "memory");
-        break;
-    default:
-        asm volatile("global_load_dwordx4 %0, %5, off sc1\n\tglobal_load_dwordx4 %1, %6, off sc1\n\t"
-                     "global_load_dwordx4 %2, %7, off sc1\n\tglobal_load_dwordx4 %3, %8, off sc1\n\t"
-                     "global_load_dwordx4 %4, %9, off sc1\n\ts_waitcnt vmcnt(0)"
-                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4])
-                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]) : "memory");
-        break;
+    }
+}
+// A KV split's partial for one 16-byte piece of the attention output: accumulator piece, maximum and sum of its head,
+// asked for together (one round trip), repeated until all three are there.
+__device__ __forceinline__ void poll_partial(const f4* pa, const float* pm, const float* pl, f4& a, float& m, float& l, Waiter& w) {
+    long long t0 = 0;
+    bool timing = false;
+    for (;;) {
+        asm volatile("global_load_dwordx4 %0, %3, off sc1\n\tglobal_load_dword %1, %4, off sc1\n\t"
+                     "global_load_dword %2, %5, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(a), "=&v"(m), "=&v"(l) : "v"(pa), "v"(pm), "v"(pl) : "memory");
+        if ((ready4(a) && !unset(m) && !unset(l)) || w.dead) break;
+        if (!timing) { timing = true; t0 = wall_clock64(); }
+        else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
     }
 }
 // A layer's table entry, read one layer ahead: lane i loads word i, and the fields are picked out of the lanes into
@@ -129,7 +133,7 @@ __device__ __forceinline__ FlowLayer unpack_layer(unsigned v) {
 }
 #undef FL_PTR
 
-constexpr int PB = 5;        // float4 pieces a thread polls at once
+constexpr int PB = 3;        // float4 pieces a thread polls at once (a round of the 512 threads covers 6144 floats)
 // n uniform in the workgroup, 1..PB; pieces past n are left as they are
 __device__ __forceinline__ void poll_batch(const f4* const (&ptr)[PB], f4 (&v)[PB], int n, Waiter& w) {
     long long t0 = 0;
@@ -158,17 +162,17 @@ __device__ __forceinline__ float stage_rms(const float* x, bool polled, const fl
     const float4* g4 = reinterpret_cast<const float4*>(gain);
     __syncthreads();                                   // the previous phase's readers of a4 are done
     float ss = 0.f;
-    for (int base = 0; base < K4; base += WG * PB) {
+    for (int base = 0; base < K4; base += FWG * PB) {
         f4 v[PB];
         float4 g[PB];
         const f4* ptr[PB];
 #pragma unroll
         for (int u = 0; u < PB; u++) {
-            const int i = min(base + u * WG + tid, K4 - 1);
+            const int i = min(base + u * FWG + tid, K4 - 1);
             ptr[u] = x4 + i;
             g[u] = g4[i];
         }
-        const int np = min(PB, (K4 - base + WG - 1) / WG);      // pieces of this round (uniform)
+        const int np = min(PB, (K4 - base + FWG - 1) / FWG);      // pieces of this round (uniform)
 #pragma unroll
         for (int u = 0; u < PB; u++) v[u] = f4{0.f, 0.f, 0.f, 0.f};
         if (polled) {
@@ -179,7 +183,7 @@ __device__ __forceinline__ float stage_rms(const float* x, bool polled, const fl
         }
 #pragma unroll
         for (int u = 0; u < PB; u++) {
-            const int i = base + u * WG + tid;
+            const int i = base + u * FWG + tid;
             if (i < K4) {
                 ss += v[u].x * v[u].x + v[u].y * v[u].y + v[u].z * v[u].z + v[u].w * v[u].w;
                 a4[slot4(i, nch)] = make_float4(v[u].x * g[u].x, v[u].y * g[u].y, v[u].z * g[u].z, v[u].w * g[u].w);
@@ -189,7 +193,9 @@ __device__ __forceinline__ float stage_rms(const float* x, bool polled, const fl
     ss = wave_sum(ss);
     if ((tid & 63) == 0) red[tid >> 6] = ss;
     __syncthreads();
-    const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+    float tot = 0.f;
+#pragma unroll
+    for (int k = 0; k < FWAVES; k++) tot += red[k];
     return __builtin_amdgcn_rsqf(tot * __builtin_amdgcn_rcpf((float)K) + eps);
 }
 
@@ -198,15 +204,15 @@ __device__ __forceinline__ void stage_plain(const float* x, int K, float4* a4, W
     const int K4 = K >> 2, nch = K >> 4, tid = threadIdx.x;
     const f4* x4 = reinterpret_cast<const f4*>(x);
     __syncthreads();
-    for (int base = 0; base < K4; base += WG * PB) {
+    for (int base = 0; base < K4; base += FWG * PB) {
         f4 v[PB];
         const f4* ptr[PB];
 #pragma unroll
-        for (int u = 0; u < PB; u++) { ptr[u] = x4 + min(base + u * WG + tid, K4 - 1); v[u] = f4{0.f, 0.f, 0.f, 0.f}; }
-        poll_batch(ptr, v, min(PB, (K4 - base + WG - 1) / WG), w);
+        for (int u = 0; u < PB; u++) { ptr[u] = x4 + min(base + u * FWG + tid, K4 - 1); v[u] = f4{0.f, 0.f, 0.f, 0.f}; }
+        poll_batch(ptr, v, min(PB, (K4 - base + FWG - 1) / FWG), w);
 #pragma unroll
         for (int u = 0; u < PB; u++) {
-            const int i = base + u * WG + tid;
+            const int i = base + u * FWG + tid;
             if (i < K4) a4[slot4(i, nch)] = tof4(v[u]);
         }
     }
@@ -247,39 +253,36 @@ __device__ __forceinline__ void dot_rows_tail(const signed char* const (&rows)[N
     }
 }
 
-constexpr int CBD = 2;       // chunks a lane prefetches per row of K = dim (rows up to 2048 weights in one batch)
 constexpr int CBF = 6;       // ... per row of K = ffnDim (rows up to 6144 weights in one batch)
-constexpr int NIB = 6;       // gate/up items (a gate row and its up row) a wave holds in flight
-constexpr int NID = 2;       // down rows a wave holds in flight
+constexpr int NIB = 24 / FWAVES;   // gate/up items (a gate row and its up row) a wave holds in flight
+constexpr int NID = 8 / FWAVES;    // down rows a wave holds in flight
 
-template <int HD>
-__global__ __launch_bounds__(WG) void flow_layers_kernel(FlowParams p) {
+// CBD: chunks a lane prefetches per row of K = dim (1: rows of up to 1024 weights in one batch, 2: up to 2048)
+template <int HD, int CBD>
+__global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     extern __shared__ float4 a4[];                     // the staged activation vector, max(dim, ffn) floats
-    __shared__ float red[4];
+    __shared__ float red[FWAVES];
     __shared__ float4 sqkv[3][HD / 4];                 // q of the head, K and V row of the current position
-    __shared__ float4 accbuf[4][HD / 4];
-    __shared__ float lbuf[4], wred[4];
+    __shared__ float4 accbuf[FWAVES][HD / 4];
+    __shared__ float lbuf[FWAVES], wred[FWAVES];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int gw = blockIdx.x * 4 + wave;              // this wave among all waves of the launch
-    const int W = gridDim.x * 4;
+    const int gw = blockIdx.x * FWAVES + wave;         // this wave among all waves of the launch
+    const int W = gridDim.x * FWAVES;
     const int dim = p.dim, kvDim = p.kvDim, ffn = p.ffn;
     const int nchD = dim >> 4, nchF = ffn >> 4;
     const FlowGeometry G = p.geo;
     const int pos = p.state ? p.state->pos : p.posImm;
     Waiter wt{p.limitTicks, p.err, false};
 
-    // attention geometry (decode attention of kernels.hip with one query head per workgroup, 256 threads)
-    // A thread group of 16 lanes holds a K/V row; a thread holds up to VU rows of its workgroup's tile.  The tile is
-    // FLOW_MIN_TILE positions and doubles until the partial slots cover the context: the fewer rows a thread has,
-    // the shorter the serial part of the phase (measured on the 0.5B shape at 100-200 positions: 128 beats 256
-    // by 5%, and beats 64 and 32, whose extra partials cost more to merge than the rows save).
-    constexpr int LPR = 16, NF = HD / 64, TG = WG / LPR, VU = 16 / NF;
+    // attention geometry (decode attention of kernels.hip with one query head per workgroup): a thread group of 16
+    // lanes holds a K/V row, a thread VU rows of its workgroup's tile of FLOW_TILE positions.  (Measured on the 0.5B
+    // shape at 100-200 positions: tiles of 128 beat 256 by 5 %, and beat 64 and 32, whose extra partials cost more to
+    // merge than the rows save; a kernel that can also take tiles of 256 is 2-3 % slower at every context for the
+    // unrolled code alone.)
+    constexpr int LPR = 16, NF = HD / 64, TG = FWG / LPR, VU = FLOW_TILE / TG, TILE = FLOW_TILE;
     const int half = HD >> 1;
-    int tile = FLOW_MIN_TILE;
-    while (pos / tile + 1 > G.smax && tile < TG * VU) tile <<= 1;
-    const int TILE = tile, VUe = tile / TG;
 
     // timing trace (diagnostic): slot b of layer l, per workgroup, in ticks of the 100 MHz wall clock
 #define FLOW_TRACE(b) do { if (p.trace && tid == 0) \
@@ -296,7 +299,7 @@ __global__ __launch_bounds__(WG) void flow_layers_kernel(FlowParams p) {
         // ------------------------------------------------------------------ q | k | v
         {
             const int nq = dim >> 1, nk = kvDim >> 1, nI = nq + 2 * nk;       // RoPE pairs of q, of k; row pairs of v
-            if (blockIdx.x * 4 < nI) {
+            if (blockIdx.x * FWAVES < nI) {
                 int it = gw;
                 int4 wr[2][CBD];
                 const signed char* rows[2] = {L.wq, L.wq};
@@ -369,7 +372,6 @@ __global__ __launch_bounds__(WG) void flow_layers_kernel(FlowParams p) {
                 float4 kreg[VU][NF], vreg[VU][NF];
 #pragma unroll
                 for (int u = 0; u < VU; u++) {
-                    if (u >= VUe) continue;             // uniform
                     const size_t ro = (size_t)min(t0 + tg + u * TG, lastRow) * rowStride + colOff;
 #pragma unroll
                     for (int j = 0; j < NF; j++) kreg[u][j] = Kc4[ro + j * 16];
@@ -436,11 +438,13 @@ __global__ __launch_bounds__(WG) void flow_layers_kernel(FlowParams p) {
                 if (lane == 0) { lbuf[wave] = lsum; wred[wave] = m; }
                 __syncthreads();
                 if (tid < HD / 4) {
-                    const float mg_ = fmaxf(fmaxf(wred[0], wred[1]), fmaxf(wred[2], wred[3]));
+                    float mg_ = wred[0];
+#pragma unroll
+                    for (int k = 1; k < FWAVES; k++) mg_ = fmaxf(mg_, wred[k]);
                     f4 r = {0.f, 0.f, 0.f, 0.f};
                     float lg = 0.f;
 #pragma unroll
-                    for (int k = 0; k < 4; k++) {
+                    for (int k = 0; k < FWAVES; k++) {
                         const float wk = exp_neg(wred[k] - mg_);
                         const float4 a = accbuf[k][tid];
                         r.x = fmaf(wk, a.x, r.x); r.y = fmaf(wk, a.y, r.y); r.z = fmaf(wk, a.z, r.z); r.w = fmaf(wk, a.w, r.w);
@@ -459,7 +463,7 @@ __global__ __launch_bounds__(WG) void flow_layers_kernel(FlowParams p) {
         // ------------------------------------------------------------------ Wo + residual
         {
             const int nI = dim;
-            if (blockIdx.x * 4 < nI) {
+            if (blockIdx.x * FWAVES < nI) {
                 int it = gw;
                 int4 wr[1][CBD];
                 const signed char* rows[1] = {L.wo};
@@ -478,14 +482,19 @@ __global__ __launch_bounds__(WG) void flow_layers_kernel(FlowParams p) {
                 {
                     const int nsplit = pos / TILE + 1;
                     const int ns = nsplit < G.smax ? nsplit : G.smax;
-                    for (int i = tid; i < (dim >> 2); i += WG) {
+                    for (int i = tid; i < (dim >> 2); i += FWG) {
                         const int h = (i * 4) / HD;
                         float M = -INFINITY, den = 0.f;
                         f4 num = {0.f, 0.f, 0.f, 0.f};
                         for (int s = 0; s < ns; s++) {
-                            const f4 a = poll4(reinterpret_cast<const f4*>(X + G.offPacc + (size_t)s * dim) + i, wt);
-                            const float ms = poll1(X + G.offPm + s * p.nHeads + h, wt);
-                            const float ls = poll1(X + G.offPl + s * p.nHeads + h, wt);
+                            f4 a;
+                            float ms, ls;
+                            const f4* pa = reinterpret_cast<const f4*>(X + G.offPacc + (size_t)s * dim) + i;
+                            // The split everybody has to wait for is waited for on the accumulator pieces alone: they are
+                            // spread over many lines, while the maxima and sums of all heads share one, and a line that
+                            // 50,000 threads keep re-reading takes its producer's store late.
+                            if (s == 0) a = poll4(pa, wt);
+                            poll_partial(pa, X + G.offPm + s * p.nHeads + h, X + G.offPl + s * p.nHeads + h, a, ms, ls, wt);
                             const float Mn = fmaxf(M, ms);
                             const float c = exp_neg(M - Mn);                    // first split: exp(-inf) = 0
                             const float wgt = exp_neg(ms - Mn);
@@ -515,7 +524,7 @@ __global__ __launch_bounds__(WG) void flow_layers_kernel(FlowParams p) {
         // ------------------------------------------------------------------ gate | up, SiLU(g) * u
         {
             const int nI = ffn;
-            if (blockIdx.x * 4 < nI) {
+            if (blockIdx.x * FWAVES < nI) {
                 int4 wr[NIB][2][CBD];
                 float sg = 0.f, su = 0.f;
                 auto issue = [&](int it0) {
@@ -565,7 +574,7 @@ __global__ __launch_bounds__(WG) void flow_layers_kernel(FlowParams p) {
         // ------------------------------------------------------------------ down + residual
         {
             const int nI = dim;
-            if (blockIdx.x * 4 < nI) {
+            if (blockIdx.x * FWAVES < nI) {
                 int4 wr[NID][1][CBF];
                 float e0 = 0.f, e1 = 0.f;
                 auto issue = [&](int it0) {
@@ -610,8 +619,8 @@ __global__ __launch_bounds__(WG) void flow_layers_kernel(FlowParams p) {
 
 FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int headDim, int maxSeq, int grid) {
     FlowGeometry g{};
-    // partial slots: one per FLOW_MIN_TILE positions, at most as many as the workgroups of the launch can serve
-    g.smax = (maxSeq + FLOW_MIN_TILE - 1) / FLOW_MIN_TILE;
+    // partial slots: one per FLOW_TILE positions, at most as many as the workgroups of the launch can serve
+    g.smax = (maxSeq + FLOW_TILE - 1) / FLOW_TILE;
     if (nHeads > 0 && g.smax > grid / nHeads) g.smax = grid / nHeads;
     if (g.smax < 1) g.smax = 1;
     auto up64 = [](int v) { return (v + 63) & ~63; };
@@ -630,8 +639,8 @@ FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int headDim,
 }
 
 int flow_min_grid(int nHeads, const FlowGeometry& g) { return nHeads * g.smax; }
-// the largest tile (16 rows a thread for heads of 64, 8 for heads of 128) times the slots covers the context
-bool flow_context_fits(int headDim, int maxSeq, const FlowGeometry& g) { return (long long)(headDim == 128 ? 128 : 256) * g.smax >= maxSeq; }
+// one workgroup per (query head, tile): the slots cover the context
+bool flow_context_fits(int maxSeq, const FlowGeometry& g) { return (long long)FLOW_TILE * g.smax >= maxSeq; }
 
 bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads, int headDim) {
     if (headDim != 64 && headDim != 128) return false;
@@ -644,11 +653,17 @@ bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads,
 hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
     if (!flow_shape_supported(p.dim, p.kvDim, p.ffn, p.nHeads, p.nKVHeads, p.headDim)) return hipErrorInvalidValue;
     if (p.l0 < 0 || p.l1 <= p.l0 || p.l1 > p.nLayersTotal || grid < flow_min_grid(p.nHeads, p.geo) ||
-        !flow_context_fits(p.headDim, p.maxSeq, p.geo) || !p.layers || !p.xchg || !p.err || !p.hidden)
+        !flow_context_fits(p.maxSeq, p.geo) || !p.layers || !p.xchg || !p.err || !p.hidden)
         return hipErrorInvalidValue;
     const size_t lds = (size_t)(p.dim > p.ffn ? p.dim : p.ffn) * sizeof(float);
-    if (p.headDim == 64) hipLaunchKernelGGL(flow_layers_kernel<64>, dim3(grid), dim3(WG), lds, s, p);
-    else hipLaunchKernelGGL(flow_layers_kernel<128>, dim3(grid), dim3(WG), lds, s, p);
+    const bool wide = p.dim > 1024;
+    if (p.headDim == 64) {
+        if (wide) hipLaunchKernelGGL((flow_layers_kernel<64, 2>), dim3(grid), dim3(FWG), lds, s, p);
+        else hipLaunchKernelGGL((flow_layers_kernel<64, 1>), dim3(grid), dim3(FWG), lds, s, p);
+    } else {
+        if (wide) hipLaunchKernelGGL((flow_layers_kernel<128, 2>), dim3(grid), dim3(FWG), lds, s, p);
+        else hipLaunchKernelGGL((flow_layers_kernel<128, 1>), dim3(grid), dim3(FWG), lds, s, p);
+    }
     return hipGetLastError();
 }
 

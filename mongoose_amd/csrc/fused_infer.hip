@@ -662,7 +662,7 @@ bool HIPFusedInference::flowEligible(int l0, int l1) const {
         cus = prop.multiProcessorCount;
     }
     const FlowGeometry g = flow_geometry(dim, kvDim, ffnDim, nHeads, headDim, maxSeq, cus);
-    return flow_min_grid(nHeads, g) <= cus && flow_context_fits(headDim, maxSeq, g);
+    return flow_min_grid(nHeads, g) <= cus && flow_context_fits(maxSeq, g);
 }
 
 int HIPFusedInference::ensureFlow() {

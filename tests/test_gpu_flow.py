@@ -5,7 +5,7 @@ their vectors over through an exchange area in device memory.
   vector, layer output), read back from the exchange area, against a float64 numpy evaluation of the layer
   (cuda_fused_infer.go:414-444 order, kernels/mongoose.cu:145-174, 856-933, 949-956, 991-1006 arithmetic);
 * tokens through the launch == the oracle's, through graph replay and eager launches, and == the fused launches';
-* contexts that need several KV splits per head, and a context long enough that the attention tile doubles;
+* contexts that need several KV splits per head, up to every partial slot in use;
 * heads of 128 with grouped KV heads;
 * automatic mode picks the launch for a many-layer small model and not for a 4-layer one;
 * a wait that runs out: the launch still ends, the call reports it, the context continues with the fused launches.
@@ -130,15 +130,20 @@ def _modes_agree(m, prompt, nDecode, what):
     return out[3]
 
 
-def test_kv_splits_and_tile_doubling_heads_of_64(hip):
-    """0.5B geometry (14 query heads on 2 KV heads, biases), 2 layers.  Up to 18 partial slots per head: positions
-    600..640 use 5-6 splits of 128 positions; from position 2304 the tile is 256."""
+def test_kv_splits_heads_of_64(hip):
+    """0.5B geometry (14 query heads on 2 KV heads, biases), 2 layers.  18 partial slots per head (256 CUs / 14 heads),
+    i.e. contexts of up to 2304 positions: positions 600..640 use 5-6 splits of 128 positions, 2260..2300 all 18.
+    A longer context does not fit the launch: the context then runs the fused launches."""
     s = H.with_layers(configs.QWEN, 2)._replace(name="qwen-geom", vocab=2048)
-    m = H.Model(s, seed=11, maxSeq=2400, eng=hip, oracle=False)
+    m = H.Model(s, seed=11, maxSeq=2304, eng=hip, oracle=False)
     print("flow: qwen geometry, positions 600..640", flush=True)
     _modes_agree(m, m.prompt(600), 40, "5-6 splits")
-    print("flow: qwen geometry, positions 2290..2330 (tile doubles at 2304)", flush=True)
-    _modes_agree(m, m.prompt(2290), 40, "tile 128 -> 256")
+    print("flow: qwen geometry, positions 2260..2300 (18 splits)", flush=True)
+    _modes_agree(m, m.prompt(2260), 40, "18 splits")
+    m.close()
+    m = H.Model(s, seed=11, maxSeq=2305, eng=hip, oracle=False)
+    assert m.hip.SetExecMode(3) == 0
+    assert not _in_use(m.hip)
     m.close()
 
 
