@@ -271,11 +271,30 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     __shared__ float4 sqkv[3][HD / 4];                 // q of the head, K and V row of the current position
     __shared__ float4 accbuf[FWAVES][HD / 4];
     __shared__ float lbuf[FWAVES], wred[FWAVES];
+    __shared__ float outbuf[NIB][FWAVES];                // a phase's results of the workgroup, stored by one wave as whole 32-byte runs
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int gw = blockIdx.x * FWAVES + wave;         // this wave among all waves of the launch
     const int W = gridDim.x * FWAVES;
+    // The rows of a workgroup's eight waves are consecutive (row = base + wave + k W), so their results go out as runs
+    // of eight floats in one store instruction of wave 0 instead of eight single-float stores from eight waves: a line
+    // of a handed-over vector is then written 4 times, not 32, while 256 workgroups keep re-reading it.
+    // Lane k < nk of every wave holds the value of its row k; all waves of the workgroup call this together.
+    // rowOff: offset of this round's rows from the first round's (the same for all waves).
+    auto store_runs = [&](float val, int nk, int nI, int rowOff, float* dst, float* dst2) {
+        if (lane < nk) outbuf[lane][wave] = val;
+        __syncthreads();
+        if (wave == 0 && lane < nk * FWAVES) {
+            const int k = lane / FWAVES, wv = lane % FWAVES;
+            const int r = blockIdx.x * FWAVES + wv + k * W + rowOff;
+            if (r < nI) {
+                const float o = outbuf[k][wv];
+                stx(dst + r, o);
+                if (dst2) dst2[r] = o;
+            }
+        }
+    };
     const int dim = p.dim, kvDim = p.kvDim, ffn = p.ffn;
     const int nchD = dim >> 4, nchF = ffn >> 4;
     const FlowGeometry G = p.geo;
@@ -521,7 +540,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     dot_rows<1, CBD>(wr, a4, nchD, lane, 0, acc);
                     if (nchD > CBD * 64) dot_rows_tail<1, CBD>(rows, a4, nchD, lane, acc);
                     const float v = wave_sum(acc[0]);
-                    if (lane == 0) stx(X + G.offX1 + it, e1 + v * e0);
+                    if (it != gw) __syncthreads();              // outbuf is free again
+                    store_runs(e1 + v * e0, 1, nI, it - gw, X + G.offX1, nullptr);
                 }
             }
         }
@@ -565,13 +585,11 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         }
                         if (lane == k) { g = acc[0]; u = acc[1]; }
                     }
-                    const int r = it0 + lane * W;
-                    if (lane < NIB && r < nI) {
-                        g = g * sg; g = g * rs;
-                        u = u * su; u = u * rs;
-                        const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f));   // mongoose.cu:949-956
-                        stx(X + G.offM + r, g * sig * u);
-                    }
+                    g = g * sg; g = g * rs;
+                    u = u * su; u = u * rs;
+                    const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f));   // mongoose.cu:949-956
+                    if (it0 != gw) __syncthreads();             // outbuf is free again
+                    store_runs(g * sig * u, NIB, nI, it0 - gw, X + G.offM, nullptr);
                 }
             }
         }
@@ -610,12 +628,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         }
                         if (lane == k) v = acc[0];
                     }
-                    const int r = it0 + lane * W;
-                    if (lane < NID && r < nI) {
-                        const float o = e1 + v * e0;
-                        stx(X + G.offX2 + r, o);
-                        if (l == p.l1 - 1) p.hidden[r] = o;
-                    }
+                    if (it0 != gw) __syncthreads();             // outbuf is free again
+                    store_runs(e1 + v * e0, NID, nI, it0 - gw, X + G.offX2, l == p.l1 - 1 ? p.hidden : nullptr);
                 }
             }
         }
