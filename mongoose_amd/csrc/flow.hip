@@ -362,16 +362,27 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     v = v + e1;
                     const float v1 = dpp_f<0x101>(v);                            // lane 0 reads lane 1: the pair's second row
                     const float cs = dpp_f<0x102>(e0), sn = dpp_f<0x102>(e1);    // lane 0 reads lane 2
-                    if (lane == 0) {
-                        float o0 = v, o1 = v1;
-                        if (kind < 2) { o0 = v * cs - v1 * sn; o1 = v * sn + v1 * cs; }      // mongoose.cu:991-1006
-                        if (kind == 0) {
-                            stx(X + G.offQ + r0, o0); stx(X + G.offQ + r1, o1);
-                        } else {                                                  // mongoose.cu:1644-1647, and the hand-over copy
-                            float* cache = (kind == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim;
-                            cache[r0] = o0; cache[r1] = o1;
-                            float* cur = X + (kind == 1 ? G.offKc : G.offVc);
-                            stx(cur + r0, o0); stx(cur + r1, o1);
+                    float o0 = v, o1 = v1;
+                    if (kind < 2) { o0 = v * cs - v1 * sn; o1 = v * sn + v1 * cs; }          // mongoose.cu:991-1006
+                    // the eight waves' rows are consecutive (first rows of the pairs, and second rows): out as runs by wave 0
+                    if (it != gw) __syncthreads();              // outbuf is free again
+                    if (lane == 0) { outbuf[0][wave] = o0; outbuf[1][wave] = o1; }
+                    __syncthreads();
+                    if (wave == 0 && lane < 2 * FWAVES) {
+                        const int k = lane / FWAVES, wv = lane % FWAVES, item = it + wv;
+                        if (item < nI) {
+                            int kd, a0, a1;
+                            if (item < nq) { kd = 0; const int j = item % half; a0 = (item - j) * 2 + j; a1 = a0 + half; }
+                            else if (item < nq + nk) { kd = 1; const int i2 = item - nq; const int j = i2 % half; a0 = (i2 - j) * 2 + j; a1 = a0 + half; }
+                            else { kd = 2; a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
+                            const int r = k ? a1 : a0;
+                            const float o = outbuf[k][wv];
+                            if (kd == 0) {
+                                stx(X + G.offQ + r, o);
+                            } else {                                              // mongoose.cu:1644-1647, and the hand-over copy
+                                ((kd == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim)[r] = o;
+                                stx(X + (kd == 1 ? G.offKc : G.offVc) + r, o);
+                            }
                         }
                     }
                 }
