@@ -487,7 +487,8 @@ class HIPFusedInference:
         rc = lib.mg_generate(self._h, _ip(p), p.size, nDecode, _ip(out), 1 if useGraph else 0)
         return rc, out[:nDecode]
 
-    def CaptureGraph(self):
+    def CaptureTokenGraph(self):
+        """mg_graph_capture: the whole-token graphs (embedding gather .. argmax) that Generate / GraphLaunch replay."""
         return lib.mg_graph_capture(self._h)
 
     def GraphLaunch(self, token, pos):

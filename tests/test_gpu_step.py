@@ -171,7 +171,7 @@ def test_graph_replay_matches_eager(hip):
     prompt = m.prompt(6)
     rc, _ = m.hip.Generate(prompt, 4, useGraph=False)
     assert rc == 0, E.last_error()
-    assert m.hip.CaptureGraph() == 0, E.last_error()
+    assert m.hip.CaptureTokenGraph() == 0, E.last_error()
     for rep in range(3):                       # several replays with eager work in between
         rc, md = m.hip.ValidateGraph(int(prompt[rep]), 9 + rep)
         assert rc == 0, E.last_error()
