@@ -38,8 +38,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
 # here, keyed by (configuration, launch); profiles/ holds the runs they come from.  They are
 # NOT measured by the run that prints them: "traffic_source" in the output says so.
 PMC_TRAFFIC_BYTES = {
-    ("qwen2.5-0.5b", "lm_head"): int((67135.0 * (262144.0 / 131102.4) + 660.7 * 1.0) * 1024),
-    ("qwen2.5-0.5b", "flow"): int((190997.2 * (262144.0 / 131102.4) + 6004.0 * 1.0) * 1024),
+    ("qwen2.5-0.5b", "lm_head"): int((67135.1 * (262144.0 / 131102.4) + 660.5 * 1.0) * 1024),
+    ("qwen2.5-0.5b", "flow"): int((187425.9 * (262144.0 / 131102.4) + 864.5 * 1.0) * 1024),
 }
 PMC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script recorded in profiles/ (constants in bench.py, not measured by this run)"
 

@@ -245,11 +245,8 @@ int mg_hidden_idx(mg_ctx* ctx);
  * workgroups hand their vectors over through device memory, wherever the model allows it
  * (Q8 weights, fp32 KV rows, heads of 64 or 128, a context of at most 128 x floor(CUs / nHeads)
  * positions: one workgroup per query head and 128 positions; otherwise as mode 1).
- * A new context is in automatic mode: as mode 3 where that launch is also the faster one --
- * at least 8 layers of at most 64 MB of weights each, i.e. steps bound by the hand-over
- * between dependent phases rather than by HBM (measured: 0.5B and 1.1B shapes 10-18 %
- * faster, the 8B shape 26 % slower than mode 1) -- and as mode 1 elsewhere.  Setting a mode
- * ends automatic mode.
+ * A new context is in mode 3 (measured against mode 1: 0.5B shape 27 % faster, 1.1B shape 30 %,
+ * 8B shape 3-4 %, a 4-layer toy 18 %).
  * The persistent launch needs all its workgroups resident at once: on a GPU shared with
  * other kernels its waits can run into their time limit; the call then returns MG_E_HIP,
  * and the context continues with the fused launches.  All modes give the same results to

@@ -93,10 +93,8 @@ public:
     int quantRounding = 0;
     // 0: one launch per reference op; 1: fused launches; 2: fused, attention launches without the L2 prefetch
     // helpers; 3: all layers of a step in one persistent launch where the model allows it (else as 1).
-    // execAuto (until a mode is set): mode 3 only where that launch is also the faster one.
     int execMode = 3;
-    bool execAuto = true;
-    void SetExecMode(int mode) { if (mode != execMode || execAuto) invalidateGraphs(); execMode = mode; execAuto = false; }
+    void SetExecMode(int mode) { if (mode != execMode) invalidateGraphs(); execMode = mode; }
 
     // shape
     int dim, kvDim, headDim, nHeads, nKVHeads, ffnDim, vocabSize, nLayers, maxSeq;

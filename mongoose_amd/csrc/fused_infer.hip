@@ -639,12 +639,6 @@ int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const
 bool HIPFusedInference::flowEligible(int l0, int l1) const {
     if (execMode != 3 || flowBroken || kvHalf) return false;
     if (!flow_shape_supported(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim)) return false;
-    if (execAuto) {
-        // Only where the step is bound by the hand-over between dependent phases, not by HBM: with hundreds of KB of
-        // weights per CU and layer the separate launches stream them faster than the persistent workgroups do.
-        const uint64_t layerBytes = (uint64_t)dim * dim * 2 + (uint64_t)kvDim * dim * 2 + (uint64_t)ffnDim * dim * 3;
-        if (nLayers < 8 || layerBytes > (64ull << 20)) return false;
-    }
     if (l1 > nLayers) l1 = nLayers;
     if (l0 < 0 || l0 >= l1) return false;
     for (int l = l0; l < l1; l++) {

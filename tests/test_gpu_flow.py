@@ -7,7 +7,7 @@ their vectors over through an exchange area in device memory.
 * tokens through the launch == the oracle's, through graph replay and eager launches, and == the fused launches';
 * contexts that need several KV splits per head, up to every partial slot in use;
 * heads of 128 with grouped KV heads;
-* automatic mode picks the launch for a many-layer small model and not for a 4-layer one;
+* a new context uses the launch; the trace diagnostic;
 * a wait that runs out: the launch still ends, the call reports it, the context continues with the fused launches.
 """
 import numpy as np
@@ -88,7 +88,7 @@ def test_tokens_match_oracle_and_fused_launches(hip):
     m = H.Model(s, seed=3, maxSeq=72, eng=hip, threads=8)
     prompt = m.prompt(8)
     ref, _ = H.oracle_generate(m, prompt, 64)
-    assert not _in_use(m.hip), "automatic mode takes the persistent launch for a 4-layer model"
+    assert _in_use(m.hip), "a new context should use the persistent launch"
     out = {}
     for mode in (1, 3):
         assert m.hip.SetExecMode(mode) == 0
@@ -165,14 +165,14 @@ def test_heads_of_128_grouped_kv(hip):
     m.close()
 
 
-def test_automatic_mode_takes_the_launch_for_many_small_layers(hip):
+def test_new_context_uses_the_launch_and_trace(hip):
     s = H.with_layers(configs.TOY, 8)
     m = H.Model(s, seed=5, maxSeq=40, eng=hip, threads=8)
     prompt = m.prompt(4)
     ref, _ = H.oracle_generate(m, prompt, 16)
     rc, t = m.hip.Generate(prompt, 16, useGraph=True)
     assert rc == 0, E.last_error()
-    assert _in_use(m.hip), "8 small layers: automatic mode should use the persistent launch"
+    assert _in_use(m.hip)
     assert t.tolist() == ref.tolist()
     rc, tr = m.hip.FlowTrace(True, read=False)
     assert rc == 0, E.last_error()
