@@ -259,19 +259,21 @@ __device__ __forceinline__ void dot_rows_tail(const signed char* const (&rows)[N
     }
 }
 
+constexpr int FLOW_MAX_ROUNDS = 8;   // rows of a matrix a wave takes at most (rounds of all waves over the matrix)
 constexpr int CBF = 6;       // ... per row of K = ffnDim (rows up to 6144 weights in one batch)
 constexpr int NIB = 24 / FWAVES;   // gate/up items (a gate row and its up row) a wave holds in flight
 constexpr int NID = 8 / FWAVES;    // down rows a wave holds in flight
 
 // CBD: chunks a lane prefetches per row of K = dim (1: rows of up to 1024 weights in one batch, 2: up to 2048)
-template <int HD, int CBD>
+// RING: gate | up and down stream their rows through a ring of register sets (rows of more than 2048 weights)
+template <int HD, int CBD, bool RING>
 __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     extern __shared__ float4 a4[];                     // the staged activation vector, max(dim, ffn) floats
     __shared__ float red[FWAVES];
     __shared__ float4 sqkv[3][HD / 4];                 // q of the head, K and V row of the current position
     __shared__ float4 accbuf[FWAVES][HD / 4];
     __shared__ float lbuf[FWAVES], wred[FWAVES];
-    __shared__ float outbuf[NIB][FWAVES];                // a phase's results of the workgroup, stored by one wave as whole 32-byte runs
+    __shared__ float outbuf[FLOW_MAX_ROUNDS][FWAVES];                // a phase's results of the workgroup, stored by one wave as whole 32-byte runs
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -561,6 +563,54 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
         // ------------------------------------------------------------------ gate | up, SiLU(g) * u
         {
             const int nI = ffn;
+            if constexpr (RING) {
+                // Long rows, several items a wave: the rows stream through a ring of register sets, the loads of step
+                // s + RD - 1 are issued before step s is multiplied (a step = one item's two rows x CB chunks a lane).
+                if (blockIdx.x * FWAVES < nI) {
+                    constexpr int RD = 4, CB = 2;
+                    int4 ring[RD][2][CB];
+                    const int nItems = gw < nI ? (nI - gw + W - 1) / W : 0;
+                    const int nb = (nchD + 64 * CB - 1) / (64 * CB);
+                    const int T = nItems * nb;
+                    auto issueStep = [&](int4 (&set)[2][CB], int st) {
+                        const int sc = min(st, T - 1);                       // past the end: the last step again (uniform loop)
+                        const int k = sc / nb, b = sc - k * nb;
+                        const size_t row = (size_t)(gw + k * W) * dim;
+                        ld_row<CB>(L.gate + row, nchD, lane, b * CB * 64, set[0]);
+                        ld_row<CB>(L.up + row, nchD, lane, b * CB * 64, set[1]);
+                    };
+                    float sg = 0.f, su = 0.f;
+                    if (T > 0) {
+#pragma unroll
+                        for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
+                        if (lane < nItems) { const int r = gw + lane * W; sg = L.sgate[r]; su = L.sup[r]; }
+                    }
+                    const float rs = stage_rms(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                    FLOW_TRACE(7);
+                    float acc[2] = {0.f, 0.f};
+                    float g = 0.f, u = 0.f;
+                    for (int s0 = 0; s0 < T; s0 += RD) {
+#pragma unroll
+                        for (int j = 0; j < RD; j++) {
+                            const int st = s0 + j;
+                            issueStep(ring[(j + RD - 1) % RD], st + RD - 1);
+                            if (st < T) {                                        // uniform in the wave
+                                const int k = st / nb, b = st - k * nb;
+                                dot_rows<2, CB>(ring[j], a4, nchD, lane, b * CB * 64, acc);
+                                if (b == nb - 1) {
+                                    const float v0 = wave_sum(acc[0]), v1 = wave_sum(acc[1]);
+                                    if (lane == k) { g = v0; u = v1; }
+                                    acc[0] = 0.f; acc[1] = 0.f;
+                                }
+                            }
+                        }
+                    }
+                    g = g * sg; g = g * rs;
+                    u = u * su; u = u * rs;
+                    const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f));   // mongoose.cu:949-956
+                    store_runs(g * sig * u, (nI + W - 1) / W, nI, 0, X + G.offM, nullptr);
+                }
+            } else
             if (blockIdx.x * FWAVES < nI) {
                 int4 wr[NIB][2][CBD];
                 float sg = 0.f, su = 0.f;
@@ -609,6 +659,47 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
         // ------------------------------------------------------------------ down + residual
         {
             const int nI = dim;
+            if constexpr (RING) {
+                if (blockIdx.x * FWAVES < nI) {
+                    constexpr int RD = 3, CB = 4;
+                    int4 ring[RD][1][CB];
+                    const int nItems = gw < nI ? (nI - gw + W - 1) / W : 0;
+                    const int nb = (nchF + 64 * CB - 1) / (64 * CB);
+                    const int T = nItems * nb;
+                    auto issueStep = [&](int4 (&set)[1][CB], int st) {
+                        const int sc = min(st, T - 1);
+                        const int k = sc / nb, b = sc - k * nb;
+                        ld_row<CB>(L.down + (size_t)(gw + k * W) * ffn, nchF, lane, b * CB * 64, set[0]);
+                    };
+                    float e0 = 0.f, e1 = 0.f;
+                    if (T > 0) {
+                        if (lane < nItems) { const int r = gw + lane * W; e0 = L.sdown[r]; e1 = poll1(X + G.offX1 + r, wt); }
+#pragma unroll
+                        for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
+                    }
+                    stage_plain(X + G.offM, ffn, a4, wt);
+                    FLOW_TRACE(9);
+                    float acc[1] = {0.f};
+                    float v = 0.f;
+                    for (int s0 = 0; s0 < T; s0 += RD) {
+#pragma unroll
+                        for (int j = 0; j < RD; j++) {
+                            const int st = s0 + j;
+                            issueStep(ring[(j + RD - 1) % RD], st + RD - 1);
+                            if (st < T) {                                        // uniform in the wave
+                                const int k = st / nb, b = st - k * nb;
+                                dot_rows<1, CB>(ring[j], a4, nchF, lane, b * CB * 64, acc);
+                                if (b == nb - 1) {
+                                    const float v0 = wave_sum(acc[0]);
+                                    if (lane == k) v = v0;
+                                    acc[0] = 0.f;
+                                }
+                            }
+                        }
+                    }
+                    store_runs(e1 + v * e0, (nI + W - 1) / W, nI, 0, X + G.offX2, l == p.l1 - 1 ? p.hidden : nullptr);
+                }
+            } else
             if (blockIdx.x * FWAVES < nI) {
                 int4 wr[NID][1][CBF];
                 float e0 = 0.f, e1 = 0.f;
@@ -684,16 +775,19 @@ bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads,
 hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
     if (!flow_shape_supported(p.dim, p.kvDim, p.ffn, p.nHeads, p.nKVHeads, p.headDim)) return hipErrorInvalidValue;
     if (p.l0 < 0 || p.l1 <= p.l0 || p.l1 > p.nLayersTotal || grid < flow_min_grid(p.nHeads, p.geo) ||
-        !flow_context_fits(p.maxSeq, p.geo) || !p.layers || !p.xchg || !p.err || !p.hidden)
+        !flow_context_fits(p.maxSeq, p.geo) || !p.layers || !p.xchg || !p.err || !p.hidden ||
+        (p.ffn + grid * FWAVES - 1) / (grid * FWAVES) > FLOW_MAX_ROUNDS)
         return hipErrorInvalidValue;
     const size_t lds = (size_t)(p.dim > p.ffn ? p.dim : p.ffn) * sizeof(float);
-    const bool wide = p.dim > 1024;
+    const bool wide = p.dim > 1024, ring = p.dim > 2048;
     if (p.headDim == 64) {
-        if (wide) hipLaunchKernelGGL((flow_layers_kernel<64, 2>), dim3(grid), dim3(FWG), lds, s, p);
-        else hipLaunchKernelGGL((flow_layers_kernel<64, 1>), dim3(grid), dim3(FWG), lds, s, p);
+        if (ring) hipLaunchKernelGGL((flow_layers_kernel<64, 2, true>), dim3(grid), dim3(FWG), lds, s, p);
+        else if (wide) hipLaunchKernelGGL((flow_layers_kernel<64, 2, false>), dim3(grid), dim3(FWG), lds, s, p);
+        else hipLaunchKernelGGL((flow_layers_kernel<64, 1, false>), dim3(grid), dim3(FWG), lds, s, p);
     } else {
-        if (wide) hipLaunchKernelGGL((flow_layers_kernel<128, 2>), dim3(grid), dim3(FWG), lds, s, p);
-        else hipLaunchKernelGGL((flow_layers_kernel<128, 1>), dim3(grid), dim3(FWG), lds, s, p);
+        if (ring) hipLaunchKernelGGL((flow_layers_kernel<128, 2, true>), dim3(grid), dim3(FWG), lds, s, p);
+        else if (wide) hipLaunchKernelGGL((flow_layers_kernel<128, 2, false>), dim3(grid), dim3(FWG), lds, s, p);
+        else hipLaunchKernelGGL((flow_layers_kernel<128, 1, false>), dim3(grid), dim3(FWG), lds, s, p);
     }
     return hipGetLastError();
 }
