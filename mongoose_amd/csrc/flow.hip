@@ -327,66 +327,79 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
         {
             const int nq = dim >> 1, nk = kvDim >> 1, nI = nq + 2 * nk;       // RoPE pairs of q, of k; row pairs of v
             if (blockIdx.x * FWAVES < nI) {
-                int it = gw;
-                int4 wr[2][CBD];
-                const signed char* rows[2] = {L.wq, L.wq};
-                int kind = 0, r0 = 0, r1 = 0;
-                float e0 = 0.f, e1 = 0.f;                // per-lane epilogue operands: lanes 0/1 scale and bias, lane 2 cos and sin
-                auto resolve = [&](int item) {
+                // The first NPI items of a wave are requested whole (CBQ chunks a lane and row) before the input is waited for;
+                // further items, and chunks past CBQ, are read where they are used.
+                constexpr int NPI = 1, CBQ = CBD;
+                int4 wr[NPI][2][CBQ];
+                const signed char* rows[NPI][2];
+                int kind[NPI], r0[NPI], r1[NPI];
+                float e0[NPI], e1[NPI];                  // per-lane epilogue operands: lanes 0/1 scale and bias, lane 2 cos and sin
+                auto resolve = [&](int4 (&w)[2][CBQ], const signed char* (&rw)[2], int& kd, int& a0, int& a1, float& f0, float& f1, int item) {
                     const signed char* Wm; const float* sc; const float* bias;
-                    if (item < nq) { kind = 0; Wm = L.wq; sc = L.sq; bias = L.bq; const int j = item % half; r0 = (item - j) * 2 + j; r1 = r0 + half; }
-                    else if (item < nq + nk) { kind = 1; Wm = L.wk; sc = L.sk; bias = L.bk; const int i2 = item - nq; const int j = i2 % half; r0 = (i2 - j) * 2 + j; r1 = r0 + half; }
-                    else { kind = 2; Wm = L.wv; sc = L.sv; bias = L.bv; r0 = (item - nq - nk) * 2; r1 = r0 + 1; }
-                    rows[0] = Wm + (size_t)r0 * dim; rows[1] = Wm + (size_t)r1 * dim;
-                    ld_row<CBD>(rows[0], nchD, lane, 0, wr[0]);
-                    ld_row<CBD>(rows[1], nchD, lane, 0, wr[1]);
-                    e0 = 1.f; e1 = 0.f;
+                    if (item < nq) { kd = 0; Wm = L.wq; sc = L.sq; bias = L.bq; const int jj = item % half; a0 = (item - jj) * 2 + jj; a1 = a0 + half; }
+                    else if (item < nq + nk) { kd = 1; Wm = L.wk; sc = L.sk; bias = L.bk; const int i2 = item - nq; const int jj = i2 % half; a0 = (i2 - jj) * 2 + jj; a1 = a0 + half; }
+                    else { kd = 2; Wm = L.wv; sc = L.sv; bias = L.bv; a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
+                    rw[0] = Wm + (size_t)a0 * dim; rw[1] = Wm + (size_t)a1 * dim;
+                    ld_row<CBQ>(rw[0], nchD, lane, 0, w[0]);
+                    ld_row<CBQ>(rw[1], nchD, lane, 0, w[1]);
+                    f0 = 1.f; f1 = 0.f;
                     if (lane < 2) {
-                        const int r = lane ? r1 : r0;
-                        e0 = sc[r];
-                        if (bias) e1 = bias[r];
+                        const int r = lane ? a1 : a0;
+                        f0 = sc[r];
+                        if (bias) f1 = bias[r];
                     }
-                    if (lane == 2 && kind < 2) { const int j = r0 % half; e0 = p.cosRow[j]; e1 = p.sinRow[j]; }
+                    if (lane == 2 && kd < 2) { const int jj = a0 % half; f0 = p.cosRow[jj]; f1 = p.sinRow[jj]; }
                 };
-                if (it < nI) resolve(it);
-                const float rs = stage_rms(xin, !first, L.g1, dim, p.eps, a4, red, wt);
-                FLOW_TRACE(1);
-                for (; it < nI; it += W) {
-                    if (it != gw) resolve(it);
+                // one item of every wave of the workgroup: dot, epilogue, the results out as runs by wave 0
+                auto finish = [&](const int4 (&w)[2][CBQ], const signed char* const (&rw)[2], int kd, float f0, float f1, float rs, int it) {
                     float acc[2] = {0.f, 0.f};
-                    dot_rows<2, CBD>(wr, a4, nchD, lane, 0, acc);
-                    if (nchD > CBD * 64) dot_rows_tail<2, CBD>(rows, a4, nchD, lane, acc);
+                    dot_rows<2, CBQ>(w, a4, nchD, lane, 0, acc);
+                    if (nchD > CBQ * 64) dot_rows_tail<2, CBQ>(rw, a4, nchD, lane, acc);
                     acc[0] = wave_sum(acc[0]);
                     acc[1] = wave_sum(acc[1]);
                     float v = lane == 1 ? acc[1] : acc[0];
-                    v = v * e0;                                                  // row scale (lanes 0 and 1)
+                    v = v * f0;                                                  // row scale (lanes 0 and 1)
                     v = v * rs;
-                    v = v + e1;
+                    v = v + f1;
                     const float v1 = dpp_f<0x101>(v);                            // lane 0 reads lane 1: the pair's second row
-                    const float cs = dpp_f<0x102>(e0), sn = dpp_f<0x102>(e1);    // lane 0 reads lane 2
+                    const float cs = dpp_f<0x102>(f0), sn = dpp_f<0x102>(f1);    // lane 0 reads lane 2
                     float o0 = v, o1 = v1;
-                    if (kind < 2) { o0 = v * cs - v1 * sn; o1 = v * sn + v1 * cs; }          // mongoose.cu:991-1006
-                    // the eight waves' rows are consecutive (first rows of the pairs, and second rows): out as runs by wave 0
+                    if (kd < 2) { o0 = v * cs - v1 * sn; o1 = v * sn + v1 * cs; }            // mongoose.cu:991-1006
+                    // the eight waves' rows are consecutive (first rows of the pairs, and second rows)
                     if (it != gw) __syncthreads();              // outbuf is free again
                     if (lane == 0) { outbuf[0][wave] = o0; outbuf[1][wave] = o1; }
                     __syncthreads();
                     if (wave == 0 && lane < 2 * FWAVES) {
                         const int k = lane / FWAVES, wv = lane % FWAVES, item = it + wv;
                         if (item < nI) {
-                            int kd, a0, a1;
-                            if (item < nq) { kd = 0; const int j = item % half; a0 = (item - j) * 2 + j; a1 = a0 + half; }
-                            else if (item < nq + nk) { kd = 1; const int i2 = item - nq; const int j = i2 % half; a0 = (i2 - j) * 2 + j; a1 = a0 + half; }
-                            else { kd = 2; a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
+                            int kk, a0, a1;
+                            if (item < nq) { kk = 0; const int jj = item % half; a0 = (item - jj) * 2 + jj; a1 = a0 + half; }
+                            else if (item < nq + nk) { kk = 1; const int i2 = item - nq; const int jj = i2 % half; a0 = (i2 - jj) * 2 + jj; a1 = a0 + half; }
+                            else { kk = 2; a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
                             const int r = k ? a1 : a0;
                             const float o = outbuf[k][wv];
-                            if (kd == 0) {
+                            if (kk == 0) {
                                 stx(X + G.offQ + r, o);
                             } else {                                              // mongoose.cu:1644-1647, and the hand-over copy
-                                ((kd == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim)[r] = o;
-                                stx(X + (kd == 1 ? G.offKc : G.offVc) + r, o);
+                                ((kk == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim)[r] = o;
+                                stx(X + (kk == 1 ? G.offKc : G.offVc) + r, o);
                             }
                         }
                     }
+                };
+#pragma unroll
+                for (int q = 0; q < NPI; q++) {
+                    kind[q] = 0; r0[q] = 0; r1[q] = 0; e0[q] = 0.f; e1[q] = 0.f; rows[q][0] = L.wq; rows[q][1] = L.wq;
+                    if (gw + q * W < nI) resolve(wr[q], rows[q], kind[q], r0[q], r1[q], e0[q], e1[q], gw + q * W);
+                }
+                const float rs = stage_rms(xin, !first, L.g1, dim, p.eps, a4, red, wt);
+                FLOW_TRACE(1);
+#pragma unroll
+                for (int q = 0; q < NPI; q++)
+                    if (blockIdx.x * FWAVES + q * W < nI) finish(wr[q], rows[q], kind[q], e0[q], e1[q], rs, gw + q * W);      // uniform in the workgroup
+                for (int it = gw + NPI * W; it - wave < nI; it += W) {         // it - wave: the same for all waves of the workgroup
+                    if (it < nI) resolve(wr[0], rows[0], kind[0], r0[0], r1[0], e0[0], e1[0], it);
+                    finish(wr[0], rows[0], kind[0], e0[0], e1[0], rs, it);
                 }
             }
         }
