@@ -27,13 +27,15 @@ struct FlowLayer {
 // the K and V rows of the current position, the attention partials of up to smax KV splits (accumulator,
 // maximum, sum), the hidden state after the attention block, the SwiGLU vector and the layer's output.
 // Every float is the pattern 0xFFFFFFFF until its producer has written it.
+constexpr int FLOW_GQA_MAX = 8;        // query heads a KV head may have for the grouped attention
 constexpr int FLOW_TILE = 128;         // positions of an attention tile: one workgroup per (query head, tile)
 struct FlowGeometry {
     int stride;
-    int offQ, offKc, offVc, offPacc, offPm, offPl, offX1, offM, offX2;
+    int offQ, offKc, offVc, offPacc, offPm, offPl, offX1, offM, offX2, offAttn;
     int smax;
+    int gqa;         // 1: an attention workgroup per (KV head, split) taking all its query heads; 0: per (query head, split)
 };
-FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int headDim, int maxSeq, int grid);
+FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int nKVHeads, int headDim, int maxSeq, int grid);
 bool flow_context_fits(int maxSeq, const FlowGeometry& g);
 
 // Trace slots of a layer, in program order: when thread 0 of a workgroup passed the point.
@@ -60,7 +62,7 @@ struct FlowParams {
 };
 
 // Workgroups the launch needs at least (one per query head and KV split) for this shape.
-int flow_min_grid(int nHeads, const FlowGeometry& g);
+int flow_min_grid(int nHeads, int nKVHeads, const FlowGeometry& g);
 bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads, int headDim);
 // grid workgroups of 512 threads, all of which must be resident at once (grid <= CUs x resident workgroups per CU).
 hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s);

@@ -266,11 +266,13 @@ constexpr int NID = 8 / FWAVES;    // down rows a wave holds in flight
 
 // CBD: chunks a lane prefetches per row of K = dim (1: rows of up to 1024 weights in one batch, 2: up to 2048)
 // RING: gate | up and down stream their rows through a ring of register sets (rows of more than 2048 weights)
-template <int HD, int CBD, bool RING>
+// GQA: an attention workgroup takes all query heads of a KV head (contexts too long for one workgroup a query head)
+template <int HD, int CBD, bool RING, bool GQA>
 __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     extern __shared__ float4 a4[];                     // the staged activation vector, max(dim, ffn) floats
     __shared__ float red[FWAVES];
-    __shared__ float4 sqkv[3][HD / 4];                 // q of the head, K and V row of the current position
+    constexpr int QHMAX = GQA ? FLOW_GQA_MAX : 1;
+    __shared__ float4 sqkv[2 + QHMAX][HD / 4];         // K and V row of the current position, q of the workgroup's heads
     __shared__ float4 accbuf[FWAVES][HD / 4];
     __shared__ float lbuf[FWAVES], wred[FWAVES];
     __shared__ float outbuf[FLOW_MAX_ROUNDS][FWAVES];                // a phase's results of the workgroup, stored by one wave as whole 32-byte runs
@@ -314,6 +316,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     // timing trace (diagnostic): slot b of layer l, per workgroup, in ticks of the 100 MHz wall clock
 #define FLOW_TRACE(b) do { if (p.trace && tid == 0) \
         p.trace[((size_t)(l - p.l0) * FLOW_TRACE_SLOTS + (b)) * gridDim.x + blockIdx.x] = wall_clock64(); } while (0)
+    // the exchange area as a buffer resource: agent-scope loads that the compiler keeps track of (used where many are
+    // wanted in flight together)
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(p.xchg, 0, (int)((size_t)p.nLayersTotal * G.stride * 4), 0x00020000);
     unsigned lw = layer_words(p.layers, p.l0, lane);
     for (int l = p.l0; l < p.l1; l++) {
         const FlowLayer L = unpack_layer(lw);
@@ -408,9 +413,12 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
         // ------------------------------------------------------------------ attention: one (head, KV split) per workgroup
         {
             const int nsplit = pos / TILE + 1;
-            const int split = blockIdx.x / p.nHeads, h = blockIdx.x % p.nHeads;
+            const int QH = GQA ? p.nHeads / p.nKVHeads : 1;            // query heads of this workgroup
+            const int unit = GQA ? p.nKVHeads : p.nHeads;
+            const int split = blockIdx.x / unit, hu = blockIdx.x % unit;
             if (split < G.smax && split < nsplit) {
-                const int kvh = h / (p.nHeads / p.nKVHeads);
+                const int kvh = GQA ? hu : hu / (p.nHeads / p.nKVHeads);
+                const int h0 = GQA ? hu * QH : hu;
                 const int tg = tid / LPR, dl = tid % LPR;
                 const int t0 = split * TILE;
                 const int len = pos + 1;
@@ -430,18 +438,28 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     for (int j = 0; j < NF; j++) vreg[u][j] = Vc4[ro + j * 16];
                 }
                 __syncthreads();
-                if (tid < 3 * (HD / 4)) {
+                if (tid < (2 + QH) * (HD / 4)) {
                     const int which = tid / (HD / 4), i = tid % (HD / 4);
-                    const float* src = which == 0 ? X + G.offQ + h * HD : X + (which == 1 ? G.offKc : G.offVc) + kvh * HD;
+                    const float* src = which >= 2 ? X + G.offQ + (h0 + which - 2) * HD : X + (which == 0 ? G.offKc : G.offVc) + kvh * HD;
                     sqkv[which][i] = tof4(poll4(reinterpret_cast<const f4*>(src) + i, wt));
                 }
                 __syncthreads();
                 FLOW_TRACE(3);
-                float4 q4[NF];
-#pragma unroll
-                for (int j = 0; j < NF; j++) q4[j] = sqkv[0][j * 16 + dl];
                 const int live = t1 - t0;
                 const float scale = 1.0f / sqrtf((float)HD);
+#pragma unroll
+                for (int u = 0; u < VU; u++) {
+                    if (t0 + tg + u * TG == pos) {          // the current position's rows come from this launch, not from the cache
+#pragma unroll
+                        for (int j = 0; j < NF; j++) { kreg[u][j] = sqkv[0][j * 16 + dl]; vreg[u][j] = sqkv[1][j * 16 + dl]; }
+                    }
+                }
+                for (int hi = 0; hi < QH; hi++) {          // the heads of the KV head in turn, on the same K / V registers
+                const int h = h0 + hi;
+                if (hi) __syncthreads();                    // accbuf, lbuf, wred are free again
+                float4 q4[NF];
+#pragma unroll
+                for (int j = 0; j < NF; j++) q4[j] = sqkv[2 + (GQA ? hi : 0)][j * 16 + dl];
                 float sc[VU];
                 float tmax = -INFINITY;
 #pragma unroll
@@ -449,10 +467,6 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     sc[u] = -INFINITY;
                     if (u * TG >= live) continue;
                     const int row = t0 + tg + u * TG;
-                    if (row == pos) {                   // the current position's rows come from this launch, not from the cache
-#pragma unroll
-                        for (int j = 0; j < NF; j++) { kreg[u][j] = sqkv[1][j * 16 + dl]; vreg[u][j] = sqkv[2][j * 16 + dl]; }
-                    }
                     float d = 0.f;
 #pragma unroll
                     for (int j = 0; j < NF; j++) {
@@ -507,9 +521,75 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         stx(X + G.offPl + split * p.nHeads + h, lg);
                     }
                 }
+                }
             }
         }
 
+        if constexpr (GQA) {
+            // Long contexts, tens of KV splits: merged once per head, by workgroup h for head h (every thread a 16-byte piece
+            // and every eighth split, eight splits' loads in flight together, then combined through LDS), and handed on as
+            // one vector -- every consumer merging all partials itself re-reads tens of KB per workgroup and layer.
+            if ((int)blockIdx.x < p.nHeads) {
+                constexpr int P4 = HD / 4, SG = FWG / P4;          // pieces of a head, split groups (thread = piece x group)
+                __shared__ float4 mnum[SG][P4];
+                __shared__ float mM[SG][P4], mden[SG][P4];
+                const int h = blockIdx.x, i = tid % P4, sg = tid / P4;
+                const int ns = min(pos / TILE + 1, G.smax);
+                const unsigned Xo = (unsigned)l * G.stride;
+                float M = -INFINITY, den = 0.f;
+                f4 num = {0.f, 0.f, 0.f, 0.f};
+                constexpr int MBG = 4;
+                for (int s1 = sg; s1 < ns; s1 += SG * MBG) {
+                    f4 a[MBG];
+                    float ms[MBG], ls[MBG];
+                    long long t0w = 0;
+                    bool timing = false;
+                    for (;;) {
+                        bool ok = true;
+#pragma unroll
+                        for (int j = 0; j < MBG; j++) {
+                            const int sj = min(s1 + j * SG, ns - 1);
+                            a[j] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (Xo + G.offPacc + (unsigned)sj * dim + h * HD + i * 4) * 4u, 0, 16));
+                            ms[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, (Xo + G.offPm + sj * p.nHeads + h) * 4u, 0, 16));
+                            ls[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, (Xo + G.offPl + sj * p.nHeads + h) * 4u, 0, 16));
+                        }
+#pragma unroll
+                        for (int j = 0; j < MBG; j++) ok = ok && ready4(a[j]) && !unset(ms[j]) && !unset(ls[j]);
+                        if (ok || wt.dead) break;
+                        if (!timing) { timing = true; t0w = wall_clock64(); }
+                        else if (wall_clock64() - t0w > wt.limit) { wt.fail(); break; }
+                        for (int z = 0; z < 4; z++) __builtin_amdgcn_s_sleep(2);
+                    }
+#pragma unroll
+                    for (int j = 0; j < MBG; j++) {
+                        if (s1 + j * SG < ns) {
+                            const float Mn = fmaxf(M, ms[j]);
+                            const float c = exp_neg(M - Mn), wgt = exp_neg(ms[j] - Mn);
+                            den = den * c + wgt * ls[j];
+                            num.x = num.x * c + wgt * a[j].x; num.y = num.y * c + wgt * a[j].y;
+                            num.z = num.z * c + wgt * a[j].z; num.w = num.w * c + wgt * a[j].w;
+                            M = Mn;
+                        }
+                    }
+                }
+                mnum[sg][i] = tof4(num); mM[sg][i] = M; mden[sg][i] = den;
+                __syncthreads();
+                if (tid < P4) {
+                    float Mg = mM[0][tid];
+                    for (int g2 = 1; g2 < SG; g2++) Mg = fmaxf(Mg, mM[g2][tid]);
+                    float dn = 0.f;
+                    f4 nm = {0.f, 0.f, 0.f, 0.f};
+                    for (int g2 = 0; g2 < SG; g2++) {
+                        const float wgt = exp_neg(mM[g2][tid] - Mg);     // a group without splits has M = -inf: weight 0
+                        const float4 a = mnum[g2][tid];
+                        dn = fmaf(wgt, mden[g2][tid], dn);
+                        nm.x = fmaf(wgt, a.x, nm.x); nm.y = fmaf(wgt, a.y, nm.y); nm.z = fmaf(wgt, a.z, nm.z); nm.w = fmaf(wgt, a.w, nm.w);
+                    }
+                    const float il = __builtin_amdgcn_rcpf(dn);
+                    stx4(reinterpret_cast<f4*>(X + G.offAttn + h * HD) + tid, f4{nm.x * il, nm.y * il, nm.z * il, nm.w * il});
+                }
+            }
+        }
         FLOW_TRACE(4);
         // ------------------------------------------------------------------ Wo + residual
         {
@@ -529,6 +609,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 };
                 if (it < nI) resolve(it);
                 // stage the attention output: merge the KV splits' partials (running maximum, as the split-KV combine)
+                if constexpr (GQA) {
+                    stage_plain(X + G.offAttn, dim, a4, wt);      // merged per head above
+                } else {
                 __syncthreads();
                 {
                     const int nsplit = pos / TILE + 1;
@@ -537,6 +620,15 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         const int h = (i * 4) / HD;
                         float M = -INFINITY, den = 0.f;
                         f4 num = {0.f, 0.f, 0.f, 0.f};
+                        auto mergeIn = [&](f4 a, float ms, float ls) {
+                            const float Mn = fmaxf(M, ms);
+                            const float c = exp_neg(M - Mn);                        // first split: exp(-inf) = 0
+                            const float wgt = exp_neg(ms - Mn);
+                            den = den * c + wgt * ls;
+                            num.x = num.x * c + wgt * a.x; num.y = num.y * c + wgt * a.y;
+                            num.z = num.z * c + wgt * a.z; num.w = num.w * c + wgt * a.w;
+                            M = Mn;
+                        };
                         for (int s = 0; s < ns; s++) {
                             f4 a;
                             float ms, ls;
@@ -546,19 +638,14 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             // 50,000 threads keep re-reading takes its producer's store late.
                             if (s == 0) a = poll4(pa, wt);
                             poll_partial(pa, X + G.offPm + s * p.nHeads + h, X + G.offPl + s * p.nHeads + h, a, ms, ls, wt);
-                            const float Mn = fmaxf(M, ms);
-                            const float c = exp_neg(M - Mn);                    // first split: exp(-inf) = 0
-                            const float wgt = exp_neg(ms - Mn);
-                            den = den * c + wgt * ls;
-                            num.x = num.x * c + wgt * a.x; num.y = num.y * c + wgt * a.y;
-                            num.z = num.z * c + wgt * a.z; num.w = num.w * c + wgt * a.w;
-                            M = Mn;
+                            mergeIn(a, ms, ls);
                         }
                         const float il = __builtin_amdgcn_rcpf(den);
                         a4[slot4(i, nchD)] = make_float4(num.x * il, num.y * il, num.z * il, num.w * il);
                     }
                 }
                 __syncthreads();
+                }
                 FLOW_TRACE(5);
                 for (; it < nI; it += W) {
                     if (it != gw) resolve(it);
@@ -752,11 +839,16 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     }
 }
 
-FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int headDim, int maxSeq, int grid) {
+FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int nKVHeads, int headDim, int maxSeq, int grid) {
     FlowGeometry g{};
-    // partial slots: one per FLOW_TILE positions, at most as many as the workgroups of the launch can serve
-    g.smax = (maxSeq + FLOW_TILE - 1) / FLOW_TILE;
-    if (nHeads > 0 && g.smax > grid / nHeads) g.smax = grid / nHeads;
+    // partial slots: one per FLOW_TILE positions, at most as many as the workgroups of the launch can serve.  One
+    // workgroup a query head where that covers the context (the shorter phase), else one a KV head, taking all its
+    // query heads in turn on one load of the K / V rows.
+    const int want = (maxSeq + FLOW_TILE - 1) / FLOW_TILE;
+    g.gqa = (nHeads > 0 && want > grid / nHeads && nKVHeads > 0 && nHeads / nKVHeads > 1 && nHeads / nKVHeads <= FLOW_GQA_MAX) ? 1 : 0;
+    const int unit = g.gqa ? nKVHeads : nHeads;
+    g.smax = want;
+    if (unit > 0 && g.smax > grid / unit) g.smax = grid / unit;
     if (g.smax < 1) g.smax = 1;
     auto up64 = [](int v) { return (v + 63) & ~63; };
     int o = 0;
@@ -769,11 +861,12 @@ FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int headDim,
     g.offX1 = o; o += up64(dim);
     g.offM = o; o += up64(ffn);
     g.offX2 = o; o += up64(dim);
+    g.offAttn = o; o += up64(dim);          // attention output merged over the splits (grouped attention only)
     g.stride = o;
     return g;
 }
 
-int flow_min_grid(int nHeads, const FlowGeometry& g) { return nHeads * g.smax; }
+int flow_min_grid(int nHeads, int nKVHeads, const FlowGeometry& g) { return (g.gqa ? nKVHeads : nHeads) * g.smax; }
 // one workgroup per (query head, tile): the slots cover the context
 bool flow_context_fits(int maxSeq, const FlowGeometry& g) { return (long long)FLOW_TILE * g.smax >= maxSeq; }
 
@@ -787,21 +880,25 @@ bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads,
 
 hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
     if (!flow_shape_supported(p.dim, p.kvDim, p.ffn, p.nHeads, p.nKVHeads, p.headDim)) return hipErrorInvalidValue;
-    if (p.l0 < 0 || p.l1 <= p.l0 || p.l1 > p.nLayersTotal || grid < flow_min_grid(p.nHeads, p.geo) ||
+    if (p.l0 < 0 || p.l1 <= p.l0 || p.l1 > p.nLayersTotal || grid < flow_min_grid(p.nHeads, p.nKVHeads, p.geo) ||
         !flow_context_fits(p.maxSeq, p.geo) || !p.layers || !p.xchg || !p.err || !p.hidden ||
-        (p.ffn + grid * FWAVES - 1) / (grid * FWAVES) > FLOW_MAX_ROUNDS)
+        (p.ffn + grid * FWAVES - 1) / (grid * FWAVES) > FLOW_MAX_ROUNDS || (size_t)p.nLayersTotal * p.geo.stride * 4 >= (1ull << 31))
         return hipErrorInvalidValue;
     const size_t lds = (size_t)(p.dim > p.ffn ? p.dim : p.ffn) * sizeof(float);
-    const bool wide = p.dim > 1024, ring = p.dim > 2048;
+    const bool wide = p.dim > 1024, ring = p.dim > 2048, gqa = p.geo.gqa != 0;
+#define FLOW_LAUNCH(HDv, CBv, RGv, GQv) hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv>), dim3(grid), dim3(FWG), lds, s, p)
+#define FLOW_LAUNCH_G(HDv, CBv, RGv) do { if (gqa) FLOW_LAUNCH(HDv, CBv, RGv, true); else FLOW_LAUNCH(HDv, CBv, RGv, false); } while (0)
     if (p.headDim == 64) {
-        if (ring) hipLaunchKernelGGL((flow_layers_kernel<64, 2, true>), dim3(grid), dim3(FWG), lds, s, p);
-        else if (wide) hipLaunchKernelGGL((flow_layers_kernel<64, 2, false>), dim3(grid), dim3(FWG), lds, s, p);
-        else hipLaunchKernelGGL((flow_layers_kernel<64, 1, false>), dim3(grid), dim3(FWG), lds, s, p);
+        if (ring) FLOW_LAUNCH_G(64, 2, true);
+        else if (wide) FLOW_LAUNCH_G(64, 2, false);
+        else FLOW_LAUNCH_G(64, 1, false);
     } else {
-        if (ring) hipLaunchKernelGGL((flow_layers_kernel<128, 2, true>), dim3(grid), dim3(FWG), lds, s, p);
-        else if (wide) hipLaunchKernelGGL((flow_layers_kernel<128, 2, false>), dim3(grid), dim3(FWG), lds, s, p);
-        else hipLaunchKernelGGL((flow_layers_kernel<128, 1, false>), dim3(grid), dim3(FWG), lds, s, p);
+        if (ring) FLOW_LAUNCH_G(128, 2, true);
+        else if (wide) FLOW_LAUNCH_G(128, 2, false);
+        else FLOW_LAUNCH_G(128, 1, false);
     }
+#undef FLOW_LAUNCH_G
+#undef FLOW_LAUNCH
     return hipGetLastError();
 }
 

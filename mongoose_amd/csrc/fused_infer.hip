@@ -655,8 +655,8 @@ bool HIPFusedInference::flowEligible(int l0, int l1) const {
         if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) { (void)hipGetLastError(); return false; }
         cus = prop.multiProcessorCount;
     }
-    const FlowGeometry g = flow_geometry(dim, kvDim, ffnDim, nHeads, headDim, maxSeq, cus);
-    return flow_min_grid(nHeads, g) <= cus && flow_context_fits(maxSeq, g);
+    const FlowGeometry g = flow_geometry(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim, maxSeq, cus);
+    return flow_min_grid(nHeads, nKVHeads, g) <= cus && flow_context_fits(maxSeq, g);
 }
 
 int HIPFusedInference::ensureFlow() {
@@ -666,7 +666,7 @@ int HIPFusedInference::ensureFlow() {
         HIPCHK(hipGetDevice(&dev));
         HIPCHK(hipGetDeviceProperties(&prop, dev));
         flowGrid = prop.multiProcessorCount;
-        flowGeo = flow_geometry(dim, kvDim, ffnDim, nHeads, headDim, maxSeq, flowGrid);
+        flowGeo = flow_geometry(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim, maxSeq, flowGrid);
         void* v = nullptr;
         HIPCHK(hipMalloc(&v, sizeof(FlowLayer) * (size_t)nLayers));
         dFlowLayers = static_cast<FlowLayer*>(v);

@@ -132,8 +132,7 @@ def _modes_agree(m, prompt, nDecode, what):
 
 def test_kv_splits_heads_of_64(hip):
     """0.5B geometry (14 query heads on 2 KV heads, biases), 2 layers.  18 partial slots per head (256 CUs / 14 heads),
-    i.e. contexts of up to 2304 positions: positions 600..640 use 5-6 splits of 128 positions, 2260..2300 all 18.
-    A longer context does not fit the launch: the context then runs the fused launches."""
+    i.e. contexts of up to 2304 positions: positions 600..640 use 5-6 splits of 128 positions, 2260..2300 all 18."""
     s = H.with_layers(configs.QWEN, 2)._replace(name="qwen-geom", vocab=2048)
     m = H.Model(s, seed=11, maxSeq=2304, eng=hip, oracle=False)
     print("flow: qwen geometry, positions 600..640", flush=True)
@@ -141,7 +140,15 @@ def test_kv_splits_heads_of_64(hip):
     print("flow: qwen geometry, positions 2260..2300 (18 splits)", flush=True)
     _modes_agree(m, m.prompt(2260), 40, "18 splits")
     m.close()
-    m = H.Model(s, seed=11, maxSeq=2305, eng=hip, oracle=False)
+    # a longer context: one attention workgroup per (KV head, split) that takes the 7 query heads of its KV head in turn
+    m = H.Model(s, seed=11, maxSeq=6000, eng=hip, oracle=False)
+    print("flow: qwen geometry, grouped attention, positions 100..130, 2990..3020 and 5950..5990", flush=True)
+    _modes_agree(m, m.prompt(100), 30, "grouped, 1 split")
+    _modes_agree(m, m.prompt(2990), 30, "grouped, 24 splits")
+    _modes_agree(m, m.prompt(5950), 40, "grouped, 47 splits")
+    m.close()
+    # 2 KV heads x 128 positions x 128 workgroup rows = 16384 positions at most
+    m = H.Model(s, seed=11, maxSeq=16385, eng=hip, oracle=False)
     assert m.hip.SetExecMode(3) == 0
     assert not _in_use(m.hip)
     m.close()
@@ -162,6 +169,11 @@ def test_heads_of_128_grouped_kv(hip):
     assert t.tolist() == ref.tolist()
     print("flow: llama-3 geometry, positions 300..330 (3 splits)", flush=True)
     _modes_agree(m, m.prompt(300), 30, "heads of 128")
+    m.close()
+    # past 8 x 128 positions: grouped attention (4 query heads a KV head), up to 32 splits
+    m = H.Model(s, seed=12, maxSeq=4096, eng=hip, oracle=False)
+    print("flow: llama-3 geometry, grouped attention, positions 4040..4090", flush=True)
+    _modes_agree(m, m.prompt(4040), 50, "heads of 128, grouped")
     m.close()
 
 
