@@ -243,10 +243,11 @@ int mg_hidden_idx(mg_ctx* ctx);
  * also fetch the following matrices into L2 with its idle workgroups (for a GPU
  * shared with other work); 3 = all layers of a step in ONE persistent launch whose
  * workgroups hand their vectors over through device memory, wherever the model allows it
- * (Q8 weights, fp32 KV rows, heads of 64 or 128, a context of at most 128 x floor(CUs / nHeads)
- * positions: one workgroup per query head and 128 positions; otherwise as mode 1).
- * A new context is in mode 3 (measured against mode 1: 0.5B shape 27 % faster, 1.1B shape 30 %,
- * 8B shape 3-4 %, a 4-layer toy 18 %).
+ * (Q8 weights, fp32 KV rows, heads of 64 or 128, a context of at most 128 x floor(CUs / nKVHeads)
+ * positions -- an attention workgroup per query head and 128 positions where that covers the context,
+ * else per KV head -- with at most 8 query heads a KV head; otherwise as mode 1).
+ * A new context is in mode 3 (measured against mode 1: 0.5B shape 37 % more tokens per second, 1.1B
+ * shape 42 %, 8B shape 12 %, also at contexts of thousands of positions).
  * The persistent launch needs all its workgroups resident at once: on a GPU shared with
  * other kernels its waits can run into their time limit; the call then returns MG_E_HIP,
  * and the context continues with the fused launches.  All modes give the same results to
