@@ -248,6 +248,9 @@ int mg_hidden_idx(mg_ctx* ctx);
  * else per KV head -- with at most 8 query heads a KV head; otherwise as mode 1).
  * A new context is in mode 3 (measured against mode 1: 0.5B shape 37 % more tokens per second, 1.1B
  * shape 42 %, 8B shape 12 %, also at contexts of thousands of positions).
+ * On every device one context at a time uses the persistent launch -- the first that needs it, until it is
+ * destroyed or set to another mode; other contexts run the fused launches meanwhile (two such launches at
+ * once could each hold part of the CUs and wait for workgroups that cannot start).
  * The persistent launch needs all its workgroups resident at once: on a GPU shared with
  * other kernels its waits can run into their time limit; the call then returns MG_E_HIP,
  * and the context continues with the fused launches.  All modes give the same results to

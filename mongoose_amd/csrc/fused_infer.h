@@ -94,7 +94,8 @@ public:
     // 0: one launch per reference op; 1: fused launches; 2: fused, attention launches without the L2 prefetch
     // helpers; 3: all layers of a step in one persistent launch where the model allows it (else as 1).
     int execMode = 3;
-    void SetExecMode(int mode) { if (mode != execMode) invalidateGraphs(); execMode = mode; }
+    void SetExecMode(int mode) { if (mode != execMode) invalidateGraphs(); execMode = mode; if (mode != 3) releaseFlow(); }
+    void releaseFlow();
 
     // shape
     int dim, kvDim, headDim, nHeads, nKVHeads, ffnDim, vocabSize, nLayers, maxSeq;
@@ -203,6 +204,7 @@ private:
     int* dHistory = nullptr;
     int* dPrompt = nullptr;
     int* hTokens = nullptr;         // pinned
+    bool graphsUseFlow = false;       // the whole-token graphs were captured with the persistent layer launch
     unsigned graphGeneration = 0;     // bumped by whatever makes captured graphs stale (weights, caches, modes)
     hipGraph_t graphFull = nullptr, graphPrompt = nullptr;
     hipGraphExec_t execFull = nullptr, execPrompt = nullptr;

@@ -1,6 +1,7 @@
 // fused_infer.hip -- HIPFusedInference and the mg_* C entry points over it.
 // Host code only (no kernels here); compiled with hipcc for the runtime API.
 #include "fused_infer.h"
+#include <mutex>
 #include "../../include/mongoose_hip.h"
 #include "host_util.h"
 #include "prefill.h"
@@ -202,6 +203,7 @@ int HIPFusedInference::slotAddr(int idx, char** out) {
 }
 
 HIPFusedInference::~HIPFusedInference() {
+    releaseFlow();
     for (HIPFusedInference** ref : backrefs) *ref = nullptr;
     if (stream) (void)hipStreamSynchronize(stream);
     invalidateGraphs();
@@ -636,6 +638,22 @@ int HIPFusedInference::enqueueLayerFused(const LayerWeights& L, int layer, const
 }
 
 // ---- all layers of a step in one persistent launch (flow.hip) ----
+// Two such launches at once on one GPU could each hold part of the CUs and wait for workgroups that cannot start,
+// until their waits run out.  So on every device one context at a time uses the launch: the first that needs it, until
+// it is destroyed or set to another mode; the others run the fused launches meanwhile.
+static std::mutex g_flowOwnerMutex;
+static const HIPFusedInference* g_flowOwner[64] = {};
+static bool claim_flow(const HIPFusedInference* f, int dev) {
+    if (dev < 0 || dev >= 64) return false;
+    std::lock_guard<std::mutex> lk(g_flowOwnerMutex);
+    if (!g_flowOwner[dev]) g_flowOwner[dev] = f;
+    return g_flowOwner[dev] == f;
+}
+void HIPFusedInference::releaseFlow() {
+    std::lock_guard<std::mutex> lk(g_flowOwnerMutex);
+    for (auto& o : g_flowOwner) if (o == this) o = nullptr;
+}
+
 bool HIPFusedInference::flowEligible(int l0, int l1) const {
     if (execMode != 3 || flowBroken || kvHalf) return false;
     if (!flow_shape_supported(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim)) return false;
@@ -656,7 +674,10 @@ bool HIPFusedInference::flowEligible(int l0, int l1) const {
         cus = prop.multiProcessorCount;
     }
     const FlowGeometry g = flow_geometry(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim, maxSeq, cus);
-    return flow_min_grid(nHeads, nKVHeads, g) <= cus && flow_context_fits(maxSeq, g);
+    if (!(flow_min_grid(nHeads, nKVHeads, g) <= cus && flow_context_fits(maxSeq, g))) return false;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return false; }
+    return claim_flow(this, dev);
 }
 
 int HIPFusedInference::ensureFlow() {
@@ -760,6 +781,7 @@ int HIPFusedInference::checkFlowError() {
     *hFlowErr = 0;
     HIPCHK(hipMemset(dFlowErr, 0, sizeof(int)));
     flowBroken = true;
+    releaseFlow();
     invalidateGraphs();
     set_error("persistent layer launch: a wait between phases ran into its time limit (workgroups not all resident at once?); "
               "this step's results are invalid, later steps use the separate launches");
@@ -959,7 +981,7 @@ int HIPFusedInference::primeGraph() {
     int rc = enqueueEmbed();
     if (rc) return rc;
     // a captured token leaves the exchange area reset for its successor; the first one finds it so here
-    if (flowEligible(0, nLayers)) HIPCHK(launch_flow_reset(flowXchg, flowGeo, 0, nLayers, stream));
+    if (graphsUseFlow) HIPCHK(launch_flow_reset(flowXchg, flowGeo, 0, nLayers, stream));
     return MG_OK;
 }
 
@@ -1021,9 +1043,11 @@ int HIPFusedInference::GraphCapture() {
     if (!built) return MG_E_NOT_BUILT;
     int rc = checkReady(this);
     if (rc) return rc;
-    if (execFull && execPrompt) return MG_OK;
+    const bool flow = flowEligible(0, nLayers);
+    if (execFull && execPrompt && graphsUseFlow == flow) return MG_OK;     // (the launch may have changed hands since the capture)
     invalidateGraphs();
-    if (flowEligible(0, nLayers)) { rc = ensureFlow(); if (rc) return rc; }     // allocations and uploads come before the capture
+    graphsUseFlow = flow;
+    if (flow) { rc = ensureFlow(); if (rc) return rc; }     // allocations and uploads come before the capture
     HIPCHK(hipStreamSynchronize(stream));
     for (int which = 0; which < 2; which++) {
         HIPCHK(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));

@@ -202,6 +202,28 @@ def test_new_context_uses_the_launch_and_trace(hip):
     m.close()
 
 
+def test_one_context_a_device_owns_the_launch(hip):
+    s = configs.TOY
+    a = H.Model(s, seed=8, maxSeq=24, eng=hip, oracle=False)
+    b = H.Model(s, seed=8, maxSeq=24, eng=hip, oracle=False)
+    prompt = a.prompt(4)
+    assert _in_use(a.hip) and not _in_use(b.hip)
+    rc, ta = a.hip.Generate(prompt, 8)
+    assert rc == 0, E.last_error()
+    rc, tb = b.hip.Generate(prompt, 8)                 # the fused launches
+    assert rc == 0, E.last_error()
+    assert ta.tolist() == tb.tolist()
+    assert a.hip.SetExecMode(1) == 0                   # gives the launch up
+    assert _in_use(b.hip) and not _in_use(a.hip)
+    assert b.hip.ResetKV() == 0
+    rc, tb2 = b.hip.Generate(prompt, 8)
+    assert rc == 0 and tb2.tolist() == ta.tolist()
+    b.close()
+    assert a.hip.SetExecMode(3) == 0
+    assert _in_use(a.hip)
+    a.close()
+
+
 def test_a_wait_that_runs_out_is_reported_and_the_context_goes_on(hip):
     s = configs.TOY
     m = H.Model(s, seed=7, maxSeq=40, eng=hip, threads=8)

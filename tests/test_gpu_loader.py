@@ -27,6 +27,7 @@ def test_set_weight_fp32_equals_set_weight_q8_of_oracle_bytes(hip, shape, mode):
     s = shape
     maxSeq = 12
     a, b = _ctx(hip, s, maxSeq), _ctx(hip, s, maxSeq)
+    assert a.SetExecMode(1) == 0 and b.SetExecMode(1) == 0       # the same launches in both (one context a device owns the persistent one)
     assert a.SetQuantRounding(mode) == 0
     assert a.SetQuantRounding(2) != 0                            # only 0 and 1 exist
     orc = ob.Oracle(s.dim, configs.kv_dim(s), s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab, s.nLayers, maxSeq,

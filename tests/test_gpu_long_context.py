@@ -95,6 +95,7 @@ def test_fused_split_kv_matches_per_op_single_split(hip, name, shape, maxSeq):
     at positions spanning several splits.  GPU only, so the cache is filled quickly."""
     a = H.load_fast(shape, seed=55, maxSeq=maxSeq, eng=hip, oracle=False)
     b = H.load_fast(shape, seed=55, maxSeq=maxSeq, eng=hip, oracle=False)
+    assert a.hip.SetExecMode(1) == 0
     assert b.hip.SetExecMode(0) == 0
     rng = np.random.default_rng(7)
     check = {0, 300, 2049, 6000, maxSeq - 1}

@@ -417,6 +417,8 @@ def test_layer_range_pipeline_with_l3_bridge_and_mailbox(hip):
     whole = H.Model(s, seed=41, maxSeq=8, eng=hip, threads=4)
     a = H.Model(s, seed=41, maxSeq=8, eng=hip, oracle=False)
     b = H.Model(s, seed=41, maxSeq=8, eng=hip, oracle=False)
+    for m in (whole, a, b):
+        assert m.hip.SetExecMode(1) == 0          # the same launches in all three (one context a device owns the persistent one)
     assert a.hip.HasL3() and a.hip.HiddenIdx() == 0
     prompt = whole.prompt(5)
     whole.orc.reset_kv()
