@@ -411,14 +411,16 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
 
         FLOW_TRACE(2);
         // ------------------------------------------------------------------ attention: one (head, KV split) per workgroup
+        // grouped only while a workgroup per query head and split would not fit the launch (positions far into a long context)
+        const bool grouped = GQA && p.nHeads * (pos / TILE + 1) > (int)gridDim.x;
         {
             const int nsplit = pos / TILE + 1;
-            const int QH = GQA ? p.nHeads / p.nKVHeads : 1;            // query heads of this workgroup
-            const int unit = GQA ? p.nKVHeads : p.nHeads;
+            const int QH = grouped ? p.nHeads / p.nKVHeads : 1;        // query heads of this workgroup
+            const int unit = grouped ? p.nKVHeads : p.nHeads;
             const int split = blockIdx.x / unit, hu = blockIdx.x % unit;
             if (split < G.smax && split < nsplit) {
-                const int kvh = GQA ? hu : hu / (p.nHeads / p.nKVHeads);
-                const int h0 = GQA ? hu * QH : hu;
+                const int kvh = grouped ? hu : hu / (p.nHeads / p.nKVHeads);
+                const int h0 = grouped ? hu * QH : hu;
                 const int tg = tid / LPR, dl = tid % LPR;
                 const int t0 = split * TILE;
                 const int len = pos + 1;
@@ -459,7 +461,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 if (hi) __syncthreads();                    // accbuf, lbuf, wred are free again
                 float4 q4[NF];
 #pragma unroll
-                for (int j = 0; j < NF; j++) q4[j] = sqkv[2 + (GQA ? hi : 0)][j * 16 + dl];
+                for (int j = 0; j < NF; j++) q4[j] = sqkv[2 + hi][j * 16 + dl];
                 float sc[VU];
                 float tmax = -INFINITY;
 #pragma unroll
@@ -525,7 +527,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             }
         }
 
-        if constexpr (GQA) {
+        if (grouped) {
             // Long contexts, tens of KV splits: merged once per head, by workgroup h for head h (every thread a 16-byte piece
             // and every eighth split, eight splits' loads in flight together, then combined through LDS), and handed on as
             // one vector -- every consumer merging all partials itself re-reads tens of KB per workgroup and layer.
@@ -609,7 +611,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 };
                 if (it < nI) resolve(it);
                 // stage the attention output: merge the KV splits' partials (running maximum, as the split-KV combine)
-                if constexpr (GQA) {
+                if (grouped) {
                     stage_plain(X + G.offAttn, dim, a4, wt);      // merged per head above
                 } else {
                 __syncthreads();
