@@ -125,13 +125,15 @@ private:
     int uploadMatQ4(int idx, DevMat& m, int rows, int cols, const uint8_t* raw, size_t nbytes);
     int setVec(int idx, float*& dst, const float* data, size_t n, size_t expect);
     int slotAddr(int idx, char** out);
-    Slab scratch, headSlab, prefillSlab;
+    Slab scratch, headSlab, prefillSlab, prefillKVSlab;
     int prefillCap = 0;             // rows the prefill buffers hold
+    int prefillKVCap = 0;           // cache rows the attention's split planes hold
+    void* pfKVSplit = nullptr;
     int* pfTokens = nullptr;
     float *pfX = nullptr, *pfQ = nullptr, *pfK = nullptr, *pfV = nullptr, *pfGate = nullptr, *pfUp = nullptr;
     void *pfHi = nullptr, *pfLo = nullptr, *pfHi2 = nullptr, *pfLo2 = nullptr;
     float* pfPartial = nullptr;
-    int ensurePrefill(int rows);
+    int ensurePrefill(int rows, int kvRows);
     std::vector<Slab> layerSlabs, kvSlabs;
     size_t slotOff[12] = {0};
     size_t layerSlabBytes = 0;

@@ -210,6 +210,7 @@ HIPFusedInference::~HIPFusedInference() {
     scratch.release();
     headSlab.release();
     prefillSlab.release();
+    prefillKVSlab.release();
     for (auto& sl : layerSlabs) sl.release();
     for (auto& sl : kvSlabs) sl.release();
     if (embedTable) (void)hipFree(embedTable);
@@ -1297,7 +1298,20 @@ int HIPFusedInference::ProfileDecode(int token, int pos, int steps, unsigned cla
 // Batched prefill (Q8): the layer of the decode step applied to T rows at
 // once, the seven projections as MFMA GEMMs.
 // ---------------------------------------------------------------------------
-int HIPFusedInference::ensurePrefill(int rows) {
+int HIPFusedInference::ensurePrefill(int rows, int kvRows) {
+    const int kvPad = (kvRows + 31) / 32 * 32;
+    if (kvPad > prefillKVCap) {                 // the attention's hi/lo planes of the cache rows [0, pos0 + T)
+        HIPCHK(hipStreamSynchronize(stream));
+        prefillKVSlab.release();
+        const int want = std::min((maxSeq + 31) / 32 * 32, std::max(kvPad, 2 * prefillKVCap));
+        prefillKVCap = 0;
+        const size_t bytes = prefill_kv_split_bytes(want, kvDim);
+        int rc = prefillKVSlab.init(bytes + 256);
+        if (rc) return rc;
+        pfKVSplit = prefillKVSlab.take(bytes);
+        if (!pfKVSplit) { set_error("prefill KV slab too small"); return MG_E_STATE; }
+        prefillKVCap = want;
+    }
     if (rows <= prefillCap) return MG_OK;
     HIPCHK(hipStreamSynchronize(stream));
     prefillSlab.release();
@@ -1341,7 +1355,7 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
             return MG_E_UNSUPPORTED;
         }
     }
-    rc = ensurePrefill(nTokens);
+    rc = ensurePrefill(nTokens, pos0 + nTokens);
     if (rc) return rc;
     const int T = nTokens;
     HIPCHK(hipStreamSynchronize(stream));
@@ -1373,7 +1387,7 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
             HIPCHK(launch_rope_store_rows(pfQ, pfK, pfV, kCache[l], vCache[l], kvHalf, cosTab, sinTab, pos0, T, dim, kvDim, headDim, stream));
         g.ropeKc = nullptr; g.ropeVc = nullptr;
         // the attention writes its rows as the hi/lo split the output projection reads
-        HIPCHK(launch_prefill_attention(pfQ, kCache[l], vCache[l], kvHalf, nullptr, pfHi, pfLo, T, pos0, maxSeq, dim, kvDim, nHeads,
+        HIPCHK(launch_prefill_attention(pfQ, kCache[l], vCache[l], kvHalf, pfKVSplit, nullptr, pfHi, pfLo, T, pos0, maxSeq, dim, kvDim, nHeads,
                                         nKVHeads, headDim, stream));
         g.K = dim; g.nseg = 1; g.q4 = L.wo.kind == WF_Q4P; g.seg[0] = seg(L.wo, nullptr, pfX);
         // where K is split, the kernel that sums the splits also writes norm2's split of the new rows

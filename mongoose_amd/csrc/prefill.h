@@ -16,10 +16,13 @@ hipError_t launch_swiglu_split(const float* gate, const float* up, int T, int K,
 hipError_t launch_rope_store_rows(float* q, const float* k, const float* v, void* Kc, void* Vc, int kvHalf, const float* cosTab,
                                   const float* sinTab, int pos0, int T, int dim, int kvDim, int headDim, hipStream_t s);
 // Causal attention of T query rows [T,dim] (rotated) at positions pos0.. over cache rows [0, pos0+T); out [T,dim]
-// and/or its hi/lo split for K = dim in launch_split_rows's layout (either may be NULL, not both).
-hipError_t launch_prefill_attention(const float* q, const void* Kc, const void* Vc, int kvHalf, float* out, void* splitHi,
-                                    void* splitLo, int T, int pos0, int rowLimit, int dim, int kvDim, int nHeads, int nKVHeads,
-                                    int headDim, hipStream_t s);
+// and/or its hi/lo split for K = dim in launch_split_rows's layout (either may be NULL, not both).  The cache rows
+// are first split into bf16 hi/lo planes in kvSplit, a workspace of prefill_kv_split_bytes(pos0 + T, kvDim) bytes
+// (16-byte aligned) that the launch owns until it has finished.
+size_t prefill_kv_split_bytes(int rows, int kvDim);
+hipError_t launch_prefill_attention(const float* q, const void* Kc, const void* Vc, int kvHalf, void* kvSplit, float* out,
+                                    void* splitHi, void* splitLo, int T, int pos0, int rowLimit, int dim, int kvDim, int nHeads,
+                                    int nKVHeads, int headDim, hipStream_t s);
 // Embedding rows of T tokens: kind 0 = Q8 row * scale, 1 = fp16 table, 2 = fp32 table, 3 = Q4_0 split-layout row.
 hipError_t launch_embed_rows(int kind, const void* table, const float* scales, const int* tokens, float* x, int T, int dim,
                              int vocab, hipStream_t s);

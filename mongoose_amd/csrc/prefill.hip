@@ -160,41 +160,102 @@ hipError_t launch_embed_rows(int kind, const void* table, const float* scales, c
 
 // ---------------------------------------------------------------------------
 // Causal attention over T query rows (mongoose.cu:251-353 for a training
-// sequence; here against the KV caches, query t at position pos0 + t).
+// sequence; here against the KV caches, query t at position pos0 + t), on the
+// bf16 matrix instruction with every fp32 operand split into two bf16 terms
+// (x = hi + lo, |x - hi - lo| <= 2^-16 |x|) and three products per pair of
+// operands (hi.hi + hi.lo + lo.hi; lo.lo is below 2^-16 of the result).
+//
+// The cache rows are split once per layer by kv_split_kernel into planes the
+// matrix instruction reads as they lie: K hi / lo as [row][kvDim], and V hi /
+// lo transposed, [kvh * HD + d][row], the rows of each group of 16 in the order
+// 0-3, 8-11, 4-7, 12-15 (see the P operand below).  Rows past pos0 + T, up to
+// the next multiple of 32, are written as zeros.
+//
 // One workgroup = 32 queries of one head; its four waves take the 32-position
 // KV tiles in turn (tile w, w+4, ...) with their own running max / sum /
-// output and are combined at the end, so the longest serial chain is a quarter
-// of the causal range.  Both products run on the fp32 matrix instruction
-// v_mfma_f32_32x32x2_f32 (exact fp32 products, fp32 accumulation), arranged
-// transposed so that a lane owns one query:
-//   S^T[kpos][q] = K . Q^T    A = K tile from LDS, B = Q rows held in registers
-//   O^T[d][q]    = V^T . P^T  A = V rows straight from the cache, B = the S^T accumulator itself
-// (C layout: lane l holds column l%32, rows 8*(i/4) + 4*(l/32) + i%4; as a B
-// operand step s wants row k = l/32 of its pair, so step s pairs exactly the
-// rows register s holds in the two lane halves.)
+// output and are combined at the end.  Arranged transposed, so that a lane
+// owns one query (C layout: lane l holds column l%32, rows 8*(i/4) + 4*(l/32)
+// + i%4 for i = 0..15):
+//   S^T[kpos][q] = K . Q^T    A = K rows (lane: row l%32, 8 d of half l/32), B = Q^T held in registers
+//   O^T[d][q]    = V^T . P^T  A = V^T rows, B = the S^T accumulator itself: as the B operand of step s2
+//                             a lane holds k slots j = 0..7 = accumulator registers 8*s2 + j, i.e. tile
+//                             positions 16*s2 + 8*(j/4) + 4*(l/32) + j%4 -- the order V^T is stored in.
 // ---------------------------------------------------------------------------
-template <int HD, typename KVT>
-__global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const KVT* Kc, const KVT* Vc, float* out,
-                                                          unsigned short* hi, unsigned short* lo, int T,
-                                                          int pos0, int dim, int kvDim, int nHeads, int nKVHeads) {
-    constexpr int KS = HD + 4;                 // LDS row stride of the K tile (floats)
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ void split8(const float (&v)[8], bf16x8_t& h, bf16x8_t& l) {
+    unsigned short hs[8], ls[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        hs[i] = f32_to_bf16_rne(v[i]);
+        ls[i] = f32_to_bf16_rne(v[i] - bf16_to_f32(hs[i]));
+    }
+    uint4 uh, ul;
+    uh.x = hs[0] | ((unsigned)hs[1] << 16); uh.y = hs[2] | ((unsigned)hs[3] << 16);
+    uh.z = hs[4] | ((unsigned)hs[5] << 16); uh.w = hs[6] | ((unsigned)hs[7] << 16);
+    ul.x = ls[0] | ((unsigned)ls[1] << 16); ul.y = ls[2] | ((unsigned)ls[3] << 16);
+    ul.z = ls[4] | ((unsigned)ls[5] << 16); ul.w = ls[6] | ((unsigned)ls[7] << 16);
+    h = __builtin_bit_cast(bf16x8_t, uh);
+    l = __builtin_bit_cast(bf16x8_t, ul);
+}
+
+// grid (rowsPad / 16, nKVHeads), HD threads: thread d of a workgroup takes column kvh * HD + d of 16 rows
+template <typename KVT>
+__global__ void kv_split_kernel(const KVT* Kc, const KVT* Vc, int rows, int kvDim, int HD, unsigned short* Khi,
+                                unsigned short* Klo, unsigned short* VThi, unsigned short* VTlo, int vtStride) {
+    const int g = blockIdx.x, col = blockIdx.y * HD + threadIdx.x;
+    unsigned short vh[16], vl[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int r = g * 16 + i;
+        const size_t o = (size_t)r * kvDim + col;
+        const float k = r < rows ? (float)Kc[o] : 0.f;
+        const float v = r < rows ? (float)Vc[o] : 0.f;
+        const unsigned short kh = f32_to_bf16_rne(k);
+        Khi[o] = kh;
+        Klo[o] = f32_to_bf16_rne(k - bf16_to_f32(kh));
+        const int idx = 8 * ((i >> 2) & 1) + (i & 3) + 4 * (i >> 3);
+        vh[idx] = f32_to_bf16_rne(v);
+        vl[idx] = f32_to_bf16_rne(v - bf16_to_f32(vh[idx]));
+    }
+    uint4* dh = reinterpret_cast<uint4*>(VThi + (size_t)col * vtStride + g * 16);
+    uint4* dl = reinterpret_cast<uint4*>(VTlo + (size_t)col * vtStride + g * 16);
+#pragma unroll
+    for (int w = 0; w < 2; w++) {
+        dh[w] = make_uint4(vh[8 * w] | ((unsigned)vh[8 * w + 1] << 16), vh[8 * w + 2] | ((unsigned)vh[8 * w + 3] << 16),
+                           vh[8 * w + 4] | ((unsigned)vh[8 * w + 5] << 16), vh[8 * w + 6] | ((unsigned)vh[8 * w + 7] << 16));
+        dl[w] = make_uint4(vl[8 * w] | ((unsigned)vl[8 * w + 1] << 16), vl[8 * w + 2] | ((unsigned)vl[8 * w + 3] << 16),
+                           vl[8 * w + 4] | ((unsigned)vl[8 * w + 5] << 16), vl[8 * w + 6] | ((unsigned)vl[8 * w + 7] << 16));
+    }
+}
+
+template <int HD>
+__global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const unsigned short* Khi, const unsigned short* Klo,
+                                                          const unsigned short* VThi, const unsigned short* VTlo, int vtStride,
+                                                          float* out, unsigned short* hi, unsigned short* lo, int T, int pos0,
+                                                          int dim, int kvDim, int nHeads, int nKVHeads) {
+    constexpr int NS = HD / 16;                // 16-wide steps of the head dimension
     constexpr int DB = HD / 32;                // 32-wide blocks of the head dimension
-    __shared__ __attribute__((aligned(16))) float lds[4][32 * KS];
+    __shared__ __attribute__((aligned(16))) float lds[4][HD * 33];
     __shared__ float wm[4][32], wl[4][32];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, half = lane >> 5;
-    const int q0 = blockIdx.x * 32, head = blockIdx.y;
+    const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * 32, head = blockIdx.y;      // the longest causal ranges start first
     const int kvh = head / (nHeads / nKVHeads);
     const int myq = q0 + col;                           // this lane's query row
     const int qpos = pos0 + min(myq, T - 1);            // its position (clamped rows are never stored)
     const float scale = 1.0f / sqrtf((float)HD);
 
-    // Q^T operand: lane holds Q[myq][2*s + half], s = 0 .. HD/2-1
-    float qreg[HD / 2];
+    // Q^T operand: step s holds Q[myq][16 s + 8 half .. + 7]
+    bf16x8_t qh[NS], ql[NS];
     {
-        const float* qr = q + (size_t)min(myq, T - 1) * dim + (size_t)head * HD + half;
+        const float* qr = q + (size_t)min(myq, T - 1) * dim + (size_t)head * HD + 8 * half;
 #pragma unroll
-        for (int s = 0; s < HD / 2; s++) qreg[s] = qr[2 * s];
+        for (int s = 0; s < NS; s++) {
+            const float4 a = *reinterpret_cast<const float4*>(qr + 16 * s), b = *reinterpret_cast<const float4*>(qr + 16 * s + 4);
+            const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+            split8(v, qh[s], ql[s]);
+        }
     }
     float16_t o[DB];
 #pragma unroll
@@ -205,42 +266,39 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const
 
     const int lastPos = pos0 + min(q0 + 31, T - 1);     // furthest position any query of the block sees
     const int nTiles = lastPos / 32 + 1;
-    float* kt = lds[wave];
+    const size_t kcol = (size_t)kvh * HD + 8 * half;
     for (int tile = wave; tile < nTiles; tile += 4) {
         const int t0 = tile * 32;
-        // K tile -> this wave's LDS (rows past lastPos are clamped; they are masked below)
+        const unsigned short* kh = Khi + (size_t)(t0 + col) * kvDim + kcol;
+        const unsigned short* kl = Klo + (size_t)(t0 + col) * kvDim + kcol;
+        float16_t sT, sX;                                // hi.hi and the two cross terms: two chains for the matrix pipe
 #pragma unroll
-        for (int i = 0; i < 32 * HD / 4 / 64; i++) {
-            const int idx = i * 64 + lane, r = idx / (HD / 4), c4 = idx % (HD / 4);
-            typedef KVT kv4_t __attribute__((ext_vector_type(4)));
-            const kv4_t kv = *reinterpret_cast<const kv4_t*>(Kc + (size_t)min(t0 + r, lastPos) * kvDim + (size_t)kvh * HD + c4 * 4);
-            *reinterpret_cast<float4*>(&kt[r * KS + c4 * 4]) = make_float4((float)kv[0], (float)kv[1], (float)kv[2], (float)kv[3]);
+        for (int e = 0; e < 16; e++) { sT[e] = 0.f; sX[e] = 0.f; }
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const bf16x8_t ah = *reinterpret_cast<const bf16x8_t*>(kh + 16 * s);
+            const bf16x8_t al = *reinterpret_cast<const bf16x8_t*>(kl + 16 * s);
+            sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, qh[s], sT, 0, 0, 0);
+            sX = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, ql[s], sX, 0, 0, 0);
+            sX = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, qh[s], sX, 0, 0, 0);
         }
-        __builtin_amdgcn_s_waitcnt(0);                   // wave-private buffer: the wave's own stores have landed
-        __builtin_amdgcn_wave_barrier();
-        float16_t sT;
-#pragma unroll
-        for (int e = 0; e < 16; e++) sT[e] = 0.f;
-#pragma unroll
-        for (int s = 0; s < HD / 2; s++)
-            sT = __builtin_amdgcn_mfma_f32_32x32x2f32(kt[col * KS + 2 * s + half], qreg[s], sT, 0, 0, 0);
         // causal mask, online softmax for this lane's query over the tile's 32 positions
         float tmax = -INFINITY;
 #pragma unroll
         for (int e = 0; e < 16; e++) {
             const int kpos = t0 + 8 * (e >> 2) + 4 * half + (e & 3);
-            sT[e] = kpos <= qpos ? sT[e] * scale : -INFINITY;
+            sT[e] = kpos <= qpos ? (sT[e] + sX[e]) * scale : -INFINITY;
             tmax = fmaxf(tmax, sT[e]);
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
         const float mNew = fmaxf(m, tmax);
         const float corr = m == -INFINITY ? 0.f : expf(m - mNew);
         float psum = 0.f;
+        float pv[16];
 #pragma unroll
         for (int e = 0; e < 16; e++) {
-            const float pv = sT[e] == -INFINITY ? 0.f : expf(sT[e] - mNew);
-            sT[e] = pv;
-            psum += pv;
+            pv[e] = sT[e] == -INFINITY ? 0.f : expf(sT[e] - mNew);
+            psum += pv[e];
         }
         psum += __shfl_xor(psum, 32, 64);
         l = l * corr + psum;
@@ -249,20 +307,26 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const
         for (int b = 0; b < DB; b++)
 #pragma unroll
             for (int e = 0; e < 16; e++) o[b][e] *= corr;
-        // O^T += V^T . P^T : step s takes positions 8*(s/4) + 4*half + s%4, which is what sT[s] holds
+        // O^T += V^T . P^T
 #pragma unroll
-        for (int s = 0; s < 16; s++) {
-            const int kpos = min(t0 + 8 * (s >> 2) + 4 * half + (s & 3), lastPos);
-            const KVT* vr = Vc + (size_t)kpos * kvDim + (size_t)kvh * HD + col;
+        for (int s2 = 0; s2 < 2; s2++) {
+            bf16x8_t ph, pl;
+            const float pp[8] = {pv[8 * s2], pv[8 * s2 + 1], pv[8 * s2 + 2], pv[8 * s2 + 3],
+                                 pv[8 * s2 + 4], pv[8 * s2 + 5], pv[8 * s2 + 6], pv[8 * s2 + 7]};
+            split8(pp, ph, pl);
 #pragma unroll
-            for (int b = 0; b < DB; b++)
-                o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32((float)vr[32 * b], sT[s], o[b], 0, 0, 0);
+            for (int b = 0; b < DB; b++) {
+                const size_t vo = (size_t)(kvh * HD + 32 * b + col) * vtStride + t0 + 16 * s2 + 8 * half;
+                const bf16x8_t vh = *reinterpret_cast<const bf16x8_t*>(VThi + vo);
+                const bf16x8_t vl = *reinterpret_cast<const bf16x8_t*>(VTlo + vo);
+                o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vh, ph, o[b], 0, 0, 0);
+                o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vh, pl, o[b], 0, 0, 0);
+                o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vl, ph, o[b], 0, 0, 0);
+            }
         }
-        __builtin_amdgcn_wave_barrier();                 // the K tile is overwritten next
     }
-    // ---- combine the four waves: O^T partials through the (now free) tile buffers ----
-    // layout in kt: [d][q] with row stride 33
-    static_assert(HD * 33 <= 32 * KS, "tile buffer too small for the partial output");
+    // ---- combine the four waves: O^T partials through LDS, [d][q] with row stride 33 ----
+    float* kt = lds[wave];
 #pragma unroll
     for (int b = 0; b < DB; b++)
 #pragma unroll
@@ -291,25 +355,36 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const
     }
 }
 
-hipError_t launch_prefill_attention(const float* q, const void* Kc, const void* Vc, int kvHalf, float* out, void* splitHi,
-                                    void* splitLo, int T, int pos0, int rowLimit, int dim, int kvDim, int nHeads, int nKVHeads,
-                                    int headDim, hipStream_t s) {
+size_t prefill_kv_split_bytes(int rows, int kvDim) {
+    const size_t rowsPad = ((size_t)rows + 31) / 32 * 32;
+    return 4 * rowsPad * (size_t)kvDim * sizeof(unsigned short);
+}
+
+hipError_t launch_prefill_attention(const float* q, const void* Kc, const void* Vc, int kvHalf, void* kvSplit, float* out,
+                                    void* splitHi, void* splitLo, int T, int pos0, int rowLimit, int dim, int kvDim, int nHeads,
+                                    int nKVHeads, int headDim, hipStream_t s) {
     if (T <= 0) return hipSuccess;
-    if ((!out && !splitHi) || (splitHi == nullptr) != (splitLo == nullptr)) return hipErrorInvalidValue;
+    if ((!out && !splitHi) || (splitHi == nullptr) != (splitLo == nullptr) || !kvSplit) return hipErrorInvalidValue;
     unsigned short* hi = static_cast<unsigned short*>(splitHi);
     unsigned short* lo = static_cast<unsigned short*>(splitLo);
     if (nKVHeads <= 0 || nHeads % nKVHeads != 0 || pos0 < 0 || pos0 + T > rowLimit || dim != nHeads * headDim ||
         kvDim != nKVHeads * headDim || (headDim != 64 && headDim != 128)) return hipErrorInvalidValue;
+    const int rows = pos0 + T, rowsPad = (rows + 31) / 32 * 32;
+    const size_t plane = (size_t)rowsPad * kvDim;
+    unsigned short* Khi = static_cast<unsigned short*>(kvSplit);
+    unsigned short *Klo = Khi + plane, *VThi = Klo + plane, *VTlo = VThi + plane;
+    const dim3 sgrid((unsigned)(rowsPad / 16), (unsigned)nKVHeads);
+    if (kvHalf) hipLaunchKernelGGL((kv_split_kernel<_Float16>), sgrid, dim3(headDim), 0, s, static_cast<const _Float16*>(Kc),
+                                   static_cast<const _Float16*>(Vc), rows, kvDim, headDim, Khi, Klo, VThi, VTlo, rowsPad);
+    else hipLaunchKernelGGL((kv_split_kernel<float>), sgrid, dim3(headDim), 0, s, static_cast<const float*>(Kc),
+                            static_cast<const float*>(Vc), rows, kvDim, headDim, Khi, Klo, VThi, VTlo, rowsPad);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
     dim3 grid((unsigned)((T + 31) / 32), (unsigned)nHeads);
-    const float* kf = static_cast<const float*>(Kc); const float* vf = static_cast<const float*>(Vc);
-    const _Float16* kh = static_cast<const _Float16*>(Kc); const _Float16* vh = static_cast<const _Float16*>(Vc);
-    if (headDim == 64) {
-        if (kvHalf) hipLaunchKernelGGL((prefill_attn_kernel<64, _Float16>), grid, dim3(256), 0, s, q, kh, vh, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
-        else hipLaunchKernelGGL((prefill_attn_kernel<64, float>), grid, dim3(256), 0, s, q, kf, vf, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
-    } else {
-        if (kvHalf) hipLaunchKernelGGL((prefill_attn_kernel<128, _Float16>), grid, dim3(256), 0, s, q, kh, vh, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
-        else hipLaunchKernelGGL((prefill_attn_kernel<128, float>), grid, dim3(256), 0, s, q, kf, vf, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
-    }
+    if (headDim == 64)
+        hipLaunchKernelGGL((prefill_attn_kernel<64>), grid, dim3(256), 0, s, q, Khi, Klo, VThi, VTlo, rowsPad, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
+    else
+        hipLaunchKernelGGL((prefill_attn_kernel<128>), grid, dim3(256), 0, s, q, Khi, Klo, VThi, VTlo, rowsPad, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
     return hipGetLastError();
 }
 
@@ -323,7 +398,6 @@ hipError_t launch_prefill_attention(const float* q, const void* Kc, const void* 
 // that share a weight tile are placed on one XCD (ids congruent mod 8), so the
 // tile comes into that XCD's L2 once.
 // ---------------------------------------------------------------------------
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 constexpr int BK = 64;
 constexpr int A_STRIDE = BK + 8;    // bf16 per LDS row (144 bytes)
 constexpr int B_STRIDE = BK + 16;   // bytes per LDS row of int8 weights (80)
@@ -594,21 +668,32 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// The large Q8 tile (256 x 256, 1024 threads) fed by direct global -> LDS loads
-// (global_load_lds_dwordx4: no register staging, no LDS store instructions)
-// through a three-stage LDS ring with K steps of 32: a stage's loads are issued
-// two steps before it is multiplied, one barrier per step.  A wave's load
-// lands as 1 KB of consecutive 16-byte slots, so the layout is made on the
-// global side: slot s of wave w holds, for A, row 16w + s/4 and piece
-// (s%4) ^ ((row>>1)&3) of the row's 64 bytes; for W (waves 0-7), row 32w + s/2
-// and piece (s%2) ^ ((row>>2)&1) of its 32 bytes.  The XOR makes every
-// fragment read (8 lanes = 128 bytes) touch all LDS banks once.  A W piece is
-// 16 consecutive k of one lane half: its low 8 bytes feed the first MFMA step,
-// its high 8 bytes the second, and the A pieces are picked to match.
-// 917 TF issued against 717 for the register-staged tile on the gate/up shape.
+// The large Q8 tile: 256 x 256, 512 threads (4 x 2 waves of 64 rows x 128
+// columns), v_mfma_f32_16x16x32_bf16, a three-stage LDS ring with K steps of 32
+// and one barrier per step.  Measured on the gate|up shape (512 x 28672 x 4096):
+// the matrix pipe and ordinary vector instructions of a SIMD do not overlap
+// here (busy cycles add up), so the loop carries as few of the latter as it
+// can, and under this load the chip clocks near 1.8 GHz, where the 16x16x32
+// form sustains 2.2 PFLOP/s on random operands against 1.84 for 32x32x16.
+//
+// * The activation planes (A hi, A lo: 16 KB a stage each) come by direct global -> LDS loads
+//   (global_load_lds_dwordx4: no registers, no LDS store instructions), issued two steps ahead.  A wave's load
+//   lands as 1 KB of consecutive 16-byte slots, so the layout is made on the global side: slot s of a
+//   load holds row r = first + s/4 and piece (s%4) ^ ((r>>1)&3) of the row's 64 bytes.
+// * The weights come through registers, 16 int8 a thread and step, requested five steps ahead (their
+//   rows come from HBM, the activations from L2), and are converted to bf16 once per workgroup --
+//   not once per wave that multiplies them -- into the stage's third plane, same layout.
+// * A fragment read is ds_read_b128 with lane l at row l%16, piece l/16: with the XOR by (row>>1)&3
+//   it is served without bank conflicts (4 cycles an instruction; (row>>2)&3 or none: 8).
+// * s_waitcnt / s_barrier are written out: the compiler's __syncthreads() waits for every outstanding
+//   load, including the ones issued for later steps.  Loads complete in order, five are issued per
+//   step (A x 4, W), so "at most five outstanding" at the top of step s means A(s) and W(s+1) landed.
+// The K steps of a workgroup must be a multiple of 4 (the register ring is unrolled by hand).
 // ---------------------------------------------------------------------------
 constexpr int RK = 32, RS = 3;
-constexpr int RING_STAGE_BYTES = 256 * 64 * 2 + 256 * 32;      // A hi + A lo + W
+constexpr int RING_PLANE = 256 * 64;                      // 256 rows x 32 bf16
+constexpr int RING_STAGE_BYTES = 3 * RING_PLANE;          // A hi, A lo, W as bf16
+typedef float float4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ bf16x8_t cvt8_i8_bf16(int lo, int hi) {
     uint4 u;
@@ -620,11 +705,11 @@ __device__ __forceinline__ bf16x8_t cvt8_i8_bf16(int lo, int hi) {
 }
 
 template <int MODE>
-__global__ __launch_bounds__(1024) void gemm_q8_ring_kernel(GemmParams p) {
+__global__ __launch_bounds__(512) void gemm_q8_ring_kernel(GemmParams p) {
     constexpr int BM = 256, BN = 256;
     extern __shared__ __attribute__((aligned(16))) unsigned char ring[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 2, wn = wave & 3;             // 4 x 4 waves, each 64 x 64
+    const int wm = wave >> 1, wn = wave & 1;             // 4 x 2 waves, each 64 rows x 128 columns
     const int numM = (p.T + BM - 1) / BM;
     const int L = blockIdx.x;
     const int grp = L / (8 * numM), rem = L % (8 * numM);
@@ -637,97 +722,127 @@ __global__ __launch_bounds__(1024) void gemm_q8_ring_kernel(GemmParams p) {
     }
     const int N = sg.N, K = p.K, T = p.T;
     // MODE 3 (gate | up -> silu(gate) * up): a tile is 128 columns of the output; its 256 weight rows
-    // alternate in blocks of 32 between the gate and the up matrix, so a wave's two 32-column MFMA
-    // blocks are the gate and the up values of the same 32 columns and the product needs no exchange.
+    // alternate in blocks of 32 between the gate and the up matrix, so a wave holds the gate and the
+    // up values of the same columns (blocks j and j + 2) and the product needs no exchange.
     const int m0 = mTile * BM, n0 = MODE == 3 ? nTile * 128 : (nTile - sg.tile0) * BN;
-    const int ksteps = K / RK;                            // K is a multiple of 32
+    const int ksteps = K / RK;
     const int ks64 = (K + 63) / 64;                       // the split planes are blocked in 64-k steps
     const int stepBeg = MODE == 2 ? blockIdx.y * p.stepsPerSplit * 2 : 0;
     const int stepEnd = MODE == 2 ? min(ksteps, stepBeg + p.stepsPerSplit * 2) : ksteps;
     const int planeRows = ((T + 127) >> 7) << 7;
 
-    const int aRowL = 16 * wave + (lane >> 2);
-    const int aSeg = (lane & 3) ^ ((aRowL >> 1) & 3);
-    const int aRowG = min(m0 + aRowL, planeRows - 1);
-    const size_t aOff = (size_t)(aRowG >> 7) * ks64 * 8192 + (size_t)(aRowG & 127) * 64 + aSeg * 8;
-    const unsigned short* aH = p.Ahi + aOff;
-    const unsigned short* aL = p.Alo + aOff;
-    const int bRowL = 32 * (wave & 7) + (lane >> 1);
-    const int bSeg = (lane & 1) ^ ((bRowL >> 2) & 1);
-    const signed char* bG = sg.W + (size_t)min(n0 + bRowL, N - 1) * K + bSeg * 16;
-    if (MODE == 3) {
-        const int blk = wave & 7;                         // this wave's 32 rows: block blk of the tile
-        const int wrow = min(n0 + (blk >> 1) * 32 + (bRowL & 31), N - 1);
-        bG = ((blk & 1) ? p.seg[1].W : p.seg[0].W) + (size_t)wrow * K + bSeg * 16;
+    // A: the wave's two loads per plane cover rows 32 wave + 16 u + lane/4, u = 0, 1
+    unsigned aOff[2];                                     // in elements of a plane (< 2^32)
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int rl = 32 * wave + 16 * u + (lane >> 2);
+        const int seg = (lane & 3) ^ ((rl >> 1) & 3);
+        const int rg = min(m0 + rl, planeRows - 1);
+        aOff[u] = (unsigned)(rg >> 7) * (unsigned)ks64 * 8192u + (unsigned)(rg & 127) * 64u + (unsigned)seg * 8u;
     }
-    const bool bWave = wave < 8;
+    // W: thread t -> tile row t/2, 16 weights (t%2)*16 .. +15 of the step = pieces 2 (t%2) and 2 (t%2) + 1 of the row
+    const int bRowL = tid >> 1, bQ = (tid & 1) * 2;
+    const signed char* bG;
+    if (MODE == 3) {
+        const int blk = bRowL >> 5;
+        const int wrow = min(n0 + (blk >> 1) * 32 + (bRowL & 31), N - 1);
+        bG = ((blk & 1) ? p.seg[1].W : p.seg[0].W) + (size_t)wrow * K + bQ * 8;
+    } else {
+        bG = sg.W + (size_t)min(n0 + bRowL, N - 1) * K + bQ * 8;
+    }
+    const unsigned bDst0 = 2 * RING_PLANE + bRowL * 64 + ((bQ ^ ((bRowL >> 1) & 3)) * 16);
+    const unsigned bDst1 = 2 * RING_PLANE + bRowL * 64 + (((bQ + 1) ^ ((bRowL >> 1) & 3)) * 16);
+    const int fr = lane & 15, fq = lane >> 4;
+    const unsigned offA = (wm * 64 + fr) * 64 + ((fq ^ ((fr >> 1) & 3)) * 16);
+    const unsigned offW = 2 * RING_PLANE + (wn * 128 + fr) * 64 + ((fq ^ ((fr >> 1) & 3)) * 16);
 
-    auto issue = [&](int step, int stage) __attribute__((always_inline)) {
+    auto issueA = [&](int step, int stage) __attribute__((always_inline)) {
         const int st = min(step, ksteps - 1);            // past the end: a harmless reload that keeps the counters uniform
-        unsigned char* base = ring + stage * RING_STAGE_BYTES;
+        unsigned char* base = ring + stage * RING_STAGE_BYTES + wave * 2048;
         const size_t ko = (size_t)(st >> 1) * 8192 + (st & 1) * 32;
-        __builtin_amdgcn_global_load_lds(aH + ko, reinterpret_cast<int4*>(base + wave * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(aL + ko, reinterpret_cast<int4*>(base + BM * 64 + wave * 1024), 16, 0, 0);
-        if (bWave) __builtin_amdgcn_global_load_lds(bG + (size_t)st * RK, reinterpret_cast<int4*>(base + BM * 128 + wave * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(p.Ahi + aOff[0] + ko, reinterpret_cast<int4*>(base), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(p.Ahi + aOff[1] + ko, reinterpret_cast<int4*>(base + 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(p.Alo + aOff[0] + ko, reinterpret_cast<int4*>(base + RING_PLANE), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(p.Alo + aOff[1] + ko, reinterpret_cast<int4*>(base + RING_PLANE + 1024), 16, 0, 0);
+    };
+    auto loadW = [&](int step) __attribute__((always_inline)) {
+        return *reinterpret_cast<const int4*>(bG + (size_t)min(step, ksteps - 1) * RK);
+    };
+    auto putW = [&](int4 w, int stage) __attribute__((always_inline)) {
+        *reinterpret_cast<bf16x8_t*>(ring + stage * RING_STAGE_BYTES + bDst0) = cvt8_i8_bf16(w.x, w.y);
+        *reinterpret_cast<bf16x8_t*>(ring + stage * RING_STAGE_BYTES + bDst1) = cvt8_i8_bf16(w.z, w.w);
     };
 
-    float16_t acc[2][2];
+    float4_t acc[4][8];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < 8; j++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+            for (int e = 0; e < 4; e++) acc[i][j][e] = 0.f;
 
-    issue(stepBeg, 0);
-    issue(stepBeg + 1, 1);
-    int stage = 0;
-    for (int step = stepBeg; step < stepEnd; step++) {
-        // this step's stage has landed; the next stage's loads may still be in flight
-        if (bWave) asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-        __syncthreads();
-        int nst = stage + 2; if (nst >= RS) nst -= RS;
-        issue(step + 2, nst);                            // refills the stage every wave finished reading before this barrier
+    auto multiply = [&](int stage) __attribute__((always_inline)) {
         const unsigned char* base = ring + stage * RING_STAGE_BYTES;
-        const int half = lane >> 5;
-        bf16x8_t b[2][2];
+        bf16x8_t b[8];
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int row = wn * 64 + j * 32 + (lane & 31);
-            const int4 w = *reinterpret_cast<const int4*>(base + BM * 128 + (row * 2 + (half ^ ((row >> 2) & 1))) * 16);
-            b[j][0] = cvt8_i8_bf16(w.x, w.y);
-            b[j][1] = cvt8_i8_bf16(w.z, w.w);
+        for (int j = 0; j < 8; j++) b[j] = *reinterpret_cast<const bf16x8_t*>(base + offW + j * 1024);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const bf16x8_t ah = *reinterpret_cast<const bf16x8_t*>(base + offA + i * 1024);
+            const bf16x8_t al = *reinterpret_cast<const bf16x8_t*>(base + RING_PLANE + offA + i * 1024);
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, b[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, b[j], acc[i][j], 0, 0, 0);
         }
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int row = wm * 64 + i * 32 + (lane & 31);
-#pragma unroll
-            for (int ksub = 0; ksub < 2; ksub++) {
-                const int slot = row * 4 + ((2 * half + ksub) ^ ((row >> 1) & 3));
-                const bf16x8_t ah = *reinterpret_cast<const bf16x8_t*>(base + slot * 16);
-                const bf16x8_t al = *reinterpret_cast<const bf16x8_t*>(base + BM * 64 + slot * 16);
-#pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, b[j][ksub], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, b[j][ksub], acc[i][j], 0, 0, 0);
-                }
-            }
-        }
-        stage = stage + 1 == RS ? 0 : stage + 1;
+    };
+
+    // W of the first four steps into the register ring, the first converted at once
+    int4 w0 = loadW(stepBeg), w1 = loadW(stepBeg + 1), w2 = loadW(stepBeg + 2), w3 = loadW(stepBeg + 3);
+    asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    putW(w0, 0);
+    issueA(stepBeg, 0);
+    w0 = loadW(stepBeg + 4);
+    issueA(stepBeg + 1, 1);
+    int stage = 0;
+    // step s: A(s) and W(s+1) have landed; barrier; W(s+1) -> stage s+1; request W(s+5) and A(s+2); multiply stage s
+#define MG_RING_STEP(WS, S)                                                                          \
+    {                                                                                                \
+        asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)\n\ts_barrier" ::: "memory");                     \
+        const int s1 = stage + 1 == RS ? 0 : stage + 1;                                              \
+        const int s2 = s1 + 1 == RS ? 0 : s1 + 1;                                                    \
+        putW(WS, s1);                                                                                \
+        WS = loadW((S) + 5);                                                                         \
+        issueA((S) + 2, s2);                                                                         \
+        multiply(stage);                                                                             \
+        stage = s1;                                                                                  \
     }
+    for (int step = stepBeg; step < stepEnd; step += 4) {
+        MG_RING_STEP(w1, step)
+        MG_RING_STEP(w2, step + 1)
+        MG_RING_STEP(w3, step + 2)
+        MG_RING_STEP(w0, step + 3)
+    }
+#undef MG_RING_STEP
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the trailing reloads must not outlive the workgroup's LDS
+
+    // C layout of the 16 x 16 blocks: lane l holds column l%16, rows 4*(l/16) + e
+    const int mrow = m0 + wm * 64 + 4 * (lane >> 4);
     if (MODE == 3) {
-        const int n = n0 + wn * 32 + (lane & 31);
-        if (n < N) {
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const int jg = (jj >> 1) * 4 + (jj & 1);      // gate blocks 0, 1, 4, 5; the up values of the same columns in jg + 2
+            const int n = n0 + (wn * 2 + (jj >> 1)) * 32 + (jj & 1) * 16 + (lane & 15);
+            if (n >= N) continue;
             const float scg = p.seg[0].scales[n], scu = p.seg[1].scales[n];
             const float big = p.seg[0].bias ? p.seg[0].bias[n] : 0.f, biu = p.seg[1].bias ? p.seg[1].bias[n] : 0.f;
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int e = 0; e < 16; e++) {
-                    const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                for (int e = 0; e < 4; e++) {
+                    const int m = mrow + i * 16 + e;
                     if (m < T) {
-                        const float g = acc[i][0][e] * scg + big, u = acc[i][1][e] * scu + biu;
+                        const float g = acc[i][jg][e] * scg + big, u = acc[i][jg + 2][e] * scu + biu;
                         const float a = g * (1.0f / (1.0f + expf(-g))) * u;        // mongoose.cu:949-956
                         const unsigned short h = f32_to_bf16_rne(a);
                         const size_t o = tiled_index(m, n, N);
@@ -739,16 +854,16 @@ __global__ __launch_bounds__(1024) void gemm_q8_ring_kernel(GemmParams p) {
         return;
     }
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int nl = wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < 8; j++) {
+        const int nl = wn * 128 + j * 16 + (lane & 15);
         const int n = n0 + nl;
         if (MODE == 2) {
             float* dst = p.partial + ((size_t)blockIdx.y * T) * p.ldPartial + (size_t)nTile * BN + nl;
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int e = 0; e < 16; e++) {
-                    const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                for (int e = 0; e < 4; e++) {
+                    const int m = mrow + i * 16 + e;
                     if (m < T) dst[(size_t)m * p.ldPartial] = acc[i][j][e];
                 }
             continue;
@@ -757,10 +872,10 @@ __global__ __launch_bounds__(1024) void gemm_q8_ring_kernel(GemmParams p) {
         const float sc = sg.scales[n];
         const float bi = sg.bias ? sg.bias[n] : 0.f;
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+            for (int e = 0; e < 4; e++) {
+                const int m = mrow + i * 16 + e;
                 if (m < T) {
                     float v = acc[i][j][e] * sc + bi;
                     float* dst = sg.Y + (size_t)m * N + n;
@@ -773,7 +888,7 @@ __global__ __launch_bounds__(1024) void gemm_q8_ring_kernel(GemmParams p) {
 
 template <int MODE>
 static hipError_t launch_ring(const GemmParams& p, dim3 grid, hipStream_t s) {
-    constexpr int bytes = RS * RING_STAGE_BYTES;          // 120 KB of the CU's 160 KB
+    constexpr int bytes = RS * RING_STAGE_BYTES;          // 144 KB of the CU's 160 KB
     static bool raised = false;                            // the default cap on dynamic LDS is 64 KB
     if (!raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q8_ring_kernel<MODE>),
@@ -781,7 +896,7 @@ static hipError_t launch_ring(const GemmParams& p, dim3 grid, hipStream_t s) {
         if (e != hipSuccess) return e;
         raised = true;
     }
-    hipLaunchKernelGGL((gemm_q8_ring_kernel<MODE>), grid, dim3(1024), bytes, s, p);
+    hipLaunchKernelGGL((gemm_q8_ring_kernel<MODE>), grid, dim3(512), bytes, s, p);
     return hipGetLastError();
 }
 
@@ -1008,7 +1123,8 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
     constexpr int BMB = Q4 ? 128 : 256, NTB = Q4 ? 512 : 1024;
     const int ksteps = (p.K + BK - 1) / BK;
     p.splitK = 1; p.stepsPerSplit = ksteps;
-    if (!Q4 && p.T > 128 && p.nseg == 2 && !residual && p.nextSwiglu && p.nextHi && p.nextLo && p.seg[0].N == p.seg[1].N) {
+    const bool ringOk = p.K % 128 == 0;          // the ring kernel takes its K steps four at a time
+    if (!Q4 && ringOk && p.T > 128 && p.nseg == 2 && !residual && p.nextSwiglu && p.nextHi && p.nextLo && p.seg[0].N == p.seg[1].N) {
         // gate | up with enough 128-column tiles to fill the chip without splitting K: the GEMM's own
         // epilogue forms silu(gate) * up and writes its hi/lo split
         const int tiles = (p.seg[0].N + 127) / 128;
@@ -1041,10 +1157,11 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
             dim3 grid((unsigned)(((tiles + 7) / 8) * 8 * numM), 1);
             if (S > 1) {
                 p.stepsPerSplit = (ksteps + S - 1) / S;
+                if (!Q4 && ringOk) p.stepsPerSplit = (p.stepsPerSplit + 1) & ~1;      // 64-k steps: an even count = 32-k steps in fours
                 S = (ksteps + p.stepsPerSplit - 1) / p.stepsPerSplit;
                 grid.y = (unsigned)S;
                 p.splitK = S; p.ldPartial = tiles * 256;
-                if constexpr (Q4 != 0) {
+                if (Q4 || !ringOk) {
                     hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 2>), grid, dim3(NTB), 0, s, p);
                 } else {
                     hipError_t e = launch_ring<2>(p, grid, s);
@@ -1053,7 +1170,7 @@ static hipError_t launch_gemm_fmt(GemmParams& p, int residual, hipStream_t s) {
                 launch_reduce(p, 256, residual, s);
                 return hipGetLastError();
             }
-            if constexpr (Q4 != 0) {
+            if (Q4 || !ringOk) {
                 if (residual) hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 1>), grid, dim3(NTB), 0, s, p);
                 else hipLaunchKernelGGL((gemm_q8_bf16x2_kernel<Q4, BMB, 256, NTB, 0>), grid, dim3(NTB), 0, s, p);
                 return hipGetLastError();
