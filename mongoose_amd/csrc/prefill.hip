@@ -161,27 +161,37 @@ hipError_t launch_embed_rows(int kind, const void* table, const float* scales, c
 // ---------------------------------------------------------------------------
 // Causal attention over T query rows (mongoose.cu:251-353 for a training
 // sequence; here against the KV caches, query t at position pos0 + t), on the
-// bf16 matrix instruction with every fp32 operand split into two bf16 terms
-// (x = hi + lo, |x - hi - lo| <= 2^-16 |x|) and three products per pair of
-// operands (hi.hi + hi.lo + lo.hi; lo.lo is below 2^-16 of the result).
+// bf16 matrix instruction v_mfma_f32_16x16x32_bf16 with every fp32 operand
+// split into two bf16 terms (x = hi + lo, |x - hi - lo| <= 2^-16 |x|) and
+// three products per pair of operands (hi.hi + hi.lo + lo.hi; lo.lo is below
+// 2^-16 of the result).
 //
 // The cache rows are split once per layer by kv_split_kernel into planes the
 // matrix instruction reads as they lie: K hi / lo as [row][kvDim], and V hi /
-// lo transposed, [kvh * HD + d][row], the rows of each group of 16 in the order
-// 0-3, 8-11, 4-7, 12-15 (see the P operand below).  Rows past pos0 + T, up to
-// the next multiple of 32, are written as zeros.
+// lo transposed, [kvh * HD + d][row], the rows of each group of 32 in the order
+// the P operand holds them (below).  Rows past pos0 + T, up to the next
+// multiple of 32, are written as zeros.
 //
-// One workgroup = 32 queries of one head; its four waves take the 32-position
-// KV tiles in turn (tile w, w+4, ...) with their own running max / sum /
-// output and are combined at the end.  Arranged transposed, so that a lane
-// owns one query (C layout: lane l holds column l%32, rows 8*(i/4) + 4*(l/32)
-// + i%4 for i = 0..15):
-//   S^T[kpos][q] = K . Q^T    A = K rows (lane: row l%32, 8 d of half l/32), B = Q^T held in registers
-//   O^T[d][q]    = V^T . P^T  A = V^T rows, B = the S^T accumulator itself: as the B operand of step s2
-//                             a lane holds k slots j = 0..7 = accumulator registers 8*s2 + j, i.e. tile
-//                             positions 16*s2 + 8*(j/4) + 4*(l/32) + j%4 -- the order V^T is stored in.
+// A workgroup = 8 waves = 4 slots x 2 tile parities.  The slots are the query
+// heads of one KV head (4 of them; fewer heads a KV head: the slots are shared
+// out over neighbouring blocks of 16 queries instead), so all waves want the
+// same K / V tiles: each step brings two 32-position tiles into LDS by direct
+// global -> LDS loads (double-buffered: the next pair is requested before the
+// current one is multiplied), and every wave reads its operands from there.
+// A wave keeps its own running max / sum / output over the tiles of its
+// parity; the two parities of a slot are combined at the end.
+//
+// Transposed, so that the softmax statistics of a query stay in four lanes
+// (C layout of a 16 x 16 block: lane l holds column l%16, rows 4*(l/16) + e):
+//   S^T[kpos][q] = K . Q^T    A = K rows (lane: row l%16, 8 d of quarter l/16 of a 32-d step), B = Q^T in registers
+//   O^T[d][q]    = V^T . P^T  A = V^T rows, B = the S^T accumulators themselves: as the B operand a lane
+//                             holds k slots 8*(l/16) + j, j = 0..7, and it has S^T for tile positions
+//                             16*(j/4) + 4*(l/16) + j%4 -- the order V^T is stored in.
+// LDS: planes of 16 rows x 64 bytes (a 32-d step of 16 K rows; 32 positions of 16 V^T rows), the 16-byte
+// piece p of row r at p ^ ((r>>1)&3): the fragment reads (lane l: row l%16, piece l/16) are conflict-free.
 // ---------------------------------------------------------------------------
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ void split8(const float (&v)[8], bf16x8_t& h, bf16x8_t& l) {
     unsigned short hs[8], ls[8];
@@ -199,29 +209,36 @@ __device__ __forceinline__ void split8(const float (&v)[8], bf16x8_t& h, bf16x8_
     l = __builtin_bit_cast(bf16x8_t, ul);
 }
 
-// grid (rowsPad / 16, nKVHeads), HD threads: thread d of a workgroup takes column kvh * HD + d of 16 rows
+// grid (rowsPad / 32, nKVHeads, 2), HD threads: thread d takes column kvh * HD + d of 32 rows of K (z = 0) or V (z = 1)
 template <typename KVT>
 __global__ void kv_split_kernel(const KVT* Kc, const KVT* Vc, int rows, int kvDim, int HD, unsigned short* Khi,
                                 unsigned short* Klo, unsigned short* VThi, unsigned short* VTlo, int vtStride) {
     const int g = blockIdx.x, col = blockIdx.y * HD + threadIdx.x;
-    unsigned short vh[16], vl[16];
+    if (blockIdx.z == 0) {
+#pragma unroll 8
+        for (int i = 0; i < 32; i++) {
+            const int r = g * 32 + i;
+            const size_t o = (size_t)r * kvDim + col;
+            const float k = r < rows ? (float)Kc[o] : 0.f;
+            const unsigned short kh = f32_to_bf16_rne(k);
+            Khi[o] = kh;
+            Klo[o] = f32_to_bf16_rne(k - bf16_to_f32(kh));
+        }
+        return;
+    }
+    unsigned short vh[32], vl[32];
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-        const int r = g * 16 + i;
-        const size_t o = (size_t)r * kvDim + col;
-        const float k = r < rows ? (float)Kc[o] : 0.f;
-        const float v = r < rows ? (float)Vc[o] : 0.f;
-        const unsigned short kh = f32_to_bf16_rne(k);
-        Khi[o] = kh;
-        Klo[o] = f32_to_bf16_rne(k - bf16_to_f32(kh));
-        const int idx = 8 * ((i >> 2) & 1) + (i & 3) + 4 * (i >> 3);
+    for (int i = 0; i < 32; i++) {
+        const int r = g * 32 + i;
+        const float v = r < rows ? (float)Vc[(size_t)r * kvDim + col] : 0.f;
+        const int idx = 8 * ((i >> 2) & 3) + (i & 3) + 4 * (i >> 4);      // position i of the tile sits at k slot idx
         vh[idx] = f32_to_bf16_rne(v);
         vl[idx] = f32_to_bf16_rne(v - bf16_to_f32(vh[idx]));
     }
-    uint4* dh = reinterpret_cast<uint4*>(VThi + (size_t)col * vtStride + g * 16);
-    uint4* dl = reinterpret_cast<uint4*>(VTlo + (size_t)col * vtStride + g * 16);
+    uint4* dh = reinterpret_cast<uint4*>(VThi + (size_t)col * vtStride + g * 32);
+    uint4* dl = reinterpret_cast<uint4*>(VTlo + (size_t)col * vtStride + g * 32);
 #pragma unroll
-    for (int w = 0; w < 2; w++) {
+    for (int w = 0; w < 4; w++) {
         dh[w] = make_uint4(vh[8 * w] | ((unsigned)vh[8 * w + 1] << 16), vh[8 * w + 2] | ((unsigned)vh[8 * w + 3] << 16),
                            vh[8 * w + 4] | ((unsigned)vh[8 * w + 5] << 16), vh[8 * w + 6] | ((unsigned)vh[8 * w + 7] << 16));
         dl[w] = make_uint4(vl[8 * w] | ((unsigned)vl[8 * w + 1] << 16), vl[8 * w + 2] | ((unsigned)vl[8 * w + 3] << 16),
@@ -230,125 +247,164 @@ __global__ void kv_split_kernel(const KVT* Kc, const KVT* Vc, int rows, int kvDi
 }
 
 template <int HD>
-__global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const unsigned short* Khi, const unsigned short* Klo,
+__global__ __launch_bounds__(512) void prefill_attn_kernel(const float* q, const unsigned short* Khi, const unsigned short* Klo,
                                                           const unsigned short* VThi, const unsigned short* VTlo, int vtStride,
                                                           float* out, unsigned short* hi, unsigned short* lo, int T, int pos0,
-                                                          int dim, int kvDim, int nHeads, int nKVHeads) {
-    constexpr int NS = HD / 16;                // 16-wide steps of the head dimension
-    constexpr int DB = HD / 32;                // 32-wide blocks of the head dimension
-    __shared__ __attribute__((aligned(16))) float lds[4][HD * 33];
-    __shared__ float wm[4][32], wl[4][32];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int col = lane & 31, half = lane >> 5;
-    const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * 32, head = blockIdx.y;      // the longest causal ranges start first
-    const int kvh = head / (nHeads / nKVHeads);
-    const int myq = q0 + col;                           // this lane's query row
-    const int qpos = pos0 + min(myq, T - 1);            // its position (clamped rows are never stored)
+                                                          int dim, int kvDim, int nHeads, int nKVHeads, int HS, int parts) {
+    constexpr int NS = HD / 32;                // 32-wide steps of the head dimension
+    constexpr int DB = HD / 16;                // 16-wide blocks of the head dimension
+    constexpr int PL = HD * 64;                // bytes of one plane of a tile: 32 rows x HD bf16 (K), HD rows x 32 bf16 (V^T)
+    constexpr int TILE_BYTES = 4 * PL;         // K hi, K lo, V^T hi, V^T lo
+    constexpr int BUF_BYTES = 2 * TILE_BYTES;  // the two tiles of a step
+    constexpr int OS = 17;                     // row stride (floats) of a wave's [d][16 q] partial output
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    __shared__ float wm[8][16], wl[8][16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int slot = wave >> 1, ph = wave & 1;
+    const int QB = 4 / HS;                                   // blocks of 16 queries a workgroup covers
+    const int QH = nHeads / nKVHeads;
+    const int kvh = blockIdx.y / parts, part = blockIdx.y % parts;
+    const int hIn = part * HS + slot % HS;                   // this wave's query head within the KV head's group
+    const int qblk = ((int)gridDim.x - 1 - (int)blockIdx.x) * QB + slot / HS;     // the longest causal ranges start first
+    const int q0 = qblk * 16;
+    const bool active = hIn < QH && q0 < T;
+    const int head = kvh * QH + min(hIn, QH - 1);
+    const int fr = lane & 15, fq = lane >> 4;
+    const int myq = min(q0 + fr, T - 1);                    // this lane's query row (clamped rows are never stored)
+    const int qpos = pos0 + myq;
     const float scale = 1.0f / sqrtf((float)HD);
 
-    // Q^T operand: step s holds Q[myq][16 s + 8 half .. + 7]
+    // Q^T operand: step ds holds Q[myq][32 ds + 8 fq .. + 7]
     bf16x8_t qh[NS], ql[NS];
     {
-        const float* qr = q + (size_t)min(myq, T - 1) * dim + (size_t)head * HD + 8 * half;
+        const float* qr = q + (size_t)myq * dim + (size_t)head * HD + 8 * fq;
 #pragma unroll
-        for (int s = 0; s < NS; s++) {
-            const float4 a = *reinterpret_cast<const float4*>(qr + 16 * s), b = *reinterpret_cast<const float4*>(qr + 16 * s + 4);
+        for (int ds = 0; ds < NS; ds++) {
+            const float4 a = *reinterpret_cast<const float4*>(qr + 32 * ds), b = *reinterpret_cast<const float4*>(qr + 32 * ds + 4);
             const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-            split8(v, qh[s], ql[s]);
+            split8(v, qh[ds], ql[ds]);
         }
     }
-    float16_t o[DB];
+    float4_t o[DB];
 #pragma unroll
     for (int b = 0; b < DB; b++)
 #pragma unroll
-        for (int e = 0; e < 16; e++) o[b][e] = 0.f;
+        for (int e = 0; e < 4; e++) o[b][e] = 0.f;
     float m = -INFINITY, l = 0.f;
 
-    const int lastPos = pos0 + min(q0 + 31, T - 1);     // furthest position any query of the block sees
-    const int nTiles = lastPos / 32 + 1;
-    const size_t kcol = (size_t)kvh * HD + 8 * half;
-    for (int tile = wave; tile < nTiles; tile += 4) {
+    // the workgroup walks the tiles its furthest query sees; a wave skips the tiles past its own block's range
+    const int wgLast = pos0 + min(((int)gridDim.x - 1 - (int)blockIdx.x) * QB * 16 + QB * 16 - 1, T - 1);
+    const int wgTiles = wgLast / 32 + 1, nSteps = (wgTiles + 1) / 2;
+    const int myLast = pos0 + min(q0 + 15, T - 1);
+    const int myTiles = active ? myLast / 32 + 1 : 0;
+
+    // loads of a step: wave w brings plane w%4 (K hi, K lo, V^T hi, V^T lo) of tile w/4: DB wave-loads of 1 KB
+    const int ltile = wave >> 2, lplane = wave & 3;
+    const int lr = lane >> 2, lpiece = (lane & 3) ^ ((lr >> 1) & 3);
+    const unsigned short* lsrc = lplane == 0 ? Khi : lplane == 1 ? Klo : lplane == 2 ? VThi : VTlo;
+    auto issue = [&](int step, int buf) __attribute__((always_inline)) {
+        const int tile = min(2 * step + ltile, wgTiles - 1);
         const int t0 = tile * 32;
-        const unsigned short* kh = Khi + (size_t)(t0 + col) * kvDim + kcol;
-        const unsigned short* kl = Klo + (size_t)(t0 + col) * kvDim + kcol;
-        float16_t sT, sX;                                // hi.hi and the two cross terms: two chains for the matrix pipe
+        unsigned char* dst = lds + buf * BUF_BYTES + ltile * TILE_BYTES + lplane * PL;
 #pragma unroll
-        for (int e = 0; e < 16; e++) { sT[e] = 0.f; sX[e] = 0.f; }
-#pragma unroll
-        for (int s = 0; s < NS; s++) {
-            const bf16x8_t ah = *reinterpret_cast<const bf16x8_t*>(kh + 16 * s);
-            const bf16x8_t al = *reinterpret_cast<const bf16x8_t*>(kl + 16 * s);
-            sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, qh[s], sT, 0, 0, 0);
-            sX = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, ql[s], sX, 0, 0, 0);
-            sX = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, qh[s], sX, 0, 0, 0);
+        for (int i = 0; i < DB; i++) {
+            const unsigned short* src;
+            if (lplane < 2) src = lsrc + (size_t)(t0 + 16 * (i & 1) + lr) * kvDim + (size_t)kvh * HD + (i >> 1) * 32 + lpiece * 8;     // plane (ds = i/2, rows 16 (i%2) ..)
+            else src = lsrc + (size_t)(kvh * HD + 16 * i + lr) * vtStride + t0 + lpiece * 8;                                        // d block i
+            __builtin_amdgcn_global_load_lds(src, reinterpret_cast<int4*>(dst + i * 1024), 16, 0, 0);
         }
-        // causal mask, online softmax for this lane's query over the tile's 32 positions
+    };
+    const unsigned foff = fr * 64 + ((fq ^ ((fr >> 1) & 3)) * 16);
+
+    issue(0, 0);
+    for (int step = 0; step < nSteps; step++) {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");     // this step's tiles have landed; the other buffer is free
+        if (step + 1 < nSteps) issue(step + 1, (step + 1) & 1);
+        const int tile = 2 * step + ph;
+        if (tile >= myTiles) continue;
+        const int t0 = tile * 32;
+        const unsigned char* base = lds + (step & 1) * BUF_BYTES + ph * TILE_BYTES;
+        float4_t sT[2], sX[2];                           // hi.hi and the two cross terms: two chains for the matrix pipe
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) { sT[kb][e] = 0.f; sX[kb][e] = 0.f; }
+#pragma unroll
+        for (int ds = 0; ds < NS; ds++)
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                const bf16x8_t ah = *reinterpret_cast<const bf16x8_t*>(base + (ds * 2 + kb) * 1024 + foff);
+                const bf16x8_t al = *reinterpret_cast<const bf16x8_t*>(base + PL + (ds * 2 + kb) * 1024 + foff);
+                sT[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, qh[ds], sT[kb], 0, 0, 0);
+                sX[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, ql[ds], sX[kb], 0, 0, 0);
+                sX[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, qh[ds], sX[kb], 0, 0, 0);
+            }
+        // causal mask, online softmax: a query's 32 scores are in the four lanes l%16 = its column
+        float sv[8];
         float tmax = -INFINITY;
 #pragma unroll
-        for (int e = 0; e < 16; e++) {
-            const int kpos = t0 + 8 * (e >> 2) + 4 * half + (e & 3);
-            sT[e] = kpos <= qpos ? (sT[e] + sX[e]) * scale : -INFINITY;
-            tmax = fmaxf(tmax, sT[e]);
+        for (int j = 0; j < 8; j++) {
+            const int kpos = t0 + 16 * (j >> 2) + 4 * fq + (j & 3);
+            sv[j] = kpos <= qpos ? (sT[j >> 2][j & 3] + sX[j >> 2][j & 3]) * scale : -INFINITY;
+            tmax = fmaxf(tmax, sv[j]);
         }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
         const float mNew = fmaxf(m, tmax);
         const float corr = m == -INFINITY ? 0.f : expf(m - mNew);
         float psum = 0.f;
-        float pv[16];
 #pragma unroll
-        for (int e = 0; e < 16; e++) {
-            pv[e] = sT[e] == -INFINITY ? 0.f : expf(sT[e] - mNew);
-            psum += pv[e];
+        for (int j = 0; j < 8; j++) {
+            sv[j] = sv[j] == -INFINITY ? 0.f : expf(sv[j] - mNew);
+            psum += sv[j];
         }
+        psum += __shfl_xor(psum, 16, 64);
         psum += __shfl_xor(psum, 32, 64);
         l = l * corr + psum;
         m = mNew;
 #pragma unroll
         for (int b = 0; b < DB; b++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) o[b][e] *= corr;
+            for (int e = 0; e < 4; e++) o[b][e] *= corr;
+        bf16x8_t pH, pL;
+        split8(sv, pH, pL);
         // O^T += V^T . P^T
 #pragma unroll
-        for (int s2 = 0; s2 < 2; s2++) {
-            bf16x8_t ph, pl;
-            const float pp[8] = {pv[8 * s2], pv[8 * s2 + 1], pv[8 * s2 + 2], pv[8 * s2 + 3],
-                                 pv[8 * s2 + 4], pv[8 * s2 + 5], pv[8 * s2 + 6], pv[8 * s2 + 7]};
-            split8(pp, ph, pl);
-#pragma unroll
-            for (int b = 0; b < DB; b++) {
-                const size_t vo = (size_t)(kvh * HD + 32 * b + col) * vtStride + t0 + 16 * s2 + 8 * half;
-                const bf16x8_t vh = *reinterpret_cast<const bf16x8_t*>(VThi + vo);
-                const bf16x8_t vl = *reinterpret_cast<const bf16x8_t*>(VTlo + vo);
-                o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vh, ph, o[b], 0, 0, 0);
-                o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vh, pl, o[b], 0, 0, 0);
-                o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vl, ph, o[b], 0, 0, 0);
-            }
+        for (int b = 0; b < DB; b++) {
+            const bf16x8_t vh = *reinterpret_cast<const bf16x8_t*>(base + 2 * PL + b * 1024 + foff);
+            const bf16x8_t vl = *reinterpret_cast<const bf16x8_t*>(base + 3 * PL + b * 1024 + foff);
+            o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vh, pH, o[b], 0, 0, 0);
+            o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vh, pL, o[b], 0, 0, 0);
+            o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vl, pH, o[b], 0, 0, 0);
         }
     }
-    // ---- combine the four waves: O^T partials through LDS, [d][q] with row stride 33 ----
-    float* kt = lds[wave];
+    // ---- combine the two parities of every slot: O^T partials through LDS, [d][q] with row stride 17 ----
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");     // every wave is done with the tiles
+    float* part_ = reinterpret_cast<float*>(lds) + wave * (HD * OS);
 #pragma unroll
     for (int b = 0; b < DB; b++)
 #pragma unroll
-        for (int e = 0; e < 16; e++) kt[(32 * b + 8 * (e >> 2) + 4 * half + (e & 3)) * 33 + col] = o[b][e];
-    if (half == 0) { wm[wave][col] = m; wl[wave][col] = l; }
+        for (int e = 0; e < 4; e++) part_[(16 * b + 4 * fq + e) * OS + fr] = o[b][e];
+    if (fq == 0) { wm[wave][fr] = m; wl[wave][fr] = l; }
     __syncthreads();
-    for (int i = tid; i < 32 * HD; i += 256) {
-        const int qq = i / HD, d = i % HD;
-        if (q0 + qq >= T) continue;
-        const float M = fmaxf(fmaxf(wm[0][qq], wm[1][qq]), fmaxf(wm[2][qq], wm[3][qq]));
-        float num = 0.f, den = 0.f;
-#pragma unroll
-        for (int w = 0; w < 4; w++) {
-            const float wgt = wm[w][qq] == -INFINITY ? 0.f : expf(wm[w][qq] - M);
-            num = fmaf(wgt, lds[w][d * 33 + qq], num);
-            den = fmaf(wgt, wl[w][qq], den);
-        }
+    for (int i = tid; i < 4 * 16 * HD; i += 512) {
+        const int sl = i / (16 * HD), qq = (i / HD) % 16, d = i % HD;
+        const int hI = part * HS + sl % HS, qrow = (((int)gridDim.x - 1 - (int)blockIdx.x) * QB + sl / HS) * 16 + qq;
+        if (hI >= QH || qrow >= T) continue;
+        const int w0 = sl * 2, w1 = sl * 2 + 1;
+        const float M = fmaxf(wm[w0][qq], wm[w1][qq]);
+        const float g0 = wm[w0][qq] == -INFINITY ? 0.f : expf(wm[w0][qq] - M);
+        const float g1 = wm[w1][qq] == -INFINITY ? 0.f : expf(wm[w1][qq] - M);
+        const float* P0 = reinterpret_cast<const float*>(lds) + w0 * (HD * OS);
+        const float* P1 = reinterpret_cast<const float*>(lds) + w1 * (HD * OS);
+        const float num = fmaf(g1, P1[d * OS + qq], g0 * P0[d * OS + qq]);
+        const float den = fmaf(g1, wl[w1][qq], g0 * wl[w0][qq]);
         const float v = num / den;
-        if (out) out[(size_t)(q0 + qq) * dim + (size_t)head * HD + d] = v;
+        const int hd = (kvh * QH + hI) * HD + d;
+        if (out) out[(size_t)qrow * dim + hd] = v;
         if (hi) {            // the output projection's hi/lo split, written here instead of by a pass of its own
             const unsigned short h = f32_to_bf16_rne(v);
-            const size_t o2 = tiled_index(q0 + qq, head * HD + d, dim);
+            const size_t o2 = tiled_index(qrow, hd, dim);
             hi[o2] = h;
             lo[o2] = f32_to_bf16_rne(v - bf16_to_f32(h));
         }
@@ -358,6 +414,24 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* q, const
 size_t prefill_kv_split_bytes(int rows, int kvDim) {
     const size_t rowsPad = ((size_t)rows + 31) / 32 * 32;
     return 4 * rowsPad * (size_t)kvDim * sizeof(unsigned short);
+}
+
+template <int HD>
+static hipError_t launch_attn(dim3 grid, hipStream_t s, const float* q, const unsigned short* Khi, const unsigned short* Klo,
+                              const unsigned short* VThi, const unsigned short* VTlo, int vtStride, float* out, unsigned short* hi,
+                              unsigned short* lo, int T, int pos0, int dim, int kvDim, int nHeads, int nKVHeads, int HS, int parts) {
+    constexpr int bytes = 2 * 2 * 4 * HD * 64;             // two buffers of two tiles of four planes (HD = 128: 128 KB)
+    static_assert(8 * HD * 17 * 4 <= bytes, "the partial outputs reuse the tile buffers");
+    static bool raised = false;                            // the default cap on dynamic LDS is 64 KB
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn_kernel<HD>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    hipLaunchKernelGGL((prefill_attn_kernel<HD>), grid, dim3(512), bytes, s, q, Khi, Klo, VThi, VTlo, vtStride, out, hi, lo, T, pos0,
+                       dim, kvDim, nHeads, nKVHeads, HS, parts);
+    return hipGetLastError();
 }
 
 hipError_t launch_prefill_attention(const float* q, const void* Kc, const void* Vc, int kvHalf, void* kvSplit, float* out,
@@ -373,19 +447,20 @@ hipError_t launch_prefill_attention(const float* q, const void* Kc, const void* 
     const size_t plane = (size_t)rowsPad * kvDim;
     unsigned short* Khi = static_cast<unsigned short*>(kvSplit);
     unsigned short *Klo = Khi + plane, *VThi = Klo + plane, *VTlo = VThi + plane;
-    const dim3 sgrid((unsigned)(rowsPad / 16), (unsigned)nKVHeads);
+    const dim3 sgrid((unsigned)(rowsPad / 32), (unsigned)nKVHeads, 2);
     if (kvHalf) hipLaunchKernelGGL((kv_split_kernel<_Float16>), sgrid, dim3(headDim), 0, s, static_cast<const _Float16*>(Kc),
                                    static_cast<const _Float16*>(Vc), rows, kvDim, headDim, Khi, Klo, VThi, VTlo, rowsPad);
     else hipLaunchKernelGGL((kv_split_kernel<float>), sgrid, dim3(headDim), 0, s, static_cast<const float*>(Kc),
                             static_cast<const float*>(Vc), rows, kvDim, headDim, Khi, Klo, VThi, VTlo, rowsPad);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    dim3 grid((unsigned)((T + 31) / 32), (unsigned)nHeads);
-    if (headDim == 64)
-        hipLaunchKernelGGL((prefill_attn_kernel<64>), grid, dim3(256), 0, s, q, Khi, Klo, VThi, VTlo, rowsPad, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
-    else
-        hipLaunchKernelGGL((prefill_attn_kernel<128>), grid, dim3(256), 0, s, q, Khi, Klo, VThi, VTlo, rowsPad, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads);
-    return hipGetLastError();
+    // four slots a workgroup: the query heads of a KV head, or (fewer than 3 heads a KV head) heads x neighbouring query blocks
+    const int QH = nHeads / nKVHeads;
+    const int HS = QH >= 3 ? 4 : QH, QB = 4 / HS, parts = (QH + HS - 1) / HS;
+    const int qblocks = (T + 15) / 16;
+    dim3 grid((unsigned)((qblocks + QB - 1) / QB), (unsigned)(nKVHeads * parts));
+    if (headDim == 64) return launch_attn<64>(grid, s, q, Khi, Klo, VThi, VTlo, rowsPad, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads, HS, parts);
+    return launch_attn<128>(grid, s, q, Khi, Klo, VThi, VTlo, rowsPad, out, hi, lo, T, pos0, dim, kvDim, nHeads, nKVHeads, HS, parts);
 }
 
 // ---------------------------------------------------------------------------
@@ -693,7 +768,6 @@ __global__ __launch_bounds__(NT) void gemm_q8_bf16x2_kernel(GemmParams p) {
 constexpr int RK = 32, RS = 3;
 constexpr int RING_PLANE = 256 * 64;                      // 256 rows x 32 bf16
 constexpr int RING_STAGE_BYTES = 3 * RING_PLANE;          // A hi, A lo, W as bf16
-typedef float float4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ bf16x8_t cvt8_i8_bf16(int lo, int hi) {
     uint4 u;
