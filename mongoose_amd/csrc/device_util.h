@@ -133,6 +133,27 @@ __device__ __forceinline__ float half_bits_to_float(unsigned short h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
 
+// Q4_0 half block: s = sum_i act_i*nib_i - 8*sum_i act_i, then acc += s * f32(d)
+// (block form kernels/infer.metal:63-75; the -8 folded as kernels/q4_simd.metal:6-19
+// does).  Element order: low nibble of byte j = element j, high nibble = element
+// j+16 of the block (GGML).
+__device__ __forceinline__ float dot_q4_half(int2 w, float d, const float4 (&av)[4], float asum, float acc) {
+    float s = -8.0f * asum;
+    unsigned q;
+    q = (unsigned)w.x; s = dot4_nib(q & 0x0f0f0f0fu, av[0], s); s = dot4_nib((q >> 4) & 0x0f0f0f0fu, av[2], s);
+    q = (unsigned)w.y; s = dot4_nib(q & 0x0f0f0f0fu, av[1], s); s = dot4_nib((q >> 4) & 0x0f0f0f0fu, av[3], s);
+    return fmaf(s, d, acc);
+}
+// The sum of a chunk's 16 activations, in the order every Q4_0 path uses.
+__device__ __forceinline__ float chunk_act_sum(const float4 (&av)[4]) {
+    float4 t;
+    t.x = (av[0].x + av[1].x) + (av[2].x + av[3].x);
+    t.y = (av[0].y + av[1].y) + (av[2].y + av[3].y);
+    t.z = (av[0].z + av[1].z) + (av[2].z + av[3].z);
+    t.w = (av[0].w + av[1].w) + (av[2].w + av[3].w);
+    return (t.x + t.y) + (t.z + t.w);
+}
+
 // ---------------------------------------------------------------------------
 // Agent-scope accesses and the decode attention's row helpers
 // ---------------------------------------------------------------------------

@@ -11,7 +11,9 @@
 
 namespace mg {
 
-// Per-layer operands, a table in device memory (Q8 weights: int8 rows + per-row float scales).
+// Per-layer operands, a table in device memory.  Q8 weights: int8 rows + per-row float scales.  Q4_0 weights (all
+// seven matrices of every layer, split layout): the matrix pointer is the nibble plane [N, K/2] and the scale pointer
+// holds the address of the fp16 d plane [N, K/32] that follows it.
 struct FlowLayer {
     const float* g1;
     const float* g2;
@@ -48,6 +50,7 @@ struct FlowParams {
     int l0, l1;                  // layers [l0, l1)
     int nLayersTotal;            // layers the table and the exchange area hold
     int dim, kvDim, ffn, nHeads, nKVHeads, headDim, maxSeq;
+    int q4;                      // 0: Q8 matrices, 1: Q4_0 matrices in the split layout
     float eps;
     const StepState* state;      // position source (NULL -> posImm)
     int posImm;

@@ -155,12 +155,20 @@ __device__ __forceinline__ void poll_batch(const f4* const (&ptr)[PB], f4 (&v)[P
     }
 }
 
-// planar LDS layout of an activation vector for 16-weight chunks (as the matvec kernels use):
-// float4 k4 of the vector sits at (k4 & 3) * nch + (k4 >> 2); lane c reads a4[pl * nch + c], pl = 0..3
-__device__ __forceinline__ int slot4(int k4, int nch) { return (k4 & 3) * nch + (k4 >> 2); }
+// planar LDS layout of an activation vector for 16-weight chunks (as the matvec kernels use): lane c reads
+// a4[pl * nch + c], pl = 0..3.  Q8: a chunk is 16 consecutive weights, float4 k4 of the vector sits at
+// (k4 & 3) * nch + (k4 >> 2).  Q4_0: a chunk is half a block (8 bytes: low nibbles = elements 8h..8h+7 of the block,
+// high nibbles = elements 16+8h..16+8h+7), planes 0/1 its low-nibble float4s, planes 2/3 its high-nibble ones.
+template <bool Q4>
+__device__ __forceinline__ int slot4(int k4, int nch) {
+    if (!Q4) return (k4 & 3) * nch + (k4 >> 2);
+    const int blk = k4 >> 3, r4 = k4 & 7;
+    return ((r4 >> 2) * 2 + (r4 & 1)) * nch + blk * 2 + ((r4 >> 1) & 1);
+}
 __device__ __forceinline__ float4 tof4(f4 v) { return make_float4(v.x, v.y, v.z, v.w); }
 
 // x (optionally polled) -> LDS as x * gain; returns 1/rms.  Leaves with a barrier done.
+template <bool Q4>
 __device__ __forceinline__ float stage_rms(const float* x, bool polled, const float* gain, int K, float eps, float4* a4,
                                            float* red, Waiter& w) {
     const int K4 = K >> 2, nch = K >> 4, tid = threadIdx.x;
@@ -192,7 +200,7 @@ __device__ __forceinline__ float stage_rms(const float* x, bool polled, const fl
             const int i = base + u * FWG + tid;
             if (i < K4) {
                 ss += v[u].x * v[u].x + v[u].y * v[u].y + v[u].z * v[u].z + v[u].w * v[u].w;
-                a4[slot4(i, nch)] = make_float4(v[u].x * g[u].x, v[u].y * g[u].y, v[u].z * g[u].z, v[u].w * g[u].w);
+                a4[slot4<Q4>(i, nch)] = make_float4(v[u].x * g[u].x, v[u].y * g[u].y, v[u].z * g[u].z, v[u].w * g[u].w);
             }
         }
     }
@@ -206,6 +214,7 @@ __device__ __forceinline__ float stage_rms(const float* x, bool polled, const fl
 }
 
 // polled x -> LDS.  Leaves with a barrier done.
+template <bool Q4>
 __device__ __forceinline__ void stage_plain(const float* x, int K, float4* a4, Waiter& w) {
     const int K4 = K >> 2, nch = K >> 4, tid = threadIdx.x;
     const f4* x4 = reinterpret_cast<const f4*>(x);
@@ -219,43 +228,67 @@ __device__ __forceinline__ void stage_plain(const float* x, int K, float4* a4, W
 #pragma unroll
         for (int u = 0; u < PB; u++) {
             const int i = base + u * FWG + tid;
-            if (i < K4) a4[slot4(i, nch)] = tof4(v[u]);
+            if (i < K4) a4[slot4<Q4>(i, nch)] = tof4(v[u]);
         }
     }
     __syncthreads();
 }
 
-// chunks c0 + lane + i*64 of an int8 row (clamped inside the row: loads are unconditional)
-template <int CB>
-__device__ __forceinline__ void ld_row(const signed char* row, int nch, int lane, int c0, int4 (&wr)[CB]) {
-#pragma unroll
-    for (int i = 0; i < CB; i++) wr[i] = reinterpret_cast<const int4*>(row)[min(c0 + lane + i * 64, nch - 1)];
+// A weight row: Q8 16-byte chunks of int8; Q4_0 (split layout: all nibble groups of the matrix, then all fp16 d)
+// 8-byte half blocks and the row of d, one per two chunks.
+struct WRow { const signed char* w; const unsigned short* d; };
+template <bool Q4>
+__device__ __forceinline__ WRow wrow(const signed char* W, const float* aux, int r, int K) {
+    if (Q4) return WRow{W + (size_t)r * (K >> 1), reinterpret_cast<const unsigned short*>(aux) + (size_t)r * (K >> 5)};
+    return WRow{W + (size_t)r * K, nullptr};
 }
-template <int NR, int CB>
+// chunks c0 + lane + i*64 of a row (clamped inside the row: loads are unconditional); a Q4_0 chunk travels as
+// {nibbles, nibbles, d bits, -}
+template <bool Q4, int CB>
+__device__ __forceinline__ void ld_row(WRow row, int nch, int lane, int c0, int4 (&wr)[CB]) {
+#pragma unroll
+    for (int i = 0; i < CB; i++) {
+        const int c = min(c0 + lane + i * 64, nch - 1);
+        if (Q4) {
+            const int2 q = reinterpret_cast<const int2*>(row.w)[c];
+            wr[i] = make_int4(q.x, q.y, (int)row.d[c >> 1], 0);
+        } else {
+            wr[i] = reinterpret_cast<const int4*>(row.w)[c];
+        }
+    }
+}
+template <bool Q4, int NR, int CB>
 __device__ __forceinline__ void dot_rows(const int4 (&wr)[NR][CB], const float4* a4, int nch, int lane, int c0, float (&acc)[NR]) {
 #pragma unroll
     for (int i = 0; i < CB; i++) {
         const int c = c0 + lane + i * 64;
         if (c < nch) {
-            const float4 a0 = a4[c], a1 = a4[nch + c], a2 = a4[2 * nch + c], a3 = a4[3 * nch + c];
+            const float4 av[4] = {a4[c], a4[nch + c], a4[2 * nch + c], a4[3 * nch + c]};
+            if (Q4) {
+                const float asum = chunk_act_sum(av);
 #pragma unroll
-            for (int r = 0; r < NR; r++) {
-                float a = acc[r];
-                a = dot4_i8(wr[r][i].x, a0, a); a = dot4_i8(wr[r][i].y, a1, a);
-                a = dot4_i8(wr[r][i].z, a2, a); a = dot4_i8(wr[r][i].w, a3, a);
-                acc[r] = a;
+                for (int r = 0; r < NR; r++)
+                    acc[r] = dot_q4_half(make_int2(wr[r][i].x, wr[r][i].y), half_bits_to_float((unsigned short)wr[r][i].z), av, asum, acc[r]);
+            } else {
+#pragma unroll
+                for (int r = 0; r < NR; r++) {
+                    float a = acc[r];
+                    a = dot4_i8(wr[r][i].x, av[0], a); a = dot4_i8(wr[r][i].y, av[1], a);
+                    a = dot4_i8(wr[r][i].z, av[2], a); a = dot4_i8(wr[r][i].w, av[3], a);
+                    acc[r] = a;
+                }
             }
         }
     }
 }
 // the rest of rows longer than the prefetched batch
-template <int NR, int CB>
-__device__ __forceinline__ void dot_rows_tail(const signed char* const (&rows)[NR], const float4* a4, int nch, int lane, float (&acc)[NR]) {
+template <bool Q4, int NR, int CB>
+__device__ __forceinline__ void dot_rows_tail(const WRow (&rows)[NR], const float4* a4, int nch, int lane, float (&acc)[NR]) {
     for (int c0 = CB * 64; c0 < nch; c0 += CB * 64) {
         int4 wr[NR][CB];
 #pragma unroll
-        for (int r = 0; r < NR; r++) ld_row<CB>(rows[r], nch, lane, c0, wr[r]);
-        dot_rows<NR, CB>(wr, a4, nch, lane, c0, acc);
+        for (int r = 0; r < NR; r++) ld_row<Q4, CB>(rows[r], nch, lane, c0, wr[r]);
+        dot_rows<Q4, NR, CB>(wr, a4, nch, lane, c0, acc);
     }
 }
 
@@ -267,7 +300,8 @@ constexpr int NID = 8 / FWAVES;    // down rows a wave holds in flight
 // CBD: chunks a lane prefetches per row of K = dim (1: rows of up to 1024 weights in one batch, 2: up to 2048)
 // RING: gate | up and down stream their rows through a ring of register sets (rows of more than 2048 weights)
 // GQA: an attention workgroup takes all query heads of a KV head (contexts too long for one workgroup a query head)
-template <int HD, int CBD, bool RING, bool GQA>
+// Q4: the seven matrices of a layer are Q4_0 in the split layout (the table's scale pointers then hold the d planes)
+template <int HD, int CBD, bool RING, bool GQA, bool Q4>
 __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     extern __shared__ float4 a4[];                     // the staged activation vector, max(dim, ffn) floats
     __shared__ float red[FWAVES];
@@ -336,30 +370,30 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 // further items, and chunks past CBQ, are read where they are used.
                 constexpr int NPI = 1, CBQ = CBD;
                 int4 wr[NPI][2][CBQ];
-                const signed char* rows[NPI][2];
+                WRow rows[NPI][2];
                 int kind[NPI], r0[NPI], r1[NPI];
                 float e0[NPI], e1[NPI];                  // per-lane epilogue operands: lanes 0/1 scale and bias, lane 2 cos and sin
-                auto resolve = [&](int4 (&w)[2][CBQ], const signed char* (&rw)[2], int& kd, int& a0, int& a1, float& f0, float& f1, int item) {
+                auto resolve = [&](int4 (&w)[2][CBQ], WRow (&rw)[2], int& kd, int& a0, int& a1, float& f0, float& f1, int item) {
                     const signed char* Wm; const float* sc; const float* bias;
                     if (item < nq) { kd = 0; Wm = L.wq; sc = L.sq; bias = L.bq; const int jj = item % half; a0 = (item - jj) * 2 + jj; a1 = a0 + half; }
                     else if (item < nq + nk) { kd = 1; Wm = L.wk; sc = L.sk; bias = L.bk; const int i2 = item - nq; const int jj = i2 % half; a0 = (i2 - jj) * 2 + jj; a1 = a0 + half; }
                     else { kd = 2; Wm = L.wv; sc = L.sv; bias = L.bv; a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
-                    rw[0] = Wm + (size_t)a0 * dim; rw[1] = Wm + (size_t)a1 * dim;
-                    ld_row<CBQ>(rw[0], nchD, lane, 0, w[0]);
-                    ld_row<CBQ>(rw[1], nchD, lane, 0, w[1]);
+                    rw[0] = wrow<Q4>(Wm, sc, a0, dim); rw[1] = wrow<Q4>(Wm, sc, a1, dim);
+                    ld_row<Q4, CBQ>(rw[0], nchD, lane, 0, w[0]);
+                    ld_row<Q4, CBQ>(rw[1], nchD, lane, 0, w[1]);
                     f0 = 1.f; f1 = 0.f;
                     if (lane < 2) {
                         const int r = lane ? a1 : a0;
-                        f0 = sc[r];
+                        if (!Q4) f0 = sc[r];
                         if (bias) f1 = bias[r];
                     }
                     if (lane == 2 && kd < 2) { const int jj = a0 % half; f0 = p.cosRow[jj]; f1 = p.sinRow[jj]; }
                 };
                 // one item of every wave of the workgroup: dot, epilogue, the results out as runs by wave 0
-                auto finish = [&](const int4 (&w)[2][CBQ], const signed char* const (&rw)[2], int kd, float f0, float f1, float rs, int it) {
+                auto finish = [&](const int4 (&w)[2][CBQ], const WRow (&rw)[2], int kd, float f0, float f1, float rs, int it) {
                     float acc[2] = {0.f, 0.f};
-                    dot_rows<2, CBQ>(w, a4, nchD, lane, 0, acc);
-                    if (nchD > CBQ * 64) dot_rows_tail<2, CBQ>(rw, a4, nchD, lane, acc);
+                    dot_rows<Q4, 2, CBQ>(w, a4, nchD, lane, 0, acc);
+                    if (nchD > CBQ * 64) dot_rows_tail<Q4, 2, CBQ>(rw, a4, nchD, lane, acc);
                     acc[0] = wave_sum(acc[0]);
                     acc[1] = wave_sum(acc[1]);
                     float v = lane == 1 ? acc[1] : acc[0];
@@ -394,10 +428,10 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 };
 #pragma unroll
                 for (int q = 0; q < NPI; q++) {
-                    kind[q] = 0; r0[q] = 0; r1[q] = 0; e0[q] = 0.f; e1[q] = 0.f; rows[q][0] = L.wq; rows[q][1] = L.wq;
+                    kind[q] = 0; r0[q] = 0; r1[q] = 0; e0[q] = 0.f; e1[q] = 0.f; rows[q][0] = wrow<Q4>(L.wq, L.sq, 0, dim); rows[q][1] = rows[q][0];
                     if (gw + q * W < nI) resolve(wr[q], rows[q], kind[q], r0[q], r1[q], e0[q], e1[q], gw + q * W);
                 }
-                const float rs = stage_rms(xin, !first, L.g1, dim, p.eps, a4, red, wt);
+                const float rs = stage_rms<Q4>(xin, !first, L.g1, dim, p.eps, a4, red, wt);
                 FLOW_TRACE(1);
 #pragma unroll
                 for (int q = 0; q < NPI; q++)
@@ -599,20 +633,20 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             if (blockIdx.x * FWAVES < nI) {
                 int it = gw;
                 int4 wr[1][CBD];
-                const signed char* rows[1] = {L.wo};
+                WRow rows[1] = {wrow<Q4>(L.wo, L.so, 0, dim)};
                 float e0 = 0.f, e1 = 0.f;
                 auto resolve = [&](int item) {
-                    rows[0] = L.wo + (size_t)item * dim;
-                    ld_row<CBD>(rows[0], nchD, lane, 0, wr[0]);
+                    rows[0] = wrow<Q4>(L.wo, L.so, item, dim);
+                    ld_row<Q4, CBD>(rows[0], nchD, lane, 0, wr[0]);
                     if (lane == 0) {
-                        e0 = L.so[item];
+                        e0 = Q4 ? 1.f : L.so[item];
                         e1 = first ? xin[item] : poll1(xin + item, wt);         // there already if this workgroup staged it for q | k | v
                     }
                 };
                 if (it < nI) resolve(it);
                 // stage the attention output: merge the KV splits' partials (running maximum, as the split-KV combine)
                 if (grouped) {
-                    stage_plain(X + G.offAttn, dim, a4, wt);      // merged per head above
+                    stage_plain<Q4>(X + G.offAttn, dim, a4, wt);      // merged per head above
                 } else {
                 __syncthreads();
                 {
@@ -643,7 +677,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             mergeIn(a, ms, ls);
                         }
                         const float il = __builtin_amdgcn_rcpf(den);
-                        a4[slot4(i, nchD)] = make_float4(num.x * il, num.y * il, num.z * il, num.w * il);
+                        a4[slot4<Q4>(i, nchD)] = make_float4(num.x * il, num.y * il, num.z * il, num.w * il);
                     }
                 }
                 __syncthreads();
@@ -652,8 +686,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 for (; it < nI; it += W) {
                     if (it != gw) resolve(it);
                     float acc[1] = {0.f};
-                    dot_rows<1, CBD>(wr, a4, nchD, lane, 0, acc);
-                    if (nchD > CBD * 64) dot_rows_tail<1, CBD>(rows, a4, nchD, lane, acc);
+                    dot_rows<Q4, 1, CBD>(wr, a4, nchD, lane, 0, acc);
+                    if (nchD > CBD * 64) dot_rows_tail<Q4, 1, CBD>(rows, a4, nchD, lane, acc);
                     const float v = wave_sum(acc[0]);
                     if (it != gw) __syncthreads();              // outbuf is free again
                     store_runs(e1 + v * e0, 1, nI, it - gw, X + G.offX1, nullptr);
@@ -677,17 +711,17 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     auto issueStep = [&](int4 (&set)[2][CB], int st) {
                         const int sc = min(st, T - 1);                       // past the end: the last step again (uniform loop)
                         const int k = sc / nb, b = sc - k * nb;
-                        const size_t row = (size_t)(gw + k * W) * dim;
-                        ld_row<CB>(L.gate + row, nchD, lane, b * CB * 64, set[0]);
-                        ld_row<CB>(L.up + row, nchD, lane, b * CB * 64, set[1]);
+                        const int row = gw + k * W;
+                        ld_row<Q4, CB>(wrow<Q4>(L.gate, L.sgate, row, dim), nchD, lane, b * CB * 64, set[0]);
+                        ld_row<Q4, CB>(wrow<Q4>(L.up, L.sup, row, dim), nchD, lane, b * CB * 64, set[1]);
                     };
                     float sg = 0.f, su = 0.f;
                     if (T > 0) {
 #pragma unroll
                         for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
-                        if (lane < nItems) { const int r = gw + lane * W; sg = L.sgate[r]; su = L.sup[r]; }
+                        if (lane < nItems) { const int r = gw + lane * W; sg = Q4 ? 1.f : L.sgate[r]; su = Q4 ? 1.f : L.sup[r]; }
                     }
-                    const float rs = stage_rms(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                    const float rs = stage_rms<Q4>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
                     FLOW_TRACE(7);
                     float acc[2] = {0.f, 0.f};
                     float g = 0.f, u = 0.f;
@@ -698,7 +732,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             issueStep(ring[(j + RD - 1) % RD], st + RD - 1);
                             if (st < T) {                                        // uniform in the wave
                                 const int k = st / nb, b = st - k * nb;
-                                dot_rows<2, CB>(ring[j], a4, nchD, lane, b * CB * 64, acc);
+                                dot_rows<Q4, 2, CB>(ring[j], a4, nchD, lane, b * CB * 64, acc);
                                 if (b == nb - 1) {
                                     const float v0 = wave_sum(acc[0]), v1 = wave_sum(acc[1]);
                                     if (lane == k) { g = v0; u = v1; }
@@ -721,14 +755,14 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     for (int k = 0; k < NIB; k++) {
                         const int r = it0 + k * W;
                         if (r < nI) {                                           // uniform in the wave
-                            ld_row<CBD>(L.gate + (size_t)r * dim, nchD, lane, 0, wr[k][0]);
-                            ld_row<CBD>(L.up + (size_t)r * dim, nchD, lane, 0, wr[k][1]);
+                            ld_row<Q4, CBD>(wrow<Q4>(L.gate, L.sgate, r, dim), nchD, lane, 0, wr[k][0]);
+                            ld_row<Q4, CBD>(wrow<Q4>(L.up, L.sup, r, dim), nchD, lane, 0, wr[k][1]);
                         }
                     }
-                    if (lane < NIB) { const int r = min(it0 + lane * W, nI - 1); sg = L.sgate[r]; su = L.sup[r]; }
+                    if (lane < NIB) { const int r = min(it0 + lane * W, nI - 1); sg = Q4 ? 1.f : L.sgate[r]; su = Q4 ? 1.f : L.sup[r]; }
                 };
                 if (gw < nI) issue(gw);
-                const float rs = stage_rms(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                const float rs = stage_rms<Q4>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
                 FLOW_TRACE(7);
                 for (int it0 = gw; it0 < nI; it0 += NIB * W) {
                     if (it0 != gw) issue(it0);
@@ -737,11 +771,11 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     for (int k = 0; k < NIB; k++) {
                         float acc[2] = {0.f, 0.f};
                         if (it0 + k * W < nI) {                                 // uniform in the wave
-                            dot_rows<2, CBD>(wr[k], a4, nchD, lane, 0, acc);
+                            dot_rows<Q4, 2, CBD>(wr[k], a4, nchD, lane, 0, acc);
                             if (nchD > CBD * 64) {
                                 const int r = it0 + k * W;
-                                const signed char* rows[2] = {L.gate + (size_t)r * dim, L.up + (size_t)r * dim};
-                                dot_rows_tail<2, CBD>(rows, a4, nchD, lane, acc);
+                                const WRow rows[2] = {wrow<Q4>(L.gate, L.sgate, r, dim), wrow<Q4>(L.up, L.sup, r, dim)};
+                                dot_rows_tail<Q4, 2, CBD>(rows, a4, nchD, lane, acc);
                             }
                             acc[0] = wave_sum(acc[0]);
                             acc[1] = wave_sum(acc[1]);
@@ -771,15 +805,15 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     auto issueStep = [&](int4 (&set)[1][CB], int st) {
                         const int sc = min(st, T - 1);
                         const int k = sc / nb, b = sc - k * nb;
-                        ld_row<CB>(L.down + (size_t)(gw + k * W) * ffn, nchF, lane, b * CB * 64, set[0]);
+                        ld_row<Q4, CB>(wrow<Q4>(L.down, L.sdown, gw + k * W, ffn), nchF, lane, b * CB * 64, set[0]);
                     };
                     float e0 = 0.f, e1 = 0.f;
                     if (T > 0) {
-                        if (lane < nItems) { const int r = gw + lane * W; e0 = L.sdown[r]; e1 = poll1(X + G.offX1 + r, wt); }
+                        if (lane < nItems) { const int r = gw + lane * W; e0 = Q4 ? 1.f : L.sdown[r]; e1 = poll1(X + G.offX1 + r, wt); }
 #pragma unroll
                         for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
                     }
-                    stage_plain(X + G.offM, ffn, a4, wt);
+                    stage_plain<Q4>(X + G.offM, ffn, a4, wt);
                     FLOW_TRACE(9);
                     float acc[1] = {0.f};
                     float v = 0.f;
@@ -790,7 +824,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             issueStep(ring[(j + RD - 1) % RD], st + RD - 1);
                             if (st < T) {                                        // uniform in the wave
                                 const int k = st / nb, b = st - k * nb;
-                                dot_rows<1, CB>(ring[j], a4, nchF, lane, b * CB * 64, acc);
+                                dot_rows<Q4, 1, CB>(ring[j], a4, nchF, lane, b * CB * 64, acc);
                                 if (b == nb - 1) {
                                     const float v0 = wave_sum(acc[0]);
                                     if (lane == k) v = v0;
@@ -809,12 +843,12 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
 #pragma unroll
                     for (int k = 0; k < NID; k++) {
                         const int r = it0 + k * W;
-                        if (r < nI) ld_row<CBF>(L.down + (size_t)r * ffn, nchF, lane, 0, wr[k][0]);      // uniform in the wave
+                        if (r < nI) ld_row<Q4, CBF>(wrow<Q4>(L.down, L.sdown, r, ffn), nchF, lane, 0, wr[k][0]);      // uniform in the wave
                     }
-                    if (lane < NID) { const int r = min(it0 + lane * W, nI - 1); e0 = L.sdown[r]; e1 = poll1(X + G.offX1 + r, wt); }
+                    if (lane < NID) { const int r = min(it0 + lane * W, nI - 1); e0 = Q4 ? 1.f : L.sdown[r]; e1 = poll1(X + G.offX1 + r, wt); }
                 };
                 if (gw < nI) issue(gw);
-                stage_plain(X + G.offM, ffn, a4, wt);
+                stage_plain<Q4>(X + G.offM, ffn, a4, wt);
                 FLOW_TRACE(9);
                 for (int it0 = gw; it0 < nI; it0 += NID * W) {
                     if (it0 != gw) issue(it0);
@@ -823,10 +857,10 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     for (int k = 0; k < NID; k++) {
                         float acc[1] = {0.f};
                         if (it0 + k * W < nI) {
-                            dot_rows<1, CBF>(wr[k], a4, nchF, lane, 0, acc);
+                            dot_rows<Q4, 1, CBF>(wr[k], a4, nchF, lane, 0, acc);
                             if (nchF > CBF * 64) {
-                                const signed char* rows[1] = {L.down + (size_t)(it0 + k * W) * ffn};
-                                dot_rows_tail<1, CBF>(rows, a4, nchF, lane, acc);
+                                const WRow rows[1] = {wrow<Q4>(L.down, L.sdown, it0 + k * W, ffn)};
+                                dot_rows_tail<Q4, 1, CBF>(rows, a4, nchF, lane, acc);
                             }
                             acc[0] = wave_sum(acc[0]);
                         }
@@ -888,8 +922,10 @@ hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
         return hipErrorInvalidValue;
     const size_t lds = (size_t)(p.dim > p.ffn ? p.dim : p.ffn) * sizeof(float);
     const bool wide = p.dim > 1024, ring = p.dim > 2048, gqa = p.geo.gqa != 0;
-#define FLOW_LAUNCH(HDv, CBv, RGv, GQv) hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv>), dim3(grid), dim3(FWG), lds, s, p)
-#define FLOW_LAUNCH_G(HDv, CBv, RGv) do { if (gqa) FLOW_LAUNCH(HDv, CBv, RGv, true); else FLOW_LAUNCH(HDv, CBv, RGv, false); } while (0)
+#define FLOW_LAUNCH(HDv, CBv, RGv, GQv, Q4v) hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v>), dim3(grid), dim3(FWG), lds, s, p)
+#define FLOW_LAUNCH_G(HDv, CBv, RGv) do { \
+        if (p.q4) { if (gqa) FLOW_LAUNCH(HDv, CBv, RGv, true, true); else FLOW_LAUNCH(HDv, CBv, RGv, false, true); } \
+        else { if (gqa) FLOW_LAUNCH(HDv, CBv, RGv, true, false); else FLOW_LAUNCH(HDv, CBv, RGv, false, false); } } while (0)
     if (p.headDim == 64) {
         if (ring) FLOW_LAUNCH_G(64, 2, true);
         else if (wide) FLOW_LAUNCH_G(64, 2, false);

@@ -663,8 +663,11 @@ bool HIPFusedInference::flowEligible(int l0, int l1) const {
     for (int l = l0; l < l1; l++) {
         const LayerWeights& L = layers[l];
         if (!layerComplete(L) || !kCache[l] || !vCache[l]) return false;
+        // one format for all matrices of all layers: Q8, or Q4_0 in the split layout (whole blocks: rows of a multiple of 32)
         const DevMat* ms[7] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.gate, &L.up, &L.down};
-        for (const DevMat* m : ms) if (m->kind != WF_Q8) return false;
+        const int kind = layers[l0].wq.kind;
+        if (kind != WF_Q8 && kind != WF_Q4P) return false;
+        for (const DevMat* m : ms) if (m->kind != kind || (kind == WF_Q4P && m->cols % 32)) return false;
     }
     // one workgroup per CU, all resident at once; a (query head, KV split) per workgroup in the attention phase
     int cus = flowGrid;
@@ -710,9 +713,14 @@ int HIPFusedInference::ensureFlow() {
             F = FlowLayer{};
             F.g1 = L.norm1; F.g2 = L.norm2;
             auto w8 = [](const DevMat& m) { return static_cast<const signed char*>(m.w); };
+            // Q8: the per-row scales; Q4_0: the fp16 d plane, which follows the nibble plane [rows, cols/2]
+            auto aux = [](const DevMat& m) -> const float* {
+                if (m.kind != WF_Q4P) return m.scales;
+                return reinterpret_cast<const float*>(static_cast<const char*>(m.w) + (size_t)m.rows * (m.cols >> 1));
+            };
             F.wq = w8(L.wq); F.wk = w8(L.wk); F.wv = w8(L.wv); F.wo = w8(L.wo); F.gate = w8(L.gate); F.up = w8(L.up); F.down = w8(L.down);
-            F.sq = L.wq.scales; F.sk = L.wk.scales; F.sv = L.wv.scales; F.so = L.wo.scales;
-            F.sgate = L.gate.scales; F.sup = L.up.scales; F.sdown = L.down.scales;
+            F.sq = aux(L.wq); F.sk = aux(L.wk); F.sv = aux(L.wv); F.so = aux(L.wo);
+            F.sgate = aux(L.gate); F.sup = aux(L.up); F.sdown = aux(L.down);
             F.bq = L.bq; F.bk = L.bk; F.bv = L.bv;
             F.Kc = kCache[l]; F.Vc = vCache[l];
         }
@@ -756,6 +764,7 @@ int HIPFusedInference::enqueueLayersFlow(int l0, int l1, const StepState* st, in
     FlowParams p{};
     p.layers = dFlowLayers; p.l0 = l0; p.l1 = l1; p.nLayersTotal = nLayers;
     p.dim = dim; p.kvDim = kvDim; p.ffn = ffnDim; p.nHeads = nHeads; p.nKVHeads = nKVHeads; p.headDim = headDim; p.maxSeq = maxSeq;
+    p.q4 = layers[l0].wq.kind == WF_Q4P ? 1 : 0;
     p.eps = eps;
     p.state = st; p.posImm = posImm;
     const int half = headDim / 2;

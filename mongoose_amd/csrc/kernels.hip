@@ -108,17 +108,6 @@ template <> struct Fmt<WF_Q8> {
         return acc;
     }
 };
-// Q4_0 half block: s = sum_i act_i*nib_i - 8*sum_i act_i, then acc += s * f32(d)
-// (block form kernels/infer.metal:63-75; the -8 folded as kernels/q4_simd.metal:6-19
-// does).  Element order: low nibble of byte j = element j, high nibble = element
-// j+16 of the block (GGML).
-__device__ __forceinline__ float dot_q4_half(int2 w, float d, const float4 (&av)[4], float asum, float acc) {
-    float s = -8.0f * asum;
-    unsigned q;
-    q = (unsigned)w.x; s = dot4_nib(q & 0x0f0f0f0fu, av[0], s); s = dot4_nib((q >> 4) & 0x0f0f0f0fu, av[2], s);
-    q = (unsigned)w.y; s = dot4_nib(q & 0x0f0f0f0fu, av[1], s); s = dot4_nib((q >> 4) & 0x0f0f0f0fu, av[3], s);
-    return fmaf(s, d, acc);
-}
 template <> struct Fmt<WF_Q4P> {
     struct Row { const int2* qs; const unsigned short* d; };
     __device__ static Row row(const MvSeg& s, int r, int K) {

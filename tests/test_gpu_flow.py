@@ -7,6 +7,8 @@ their vectors over through an exchange area in device memory.
 * tokens through the launch == the oracle's, through graph replay and eager launches, and == the fused launches';
 * contexts that need several KV splits per head, up to every partial slot in use;
 * heads of 128 with grouped KV heads;
+* Q4_0 matrices (split layout, half-block chunks) through the same launch: every handed-over vector, tokens against
+  the oracle, rows of one and of two chunks a lane, the ring variant, biases;
 * a new context uses the launch; the trace diagnostic;
 * a wait that runs out: the launch still ends, the call reports it, the context continues with the fused launches.
 """
@@ -27,9 +29,10 @@ def _in_use(hipctx):
     return hipctx.FlowInUse()
 
 
-def test_every_handed_over_vector_matches_numpy(hip):
+@pytest.mark.parametrize("fmt", ["q8", "q4_0"])
+def test_every_handed_over_vector_matches_numpy(hip, fmt):
     s = H.with_layers(configs.TOY, 1)
-    m = H.Model(s, seed=1, maxSeq=72, eng=hip, threads=8, keep_dequant=True)
+    m = H.Model(s, seed=1, maxSeq=72, eng=hip, threads=8, keep_dequant=True, fmt=fmt)
     assert m.hip.SetExecMode(3) == 0
     D = {k: v.astype(np.float64) for k, v in m.dequant.items()}
     hd, half = s.headDim, s.headDim // 2
@@ -83,9 +86,10 @@ def test_every_handed_over_vector_matches_numpy(hip):
     m.close()
 
 
-def test_tokens_match_oracle_and_fused_launches(hip):
+@pytest.mark.parametrize("fmt", ["q8", "q4_0"])
+def test_tokens_match_oracle_and_fused_launches(hip, fmt):
     s = configs.TOY
-    m = H.Model(s, seed=3, maxSeq=72, eng=hip, threads=8)
+    m = H.Model(s, seed=3, maxSeq=72, eng=hip, threads=8, fmt=fmt)
     prompt = m.prompt(8)
     ref, _ = H.oracle_generate(m, prompt, 64)
     assert _in_use(m.hip), "a new context should use the persistent launch"
@@ -151,6 +155,46 @@ def test_kv_splits_heads_of_64(hip):
     m = H.Model(s, seed=11, maxSeq=16385, eng=hip, oracle=False)
     assert m.hip.SetExecMode(3) == 0
     assert not _in_use(m.hip)
+    m.close()
+
+
+def test_q4_0_qwen_geometry_and_ring(hip):
+    """Q4_0 matrices through the persistent launch at the 0.5B geometry (biases, 14 query heads on 2 KV heads, rows of
+    896 = 56 half-block chunks, fp16 embedding table) and at rows of 4096 weights, which stream through the register
+    ring: tokens against the oracle, then against the fused launches over positions that need several KV splits."""
+    s = H.with_layers(configs.QWEN_Q4, 2)._replace(name="qwen-q4-geom", vocab=2048)
+    m = H.Model(s, seed=21, maxSeq=400, eng=hip, threads=8)
+    print("flow: qwen geometry, Q4_0, 6 + 10 against the oracle", flush=True)
+    prompt = m.prompt(6)
+    ref, _ = H.oracle_generate(m, prompt, 10)
+    rc, t = m.hip.Generate(prompt, 10, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert _in_use(m.hip), "Q4_0 layers should run in the persistent launch"
+    assert t.tolist() == ref.tolist(), H.first_divergence(t, ref)
+    print("flow: qwen geometry, Q4_0, positions 300..340 (3 splits)", flush=True)
+    _modes_agree(m, m.prompt(300), 40, "Q4_0, 3 splits")
+    m.close()
+    s = H.with_layers(configs.LLAMA3_8B, 2)._replace(name="l3-q4-geom", ffnDim=4864, vocab=1024, tied=True)
+    m = H.Model(s, seed=22, maxSeq=200, eng=hip, threads=16, fmt="q4_0")
+    print("flow: rows of 4096 and 4864 weights (ring), Q4_0, 6 + 8 against the oracle", flush=True)
+    prompt = m.prompt(6)
+    ref, _ = H.oracle_generate(m, prompt, 8)
+    rc, t = m.hip.Generate(prompt, 8, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert _in_use(m.hip)
+    assert t.tolist() == ref.tolist(), H.first_divergence(t, ref)
+    _modes_agree(m, m.prompt(150), 30, "Q4_0 ring, 2 splits")
+    m.close()
+    # TinyLlama's row lengths (2048 = two chunks a lane, 5632 in the down projection), no ring
+    s = H.with_layers(configs.TINYLLAMA, 2)._replace(name="tiny-q4-geom", vocab=1024, tied=True)
+    m = H.Model(s, seed=23, maxSeq=64, eng=hip, threads=16, fmt="q4_0")
+    print("flow: rows of 2048 and 5632 weights, Q4_0, 6 + 8 against the oracle", flush=True)
+    prompt = m.prompt(6)
+    ref, _ = H.oracle_generate(m, prompt, 8)
+    rc, t = m.hip.Generate(prompt, 8, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert _in_use(m.hip)
+    assert t.tolist() == ref.tolist(), H.first_divergence(t, ref)
     m.close()
 
 

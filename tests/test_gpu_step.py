@@ -270,7 +270,8 @@ def test_streaming_matches_resident(hip):
         rc = st.StreamForwardToken(pos, h, s.nLayers, ptrs, sizes, logits)
         assert rc == 0, E.last_error()
         assert H.rel_err(logits, lg) < LOGIT_TOL, pos
-    # resident path on the same positions gives the same logits as streaming
+    # resident path on the same positions gives the same logits as streaming (which runs the fused launches)
+    assert m.hip.SetExecMode(1) == 0
     assert m.hip.ResetKV() == 0
     for pos in range(5):
         logits2 = np.empty(s.vocab, np.float32)
