@@ -313,7 +313,7 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds of CPU baseline work (0 = skip)")
     ap.add_argument("--profile-steps", type=int, default=20)
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--exec-mode", type=int, default=-1, choices=[-1, 0, 1, 2, 3],
+    ap.add_argument("--exec-mode", type=int, default=-1, choices=[-1, 0, 1, 2, 3, 4],
                     help="-1 = the library's automatic choice (default); 1 = fused launches; 2 = the same without the L2 prefetch by "
                          "the attention launch's idle workgroups; 3 = one persistent launch for all layers wherever the model allows it")
     ap.add_argument("--context", type=int, default=0,

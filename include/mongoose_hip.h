@@ -243,10 +243,13 @@ int mg_hidden_idx(mg_ctx* ctx);
  * also fetch the following matrices into L2 with its idle workgroups (for a GPU
  * shared with other work); 3 = all layers of a step in ONE persistent launch whose
  * workgroups hand their vectors over through device memory, wherever the model allows it
- * (Q8 weights, fp32 KV rows, heads of 64 or 128, a context of at most 128 x floor(CUs / nKVHeads)
- * positions -- an attention workgroup per query head and 128 positions where that covers the context,
- * else per KV head -- with at most 8 query heads a KV head; otherwise as mode 1).
- * A new context is in mode 3 (measured against mode 1: 0.5B shape 37 % more tokens per second, 1.1B
+ * (all matrices of the layers Q8, or all Q4_0; fp32 KV rows, heads of 64 or 128, a context of at most
+ * 128 x floor(CUs / nKVHeads) positions -- an attention workgroup per query head and 128 positions where
+ * that covers the context, else per KV head -- with at most 8 query heads a KV head; otherwise as mode 1).
+ * In mode 3, 32 of the launch's workgroups compute nothing and instead read the weights that the others
+ * will want next into the L2s, where a layer is small enough for that to pay (0.5B shape: 8 % faster);
+ * 4 = mode 3 with every workgroup computing (bit-identical results; for comparison).
+ * A new context is in mode 3 (measured against mode 1: 0.5B shape 50 % more tokens per second, 1.1B
  * shape 42 %, 8B shape 12 %, also at contexts of thousands of positions).
  * On every device one context at a time uses the persistent launch -- the first that needs it, until it is
  * destroyed or set to another mode; other contexts run the fused launches meanwhile (two such launches at

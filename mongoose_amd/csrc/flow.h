@@ -51,6 +51,7 @@ struct FlowParams {
     int nLayersTotal;            // layers the table and the exchange area hold
     int dim, kvDim, ffn, nHeads, nKVHeads, headDim, maxSeq;
     int q4;                      // 0: Q8 matrices, 1: Q4_0 matrices in the split layout
+    int nCompute;                // workgroups 0 .. nCompute-1 compute (geo is laid out for them), the rest of the grid prefetches
     float eps;
     const StepState* state;      // position source (NULL -> posImm)
     int posImm;
@@ -64,10 +65,14 @@ struct FlowParams {
     long long* trace;            // optional (diagnostic): wall-clock ticks [layer][FLOW_TRACE_SLOTS][workgroup], see FLOW_TRACE_NAMES
 };
 
-// Workgroups the launch needs at least (one per query head and KV split) for this shape.
+// Of `cus` workgroups that can be resident at once, how many the launch sets aside to prefetch weights into the L2s
+// (0 where that does not pay: layers too large for the L2s, or a phase that would need another round of the waves).
+int flow_prefetch_workgroups(int cus, size_t layerBytes, int dim, int kvDim, int ffn);
+// Computing workgroups the launch needs at least (one per query head and KV split) for this shape.
 int flow_min_grid(int nHeads, int nKVHeads, const FlowGeometry& g);
 bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads, int headDim);
-// grid workgroups of 512 threads, all of which must be resident at once (grid <= CUs x resident workgroups per CU).
+// grid workgroups of 512 threads, all of which must be resident at once (grid <= CUs x resident workgroups per CU);
+// grid - p.nCompute of them prefetch (0, or a multiple of 8 with nCompute a multiple of 8 as well).
 hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s);
 // Fills the blocks of layers [l0, l1) with the "not written yet" pattern.
 hipError_t launch_flow_reset(float* xchg, const FlowGeometry& g, int l0, int l1, hipStream_t s);

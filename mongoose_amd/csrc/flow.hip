@@ -292,6 +292,42 @@ __device__ __forceinline__ void dot_rows_tail(const WRow (&rows)[NR], const floa
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Prefetch role.  The last workgroups of the launch compute nothing: they read the rows that the computing
+// workgroups of their own XCD are going to want, one phase to one layer ahead of them, so that those find their
+// weights in the XCD's L2 instead of in HBM.  (The computing workgroups cannot do this for themselves: a CU's loads
+// come back in order, so the polls of a hand-over would queue behind their own prefetch.)  The dispatcher places
+// workgroup i on XCD i & 7; the eight waves of computing workgroup w take rows 8g .. 8g+7 of a matrix for every run
+// g with g % nC == w, so with nC a multiple of 8 run g belongs to XCD g & 7.
+// ---------------------------------------------------------------------------------------------------------------
+typedef int pfv4 __attribute__((ext_vector_type(4)));
+struct Prefetcher {
+    int x, rank, nRank, tid;     // XCD, this workgroup among the XCD's prefetchers, their number, thread
+    pfv4 sink;
+    // bytes [b0, b1) of base, 16 bytes a thread and step; b0 a multiple of 16, the tail rounded down
+    __device__ __forceinline__ void span(const char* base, size_t b0, size_t b1) {
+        b1 &= ~(size_t)15;
+        for (size_t o = b0 + (size_t)tid * 16; o < b1; o += (size_t)FWG * 16)
+            asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(sink) : "v"(base + o) : "memory");
+    }
+    // runs of `run` rows of rowBytes each; run g of the matrix goes to XCD g & 7, then to the XCD's prefetchers in turn
+    __device__ __forceinline__ void rows(const void* base, size_t rowBytes, int nRows, int run) {
+        if (!base) return;
+        const size_t total = (size_t)nRows * rowBytes, rb = (size_t)run * rowBytes;
+        const int nRuns = (nRows + run - 1) / run;
+        for (int g = x + 8 * rank; g < nRuns; g += 8 * nRank) {
+            const size_t b0 = (size_t)g * rb;
+            span(static_cast<const char*>(base), b0 & ~(size_t)15, b0 + rb < total ? b0 + rb : total);
+        }
+    }
+    // a small array every workgroup of the XCD reads (scales, gains, biases): the XCD's first prefetcher takes it whole
+    __device__ __forceinline__ void whole(const void* base, size_t bytes) {
+        if (!base || rank != 0) return;
+        span(static_cast<const char*>(base), 0, bytes);
+    }
+    __device__ __forceinline__ void drain() { asm volatile("s_waitcnt vmcnt(0)" : "+v"(sink) : : "memory"); }
+};
+
 constexpr int FLOW_MAX_ROUNDS = 8;   // rows of a matrix a wave takes at most (rounds of all waves over the matrix)
 constexpr int CBF = 6;       // ... per row of K = ffnDim (rows up to 6144 weights in one batch)
 constexpr int NIB = 24 / FWAVES;   // gate/up items (a gate row and its up row) a wave holds in flight
@@ -313,8 +349,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int gw = blockIdx.x * FWAVES + wave;         // this wave among all waves of the launch
-    const int W = gridDim.x * FWAVES;
+    const int nC = p.nCompute;                         // workgroups that compute; those after them prefetch
+    const int gw = blockIdx.x * FWAVES + wave;         // this wave among all computing waves of the launch
+    const int W = nC * FWAVES;
     // The rows of a workgroup's eight waves are consecutive (row = base + wave + k W), so their results go out as runs
     // of eight floats in one store instruction of wave 0 instead of eight single-float stores from eight waves: a line
     // of a handed-over vector is then written 4 times, not 32, while 256 workgroups keep re-reading it.
@@ -339,6 +376,63 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     const int pos = p.state ? p.state->pos : p.posImm;
     Waiter wt{p.limitTicks, p.err, false};
 
+    if ((int)blockIdx.x >= nC) {
+        // ---- prefetch role (see Prefetcher): per layer three jobs, each released by a vector of the layer before ----
+        const int pi = (int)blockIdx.x - nC;
+        Prefetcher pf{pi & 7, pi >> 3, ((int)gridDim.x - nC) >> 3, tid, {0, 0, 0, 0}};
+        const size_t rbD = Q4 ? dim >> 1 : dim, rbF = Q4 ? ffn >> 1 : ffn;      // bytes of a row of dim / of ffn weights
+        const size_t rdD = dim >> 4, rdF = ffn >> 4;                             // ... of its fp16 d values (Q4_0)
+        const int halfHd = HD >> 1;
+        unsigned lwp = layer_words(p.layers, p.l0, lane);
+        for (int l = p.l0; l < p.l1; l++) {
+            const FlowLayer L = unpack_layer(lwp);
+            if (l + 1 < p.l1) lwp = layer_words(p.layers, l + 1, lane);
+            const float* Xp = p.xchg + (size_t)(l - 1) * G.stride;               // the layer before (not for the first)
+            // (Measured at the 0.5B shape: releasing every job a phase earlier or later, and 24 to 48 prefetching
+            // workgroups, all give the same step time within 0.5 %; 16 are too few, 64 cost more than they bring.)
+            auto release = [&](int off) {
+                if (l == p.l0) return;
+                if (tid == 0) (void)poll1(Xp + off, wt);
+                __syncthreads();
+            };
+            release(G.offX1);              // the layer before is past its Wo: q | k | v and Wo of this one
+            {
+                const int nq = dim >> 1, nk = kvDim >> 1, nI = nq + 2 * nk;
+                for (int g = pf.x + 8 * pf.rank; g * 8 < nI; g += 8 * pf.nRank) {
+                    const int item = g * 8;
+                    const signed char* Wm; const float* aux; int a0, a1;
+                    if (item < nq) { Wm = L.wq; aux = L.sq; const int jj = item % halfHd; a0 = (item - jj) * 2 + jj; a1 = a0 + halfHd; }
+                    else if (item < nq + nk) { Wm = L.wk; aux = L.sk; const int i2 = item - nq; const int jj = i2 % halfHd; a0 = (i2 - jj) * 2 + jj; a1 = a0 + halfHd; }
+                    else { Wm = L.wv; aux = L.sv; a0 = (item - nq - nk) * 2; a1 = a0 + 8; }
+                    const char* wb = reinterpret_cast<const char*>(Wm);
+                    pf.span(wb, (size_t)a0 * rbD, (size_t)(a0 + 8) * rbD);
+                    pf.span(wb, (size_t)a1 * rbD, (size_t)(a1 + 8) * rbD);
+                    if (Q4) {
+                        const char* db = reinterpret_cast<const char*>(aux);
+                        pf.span(db, ((size_t)a0 * rdD) & ~(size_t)15, (size_t)(a0 + 8) * rdD);
+                        pf.span(db, ((size_t)a1 * rdD) & ~(size_t)15, (size_t)(a1 + 8) * rdD);
+                    }
+                }
+                if (!Q4) { pf.whole(L.sq, (size_t)dim * 4); pf.whole(L.sk, (size_t)kvDim * 4); pf.whole(L.sv, (size_t)kvDim * 4); }
+                pf.whole(L.bq, (size_t)dim * 4); pf.whole(L.bk, (size_t)kvDim * 4); pf.whole(L.bv, (size_t)kvDim * 4);
+                pf.whole(L.g1, (size_t)dim * 4);
+                pf.rows(L.wo, rbD, dim, 8);
+                if (Q4) pf.rows(L.so, rdD, dim, 8); else pf.whole(L.so, (size_t)dim * 4);
+            }
+            release(G.offM);               // ... past its gate | up: gate | up of this one
+            pf.rows(L.gate, rbD, ffn, 8);
+            pf.rows(L.up, rbD, ffn, 8);
+            if (Q4) { pf.rows(L.sgate, rdD, ffn, 8); pf.rows(L.sup, rdD, ffn, 8); }
+            else { pf.whole(L.sgate, (size_t)ffn * 4); pf.whole(L.sup, (size_t)ffn * 4); }
+            pf.whole(L.g2, (size_t)dim * 4);
+            release(G.offX2);              // ... done: the down projection of this one
+            pf.rows(L.down, rbF, dim, 8);
+            if (Q4) pf.rows(L.sdown, rdF, dim, 8); else pf.whole(L.sdown, (size_t)dim * 4);
+        }
+        pf.drain();
+        return;
+    }
+
     // attention geometry (decode attention of kernels.hip with one query head per workgroup): a thread group of 16
     // lanes holds a K/V row, a thread VU rows of its workgroup's tile of FLOW_TILE positions.  (Measured on the 0.5B
     // shape at 100-200 positions: tiles of 128 beat 256 by 5 %, and beat 64 and 32, whose extra partials cost more to
@@ -349,7 +443,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
 
     // timing trace (diagnostic): slot b of layer l, per workgroup, in ticks of the 100 MHz wall clock
 #define FLOW_TRACE(b) do { if (p.trace && tid == 0) \
-        p.trace[((size_t)(l - p.l0) * FLOW_TRACE_SLOTS + (b)) * gridDim.x + blockIdx.x] = wall_clock64(); } while (0)
+        p.trace[((size_t)(l - p.l0) * FLOW_TRACE_SLOTS + (b)) * nC + blockIdx.x] = wall_clock64(); } while (0)
     // the exchange area as a buffer resource: agent-scope loads that the compiler keeps track of (used where many are
     // wanted in flight together)
     const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(p.xchg, 0, (int)((size_t)p.nLayersTotal * G.stride * 4), 0x00020000);
@@ -446,7 +540,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
         FLOW_TRACE(2);
         // ------------------------------------------------------------------ attention: one (head, KV split) per workgroup
         // grouped only while a workgroup per query head and split would not fit the launch (positions far into a long context)
-        const bool grouped = GQA && p.nHeads * (pos / TILE + 1) > (int)gridDim.x;
+        const bool grouped = GQA && p.nHeads * (pos / TILE + 1) > nC;
         {
             const int nsplit = pos / TILE + 1;
             const int QH = grouped ? p.nHeads / p.nKVHeads : 1;        // query heads of this workgroup
@@ -902,6 +996,20 @@ FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int nKVHeads
     return g;
 }
 
+// Of `cus` resident workgroups, how many prefetch instead of computing (a multiple of 8: the same number on every
+// XCD).  They pay where a layer is a chain of latencies rather than a stream of bytes: a layer's share of an XCD must
+// fit its 4 MB L2 beside the share in use (beyond that the prefetched lines push each other out: 1.1B shape 0.453 ->
+// 0.494 ms/token with them), and no phase may need more rounds of the computing waves than it would with all
+// workgroups computing (8B shape: eight rounds of gate | up instead of seven).  layerBytes: weights of one layer.
+int flow_prefetch_workgroups(int cus, size_t layerBytes, int dim, int kvDim, int ffn) {
+    const int n = 32;
+    if (cus < 128 || cus % 8 || layerBytes / 8 > ((size_t)5 << 19)) return 0;       // 2.5 MB an XCD
+    auto rounds = [](int items, int wgs) { return (items + wgs * FWAVES - 1) / (wgs * FWAVES); };
+    const int items[3] = {dim / 2 + kvDim, dim, ffn};                               // q | k | v pairs, Wo / down rows, gate | up rows
+    for (int it : items) if (rounds(it, cus - n) != rounds(it, cus)) return 0;
+    return n;
+}
+
 int flow_min_grid(int nHeads, int nKVHeads, const FlowGeometry& g) { return (g.gqa ? nKVHeads : nHeads) * g.smax; }
 // one workgroup per (query head, tile): the slots cover the context
 bool flow_context_fits(int maxSeq, const FlowGeometry& g) { return (long long)FLOW_TILE * g.smax >= maxSeq; }
@@ -916,9 +1024,11 @@ bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads,
 
 hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
     if (!flow_shape_supported(p.dim, p.kvDim, p.ffn, p.nHeads, p.nKVHeads, p.headDim)) return hipErrorInvalidValue;
-    if (p.l0 < 0 || p.l1 <= p.l0 || p.l1 > p.nLayersTotal || grid < flow_min_grid(p.nHeads, p.nKVHeads, p.geo) ||
+    const int nC = p.nCompute;
+    if (nC <= 0 || nC > grid || ((grid - nC) && (nC % 8 || (grid - nC) % 8))) return hipErrorInvalidValue;
+    if (p.l0 < 0 || p.l1 <= p.l0 || p.l1 > p.nLayersTotal || nC < flow_min_grid(p.nHeads, p.nKVHeads, p.geo) ||
         !flow_context_fits(p.maxSeq, p.geo) || !p.layers || !p.xchg || !p.err || !p.hidden ||
-        (p.ffn + grid * FWAVES - 1) / (grid * FWAVES) > FLOW_MAX_ROUNDS || (size_t)p.nLayersTotal * p.geo.stride * 4 >= (1ull << 31))
+        (p.ffn + nC * FWAVES - 1) / (nC * FWAVES) > FLOW_MAX_ROUNDS || (size_t)p.nLayersTotal * p.geo.stride * 4 >= (1ull << 31))
         return hipErrorInvalidValue;
     const size_t lds = (size_t)(p.dim > p.ffn ? p.dim : p.ffn) * sizeof(float);
     const bool wide = p.dim > 1024, ring = p.dim > 2048, gqa = p.geo.gqa != 0;

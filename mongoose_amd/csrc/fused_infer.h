@@ -94,7 +94,13 @@ public:
     // 0: one launch per reference op; 1: fused launches; 2: fused, attention launches without the L2 prefetch
     // helpers; 3: all layers of a step in one persistent launch where the model allows it (else as 1).
     int execMode = 3;
-    void SetExecMode(int mode) { if (mode != execMode) invalidateGraphs(); execMode = mode; if (mode != 3) releaseFlow(); }
+    void SetExecMode(int mode) {
+        if (mode != execMode) invalidateGraphs();
+        if ((mode == 3 || mode == 4) && mode != execMode) flowRegeometry();    // the two differ in the launch's geometry
+        execMode = mode;
+        if (mode != 3 && mode != 4) releaseFlow();
+    }
+    void flowRegeometry();
     void releaseFlow();
 
     // shape
@@ -174,10 +180,12 @@ private:
     FlowLayer* dFlowLayers = nullptr;
     int* dFlowErr = nullptr;
     int* hFlowErr = nullptr;        // pinned
-    int flowGrid = 0;
+    int flowGrid = 0;         // workgroups of the persistent launch (one per CU)
+    int flowCompute = 0;      // ... of which compute (the others prefetch weights)
     bool flowTableDirty = true;
     bool flowBroken = false;        // a wait ran into its limit once: the separate launches are used from then on
     bool flowEligible(int l0, int l1) const;
+    int flowComputeWgs(int cus) const;
     int ensureFlow();
     int enqueueLayersFlow(int l0, int l1, const StepState* st, int posImm, bool resetFirst);
     int checkFlowError();

@@ -555,7 +555,7 @@ MvParams HIPFusedInference::downParams(const LayerWeights& L) const {
 // launch before): it need not be in by the end of this launch.
 void HIPFusedInference::planPrefetch(const LayerWeights& L, const LayerWeights* next, int layer, PfJob& job) const {
     job = PfJob{};
-    if (execMode != 1 && execMode != 3) return;
+    if (execMode != 1 && execMode != 3 && execMode != 4) return;
     const size_t budget = (size_t)12 << 20;       // measured: 10.6 MB make the attention launch 0.3 us longer, 15 MB 3 us
     const size_t l2 = (size_t)24 << 20;           // of 8 x 4 MB
     const LayerWeights* N = nullptr;
@@ -655,8 +655,38 @@ void HIPFusedInference::releaseFlow() {
     for (auto& o : g_flowOwner) if (o == this) o = nullptr;
 }
 
+// Modes 3 and 4 lay the launch out for different numbers of computing workgroups: drop what was sized for the other
+// (ensureFlow builds it again).
+void HIPFusedInference::flowRegeometry() {
+    if (!dFlowLayers) return;
+    if (stream) (void)hipStreamSynchronize(stream);
+    (void)hipFree(dFlowLayers); dFlowLayers = nullptr;
+    if (flowXchg) { (void)hipFree(flowXchg); flowXchg = nullptr; }
+    if (dFlowErr) { (void)hipFree(dFlowErr); dFlowErr = nullptr; }
+    if (hFlowErr) { (void)hipHostFree(hFlowErr); hFlowErr = nullptr; }
+    if (flowTrace) { (void)hipFree(flowTrace); flowTrace = nullptr; }
+    flowGrid = 0; flowCompute = 0;
+}
+
+// Of cus resident workgroups, how many compute: all but the prefetchers where the attention phase (one workgroup per
+// head and KV split) then still covers the context, else all of them; 0 if the launch cannot cover it at all.
+int HIPFusedInference::flowComputeWgs(int cus) const {
+    size_t layerBytes = 0;
+    if (!layers.empty()) {
+        const LayerWeights& L = layers[0];
+        layerBytes = L.wq.bytes + L.wk.bytes + L.wv.bytes + L.wo.bytes + L.gate.bytes + L.up.bytes + L.down.bytes;
+    }
+    const int pf = execMode == 4 ? 0 : flow_prefetch_workgroups(cus, layerBytes, dim, kvDim, ffnDim);
+    const int tries[2] = {cus - pf, cus};
+    for (int nC : tries) {
+        const FlowGeometry g = flow_geometry(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim, maxSeq, nC);
+        if (flow_min_grid(nHeads, nKVHeads, g) <= nC && flow_context_fits(maxSeq, g)) return nC;
+    }
+    return 0;
+}
+
 bool HIPFusedInference::flowEligible(int l0, int l1) const {
-    if (execMode != 3 || flowBroken || kvHalf) return false;
+    if ((execMode != 3 && execMode != 4) || flowBroken || kvHalf) return false;
     if (!flow_shape_supported(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim)) return false;
     if (l1 > nLayers) l1 = nLayers;
     if (l0 < 0 || l0 >= l1) return false;
@@ -677,8 +707,7 @@ bool HIPFusedInference::flowEligible(int l0, int l1) const {
         if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) { (void)hipGetLastError(); return false; }
         cus = prop.multiProcessorCount;
     }
-    const FlowGeometry g = flow_geometry(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim, maxSeq, cus);
-    if (!(flow_min_grid(nHeads, nKVHeads, g) <= cus && flow_context_fits(maxSeq, g))) return false;
+    if (flowComputeWgs(cus) == 0) return false;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return false; }
     return claim_flow(this, dev);
@@ -691,7 +720,8 @@ int HIPFusedInference::ensureFlow() {
         HIPCHK(hipGetDevice(&dev));
         HIPCHK(hipGetDeviceProperties(&prop, dev));
         flowGrid = prop.multiProcessorCount;
-        flowGeo = flow_geometry(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim, maxSeq, flowGrid);
+        flowCompute = flowComputeWgs(flowGrid);
+        flowGeo = flow_geometry(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim, maxSeq, flowCompute);
         void* v = nullptr;
         HIPCHK(hipMalloc(&v, sizeof(FlowLayer) * (size_t)nLayers));
         dFlowLayers = static_cast<FlowLayer*>(v);
@@ -737,9 +767,9 @@ int HIPFusedInference::ensureFlow() {
 int HIPFusedInference::FlowTrace(int enable, long long* out, size_t cap, int* dims) {
     if (!flowEligible(0, nLayers)) { set_error("flow trace: the persistent launch is not in use for this model (exec mode, weight kinds, shape)"); return MG_E_STATE; }
     if (int rc = ensureFlow()) return rc;
-    const size_t n = (size_t)nLayers * FLOW_TRACE_SLOTS * (size_t)flowGrid;
+    const size_t n = (size_t)nLayers * FLOW_TRACE_SLOTS * (size_t)flowCompute;
     HIPCHK(hipStreamSynchronize(stream));
-    if (dims) { dims[0] = nLayers; dims[1] = FLOW_TRACE_SLOTS; dims[2] = flowGrid; }
+    if (dims) { dims[0] = nLayers; dims[1] = FLOW_TRACE_SLOTS; dims[2] = flowCompute; }
     if (enable && !flowTrace) {
         void* v = nullptr;
         HIPCHK(hipMalloc(&v, sizeof(long long) * n));
@@ -765,6 +795,7 @@ int HIPFusedInference::enqueueLayersFlow(int l0, int l1, const StepState* st, in
     p.layers = dFlowLayers; p.l0 = l0; p.l1 = l1; p.nLayersTotal = nLayers;
     p.dim = dim; p.kvDim = kvDim; p.ffn = ffnDim; p.nHeads = nHeads; p.nKVHeads = nKVHeads; p.headDim = headDim; p.maxSeq = maxSeq;
     p.q4 = layers[l0].wq.kind == WF_Q4P ? 1 : 0;
+    p.nCompute = flowCompute;
     p.eps = eps;
     p.state = st; p.posImm = posImm;
     const int half = headDim / 2;
@@ -1513,7 +1544,7 @@ int mg_swap_hidden_buffer(mg_ctx* c) { CTX(c); return f->SwapHiddenBuffer(); }
 int mg_hidden_idx(mg_ctx* c) { CTX(c); return f->hiddenIdx; }
 int mg_set_exec_mode(mg_ctx* c, int mode) {
     CTX(c);
-    if (mode < 0 || mode > 3) { mg::set_error("exec mode must be 0, 1, 2 or 3"); return MG_E_ARG; }
+    if (mode < 0 || mode > 4) { mg::set_error("exec mode must be 0, 1, 2, 3 or 4"); return MG_E_ARG; }
     f->SetExecMode(mode);
     return MG_OK;
 }

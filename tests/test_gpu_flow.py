@@ -198,6 +198,43 @@ def test_q4_0_qwen_geometry_and_ring(hip):
     m.close()
 
 
+@pytest.mark.parametrize("fmt", ["q8", "q4_0"])
+def test_prefetching_workgroups_change_nothing(hip, fmt):
+    """Exec mode 3 sets 32 workgroups of the launch aside to read the coming weights into the L2s (0.5B geometry: a layer
+    fits); mode 4 lets every workgroup compute.  A row is multiplied by one wave in the same order either way, so the
+    logits are identical bit for bit, at one KV split and at several."""
+    s = H.with_layers(configs.QWEN if fmt == "q8" else configs.QWEN_Q4, 3)._replace(vocab=2048)
+    m = H.Model(s, seed=31, maxSeq=400, eng=hip, oracle=False)
+    prompt = m.prompt(300)
+    outs = {}
+    for mode in (3, 4):
+        assert m.hip.SetExecMode(mode) == 0
+        assert m.hip.ResetKV() == 0
+        assert _in_use(m.hip)
+        logits = np.empty(s.vocab, np.float32)
+        res = []
+        for pos in range(300):
+            last = pos in (0, 1, 127, 128, 298, 299)
+            rc, nxt = m.hip.DecodeToken(int(prompt[pos]), pos, logits if last else None)
+            assert rc == 0, E.last_error()
+            if last:
+                res.append((nxt, logits.copy()))
+        outs[mode] = res
+    for (n3, l3), (n4, l4) in zip(outs[3], outs[4]):
+        assert n3 == n4 and np.array_equal(l3, l4)
+    # and through graph replay after the switch back
+    assert m.hip.SetExecMode(3) == 0
+    assert m.hip.ResetKV() == 0
+    rc, t3 = m.hip.Generate(prompt[:8], 24, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert m.hip.SetExecMode(4) == 0
+    assert m.hip.ResetKV() == 0
+    rc, t4 = m.hip.Generate(prompt[:8], 24, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert t3.tolist() == t4.tolist()
+    m.close()
+
+
 def test_heads_of_128_grouped_kv(hip):
     """Llama-3-8B attention geometry (32 query heads of 128 on 8 KV heads, dim 4096: rows of two chunks a lane), 2
     layers, FFN and vocabulary cut: 8 partial slots, tile 128."""
