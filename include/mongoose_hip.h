@@ -98,6 +98,22 @@ void mongoose_q4_0_matvec(const float* act, const void* w_q4_0, float* out, int 
 void mongoose_q4_0_repack(const void* w_q4_0, void* planar, int N, int K, void* stream);
 void mongoose_q4_0_matvec_planar(const float* act, const void* planar, float* out, int N, int K, void* stream);
 
+/* The integer ("dp4a") forms of the Q4_0 matvec: kernels.go:66-70 (typedefs, same argument order), wrappers
+ * kernels.go:985-1017, dispatch cuda_fused_infer_q4.go:611-673.  The reference's CUDA bodies of these five are not
+ * in its tree; its Go side fixes the calling sequence and the scratch size, (K/32)*40 bytes
+ * (cuda_fused_infer.go:176), "Q8_1 blocks" (kernels.go:993).  Here a block of 32 activations is
+ *     { float d = max|x|/127;  float s = d * sum(q);  int8 q[32] = round-half-away(x/d) }      (40 bytes)
+ * and a row of block_q4_0 weights against it is GGML's vec_dot_q4_0_q8_1,
+ *     out[r] = sum_b f32(d4) * (d8 * sum_i nib_i * q_i - 8 * s8),
+ * on the packed int8 dot instruction.  Results differ from mongoose_q4_0_matvec by the activation rounding only
+ * (about 1e-2 relative on N(0,1) activations).  q8 buffers: 8-byte aligned, (K/32)*40 bytes a vector; batch forms
+ * take B contiguous vectors and write out[B, N]. */
+void mongoose_q8_quantize_act(const float* act, void* q8_out, int K, void* stream);
+void mongoose_q8_quantize_act_batch(const float* acts, void* q8_out, int K, int B, void* stream);
+void mongoose_q4_0_matvec_dp4a(const float* act, const void* w_q4_0, float* out, int N, int K, void* q8_scratch, void* stream);
+void mongoose_q4_0_matvec_dp4a_preq(const void* w_q4_0, const void* q8_act, float* out, int N, int K, void* stream);
+void mongoose_q4_0_matvec_dp4a_batch(const void* w_q4_0, const void* q8_acts, float* out, int N, int K, int B, void* stream);
+
 /* kernels.go:31, mongoose.cu:991-1013.  In place on x[seqLen, dim]; rotate-half
  * pairs (j, j+headDim/2); row `pos` of x uses table row `pos`. */
 void mongoose_rope(float* x, const float* cosTab, const float* sinTab, int seqLen, int dim, int headDim, int nHeads, void* stream);
@@ -259,6 +275,15 @@ int mg_hidden_idx(mg_ctx* ctx);
  * and the context continues with the fused launches.  All modes give the same results to
  * rounding. */
 int mg_set_exec_mode(mg_ctx* ctx, int mode);
+
+/* q4Matvec / q4MatvecPreq / q8QuantizeAct, cuda_fused_infer_q4.go:611-673: in the op-by-op loop (exec mode 0; any
+ * other mode: MG_E_STATE) Q4_0 matrices are multiplied in the integer form -- the activation vector quantized to
+ * int8 blocks (once for q, k, v and once for gate, up, as :161-173 and :208-212 do), then the packed int8 dot
+ * products of mongoose_q4_0_matvec_dp4a_preq; Wo, down and lm_head quantize their own input (:197, :222, :601).
+ * Off by default: the result carries the activation rounding (logits within about 1e-2 of the fp32-activation
+ * path, not within its 1e-3 bar), which is why the fused and persistent launches keep fp32 activations.  Setting
+ * another exec mode switches it off. */
+int mg_set_q4_act_quant(mg_ctx* ctx, int on);
 
 /* Whole token on the device: embedding gather -> layers -> final norm ->
  * lm_head -> greedy argmax (lowest index on ties).  logitsOut may be NULL. */

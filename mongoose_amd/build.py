@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmongoose_hip.so")
 
-SOURCES = ["kernels.hip", "flow.hip", "prefill.hip", "abi.hip", "fused_infer.hip", "stream_infer.hip", "host_quant.cpp"]
+SOURCES = ["kernels.hip", "flow.hip", "prefill.hip", "q4_dp4a.hip", "abi.hip", "fused_infer.hip", "stream_infer.hip", "host_quant.cpp"]
 
 # -packed-fp32-ops off: hipcc must not form v_pk_*_f32 from float code on this target.
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -158,6 +158,31 @@ void mongoose_q4_0_matvec_planar(const float* act, const void* planar, float* ou
     note(mg::launch_matvec(mg::WF_Q4P, mg::EPI_STORE, mg::PRO_PLAIN, p, nullptr, S(stream)));
 }
 
+// kernels.go:66-70, 985-1017: the integer (dp4a) forms of the Q4_0 matvec.  The reference's CUDA bodies are not in
+// its tree; block format and arithmetic are documented in q4_dp4a.hip.
+void mongoose_q8_quantize_act(const float* act, void* q8_out, int K, void* stream) {
+    if (K <= 0) return;
+    note(mg::launch_q8_quantize_act(act, q8_out, K, 1, S(stream)));
+}
+void mongoose_q8_quantize_act_batch(const float* acts, void* q8_out, int K, int B, void* stream) {
+    if (K <= 0 || B <= 0) return;
+    note(mg::launch_q8_quantize_act(acts, q8_out, K, B, S(stream)));
+}
+void mongoose_q4_0_matvec_dp4a_preq(const void* w, const void* q8_act, float* out, int N, int K, void* stream) {
+    if (N <= 0 || K <= 0) return;
+    note(mg::launch_q4_0_dp4a(w, false, q8_act, out, N, K, 1, S(stream)));
+}
+void mongoose_q4_0_matvec_dp4a(const float* act, const void* w, float* out, int N, int K, void* q8_scratch, void* stream) {
+    if (N <= 0 || K <= 0) return;
+    hipError_t e = mg::launch_q8_quantize_act(act, q8_scratch, K, 1, S(stream));
+    if (e == hipSuccess) e = mg::launch_q4_0_dp4a(w, false, q8_scratch, out, N, K, 1, S(stream));
+    note(e);
+}
+void mongoose_q4_0_matvec_dp4a_batch(const void* w, const void* q8_acts, float* out, int N, int K, int B, void* stream) {
+    if (N <= 0 || K <= 0 || B <= 0) return;
+    note(mg::launch_q4_0_dp4a(w, false, q8_acts, out, N, K, B, S(stream)));
+}
+
 void mongoose_rope(float* x, const float* cosTab, const float* sinTab, int seqLen, int dim, int headDim, int nHeads, void* stream) {
     note(mg::launch_rope(x, cosTab, sinTab, seqLen, dim, headDim, nHeads, S(stream)));
 }

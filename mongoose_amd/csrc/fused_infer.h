@@ -94,10 +94,12 @@ public:
     // 0: one launch per reference op; 1: fused launches; 2: fused, attention launches without the L2 prefetch
     // helpers; 3: all layers of a step in one persistent launch where the model allows it (else as 1).
     int execMode = 3;
+    int SetQ4ActQuant(int on);
     void SetExecMode(int mode) {
         if (mode != execMode) invalidateGraphs();
         if ((mode == 3 || mode == 4) && mode != execMode) flowRegeometry();    // the two differ in the launch's geometry
         execMode = mode;
+        if (mode != 0) q4ActQuant = false;      // only the op-by-op loop has the integer matvecs
         if (mode != 3 && mode != 4) releaseFlow();
     }
     void flowRegeometry();
@@ -186,6 +188,8 @@ private:
     bool flowBroken = false;        // a wait ran into its limit once: the separate launches are used from then on
     bool flowEligible(int l0, int l1) const;
     int flowComputeWgs(int cus) const;
+    bool q4ActQuant = false;      // exec mode 0: Q4_0 matrices through the int8-activation matvecs
+    void* q8Scratch = nullptr;    // (max(dim, ffnDim)/32)*40 bytes of activation blocks (cuda_fused_infer.go:175-179)
     int ensureFlow();
     int enqueueLayersFlow(int l0, int l1, const StepState* st, int posImm, bool resetFirst);
     int checkFlowError();

@@ -214,6 +214,7 @@ HIPFusedInference::~HIPFusedInference() {
     for (auto& sl : layerSlabs) sl.release();
     for (auto& sl : kvSlabs) sl.release();
     if (embedTable) (void)hipFree(embedTable);
+    if (q8Scratch) (void)hipFree(q8Scratch);
     if (dFlowLayers) (void)hipFree(dFlowLayers);
     if (flowXchg) (void)hipFree(flowXchg);
     if (dFlowErr) (void)hipFree(dFlowErr);
@@ -465,7 +466,13 @@ static bool layerComplete(const LayerWeights& L) {
 int HIPFusedInference::enqueueLayerPerOp(const LayerWeights& L, int layer, int pos) {
     float* h = hidden[hiddenIdx];
     const int half = headDim / 2;
-    auto mv = [&](const DevMat& m, const float* act, float* out) -> hipError_t {
+    // requant: the activation vector is quantized into the int8 scratch first (false: it still holds this vector's
+    // blocks -- the reference quantizes once for q, k, v and once for gate, up: cuda_fused_infer_q4.go:161-173, 208-212)
+    auto mv = [&](const DevMat& m, const float* act, float* out, bool requant = true) -> hipError_t {
+        if (q4ActQuant && m.kind == WF_Q4P) {                  // q4Matvec / q4MatvecPreq, cuda_fused_infer_q4.go:611-673
+            if (requant) { hipError_t e = launch_q8_quantize_act(act, q8Scratch, m.cols, 1, stream); if (e != hipSuccess) return e; }
+            return launch_q4_0_dp4a(m.w, true, q8Scratch, out, m.rows, m.cols, 1, stream);
+        }
         MvParams p{};
         p.seg[0] = MvSeg{m.w, m.scales, nullptr, out, m.rows};
         p.nseg = 1; p.K = m.cols; p.act = act;
@@ -473,8 +480,8 @@ int HIPFusedInference::enqueueLayerPerOp(const LayerWeights& L, int layer, int p
     };
     HIPCHK(launch_rmsnorm_out(h, normed, L.norm1, 1, dim, eps, stream));
     HIPCHK(mv(L.wq, normed, Q));
-    HIPCHK(mv(L.wk, normed, K));
-    HIPCHK(mv(L.wv, normed, V));
+    HIPCHK(mv(L.wk, normed, K, L.wq.kind != WF_Q4P));
+    HIPCHK(mv(L.wv, normed, V, L.wq.kind != WF_Q4P));
     if (L.bq) HIPCHK(launch_add_inplace(Q, L.bq, dim, stream));
     if (L.bk) HIPCHK(launch_add_inplace(K, L.bk, kvDim, stream));
     if (L.bv) HIPCHK(launch_add_inplace(V, L.bv, kvDim, stream));
@@ -499,7 +506,7 @@ int HIPFusedInference::enqueueLayerPerOp(const LayerWeights& L, int layer, int p
     HIPCHK(launch_add_inplace(h, proj, dim, stream));
     HIPCHK(launch_rmsnorm_out(h, normed2, L.norm2, 1, dim, eps, stream));
     HIPCHK(mv(L.gate, normed2, gatePre));
-    HIPCHK(mv(L.up, normed2, upOut));
+    HIPCHK(mv(L.up, normed2, upOut, L.gate.kind != WF_Q4P));
     HIPCHK(launch_silu_gate_mul(gatePre, upOut, ffnMid, ffnDim, stream));
     HIPCHK(mv(L.down, ffnMid, proj));
     HIPCHK(launch_add_inplace(h, proj, dim, stream));
@@ -653,6 +660,18 @@ static bool claim_flow(const HIPFusedInference* f, int dev) {
 void HIPFusedInference::releaseFlow() {
     std::lock_guard<std::mutex> lk(g_flowOwnerMutex);
     for (auto& o : g_flowOwner) if (o == this) o = nullptr;
+}
+
+// The reference's integer Q4_0 matvecs in the op-by-op loop (exec mode 0): activations quantized to int8 blocks.
+int HIPFusedInference::SetQ4ActQuant(int on) {
+    if (!built) return MG_E_NOT_BUILT;
+    if (on && execMode != 0) { set_error("SetQ4ActQuant: only the op-by-op loop (exec mode 0) has the integer matvecs"); return MG_E_STATE; }
+    if (on && !q8Scratch) {
+        const int q8MaxK = std::max(dim, ffnDim);                      // cuda_fused_infer.go:175-176
+        HIPCHK(hipMalloc(&q8Scratch, (size_t)(q8MaxK / 32 + 1) * 40));
+    }
+    q4ActQuant = on != 0;
+    return MG_OK;
 }
 
 // Modes 3 and 4 lay the launch out for different numbers of computing workgroups: drop what was sized for the other
@@ -845,6 +864,19 @@ int HIPFusedInference::enqueueLayer(const LayerWeights& L, int layer, const Step
 // argmax folded into the matvec epilogue.
 int HIPFusedInference::enqueueFinal(bool withArgmax) {
     if (!finalNorm || !lmHead.w) { set_error("final norm / lm_head not set"); return MG_E_STATE; }
+    if (execMode == 0 && q4ActQuant && lmHead.kind == WF_Q4P) {
+        // the reference's tail with its integer matvec (cuda_fused_infer_q4.go:600-601): norm, quantize, lm_head; then
+        // the argmax over the finished logits
+        HIPCHK(launch_rmsnorm_out(hidden[hiddenIdx], normed, finalNorm, 1, dim, eps, stream));
+        HIPCHK(launch_q8_quantize_act(normed, q8Scratch, dim, 1, stream));
+        HIPCHK(launch_q4_0_dp4a(lmHead.w, true, q8Scratch, logits, vocabSize, dim, 1, stream));
+        if (withArgmax) {
+            const int parts = std::max(1, std::min(std::min(amaxParts, 256), (vocabSize + 255) / 256));
+            HIPCHK(launch_argmax_slices(logits, vocabSize, parts, amaxVal, amaxIdx, stream));
+            HIPCHK(launch_argmax_finish(amaxVal, amaxIdx, parts, dState, nullptr, dHistory, maxSeq + 1, vocabSize, ropeRef(), embedRef(), stream));
+        }
+        return MG_OK;
+    }
     MvParams p{};
     p.seg[0] = MvSeg{lmHead.w, lmHead.scales, nullptr, logits, vocabSize};
     p.nseg = 1; p.K = dim; p.act = hidden[hiddenIdx]; p.gain = finalNorm; p.eps = eps;
@@ -1548,6 +1580,7 @@ int mg_set_exec_mode(mg_ctx* c, int mode) {
     f->SetExecMode(mode);
     return MG_OK;
 }
+int mg_set_q4_act_quant(mg_ctx* c, int on) { CTX(c); return f->SetQ4ActQuant(on); }
 int mg_decode_token(mg_ctx* c, int token, int pos, int* next, float* logitsOut) { CTX(c); return f->DecodeToken(token, pos, next, logitsOut); }
 int mg_generate(mg_ctx* c, const int* prompt, int nPrompt, int nDecode, int* out, int useGraph) {
     CTX(c); return f->Generate(prompt, nPrompt, nDecode, out, useGraph != 0);

@@ -140,6 +140,12 @@ hipError_t launch_q4_0_repack(const void* raw, void* planar, int N, int K, hipSt
 hipError_t launch_matvec_generic_q8(const float* act, const void* w, const float* scales, float* out, int N, int K, int div127, hipStream_t s);
 hipError_t launch_fill_zero(void* ptr, size_t bytes, hipStream_t s);
 
+// q4_dp4a.hip: int8 activation blocks (40 bytes per 32 activations: float d, float d*sum(q), int8 q[32]) and the
+// Q4_0 matvec on the packed int8 dot instruction.  batch vectors / results are contiguous.
+hipError_t launch_q8_quantize_act(const float* act, void* q8out, int K, int batch, hipStream_t s);
+hipError_t launch_q4_0_dp4a(const void* w, bool planar, const void* q8, float* out, int N, int K, int batch, hipStream_t s);
+hipError_t launch_argmax_slices(const float* x, int n, int nparts, float* pv, int* pi, hipStream_t s);
+
 // Embedding row of state->token into x[dim]: kind 0 = Q8 row * scale (tied
 // lm_head), 1 = fp16 table, 2 = fp32 table, 3 = Q4_0 split-layout row.
 hipError_t launch_embed_token(int kind, const void* table, const float* scales, const StepState* state,

@@ -185,6 +185,31 @@ def KQ4_0MatvecPlanar(act, planar, out, N, K):
     lib.mongoose_q4_0_matvec_planar(_p(act), _p(planar), _p(out), N, K, None)
 
 
+def KQ8QuantizeAct(act, q8Out, K):
+    """kernels.go:993-996: fp32 activations -> int8 blocks, (K/32)*40 bytes."""
+    lib.mongoose_q8_quantize_act(_p(act), _p(q8Out), K, None)
+
+
+def KQ8QuantizeActBatch(acts, q8Out, K, B):
+    """kernels.go:1011-1014."""
+    lib.mongoose_q8_quantize_act_batch(_p(acts), _p(q8Out), K, B, None)
+
+
+def KQ4_0MatvecDP4A(act, w, out, scratch, N, K):
+    """kernels.go:985-988 (scratch: (K/32)*40 bytes)."""
+    lib.mongoose_q4_0_matvec_dp4a(_p(act), _p(w), _p(out), N, K, _p(scratch), None)
+
+
+def KQ4_0MatvecDP4APreq(w, q8Act, out, N, K):
+    """kernels.go:998-1001."""
+    lib.mongoose_q4_0_matvec_dp4a_preq(_p(w), _p(q8Act), _p(out), N, K, None)
+
+
+def KQ4_0MatvecDP4ABatch(w, q8Acts, out, N, K, B):
+    """kernels.go:1006-1009."""
+    lib.mongoose_q4_0_matvec_dp4a_batch(_p(w), _p(q8Acts), _p(out), N, K, B, None)
+
+
 def KRoPE(x, cos, sin, seqLen, dim, headDim, nHeads):
     lib.mongoose_rope(_p(x), _p(cos), _p(sin), seqLen, dim, headDim, nHeads, None)
 
@@ -426,8 +451,13 @@ class HIPFusedInference:
 
     def SetExecMode(self, mode):
         """0 = one launch per reference op, 1 = fused launches, 2 = fused without the L2 prefetch helpers,
-        3 (default) = all layers in one persistent launch where the model allows it."""
+        3 (default) = all layers in one persistent launch where the model allows it, 4 = mode 3 without the
+        workgroups that prefetch weights."""
         return lib.mg_set_exec_mode(self._h, mode)
+
+    def SetQ4ActQuant(self, on):
+        """cuda_fused_infer_q4.go:611-673: Q4_0 matrices through the int8-activation (dp4a) matvecs; exec mode 0 only."""
+        return lib.mg_set_q4_act_quant(self._h, 1 if on else 0)
 
     # L3 bridge and mailbox (cuda_fused_infer.go:556-737)
     def QueueHiddenToL3(self):

@@ -62,6 +62,11 @@ _sig("mongoose_embed_gather", None, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_dequant_int8_to_fp32", None, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_dequant_q8_rowscale", None, _p, _p, _p, c_int, c_int, _p)
 _sig("mongoose_dequant_q4_0", None, _p, _p, c_int, c_int, _p)
+_sig("mongoose_q8_quantize_act", None, _p, _p, c_int, _p)
+_sig("mongoose_q8_quantize_act_batch", None, _p, _p, c_int, c_int, _p)
+_sig("mongoose_q4_0_matvec_dp4a", None, _p, _p, _p, c_int, c_int, _p, _p)
+_sig("mongoose_q4_0_matvec_dp4a_preq", None, _p, _p, _p, c_int, c_int, _p)
+_sig("mongoose_q4_0_matvec_dp4a_batch", None, _p, _p, _p, c_int, c_int, c_int, _p)
 _sig("mongoose_q8_gemm", None, _p, _p, _p, _p, _p, c_int, c_int, c_int, c_int, _p, c_size_t, _p)
 _sig("mg_q8_gemm_noalloc", c_int, _p, _p, _p, _p, _p, c_int, c_int, c_int, c_int, _p)
 _sig("mg_q8_gemm_noalloc_max_bytes", c_size_t)
@@ -78,6 +83,7 @@ _sig("mg_num_weights", c_int, c_void_p)
 _sig("mg_set_weight", c_int, c_void_p, c_int, _f, c_size_t)
 _sig("mg_set_weight_q8", c_int, c_void_p, c_int, POINTER(c_int8), _f)
 _sig("mg_set_weight_q4_0", c_int, c_void_p, c_int, POINTER(c_uint8), c_size_t)
+_sig("mg_set_q4_act_quant", c_int, c_void_p, c_int)
 _sig("mg_set_quant_rounding", c_int, c_void_p, c_int)
 _sig("mg_set_embedding_f16", c_int, c_void_p, POINTER(c_uint16))
 _sig("mg_set_embedding_f32", c_int, c_void_p, _f)

@@ -56,12 +56,15 @@ _sig("orc_set_embed_f16", None, c_void_p, POINTER(c_uint16))
 _sig("orc_set_embed_f32", None, c_void_p, _f)
 _sig("orc_reset_kv", None, c_void_p)
 _sig("orc_set_kv_f16", None, c_void_p, c_int)
+_sig("orc_set_q4_act_quant", None, c_void_p, c_int)
+_sig("orc_q8_quantize_act", None, _f, POINTER(c_uint8), c_int)
 _sig("orc_embed", c_int, c_void_p, c_int, _f)
 _sig("orc_argmax", c_int, _f, c_int)
 for pfx, real in (("orc32", _f), ("orc64", _d)):
     _sig(pfx + "_rmsnorm_out", None, real, _f, c_int, c_float, real)
     _sig(pfx + "_q8_matvec", None, real, POINTER(c_int8), _f, real, c_int, c_int, c_int)
     _sig(pfx + "_q4_0_matvec", None, real, POINTER(c_uint8), real, c_int, c_int, c_int)
+    _sig(pfx + "_q4_0_matvec_q8act", None, POINTER(c_uint8), POINTER(c_uint8), real, c_int, c_int, c_int)
     _sig(pfx + "_rope", None, real, _f, _f, c_int, c_int)
     _sig(pfx + "_decode_attention", None, real, real, real, real, c_int, c_int, c_int, c_int, c_int, real)
     _sig(pfx + "_silu_gate_mul", None, real, real, real, c_int)
@@ -160,6 +163,24 @@ def q4_0_matvec(act, blocks, N, K, shadow=False, threads=1):
     return out
 
 
+def q8_quantize_act(act):
+    """fp32 activations [K] -> int8 blocks, (K/32)*40 bytes: float d, float d*sum(q), int8 q[32]."""
+    act = f32(act)
+    out = np.empty(act.size // 32 * 40, np.uint8)
+    lib.orc_q8_quantize_act(fp(act), u8p(out), act.size)
+    return out
+
+
+def q4_0_matvec_q8act(q8, blocks, N, K, shadow=False, threads=1):
+    """Raw GGUF Q4_0 rows against quantized activation blocks (the integer matvec)."""
+    pfx, dt, p = _real(shadow)
+    q8 = np.ascontiguousarray(q8, np.uint8)
+    blocks = np.ascontiguousarray(blocks, np.uint8)
+    out = np.empty(N, dt)
+    getattr(lib, pfx + "_q4_0_matvec_q8act")(u8p(q8), u8p(blocks), p(out), N, K, threads)
+    return out
+
+
 def rope(x, cosRow, sinRow, nHeads, headDim, shadow=False):
     pfx, dt, p = _real(shadow)
     x = np.array(x, dtype=dt, order="C")
@@ -254,6 +275,9 @@ class Oracle:
 
     def set_kv_f16(self, on):
         lib.orc_set_kv_f16(self.h, 1 if on else 0)
+
+    def set_q4_act_quant(self, on):
+        lib.orc_set_q4_act_quant(self.h, 1 if on else 0)
 
     def embed(self, tok):
         out = np.empty(self.dim, np.float32)

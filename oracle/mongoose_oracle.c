@@ -39,6 +39,12 @@
  *                        pairs, (nib-8)*s/7); pinned by unit activations that pick single
  *                        nibbles and by orc_matmul over the densely dequantized matrix
  *   orcNN_fused_add_rmsnorm  kernels/mongoose.cu:372-404; pinned by orc_rmsnorm on a+b
+ *   orc_q8_quantize_act / orcNN_q4_0_matvec_q8act / orc_set_q4_act_quant
+ *                        the integer ("dp4a") Q4_0 matvec, kernels.go:66-70, 985-1017, dispatch
+ *                        cuda_fused_infer_q4.go:611-673.  The CUDA bodies are absent from the reference:
+ *                        PARITY UNPINNED by it.  Restated from GGML's block_q8_1 / vec_dot_q4_0_q8_1 (fp32
+ *                        block fields, the 40-byte block the reference's scratch size implies); pinned by
+ *                        closed forms and by equality with the fp32 matvec on the dequantized blocks.
  *   embedding gather, argmax   no reference function (the reference's caller does
  *                        both on the host); textbook semantics, lowest index on ties.
  *
@@ -254,6 +260,35 @@ ORC_API void orc_dequant_q4_0(const uint8_t* blocks, int rows, int cols, float* 
     }
 }
 
+/* Activation blocks of the integer ("dp4a") Q4_0 matvec, kernels.go:68,993-996 (KQ8QuantizeAct: "quantizes fp32
+ * activation to Q8_1 blocks"); scratch size (K/32)*40 bytes, cuda_fused_infer.go:176.  The reference's CUDA body is
+ * not in its tree: PARITY UNPINNED by the reference.  The block is GGML's block_q8_1 (quantize_row_q8_1_ref) with
+ * fp32 fields, which is what 40 bytes hold: float d = amax/127, float s = d * sum(q), int8 q[32] =
+ * roundf(x * (1/d)) (round half away from zero); a zero block has d = s = 0.  Pinned by closed forms in the tests
+ * (amax maps to +-127, reconstruction error <= d/2, s == d * sum q, zero block) and an independent numpy
+ * restatement. */
+ORC_API void orc_q8_quantize_act(const float* act, uint8_t* out, int K) {
+    int nb = K / 32;
+    for (int b = 0; b < nb; b++) {
+        const float* x = act + (size_t)b * 32;
+        uint8_t* y = out + (size_t)b * 40;
+        float amax = 0.0f;
+        for (int j = 0; j < 32; j++) { float v = fabsf(x[j]); if (v > amax) amax = v; }
+        float d = amax / 127.0f;
+        float id = d != 0.0f ? 1.0f / d : 0.0f;
+        int sum = 0;
+        int8_t* q = (int8_t*)(y + 8);
+        for (int j = 0; j < 32; j++) {
+            int v = (int)roundf(x[j] * id);
+            q[j] = (int8_t)v;
+            sum += v;
+        }
+        float s = d * (float)sum;
+        memcpy(y, &d, 4);
+        memcpy(y + 4, &s, 4);
+    }
+}
+
 /* cuda_fused_infer.go:181-192  angle in double, tables stored as float. */
 ORC_API void orc_rope_tables(int maxSeq, int headDim, double theta, float* cosT, float* sinT) {
     int half = headDim / 2;
@@ -293,6 +328,7 @@ typedef struct {
     float *kc32, *vc32;       /* [nLayers, maxSeq, kvDim] float caches */
     double *kc64, *vc64;      /* double shadow caches */
     int kv_f16;               /* K/V rows rounded to fp16 (RNE) when written: models an fp16 KV cache */
+    int q4_act_quant;         /* Q4_0 matrices through the int8-activation matvec (cuda_fused_infer_q4.go:611-673) */
     int threads;
 } orc_ctx;
 
@@ -407,6 +443,11 @@ ORC_API void orc_set_embed_f32(orc_ctx* c, const float* table) {
  * for compressed ones, kernels.go:71-72).  The rounding is the pinned orc_f32_to_f16; everything
  * around it is the unchanged step, so the option is pinned by those two. */
 ORC_API void orc_set_kv_f16(orc_ctx* c, int on) { c->kv_f16 = on ? 1 : 0; }
+
+/* The step with the reference's integer Q4_0 matvecs (q4Matvec / q4MatvecPreq, cuda_fused_infer_q4.go:611-673):
+ * every Q4_0 matrix sees its input quantized by orc_q8_quantize_act.  The reference quantizes once for q, k, v and
+ * once for gate, up (:161-173, :208-212); quantizing per matrix gives the same blocks. */
+ORC_API void orc_set_q4_act_quant(orc_ctx* c, int on) { c->q4_act_quant = on ? 1 : 0; }
 
 ORC_API void orc_reset_kv(orc_ctx* c) {
     size_t kvn = (size_t)c->nLayers * c->maxSeq * c->kvDim;

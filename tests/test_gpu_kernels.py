@@ -289,3 +289,68 @@ def test_zero_fill_unaligned(hip):
     want[3:25] = 0
     assert np.array_equal(got, want)
     d.Release()
+
+
+# ---------------------------------------------------------------------------
+# The integer ("dp4a") forms of the Q4_0 matvec (kernels.go:66-70, 985-1017).
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("K,B", [(32, 1), (896, 1), (4864, 1), (14336, 1), (896, 5)])
+def test_q8_quantize_act_bytes_equal_the_oracle(hip, K, B):
+    """Activation blocks (40 bytes per 32 values): the same bytes as the oracle's, zero blocks and single spikes
+    included; the batch form quantizes B contiguous vectors."""
+    x = rng.standard_normal(K * B).astype(np.float32)
+    x[:32] = 0.0
+    if K >= 96:
+        x[32:64] = 0.0
+        x[40] = 7.25
+    want = np.concatenate([ob.q8_quantize_act(x[b * K:(b + 1) * K]) for b in range(B)])
+    dx = _up(hip, x)
+    dq = hip.UploadRawBytes(np.full(want.size, 0xAA, np.uint8))
+    if B == 1:
+        E.KQ8QuantizeAct(dx, dq, K)
+    else:
+        E.KQ8QuantizeActBatch(dx, dq, K, B)
+    _check()
+    assert np.array_equal(hip.DownloadRawBytes(dq), want)
+    dx.Release()
+    dq.Release()
+
+
+@pytest.mark.parametrize("N,K", [(896, 896), (128, 896), (4864, 896), (896, 4864), (1001, 64), (4096, 14336)])
+def test_q4_0_matvec_dp4a_forms(hip, N, K):
+    """mongoose_q4_0_matvec_dp4a (quantizes into the caller's scratch), _preq (takes quantized blocks) and _batch against
+    the oracle's integer matvec at 1e-5 (the integer block sums are exact; the floats differ by summation order), and
+    against the fp32-activation matvec within the activation rounding (what the reference's own check logs,
+    cuda_fused_infer_q4.go:633-662)."""
+    print(f"q4_0 dp4a N={N} K={K}", flush=True)
+    w = E.synth_normal(18, N * 19 + K, 0.02, (N, K))
+    blocks = ob.quantize_q4_0(w)
+    B = 3
+    acts = rng.standard_normal(K * B).astype(np.float32)
+    q8 = [ob.q8_quantize_act(acts[b * K:(b + 1) * K]) for b in range(B)]
+    ref = [ob.q4_0_matvec_q8act(q8[b], blocks, N, K, shadow=True, threads=8) for b in range(B)]
+    dw, da = _up(hip, blocks), _up(hip, acts)
+    dscratch = hip.UploadRawBytes(np.zeros(K // 32 * 40, np.uint8))
+    dout = hip.Zeros([N])
+    E.KQ4_0MatvecDP4A(da, dw, dout, dscratch, N, K)
+    _check()
+    got = hip.ToHost(dout)
+    assert H.rel_err(got, ref[0]) < 1e-5
+    assert np.array_equal(hip.DownloadRawBytes(dscratch), q8[0])
+    exact = ob.q4_0_matvec(acts[:K], blocks, N, K, shadow=True, threads=8)
+    assert H.rel_err(got, exact) < 3e-2
+    dout2 = hip.Zeros([N])
+    E.KQ4_0MatvecDP4APreq(dw, dscratch, dout2, N, K)
+    _check()
+    assert np.array_equal(hip.ToHost(dout2), got)
+    dq8 = hip.UploadRawBytes(np.zeros(K // 32 * 40 * B, np.uint8))
+    E.KQ8QuantizeActBatch(da, dq8, K, B)
+    doutB = hip.Zeros([B * N])
+    E.KQ4_0MatvecDP4ABatch(dw, dq8, doutB, N, K, B)
+    _check()
+    gotB = hip.ToHost(doutB).reshape(B, N)
+    for b in range(B):
+        assert H.rel_err(gotB[b], ref[b]) < 1e-5, b
+    assert np.array_equal(gotB[0], got)
+    for t in (dw, da, dscratch, dout, dout2, dq8, doutB):
+        t.Release()

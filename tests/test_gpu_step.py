@@ -451,3 +451,53 @@ def test_layer_range_pipeline_with_l3_bridge_and_mailbox(hip):
     assert np.array_equal(a.hip.GetL3Hidden(), a.hip.ExportHidden())
     for m in (whole, a, b):
         m.close()
+
+
+def test_q4_act_quant_step_matches_the_oracle_with_the_same_option(hip):
+    """mg_set_q4_act_quant: the op-by-op loop with the reference's integer Q4_0 matvecs (q4Matvec / q4MatvecPreq /
+    q8QuantizeAct, cuda_fused_infer_q4.go:611-673) against the oracle run with the same activation quantization.
+    Rounding activations to int8 makes the step discontinuous: an activation that two correct fp32 evaluations place
+    on either side of a rounding boundary moves by a whole step (1/127 of its block's maximum), so the bar here is
+    5e-3 on the logits of a teacher-forced stream and tokens equal up to near-ties at that bar, not the 1e-3 /
+    identical tokens of the fp32-activation paths.  The fp32-activation step is close (activation rounding) but not
+    equal; any other exec mode refuses the option."""
+    s = H.with_layers(configs.QWEN_Q4, 3)._replace(vocab=2048)
+    m = H.Model(s, seed=61, maxSeq=32, eng=hip, threads=8)
+    assert m.hip.SetQ4ActQuant(True) != 0 and "exec mode 0" in E.last_error()
+    assert m.hip.SetExecMode(0) == 0
+    prompt = m.prompt(6)
+    stream = [int(t) for t in prompt] + [int(t) for t in m.prompt(16)[6:]]
+
+    def forced_logits():
+        assert m.hip.ResetKV() == 0
+        out = []
+        lg = np.empty(s.vocab, np.float32)
+        for pos, tok in enumerate(stream):
+            rc, _ = m.hip.DecodeToken(tok, pos, lg)
+            assert rc == 0, E.last_error()
+            out.append(lg.copy())
+        return out
+
+    plain = forced_logits()
+    assert m.hip.SetQ4ActQuant(True) == 0, E.last_error()
+    quant = forced_logits()
+    m.orc.set_q4_act_quant(True)
+    m.orc.reset_kv()
+    worst = 0.0
+    for pos, tok in enumerate(stream):
+        _, lg, _ = m.orc.decode_token(tok, pos, shadow=True)
+        worst = max(worst, H.rel_err(quant[pos], lg))
+        d = H.rel_err(quant[pos], plain[pos])
+        assert 1e-5 < d < 5e-2, (pos, d)
+    assert worst < 5e-3, worst
+    # greedy tokens: the oracle's, up to near-ties at the same bar
+    ref, _ = H.oracle_generate(m, prompt, 12)
+    assert m.hip.ResetKV() == 0
+    rc, toks = m.hip.Generate(prompt, 12, useGraph=False)
+    assert rc == 0, E.last_error()
+    H.assert_same_tokens_or_near_tie(m, prompt, ref, toks, "integer Q4_0 matvecs", tol=5e-3)
+    # leaving the op-by-op loop switches the option off
+    assert m.hip.SetExecMode(1) == 0
+    again = forced_logits()
+    assert H.rel_err(again[-1], plain[-1]) < 1e-4
+    m.close()

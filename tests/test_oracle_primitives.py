@@ -340,3 +340,89 @@ def test_fused_add_rmsnorm_is_rmsnorm_of_the_sum():
     s = a.astype(np.float64) + b.astype(np.float64)
     want64 = s / np.sqrt((s * s).mean() + 1e-6) * g
     assert H_rel(ob.fused_add_rmsnorm(a, b, g, 1e-6, shadow=True), want64) < 1e-12
+
+
+# ---------------------------------------------------------------------------
+# The integer ("dp4a") Q4_0 matvec: activation blocks and the block dot product
+# (kernels.go:66-70, 985-1017; the CUDA bodies are absent from the reference, so these
+# closed forms and the independent restatement are what pins the oracle's functions).
+# ---------------------------------------------------------------------------
+def _np_q8_blocks(x):
+    """Independent numpy restatement of the activation quantizer: per 32 values d = amax/127 (float32),
+    q = round half away from zero of x * (1/d), s = d * sum(q)."""
+    x = np.asarray(x, np.float32).reshape(-1, 32)
+    amax = np.abs(x).max(axis=1)
+    d = (amax / np.float32(127.0)).astype(np.float32)
+    idv = np.zeros_like(d)
+    nz = d != 0
+    idv[nz] = (np.float32(1.0) / d[nz]).astype(np.float32)
+    v = (x * idv[:, None]).astype(np.float32).astype(np.float64)
+    q = (np.sign(v) * np.floor(np.abs(v) + 0.5)).astype(np.int32)
+    s = (d * q.sum(axis=1).astype(np.float32)).astype(np.float32)
+    return d, s, q.astype(np.int8)
+
+
+def _split_q8(blocks):
+    b = np.asarray(blocks, np.uint8).reshape(-1, 40)
+    return b[:, :4].copy().view(np.float32)[:, 0], b[:, 4:8].copy().view(np.float32)[:, 0], b[:, 8:].copy().view(np.int8)
+
+
+def test_q8_activation_blocks_closed_forms_and_numpy():
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal(32 * 40).astype(np.float32)
+    x[64:96] = 0.0                                  # a zero block
+    x[96:128] = 0.0
+    x[100] = -3.5                                   # a single spike: it alone maps to -127
+    x[128:160] = 1e-30                              # tiny equal values: all +127
+    d, s, q = _split_q8(ob.q8_quantize_act(x))
+    nd, ns, nq = _np_q8_blocks(x)
+    assert np.array_equal(d, nd) and np.array_equal(s, ns) and np.array_equal(q, nq)
+    xb = x.reshape(-1, 32)
+    assert d[2] == 0 and s[2] == 0 and not q[2].any()
+    assert q[3][4] == -127 and np.count_nonzero(q[3]) == 1 and d[3] == np.float32(3.5) / np.float32(127)
+    assert (q[4] == 127).all()
+    for b in range(xb.shape[0]):
+        if d[b] == 0:
+            continue
+        i = int(np.abs(xb[b]).argmax())
+        assert abs(int(q[b][i])) == 127                               # the extreme maps to +-127
+        assert np.abs(xb[b] - q[b].astype(np.float64) * d[b]).max() <= 0.5 * d[b] * (1 + 1e-6)
+        assert s[b] == np.float32(d[b] * np.float32(q[b].astype(np.int64).sum()))
+
+
+def test_integer_q4_0_matvec_is_the_fp32_matvec_on_the_quantized_activations():
+    """sum_b d4 (d8 sumi - 8 s8) == sum_k deq(W)[r,k] * (q[k] d8[block of k]) in exact arithmetic: the double shadow of
+    the integer form against the (pinned) fp32-activation matvec fed the dequantized activation blocks."""
+    rng = np.random.default_rng(78)
+    N, K = 37, 896
+    w = rng.standard_normal((N, K)).astype(np.float32) * 0.02
+    blocks = ob.quantize_q4_0(w)
+    act = rng.standard_normal(K).astype(np.float32)
+    q8 = ob.q8_quantize_act(act)
+    d, s, q = _split_q8(q8)
+    act_hat = (q.astype(np.float64) * d.astype(np.float64)[:, None]).reshape(-1)
+    want = ob.q4_0_matvec(act_hat, blocks, N, K, shadow=True)
+    got64 = ob.q4_0_matvec_q8act(q8, blocks, N, K, shadow=True)
+    got32 = ob.q4_0_matvec_q8act(q8, blocks, N, K)
+    den = np.abs(want).max()
+    assert np.abs(got64 - want).max() / den < 1e-6          # s8 is d*sum rounded to float: 6e-8 of the -8 term
+    assert np.abs(got32 - want).max() / den < 1e-5
+    # and it is the fp32-activation result up to the activation rounding (half a step of 1/127 of the block maximum)
+    exact = ob.q4_0_matvec(act, blocks, N, K, shadow=True)
+    err = np.abs(got64 - exact).max() / np.abs(exact).max()
+    assert 1e-5 < err < 3e-2, err
+
+
+def test_integer_q4_0_matvec_element_order():
+    """One activation per run: it quantizes to +127 with d = x/127, so row r gives d4 * (nib - 8) * x -- which picks
+    the nibble that belongs to element k (low nibble of byte j = element j, high nibble = element j + 16)."""
+    rng = np.random.default_rng(79)
+    N, K = 3, 64
+    w = rng.standard_normal((N, K)).astype(np.float32)
+    blocks = ob.quantize_q4_0(w)
+    deq = ob.dequant_q4_0(blocks, N, K)
+    for k in (0, 1, 15, 16, 17, 31, 32, 47, 63):
+        act = np.zeros(K, np.float32)
+        act[k] = 2.5
+        got = ob.q4_0_matvec_q8act(ob.q8_quantize_act(act), blocks, N, K, shadow=True)
+        assert np.allclose(got, deq[:, k].astype(np.float64) * 2.5, rtol=1e-6, atol=1e-6), k     # a nibble of 8: zero up to the rounding of s = d * sum(q)

@@ -229,3 +229,25 @@ def test_threaded_attention_changes_nothing():
             assert (x[0] == y[0]).all() and (x[1] == y[1]).all()
     a.close()
     b.close()
+
+
+def test_step_with_integer_q4_0_matvecs_tracks_the_fp32_activation_step():
+    """orc_set_q4_act_quant: every Q4_0 matrix sees int8 activation blocks (cuda_fused_infer_q4.go:611-673).  Same
+    step otherwise, so the logits stay within the activation rounding of the fp32-activation step and are not equal."""
+    from mongoose_amd import configs
+    from tests import helpers as H
+    s = H.with_layers(configs.TOY, 2)._replace(fmt="q4_0", name="toy-q4")
+    a = H.Model(s, seed=5, maxSeq=8, threads=4)
+    b = H.Model(s, seed=5, maxSeq=8, threads=4)
+    b.orc.set_q4_act_quant(True)
+    prompt = a.prompt(4)
+    for pos in range(4):
+        h = a.orc.embed(prompt[pos])
+        _, la, _ = a.orc.step(h, pos, shadow=True)
+        _, lb, _ = b.orc.step(h, pos, shadow=True)
+        _, lb32, _ = b.orc.step(h, pos)
+        err = H.rel_err(lb, la)
+        assert 1e-5 < err < 5e-2, (pos, err)
+        assert H.rel_err(lb32, lb) < 1e-4
+    a.close()
+    b.close()
