@@ -268,6 +268,15 @@ def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_gra
         if att and "GBps" in att[0]:
             run["attention_KV_GBps"] = att[0]["GBps"]
         res["runs"].append(run)
+    # K/V read rate of the launches in use at a long context: the extra K/V bytes a step reads there, over the extra
+    # time it takes, against the first (short) context of the same run
+    for run in res["runs"][1:]:
+        base = res["runs"][0]
+        dms = run["ms_per_step"] - base["ms_per_step"]
+        dbytes = (configs.kv_bytes_at(s, run["start_position"] + K // 2) - configs.kv_bytes_at(s, base["start_position"] + K // 2)) // (2 if kv_f16 else 1)
+        if dms > 0 and dbytes > 0:
+            run["KV_GBps_from_step_delta"] = round(dbytes / (dms * 1e-3) / 1e9, 1)
+            run["KV_GBps_note"] = f"extra K/V bytes over extra step time against start_position {base['start_position']}"
     if prefill > 0:
         ptoks = E.synth_tokens(seed, 20_000_003, s.vocab, prefill)
         times = []

@@ -391,6 +391,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             // (Measured at the 0.5B shape: releasing every job a phase earlier or later, and 24 to 48 prefetching
             // workgroups, all give the same step time within 0.5 %; 16 are too few, 64 cost more than they bring.)
             auto release = [&](int off) {
+                pf.drain();                // the job before has landed (its loads' destination register is still pf.sink)
                 if (l == p.l0) return;
                 if (tid == 0) (void)poll1(Xp + off, wt);
                 __syncthreads();
@@ -546,6 +547,23 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             const int QH = grouped ? p.nHeads / p.nKVHeads : 1;        // query heads of this workgroup
             const int unit = grouped ? p.nKVHeads : p.nHeads;
             const int split = blockIdx.x / unit, hu = blockIdx.x % unit;
+            if constexpr (RING) {
+                // Long rows, two or more Wo rows a wave, of which only the first half-row is requested ahead: a workgroup
+                // with no attention to do (and no partials to merge per head) reads its waves' Wo rows into its XCD's L2
+                // now.  Its next poll, for the attention's partials, is microseconds away (8B shape: 1.828 -> 1.810 ms a token;
+                // the same for the rest of the q | k | v rows ahead of the layer's first poll gains nothing).
+                if (!(split < G.smax && split < nsplit) && !(grouped && (int)blockIdx.x < p.nHeads)) {
+                    pfv4 sink = {0, 0, 0, 0};
+                    const size_t rb = Q4 ? dim >> 1 : dim;
+                    for (int r = gw; r < dim; r += W) {
+                        const char* row = reinterpret_cast<const char*>(L.wo) + (size_t)r * rb;
+                        for (size_t o = (size_t)lane * 16; o < rb; o += 1024)
+                            asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(sink) : "v"(row + o) : "memory");
+                    }
+                    // the loads write into sink: it must stay allocated until they have landed
+                    asm volatile("s_waitcnt vmcnt(0)" : "+v"(sink) : : "memory");
+                }
+            }
             if (split < G.smax && split < nsplit) {
                 const int kvh = grouped ? hu : hu / (p.nHeads / p.nKVHeads);
                 const int h0 = grouped ? hu * QH : hu;

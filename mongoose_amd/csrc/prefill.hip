@@ -209,15 +209,17 @@ __device__ __forceinline__ void split8(const float (&v)[8], bf16x8_t& h, bf16x8_
     l = __builtin_bit_cast(bf16x8_t, ul);
 }
 
-// grid (rowsPad / 32, nKVHeads, 2), HD threads: thread d takes column kvh * HD + d of 32 rows of K (z = 0) or V (z = 1)
+// grid (rowsPad / 32, nKVHeads, 2), (HD, 4) threads: thread (d, w) takes column kvh * HD + d of a quarter of the 32
+// rows of K (z = 0: rows 8w .. 8w+7) or V (z = 1: the eight rows whose values make up 16-byte piece w of the column's
+// transposed group)
 template <typename KVT>
 __global__ void kv_split_kernel(const KVT* Kc, const KVT* Vc, int rows, int kvDim, int HD, unsigned short* Khi,
                                 unsigned short* Klo, unsigned short* VThi, unsigned short* VTlo, int vtStride) {
-    const int g = blockIdx.x, col = blockIdx.y * HD + threadIdx.x;
+    const int g = blockIdx.x, col = blockIdx.y * HD + threadIdx.x, w = threadIdx.y;
     if (blockIdx.z == 0) {
-#pragma unroll 8
-        for (int i = 0; i < 32; i++) {
-            const int r = g * 32 + i;
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const int r = g * 32 + 8 * w + t;
             const size_t o = (size_t)r * kvDim + col;
             const float k = r < rows ? (float)Kc[o] : 0.f;
             const unsigned short kh = f32_to_bf16_rne(k);
@@ -226,24 +228,23 @@ __global__ void kv_split_kernel(const KVT* Kc, const KVT* Vc, int rows, int kvDi
         }
         return;
     }
-    unsigned short vh[32], vl[32];
+    // position i of the tile sits at k slot 8 * ((i >> 2) & 3) + (i & 3) + 4 * (i >> 4): piece w holds positions
+    // 4w .. 4w+3 and 16+4w .. 16+4w+3
+    unsigned short vh[8], vl[8];
 #pragma unroll
-    for (int i = 0; i < 32; i++) {
+    for (int t = 0; t < 8; t++) {
+        const int i = t < 4 ? 4 * w + t : 16 + 4 * w + (t - 4);
         const int r = g * 32 + i;
         const float v = r < rows ? (float)Vc[(size_t)r * kvDim + col] : 0.f;
-        const int idx = 8 * ((i >> 2) & 3) + (i & 3) + 4 * (i >> 4);      // position i of the tile sits at k slot idx
-        vh[idx] = f32_to_bf16_rne(v);
-        vl[idx] = f32_to_bf16_rne(v - bf16_to_f32(vh[idx]));
+        vh[t] = f32_to_bf16_rne(v);
+        vl[t] = f32_to_bf16_rne(v - bf16_to_f32(vh[t]));
     }
     uint4* dh = reinterpret_cast<uint4*>(VThi + (size_t)col * vtStride + g * 32);
     uint4* dl = reinterpret_cast<uint4*>(VTlo + (size_t)col * vtStride + g * 32);
-#pragma unroll
-    for (int w = 0; w < 4; w++) {
-        dh[w] = make_uint4(vh[8 * w] | ((unsigned)vh[8 * w + 1] << 16), vh[8 * w + 2] | ((unsigned)vh[8 * w + 3] << 16),
-                           vh[8 * w + 4] | ((unsigned)vh[8 * w + 5] << 16), vh[8 * w + 6] | ((unsigned)vh[8 * w + 7] << 16));
-        dl[w] = make_uint4(vl[8 * w] | ((unsigned)vl[8 * w + 1] << 16), vl[8 * w + 2] | ((unsigned)vl[8 * w + 3] << 16),
-                           vl[8 * w + 4] | ((unsigned)vl[8 * w + 5] << 16), vl[8 * w + 6] | ((unsigned)vl[8 * w + 7] << 16));
-    }
+    dh[w] = make_uint4(vh[0] | ((unsigned)vh[1] << 16), vh[2] | ((unsigned)vh[3] << 16),
+                       vh[4] | ((unsigned)vh[5] << 16), vh[6] | ((unsigned)vh[7] << 16));
+    dl[w] = make_uint4(vl[0] | ((unsigned)vl[1] << 16), vl[2] | ((unsigned)vl[3] << 16),
+                       vl[4] | ((unsigned)vl[5] << 16), vl[6] | ((unsigned)vl[7] << 16));
 }
 
 template <int HD>
@@ -448,9 +449,9 @@ hipError_t launch_prefill_attention(const float* q, const void* Kc, const void* 
     unsigned short* Khi = static_cast<unsigned short*>(kvSplit);
     unsigned short *Klo = Khi + plane, *VThi = Klo + plane, *VTlo = VThi + plane;
     const dim3 sgrid((unsigned)(rowsPad / 32), (unsigned)nKVHeads, 2);
-    if (kvHalf) hipLaunchKernelGGL((kv_split_kernel<_Float16>), sgrid, dim3(headDim), 0, s, static_cast<const _Float16*>(Kc),
+    if (kvHalf) hipLaunchKernelGGL((kv_split_kernel<_Float16>), sgrid, dim3(headDim, 4), 0, s, static_cast<const _Float16*>(Kc),
                                    static_cast<const _Float16*>(Vc), rows, kvDim, headDim, Khi, Klo, VThi, VTlo, rowsPad);
-    else hipLaunchKernelGGL((kv_split_kernel<float>), sgrid, dim3(headDim), 0, s, static_cast<const float*>(Kc),
+    else hipLaunchKernelGGL((kv_split_kernel<float>), sgrid, dim3(headDim, 4), 0, s, static_cast<const float*>(Kc),
                             static_cast<const float*>(Vc), rows, kvDim, headDim, Khi, Klo, VThi, VTlo, rowsPad);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
