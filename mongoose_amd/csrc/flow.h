@@ -51,6 +51,7 @@ struct FlowParams {
     int nLayersTotal;            // layers the table and the exchange area hold
     int dim, kvDim, ffn, nHeads, nKVHeads, headDim, maxSeq;
     int q4;                      // 0: Q8 matrices, 1: Q4_0 matrices in the split layout
+    int idleWoRows, idleGateUpRows;   // leading rows of Wo / of gate and up that workgroups idle during the attention read into the L2s
     int nCompute;                // workgroups 0 .. nCompute-1 compute (geo is laid out for them), the rest of the grid prefetches
     float eps;
     const StepState* state;      // position source (NULL -> posImm)

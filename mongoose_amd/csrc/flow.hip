@@ -547,21 +547,34 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             const int QH = grouped ? p.nHeads / p.nKVHeads : 1;        // query heads of this workgroup
             const int unit = grouped ? p.nKVHeads : p.nHeads;
             const int split = blockIdx.x / unit, hu = blockIdx.x % unit;
-            if constexpr (RING) {
-                // Long rows, two or more Wo rows a wave, of which only the first half-row is requested ahead: a workgroup
-                // with no attention to do (and no partials to merge per head) reads its waves' Wo rows into its XCD's L2
-                // now.  Its next poll, for the attention's partials, is microseconds away (8B shape: 1.828 -> 1.810 ms a token;
-                // the same for the rest of the q | k | v rows ahead of the layer's first poll gains nothing).
-                if (!(split < G.smax && split < nsplit) && !(grouped && (int)blockIdx.x < p.nHeads)) {
-                    pfv4 sink = {0, 0, 0, 0};
-                    const size_t rb = Q4 ? dim >> 1 : dim;
-                    for (int r = gw; r < dim; r += W) {
-                        const char* row = reinterpret_cast<const char*>(L.wo) + (size_t)r * rb;
-                        for (size_t o = (size_t)lane * 16; o < rb; o += 1024)
-                            asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(sink) : "v"(row + o) : "memory");
+            // Workgroups with no attention to do (and no partials to merge per head) read, into their XCD's L2, rows that the
+            // XCD's workgroups will want after it -- their next poll, for the attention's partials, is microseconds away, and
+            // HBM would be idle meanwhile.  p.idleWoRows: Wo (rows of more than 2048 weights, of which a wave requests only
+            // the first half-row ahead); p.idleGateUpRows: the leading rows of gate and of up -- all of them where both
+            // matrices fit the L2s (1.1B shape: 0.465 -> 0.436 ms a token; the down projection on top overflows the L2s:
+            // 0.470), else half of the first round of rows, which is what a phase waits for before it streams (8B shape
+            // with both: 1.845 -> 1.790; the whole first round 1.804, a quarter 1.800).
+            // Only while at least half the launch is idle (short contexts), and only without dedicated prefetchers.
+            if ((p.idleWoRows > 0 || p.idleGateUpRows > 0) && nC == (int)gridDim.x) {
+                const int live = nsplit < G.smax ? nsplit : G.smax;
+                int nBusy = unit * live;
+                if (grouped && nBusy < p.nHeads) nBusy = p.nHeads;
+                nBusy = (nBusy + 7) & ~7;
+                if ((int)blockIdx.x >= nBusy && 2 * ((int)gridDim.x - nBusy) >= (int)gridDim.x) {
+                    Prefetcher pf{(int)blockIdx.x & 7, ((int)blockIdx.x - nBusy) >> 3, ((int)gridDim.x - nBusy) >> 3, tid, {0, 0, 0, 0}};
+                    const size_t rbD = Q4 ? dim >> 1 : dim, rdD = dim >> 4;
+                    // (a workgroup without q | k | v rows gets here at the top of the layer; holding it back until q | k | v is
+                    // through measures slower: 1.1B shape 0.453 against 0.435 ms a token)
+                    if (p.idleWoRows > 0) {
+                        pf.rows(L.wo, rbD, p.idleWoRows, 8);
+                        if (Q4) pf.rows(L.so, rdD, p.idleWoRows, 8);
                     }
-                    // the loads write into sink: it must stay allocated until they have landed
-                    asm volatile("s_waitcnt vmcnt(0)" : "+v"(sink) : : "memory");
+                    if (p.idleGateUpRows > 0) {
+                        pf.rows(L.gate, rbD, p.idleGateUpRows, 8);
+                        pf.rows(L.up, rbD, p.idleGateUpRows, 8);
+                        if (Q4) { pf.rows(L.sgate, rdD, p.idleGateUpRows, 8); pf.rows(L.sup, rdD, p.idleGateUpRows, 8); }
+                    }
+                    pf.drain();
                 }
             }
             if (split < G.smax && split < nsplit) {

@@ -815,6 +815,14 @@ int HIPFusedInference::enqueueLayersFlow(int l0, int l1, const StepState* st, in
     p.dim = dim; p.kvDim = kvDim; p.ffn = ffnDim; p.nHeads = nHeads; p.nKVHeads = nKVHeads; p.headDim = headDim; p.maxSeq = maxSeq;
     p.q4 = layers[l0].wq.kind == WF_Q4P ? 1 : 0;
     p.nCompute = flowCompute;
+    {
+        // attention-idle prefetch: Wo where a wave holds only part of its rows ahead (rows of more than 2048 weights); gate
+        // and up whole where both fit the L2s beside what is in use (3 MB an XCD), else half of their first round of rows
+        const LayerWeights& L0 = layers[l0];
+        p.idleWoRows = dim > 2048 ? dim : 0;
+        const int firstRound = std::min(ffnDim, flowCompute * 8);
+        p.idleGateUpRows = (L0.gate.bytes + L0.up.bytes) / 8 <= ((size_t)3 << 20) ? ffnDim : (firstRound / 2) & ~63;
+    }
     p.eps = eps;
     p.state = st; p.posImm = posImm;
     const int half = headDim / 2;
