@@ -52,6 +52,7 @@ struct FlowParams {
     int dim, kvDim, ffn, nHeads, nKVHeads, headDim, maxSeq;
     int q4;                      // 0: Q8 matrices, 1: Q4_0 matrices in the split layout
     int idleWoRows, idleGateUpRows;   // leading rows of Wo / of gate and up that workgroups idle during the attention read into the L2s
+    int downSplit;               // the down projection's rows are shared by two waves each (few rows, long ones)
     int nCompute;                // workgroups 0 .. nCompute-1 compute (geo is laid out for them), the rest of the grid prefetches
     float eps;
     const StepState* state;      // position source (NULL -> posImm)

@@ -281,6 +281,37 @@ __device__ __forceinline__ void dot_rows(const int4 (&wr)[NR][CB], const float4*
         }
     }
 }
+// the same over the chunks [.., cHi) of a row only (a row shared by two waves); nch stays the stride of the staged planes
+template <bool Q4, int CB>
+__device__ __forceinline__ void ld_row_rng(WRow row, int cHi, int lane, int c0, int4 (&wr)[CB]) {
+#pragma unroll
+    for (int i = 0; i < CB; i++) {
+        const int c = min(c0 + lane + i * 64, cHi - 1);
+        if (Q4) {
+            const int2 q = reinterpret_cast<const int2*>(row.w)[c];
+            wr[i] = make_int4(q.x, q.y, (int)row.d[c >> 1], 0);
+        } else {
+            wr[i] = reinterpret_cast<const int4*>(row.w)[c];
+        }
+    }
+}
+template <bool Q4, int CB>
+__device__ __forceinline__ float dot_row_rng(const int4 (&wr)[CB], const float4* a4, int nch, int cHi, int lane, int c0, float acc) {
+#pragma unroll
+    for (int i = 0; i < CB; i++) {
+        const int c = c0 + lane + i * 64;
+        if (c < cHi) {
+            const float4 av[4] = {a4[c], a4[nch + c], a4[2 * nch + c], a4[3 * nch + c]};
+            if (Q4) {
+                acc = dot_q4_half(make_int2(wr[i].x, wr[i].y), half_bits_to_float((unsigned short)wr[i].z), av, chunk_act_sum(av), acc);
+            } else {
+                acc = dot4_i8(wr[i].x, av[0], acc); acc = dot4_i8(wr[i].y, av[1], acc);
+                acc = dot4_i8(wr[i].z, av[2], acc); acc = dot4_i8(wr[i].w, av[3], acc);
+            }
+        }
+    }
+    return acc;
+}
 // the rest of rows longer than the prefetched batch
 template <bool Q4, int NR, int CB>
 __device__ __forceinline__ void dot_rows_tail(const WRow (&rows)[NR], const float4* a4, int nch, int lane, float (&acc)[NR]) {
@@ -432,8 +463,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             else { pf.whole(L.sgate, (size_t)ffn * 4); pf.whole(L.sup, (size_t)ffn * 4); }
             pf.whole(L.g2, (size_t)dim * 4);
             release(G.offX2);              // ... done: the down projection of this one
-            pf.rows(L.down, rbF, dim, 8);
-            if (Q4) pf.rows(L.sdown, rdF, dim, 8); else pf.whole(L.sdown, (size_t)dim * 4);
+            const int drun = p.downSplit ? FWAVES / 2 : FWAVES;      // rows of the down projection a workgroup takes
+            pf.rows(L.down, rbF, dim, drun);
+            if (Q4) pf.rows(L.sdown, rdF, dim, drun); else pf.whole(L.sdown, (size_t)dim * 4);
         }
         pf.drain();
         return;
@@ -964,6 +996,44 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         }
                     }
                     store_runs(e1 + v * e0, (nI + W - 1) / W, nI, 0, X + G.offX2, l == p.l1 - 1 ? p.hidden : nullptr);
+                }
+            } else if (p.downSplit) {
+                // Few rows (at most half as many as computing waves): a row is shared by two neighbouring waves of a
+                // workgroup, each taking half of its chunks, and every workgroup with rows has half as many -- the
+                // multiplications of this phase, its longest rows, take half as long (0.5B shape 0.366 -> 0.360 ms a
+                // token).  One round.
+                if ((int)blockIdx.x * (FWAVES / 2) < nI) {
+                    constexpr int CBH = CBF / 2;
+                    const int row = min(gw >> 1, nI - 1), hf = wave & 1;
+                    const int nHalf = (nchF + 1) >> 1;
+                    const int c0 = hf ? nHalf : 0, cHi = hf ? nchF : nHalf;
+                    const WRow rw = wrow<Q4>(L.down, L.sdown, row, ffn);
+                    int4 wr[CBH];
+                    ld_row_rng<Q4, CBH>(rw, cHi, lane, c0, wr);
+                    float e0 = 0.f, e1 = 0.f;
+                    if (wave == 0 && lane < FWAVES / 2) {
+                        const int r = min((int)blockIdx.x * (FWAVES / 2) + lane, nI - 1);
+                        e0 = Q4 ? 1.f : L.sdown[r];
+                        e1 = poll1(X + G.offX1 + r, wt);
+                    }
+                    stage_plain<Q4>(X + G.offM, ffn, a4, wt);
+                    FLOW_TRACE(9);
+                    float acc = dot_row_rng<Q4, CBH>(wr, a4, nchF, cHi, lane, c0, 0.f);
+                    for (int cc = c0 + CBH * 64; cc < cHi; cc += CBH * 64) {
+                        ld_row_rng<Q4, CBH>(rw, cHi, lane, cc, wr);
+                        acc = dot_row_rng<Q4, CBH>(wr, a4, nchF, cHi, lane, cc, acc);
+                    }
+                    acc = wave_sum(acc);
+                    if (lane == 0) outbuf[0][wave] = acc;
+                    __syncthreads();
+                    if (wave == 0 && lane < FWAVES / 2) {
+                        const int r = (int)blockIdx.x * (FWAVES / 2) + lane;
+                        if (r < nI) {
+                            const float o = e1 + (outbuf[0][2 * lane] + outbuf[0][2 * lane + 1]) * e0;
+                            stx(X + G.offX2 + r, o);
+                            if (l == p.l1 - 1) p.hidden[r] = o;
+                        }
+                    }
                 }
             } else
             if (blockIdx.x * FWAVES < nI) {

@@ -815,6 +815,7 @@ int HIPFusedInference::enqueueLayersFlow(int l0, int l1, const StepState* st, in
     p.dim = dim; p.kvDim = kvDim; p.ffn = ffnDim; p.nHeads = nHeads; p.nKVHeads = nKVHeads; p.headDim = headDim; p.maxSeq = maxSeq;
     p.q4 = layers[l0].wq.kind == WF_Q4P ? 1 : 0;
     p.nCompute = flowCompute;
+    p.downSplit = (dim <= 2048 && 2 * dim <= flowCompute * 8 && ffnDim >= 2048) ? 1 : 0;
     {
         // attention-idle prefetch: Wo where a wave holds only part of its rows ahead (rows of more than 2048 weights); gate
         // and up whole where both fit the L2s beside what is in use (3 MB an XCD), else half of their first round of rows
