@@ -39,7 +39,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
 # NOT measured by the run that prints them: "traffic_source" in the output says so.
 PMC_TRAFFIC_BYTES = {
     ("qwen2.5-0.5b", "lm_head"): int((67135.1 * (262144.0 / 131102.4) + 660.5 * 1.0) * 1024),
-    ("qwen2.5-0.5b", "flow"): int((190112.3 * (262144.0 / 131102.4) + 864.5 * 1.0) * 1024),
+    ("qwen2.5-0.5b", "flow"): int((190867.0 * (262144.0 / 131102.4) + 952.0 * 1.0) * 1024),
     ("llama-3-8b", "lm_head"): int((257245.0 * (262144.0 / 131102.4) + 715.6 * 1.0) * 1024),
     ("llama-3-8b", "flow"): int((3510548.2 * (262144.0 / 131102.4) + 4432.0 * 1.0) * 1024),
 }
