@@ -73,6 +73,24 @@ __device__ __forceinline__ float wave_sum(float v) {
     v += dpp_f<0x128>(v);
     return rows_sum(v);
 }
+// Two sums over the wave for the price of little more than one: the first exchange folds them into one register
+// (lanes 0..31 carry a, lanes 32..63 carry b), the rest reduces within the halves.  Returns sum(a) in lanes 0..31 and
+// sum(b) in lanes 32..63.
+__device__ __forceinline__ float wave_sum2(float a, float b) {
+    row_swap32(a, b);                      // a: [a low half | b low half], b: [a high half | b high half]
+    float t = a + b;
+    float x = t, y = t;
+    row_swap16(x, y);
+    t = x + y;
+    t += dpp_f<0xB1>(t);
+    t += dpp_f<0x4E>(t);
+    t += dpp_f<0x124>(t);
+    t += dpp_f<0x128>(t);
+    return t;
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
 __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, dpp_f<0xB1>(v));
     v = fmaxf(v, dpp_f<0x4E>(v));

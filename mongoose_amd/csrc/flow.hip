@@ -526,9 +526,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     float acc[2] = {0.f, 0.f};
                     dot_rows<Q4, 2, CBQ>(w, a4, nchD, lane, 0, acc);
                     if (nchD > CBQ * 64) dot_rows_tail<Q4, 2, CBQ>(rw, a4, nchD, lane, acc);
-                    acc[0] = wave_sum(acc[0]);
-                    acc[1] = wave_sum(acc[1]);
-                    float v = lane == 1 ? acc[1] : acc[0];
+                    const float t = wave_sum2(acc[0], acc[1]);
+                    float v = lane == 1 ? lane_value(t, 32) : t;
                     v = v * f0;                                                  // row scale (lanes 0 and 1)
                     v = v * rs;
                     v = v + f1;
@@ -896,7 +895,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                 const int k = st / nb, b = st - k * nb;
                                 dot_rows<Q4, 2, CB>(ring[j], a4, nchD, lane, b * CB * 64, acc);
                                 if (b == nb - 1) {
-                                    const float v0 = wave_sum(acc[0]), v1 = wave_sum(acc[1]);
+                                    const float t = wave_sum2(acc[0], acc[1]);
+                                    const float v0 = lane_value(t, 0), v1 = lane_value(t, 32);
                                     if (lane == k) { g = v0; u = v1; }
                                     acc[0] = 0.f; acc[1] = 0.f;
                                 }
@@ -939,8 +939,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                 const WRow rows[2] = {wrow<Q4>(L.gate, L.sgate, r, dim), wrow<Q4>(L.up, L.sup, r, dim)};
                                 dot_rows_tail<Q4, 2, CBD>(rows, a4, nchD, lane, acc);
                             }
-                            acc[0] = wave_sum(acc[0]);
-                            acc[1] = wave_sum(acc[1]);
+                            const float t = wave_sum2(acc[0], acc[1]);
+                            acc[0] = lane_value(t, 0);
+                            acc[1] = lane_value(t, 32);
                         }
                         if (lane == k) { g = acc[0]; u = acc[1]; }
                     }
