@@ -374,8 +374,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     __shared__ float red[FWAVES];
     constexpr int QHMAX = GQA ? FLOW_GQA_MAX : 1;
     __shared__ float4 sqkv[2 + QHMAX][HD / 4];         // K and V row of the current position, q of the workgroup's heads
-    __shared__ float4 accbuf[FWAVES][HD / 4];
-    __shared__ float lbuf[FWAVES], wred[FWAVES];
+    __shared__ float4 accbuf[QHMAX][FWAVES][HD / 4];   // per query head of the workgroup: the waves' partial outputs, sums, maxima
+    __shared__ float lbuf[QHMAX][FWAVES], wred[QHMAX][FWAVES];
     __shared__ float outbuf[FLOW_MAX_ROUNDS][FWAVES];                // a phase's results of the workgroup, stored by one wave as whole 32-byte runs
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -652,8 +652,6 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     }
                 }
                 for (int hi = 0; hi < QH; hi++) {          // the heads of the KV head in turn, on the same K / V registers
-                const int h = h0 + hi;
-                if (hi) __syncthreads();                    // accbuf, lbuf, wred are free again
                 float4 q4[NF];
 #pragma unroll
                 for (int j = 0; j < NF; j++) q4[j] = sqkv[2 + hi][j * 16 + dl];
@@ -694,30 +692,32 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
 #pragma unroll
                 for (int j = 0; j < NF; j++) {
                     acc[j].x = tg_sum(acc[j].x); acc[j].y = tg_sum(acc[j].y); acc[j].z = tg_sum(acc[j].z); acc[j].w = tg_sum(acc[j].w);
-                    if (lane < LPR) accbuf[wave][j * 16 + dl] = acc[j];
+                    if (lane < LPR) accbuf[hi][wave][j * 16 + dl] = acc[j];
                 }
                 lsum = tg_sum(lsum);
-                if (lane == 0) { lbuf[wave] = lsum; wred[wave] = m; }
+                if (lane == 0) { lbuf[hi][wave] = lsum; wred[hi][wave] = m; }
+                }
+                // the waves' partials of all the workgroup's heads combined together: one barrier, a thread per head and piece
                 __syncthreads();
-                if (tid < HD / 4) {
-                    float mg_ = wred[0];
+                if (tid < QH * (HD / 4)) {
+                    const int hq = tid / (HD / 4), i = tid % (HD / 4), h = h0 + hq;
+                    float mg_ = wred[hq][0];
 #pragma unroll
-                    for (int k = 1; k < FWAVES; k++) mg_ = fmaxf(mg_, wred[k]);
+                    for (int k = 1; k < FWAVES; k++) mg_ = fmaxf(mg_, wred[hq][k]);
                     f4 r = {0.f, 0.f, 0.f, 0.f};
                     float lg = 0.f;
 #pragma unroll
                     for (int k = 0; k < FWAVES; k++) {
-                        const float wk = exp_neg(wred[k] - mg_);
-                        const float4 a = accbuf[k][tid];
+                        const float wk = exp_neg(wred[hq][k] - mg_);
+                        const float4 a = accbuf[hq][k][i];
                         r.x = fmaf(wk, a.x, r.x); r.y = fmaf(wk, a.y, r.y); r.z = fmaf(wk, a.z, r.z); r.w = fmaf(wk, a.w, r.w);
-                        lg = fmaf(wk, lbuf[k], lg);
+                        lg = fmaf(wk, lbuf[hq][k], lg);
                     }
-                    stx4(reinterpret_cast<f4*>(X + G.offPacc + (size_t)split * dim + h * HD) + tid, r);
-                    if (tid == 0) {
+                    stx4(reinterpret_cast<f4*>(X + G.offPacc + (size_t)split * dim + h * HD) + i, r);
+                    if (i == 0) {
                         stx(X + G.offPm + split * p.nHeads + h, mg_);
                         stx(X + G.offPl + split * p.nHeads + h, lg);
                     }
-                }
                 }
             }
         }
