@@ -580,9 +580,23 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
         const bool grouped = GQA && p.nHeads * (pos / TILE + 1) > nC;
         {
             const int nsplit = pos / TILE + 1;
-            const int QH = grouped ? p.nHeads / p.nKVHeads : 1;        // query heads of this workgroup
-            const int unit = grouped ? p.nKVHeads : p.nHeads;
+            // Grouped: the query heads of a KV head are shared out over as many workgroups as the launch has left for
+            // them at this position (each loads the K / V rows once and takes its heads in turn), so a workgroup takes as
+            // few heads as possible: qhMax heads a workgroup, `sub` workgroups a KV head and split.
+            const int Gq = p.nHeads / p.nKVHeads;
+            int qhMax = 1, sub = Gq;
+            if (grouped) {
+                qhMax = Gq; sub = 1;
+                const int live = nsplit < G.smax ? nsplit : G.smax;
+                for (int q = 2; q < Gq; q++) {
+                    const int sb = (Gq + q - 1) / q;
+                    if (p.nKVHeads * sb * live <= nC) { qhMax = q; sub = sb; break; }
+                }
+            }
+            const int unit = grouped ? p.nKVHeads * sub : p.nHeads;
             const int split = blockIdx.x / unit, hu = blockIdx.x % unit;
+            const int hg = grouped ? hu % sub : 0;                         // which of the KV head's groups of query heads
+            const int QH = grouped ? min(qhMax, Gq - hg * qhMax) : 1;      // query heads of this workgroup
             // Workgroups with no attention to do (and no partials to merge per head) read, into their XCD's L2, rows that the
             // XCD's workgroups will want after it -- their next poll, for the attention's partials, is microseconds away, and
             // HBM would be idle meanwhile.  p.idleWoRows: Wo (rows of more than 2048 weights, of which a wave requests only
@@ -614,8 +628,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 }
             }
             if (split < G.smax && split < nsplit) {
-                const int kvh = grouped ? hu : hu / (p.nHeads / p.nKVHeads);
-                const int h0 = grouped ? hu * QH : hu;
+                const int kvh = grouped ? hu / sub : hu / Gq;
+                const int h0 = grouped ? kvh * Gq + hg * qhMax : hu;
                 const int tg = tid / LPR, dl = tid % LPR;
                 const int t0 = split * TILE;
                 const int len = pos + 1;
