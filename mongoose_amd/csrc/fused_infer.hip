@@ -33,15 +33,6 @@ const std::string& get_error() { return g_err; }
         if (!(cond)) { set_error(msg); return MG_E_ARG; }                                 \
     } while (0)
 
-template <typename T>
-static int devAlloc(T*& p, size_t count, bool zero) {
-    void* v = nullptr;
-    HIPCHK(hipMalloc(&v, count * sizeof(T) ? count * sizeof(T) : 1));
-    if (zero) HIPCHK(hipMemset(v, 0, count * sizeof(T)));
-    p = static_cast<T*>(v);
-    return MG_OK;
-}
-
 HIPFusedInference* HIPFusedInference::New(int dim, int kvDim, int headDim, int nHeads, int nKVHeads, int ffnDim,
                                           int vocabSize, int nLayers, int maxSeq, double ropeTheta, float eps) {
     if (dim <= 0 || kvDim <= 0 || nHeads <= 0 || nKVHeads <= 0 || ffnDim <= 0 || vocabSize <= 0 || nLayers <= 0 ||
@@ -793,7 +784,8 @@ int HIPFusedInference::FlowTrace(int enable, long long* out, size_t cap, int* di
         void* v = nullptr;
         HIPCHK(hipMalloc(&v, sizeof(long long) * n));
         flowTrace = static_cast<long long*>(v);
-        HIPCHK(hipMemset(v, 0, sizeof(long long) * n));
+        HIPCHK(hipMemsetAsync(v, 0, sizeof(long long) * n, stream));
+        HIPCHK(hipStreamSynchronize(stream));
         invalidateGraphs();
     }
     if (out && flowTrace) {
@@ -852,7 +844,8 @@ int HIPFusedInference::checkFlowError() {
     HIPCHK(hipMemcpy(hFlowErr, dFlowErr, sizeof(int), hipMemcpyDeviceToHost));
     if (*hFlowErr == 0) return MG_OK;
     *hFlowErr = 0;
-    HIPCHK(hipMemset(dFlowErr, 0, sizeof(int)));
+    HIPCHK(hipMemsetAsync(dFlowErr, 0, sizeof(int), stream));
+    HIPCHK(hipStreamSynchronize(stream));
     flowBroken = true;
     releaseFlow();
     invalidateGraphs();
