@@ -24,6 +24,45 @@ constexpr int FWAVES = 8;                 // waves of a workgroup (two a SIMD: a
 constexpr int FWG = 64 * FWAVES;
 typedef float f4 __attribute__((ext_vector_type(4)));
 
+// The pointers of the layer table are read from memory, so the compiler takes them for generic pointers and loads
+// through them with FLAT instructions, which count as LDS operations as well (a wait for an LDS read then also waits
+// for the weights in flight).  What is loaded through them is loaded through explicitly global pointers instead.
+typedef int gv4i __attribute__((ext_vector_type(4)));
+typedef int gv2i __attribute__((ext_vector_type(2)));
+template <bool GL>
+__device__ __forceinline__ int4 ldg_i4(const void* p, size_t i) {
+    if (!GL) return static_cast<const int4*>(p)[i];
+    const gv4i t = ((const gv4i __attribute__((address_space(1)))*)p)[i];
+    return make_int4(t.x, t.y, t.z, t.w);
+}
+template <bool GL>
+__device__ __forceinline__ int2 ldg_i2(const void* p, size_t i) {
+    if (!GL) return static_cast<const int2*>(p)[i];
+    const gv2i t = ((const gv2i __attribute__((address_space(1)))*)p)[i];
+    return make_int2(t.x, t.y);
+}
+template <bool GL>
+__device__ __forceinline__ unsigned short ldg_u16(const void* p, size_t i) {
+    if (!GL) return static_cast<const unsigned short*>(p)[i];
+    return ((const unsigned short __attribute__((address_space(1)))*)p)[i];
+}
+template <bool GL>
+__device__ __forceinline__ void stg_f(float* p, size_t i, float v) {
+    if (!GL) { p[i] = v; return; }
+    ((float __attribute__((address_space(1)))*)p)[i] = v;
+}
+template <bool GL>
+__device__ __forceinline__ float ldg_f(const float* p, size_t i) {
+    if (!GL) return p[i];
+    return ((const float __attribute__((address_space(1)))*)p)[i];
+}
+template <bool GL>
+__device__ __forceinline__ float4 ldg_f4(const void* p, size_t i) {
+    if (!GL) return static_cast<const float4*>(p)[i];
+    const f4 t = ((const f4 __attribute__((address_space(1)))*)p)[i];
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+
 __device__ __forceinline__ bool unset(float v) { return __builtin_bit_cast(unsigned, v) == XSENT; }
 __device__ __forceinline__ float canon(float v) { return unset(v) ? __builtin_bit_cast(float, 0x7FC00000u) : v; }
 __device__ __forceinline__ bool ready4(f4 v) { return !(unset(v.x) || unset(v.y) || unset(v.z) || unset(v.w)); }
@@ -168,7 +207,7 @@ __device__ __forceinline__ int slot4(int k4, int nch) {
 __device__ __forceinline__ float4 tof4(f4 v) { return make_float4(v.x, v.y, v.z, v.w); }
 
 // x (optionally polled) -> LDS as x * gain; returns 1/rms.  Leaves with a barrier done.
-template <bool Q4>
+template <bool GL, bool Q4>
 __device__ __forceinline__ float stage_rms(const float* x, bool polled, const float* gain, int K, float eps, float4* a4,
                                            float* red, Waiter& w) {
     const int K4 = K >> 2, nch = K >> 4, tid = threadIdx.x;
@@ -184,7 +223,7 @@ __device__ __forceinline__ float stage_rms(const float* x, bool polled, const fl
         for (int u = 0; u < PB; u++) {
             const int i = min(base + u * FWG + tid, K4 - 1);
             ptr[u] = x4 + i;
-            g[u] = g4[i];
+            g[u] = ldg_f4<GL>(g4, i);
         }
         const int np = max(0, min(PB, (K4 - base - tid + FWG - 1) / FWG));      // this thread's pieces of the round
 #pragma unroll
@@ -237,6 +276,7 @@ __device__ __forceinline__ void stage_plain(const float* x, int K, float4* a4, W
 // A weight row: Q8 16-byte chunks of int8; Q4_0 (split layout: all nibble groups of the matrix, then all fp16 d)
 // 8-byte half blocks and the row of d, one per two chunks.
 struct WRow { const signed char* w; const unsigned short* d; };
+
 template <bool Q4>
 __device__ __forceinline__ WRow wrow(const signed char* W, const float* aux, int r, int K) {
     if (Q4) return WRow{W + (size_t)r * (K >> 1), reinterpret_cast<const unsigned short*>(aux) + (size_t)r * (K >> 5)};
@@ -244,16 +284,16 @@ __device__ __forceinline__ WRow wrow(const signed char* W, const float* aux, int
 }
 // chunks c0 + lane + i*64 of a row (clamped inside the row: loads are unconditional); a Q4_0 chunk travels as
 // {nibbles, nibbles, d bits, -}
-template <bool Q4, int CB>
+template <bool GL, bool Q4, int CB>
 __device__ __forceinline__ void ld_row(WRow row, int nch, int lane, int c0, int4 (&wr)[CB]) {
 #pragma unroll
     for (int i = 0; i < CB; i++) {
         const int c = min(c0 + lane + i * 64, nch - 1);
         if (Q4) {
-            const int2 q = reinterpret_cast<const int2*>(row.w)[c];
-            wr[i] = make_int4(q.x, q.y, (int)row.d[c >> 1], 0);
+            const int2 q = ldg_i2<GL>(row.w, c);
+            wr[i] = make_int4(q.x, q.y, (int)ldg_u16<GL>(row.d, c >> 1), 0);
         } else {
-            wr[i] = reinterpret_cast<const int4*>(row.w)[c];
+            wr[i] = ldg_i4<GL>(row.w, c);
         }
     }
 }
@@ -282,16 +322,16 @@ __device__ __forceinline__ void dot_rows(const int4 (&wr)[NR][CB], const float4*
     }
 }
 // the same over the chunks [.., cHi) of a row only (a row shared by two waves); nch stays the stride of the staged planes
-template <bool Q4, int CB>
+template <bool GL, bool Q4, int CB>
 __device__ __forceinline__ void ld_row_rng(WRow row, int cHi, int lane, int c0, int4 (&wr)[CB]) {
 #pragma unroll
     for (int i = 0; i < CB; i++) {
         const int c = min(c0 + lane + i * 64, cHi - 1);
         if (Q4) {
-            const int2 q = reinterpret_cast<const int2*>(row.w)[c];
-            wr[i] = make_int4(q.x, q.y, (int)row.d[c >> 1], 0);
+            const int2 q = ldg_i2<GL>(row.w, c);
+            wr[i] = make_int4(q.x, q.y, (int)ldg_u16<GL>(row.d, c >> 1), 0);
         } else {
-            wr[i] = reinterpret_cast<const int4*>(row.w)[c];
+            wr[i] = ldg_i4<GL>(row.w, c);
         }
     }
 }
@@ -313,12 +353,12 @@ __device__ __forceinline__ float dot_row_rng(const int4 (&wr)[CB], const float4*
     return acc;
 }
 // the rest of rows longer than the prefetched batch
-template <bool Q4, int NR, int CB>
+template <bool GL, bool Q4, int NR, int CB>
 __device__ __forceinline__ void dot_rows_tail(const WRow (&rows)[NR], const float4* a4, int nch, int lane, float (&acc)[NR]) {
     for (int c0 = CB * 64; c0 < nch; c0 += CB * 64) {
         int4 wr[NR][CB];
 #pragma unroll
-        for (int r = 0; r < NR; r++) ld_row<Q4, CB>(rows[r], nch, lane, c0, wr[r]);
+        for (int r = 0; r < NR; r++) ld_row<GL, Q4, CB>(rows[r], nch, lane, c0, wr[r]);
         dot_rows<Q4, NR, CB>(wr, a4, nch, lane, c0, acc);
     }
 }
@@ -373,6 +413,10 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     extern __shared__ float4 a4[];                     // the staged activation vector, max(dim, ffn) floats
     __shared__ float red[FWAVES];
     constexpr int QHMAX = GQA ? FLOW_GQA_MAX : 1;
+    // Rows of up to 1024 weights are requested whole before a hand-over and multiplied after all of them have arrived:
+    // no load is in flight across an LDS read, and the generic loads measure 1.6 % faster there (0.5B shape); longer
+    // rows stream (remainders, rings), and the explicitly global loads measure 1.7 % (1.1B) and 2.7 % (8B) faster.
+    constexpr bool GL = CBD > 1;
     __shared__ float4 sqkv[2 + QHMAX][HD / 4];         // K and V row of the current position, q of the workgroup's heads
     __shared__ float4 accbuf[QHMAX][FWAVES][HD / 4];   // per query head of the workgroup: the waves' partial outputs, sums, maxima
     __shared__ float lbuf[QHMAX][FWAVES], wred[QHMAX][FWAVES];
@@ -511,13 +555,13 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     else if (item < nq + nk) { kd = 1; Wm = L.wk; sc = L.sk; bias = L.bk; const int i2 = item - nq; const int jj = i2 % half; a0 = (i2 - jj) * 2 + jj; a1 = a0 + half; }
                     else { kd = 2; Wm = L.wv; sc = L.sv; bias = L.bv; a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
                     rw[0] = wrow<Q4>(Wm, sc, a0, dim); rw[1] = wrow<Q4>(Wm, sc, a1, dim);
-                    ld_row<Q4, CBQ>(rw[0], nchD, lane, 0, w[0]);
-                    ld_row<Q4, CBQ>(rw[1], nchD, lane, 0, w[1]);
+                    ld_row<GL, Q4, CBQ>(rw[0], nchD, lane, 0, w[0]);
+                    ld_row<GL, Q4, CBQ>(rw[1], nchD, lane, 0, w[1]);
                     f0 = 1.f; f1 = 0.f;
                     if (lane < 2) {
                         const int r = lane ? a1 : a0;
-                        if (!Q4) f0 = sc[r];
-                        if (bias) f1 = bias[r];
+                        if (!Q4) f0 = ldg_f<GL>(sc, r);
+                        if (bias) f1 = ldg_f<GL>(bias, r);
                     }
                     if (lane == 2 && kd < 2) { const int jj = a0 % half; f0 = p.cosRow[jj]; f1 = p.sinRow[jj]; }
                 };
@@ -525,7 +569,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 auto finish = [&](const int4 (&w)[2][CBQ], const WRow (&rw)[2], int kd, float f0, float f1, float rs, int it) {
                     float acc[2] = {0.f, 0.f};
                     dot_rows<Q4, 2, CBQ>(w, a4, nchD, lane, 0, acc);
-                    if (nchD > CBQ * 64) dot_rows_tail<Q4, 2, CBQ>(rw, a4, nchD, lane, acc);
+                    if (nchD > CBQ * 64) dot_rows_tail<GL, Q4, 2, CBQ>(rw, a4, nchD, lane, acc);
                     const float t = wave_sum2(acc[0], acc[1]);
                     float v = lane == 1 ? lane_value(t, 32) : t;
                     v = v * f0;                                                  // row scale (lanes 0 and 1)
@@ -551,7 +595,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             if (kk == 0) {
                                 stx(X + G.offQ + r, o);
                             } else {                                              // mongoose.cu:1644-1647, and the hand-over copy
-                                ((kk == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim)[r] = o;
+                                stg_f<GL>(kk == 1 ? L.Kc : L.Vc, (size_t)pos * kvDim + r, o);
                                 stx(X + (kk == 1 ? G.offKc : G.offVc) + r, o);
                             }
                         }
@@ -562,7 +606,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     kind[q] = 0; r0[q] = 0; r1[q] = 0; e0[q] = 0.f; e1[q] = 0.f; rows[q][0] = wrow<Q4>(L.wq, L.sq, 0, dim); rows[q][1] = rows[q][0];
                     if (gw + q * W < nI) resolve(wr[q], rows[q], kind[q], r0[q], r1[q], e0[q], e1[q], gw + q * W);
                 }
-                const float rs = stage_rms<Q4>(xin, !first, L.g1, dim, p.eps, a4, red, wt);
+                const float rs = stage_rms<GL, Q4>(xin, !first, L.g1, dim, p.eps, a4, red, wt);
                 FLOW_TRACE(1);
 #pragma unroll
                 for (int q = 0; q < NPI; q++)
@@ -644,9 +688,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 for (int u = 0; u < VU; u++) {
                     const size_t ro = (size_t)min(t0 + tg + u * TG, lastRow) * rowStride + colOff;
 #pragma unroll
-                    for (int j = 0; j < NF; j++) kreg[u][j] = Kc4[ro + j * 16];
+                    for (int j = 0; j < NF; j++) kreg[u][j] = ldg_f4<GL>(Kc4, ro + j * 16);
 #pragma unroll
-                    for (int j = 0; j < NF; j++) vreg[u][j] = Vc4[ro + j * 16];
+                    for (int j = 0; j < NF; j++) vreg[u][j] = ldg_f4<GL>(Vc4, ro + j * 16);
                 }
                 __syncthreads();
                 if (tid < (2 + QH) * (HD / 4)) {
@@ -812,9 +856,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 float e0 = 0.f, e1 = 0.f;
                 auto resolve = [&](int item) {
                     rows[0] = wrow<Q4>(L.wo, L.so, item, dim);
-                    ld_row<Q4, CBD>(rows[0], nchD, lane, 0, wr[0]);
+                    ld_row<GL, Q4, CBD>(rows[0], nchD, lane, 0, wr[0]);
                     if (lane == 0) {
-                        e0 = Q4 ? 1.f : L.so[item];
+                        e0 = Q4 ? 1.f : ldg_f<GL>(L.so, item);
                         e1 = first ? xin[item] : poll1(xin + item, wt);         // there already if this workgroup staged it for q | k | v
                     }
                 };
@@ -862,7 +906,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     if (it != gw) resolve(it);
                     float acc[1] = {0.f};
                     dot_rows<Q4, 1, CBD>(wr, a4, nchD, lane, 0, acc);
-                    if (nchD > CBD * 64) dot_rows_tail<Q4, 1, CBD>(rows, a4, nchD, lane, acc);
+                    if (nchD > CBD * 64) dot_rows_tail<GL, Q4, 1, CBD>(rows, a4, nchD, lane, acc);
                     const float v = wave_sum(acc[0]);
                     if (it != gw) __syncthreads();              // outbuf is free again
                     store_runs(e1 + v * e0, 1, nI, it - gw, X + G.offX1, nullptr);
@@ -887,16 +931,16 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         const int sc = min(st, T - 1);                       // past the end: the last step again (uniform loop)
                         const int k = sc / nb, b = sc - k * nb;
                         const int row = gw + k * W;
-                        ld_row<Q4, CB>(wrow<Q4>(L.gate, L.sgate, row, dim), nchD, lane, b * CB * 64, set[0]);
-                        ld_row<Q4, CB>(wrow<Q4>(L.up, L.sup, row, dim), nchD, lane, b * CB * 64, set[1]);
+                        ld_row<GL, Q4, CB>(wrow<Q4>(L.gate, L.sgate, row, dim), nchD, lane, b * CB * 64, set[0]);
+                        ld_row<GL, Q4, CB>(wrow<Q4>(L.up, L.sup, row, dim), nchD, lane, b * CB * 64, set[1]);
                     };
                     float sg = 0.f, su = 0.f;
                     if (T > 0) {
 #pragma unroll
                         for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
-                        if (lane < nItems) { const int r = gw + lane * W; sg = Q4 ? 1.f : L.sgate[r]; su = Q4 ? 1.f : L.sup[r]; }
+                        if (lane < nItems) { const int r = gw + lane * W; sg = Q4 ? 1.f : ldg_f<GL>(L.sgate, r); su = Q4 ? 1.f : ldg_f<GL>(L.sup, r); }
                     }
-                    const float rs = stage_rms<Q4>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                    const float rs = stage_rms<GL, Q4>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
                     FLOW_TRACE(7);
                     float acc[2] = {0.f, 0.f};
                     float g = 0.f, u = 0.f;
@@ -931,14 +975,14 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     for (int k = 0; k < NIB; k++) {
                         const int r = it0 + k * W;
                         if (r < nI) {                                           // uniform in the wave
-                            ld_row<Q4, CBD>(wrow<Q4>(L.gate, L.sgate, r, dim), nchD, lane, 0, wr[k][0]);
-                            ld_row<Q4, CBD>(wrow<Q4>(L.up, L.sup, r, dim), nchD, lane, 0, wr[k][1]);
+                            ld_row<GL, Q4, CBD>(wrow<Q4>(L.gate, L.sgate, r, dim), nchD, lane, 0, wr[k][0]);
+                            ld_row<GL, Q4, CBD>(wrow<Q4>(L.up, L.sup, r, dim), nchD, lane, 0, wr[k][1]);
                         }
                     }
-                    if (lane < NIB) { const int r = min(it0 + lane * W, nI - 1); sg = Q4 ? 1.f : L.sgate[r]; su = Q4 ? 1.f : L.sup[r]; }
+                    if (lane < NIB) { const int r = min(it0 + lane * W, nI - 1); sg = Q4 ? 1.f : ldg_f<GL>(L.sgate, r); su = Q4 ? 1.f : ldg_f<GL>(L.sup, r); }
                 };
                 if (gw < nI) issue(gw);
-                const float rs = stage_rms<Q4>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                const float rs = stage_rms<GL, Q4>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
                 FLOW_TRACE(7);
                 for (int it0 = gw; it0 < nI; it0 += NIB * W) {
                     if (it0 != gw) issue(it0);
@@ -951,7 +995,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             if (nchD > CBD * 64) {
                                 const int r = it0 + k * W;
                                 const WRow rows[2] = {wrow<Q4>(L.gate, L.sgate, r, dim), wrow<Q4>(L.up, L.sup, r, dim)};
-                                dot_rows_tail<Q4, 2, CBD>(rows, a4, nchD, lane, acc);
+                                dot_rows_tail<GL, Q4, 2, CBD>(rows, a4, nchD, lane, acc);
                             }
                             const float t = wave_sum2(acc[0], acc[1]);
                             acc[0] = lane_value(t, 0);
@@ -982,11 +1026,11 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     auto issueStep = [&](int4 (&set)[1][CB], int st) {
                         const int sc = min(st, T - 1);
                         const int k = sc / nb, b = sc - k * nb;
-                        ld_row<Q4, CB>(wrow<Q4>(L.down, L.sdown, gw + k * W, ffn), nchF, lane, b * CB * 64, set[0]);
+                        ld_row<GL, Q4, CB>(wrow<Q4>(L.down, L.sdown, gw + k * W, ffn), nchF, lane, b * CB * 64, set[0]);
                     };
                     float e0 = 0.f, e1 = 0.f;
                     if (T > 0) {
-                        if (lane < nItems) { const int r = gw + lane * W; e0 = Q4 ? 1.f : L.sdown[r]; e1 = poll1(X + G.offX1 + r, wt); }
+                        if (lane < nItems) { const int r = gw + lane * W; e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r); e1 = poll1(X + G.offX1 + r, wt); }
 #pragma unroll
                         for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
                     }
@@ -1024,18 +1068,18 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     const int c0 = hf ? nHalf : 0, cHi = hf ? nchF : nHalf;
                     const WRow rw = wrow<Q4>(L.down, L.sdown, row, ffn);
                     int4 wr[CBH];
-                    ld_row_rng<Q4, CBH>(rw, cHi, lane, c0, wr);
+                    ld_row_rng<GL, Q4, CBH>(rw, cHi, lane, c0, wr);
                     float e0 = 0.f, e1 = 0.f;
                     if (wave == 0 && lane < FWAVES / 2) {
                         const int r = min((int)blockIdx.x * (FWAVES / 2) + lane, nI - 1);
-                        e0 = Q4 ? 1.f : L.sdown[r];
+                        e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r);
                         e1 = poll1(X + G.offX1 + r, wt);
                     }
                     stage_plain<Q4>(X + G.offM, ffn, a4, wt);
                     FLOW_TRACE(9);
                     float acc = dot_row_rng<Q4, CBH>(wr, a4, nchF, cHi, lane, c0, 0.f);
                     for (int cc = c0 + CBH * 64; cc < cHi; cc += CBH * 64) {
-                        ld_row_rng<Q4, CBH>(rw, cHi, lane, cc, wr);
+                        ld_row_rng<GL, Q4, CBH>(rw, cHi, lane, cc, wr);
                         acc = dot_row_rng<Q4, CBH>(wr, a4, nchF, cHi, lane, cc, acc);
                     }
                     acc = wave_sum(acc);
@@ -1058,9 +1102,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
 #pragma unroll
                     for (int k = 0; k < NID; k++) {
                         const int r = it0 + k * W;
-                        if (r < nI) ld_row<Q4, CBF>(wrow<Q4>(L.down, L.sdown, r, ffn), nchF, lane, 0, wr[k][0]);      // uniform in the wave
+                        if (r < nI) ld_row<GL, Q4, CBF>(wrow<Q4>(L.down, L.sdown, r, ffn), nchF, lane, 0, wr[k][0]);      // uniform in the wave
                     }
-                    if (lane < NID) { const int r = min(it0 + lane * W, nI - 1); e0 = Q4 ? 1.f : L.sdown[r]; e1 = poll1(X + G.offX1 + r, wt); }
+                    if (lane < NID) { const int r = min(it0 + lane * W, nI - 1); e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r); e1 = poll1(X + G.offX1 + r, wt); }
                 };
                 if (gw < nI) issue(gw);
                 stage_plain<Q4>(X + G.offM, ffn, a4, wt);
@@ -1075,7 +1119,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             dot_rows<Q4, 1, CBF>(wr[k], a4, nchF, lane, 0, acc);
                             if (nchF > CBF * 64) {
                                 const WRow rows[1] = {wrow<Q4>(L.down, L.sdown, it0 + k * W, ffn)};
-                                dot_rows_tail<Q4, 1, CBF>(rows, a4, nchF, lane, acc);
+                                dot_rows_tail<GL, Q4, 1, CBF>(rows, a4, nchF, lane, acc);
                             }
                             acc[0] = wave_sum(acc[0]);
                         }
