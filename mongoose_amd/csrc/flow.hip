@@ -922,7 +922,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 // Long rows, several items a wave: the rows stream through a ring of register sets, the loads of step
                 // s + RD - 1 are issued before step s is multiplied (a step = one item's two rows x CB chunks a lane).
                 if (blockIdx.x * FWAVES < nI) {
-                    constexpr int RD = 4, CB = 2;
+                    constexpr int RD = 3, CB = 2;
                     int4 ring[RD][2][CB];
                     const int nItems = gw < nI ? (nI - gw + W - 1) / W : 0;
                     const int nb = (nchD + 64 * CB - 1) / (64 * CB);
