@@ -265,8 +265,8 @@ int mg_hidden_idx(mg_ctx* ctx);
  * In mode 3, 32 of the launch's workgroups compute nothing and instead read the weights that the others
  * will want next into the L2s, where a layer is small enough for that to pay (0.5B shape: 8 % faster);
  * 4 = mode 3 with every workgroup computing (bit-identical results; for comparison).
- * A new context is in mode 3 (measured against mode 1: 0.5B shape 53 % more tokens per second, 1.1B
- * shape 52 %, 8B shape 14 %, also at contexts of thousands of positions).
+ * A new context is in mode 3 (measured against mode 1: 0.5B shape 56 % more tokens per second, 1.1B
+ * shape 59 %, 8B shape 20 %, also at contexts of thousands of positions).
  * On every device one context at a time uses the persistent launch -- the first that needs it, until it is
  * destroyed or set to another mode; other contexts run the fused launches meanwhile (two such launches at
  * once could each hold part of the CUs and wait for workgroups that cannot start).
