@@ -194,6 +194,62 @@ __device__ __forceinline__ void poll_batch(const f4* const (&ptr)[PB], f4 (&v)[P
     }
 }
 
+// The same for up to eight pieces (the 8B shape's down projection takes 14336 staged values: seven pieces a thread,
+// three rounds of poll_batch -- three dependent round trips; this is one).
+constexpr int PBW = 8;
+__device__ __forceinline__ void ldx4_w(const f4* const (&p)[PBW], f4 (&v)[PBW], int n) {
+    switch (n) {
+    case 1:
+        asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]) : "v"(p[0]) : "memory");
+        break;
+    case 2:
+        asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %3, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]) : "v"(p[0]), "v"(p[1]) : "memory");
+        break;
+    case 3:
+        asm volatile("global_load_dwordx4 %0, %3, off sc1\n\tglobal_load_dwordx4 %1, %4, off sc1\n\tglobal_load_dwordx4 %2, %5, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]) : "v"(p[0]), "v"(p[1]), "v"(p[2]) : "memory");
+        break;
+    case 4:
+        asm volatile("global_load_dwordx4 %0, %4, off sc1\n\tglobal_load_dwordx4 %1, %5, off sc1\n\tglobal_load_dwordx4 %2, %6, off sc1\n\tglobal_load_dwordx4 %3, %7, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]) : "memory");
+        break;
+    case 5:
+        asm volatile("global_load_dwordx4 %0, %5, off sc1\n\tglobal_load_dwordx4 %1, %6, off sc1\n\tglobal_load_dwordx4 %2, %7, off sc1\n\tglobal_load_dwordx4 %3, %8, off sc1\n\tglobal_load_dwordx4 %4, %9, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]) : "memory");
+        break;
+    case 6:
+        asm volatile("global_load_dwordx4 %0, %6, off sc1\n\tglobal_load_dwordx4 %1, %7, off sc1\n\tglobal_load_dwordx4 %2, %8, off sc1\n\tglobal_load_dwordx4 %3, %9, off sc1\n\tglobal_load_dwordx4 %4, %10, off sc1\n\tglobal_load_dwordx4 %5, %11, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]) : "memory");
+        break;
+    case 7:
+        asm volatile("global_load_dwordx4 %0, %7, off sc1\n\tglobal_load_dwordx4 %1, %8, off sc1\n\tglobal_load_dwordx4 %2, %9, off sc1\n\tglobal_load_dwordx4 %3, %10, off sc1\n\tglobal_load_dwordx4 %4, %11, off sc1\n\tglobal_load_dwordx4 %5, %12, off sc1\n\tglobal_load_dwordx4 %6, %13, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]) : "memory");
+        break;
+    case 8:
+        asm volatile("global_load_dwordx4 %0, %8, off sc1\n\tglobal_load_dwordx4 %1, %9, off sc1\n\tglobal_load_dwordx4 %2, %10, off sc1\n\tglobal_load_dwordx4 %3, %11, off sc1\n\tglobal_load_dwordx4 %4, %12, off sc1\n\tglobal_load_dwordx4 %5, %13, off sc1\n\tglobal_load_dwordx4 %6, %14, off sc1\n\tglobal_load_dwordx4 %7, %15, off sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]) : "memory");
+        break;
+    default: break;
+    }
+}
+__device__ __forceinline__ void poll_batch_w(const f4* const (&ptr)[PBW], f4 (&v)[PBW], int n, Waiter& w) {
+    long long t0 = 0;
+    bool timing = false;
+    if (n <= 0) return;
+    for (;;) {
+        ldx4_w(ptr, v, n);
+        bool ok = true;
+#pragma unroll
+        for (int i = 0; i < PBW; i++) ok = ok && (i >= n || ready4(v[i]));
+        if (ok || w.dead) break;
+        if (!timing) { timing = true; t0 = wall_clock64(); }
+        else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
+        for (int z = 0; z < 8; z++) __builtin_amdgcn_s_sleep(2);
+    }
+}
+
 // planar LDS layout of an activation vector for 16-weight chunks (as the matvec kernels use): lane c reads
 // a4[pl * nch + c], pl = 0..3.  Q8: a chunk is 16 consecutive weights, float4 k4 of the vector sits at
 // (k4 & 3) * nch + (k4 >> 2).  Q4_0: a chunk is half a block (8 bytes: low nibbles = elements 8h..8h+7 of the block,
@@ -266,6 +322,27 @@ __device__ __forceinline__ void stage_plain(const float* x, int K, float4* a4, W
         poll_batch(ptr, v, max(0, min(PB, (K4 - base - tid + FWG - 1) / FWG)), w);
 #pragma unroll
         for (int u = 0; u < PB; u++) {
+            const int i = base + u * FWG + tid;
+            if (i < K4) a4[slot4<Q4>(i, nch)] = tof4(v[u]);
+        }
+    }
+    __syncthreads();
+}
+
+// stage_plain with up to eight pieces a thread in one round trip.
+template <bool Q4>
+__device__ __forceinline__ void stage_plain_w(const float* x, int K, float4* a4, Waiter& w) {
+    const int K4 = K >> 2, nch = K >> 4, tid = threadIdx.x;
+    const f4* x4 = reinterpret_cast<const f4*>(x);
+    __syncthreads();
+    for (int base = 0; base < K4; base += FWG * PBW) {
+        f4 v[PBW];
+        const f4* ptr[PBW];
+#pragma unroll
+        for (int u = 0; u < PBW; u++) { ptr[u] = x4 + min(base + u * FWG + tid, K4 - 1); v[u] = f4{0.f, 0.f, 0.f, 0.f}; }
+        poll_batch_w(ptr, v, max(0, min(PBW, (K4 - base - tid + FWG - 1) / FWG)), w);
+#pragma unroll
+        for (int u = 0; u < PBW; u++) {
             const int i = base + u * FWG + tid;
             if (i < K4) a4[slot4<Q4>(i, nch)] = tof4(v[u]);
         }
@@ -1034,7 +1111,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
 #pragma unroll
                         for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
                     }
-                    stage_plain<Q4>(X + G.offM, ffn, a4, wt);
+                    stage_plain_w<Q4>(X + G.offM, ffn, a4, wt);
                     FLOW_TRACE(9);
                     float acc[1] = {0.f};
                     float v = 0.f;
