@@ -258,6 +258,24 @@ def test_heads_of_128_grouped_kv(hip):
     m.close()
 
 
+@pytest.mark.parametrize("ffn", [15360, 9216])
+def test_streamed_rows_wide_ffn(hip, ffn):
+    """Rows of 4096 weights with the widest FFN the launch takes (15360: seven or eight staged pieces a thread for the
+    down projection, seven or eight rounds of gate|up rows) and one whose pieces do not come out even (9216: four or five a thread):
+    tokens against the oracle, then against the fused launches at two KV splits."""
+    s = H.with_layers(configs.LLAMA3_8B, 2)._replace(name=f"l3-ffn{ffn}", ffnDim=ffn, vocab=1024, tied=True)
+    m = H.Model(s, seed=31, maxSeq=200, eng=hip, threads=16)
+    print(f"flow: rows of 4096, ffn {ffn}, 4 + 6 against the oracle", flush=True)
+    prompt = m.prompt(4)
+    ref, _ = H.oracle_generate(m, prompt, 6)
+    rc, t = m.hip.Generate(prompt, 6, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert _in_use(m.hip)
+    assert t.tolist() == ref.tolist(), H.first_divergence(t, ref)
+    _modes_agree(m, m.prompt(140), 20, f"ffn {ffn}, 2 splits")
+    m.close()
+
+
 def test_new_context_uses_the_launch_and_trace(hip):
     s = H.with_layers(configs.TOY, 8)
     m = H.Model(s, seed=5, maxSeq=40, eng=hip, threads=8)
