@@ -276,6 +276,28 @@ def test_streamed_rows_wide_ffn(hip, ffn):
     m.close()
 
 
+@pytest.mark.parametrize("fmt", ["q8", "q4_0"])
+@pytest.mark.parametrize("name,dim,heads,kv,hd,ffn", [
+    ("rows-3072", 3072, 24, 8, 128, 8192),      # streamed rows whose second request a lane is half empty
+    ("rows-1536", 1536, 24, 4, 64, 4096),       # two requests a lane, the second used by half the lanes
+    ("rows-640", 640, 10, 2, 64, 1792),         # one request a lane, partly used
+])
+def test_row_lengths_between_the_tuned_ones(hip, fmt, name, dim, heads, kv, hd, ffn):
+    """Row lengths that are not a whole number of 1024-weight requests: tokens against the oracle through the
+    persistent launch, then against the fused launches at two KV splits."""
+    s = configs.Shape(name, 2, dim, heads, kv, hd, ffn, 1024, 1e-5, 5e5, True, True, "q8")
+    m = H.Model(s, seed=37, maxSeq=200, eng=hip, threads=16, fmt=fmt)
+    print(f"flow: {name} {fmt}, 4 + 6 against the oracle", flush=True)
+    prompt = m.prompt(4)
+    ref, _ = H.oracle_generate(m, prompt, 6)
+    rc, t = m.hip.Generate(prompt, 6, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert _in_use(m.hip)
+    H.assert_same_tokens_or_near_tie(m, prompt, t, ref, f"{name} {fmt}")
+    _modes_agree(m, m.prompt(140), 20, f"{name} {fmt}, 2 splits")
+    m.close()
+
+
 def test_new_context_uses_the_launch_and_trace(hip):
     s = H.with_layers(configs.TOY, 8)
     m = H.Model(s, seed=5, maxSeq=40, eng=hip, threads=8)
