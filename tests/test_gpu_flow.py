@@ -9,6 +9,7 @@ their vectors over through an exchange area in device memory.
 * heads of 128 with grouped KV heads;
 * Q4_0 matrices (split layout, half-block chunks) through the same launch: every handed-over vector, tokens against
   the oracle, rows of one and of two chunks a lane, the ring variant, biases;
+* the widest FFN the launch takes, an FFN whose staged pieces come out uneven, row lengths between the tuned shapes;
 * a new context uses the launch; the trace diagnostic;
 * a wait that runs out: the launch still ends, the call reports it, the context continues with the fused launches.
 """
