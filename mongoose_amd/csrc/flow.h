@@ -40,6 +40,8 @@ struct FlowGeometry {
 FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int nKVHeads, int headDim, int maxSeq, int grid);
 bool flow_context_fits(int maxSeq, const FlowGeometry& g);
 
+constexpr size_t FLOW_ERR_BYTES = 4096;
+
 // Trace slots of a layer, in program order: when thread 0 of a workgroup passed the point.
 constexpr int FLOW_TRACE_SLOTS = 11;
 #define FLOW_TRACE_NAMES "layer-top", "qkv-input-staged", "qkv-done", "q-k-v-rows-in", "attention-done", "attention-merged", \
@@ -62,7 +64,8 @@ struct FlowParams {
     float* hidden;               // input of layer l0 and output of layer l1-1 [dim]
     float* xchg;                 // exchange area, geo.stride floats per layer (indexed by layer)
     FlowGeometry geo;
-    int* err;                    // set to 1 when a wait ran into its time limit
+    int* err;                    // FLOW_ERR_BYTES of zeros: word 0 is set to 1 when a wait ran into its time limit; bytes
+                                 // 256 .. 2304 are the idle lines (never written; polls with nothing to ask for go there)
     long long limitTicks;        // per wait, in ticks of the 100 MHz wall clock
     long long* trace;            // optional (diagnostic): wall-clock ticks [layer][FLOW_TRACE_SLOTS][workgroup], see FLOW_TRACE_NAMES
 };
@@ -73,6 +76,9 @@ int flow_prefetch_workgroups(int cus, size_t layerBytes, int dim, int kvDim, int
 // Computing workgroups the launch needs at least (one per query head and KV split) for this shape.
 int flow_min_grid(int nHeads, int nKVHeads, const FlowGeometry& g);
 bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads, int headDim);
+// With nCompute computing workgroups: no phase needs more rounds of the waves than the kernel holds results for, and
+// the grouped attention has a workgroup per query head for its merge.
+bool flow_grid_fits(int ffn, int nHeads, const FlowGeometry& g, int nCompute);
 // grid workgroups of 512 threads, all of which must be resident at once (grid <= CUs x resident workgroups per CU);
 // grid - p.nCompute of them prefetch (0, or a multiple of 8 with nCompute a multiple of 8 as well).
 hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s);

@@ -71,6 +71,7 @@ struct Waiter {
     long long limit;
     int* err;
     bool dead;
+    const f4* idle;      // a line nothing writes during the launch (see poll_batch)
     __device__ __forceinline__ void fail() {
         dead = true;
         __hip_atomic_store(err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -111,25 +112,16 @@ __device__ __forceinline__ float poll1(const float* p, Waiter& w) {
     }
     return v;
 }
-// The first n of three pieces with all their loads in flight at once: one memory round trip instead of n.
-// Loads and the wait for them are one asm statement each time -- with the wait in a statement of its own the
+// Three pieces with all their loads in flight at once: one memory round trip instead of three.
+// Loads and the wait for them are one asm statement -- with the wait in a statement of its own the
 // compiler is free to copy a destination register between the two, i.e. before the data has arrived.
-__device__ __forceinline__ void ldx4_n(const f4* const (&p)[3], f4 (&v)[3], int n) {
-    switch (n) {
-    case 1:
-        asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(v[0]) : "v"(p[0]) : "memory");
-        break;
-    case 2:
-        asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %3, off sc1\n\ts_waitcnt vmcnt(0)"
-                     : "=&v"(v[0]), "=&v"(v[1]) : "v"(p[0]), "v"(p[1]) : "memory");
-        break;
-    default:
-        asm volatile("global_load_dwordx4 %0, %3, off sc1\n\tglobal_load_dwordx4 %1, %4, off sc1\n\t"
-                     "global_load_dwordx4 %2, %5, off sc1\n\ts_waitcnt vmcnt(0)"
-                     : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]) : "v"(p[0]), "v"(p[1]), "v"(p[2]) : "memory");
-        break;
-    }
+__device__ __forceinline__ void ldx4_3(const f4* const (&p)[3], f4 (&v)[3]) {
+    asm volatile("global_load_dwordx4 %0, %3, off sc1\n\tglobal_load_dwordx4 %1, %4, off sc1\n\t"
+                 "global_load_dwordx4 %2, %5, off sc1\n\ts_waitcnt vmcnt(0)"
+                 : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]) : "v"(p[0]), "v"(p[1]), "v"(p[2]) : "memory");
 }
+__device__ __forceinline__ unsigned unset1(float v) { return __builtin_bit_cast(unsigned, v) == XSENT ? 1u : 0u; }
+__device__ __forceinline__ unsigned unset4(f4 v) { return unset1(v.x) | unset1(v.y) | unset1(v.z) | unset1(v.w); }
 // A KV split's partial for one 16-byte piece of the attention output: accumulator piece, maximum and sum of its head,
 // asked for together (one round trip), repeated until all three are there.
 __device__ __forceinline__ void poll_partial(const f4* pa, const float* pm, const float* pl, f4& a, float& m, float& l, Waiter& w) {
@@ -139,7 +131,8 @@ __device__ __forceinline__ void poll_partial(const f4* pa, const float* pm, cons
         asm volatile("global_load_dwordx4 %0, %3, off sc1\n\tglobal_load_dword %1, %4, off sc1\n\t"
                      "global_load_dword %2, %5, off sc1\n\ts_waitcnt vmcnt(0)"
                      : "=&v"(a), "=&v"(m), "=&v"(l) : "v"(pa), "v"(pm), "v"(pl) : "memory");
-        if ((ready4(a) && !unset(m) && !unset(l)) || w.dead) break;
+        const unsigned missing = unset4(a) | unset1(m) | unset1(l);
+        if (!missing || w.dead) break;
         if (!timing) { timing = true; t0 = wall_clock64(); }
         else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
     }
@@ -173,19 +166,35 @@ __device__ __forceinline__ FlowLayer unpack_layer(unsigned v) {
 #undef FL_PTR
 
 constexpr int PB = 3;        // float4 pieces a thread polls at once (a round of the 512 threads covers 6144 floats)
-// n: this thread's pieces of the round, 0..PB (a thread past the end of the vector asks for nothing: clamped to the
-// last piece instead, hundreds of threads of every workgroup would re-read that one line while its producers are
-// still storing to it); pieces past n are left as they are
+// Every polling loop here has one shape: a straight loop around ONE asm statement (a fixed number of loads and their
+// wait), whose results are tested together as one word; nothing inside the loop chooses between asm statements.
+// poll_batch always asks for PB pieces: a thread with fewer pieces of the vector left (n < PB) points the others at its
+// workgroup's idle line (Waiter::idle: memory that nothing writes during the launch, so those loads hit in the L2
+// and never in a line that producers are storing to) and ignores what comes back.  A thread with no piece at all
+// asks for nothing: clamped to the vector's last piece instead, hundreds of threads of every workgroup would re-read
+// that one line while its producers are still storing to it.
+// SINGLE (fixed where the kernel variant is chosen): the vector has at most one piece a thread (512 pieces), and the
+// loop asks for one.
+template <bool SINGLE>
 __device__ __forceinline__ void poll_batch(const f4* const (&ptr)[PB], f4 (&v)[PB], int n, Waiter& w) {
+    static_assert(PB == 3, "the readiness word below names three pieces");
     long long t0 = 0;
     bool timing = false;
     if (n <= 0) return;
+    if constexpr (SINGLE) {
+        for (;;) {
+            v[0] = ldx4(ptr[0]);
+            if (!unset4(v[0]) || w.dead) break;
+            if (!timing) { timing = true; t0 = wall_clock64(); }
+            else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
+            for (int z = 0; z < 8; z++) __builtin_amdgcn_s_sleep(2);
+        }
+        return;
+    }
     for (;;) {
-        ldx4_n(ptr, v, n);
-        bool ok = true;
-#pragma unroll
-        for (int i = 0; i < PB; i++) ok = ok && (i >= n || ready4(v[i]));
-        if (ok || w.dead) break;
+        ldx4_3(ptr, v);
+        const unsigned missing = unset4(v[0]) | (n > 1 ? unset4(v[1]) : 0u) | (n > 2 ? unset4(v[2]) : 0u);
+        if (!missing || w.dead) break;
         if (!timing) { timing = true; t0 = wall_clock64(); }
         else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
         // 256 workgroups re-reading a vector load the lines its producers are still storing to: a pause of ~0.4 us
@@ -234,19 +243,33 @@ __device__ __forceinline__ void ldx4_w(const f4* const (&p)[PBW], f4 (&v)[PBW], 
     default: break;
     }
 }
-__device__ __forceinline__ void poll_batch_w(const f4* const (&ptr)[PBW], f4 (&v)[PBW], int n, Waiter& w) {
+template <int N>
+__device__ __forceinline__ void poll_fixed_w(const f4* const (&ptr)[PBW], f4 (&v)[PBW], Waiter& w) {
     long long t0 = 0;
     bool timing = false;
-    if (n <= 0) return;
     for (;;) {
-        ldx4_w(ptr, v, n);
-        bool ok = true;
+        ldx4_w(ptr, v, N);
+        unsigned missing = 0;
 #pragma unroll
-        for (int i = 0; i < PBW; i++) ok = ok && (i >= n || ready4(v[i]));
-        if (ok || w.dead) break;
+        for (int i = 0; i < N; i++) missing |= unset4(v[i]);
+        if (!missing || w.dead) break;
         if (!timing) { timing = true; t0 = wall_clock64(); }
         else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
         for (int z = 0; z < 8; z++) __builtin_amdgcn_s_sleep(2);
+    }
+}
+__device__ __forceinline__ void poll_batch_w(const f4* const (&ptr)[PBW], f4 (&v)[PBW], int n, Waiter& w) {
+    static_assert(PBW == 8, "one case per batch size");
+    switch (n < PBW ? n : PBW) {
+    case 1: poll_fixed_w<1>(ptr, v, w); break;
+    case 2: poll_fixed_w<2>(ptr, v, w); break;
+    case 3: poll_fixed_w<3>(ptr, v, w); break;
+    case 4: poll_fixed_w<4>(ptr, v, w); break;
+    case 5: poll_fixed_w<5>(ptr, v, w); break;
+    case 6: poll_fixed_w<6>(ptr, v, w); break;
+    case 7: poll_fixed_w<7>(ptr, v, w); break;
+    case 8: poll_fixed_w<8>(ptr, v, w); break;
+    default: break;
     }
 }
 
@@ -263,7 +286,8 @@ __device__ __forceinline__ int slot4(int k4, int nch) {
 __device__ __forceinline__ float4 tof4(f4 v) { return make_float4(v.x, v.y, v.z, v.w); }
 
 // x (optionally polled) -> LDS as x * gain; returns 1/rms.  Leaves with a barrier done.
-template <bool GL, bool Q4>
+// SINGLE: K <= 2048, one piece a thread
+template <bool GL, bool Q4, bool SINGLE>
 __device__ __forceinline__ float stage_rms(const float* x, bool polled, const float* gain, int K, float eps, float4* a4,
                                            float* red, Waiter& w) {
     const int K4 = K >> 2, nch = K >> 4, tid = threadIdx.x;
@@ -277,15 +301,15 @@ __device__ __forceinline__ float stage_rms(const float* x, bool polled, const fl
         const f4* ptr[PB];
 #pragma unroll
         for (int u = 0; u < PB; u++) {
-            const int i = min(base + u * FWG + tid, K4 - 1);
-            ptr[u] = x4 + i;
-            g[u] = ldg_f4<GL>(g4, i);
+            const int i = base + u * FWG + tid;
+            ptr[u] = i < K4 ? x4 + i : w.idle;
+            g[u] = ldg_f4<GL>(g4, min(i, K4 - 1));
         }
         const int np = max(0, min(PB, (K4 - base - tid + FWG - 1) / FWG));      // this thread's pieces of the round
 #pragma unroll
         for (int u = 0; u < PB; u++) v[u] = f4{0.f, 0.f, 0.f, 0.f};
         if (polled) {
-            poll_batch(ptr, v, np, w);
+            poll_batch<SINGLE>(ptr, v, np, w);
         } else {
 #pragma unroll
             for (int u = 0; u < PB; u++) if (u < np) v[u] = *ptr[u];
@@ -309,7 +333,7 @@ __device__ __forceinline__ float stage_rms(const float* x, bool polled, const fl
 }
 
 // polled x -> LDS.  Leaves with a barrier done.
-template <bool Q4>
+template <bool Q4, bool SINGLE>
 __device__ __forceinline__ void stage_plain(const float* x, int K, float4* a4, Waiter& w) {
     const int K4 = K >> 2, nch = K >> 4, tid = threadIdx.x;
     const f4* x4 = reinterpret_cast<const f4*>(x);
@@ -318,8 +342,8 @@ __device__ __forceinline__ void stage_plain(const float* x, int K, float4* a4, W
         f4 v[PB];
         const f4* ptr[PB];
 #pragma unroll
-        for (int u = 0; u < PB; u++) { ptr[u] = x4 + min(base + u * FWG + tid, K4 - 1); v[u] = f4{0.f, 0.f, 0.f, 0.f}; }
-        poll_batch(ptr, v, max(0, min(PB, (K4 - base - tid + FWG - 1) / FWG)), w);
+        for (int u = 0; u < PB; u++) { const int i = base + u * FWG + tid; ptr[u] = i < K4 ? x4 + i : w.idle; v[u] = f4{0.f, 0.f, 0.f, 0.f}; }
+        poll_batch<SINGLE>(ptr, v, max(0, min(PB, (K4 - base - tid + FWG - 1) / FWG)), w);
 #pragma unroll
         for (int u = 0; u < PB; u++) {
             const int i = base + u * FWG + tid;
@@ -448,15 +472,17 @@ __device__ __forceinline__ void dot_rows_tail(const WRow (&rows)[NR], const floa
 // workgroup i on XCD i & 7; the eight waves of computing workgroup w take rows 8g .. 8g+7 of a matrix for every run
 // g with g % nC == w, so with nC a multiple of 8 run g belongs to XCD g & 7.
 // ---------------------------------------------------------------------------------------------------------------
-typedef int pfv4 __attribute__((ext_vector_type(4)));
+// The fetches are loads straight into LDS (global_load_lds_dwordx4: 1 KB a wave and instruction, no destination
+// register), all into one 1 KB scrap area that nothing reads: nothing the compiler allocates can be overwritten
+// by a load that returns late, whatever it does with its registers between the issue and the wait.
 struct Prefetcher {
     int x, rank, nRank, tid;     // XCD, this workgroup among the XCD's prefetchers, their number, thread
-    pfv4 sink;
+    int4* scrap;                 // LDS, 1 KB
     // bytes [b0, b1) of base, 16 bytes a thread and step; b0 a multiple of 16, the tail rounded down
     __device__ __forceinline__ void span(const char* base, size_t b0, size_t b1) {
         b1 &= ~(size_t)15;
         for (size_t o = b0 + (size_t)tid * 16; o < b1; o += (size_t)FWG * 16)
-            asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(sink) : "v"(base + o) : "memory");
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const int4*>(base + o), scrap, 16, 0, 0);
     }
     // runs of `run` rows of rowBytes each; run g of the matrix goes to XCD g & 7, then to the XCD's prefetchers in turn
     __device__ __forceinline__ void rows(const void* base, size_t rowBytes, int nRows, int run) {
@@ -473,7 +499,8 @@ struct Prefetcher {
         if (!base || rank != 0) return;
         span(static_cast<const char*>(base), 0, bytes);
     }
-    __device__ __forceinline__ void drain() { asm volatile("s_waitcnt vmcnt(0)" : "+v"(sink) : : "memory"); }
+    // everything requested so far has landed (in the L2 on its way): nothing of it can arrive in the scrap area later
+    __device__ __forceinline__ void drain() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 };
 
 constexpr int FLOW_MAX_ROUNDS = 8;   // rows of a matrix a wave takes at most (rounds of all waves over the matrix)
@@ -498,6 +525,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     __shared__ float4 accbuf[QHMAX][FWAVES][HD / 4];   // per query head of the workgroup: the waves' partial outputs, sums, maxima
     __shared__ float lbuf[QHMAX][FWAVES], wred[QHMAX][FWAVES];
     __shared__ float outbuf[FLOW_MAX_ROUNDS][FWAVES];                // a phase's results of the workgroup, stored by one wave as whole 32-byte runs
+    __shared__ int4 pfScrap[64];                       // where the prefetching loads land (never read)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -526,12 +554,13 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     const int nchD = dim >> 4, nchF = ffn >> 4;
     const FlowGeometry G = p.geo;
     const int pos = p.state ? p.state->pos : p.posImm;
-    Waiter wt{p.limitTicks, p.err, false};
+    // (the idle lines follow the error word's 256 bytes: 16 lines of 128 bytes, two workgroups of an XCD on each)
+    Waiter wt{p.limitTicks, p.err, false, reinterpret_cast<const f4*>(reinterpret_cast<const char*>(p.err) + 256 + ((blockIdx.x >> 3) & 15) * 128)};
 
     if ((int)blockIdx.x >= nC) {
         // ---- prefetch role (see Prefetcher): per layer three jobs, each released by a vector of the layer before ----
         const int pi = (int)blockIdx.x - nC;
-        Prefetcher pf{pi & 7, pi >> 3, ((int)gridDim.x - nC) >> 3, tid, {0, 0, 0, 0}};
+        Prefetcher pf{pi & 7, pi >> 3, ((int)gridDim.x - nC) >> 3, tid, pfScrap};
         const size_t rbD = Q4 ? dim >> 1 : dim, rbF = Q4 ? ffn >> 1 : ffn;      // bytes of a row of dim / of ffn weights
         const size_t rdD = dim >> 4, rdF = ffn >> 4;                             // ... of its fp16 d values (Q4_0)
         const int halfHd = HD >> 1;
@@ -543,7 +572,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             // (Measured at the 0.5B shape: releasing every job a phase earlier or later, and 24 to 48 prefetching
             // workgroups, all give the same step time within 0.5 %; 16 are too few, 64 cost more than they bring.)
             auto release = [&](int off) {
-                pf.drain();                // the job before has landed (its loads' destination register is still pf.sink)
+                pf.drain();                // the job before has landed
                 if (l == p.l0) return;
                 if (tid == 0) (void)poll1(Xp + off, wt);
                 __syncthreads();
@@ -683,7 +712,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     kind[q] = 0; r0[q] = 0; r1[q] = 0; e0[q] = 0.f; e1[q] = 0.f; rows[q][0] = wrow<Q4>(L.wq, L.sq, 0, dim); rows[q][1] = rows[q][0];
                     if (gw + q * W < nI) resolve(wr[q], rows[q], kind[q], r0[q], r1[q], e0[q], e1[q], gw + q * W);
                 }
-                const float rs = stage_rms<GL, Q4>(xin, !first, L.g1, dim, p.eps, a4, red, wt);
+                const float rs = stage_rms<GL, Q4, !RING>(xin, !first, L.g1, dim, p.eps, a4, red, wt);
                 FLOW_TRACE(1);
 #pragma unroll
                 for (int q = 0; q < NPI; q++)
@@ -732,7 +761,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 if (grouped && nBusy < p.nHeads) nBusy = p.nHeads;
                 nBusy = (nBusy + 7) & ~7;
                 if ((int)blockIdx.x >= nBusy && 2 * ((int)gridDim.x - nBusy) >= (int)gridDim.x) {
-                    Prefetcher pf{(int)blockIdx.x & 7, ((int)blockIdx.x - nBusy) >> 3, ((int)gridDim.x - nBusy) >> 3, tid, {0, 0, 0, 0}};
+                    Prefetcher pf{(int)blockIdx.x & 7, ((int)blockIdx.x - nBusy) >> 3, ((int)gridDim.x - nBusy) >> 3, tid, pfScrap};
                     const size_t rbD = Q4 ? dim >> 1 : dim, rdD = dim >> 4;
                     // (a workgroup without q | k | v rows gets here at the top of the layer; holding it back until q | k | v is
                     // through measures slower: 1.1B shape 0.453 against 0.435 ms a token)
@@ -877,7 +906,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     long long t0w = 0;
                     bool timing = false;
                     for (;;) {
-                        bool ok = true;
+                        unsigned missing = 0;
 #pragma unroll
                         for (int j = 0; j < MBG; j++) {
                             const int sj = min(s1 + j * SG, ns - 1);
@@ -886,8 +915,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             ls[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, (Xo + G.offPl + sj * p.nHeads + h) * 4u, 0, 16));
                         }
 #pragma unroll
-                        for (int j = 0; j < MBG; j++) ok = ok && ready4(a[j]) && !unset(ms[j]) && !unset(ls[j]);
-                        if (ok || wt.dead) break;
+                        for (int j = 0; j < MBG; j++) missing |= unset4(a[j]) | unset1(ms[j]) | unset1(ls[j]);
+                        if (!missing || wt.dead) break;
                         if (!timing) { timing = true; t0w = wall_clock64(); }
                         else if (wall_clock64() - t0w > wt.limit) { wt.fail(); break; }
                         for (int z = 0; z < 4; z++) __builtin_amdgcn_s_sleep(2);
@@ -942,7 +971,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 if (it < nI) resolve(it);
                 // stage the attention output: merge the KV splits' partials (running maximum, as the split-KV combine)
                 if (grouped) {
-                    stage_plain<Q4>(X + G.offAttn, dim, a4, wt);      // merged per head above
+                    stage_plain<Q4, !RING>(X + G.offAttn, dim, a4, wt);      // merged per head above
                 } else {
                 __syncthreads();
                 {
@@ -1017,7 +1046,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
                         if (lane < nItems) { const int r = gw + lane * W; sg = Q4 ? 1.f : ldg_f<GL>(L.sgate, r); su = Q4 ? 1.f : ldg_f<GL>(L.sup, r); }
                     }
-                    const float rs = stage_rms<GL, Q4>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                    const float rs = stage_rms<GL, Q4, !RING>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
                     FLOW_TRACE(7);
                     float acc[2] = {0.f, 0.f};
                     float g = 0.f, u = 0.f;
@@ -1059,7 +1088,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     if (lane < NIB) { const int r = min(it0 + lane * W, nI - 1); sg = Q4 ? 1.f : ldg_f<GL>(L.sgate, r); su = Q4 ? 1.f : ldg_f<GL>(L.sup, r); }
                 };
                 if (gw < nI) issue(gw);
-                const float rs = stage_rms<GL, Q4>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                const float rs = stage_rms<GL, Q4, !RING>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
                 FLOW_TRACE(7);
                 for (int it0 = gw; it0 < nI; it0 += NIB * W) {
                     if (it0 != gw) issue(it0);
@@ -1152,7 +1181,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r);
                         e1 = poll1(X + G.offX1 + r, wt);
                     }
-                    stage_plain<Q4>(X + G.offM, ffn, a4, wt);
+                    stage_plain<Q4, false>(X + G.offM, ffn, a4, wt);
                     FLOW_TRACE(9);
                     float acc = dot_row_rng<Q4, CBH>(wr, a4, nchF, cHi, lane, c0, 0.f);
                     for (int cc = c0 + CBH * 64; cc < cHi; cc += CBH * 64) {
@@ -1184,7 +1213,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     if (lane < NID) { const int r = min(it0 + lane * W, nI - 1); e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r); e1 = poll1(X + G.offX1 + r, wt); }
                 };
                 if (gw < nI) issue(gw);
-                stage_plain<Q4>(X + G.offM, ffn, a4, wt);
+                stage_plain<Q4, false>(X + G.offM, ffn, a4, wt);
                 FLOW_TRACE(9);
                 for (int it0 = gw; it0 < nI; it0 += NID * W) {
                     if (it0 != gw) issue(it0);
@@ -1256,9 +1285,17 @@ int flow_min_grid(int nHeads, int nKVHeads, const FlowGeometry& g) { return (g.g
 // one workgroup per (query head, tile): the slots cover the context
 bool flow_context_fits(int maxSeq, const FlowGeometry& g) { return (long long)FLOW_TILE * g.smax >= maxSeq; }
 
+bool flow_grid_fits(int ffn, int nHeads, const FlowGeometry& g, int nCompute) {
+    if (nCompute <= 0) return false;
+    if ((ffn + nCompute * FWAVES - 1) / (nCompute * FWAVES) > FLOW_MAX_ROUNDS) return false;
+    if (g.gqa && nHeads > nCompute) return false;
+    return true;
+}
+
 bool flow_shape_supported(int dim, int kvDim, int ffn, int nHeads, int nKVHeads, int headDim) {
     if (headDim != 64 && headDim != 128) return false;
-    // the staged vector and the kernel's own 4 KB of LDS stay inside a 64 KB allocation
+    // LDS: the staged vector (dynamic, up to 60 KB) beside the kernel's own arrays (4 to 7 KB; 33 to 52 KB in the
+    // variants with grouped attention, which keep every query head's partials) stays inside the CU's 160 KB
     if (dim % 16 || ffn % 16 || kvDim % 16 || dim > 15360 || ffn > 15360) return false;
     if (nKVHeads <= 0 || nHeads % nKVHeads || nHeads * headDim != dim || nKVHeads * headDim != kvDim) return false;
     return true;
@@ -1270,7 +1307,7 @@ hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
     if (nC <= 0 || nC > grid || ((grid - nC) && (nC % 8 || (grid - nC) % 8))) return hipErrorInvalidValue;
     if (p.l0 < 0 || p.l1 <= p.l0 || p.l1 > p.nLayersTotal || nC < flow_min_grid(p.nHeads, p.nKVHeads, p.geo) ||
         !flow_context_fits(p.maxSeq, p.geo) || !p.layers || !p.xchg || !p.err || !p.hidden ||
-        (p.ffn + nC * FWAVES - 1) / (nC * FWAVES) > FLOW_MAX_ROUNDS || (size_t)p.nLayersTotal * p.geo.stride * 4 >= (1ull << 31))
+        !flow_grid_fits(p.ffn, p.nHeads, p.geo, nC) || (size_t)p.nLayersTotal * p.geo.stride * 4 >= (1ull << 31))
         return hipErrorInvalidValue;
     const size_t lds = (size_t)(p.dim > p.ffn ? p.dim : p.ffn) * sizeof(float);
     const bool wide = p.dim > 1024, ring = p.dim > 2048, gqa = p.geo.gqa != 0;

@@ -98,6 +98,7 @@ public:
     void SetExecMode(int mode) {
         if (mode != execMode) invalidateGraphs();
         if ((mode == 3 || mode == 4) && mode != execMode) flowRegeometry();    // the two differ in the launch's geometry
+        if (mode == 3 || mode == 4) flowBroken = false;      // asked for again by name: a wait that ran out earlier no longer bars it
         execMode = mode;
         if (mode != 0) q4ActQuant = false;      // only the op-by-op loop has the integer matvecs
         if (mode != 3 && mode != 4) releaseFlow();

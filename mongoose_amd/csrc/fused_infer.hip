@@ -649,6 +649,14 @@ static bool claim_flow(const HIPFusedInference* f, int dev) {
     return g_flowOwner[dev] == f;
 }
 void HIPFusedInference::releaseFlow() {
+    bool owner = false;
+    {
+        std::lock_guard<std::mutex> lk(g_flowOwnerMutex);
+        for (auto& o : g_flowOwner) if (o == this) owner = true;
+    }
+    if (!owner) return;
+    // the launch changes hands only once this context's last one has ended: the next owner's launch must not meet it on the GPU
+    if (stream) (void)hipStreamSynchronize(stream);
     std::lock_guard<std::mutex> lk(g_flowOwnerMutex);
     for (auto& o : g_flowOwner) if (o == this) o = nullptr;
 }
@@ -690,7 +698,9 @@ int HIPFusedInference::flowComputeWgs(int cus) const {
     const int tries[2] = {cus - pf, cus};
     for (int nC : tries) {
         const FlowGeometry g = flow_geometry(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim, maxSeq, nC);
-        if (flow_min_grid(nHeads, nKVHeads, g) <= nC && flow_context_fits(maxSeq, g)) return nC;
+        // (the same limits as launch_flow_layers checks: a shape it would refuse runs the fused launches instead)
+        if (flow_min_grid(nHeads, nKVHeads, g) <= nC && flow_context_fits(maxSeq, g) && flow_grid_fits(ffnDim, nHeads, g, nC) &&
+            (size_t)nLayers * g.stride * 4 < (1ull << 31)) return nC;
     }
     return 0;
 }
@@ -737,9 +747,9 @@ int HIPFusedInference::ensureFlow() {
         dFlowLayers = static_cast<FlowLayer*>(v);
         HIPCHK(hipMalloc(&v, sizeof(float) * (size_t)nLayers * flowGeo.stride));
         flowXchg = static_cast<float*>(v);
-        HIPCHK(hipMalloc(&v, 256));
+        HIPCHK(hipMalloc(&v, FLOW_ERR_BYTES));
         dFlowErr = static_cast<int*>(v);
-        HIPCHK(hipMemsetAsync(dFlowErr, 0, 256, stream));
+        HIPCHK(hipMemsetAsync(dFlowErr, 0, FLOW_ERR_BYTES, stream));
         HIPCHK(hipHostMalloc(&v, 64, hipHostMallocDefault));
         hFlowErr = static_cast<int*>(v);
         *hFlowErr = 0;
@@ -914,7 +924,8 @@ int HIPFusedInference::PartialStep(const float* hiddenIn, int pos, int layerStar
         HIPCHK(hipStreamSynchronize(stream));
         HIPCHK(hipMemcpy(h, hiddenIn, (size_t)dim * 4, hipMemcpyHostToDevice));      // :395
     }
-    if (flowEligible(layerStart, layerEnd)) {
+    const bool flow = flowEligible(layerStart, layerEnd);
+    if (flow) {
         int rc = ensureFlow();
         if (rc == 0) rc = enqueueLayersFlow(layerStart, layerEnd, nullptr, pos, true);
         if (rc) return rc;
@@ -939,7 +950,13 @@ int HIPFusedInference::PartialStep(const float* hiddenIn, int pos, int layerStar
         int rc = checkFlowError();
         if (rc) return rc;
     }
-    return MG_OK;      // nothing read back: the launches stay queued (the reference does not sync here either)
+    // Nothing read back: the launches stay queued (the reference does not sync here either) -- except after a
+    // persistent launch, whose waits may have run out: that is reported by the call whose step it spoiled.
+    if (flow && !(layerEnd >= nLayers && logitsOut && finalNorm) && !(hiddenOut && layerEnd < nLayers)) {
+        HIPCHK(hipStreamSynchronize(stream));
+        return checkFlowError();
+    }
+    return MG_OK;
 }
 
 // ---- L3 bridge and mailbox (cuda_fused_infer.go:556-737) ----

@@ -955,9 +955,9 @@ __device__ __forceinline__ float4 ld_kv4(const void* base, size_t idx4) {
 
 // A helper workgroup of the attention launch (grid rows past the splits): its waves fetch their share
 // of one region each into this XCD's L2.  Two scalar loads (the wave table, one region) come before
-// the first fetch; the loads all land in one register that nothing reads, and none is waited for
-// before the last one is out.
-typedef int pf_v4i __attribute__((ext_vector_type(4)));
+// the first fetch; the loads go straight into a 1 KB scrap area of LDS that nothing reads
+// (global_load_lds_dwordx4: no destination register that a late load could overwrite), and none is
+// waited for before the last one is out.
 __device__ __forceinline__ void prefetch_helper(const PfJob& job, int firstFlat, int nWaves) {
     const int lane = threadIdx.x & 63;
     const int flatId = blockIdx.x + blockIdx.y * gridDim.x;      // dispatch order: XCD = flatId & 7
@@ -983,15 +983,15 @@ __device__ __forceinline__ void prefetch_helper(const PfJob& job, int firstFlat,
     const int grp = lw >> R.splitLog2;
     const int ngrp = nw >> R.splitLog2;
     if (grp >= ngrp) return;
-    pf_v4i sink = {0, 0, 0, 0};
+    __shared__ int4 scrap[64];
     for (int q = q0 + qs * grp; q < nruns; q += qs * ngrp) {
         const unsigned b0 = (unsigned)q * R.runBytes;
         unsigned b1 = b0 + R.runBytes;
         b1 = b1 < end ? (b1 + 15u) & ~15u : end;
         for (unsigned o = (b0 & ~15u) + (unsigned)sub * 1024 + lane * 16; o < b1; o += 1024u << R.splitLog2)
-            asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(sink) : "v"(R.base + o) : "memory");
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const int4*>(R.base + o), scrap, 16, 0, 0);
     }
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(sink) : : "memory");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 template <int HD, int GMAX, bool KVH, int AWG = WG>

@@ -50,7 +50,7 @@ class Model:
     """Oracle and/or HIP context holding the same synthetic model."""
 
     def __init__(self, s, seed, maxSeq, eng=None, oracle=True, threads=8, fmt=None, keep_dequant=False, kv_f16=False):
-        self.s, self.seed, self.maxSeq = s, seed, maxSeq
+        self.s, self.seed, self.maxSeq, self.eng = s, seed, maxSeq, eng
         fmt = fmt or s.fmt
         kv = configs.kv_dim(s)
         self.orc = ob.Oracle(s.dim, kv, s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab, s.nLayers, maxSeq,
@@ -170,7 +170,7 @@ def load_fast(s, seed, maxSeq, eng, oracle=True, threads=16, kv_f16=False):
     """A Model whose matrices are quantized by the library's parallel host quantizer (bit-identical to
     the oracle's, checked on the CPU) and shared with the oracle: for the multi-gigabyte shapes."""
     m = Model.__new__(Model)
-    m.s, m.seed, m.maxSeq = s, seed, maxSeq
+    m.s, m.seed, m.maxSeq, m.eng = s, seed, maxSeq, eng
     kv = configs.kv_dim(s)
     m.orc = ob.Oracle(s.dim, kv, s.headDim, s.nHeads, s.nKVHeads, s.ffnDim, s.vocab, s.nLayers, maxSeq,
                       s.theta, s.eps, threads=threads) if oracle else None

@@ -122,16 +122,31 @@ def test_tokens_match_oracle_and_fused_launches(hip, fmt):
 
 
 def _modes_agree(m, prompt, nDecode, what):
-    out = {}
+    """The same prompt and decode run through the fused launches (exec mode 1) and the persistent launch (3):
+    identical greedy tokens, and -- tokens alone need not show a dropped or mis-weighted KV split -- the logits
+    and the hidden state of one more step at the position after the run agree to rounding (the two differ in
+    the order in which the splits' partials are merged, nothing else)."""
+    out, last = {}, {}
+    s = m.s
     for mode in (1, 3):
         assert m.hip.SetExecMode(mode) == 0
         assert m.hip.ResetKV() == 0
         rc, t = m.hip.GeneratePrefill(prompt, nDecode)
         assert rc == 0, E.last_error()
+        assert _in_use(m.hip) == (mode == 3)
         out[mode] = t
-    assert _in_use(m.hip)
+        pos = len(prompt) + nDecode - 1                     # the cache holds positions 0 .. pos - 1
+        if pos < m.maxSeq:
+            logits = np.empty(s.vocab, np.float32)
+            rc, _ = m.hip.DecodeToken(int(t[-1]), pos, logits)
+            assert rc == 0, E.last_error()
+            last[mode] = (logits, m.hip.ExportHidden())
     i = H.first_divergence(out[3], out[1])
     assert i is None, f"{what}: persistent launch and fused launches part at token {i}"
+    if last:
+        el, eh = H.rel_err(last[3][0], last[1][0]), H.rel_err(last[3][1], last[1][1])
+        print(f"  {what}: modes 3 vs 1 at the next position: logits {el:.2e}, hidden {eh:.2e}", flush=True)
+        assert el < 1e-5 and eh < 1e-5, f"{what}: logits {el:.2e} / hidden {eh:.2e} between the two launches"
     return out[3]
 
 

@@ -128,3 +128,32 @@ def test_llama3_8b_full_prefill_512_then_256_decode(hip):
         gap = abs(float(logits[a]) - float(logits[b])) / float(np.abs(logits).max())
         assert gap < 1e-3, (i, a, b, gap)
     m.close()
+
+
+def test_llama3_8b_full_depth_at_4000_positions_both_launches(hip):
+    """All 32 layers at the long-context leg of the benchmark (maxSeq 4082: the persistent launch's grouped attention
+    at heads of 128 with the real FFN of 14336, 32 KV splits): the cache is filled by a batched prefill of 4000
+    tokens, then 32 tokens are decoded through the persistent launch (exec mode 3) and through the fused launches
+    (exec mode 1, whose attention kernel is oracle-checked at this geometry up to position 4099 in
+    test_gpu_long_context.py): same tokens, and logits / hidden state of the following step within 1e-4.  The oracle
+    itself would need hours to reach position 4000 at this size."""
+    s = configs.LLAMA3_8B
+    m = H.load_fast(s, seed=20254, maxSeq=4082, eng=hip, oracle=False)
+    prompt = m.prompt(4000)
+    out, last = {}, {}
+    logits = np.empty(s.vocab, np.float32)
+    for mode in (3, 1):
+        print(f"llama-3-8b at 4000 positions: exec mode {mode}", flush=True)
+        assert m.hip.SetExecMode(mode) == 0
+        assert m.hip.ResetKV() == 0
+        rc, t = m.hip.GeneratePrefill(prompt, 32)
+        assert rc == 0, E.last_error()
+        assert m.hip.FlowInUse() == (mode == 3)
+        rc, _ = m.hip.DecodeToken(int(t[-1]), 4031, logits)
+        assert rc == 0, E.last_error()
+        out[mode], last[mode] = t.tolist(), (logits.copy(), m.hip.ExportHidden())
+    el, eh = H.rel_err(last[3][0], last[1][0]), H.rel_err(last[3][1], last[1][1])
+    print(f"llama-3-8b at 4000 positions: modes 3 vs 1: logits {el:.2e}, hidden {eh:.2e}", flush=True)
+    assert out[3] == out[1], H.first_divergence(out[3], out[1])
+    assert el < 1e-4 and eh < 1e-4
+    m.close()
