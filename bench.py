@@ -48,6 +48,7 @@ PMC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script record
 LAUNCH_NAMES = {0: "embed_gather", 1: "norm+qkv", 2: "rope+kvwrite+attention", 3: "wo+residual", 4: "norm+gate_up+swiglu",
                 5: "down+residual", 6: "norm+lm_head+argmax_partials", 7: "argmax_finish"}
 FLOW_NAME = "persistent layer launch (all layers: norm, q|k|v, RoPE, KV write, attention, Wo, gate|up, SwiGLU, down)"
+TOKEN_NAME = "persistent launch, whole tokens (embedding gather, all layers, final norm, lm_head, argmax)"
 
 
 def slot_shape(s, kv, idx):
@@ -156,7 +157,7 @@ def cpu_baseline(E, np, s, seed, prompt, first_tokens, budget_s, kv_f16=False):
             break
     el = time.perf_counter() - t0
     orc.close()
-    return {"value": done / el, "unit": "tok/s", "cores": 1, "kind": "port",
+    return {"value": done / el, "unit": "tok/s", "cores": 1, "host_cores": os.cpu_count(), "kind": "port",
             "sample": f"{done} tokens (positions 0..{done - 1} of the same prompt+decode stream) in {el:.1f} s, "
                       f"single thread; C restatement of the Go CPU engine, not the Go binary (no Go toolchain)",
             "tokens_match_gpu": bool(match)}
@@ -174,6 +175,7 @@ def launch_table(f, configs, s, first_tok, pos, steps, ms_per_step, kv_f16):
     rc, cls_ms, cls_n = f.ProfileDecode(first_tok, pos, steps)
     assert rc == 0
     flow = f.FlowInUse()
+    tail = flow and f.FlowTailInUse()
 
     def mat(n, k):
         return n * k + 4 * n if s.fmt == "q8" else n * (k // 32) * 18
@@ -181,7 +183,8 @@ def launch_table(f, configs, s, first_tok, pos, steps, ms_per_step, kv_f16):
     kvb = 2 * (p_prof + 1) * kv * (2 if kv_f16 else 4)
     layer_w = mat(s.dim, s.dim) * 2 + 2 * mat(kv, s.dim) + 2 * mat(s.ffnDim, s.dim) + mat(s.dim, s.ffnDim) + 8 * s.dim
     cls_bytes = {
-        1: (layer_w + kvb) * s.nLayers if flow else mat(s.dim, s.dim) + 2 * mat(kv, s.dim) + 4 * s.dim,
+        1: ((layer_w + kvb) * s.nLayers + (mat(s.vocab, s.dim) + 4 * s.dim if tail else 0)) if flow
+           else mat(s.dim, s.dim) + 2 * mat(kv, s.dim) + 4 * s.dim,
         2: kvb,
         3: mat(s.dim, s.dim),
         4: 2 * mat(s.ffnDim, s.dim) + 4 * s.dim,
@@ -196,7 +199,7 @@ def launch_table(f, configs, s, first_tok, pos, steps, ms_per_step, kv_f16):
             continue
         ms = float(cls_ms[c])
         # share of the eager step's launch time (events between launches; a replayed graph runs the same kernels closer together)
-        e = {"launch": FLOW_NAME if (flow and c == 1) else LAUNCH_NAMES[c], "cls": c, "per_token": n, "avg_us": round(ms * 1e3, 3),
+        e = {"launch": (TOKEN_NAME if tail else FLOW_NAME) if (flow and c == 1) else LAUNCH_NAMES[c], "cls": c, "per_token": n, "avg_us": round(ms * 1e3, 3),
              "share_of_step": round(ms * n / total, 4) if total > 0 else None}
         if c in cls_bytes and ms > 0:
             e["bytes"] = int(cls_bytes[c])
@@ -204,6 +207,65 @@ def launch_table(f, configs, s, first_tok, pos, steps, ms_per_step, kv_f16):
             e["frac_of_peak"] = round(e["GBps"] / HBM_PEAK_GBS, 4)
         rows.append(e)
     return rows
+
+
+def phase_table(f, np, configs, s, first_tok, pos, kv_f16, steps=8):
+    """Per-phase times inside the persistent launch from its own trace (100 MHz wall clock stamps per workgroup): for
+    every matvec phase of a layer and for the lm_head, the bytes the phase reads over the time from the first workgroup
+    having its input staged to the last workgroup being done (median over the layers of the last traced token)."""
+    kv = configs.kv_dim(s)
+    rc, _ = f.FlowTrace(True)
+    if rc != 0:
+        return None
+    rc, _ = f.TimedDecode(first_tok, pos, steps, useGraph=True)
+    assert rc == 0
+    rc, tr = f.FlowTrace(True, read=True)
+    assert rc == 0
+    tt = None
+    if f.FlowTailInUse():
+        rc, tt = f.FlowTailTrace()
+        assert rc == 0
+    f.FlowTrace(False)
+
+    def mat(n, k):
+        return n * k + 4 * n if s.fmt == "q8" else n * (k // 32) * 18
+    p_last = pos + steps - 1
+    spans = [("norm+q|k|v (+bias, RoPE, KV write)", 1, 2, mat(s.dim, s.dim) + 2 * mat(kv, s.dim) + 4 * s.dim),
+             ("attention", 3, 4, 2 * (p_last + 1) * kv * (2 if kv_f16 else 4)),
+             ("Wo+residual", 5, 6, mat(s.dim, s.dim)),
+             ("norm+gate|up+SwiGLU", 7, 8, 2 * mat(s.ffnDim, s.dim) + 4 * s.dim),
+             ("down+residual", 9, 10, mat(s.dim, s.ffnDim))]
+    nL = tr.shape[0]
+    rows = []
+    tot_phase = 0.0
+    for name, a, b, nbytes in spans:
+        us = []
+        for l in range(1 if nL > 1 else 0, nL):
+            ta, tb = tr[l, a][tr[l, a] > 0], tr[l, b][tr[l, b] > 0]
+            if ta.size and tb.size:
+                us.append((float(tb.max()) - float(ta.min())) / 100.0)
+        if not us:
+            continue
+        u = float(np.median(us))
+        tot_phase += u
+        rows.append({"phase": name, "bytes": int(nbytes), "us": round(u, 2), "GBps": round(nbytes / u / 1e3, 1),
+                     "frac_of_peak": round(nbytes / u / 1e3 / HBM_PEAK_GBS, 4)})
+    layer_us = float(np.median(np.diff(np.median(tr[:, 0, :], axis=1)))) / 100.0 if nL > 1 else None
+    out = {"position": p_last, "layer_us": round(layer_us, 2) if layer_us else None,
+           "hand_overs_and_waits_us": round(layer_us - tot_phase, 2) if layer_us else None, "phases": rows,
+           "note": "input staged by the first workgroup -> last workgroup done, per phase; a phase's weights may already be in "
+                   "the L2s (read there by the prefetching workgroups during earlier phases), so a phase can exceed the HBM peak"}
+    if tt is not None:
+        lm = mat(s.vocab, s.dim) + 4 * s.dim
+        staged, done, known = tt[1][tt[1] > 0], tt[4][tt[4] > 0], tt[3][tt[3] > 0]
+        u = (float(done.max()) - float(staged.min())) / 100.0
+        um = (float(np.median(done)) - float(np.median(staged))) / 100.0
+        out["lm_head"] = {"phase": "final norm+lm_head+argmax partials", "bytes": int(lm), "us": round(u, 2),
+                          "GBps": round(lm / u / 1e3, 1), "frac_of_peak": round(lm / u / 1e3 / HBM_PEAK_GBS, 4),
+                          "us_median_workgroup": round(um, 2),
+                          "frac_of_peak_median_workgroup": round(lm / um / 1e3 / HBM_PEAK_GBS, 4),
+                          "token_known_after_us": round((float(known.max()) - float(done.max())) / 100.0, 2)}
+    return out
 
 
 def check_tokens(E, orc, prompt, toks, budget_s):
@@ -225,17 +287,20 @@ def check_tokens(E, orc, prompt, toks, budget_s):
 
 
 def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_graph=True, exec_mode=None, kv_f16=False,
-            prefill=0, oracle_threads=0, check_budget_s=8.0, want_mode1_table=True, keep=False):
+            prefill=0, oracle_threads=0, check_budget_s=8.0, want_mode1_table=True, keep=False, tokens_per_launch=None,
+            want_phases=True, flow_tail=True, stream_tokens=0):
     """One configuration: load, warm up on the W prompt positions, time K decode steps at each start position of
     `contexts` (0 = right after the prompt), per-launch table, optional batched prefill, optional token check."""
     from oracle import binding as ob
     P = [max(c, W) for c in contexts]
-    maxSeq = max(max(P) + K + profile_steps + 8, prefill + 8, W + 56)
+    maxSeq = max(max(P) + K + profile_steps + 16, prefill + 8, W + 56)
     orc = oracle_for(ob, configs, s, W + 72, oracle_threads) if oracle_threads else None
     t_load = time.perf_counter()
     f = load_model(E, np, s, seed, maxSeq, eng, oracle=orc, kv_f16=kv_f16)
     if exec_mode is not None and f.SetExecMode(exec_mode) != 0:
         raise SystemExit("bench.py: " + E.last_error())
+    if not flow_tail:
+        f.SetFlowTail(False)
     t_load = time.perf_counter() - t_load
     prompt = E.synth_tokens(seed, 20_000_003, s.vocab, W)
     rc, first = f.Generate(prompt, 1, useGraph=use_graph)
@@ -243,9 +308,17 @@ def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_gra
     wbytes = configs.weight_bytes_per_token(s)
     assert f.WeightBytesPerToken() == wbytes
     flow = f.FlowInUse()
-    res = {"exec": ("persistent layer launch + lm_head + argmax" if flow else "fused launches (5 a layer)") +
-                   (", hipGraph replay" if use_graph else ", eager"),
-           "weight_bytes_per_token": int(wbytes), "load_s": round(t_load, 1), "runs": []}
+    tail = flow and f.FlowTailInUse()
+    if tokens_per_launch is not None and f.SetTokensPerLaunch(tokens_per_launch) != 0:
+        raise SystemExit("bench.py: " + E.last_error())
+    tpl = f.TokensPerLaunch() if tail and use_graph else 1
+    if tail:
+        how = f"persistent launch running whole tokens, {tpl} tokens a launch" if tpl > 1 else \
+              "persistent launch running a whole token, one launch a token" + (" (hipGraph replay)" if use_graph else " (eager)")
+    else:
+        how = ("persistent layer launch + lm_head + argmax" if flow else "fused launches (5 a layer)") + \
+              (", hipGraph replay" if use_graph else ", eager")
+    res = {"exec": how, "weight_bytes_per_token": int(wbytes), "load_s": round(t_load, 1), "runs": []}
     for P0 in P:
         rc, ms = f.TimedDecode(int(first[0]), P0, K, useGraph=use_graph)
         assert rc == 0, E.last_error()
@@ -253,7 +326,17 @@ def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_gra
         step_bytes = wbytes + configs.kv_bytes_at(s, P0 + K // 2) // (2 if kv_f16 else 1)
         run = {"start_position": P0, "steps": K, "ms_per_step": round(ms_step, 5), "tok_per_s": round(K / (ms / 1e3), 1),
                "step_bytes": int(step_bytes), "step_GBps": round(step_bytes / (ms_step * 1e-3) / 1e9, 1),
-               "step_roofline_frac": round(step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+               "step_roofline_frac": round(step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+               "launches": (K + tpl - 1) // tpl}
+        if tail and tpl > 1:
+            # the same steps as replays of the captured one-token graph (one launch a token)
+            assert f.SetTokensPerLaunch(1) == 0
+            rc, msg = f.TimedDecode(int(first[0]), P0, K, useGraph=use_graph)
+            assert rc == 0, E.last_error()
+            assert f.SetTokensPerLaunch(tpl) == 0
+            run["graph_replay_one_token_a_launch_ms_per_step"] = round(msg / K, 5)
+        if flow and want_phases:
+            run["in_launch_phases"] = phase_table(f, np, configs, s, int(first[0]), P0 + K, kv_f16)
         table = launch_table(f, configs, s, int(first[0]), P0 + K, profile_steps, ms_step, kv_f16)
         run["kernels"] = table
         if flow and want_mode1_table:
@@ -264,6 +347,22 @@ def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_gra
             run["kernels_fused_launches"] = launch_table(f, configs, s, int(first[0]), P0 + K, profile_steps, ms1 / K, kv_f16)
             assert f.SetExecMode(3 if exec_mode is None else exec_mode) == 0
             table = run["kernels_fused_launches"]
+        if flow and P0 > W:
+            # a long context is beyond the oracle's budget: the tokens of the launch that was timed against the fused
+            # launches' (whose attention kernel the tests check against the oracle at this geometry), same positions
+            seqs = {}
+            for md in (3 if exec_mode is None else exec_mode, 1):
+                assert f.SetExecMode(md) == 0
+                tok, seq = int(first[0]), []
+                for i in range(12):
+                    rc, tok = f.DecodeToken(tok, P0 + i)
+                    assert rc == 0, E.last_error()
+                    seq.append(tok)
+                seqs[md] = seq
+            assert f.SetExecMode(3 if exec_mode is None else exec_mode) == 0
+            a_, b_ = list(seqs.values())
+            run["tokens_match_fused_launches"] = bool(a_ == b_)
+            run["tokens_compared"] = len(a_)
         att = [e for e in table if e["cls"] == 2]
         if att and "GBps" in att[0]:
             run["attention_KV_GBps"] = att[0]["GBps"]
@@ -305,11 +404,49 @@ def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_gra
         assert rc == 0, E.last_error()
     if orc is not None:
         res.update(check_tokens(E, orc, cprompt, toks, check_budget_s))
+        res["tokens_checked_at"] = "positions 3.. of a 4-token prompt + 48 decode tokens (short context)"
         orc.close()
+    if stream_tokens > 0 and s.fmt == "q4_0":
+        res["stream"] = stream_leg(E, np, configs, f, s, seed, stream_tokens)
     if keep:
         return res, f, prompt, first, toks
     f.Close()
     return res
+
+
+def stream_leg(E, np, configs, f, s, seed, n):
+    """n tokens through the weight-streaming front end (every layer's Q4_0 blocks cross PCIe per token)."""
+    kv = configs.kv_dim(s)
+    st = f.StreamBuild()
+    assert st is not None, E.last_error()
+    ptrs, sizes = [], []
+    for l in range(s.nLayers):
+        for w in range(12):
+            idx = l * 12 + w
+            rows, cols = slot_shape(s, kv, idx)
+            if cols == 1:
+                ptrs.append(gen_slot(E, np, s, kv, seed, idx) if (w not in (4, 5, 6) or s.bias) else None)
+            else:
+                blk = E.quantize_q4_0(gen_slot(E, np, s, kv, seed, idx))
+                ptrs.append(blk)
+                sizes.append(blk.size)
+    layer_bytes = sum(a.nbytes for a in ptrs if a is not None)
+    assert f.ResetKV() == 0
+    h0 = np.zeros(s.dim, np.float32)
+    h0[:] = E.synth_normal(seed, 30_000_001, 0.02, (s.dim,))
+    logits = np.empty(s.vocab, np.float32)
+    for pos in range(2):                               # warm the staging buffers
+        assert st.StreamForwardToken(pos, h0, s.nLayers, ptrs, sizes, logits) == 0, E.last_error()
+    t0 = time.perf_counter()
+    for i in range(n):
+        assert st.StreamForwardToken(2 + i, h0, s.nLayers, ptrs, sizes, logits) == 0, E.last_error()
+    el = time.perf_counter() - t0
+    st.Close()
+    return {"tokens": n, "ms_per_token": round(el / n * 1e3, 3),
+            "tok_per_s": round(n / el, 1), "host_to_device_bytes_per_token": int(layer_bytes),
+            "host_to_device_GBps": round(layer_bytes * n / el / 1e9, 2),
+            "note": "host wall clock; every token stages all layers from pageable host memory through two pinned "
+                    "buffers into two device sets (copy of layer l+1 overlaps compute of layer l); logits read back each token"}
 
 
 def main():
@@ -338,6 +475,10 @@ def main():
                          "every layer's weights cross PCIe per token; extra 'stream' object)")
     ap.add_argument("--flow-trace", action="store_true",
                     help="also record the persistent layer launch's per-workgroup timeline (extra 'flow_trace' object)")
+    ap.add_argument("--tokens-per-launch", type=int, default=0,
+                    help="tokens the persistent launch runs per launch (0 = the library's default, 64; 1 = a launch per token)")
+    ap.add_argument("--no-flow-tail", action="store_true",
+                    help="lm_head and argmax as launches of their own behind the persistent layer launch (for comparisons)")
     ap.add_argument("--no-configs", action="store_true",
                     help="only the configuration named by --config (no 'configs' object with the other benchmark configurations)")
     args = ap.parse_args()
@@ -361,19 +502,16 @@ def main():
     mode = None if args.exec_mode < 0 else args.exec_mode
     res, f, prompt, first, toks = measure(E, np, configs, eng, s, args.seed, W, K, [args.context], args.profile_steps,
                                           use_graph=use_graph, exec_mode=mode, kv_f16=kv_f16, prefill=args.prefill,
-                                          oracle_threads=0, keep=True)
+                                          oracle_threads=0, keep=True, tokens_per_launch=args.tokens_per_launch or None,
+                                          flow_tail=not args.no_flow_tail)
     run = res["runs"][0]
     P0 = run["start_position"]
     ms_per_step = run["ms_per_step"]
     toks_per_s = K / (ms_per_step * K / 1e3)
     flow = f.FlowInUse()
 
-    # the launch that takes most of the step, and the lm_head matvec, once more with events around them alone
-    # (less event overhead inside their intervals)
+    tail = flow and f.FlowTailInUse()
     table = run["kernels"]
-    dom = max(table, key=lambda e: e["avg_us"] * e["per_token"])
-    rc, only, _ = f.ProfileDecode(int(first[0]), P0 + K, args.profile_steps, classMask=(1 << dom["cls"]) | (1 << 6))
-    assert rc == 0, E.last_error()
 
     def roof(entry, ms, key):
         sec = ms * 1e-3
@@ -384,9 +522,39 @@ def main():
                 "launches_timed": int(args.profile_steps) * entry["per_token"],
                 "traffic": PMC_TRAFFIC_BYTES.get((s.name, key)),
                 "traffic_source": PMC_SOURCE if (s.name, key) in PMC_TRAFFIC_BYTES else None}
-    roofline = roof(dom, float(only[dom["cls"]]), "flow" if (flow and dom["cls"] == 1) else LAUNCH_NAMES[dom["cls"]])
-    lm = [e for e in table if e["cls"] == 6][0]
-    matvec = roof(lm, float(only[6]), "lm_head")
+    if tail:
+        # The step is one kernel: the launch that runs whole tokens.  Its average duration is the timed region itself (HIP
+        # events on the context's stream around the K steps), divided by the launches it took.
+        launches = run["launches"]
+        sec = ms_per_step * 1e-3 * K / launches
+        b = run["step_bytes"] * K / launches
+        tr_b = PMC_TRAFFIC_BYTES.get((s.name, "token"))
+        roofline = {"bound": "hbm", "kernel": TOKEN_NAME, "achieved": round(b / sec / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(b / sec / 1e9 / HBM_PEAK_GBS, 4), "bytes_per_launch": int(b), "avg_launch_us": round(sec * 1e6, 2),
+                    "tokens_per_launch": round(K / launches, 2), "launches_timed": launches, "share_of_step": 1.0,
+                    "traffic": int(tr_b * K / launches) if tr_b else None,
+                    "traffic_source": PMC_SOURCE if tr_b else None,
+                    "traffic_note": None if tr_b else "not collected for this kernel"}
+        ph = run.get("in_launch_phases") or {}
+        lmh = ph.get("lm_head")
+        sep = [e for e in (run.get("kernels_fused_launches") or []) if e["cls"] == 6]
+        matvec = None
+        if lmh:
+            matvec = {"bound": "hbm", "kernel": "final norm + lm_head + argmax partials, a phase of the persistent launch",
+                      "achieved": lmh["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": lmh["frac_of_peak"],
+                      "bytes": lmh["bytes"], "us": lmh["us"],
+                      "timed_by": "the launch's own 100 MHz wall-clock stamps: first workgroup's input staged -> last workgroup's last wave done",
+                      "median_workgroup": {"us": lmh["us_median_workgroup"], "frac": lmh["frac_of_peak_median_workgroup"]},
+                      "as_a_launch_of_its_own_event_timed": sep[0] if sep else None}
+    else:
+        # the launch that takes most of the step, and the lm_head matvec, once more with events around them alone
+        # (less event overhead inside their intervals)
+        dom = max(table, key=lambda e: e["avg_us"] * e["per_token"])
+        rc, only, _ = f.ProfileDecode(int(first[0]), P0 + K, args.profile_steps, classMask=(1 << dom["cls"]) | (1 << 6))
+        assert rc == 0, E.last_error()
+        roofline = roof(dom, float(only[dom["cls"]]), "flow" if (flow and dom["cls"] == 1) else LAUNCH_NAMES[dom["cls"]])
+        lm = [e for e in table if e["cls"] == 6][0]
+        matvec = roof(lm, float(only[6]), "lm_head")
 
     flow_trace = None
     if args.flow_trace and flow:
@@ -423,37 +591,7 @@ def main():
             print("bench.py: --stream needs a Q4_0 configuration (the streaming front end takes GGUF block_q4_0 layers)",
                   file=sys.stderr)
             sys.exit(2)
-        kv = configs.kv_dim(s)
-        st = f.StreamBuild()
-        assert st is not None, E.last_error()
-        ptrs, sizes = [], []
-        for l in range(s.nLayers):
-            for w in range(12):
-                idx = l * 12 + w
-                rows, cols = slot_shape(s, kv, idx)
-                if cols == 1:
-                    ptrs.append(gen_slot(E, np, s, kv, args.seed, idx) if (w not in (4, 5, 6) or s.bias) else None)
-                else:
-                    blk = E.quantize_q4_0(gen_slot(E, np, s, kv, args.seed, idx))
-                    ptrs.append(blk)
-                    sizes.append(blk.size)
-        layer_bytes = sum(a.nbytes for a in ptrs if a is not None)
-        assert f.ResetKV() == 0
-        h0 = np.zeros(s.dim, np.float32)
-        h0[:] = E.synth_normal(args.seed, 30_000_001, 0.02, (s.dim,))
-        logits = np.empty(s.vocab, np.float32)
-        for pos in range(2):                               # warm the staging buffers
-            assert st.StreamForwardToken(pos, h0, s.nLayers, ptrs, sizes, logits) == 0, E.last_error()
-        t0 = time.perf_counter()
-        for i in range(args.stream):
-            assert st.StreamForwardToken(2 + i, h0, s.nLayers, ptrs, sizes, logits) == 0, E.last_error()
-        el = time.perf_counter() - t0
-        st.Close()
-        stream = {"tokens": args.stream, "ms_per_token": round(el / args.stream * 1e3, 3),
-                  "tok_per_s": round(args.stream / el, 1), "host_to_device_bytes_per_token": int(layer_bytes),
-                  "host_to_device_GBps": round(layer_bytes * args.stream / el / 1e9, 2),
-                  "note": "host wall clock; every token stages all layers from pageable host memory through two pinned "
-                          "buffers into two device sets (copy of layer l+1 overlaps compute of layer l); logits read back each token"}
+        stream = stream_leg(E, np, configs, f, s, args.seed, args.stream)
     f.Close()
 
     cpu = None
@@ -465,13 +603,13 @@ def main():
         others = {}
         plan = [("toy", dict(K=200, contexts=[0], threads=8)),
                 ("tinyllama-1.1b", dict(K=50, contexts=[0], threads=16)),
-                ("qwen2.5-0.5b-q4_0", dict(K=200, contexts=[0], threads=16)),
+                ("qwen2.5-0.5b-q4_0", dict(K=200, contexts=[0], threads=16, stream=20)),
                 ("llama-3-8b", dict(K=64, contexts=[0, 4000], threads=16, prefill=512))]
         for name, o in plan:
             print(f"bench.py: configuration {name}", file=sys.stderr, flush=True)
             others[name] = measure(E, np, configs, eng, configs.BY_NAME[name], args.seed + 1, 16, o["K"], o["contexts"],
                                    10, use_graph=True, prefill=o.get("prefill", 0), oracle_threads=o["threads"],
-                                   check_budget_s=10.0)
+                                   check_budget_s=10.0, stream_tokens=o.get("stream", 0))
 
     out = {
         "metric": "Q8 decode tok/s (bs=1, Qwen2.5-0.5B shape) + matvec HBM GB/s % of peak" if s.name == "qwen2.5-0.5b"
@@ -486,6 +624,8 @@ def main():
         "roofline": roofline, "matvec": matvec, "kernels": run["kernels"],
         "kernels_fused_launches": run.get("kernels_fused_launches"),
         "fused_launches_ms_per_step": run.get("fused_launches_ms_per_step"),
+        "graph_replay_one_token_a_launch_ms_per_step": run.get("graph_replay_one_token_a_launch_ms_per_step"),
+        "in_launch_phases": run.get("in_launch_phases"),
         "cpu_baseline": cpu, "prefill": res.get("prefill"), "stream": stream, "flow_trace": flow_trace, "configs": others,
         "load_s": res["load_s"], "device": eng.Name(),
     }

@@ -401,6 +401,25 @@ int mg_flow_in_use(mg_ctx* ctx);
  * persistent launch is not in use for the model. */
 int mg_flow_trace(mg_ctx* ctx, int enable, long long* out, size_t cap, int* dims);
 
+/* Whole tokens inside the persistent launch.  Where the launch is in use (mg_flow_in_use), the lm_head has
+ * the layers' weight format and final norm and lm_head are set, a token's embedding gather, its layers, the
+ * final norm, the lm_head matvec and the greedy argmax (cuda_fused_infer.go:446-450 plus what the
+ * reference's caller does with the logits) all run in that one launch, and the calls that ask for a run
+ * of tokens (mg_generate with useGraph, mg_timed_decode with useGraph, mg_generate_prefill) put up to
+ * `n` tokens into each launch (default 64): the next token is chosen on the device and the launch goes on
+ * with it.  n = 1: a launch (or a replay of the captured one-launch graph) per token.
+ * mg_set_flow_tail(ctx, 0) goes back to separate lm_head and argmax launches behind the layers' launch
+ * (for comparisons).  mg_flow_tail_in_use: 1 when tokens run that way as things stand.
+ * mg_flow_tail_trace: with mg_flow_trace enabled, the tail's six points (tail top; final norm input
+ * staged; lm_head done by the workgroup's first wave; token known; lm_head done by all its waves; all
+ * workgroups' argmax partials in) of the last token a launch ran, ticks [point][workgroup], dims[2] =
+ * {6, workgroups}.  No counterparts in the reference. */
+int mg_set_flow_tail(mg_ctx* ctx, int on);
+int mg_set_tokens_per_launch(mg_ctx* ctx, int n);
+int mg_tokens_per_launch(mg_ctx* ctx);
+int mg_flow_tail_in_use(mg_ctx* ctx);
+int mg_flow_tail_trace(mg_ctx* ctx, long long* out, size_t cap, int* dims);
+
 /* Time limit of each wait inside the persistent launch, in ticks of the 100 MHz wall clock (default
  * 5,000,000 = 50 ms).  A workgroup whose wait runs out stops waiting for the rest of the launch, the
  * launch ends normally with an error flag set, the call that issued it returns MG_E_HIP and the

@@ -172,6 +172,24 @@ __device__ __forceinline__ float chunk_act_sum(const float4 (&av)[4]) {
     return (t.x + t.y) + (t.z + t.w);
 }
 
+// Element i of token tok's embedding row.  kind 0: int8 rows [vocab, dim] times the row's scale (a tied Q8 lm_head),
+// 1: fp16 table, 2: fp32 table, 3: Q4_0 in the split layout (nibble plane [vocab, dim/2], then the fp16 d plane).
+__device__ __forceinline__ float embed_value(int kind, const void* table, const float* scales, int tok, int dim, int vocab, int i) {
+    if (kind == 0) {
+        const signed char* q = static_cast<const signed char*>(table) + (size_t)tok * dim;
+        return (float)q[i] * scales[tok];
+    }
+    if (kind == 1) return half_bits_to_float((static_cast<const unsigned short*>(table) + (size_t)tok * dim)[i]);
+    if (kind == 2) return static_cast<const float*>(table)[(size_t)tok * dim + i];
+    const unsigned char* base = static_cast<const unsigned char*>(table);
+    const unsigned char* qs = base + (size_t)tok * (dim >> 1);
+    const unsigned short* dpl = reinterpret_cast<const unsigned short*>(base + (size_t)vocab * (dim >> 1)) + (size_t)tok * (dim >> 5);
+    const int b = i >> 5, j = i & 31;
+    const unsigned char q = qs[b * 16 + (j & 15)];
+    const int nib = j < 16 ? (q & 0x0f) : (q >> 4);
+    return (float)(nib - 8) * half_bits_to_float(dpl[b]);
+}
+
 // ---------------------------------------------------------------------------
 // Agent-scope accesses and the decode attention's row helpers
 // ---------------------------------------------------------------------------

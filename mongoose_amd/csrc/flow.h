@@ -25,6 +25,24 @@ struct FlowLayer {
     float* Kc; float* Vc;                                    // fp32 caches [maxSeq, kvDim]
 };
 
+// Operands of the tail of a token (final norm, lm_head, greedy argmax, the next token's embedding), a struct in device
+// memory.  The lm_head has the format of the layers' matrices (pointer pair as in FlowLayer).
+struct FlowTail {
+    const float* finalGain;
+    const signed char* lmW; const float* lmAux;
+    float* logits;               // [vocab], every token's logits (the last token's remain)
+    const void* embTable;        // embKind 0: the lm_head's int8 rows (embScales = its row scales), 1: fp16 table,
+    const float* embScales;      //         2: fp32 table, 3: the lm_head's Q4_0 planes
+    const float* cosTab; const float* sinTab;    // [maxSeq, headDim/2]
+    StepState* state;            // read at the start (pos, token, count, nPrompt), written at the end of the launch
+    int* history;                // greedy tokens go to history[count ..]
+    const int* prompt;           // while pos + 1 < nPrompt the next token is prompt[pos + 1] (optional)
+    float* amax;                 // argmax exchange: [2][grid] slots of FLOW_AMAX_STRIDE floats (value, index, rest unused),
+                                 // part of the exchange allocation
+    float* ropeCur;              // cos then sin row of the position after the launch (optional)
+    int embKind, vocab, historyCap;
+};
+
 // Exchange area: per layer one block of `stride` floats holding, at the offsets below, the rotated query,
 // the K and V rows of the current position, the attention partials of up to smax KV splits (accumulator,
 // maximum, sum), the hidden state after the attention block, the SwiGLU vector and the layer's output.
@@ -41,6 +59,7 @@ FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int nKVHeads
 bool flow_context_fits(int maxSeq, const FlowGeometry& g);
 
 constexpr size_t FLOW_ERR_BYTES = 4096;
+constexpr int FLOW_AMAX_STRIDE = 32;   // floats between two workgroups' argmax slots: a 128-byte line each
 
 // Trace slots of a layer, in program order: when thread 0 of a workgroup passed the point.
 constexpr int FLOW_TRACE_SLOTS = 11;
@@ -67,8 +86,13 @@ struct FlowParams {
     int* err;                    // FLOW_ERR_BYTES of zeros: word 0 is set to 1 when a wait ran into its time limit; bytes
                                  // 256 .. 2304 are the idle lines (never written; polls with nothing to ask for go there)
     long long limitTicks;        // per wait, in ticks of the 100 MHz wall clock
-    long long* trace;            // optional (diagnostic): wall-clock ticks [layer][FLOW_TRACE_SLOTS][workgroup], see FLOW_TRACE_NAMES
+    long long* trace;            // optional (diagnostic): wall-clock ticks [layer][FLOW_TRACE_SLOTS][workgroup], see FLOW_TRACE_NAMES;
+                                 // in token mode one more "layer" for the tail: FLOW_TAIL_TRACE_NAMES
+    int nTokens;                 // 0: layers [l0, l1) of one step, hidden in and out; n >= 1: token mode -- n whole tokens from the
+                                 // device state on (all layers; xchg holds two halves and the argmax exchange; state != NULL)
+    const FlowTail* tail;        // token mode
 };
+#define FLOW_TAIL_TRACE_NAMES "tail-top", "final-input-staged", "lm-head-done", "token-known", "all-waves-done", "partials-in"
 
 // Of `cus` workgroups that can be resident at once, how many the launch sets aside to prefetch weights into the L2s
 // (0 where that does not pay: layers too large for the L2s, or a phase that would need another round of the waves).
@@ -82,7 +106,16 @@ bool flow_grid_fits(int ffn, int nHeads, const FlowGeometry& g, int nCompute);
 // grid workgroups of 512 threads, all of which must be resident at once (grid <= CUs x resident workgroups per CU);
 // grid - p.nCompute of them prefetch (0, or a multiple of 8 with nCompute a multiple of 8 as well).
 hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s);
-// Fills the blocks of layers [l0, l1) with the "not written yet" pattern.
+// Fills the blocks of layers [l0, l1) (of the first half) with the "not written yet" pattern.
 hipError_t launch_flow_reset(float* xchg, const FlowGeometry& g, int l0, int l1, hipStream_t s);
+// Floats of the whole exchange allocation: two halves of nLayers blocks (token mode alternates between them; launches
+// over a range of layers use the first) and the argmax exchange [2][grid] pairs behind them.
+size_t flow_xchg_floats(const FlowGeometry& g, int nLayers, int grid);
+inline float* flow_amax_area(float* xchg, const FlowGeometry& g, int nLayers) { return xchg + (size_t)2 * nLayers * g.stride; }
+// ... all of it (before the first token-mode launch after the position was set by the host).
+hipError_t launch_flow_reset_all(float* xchg, const FlowGeometry& g, int nLayers, int grid, hipStream_t s);
+// LDS a workgroup of the launch takes (an upper bound: dynamic part plus the variant's own arrays); token mode keeps
+// the token's embedding beside the staged vector.  Must stay within the CU's 160 KB.
+size_t flow_lds_bytes(int dim, int ffn, int headDim, int gqa, bool tokenMode);
 
 }  // namespace mg

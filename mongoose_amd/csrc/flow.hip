@@ -164,6 +164,36 @@ __device__ __forceinline__ FlowLayer unpack_layer(unsigned v) {
     return L;
 }
 #undef FL_PTR
+// The tail's operands (FlowTail), read the same way: one word a lane, fields picked out where they are used.
+__device__ __forceinline__ unsigned tail_words(const FlowTail* t, int lane) {
+    static_assert(sizeof(FlowTail) <= 64 * 4, "one word a lane");
+    const unsigned* q = reinterpret_cast<const unsigned*>(t);
+    return q[lane < (int)(sizeof(FlowTail) / 4) ? lane : 0];
+}
+#define TW_PTR(T, field) lane_ptr<T>(tw, (int)(offsetof(FlowTail, field) / 4))
+#define TW_INT(field) __builtin_amdgcn_readlane((int)tw, (int)(offsetof(FlowTail, field) / 4))
+
+// An argmax partial: value (low word) and index (high word) travel as one 8-byte store and one 8-byte load; a
+// workgroup's partial has a 128-byte line of its own (FLOW_AMAX_STRIDE floats), written once a token.
+__device__ __forceinline__ void store_arg(float* slot, float v, int i) {
+    const unsigned long long w = (unsigned long long)__builtin_bit_cast(unsigned, canon(v)) | ((unsigned long long)(unsigned)i << 32);
+    asm volatile("global_store_dwordx2 %0, %1, off sc1" : : "v"(slot), "v"(w) : "memory");
+}
+struct ArgPart { float v; int i; };
+__device__ __forceinline__ ArgPart poll_arg(const float* p, Waiter& w) {
+    unsigned long long x;
+    long long t0 = 0;
+    bool timing = false;
+    for (;;) {
+        asm volatile("global_load_dwordx2 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(x) : "v"(p) : "memory");
+        const unsigned missing = ((unsigned)x == XSENT ? 1u : 0u) | ((unsigned)(x >> 32) == XSENT ? 1u : 0u);
+        if (!missing || w.dead) break;
+        if (!timing) { timing = true; t0 = wall_clock64(); }
+        else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
+        for (int z = 0; z < 4; z++) __builtin_amdgcn_s_sleep(2);
+    }
+    return ArgPart{__builtin_bit_cast(float, (unsigned)x), (int)(unsigned)(x >> 32)};
+}
 
 constexpr int PB = 3;        // float4 pieces a thread polls at once (a round of the 512 threads covers 6144 floats)
 // Every polling loop here has one shape: a straight loop around ONE asm statement (a fixed number of loads and their
@@ -526,11 +556,13 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     __shared__ float lbuf[QHMAX][FWAVES], wred[QHMAX][FWAVES];
     __shared__ float outbuf[FLOW_MAX_ROUNDS][FWAVES];                // a phase's results of the workgroup, stored by one wave as whole 32-byte runs
     __shared__ int4 pfScrap[64];                       // where the prefetching loads land (never read)
+    __shared__ float tailV[FWAVES];                    // the tail's argmax: the waves' best values and indices
+    __shared__ int tailI[FWAVES];
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int tid = threadIdx.x, lane = tid & 63;
+    int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nC = p.nCompute;                         // workgroups that compute; those after them prefetch
-    const int gw = blockIdx.x * FWAVES + wave;         // this wave among all computing waves of the launch
+    int gw = blockIdx.x * FWAVES + wave;               // this wave among all computing waves of the launch
     const int W = nC * FWAVES;
     // The rows of a workgroup's eight waves are consecutive (row = base + wave + k W), so their results go out as runs
     // of eight floats in one store instruction of wave 0 instead of eight single-float stores from eight waves: a line
@@ -550,76 +582,11 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             }
         }
     };
-    const int dim = p.dim, kvDim = p.kvDim, ffn = p.ffn;
-    const int nchD = dim >> 4, nchF = ffn >> 4;
+    int dim = p.dim, kvDim = p.kvDim, ffn = p.ffn;
+    int nchD = dim >> 4, nchF = ffn >> 4;
     const FlowGeometry G = p.geo;
-    const int pos = p.state ? p.state->pos : p.posImm;
     // (the idle lines follow the error word's 256 bytes: 16 lines of 128 bytes, two workgroups of an XCD on each)
     Waiter wt{p.limitTicks, p.err, false, reinterpret_cast<const f4*>(reinterpret_cast<const char*>(p.err) + 256 + ((blockIdx.x >> 3) & 15) * 128)};
-
-    if ((int)blockIdx.x >= nC) {
-        // ---- prefetch role (see Prefetcher): per layer three jobs, each released by a vector of the layer before ----
-        const int pi = (int)blockIdx.x - nC;
-        Prefetcher pf{pi & 7, pi >> 3, ((int)gridDim.x - nC) >> 3, tid, pfScrap};
-        const size_t rbD = Q4 ? dim >> 1 : dim, rbF = Q4 ? ffn >> 1 : ffn;      // bytes of a row of dim / of ffn weights
-        const size_t rdD = dim >> 4, rdF = ffn >> 4;                             // ... of its fp16 d values (Q4_0)
-        const int halfHd = HD >> 1;
-        unsigned lwp = layer_words(p.layers, p.l0, lane);
-        for (int l = p.l0; l < p.l1; l++) {
-            const FlowLayer L = unpack_layer(lwp);
-            if (l + 1 < p.l1) lwp = layer_words(p.layers, l + 1, lane);
-            const float* Xp = p.xchg + (size_t)(l - 1) * G.stride;               // the layer before (not for the first)
-            // (Measured at the 0.5B shape: releasing every job a phase earlier or later, and 24 to 48 prefetching
-            // workgroups, all give the same step time within 0.5 %; 16 are too few, 64 cost more than they bring.)
-            auto release = [&](int off) {
-                pf.drain();                // the job before has landed
-                if (l == p.l0) return;
-                if (tid == 0) (void)poll1(Xp + off, wt);
-                __syncthreads();
-            };
-            release(G.offX1);              // the layer before is past its Wo: q | k | v and Wo of this one
-            {
-                const int nq = dim >> 1, nk = kvDim >> 1, nI = nq + 2 * nk;
-                for (int g = pf.x + 8 * pf.rank; g * 8 < nI; g += 8 * pf.nRank) {
-                    const int item = g * 8;
-                    const signed char* Wm; const float* aux; int a0, a1;
-                    if (item < nq) { Wm = L.wq; aux = L.sq; const int jj = item % halfHd; a0 = (item - jj) * 2 + jj; a1 = a0 + halfHd; }
-                    else if (item < nq + nk) { Wm = L.wk; aux = L.sk; const int i2 = item - nq; const int jj = i2 % halfHd; a0 = (i2 - jj) * 2 + jj; a1 = a0 + halfHd; }
-                    else { Wm = L.wv; aux = L.sv; a0 = (item - nq - nk) * 2; a1 = a0 + 8; }
-                    const char* wb = reinterpret_cast<const char*>(Wm);
-                    pf.span(wb, (size_t)a0 * rbD, (size_t)(a0 + 8) * rbD);
-                    pf.span(wb, (size_t)a1 * rbD, (size_t)(a1 + 8) * rbD);
-                    if (Q4) {
-                        const char* db = reinterpret_cast<const char*>(aux);
-                        pf.span(db, ((size_t)a0 * rdD) & ~(size_t)15, (size_t)(a0 + 8) * rdD);
-                        pf.span(db, ((size_t)a1 * rdD) & ~(size_t)15, (size_t)(a1 + 8) * rdD);
-                    }
-                }
-                if (!Q4) { pf.whole(L.sq, (size_t)dim * 4); pf.whole(L.sk, (size_t)kvDim * 4); pf.whole(L.sv, (size_t)kvDim * 4); }
-                pf.whole(L.bq, (size_t)dim * 4); pf.whole(L.bk, (size_t)kvDim * 4); pf.whole(L.bv, (size_t)kvDim * 4);
-                pf.whole(L.g1, (size_t)dim * 4);
-                pf.rows(L.wo, rbD, dim, 8);
-                if (Q4) pf.rows(L.so, rdD, dim, 8); else pf.whole(L.so, (size_t)dim * 4);
-                // the K / V rows of the earlier positions (the attention workgroups of every XCD read them; the row of the
-                // current position comes through the exchange area), while they are a small part of an L2: 0.5B shape at
-                // positions 16 .. 216 0.3766 -> 0.3710 ms a token
-                const size_t kvBytes = (size_t)pos * kvDim * 4;
-                if (kvBytes <= ((size_t)512 << 10)) { pf.whole(L.Kc, kvBytes); pf.whole(L.Vc, kvBytes); }
-            }
-            release(G.offM);               // ... past its gate | up: gate | up of this one
-            pf.rows(L.gate, rbD, ffn, 8);
-            pf.rows(L.up, rbD, ffn, 8);
-            if (Q4) { pf.rows(L.sgate, rdD, ffn, 8); pf.rows(L.sup, rdD, ffn, 8); }
-            else { pf.whole(L.sgate, (size_t)ffn * 4); pf.whole(L.sup, (size_t)ffn * 4); }
-            pf.whole(L.g2, (size_t)dim * 4);
-            release(G.offX2);              // ... done: the down projection of this one
-            const int drun = p.downSplit ? FWAVES / 2 : FWAVES;      // rows of the down projection a workgroup takes
-            pf.rows(L.down, rbF, dim, drun);
-            if (Q4) pf.rows(L.sdown, rdF, dim, drun); else pf.whole(L.sdown, (size_t)dim * 4);
-        }
-        pf.drain();
-        return;
-    }
 
     // attention geometry (decode attention of kernels.hip with one query head per workgroup): a thread group of 16
     // lanes holds a K/V row, a thread VU rows of its workgroup's tile of FLOW_TILE positions.  (Measured on the 0.5B
@@ -630,613 +597,876 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     const int half = HD >> 1;
 
     // timing trace (diagnostic): slot b of layer l, per workgroup, in ticks of the 100 MHz wall clock
-#define FLOW_TRACE(b) do { if (p.trace && tid == 0) \
+#define FLOW_TRACE(b) do { if (p.trace && tid == 0 && (int)blockIdx.x < nC) \
         p.trace[((size_t)(l - p.l0) * FLOW_TRACE_SLOTS + (b)) * nC + blockIdx.x] = wall_clock64(); } while (0)
     // the exchange area as a buffer resource: agent-scope loads that the compiler keeps track of (used where many are
     // wanted in flight together)
-    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(p.xchg, 0, (int)((size_t)p.nLayersTotal * G.stride * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(p.xchg, 0, (int)((size_t)p.nLayersTotal * G.stride * 4 * (p.nTokens > 0 ? 2 : 1)), 0x00020000);
     unsigned lw = layer_words(p.layers, p.l0, lane);
-    for (int l = p.l0; l < p.l1; l++) {
-        const FlowLayer L = unpack_layer(lw);
-        if (l + 1 < p.l1) lw = layer_words(p.layers, l + 1, lane);
-        FLOW_TRACE(0);
-        float* X = p.xchg + (size_t)l * G.stride;
-        const bool first = l == p.l0;
-        const float* xin = first ? p.hidden : p.xchg + (size_t)(l - 1) * G.stride + G.offX2;
 
-        // ------------------------------------------------------------------ q | k | v
-        {
-            const int nq = dim >> 1, nk = kvDim >> 1, nI = nq + 2 * nk;       // RoPE pairs of q, of k; row pairs of v
-            if (blockIdx.x * FWAVES < nI) {
-                // The first NPI items of a wave are requested whole (CBQ chunks a lane and row) before the input is waited for;
-                // further items, and chunks past CBQ, are read where they are used.
-                constexpr int NPI = 1, CBQ = CBD;
-                int4 wr[NPI][2][CBQ];
-                WRow rows[NPI][2];
-                int kind[NPI], r0[NPI], r1[NPI];
-                float e0[NPI], e1[NPI];                  // per-lane epilogue operands: lanes 0/1 scale and bias, lane 2 cos and sin
-                auto resolve = [&](int4 (&w)[2][CBQ], WRow (&rw)[2], int& kd, int& a0, int& a1, float& f0, float& f1, int item) {
-                    const signed char* Wm; const float* sc; const float* bias;
-                    if (item < nq) { kd = 0; Wm = L.wq; sc = L.sq; bias = L.bq; const int jj = item % half; a0 = (item - jj) * 2 + jj; a1 = a0 + half; }
-                    else if (item < nq + nk) { kd = 1; Wm = L.wk; sc = L.sk; bias = L.bk; const int i2 = item - nq; const int jj = i2 % half; a0 = (i2 - jj) * 2 + jj; a1 = a0 + half; }
-                    else { kd = 2; Wm = L.wv; sc = L.sv; bias = L.bv; a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
-                    rw[0] = wrow<Q4>(Wm, sc, a0, dim); rw[1] = wrow<Q4>(Wm, sc, a1, dim);
-                    ld_row<GL, Q4, CBQ>(rw[0], nchD, lane, 0, w[0]);
-                    ld_row<GL, Q4, CBQ>(rw[1], nchD, lane, 0, w[1]);
-                    f0 = 1.f; f1 = 0.f;
-                    if (lane < 2) {
-                        const int r = lane ? a1 : a0;
-                        if (!Q4) f0 = ldg_f<GL>(sc, r);
-                        if (bias) f1 = ldg_f<GL>(bias, r);
-                    }
-                    if (lane == 2 && kd < 2) { const int jj = a0 % half; f0 = p.cosRow[jj]; f1 = p.sinRow[jj]; }
-                };
-                // one item of every wave of the workgroup: dot, epilogue, the results out as runs by wave 0
-                auto finish = [&](const int4 (&w)[2][CBQ], const WRow (&rw)[2], int kd, float f0, float f1, float rs, int it) {
-                    float acc[2] = {0.f, 0.f};
-                    dot_rows<Q4, 2, CBQ>(w, a4, nchD, lane, 0, acc);
-                    if (nchD > CBQ * 64) dot_rows_tail<GL, Q4, 2, CBQ>(rw, a4, nchD, lane, acc);
-                    const float t = wave_sum2(acc[0], acc[1]);
-                    float v = lane == 1 ? lane_value(t, 32) : t;
-                    v = v * f0;                                                  // row scale (lanes 0 and 1)
-                    v = v * rs;
-                    v = v + f1;
-                    const float v1 = dpp_f<0x101>(v);                            // lane 0 reads lane 1: the pair's second row
-                    const float cs = dpp_f<0x102>(f0), sn = dpp_f<0x102>(f1);    // lane 0 reads lane 2
-                    float o0 = v, o1 = v1;
-                    if (kd < 2) { o0 = v * cs - v1 * sn; o1 = v * sn + v1 * cs; }            // mongoose.cu:991-1006
-                    // the eight waves' rows are consecutive (first rows of the pairs, and second rows)
-                    if (it != gw) __syncthreads();              // outbuf is free again
-                    if (lane == 0) { outbuf[0][wave] = o0; outbuf[1][wave] = o1; }
+    // Token mode (p.nTokens > 0): the launch runs whole tokens -- the embedding of the token in the device state, all
+    // layers, and the tail (final norm, lm_head, greedy argmax; cuda_fused_infer.go:446-450 and what the reference's
+    // caller does with the logits), nTokens of them, every token's successor chosen on the device.  The exchange area
+    // then has two halves, used by even and by odd positions: during a token's tail all workgroups reset the other
+    // half for the token after it.  (Nothing of the token before is read any more once a workgroup has got there:
+    // every workgroup reads every workgroup's argmax partial, so a token starts only when all are through the last.)
+    const bool tokens = p.nTokens > 0;
+    const int nTok = tokens ? p.nTokens : 1;
+    const unsigned tw = tokens ? tail_words(p.tail, lane) : 0u;
+    int pos = p.state ? p.state->pos : p.posImm;
+    int tok = tokens ? p.state->token : 0;
+    const int count0 = tokens ? p.state->count : 0, nPrompt = tokens ? p.state->nPrompt : 0;
+    const size_t halfFloats = (size_t)p.nLayersTotal * G.stride;
+    float* const xemb = reinterpret_cast<float*>(a4) + (dim > ffn ? dim : ffn);      // the token's embedding (token mode)
+    for (int tk = 0; tk < nTok; tk++) {
+        // Nothing that depends on the thread or on the shape is to be computed once for all tokens and kept in registers
+        // across the whole launch (hundreds of addresses and offsets otherwise are): every token derives them again.
+        asm volatile("" : "+v"(tid), "+v"(lane));
+        asm volatile("" : "+s"(wave), "+s"(gw), "+s"(dim), "+s"(kvDim), "+s"(ffn), "+s"(nchD), "+s"(nchF));
+        float* const xb = p.xchg + (tokens ? (size_t)(pos & 1) * halfFloats : (size_t)0);
+        const unsigned xoff = tokens ? (unsigned)((size_t)(pos & 1) * halfFloats) : 0u;
+        const float* cosRow = p.cosRow;
+        const float* sinRow = p.sinRow;
+        if (tokens) {
+            cosRow = TW_PTR(const float, cosTab) + (size_t)pos * half;
+            sinRow = TW_PTR(const float, sinTab) + (size_t)pos * half;
+            const void* et = TW_PTR(const void, embTable);
+            const float* es = TW_PTR(const float, embScales);
+            const int ek = TW_INT(embKind), vocab = TW_INT(vocab);
+            __syncthreads();                               // the token before has no reader of xemb left
+            const int tc = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+            for (int i = tid; i < dim; i += FWG) xemb[i] = embed_value(ek, et, es, tc, dim, vocab, i);
+            __syncthreads();
+        }
+
+        if ((int)blockIdx.x >= nC) {
+            // ---- prefetch role (see Prefetcher): per layer three jobs, each released by a vector of the layer before ----
+            const int pi = (int)blockIdx.x - nC;
+            Prefetcher pf{pi & 7, pi >> 3, ((int)gridDim.x - nC) >> 3, tid, pfScrap};
+            const size_t rbD = Q4 ? dim >> 1 : dim, rbF = Q4 ? ffn >> 1 : ffn;      // bytes of a row of dim / of ffn weights
+            const size_t rdD = dim >> 4, rdF = ffn >> 4;                             // ... of its fp16 d values (Q4_0)
+            const int halfHd = HD >> 1;
+            for (int l = p.l0; l < p.l1; l++) {
+                const FlowLayer L = unpack_layer(lw);
+                if (l + 1 < p.l1) lw = layer_words(p.layers, l + 1, lane);
+                else if (tk + 1 < nTok) lw = layer_words(p.layers, p.l0, lane);
+                const float* Xp = xb + (size_t)(l - 1) * G.stride;               // the layer before (not for the first)
+                // (Measured at the 0.5B shape: releasing every job a phase earlier or later, and 24 to 48 prefetching
+                // workgroups, all give the same step time within 0.5 %; 16 are too few, 64 cost more than they bring.)
+                auto release = [&](int off) {
+                    pf.drain();                // the job before has landed
+                    if (l == p.l0) return;
+                    if (tid == 0) (void)poll1(Xp + off, wt);
                     __syncthreads();
-                    if (wave == 0 && lane < 2 * FWAVES) {
-                        const int k = lane / FWAVES, wv = lane % FWAVES, item = it + wv;
-                        if (item < nI) {
-                            int kk, a0, a1;
-                            if (item < nq) { kk = 0; const int jj = item % half; a0 = (item - jj) * 2 + jj; a1 = a0 + half; }
-                            else if (item < nq + nk) { kk = 1; const int i2 = item - nq; const int jj = i2 % half; a0 = (i2 - jj) * 2 + jj; a1 = a0 + half; }
-                            else { kk = 2; a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
-                            const int r = k ? a1 : a0;
-                            const float o = outbuf[k][wv];
-                            if (kk == 0) {
-                                stx(X + G.offQ + r, o);
-                            } else {                                              // mongoose.cu:1644-1647, and the hand-over copy
-                                stg_f<GL>(kk == 1 ? L.Kc : L.Vc, (size_t)pos * kvDim + r, o);
-                                stx(X + (kk == 1 ? G.offKc : G.offVc) + r, o);
+                };
+                release(G.offX1);              // the layer before is past its Wo: q | k | v and Wo of this one
+                {
+                    const int nq = dim >> 1, nk = kvDim >> 1, nI = nq + 2 * nk;
+                    for (int g = pf.x + 8 * pf.rank; g * 8 < nI; g += 8 * pf.nRank) {
+                        const int item = g * 8;
+                        const signed char* Wm; const float* aux; int a0, a1;
+                        if (item < nq) { Wm = L.wq; aux = L.sq; const int jj = item % halfHd; a0 = (item - jj) * 2 + jj; a1 = a0 + halfHd; }
+                        else if (item < nq + nk) { Wm = L.wk; aux = L.sk; const int i2 = item - nq; const int jj = i2 % halfHd; a0 = (i2 - jj) * 2 + jj; a1 = a0 + halfHd; }
+                        else { Wm = L.wv; aux = L.sv; a0 = (item - nq - nk) * 2; a1 = a0 + 8; }
+                        const char* wb = reinterpret_cast<const char*>(Wm);
+                        pf.span(wb, (size_t)a0 * rbD, (size_t)(a0 + 8) * rbD);
+                        pf.span(wb, (size_t)a1 * rbD, (size_t)(a1 + 8) * rbD);
+                        if (Q4) {
+                            const char* db = reinterpret_cast<const char*>(aux);
+                            pf.span(db, ((size_t)a0 * rdD) & ~(size_t)15, (size_t)(a0 + 8) * rdD);
+                            pf.span(db, ((size_t)a1 * rdD) & ~(size_t)15, (size_t)(a1 + 8) * rdD);
+                        }
+                    }
+                    if (!Q4) { pf.whole(L.sq, (size_t)dim * 4); pf.whole(L.sk, (size_t)kvDim * 4); pf.whole(L.sv, (size_t)kvDim * 4); }
+                    pf.whole(L.bq, (size_t)dim * 4); pf.whole(L.bk, (size_t)kvDim * 4); pf.whole(L.bv, (size_t)kvDim * 4);
+                    pf.whole(L.g1, (size_t)dim * 4);
+                    pf.rows(L.wo, rbD, dim, 8);
+                    if (Q4) pf.rows(L.so, rdD, dim, 8); else pf.whole(L.so, (size_t)dim * 4);
+                    // the K / V rows of the earlier positions (the attention workgroups of every XCD read them; the row of the
+                    // current position comes through the exchange area), while they are a small part of an L2: 0.5B shape at
+                    // positions 16 .. 216 0.3766 -> 0.3710 ms a token
+                    const size_t kvBytes = (size_t)pos * kvDim * 4;
+                    if (kvBytes <= ((size_t)512 << 10)) { pf.whole(L.Kc, kvBytes); pf.whole(L.Vc, kvBytes); }
+                }
+                release(G.offM);               // ... past its gate | up: gate | up of this one
+                pf.rows(L.gate, rbD, ffn, 8);
+                pf.rows(L.up, rbD, ffn, 8);
+                if (Q4) { pf.rows(L.sgate, rdD, ffn, 8); pf.rows(L.sup, rdD, ffn, 8); }
+                else { pf.whole(L.sgate, (size_t)ffn * 4); pf.whole(L.sup, (size_t)ffn * 4); }
+                pf.whole(L.g2, (size_t)dim * 4);
+                release(G.offX2);              // ... done: the down projection of this one
+                const int drun = p.downSplit ? FWAVES / 2 : FWAVES;      // rows of the down projection a workgroup takes
+                pf.rows(L.down, rbF, dim, drun);
+                if (Q4) pf.rows(L.sdown, rdF, dim, drun); else pf.whole(L.sdown, (size_t)dim * 4);
+            }
+            pf.drain();
+        } else {
+            for (int l = p.l0; l < p.l1; l++) {
+                // (the same per layer: offsets that do not depend on the layer would otherwise be kept across all phases, and
+                // the phases' own working sets then no longer fit the registers)
+                asm volatile("" : "+v"(tid), "+v"(lane));
+                asm volatile("" : "+s"(wave), "+s"(gw), "+s"(dim), "+s"(kvDim), "+s"(ffn), "+s"(nchD), "+s"(nchF));
+                const FlowLayer L = unpack_layer(lw);
+                if (l + 1 < p.l1) lw = layer_words(p.layers, l + 1, lane);
+                else if (tk + 1 < nTok) lw = layer_words(p.layers, p.l0, lane);
+                FLOW_TRACE(0);
+                float* X = xb + (size_t)l * G.stride;
+                const bool first = l == p.l0;
+                const float* xin = first ? (tokens ? xemb : p.hidden) : xb + (size_t)(l - 1) * G.stride + G.offX2;
+
+                // ------------------------------------------------------------------ q | k | v
+                {
+                    const int nq = dim >> 1, nk = kvDim >> 1, nI = nq + 2 * nk;       // RoPE pairs of q, of k; row pairs of v
+                    if (blockIdx.x * FWAVES < nI) {
+                        // The first NPI items of a wave are requested whole (CBQ chunks a lane and row) before the input is waited for;
+                        // further items, and chunks past CBQ, are read where they are used.
+                        constexpr int NPI = 1, CBQ = CBD;
+                        int4 wr[NPI][2][CBQ];
+                        WRow rows[NPI][2];
+                        int kind[NPI], r0[NPI], r1[NPI];
+                        float e0[NPI], e1[NPI];                  // per-lane epilogue operands: lanes 0/1 scale and bias, lane 2 cos and sin
+                        auto resolve = [&](int4 (&w)[2][CBQ], WRow (&rw)[2], int& kd, int& a0, int& a1, float& f0, float& f1, int item) {
+                            const signed char* Wm; const float* sc; const float* bias;
+                            if (item < nq) { kd = 0; Wm = L.wq; sc = L.sq; bias = L.bq; const int jj = item % half; a0 = (item - jj) * 2 + jj; a1 = a0 + half; }
+                            else if (item < nq + nk) { kd = 1; Wm = L.wk; sc = L.sk; bias = L.bk; const int i2 = item - nq; const int jj = i2 % half; a0 = (i2 - jj) * 2 + jj; a1 = a0 + half; }
+                            else { kd = 2; Wm = L.wv; sc = L.sv; bias = L.bv; a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
+                            rw[0] = wrow<Q4>(Wm, sc, a0, dim); rw[1] = wrow<Q4>(Wm, sc, a1, dim);
+                            ld_row<GL, Q4, CBQ>(rw[0], nchD, lane, 0, w[0]);
+                            ld_row<GL, Q4, CBQ>(rw[1], nchD, lane, 0, w[1]);
+                            f0 = 1.f; f1 = 0.f;
+                            if (lane < 2) {
+                                const int r = lane ? a1 : a0;
+                                if (!Q4) f0 = ldg_f<GL>(sc, r);
+                                if (bias) f1 = ldg_f<GL>(bias, r);
                             }
+                            if (lane == 2 && kd < 2) { const int jj = a0 % half; f0 = cosRow[jj]; f1 = sinRow[jj]; }
+                        };
+                        // one item of every wave of the workgroup: dot, epilogue, the results out as runs by wave 0
+                        auto finish = [&](const int4 (&w)[2][CBQ], const WRow (&rw)[2], int kd, float f0, float f1, float rs, int it) {
+                            float acc[2] = {0.f, 0.f};
+                            dot_rows<Q4, 2, CBQ>(w, a4, nchD, lane, 0, acc);
+                            if (nchD > CBQ * 64) dot_rows_tail<GL, Q4, 2, CBQ>(rw, a4, nchD, lane, acc);
+                            const float t = wave_sum2(acc[0], acc[1]);
+                            float v = lane == 1 ? lane_value(t, 32) : t;
+                            v = v * f0;                                                  // row scale (lanes 0 and 1)
+                            v = v * rs;
+                            v = v + f1;
+                            const float v1 = dpp_f<0x101>(v);                            // lane 0 reads lane 1: the pair's second row
+                            const float cs = dpp_f<0x102>(f0), sn = dpp_f<0x102>(f1);    // lane 0 reads lane 2
+                            float o0 = v, o1 = v1;
+                            if (kd < 2) { o0 = v * cs - v1 * sn; o1 = v * sn + v1 * cs; }            // mongoose.cu:991-1006
+                            // the eight waves' rows are consecutive (first rows of the pairs, and second rows)
+                            if (it != gw) __syncthreads();              // outbuf is free again
+                            if (lane == 0) { outbuf[0][wave] = o0; outbuf[1][wave] = o1; }
+                            __syncthreads();
+                            if (wave == 0 && lane < 2 * FWAVES) {
+                                const int k = lane / FWAVES, wv = lane % FWAVES, item = it + wv;
+                                if (item < nI) {
+                                    int kk, a0, a1;
+                                    if (item < nq) { kk = 0; const int jj = item % half; a0 = (item - jj) * 2 + jj; a1 = a0 + half; }
+                                    else if (item < nq + nk) { kk = 1; const int i2 = item - nq; const int jj = i2 % half; a0 = (i2 - jj) * 2 + jj; a1 = a0 + half; }
+                                    else { kk = 2; a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
+                                    const int r = k ? a1 : a0;
+                                    const float o = outbuf[k][wv];
+                                    if (kk == 0) {
+                                        stx(X + G.offQ + r, o);
+                                    } else {                                              // mongoose.cu:1644-1647, and the hand-over copy
+                                        // (write-through: the next token of the same launch reads the row on other XCDs)
+                                        st_agent((kk == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim + r, o);
+                                        stx(X + (kk == 1 ? G.offKc : G.offVc) + r, o);
+                                    }
+                                }
+                            }
+                        };
+#pragma unroll
+                        for (int q = 0; q < NPI; q++) {
+                            kind[q] = 0; r0[q] = 0; r1[q] = 0; e0[q] = 0.f; e1[q] = 0.f; rows[q][0] = wrow<Q4>(L.wq, L.sq, 0, dim); rows[q][1] = rows[q][0];
+                            if (gw + q * W < nI) resolve(wr[q], rows[q], kind[q], r0[q], r1[q], e0[q], e1[q], gw + q * W);
+                        }
+                        const float rs = stage_rms<GL, Q4, !RING>(xin, !first, L.g1, dim, p.eps, a4, red, wt);
+                        FLOW_TRACE(1);
+#pragma unroll
+                        for (int q = 0; q < NPI; q++)
+                            if (blockIdx.x * FWAVES + q * W < nI) finish(wr[q], rows[q], kind[q], e0[q], e1[q], rs, gw + q * W);      // uniform in the workgroup
+                        for (int it = gw + NPI * W; it - wave < nI; it += W) {         // it - wave: the same for all waves of the workgroup
+                            if (it < nI) resolve(wr[0], rows[0], kind[0], r0[0], r1[0], e0[0], e1[0], it);
+                            finish(wr[0], rows[0], kind[0], e0[0], e1[0], rs, it);
                         }
                     }
-                };
-#pragma unroll
-                for (int q = 0; q < NPI; q++) {
-                    kind[q] = 0; r0[q] = 0; r1[q] = 0; e0[q] = 0.f; e1[q] = 0.f; rows[q][0] = wrow<Q4>(L.wq, L.sq, 0, dim); rows[q][1] = rows[q][0];
-                    if (gw + q * W < nI) resolve(wr[q], rows[q], kind[q], r0[q], r1[q], e0[q], e1[q], gw + q * W);
                 }
-                const float rs = stage_rms<GL, Q4, !RING>(xin, !first, L.g1, dim, p.eps, a4, red, wt);
-                FLOW_TRACE(1);
-#pragma unroll
-                for (int q = 0; q < NPI; q++)
-                    if (blockIdx.x * FWAVES + q * W < nI) finish(wr[q], rows[q], kind[q], e0[q], e1[q], rs, gw + q * W);      // uniform in the workgroup
-                for (int it = gw + NPI * W; it - wave < nI; it += W) {         // it - wave: the same for all waves of the workgroup
-                    if (it < nI) resolve(wr[0], rows[0], kind[0], r0[0], r1[0], e0[0], e1[0], it);
-                    finish(wr[0], rows[0], kind[0], e0[0], e1[0], rs, it);
-                }
-            }
-        }
 
-        FLOW_TRACE(2);
-        // ------------------------------------------------------------------ attention: one (head, KV split) per workgroup
-        // grouped only while a workgroup per query head and split would not fit the launch (positions far into a long context)
-        const bool grouped = GQA && p.nHeads * (pos / TILE + 1) > nC;
-        {
-            const int nsplit = pos / TILE + 1;
-            // Grouped: the query heads of a KV head are shared out over as many workgroups as the launch has left for
-            // them at this position (each loads the K / V rows once and takes its heads in turn), so a workgroup takes as
-            // few heads as possible: qhMax heads a workgroup, `sub` workgroups a KV head and split.
-            const int Gq = p.nHeads / p.nKVHeads;
-            int qhMax = 1, sub = Gq;
-            if (grouped) {
-                qhMax = Gq; sub = 1;
-                const int live = nsplit < G.smax ? nsplit : G.smax;
-                for (int q = 2; q < Gq; q++) {
-                    const int sb = (Gq + q - 1) / q;
-                    if (p.nKVHeads * sb * live <= nC) { qhMax = q; sub = sb; break; }
-                }
-            }
-            const int unit = grouped ? p.nKVHeads * sub : p.nHeads;
-            const int split = blockIdx.x / unit, hu = blockIdx.x % unit;
-            const int hg = grouped ? hu % sub : 0;                         // which of the KV head's groups of query heads
-            const int QH = grouped ? min(qhMax, Gq - hg * qhMax) : 1;      // query heads of this workgroup
-            // Workgroups with no attention to do (and no partials to merge per head) read, into their XCD's L2, rows that the
-            // XCD's workgroups will want after it -- their next poll, for the attention's partials, is microseconds away, and
-            // HBM would be idle meanwhile.  p.idleWoRows: Wo (rows of more than 2048 weights, of which a wave requests only
-            // the first half-row ahead); p.idleGateUpRows: the leading rows of gate and of up -- all of them where both
-            // matrices fit the L2s (1.1B shape: 0.465 -> 0.436 ms a token; the down projection on top overflows the L2s:
-            // 0.470), else half of the first round of rows, which is what a phase waits for before it streams (8B shape
-            // with both: 1.845 -> 1.790; the whole first round 1.804, a quarter 1.800).
-            // Only while at least half the launch is idle (short contexts), and only without dedicated prefetchers.
-            if ((p.idleWoRows > 0 || p.idleGateUpRows > 0) && nC == (int)gridDim.x) {
-                const int live = nsplit < G.smax ? nsplit : G.smax;
-                int nBusy = unit * live;
-                if (grouped && nBusy < p.nHeads) nBusy = p.nHeads;
-                nBusy = (nBusy + 7) & ~7;
-                if ((int)blockIdx.x >= nBusy && 2 * ((int)gridDim.x - nBusy) >= (int)gridDim.x) {
-                    Prefetcher pf{(int)blockIdx.x & 7, ((int)blockIdx.x - nBusy) >> 3, ((int)gridDim.x - nBusy) >> 3, tid, pfScrap};
-                    const size_t rbD = Q4 ? dim >> 1 : dim, rdD = dim >> 4;
-                    // (a workgroup without q | k | v rows gets here at the top of the layer; holding it back until q | k | v is
-                    // through measures slower: 1.1B shape 0.453 against 0.435 ms a token)
-                    if (p.idleWoRows > 0) {
-                        pf.rows(L.wo, rbD, p.idleWoRows, 8);
-                        if (Q4) pf.rows(L.so, rdD, p.idleWoRows, 8);
-                    }
-                    if (p.idleGateUpRows > 0) {
-                        pf.rows(L.gate, rbD, p.idleGateUpRows, 8);
-                        pf.rows(L.up, rbD, p.idleGateUpRows, 8);
-                        if (Q4) { pf.rows(L.sgate, rdD, p.idleGateUpRows, 8); pf.rows(L.sup, rdD, p.idleGateUpRows, 8); }
-                    }
-                    pf.drain();
-                }
-            }
-            if (split < G.smax && split < nsplit) {
-                const int kvh = grouped ? hu / sub : hu / Gq;
-                const int h0 = grouped ? kvh * Gq + hg * qhMax : hu;
-                const int tg = tid / LPR, dl = tid % LPR;
-                const int t0 = split * TILE;
-                const int len = pos + 1;
-                const int t1 = min(len, t0 + TILE);
-                const int lastRow = p.maxSeq - 1;
-                const size_t rowStride = (size_t)kvDim / 4;
-                const size_t colOff = (size_t)(kvh * HD) / 4 + dl;
-                const float4* Kc4 = reinterpret_cast<const float4*>(L.Kc);
-                const float4* Vc4 = reinterpret_cast<const float4*>(L.Vc);
-                float4 kreg[VU][NF], vreg[VU][NF];
-#pragma unroll
-                for (int u = 0; u < VU; u++) {
-                    const size_t ro = (size_t)min(t0 + tg + u * TG, lastRow) * rowStride + colOff;
-#pragma unroll
-                    for (int j = 0; j < NF; j++) kreg[u][j] = ldg_f4<GL>(Kc4, ro + j * 16);
-#pragma unroll
-                    for (int j = 0; j < NF; j++) vreg[u][j] = ldg_f4<GL>(Vc4, ro + j * 16);
-                }
-                __syncthreads();
-                if (tid < (2 + QH) * (HD / 4)) {
-                    const int which = tid / (HD / 4), i = tid % (HD / 4);
-                    const float* src = which >= 2 ? X + G.offQ + (h0 + which - 2) * HD : X + (which == 0 ? G.offKc : G.offVc) + kvh * HD;
-                    sqkv[which][i] = tof4(poll4(reinterpret_cast<const f4*>(src) + i, wt));
-                }
-                __syncthreads();
-                FLOW_TRACE(3);
-                const int live = t1 - t0;
-                const float scale = 1.0f / sqrtf((float)HD);
-#pragma unroll
-                for (int u = 0; u < VU; u++) {
-                    if (t0 + tg + u * TG == pos) {          // the current position's rows come from this launch, not from the cache
-#pragma unroll
-                        for (int j = 0; j < NF; j++) { kreg[u][j] = sqkv[0][j * 16 + dl]; vreg[u][j] = sqkv[1][j * 16 + dl]; }
-                    }
-                }
-                for (int hi = 0; hi < QH; hi++) {          // the heads of the KV head in turn, on the same K / V registers
-                float4 q4[NF];
-#pragma unroll
-                for (int j = 0; j < NF; j++) q4[j] = sqkv[2 + hi][j * 16 + dl];
-                float sc[VU];
-                float tmax = -INFINITY;
-#pragma unroll
-                for (int u = 0; u < VU; u++) {
-                    sc[u] = -INFINITY;
-                    if (u * TG >= live) continue;
-                    const int row = t0 + tg + u * TG;
-                    float d = 0.f;
-#pragma unroll
-                    for (int j = 0; j < NF; j++) {
-                        d = fmaf(q4[j].x, kreg[u][j].x, d); d = fmaf(q4[j].y, kreg[u][j].y, d);
-                        d = fmaf(q4[j].z, kreg[u][j].z, d); d = fmaf(q4[j].w, kreg[u][j].w, d);
-                    }
-                    d = row_sum16(d);
-                    sc[u] = row < t1 ? d * scale : -INFINITY;
-                    tmax = fmaxf(tmax, sc[u]);
-                }
-                const float m = tg_max(tmax);               // the wave's maximum
-                const float mRef = m == -INFINITY ? 0.f : m;
-                float4 acc[NF];
-#pragma unroll
-                for (int j = 0; j < NF; j++) acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-                float lsum = 0.f;
-#pragma unroll
-                for (int u = 0; u < VU; u++) {
-                    if (u * TG >= live) continue;
-                    const float pv = exp_neg(sc[u] - mRef);
-                    lsum += pv;
-#pragma unroll
-                    for (int j = 0; j < NF; j++) {
-                        acc[j].x = fmaf(pv, vreg[u][j].x, acc[j].x); acc[j].y = fmaf(pv, vreg[u][j].y, acc[j].y);
-                        acc[j].z = fmaf(pv, vreg[u][j].z, acc[j].z); acc[j].w = fmaf(pv, vreg[u][j].w, acc[j].w);
-                    }
-                }
-#pragma unroll
-                for (int j = 0; j < NF; j++) {
-                    acc[j].x = tg_sum(acc[j].x); acc[j].y = tg_sum(acc[j].y); acc[j].z = tg_sum(acc[j].z); acc[j].w = tg_sum(acc[j].w);
-                    if (lane < LPR) accbuf[hi][wave][j * 16 + dl] = acc[j];
-                }
-                lsum = tg_sum(lsum);
-                if (lane == 0) { lbuf[hi][wave] = lsum; wred[hi][wave] = m; }
-                }
-                // the waves' partials of all the workgroup's heads combined together: one barrier, a thread per head and piece
-                __syncthreads();
-                if (tid < QH * (HD / 4)) {
-                    const int hq = tid / (HD / 4), i = tid % (HD / 4), h = h0 + hq;
-                    float mg_ = wred[hq][0];
-#pragma unroll
-                    for (int k = 1; k < FWAVES; k++) mg_ = fmaxf(mg_, wred[hq][k]);
-                    f4 r = {0.f, 0.f, 0.f, 0.f};
-                    float lg = 0.f;
-#pragma unroll
-                    for (int k = 0; k < FWAVES; k++) {
-                        const float wk = exp_neg(wred[hq][k] - mg_);
-                        const float4 a = accbuf[hq][k][i];
-                        r.x = fmaf(wk, a.x, r.x); r.y = fmaf(wk, a.y, r.y); r.z = fmaf(wk, a.z, r.z); r.w = fmaf(wk, a.w, r.w);
-                        lg = fmaf(wk, lbuf[hq][k], lg);
-                    }
-                    stx4(reinterpret_cast<f4*>(X + G.offPacc + (size_t)split * dim + h * HD) + i, r);
-                    if (i == 0) {
-                        stx(X + G.offPm + split * p.nHeads + h, mg_);
-                        stx(X + G.offPl + split * p.nHeads + h, lg);
-                    }
-                }
-            }
-        }
-
-        if (grouped) {
-            // Long contexts, tens of KV splits: merged once per head, by workgroup h for head h (every thread a 16-byte piece
-            // and every eighth split, eight splits' loads in flight together, then combined through LDS), and handed on as
-            // one vector -- every consumer merging all partials itself re-reads tens of KB per workgroup and layer.
-            if ((int)blockIdx.x < p.nHeads) {
-                constexpr int P4 = HD / 4, SG = FWG / P4;          // pieces of a head, split groups (thread = piece x group)
-                __shared__ float4 mnum[SG][P4];
-                __shared__ float mM[SG][P4], mden[SG][P4];
-                const int h = blockIdx.x, i = tid % P4, sg = tid / P4;
-                const int ns = min(pos / TILE + 1, G.smax);
-                const unsigned Xo = (unsigned)l * G.stride;
-                float M = -INFINITY, den = 0.f;
-                f4 num = {0.f, 0.f, 0.f, 0.f};
-                constexpr int MBG = 4;
-                for (int s1 = sg; s1 < ns; s1 += SG * MBG) {
-                    f4 a[MBG];
-                    float ms[MBG], ls[MBG];
-                    long long t0w = 0;
-                    bool timing = false;
-                    for (;;) {
-                        unsigned missing = 0;
-#pragma unroll
-                        for (int j = 0; j < MBG; j++) {
-                            const int sj = min(s1 + j * SG, ns - 1);
-                            a[j] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (Xo + G.offPacc + (unsigned)sj * dim + h * HD + i * 4) * 4u, 0, 16));
-                            ms[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, (Xo + G.offPm + sj * p.nHeads + h) * 4u, 0, 16));
-                            ls[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, (Xo + G.offPl + sj * p.nHeads + h) * 4u, 0, 16));
-                        }
-#pragma unroll
-                        for (int j = 0; j < MBG; j++) missing |= unset4(a[j]) | unset1(ms[j]) | unset1(ls[j]);
-                        if (!missing || wt.dead) break;
-                        if (!timing) { timing = true; t0w = wall_clock64(); }
-                        else if (wall_clock64() - t0w > wt.limit) { wt.fail(); break; }
-                        for (int z = 0; z < 4; z++) __builtin_amdgcn_s_sleep(2);
-                    }
-#pragma unroll
-                    for (int j = 0; j < MBG; j++) {
-                        if (s1 + j * SG < ns) {
-                            const float Mn = fmaxf(M, ms[j]);
-                            const float c = exp_neg(M - Mn), wgt = exp_neg(ms[j] - Mn);
-                            den = den * c + wgt * ls[j];
-                            num.x = num.x * c + wgt * a[j].x; num.y = num.y * c + wgt * a[j].y;
-                            num.z = num.z * c + wgt * a[j].z; num.w = num.w * c + wgt * a[j].w;
-                            M = Mn;
-                        }
-                    }
-                }
-                mnum[sg][i] = tof4(num); mM[sg][i] = M; mden[sg][i] = den;
-                __syncthreads();
-                if (tid < P4) {
-                    float Mg = mM[0][tid];
-                    for (int g2 = 1; g2 < SG; g2++) Mg = fmaxf(Mg, mM[g2][tid]);
-                    float dn = 0.f;
-                    f4 nm = {0.f, 0.f, 0.f, 0.f};
-                    for (int g2 = 0; g2 < SG; g2++) {
-                        const float wgt = exp_neg(mM[g2][tid] - Mg);     // a group without splits has M = -inf: weight 0
-                        const float4 a = mnum[g2][tid];
-                        dn = fmaf(wgt, mden[g2][tid], dn);
-                        nm.x = fmaf(wgt, a.x, nm.x); nm.y = fmaf(wgt, a.y, nm.y); nm.z = fmaf(wgt, a.z, nm.z); nm.w = fmaf(wgt, a.w, nm.w);
-                    }
-                    const float il = __builtin_amdgcn_rcpf(dn);
-                    stx4(reinterpret_cast<f4*>(X + G.offAttn + h * HD) + tid, f4{nm.x * il, nm.y * il, nm.z * il, nm.w * il});
-                }
-            }
-        }
-        FLOW_TRACE(4);
-        // ------------------------------------------------------------------ Wo + residual
-        {
-            const int nI = dim;
-            if (blockIdx.x * FWAVES < nI) {
-                int it = gw;
-                int4 wr[1][CBD];
-                WRow rows[1] = {wrow<Q4>(L.wo, L.so, 0, dim)};
-                float e0 = 0.f, e1 = 0.f;
-                auto resolve = [&](int item) {
-                    rows[0] = wrow<Q4>(L.wo, L.so, item, dim);
-                    ld_row<GL, Q4, CBD>(rows[0], nchD, lane, 0, wr[0]);
-                    if (lane == 0) {
-                        e0 = Q4 ? 1.f : ldg_f<GL>(L.so, item);
-                        e1 = first ? xin[item] : poll1(xin + item, wt);         // there already if this workgroup staged it for q | k | v
-                    }
-                };
-                if (it < nI) resolve(it);
-                // stage the attention output: merge the KV splits' partials (running maximum, as the split-KV combine)
-                if (grouped) {
-                    stage_plain<Q4, !RING>(X + G.offAttn, dim, a4, wt);      // merged per head above
-                } else {
-                __syncthreads();
+                FLOW_TRACE(2);
+                // ------------------------------------------------------------------ attention: one (head, KV split) per workgroup
+                // grouped only while a workgroup per query head and split would not fit the launch (positions far into a long context)
+                const bool grouped = GQA && p.nHeads * (pos / TILE + 1) > nC;
                 {
                     const int nsplit = pos / TILE + 1;
-                    const int ns = nsplit < G.smax ? nsplit : G.smax;
-                    for (int i = tid; i < (dim >> 2); i += FWG) {
-                        const int h = (i * 4) / HD;
+                    // Grouped: the query heads of a KV head are shared out over as many workgroups as the launch has left for
+                    // them at this position (each loads the K / V rows once and takes its heads in turn), so a workgroup takes as
+                    // few heads as possible: qhMax heads a workgroup, `sub` workgroups a KV head and split.
+                    const int Gq = p.nHeads / p.nKVHeads;
+                    int qhMax = 1, sub = Gq;
+                    if (grouped) {
+                        qhMax = Gq; sub = 1;
+                        const int live = nsplit < G.smax ? nsplit : G.smax;
+                        for (int q = 2; q < Gq; q++) {
+                            const int sb = (Gq + q - 1) / q;
+                            if (p.nKVHeads * sb * live <= nC) { qhMax = q; sub = sb; break; }
+                        }
+                    }
+                    const int unit = grouped ? p.nKVHeads * sub : p.nHeads;
+                    const int split = blockIdx.x / unit, hu = blockIdx.x % unit;
+                    const int hg = grouped ? hu % sub : 0;                         // which of the KV head's groups of query heads
+                    const int QH = grouped ? min(qhMax, Gq - hg * qhMax) : 1;      // query heads of this workgroup
+                    // Workgroups with no attention to do (and no partials to merge per head) read, into their XCD's L2, rows that the
+                    // XCD's workgroups will want after it -- their next poll, for the attention's partials, is microseconds away, and
+                    // HBM would be idle meanwhile.  p.idleWoRows: Wo (rows of more than 2048 weights, of which a wave requests only
+                    // the first half-row ahead); p.idleGateUpRows: the leading rows of gate and of up -- all of them where both
+                    // matrices fit the L2s (1.1B shape: 0.465 -> 0.436 ms a token; the down projection on top overflows the L2s:
+                    // 0.470), else half of the first round of rows, which is what a phase waits for before it streams (8B shape
+                    // with both: 1.845 -> 1.790; the whole first round 1.804, a quarter 1.800).
+                    // Only while at least half the launch is idle (short contexts), and only without dedicated prefetchers.
+                    if ((p.idleWoRows > 0 || p.idleGateUpRows > 0) && nC == (int)gridDim.x) {
+                        const int live = nsplit < G.smax ? nsplit : G.smax;
+                        int nBusy = unit * live;
+                        if (grouped && nBusy < p.nHeads) nBusy = p.nHeads;
+                        nBusy = (nBusy + 7) & ~7;
+                        if ((int)blockIdx.x >= nBusy && 2 * ((int)gridDim.x - nBusy) >= (int)gridDim.x) {
+                            Prefetcher pf{(int)blockIdx.x & 7, ((int)blockIdx.x - nBusy) >> 3, ((int)gridDim.x - nBusy) >> 3, tid, pfScrap};
+                            const size_t rbD = Q4 ? dim >> 1 : dim, rdD = dim >> 4;
+                            // (a workgroup without q | k | v rows gets here at the top of the layer; holding it back until q | k | v is
+                            // through measures slower: 1.1B shape 0.453 against 0.435 ms a token)
+                            if (p.idleWoRows > 0) {
+                                pf.rows(L.wo, rbD, p.idleWoRows, 8);
+                                if (Q4) pf.rows(L.so, rdD, p.idleWoRows, 8);
+                            }
+                            if (p.idleGateUpRows > 0) {
+                                pf.rows(L.gate, rbD, p.idleGateUpRows, 8);
+                                pf.rows(L.up, rbD, p.idleGateUpRows, 8);
+                                if (Q4) { pf.rows(L.sgate, rdD, p.idleGateUpRows, 8); pf.rows(L.sup, rdD, p.idleGateUpRows, 8); }
+                            }
+                            pf.drain();
+                        }
+                    }
+                    if (split < G.smax && split < nsplit) {
+                        const int kvh = grouped ? hu / sub : hu / Gq;
+                        const int h0 = grouped ? kvh * Gq + hg * qhMax : hu;
+                        const int tg = tid / LPR, dl = tid % LPR;
+                        const int t0 = split * TILE;
+                        const int len = pos + 1;
+                        const int t1 = min(len, t0 + TILE);
+                        const size_t rowStride = (size_t)kvDim / 4;
+                        const size_t colOff = (size_t)(kvh * HD) / 4 + dl;
+                        const float4* Kc4 = reinterpret_cast<const float4*>(L.Kc);
+                        const float4* Vc4 = reinterpret_cast<const float4*>(L.Vc);
+                        float4 kreg[VU][NF], vreg[VU][NF];
+                        // Only rows of earlier positions are read from the caches (the current one comes through the exchange
+                        // area, the loads of later ones go to the idle line): a cache line is never fetched into an L2 before its
+                        // row has been written -- in token mode that row is written later in this same launch, by a workgroup of
+                        // another XCD, and a line fetched early would be served stale from then on.
+                        const float4* idle4 = reinterpret_cast<const float4*>(wt.idle) + dl;
+#pragma unroll
+                        for (int u = 0; u < VU; u++) {
+                            const int row = t0 + tg + u * TG;
+                            const size_t ro = (size_t)row * rowStride + colOff;
+                            const float4* kp = row < pos ? Kc4 + ro : idle4;
+                            const float4* vp = row < pos ? Vc4 + ro : idle4;
+#pragma unroll
+                            for (int j = 0; j < NF; j++) kreg[u][j] = ldg_f4<GL>(kp, j * 16);
+#pragma unroll
+                            for (int j = 0; j < NF; j++) vreg[u][j] = ldg_f4<GL>(vp, j * 16);
+                        }
+                        __syncthreads();
+                        if (tid < (2 + QH) * (HD / 4)) {
+                            const int which = tid / (HD / 4), i = tid % (HD / 4);
+                            const float* src = which >= 2 ? X + G.offQ + (h0 + which - 2) * HD : X + (which == 0 ? G.offKc : G.offVc) + kvh * HD;
+                            sqkv[which][i] = tof4(poll4(reinterpret_cast<const f4*>(src) + i, wt));
+                        }
+                        __syncthreads();
+                        FLOW_TRACE(3);
+                        const int live = t1 - t0;
+                        const float scale = 1.0f / sqrtf((float)HD);
+#pragma unroll
+                        for (int u = 0; u < VU; u++) {
+                            if (t0 + tg + u * TG == pos) {          // the current position's rows come from this launch, not from the cache
+#pragma unroll
+                                for (int j = 0; j < NF; j++) { kreg[u][j] = sqkv[0][j * 16 + dl]; vreg[u][j] = sqkv[1][j * 16 + dl]; }
+                            }
+                        }
+                        for (int hi = 0; hi < QH; hi++) {          // the heads of the KV head in turn, on the same K / V registers
+                        float4 q4[NF];
+#pragma unroll
+                        for (int j = 0; j < NF; j++) q4[j] = sqkv[2 + hi][j * 16 + dl];
+                        float sc[VU];
+                        float tmax = -INFINITY;
+#pragma unroll
+                        for (int u = 0; u < VU; u++) {
+                            sc[u] = -INFINITY;
+                            if (u * TG >= live) continue;
+                            const int row = t0 + tg + u * TG;
+                            float d = 0.f;
+#pragma unroll
+                            for (int j = 0; j < NF; j++) {
+                                d = fmaf(q4[j].x, kreg[u][j].x, d); d = fmaf(q4[j].y, kreg[u][j].y, d);
+                                d = fmaf(q4[j].z, kreg[u][j].z, d); d = fmaf(q4[j].w, kreg[u][j].w, d);
+                            }
+                            d = row_sum16(d);
+                            sc[u] = row < t1 ? d * scale : -INFINITY;
+                            tmax = fmaxf(tmax, sc[u]);
+                        }
+                        const float m = tg_max(tmax);               // the wave's maximum
+                        const float mRef = m == -INFINITY ? 0.f : m;
+                        float4 acc[NF];
+#pragma unroll
+                        for (int j = 0; j < NF; j++) acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                        float lsum = 0.f;
+#pragma unroll
+                        for (int u = 0; u < VU; u++) {
+                            if (u * TG >= live) continue;
+                            const float pv = exp_neg(sc[u] - mRef);
+                            lsum += pv;
+#pragma unroll
+                            for (int j = 0; j < NF; j++) {
+                                acc[j].x = fmaf(pv, vreg[u][j].x, acc[j].x); acc[j].y = fmaf(pv, vreg[u][j].y, acc[j].y);
+                                acc[j].z = fmaf(pv, vreg[u][j].z, acc[j].z); acc[j].w = fmaf(pv, vreg[u][j].w, acc[j].w);
+                            }
+                        }
+#pragma unroll
+                        for (int j = 0; j < NF; j++) {
+                            acc[j].x = tg_sum(acc[j].x); acc[j].y = tg_sum(acc[j].y); acc[j].z = tg_sum(acc[j].z); acc[j].w = tg_sum(acc[j].w);
+                            if (lane < LPR) accbuf[hi][wave][j * 16 + dl] = acc[j];
+                        }
+                        lsum = tg_sum(lsum);
+                        if (lane == 0) { lbuf[hi][wave] = lsum; wred[hi][wave] = m; }
+                        }
+                        // the waves' partials of all the workgroup's heads combined together: one barrier, a thread per head and piece
+                        __syncthreads();
+                        if (tid < QH * (HD / 4)) {
+                            const int hq = tid / (HD / 4), i = tid % (HD / 4), h = h0 + hq;
+                            float mg_ = wred[hq][0];
+#pragma unroll
+                            for (int k = 1; k < FWAVES; k++) mg_ = fmaxf(mg_, wred[hq][k]);
+                            f4 r = {0.f, 0.f, 0.f, 0.f};
+                            float lg = 0.f;
+#pragma unroll
+                            for (int k = 0; k < FWAVES; k++) {
+                                const float wk = exp_neg(wred[hq][k] - mg_);
+                                const float4 a = accbuf[hq][k][i];
+                                r.x = fmaf(wk, a.x, r.x); r.y = fmaf(wk, a.y, r.y); r.z = fmaf(wk, a.z, r.z); r.w = fmaf(wk, a.w, r.w);
+                                lg = fmaf(wk, lbuf[hq][k], lg);
+                            }
+                            stx4(reinterpret_cast<f4*>(X + G.offPacc + (size_t)split * dim + h * HD) + i, r);
+                            if (i == 0) {
+                                stx(X + G.offPm + split * p.nHeads + h, mg_);
+                                stx(X + G.offPl + split * p.nHeads + h, lg);
+                            }
+                        }
+                    }
+                }
+
+                if (grouped) {
+                    // Long contexts, tens of KV splits: merged once per head, by workgroup h for head h (every thread a 16-byte piece
+                    // and every eighth split, eight splits' loads in flight together, then combined through LDS), and handed on as
+                    // one vector -- every consumer merging all partials itself re-reads tens of KB per workgroup and layer.
+                    if ((int)blockIdx.x < p.nHeads) {
+                        constexpr int P4 = HD / 4, SG = FWG / P4;          // pieces of a head, split groups (thread = piece x group)
+                        __shared__ float4 mnum[SG][P4];
+                        __shared__ float mM[SG][P4], mden[SG][P4];
+                        const int h = blockIdx.x, i = tid % P4, sg = tid / P4;
+                        const int ns = min(pos / TILE + 1, G.smax);
+                        const unsigned Xo = xoff + (unsigned)l * G.stride;
                         float M = -INFINITY, den = 0.f;
                         f4 num = {0.f, 0.f, 0.f, 0.f};
-                        auto mergeIn = [&](f4 a, float ms, float ls) {
-                            const float Mn = fmaxf(M, ms);
-                            const float c = exp_neg(M - Mn);                        // first split: exp(-inf) = 0
-                            const float wgt = exp_neg(ms - Mn);
-                            den = den * c + wgt * ls;
-                            num.x = num.x * c + wgt * a.x; num.y = num.y * c + wgt * a.y;
-                            num.z = num.z * c + wgt * a.z; num.w = num.w * c + wgt * a.w;
-                            M = Mn;
+                        constexpr int MBG = 4;
+                        for (int s1 = sg; s1 < ns; s1 += SG * MBG) {
+                            f4 a[MBG];
+                            float ms[MBG], ls[MBG];
+                            long long t0w = 0;
+                            bool timing = false;
+                            for (;;) {
+                                unsigned missing = 0;
+#pragma unroll
+                                for (int j = 0; j < MBG; j++) {
+                                    const int sj = min(s1 + j * SG, ns - 1);
+                                    a[j] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (Xo + G.offPacc + (unsigned)sj * dim + h * HD + i * 4) * 4u, 0, 16));
+                                    ms[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, (Xo + G.offPm + sj * p.nHeads + h) * 4u, 0, 16));
+                                    ls[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, (Xo + G.offPl + sj * p.nHeads + h) * 4u, 0, 16));
+                                }
+#pragma unroll
+                                for (int j = 0; j < MBG; j++) missing |= unset4(a[j]) | unset1(ms[j]) | unset1(ls[j]);
+                                if (!missing || wt.dead) break;
+                                if (!timing) { timing = true; t0w = wall_clock64(); }
+                                else if (wall_clock64() - t0w > wt.limit) { wt.fail(); break; }
+                                for (int z = 0; z < 4; z++) __builtin_amdgcn_s_sleep(2);
+                            }
+#pragma unroll
+                            for (int j = 0; j < MBG; j++) {
+                                if (s1 + j * SG < ns) {
+                                    const float Mn = fmaxf(M, ms[j]);
+                                    const float c = exp_neg(M - Mn), wgt = exp_neg(ms[j] - Mn);
+                                    den = den * c + wgt * ls[j];
+                                    num.x = num.x * c + wgt * a[j].x; num.y = num.y * c + wgt * a[j].y;
+                                    num.z = num.z * c + wgt * a[j].z; num.w = num.w * c + wgt * a[j].w;
+                                    M = Mn;
+                                }
+                            }
+                        }
+                        mnum[sg][i] = tof4(num); mM[sg][i] = M; mden[sg][i] = den;
+                        __syncthreads();
+                        if (tid < P4) {
+                            float Mg = mM[0][tid];
+                            for (int g2 = 1; g2 < SG; g2++) Mg = fmaxf(Mg, mM[g2][tid]);
+                            float dn = 0.f;
+                            f4 nm = {0.f, 0.f, 0.f, 0.f};
+                            for (int g2 = 0; g2 < SG; g2++) {
+                                const float wgt = exp_neg(mM[g2][tid] - Mg);     // a group without splits has M = -inf: weight 0
+                                const float4 a = mnum[g2][tid];
+                                dn = fmaf(wgt, mden[g2][tid], dn);
+                                nm.x = fmaf(wgt, a.x, nm.x); nm.y = fmaf(wgt, a.y, nm.y); nm.z = fmaf(wgt, a.z, nm.z); nm.w = fmaf(wgt, a.w, nm.w);
+                            }
+                            const float il = __builtin_amdgcn_rcpf(dn);
+                            stx4(reinterpret_cast<f4*>(X + G.offAttn + h * HD) + tid, f4{nm.x * il, nm.y * il, nm.z * il, nm.w * il});
+                        }
+                    }
+                }
+                FLOW_TRACE(4);
+                // ------------------------------------------------------------------ Wo + residual
+                {
+                    const int nI = dim;
+                    if (blockIdx.x * FWAVES < nI) {
+                        int it = gw;
+                        int4 wr[1][CBD];
+                        WRow rows[1] = {wrow<Q4>(L.wo, L.so, 0, dim)};
+                        float e0 = 0.f, e1 = 0.f;
+                        auto resolve = [&](int item) {
+                            rows[0] = wrow<Q4>(L.wo, L.so, item, dim);
+                            ld_row<GL, Q4, CBD>(rows[0], nchD, lane, 0, wr[0]);
+                            if (lane == 0) {
+                                e0 = Q4 ? 1.f : ldg_f<GL>(L.so, item);
+                                e1 = first ? xin[item] : poll1(xin + item, wt);         // there already if this workgroup staged it for q | k | v
+                            }
                         };
-                        for (int s = 0; s < ns; s++) {
-                            f4 a;
-                            float ms, ls;
-                            const f4* pa = reinterpret_cast<const f4*>(X + G.offPacc + (size_t)s * dim) + i;
-                            // The split everybody has to wait for is waited for on the accumulator pieces alone: they are
-                            // spread over many lines, while the maxima and sums of all heads share one, and a line that
-                            // 50,000 threads keep re-reading takes its producer's store late.
-                            if (s == 0) a = poll4(pa, wt);
-                            poll_partial(pa, X + G.offPm + s * p.nHeads + h, X + G.offPl + s * p.nHeads + h, a, ms, ls, wt);
-                            mergeIn(a, ms, ls);
-                        }
-                        const float il = __builtin_amdgcn_rcpf(den);
-                        a4[slot4<Q4>(i, nchD)] = make_float4(num.x * il, num.y * il, num.z * il, num.w * il);
-                    }
-                }
-                __syncthreads();
-                }
-                FLOW_TRACE(5);
-                for (; it < nI; it += W) {
-                    if (it != gw) resolve(it);
-                    float acc[1] = {0.f};
-                    dot_rows<Q4, 1, CBD>(wr, a4, nchD, lane, 0, acc);
-                    if (nchD > CBD * 64) dot_rows_tail<GL, Q4, 1, CBD>(rows, a4, nchD, lane, acc);
-                    const float v = wave_sum(acc[0]);
-                    if (it != gw) __syncthreads();              // outbuf is free again
-                    store_runs(e1 + v * e0, 1, nI, it - gw, X + G.offX1, nullptr);
-                }
-            }
-        }
-
-        FLOW_TRACE(6);
-        // ------------------------------------------------------------------ gate | up, SiLU(g) * u
-        {
-            const int nI = ffn;
-            if constexpr (RING) {
-                // Long rows, several items a wave: the rows stream through a ring of register sets, the loads of step
-                // s + RD - 1 are issued before step s is multiplied (a step = one item's two rows x CB chunks a lane).
-                if (blockIdx.x * FWAVES < nI) {
-                    constexpr int RD = 3, CB = 2;
-                    int4 ring[RD][2][CB];
-                    const int nItems = gw < nI ? (nI - gw + W - 1) / W : 0;
-                    const int nb = (nchD + 64 * CB - 1) / (64 * CB);
-                    const int T = nItems * nb;
-                    auto issueStep = [&](int4 (&set)[2][CB], int st) {
-                        const int sc = min(st, T - 1);                       // past the end: the last step again (uniform loop)
-                        const int k = sc / nb, b = sc - k * nb;
-                        const int row = gw + k * W;
-                        ld_row<GL, Q4, CB>(wrow<Q4>(L.gate, L.sgate, row, dim), nchD, lane, b * CB * 64, set[0]);
-                        ld_row<GL, Q4, CB>(wrow<Q4>(L.up, L.sup, row, dim), nchD, lane, b * CB * 64, set[1]);
-                    };
-                    float sg = 0.f, su = 0.f;
-                    if (T > 0) {
-#pragma unroll
-                        for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
-                        if (lane < nItems) { const int r = gw + lane * W; sg = Q4 ? 1.f : ldg_f<GL>(L.sgate, r); su = Q4 ? 1.f : ldg_f<GL>(L.sup, r); }
-                    }
-                    const float rs = stage_rms<GL, Q4, !RING>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
-                    FLOW_TRACE(7);
-                    float acc[2] = {0.f, 0.f};
-                    float g = 0.f, u = 0.f;
-                    for (int s0 = 0; s0 < T; s0 += RD) {
-#pragma unroll
-                        for (int j = 0; j < RD; j++) {
-                            const int st = s0 + j;
-                            issueStep(ring[(j + RD - 1) % RD], st + RD - 1);
-                            if (st < T) {                                        // uniform in the wave
-                                const int k = st / nb, b = st - k * nb;
-                                dot_rows<Q4, 2, CB>(ring[j], a4, nchD, lane, b * CB * 64, acc);
-                                if (b == nb - 1) {
-                                    const float t = wave_sum2(acc[0], acc[1]);
-                                    const float v0 = lane_value(t, 0), v1 = lane_value(t, 32);
-                                    if (lane == k) { g = v0; u = v1; }
-                                    acc[0] = 0.f; acc[1] = 0.f;
+                        if (it < nI) resolve(it);
+                        // stage the attention output: merge the KV splits' partials (running maximum, as the split-KV combine)
+                        if (grouped) {
+                            stage_plain<Q4, !RING>(X + G.offAttn, dim, a4, wt);      // merged per head above
+                        } else {
+                        __syncthreads();
+                        {
+                            const int nsplit = pos / TILE + 1;
+                            const int ns = nsplit < G.smax ? nsplit : G.smax;
+                            for (int i = tid; i < (dim >> 2); i += FWG) {
+                                const int h = (i * 4) / HD;
+                                float M = -INFINITY, den = 0.f;
+                                f4 num = {0.f, 0.f, 0.f, 0.f};
+                                auto mergeIn = [&](f4 a, float ms, float ls) {
+                                    const float Mn = fmaxf(M, ms);
+                                    const float c = exp_neg(M - Mn);                        // first split: exp(-inf) = 0
+                                    const float wgt = exp_neg(ms - Mn);
+                                    den = den * c + wgt * ls;
+                                    num.x = num.x * c + wgt * a.x; num.y = num.y * c + wgt * a.y;
+                                    num.z = num.z * c + wgt * a.z; num.w = num.w * c + wgt * a.w;
+                                    M = Mn;
+                                };
+                                for (int s = 0; s < ns; s++) {
+                                    f4 a;
+                                    float ms, ls;
+                                    const f4* pa = reinterpret_cast<const f4*>(X + G.offPacc + (size_t)s * dim) + i;
+                                    // The split everybody has to wait for is waited for on the accumulator pieces alone: they are
+                                    // spread over many lines, while the maxima and sums of all heads share one, and a line that
+                                    // 50,000 threads keep re-reading takes its producer's store late.
+                                    if (s == 0) a = poll4(pa, wt);
+                                    poll_partial(pa, X + G.offPm + s * p.nHeads + h, X + G.offPl + s * p.nHeads + h, a, ms, ls, wt);
+                                    mergeIn(a, ms, ls);
                                 }
+                                const float il = __builtin_amdgcn_rcpf(den);
+                                a4[slot4<Q4>(i, nchD)] = make_float4(num.x * il, num.y * il, num.z * il, num.w * il);
                             }
                         }
-                    }
-                    g = g * sg; g = g * rs;
-                    u = u * su; u = u * rs;
-                    const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f));   // mongoose.cu:949-956
-                    store_runs(g * sig * u, (nI + W - 1) / W, nI, 0, X + G.offM, nullptr);
-                }
-            } else
-            if (blockIdx.x * FWAVES < nI) {
-                int4 wr[NIB][2][CBD];
-                float sg = 0.f, su = 0.f;
-                auto issue = [&](int it0) {
-#pragma unroll
-                    for (int k = 0; k < NIB; k++) {
-                        const int r = it0 + k * W;
-                        if (r < nI) {                                           // uniform in the wave
-                            ld_row<GL, Q4, CBD>(wrow<Q4>(L.gate, L.sgate, r, dim), nchD, lane, 0, wr[k][0]);
-                            ld_row<GL, Q4, CBD>(wrow<Q4>(L.up, L.sup, r, dim), nchD, lane, 0, wr[k][1]);
+                        __syncthreads();
+                        }
+                        FLOW_TRACE(5);
+                        for (; it < nI; it += W) {
+                            if (it != gw) resolve(it);
+                            float acc[1] = {0.f};
+                            dot_rows<Q4, 1, CBD>(wr, a4, nchD, lane, 0, acc);
+                            if (nchD > CBD * 64) dot_rows_tail<GL, Q4, 1, CBD>(rows, a4, nchD, lane, acc);
+                            const float v = wave_sum(acc[0]);
+                            if (it != gw) __syncthreads();              // outbuf is free again
+                            store_runs(e1 + v * e0, 1, nI, it - gw, X + G.offX1, nullptr);
                         }
                     }
-                    if (lane < NIB) { const int r = min(it0 + lane * W, nI - 1); sg = Q4 ? 1.f : ldg_f<GL>(L.sgate, r); su = Q4 ? 1.f : ldg_f<GL>(L.sup, r); }
-                };
-                if (gw < nI) issue(gw);
-                const float rs = stage_rms<GL, Q4, !RING>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
-                FLOW_TRACE(7);
-                for (int it0 = gw; it0 < nI; it0 += NIB * W) {
-                    if (it0 != gw) issue(it0);
-                    float g = 0.f, u = 0.f;
+                }
+
+                FLOW_TRACE(6);
+                // ------------------------------------------------------------------ gate | up, SiLU(g) * u
+                {
+                    const int nI = ffn;
+                    if constexpr (RING) {
+                        // Long rows, several items a wave: the rows stream through a ring of register sets, the loads of step
+                        // s + RD - 1 are issued before step s is multiplied (a step = one item's two rows x CB chunks a lane).
+                        if (blockIdx.x * FWAVES < nI) {
+                            constexpr int RD = 3, CB = 2;
+                            int4 ring[RD][2][CB];
+                            const int nItems = gw < nI ? (nI - gw + W - 1) / W : 0;
+                            const int nb = (nchD + 64 * CB - 1) / (64 * CB);
+                            const int T = nItems * nb;
+                            auto issueStep = [&](int4 (&set)[2][CB], int st) {
+                                const int sc = min(st, T - 1);                       // past the end: the last step again (uniform loop)
+                                const int k = sc / nb, b = sc - k * nb;
+                                const int row = gw + k * W;
+                                ld_row<GL, Q4, CB>(wrow<Q4>(L.gate, L.sgate, row, dim), nchD, lane, b * CB * 64, set[0]);
+                                ld_row<GL, Q4, CB>(wrow<Q4>(L.up, L.sup, row, dim), nchD, lane, b * CB * 64, set[1]);
+                            };
+                            float sg = 0.f, su = 0.f;
+                            if (T > 0) {
 #pragma unroll
-                    for (int k = 0; k < NIB; k++) {
-                        float acc[2] = {0.f, 0.f};
-                        if (it0 + k * W < nI) {                                 // uniform in the wave
-                            dot_rows<Q4, 2, CBD>(wr[k], a4, nchD, lane, 0, acc);
-                            if (nchD > CBD * 64) {
+                                for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
+                                if (lane < nItems) { const int r = gw + lane * W; sg = Q4 ? 1.f : ldg_f<GL>(L.sgate, r); su = Q4 ? 1.f : ldg_f<GL>(L.sup, r); }
+                            }
+                            const float rs = stage_rms<GL, Q4, !RING>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                            FLOW_TRACE(7);
+                            float acc[2] = {0.f, 0.f};
+                            float g = 0.f, u = 0.f;
+                            for (int s0 = 0; s0 < T; s0 += RD) {
+#pragma unroll
+                                for (int j = 0; j < RD; j++) {
+                                    const int st = s0 + j;
+                                    issueStep(ring[(j + RD - 1) % RD], st + RD - 1);
+                                    if (st < T) {                                        // uniform in the wave
+                                        const int k = st / nb, b = st - k * nb;
+                                        dot_rows<Q4, 2, CB>(ring[j], a4, nchD, lane, b * CB * 64, acc);
+                                        if (b == nb - 1) {
+                                            const float t = wave_sum2(acc[0], acc[1]);
+                                            const float v0 = lane_value(t, 0), v1 = lane_value(t, 32);
+                                            if (lane == k) { g = v0; u = v1; }
+                                            acc[0] = 0.f; acc[1] = 0.f;
+                                        }
+                                    }
+                                }
+                            }
+                            g = g * sg; g = g * rs;
+                            u = u * su; u = u * rs;
+                            const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f));   // mongoose.cu:949-956
+                            store_runs(g * sig * u, (nI + W - 1) / W, nI, 0, X + G.offM, nullptr);
+                        }
+                    } else
+                    if (blockIdx.x * FWAVES < nI) {
+                        int4 wr[NIB][2][CBD];
+                        float sg = 0.f, su = 0.f;
+                        auto issue = [&](int it0) {
+#pragma unroll
+                            for (int k = 0; k < NIB; k++) {
                                 const int r = it0 + k * W;
-                                const WRow rows[2] = {wrow<Q4>(L.gate, L.sgate, r, dim), wrow<Q4>(L.up, L.sup, r, dim)};
-                                dot_rows_tail<GL, Q4, 2, CBD>(rows, a4, nchD, lane, acc);
+                                if (r < nI) {                                           // uniform in the wave
+                                    ld_row<GL, Q4, CBD>(wrow<Q4>(L.gate, L.sgate, r, dim), nchD, lane, 0, wr[k][0]);
+                                    ld_row<GL, Q4, CBD>(wrow<Q4>(L.up, L.sup, r, dim), nchD, lane, 0, wr[k][1]);
+                                }
                             }
-                            const float t = wave_sum2(acc[0], acc[1]);
-                            acc[0] = lane_value(t, 0);
-                            acc[1] = lane_value(t, 32);
+                            if (lane < NIB) { const int r = min(it0 + lane * W, nI - 1); sg = Q4 ? 1.f : ldg_f<GL>(L.sgate, r); su = Q4 ? 1.f : ldg_f<GL>(L.sup, r); }
+                        };
+                        if (gw < nI) issue(gw);
+                        const float rs = stage_rms<GL, Q4, !RING>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                        FLOW_TRACE(7);
+                        for (int it0 = gw; it0 < nI; it0 += NIB * W) {
+                            if (it0 != gw) issue(it0);
+                            float g = 0.f, u = 0.f;
+#pragma unroll
+                            for (int k = 0; k < NIB; k++) {
+                                float acc[2] = {0.f, 0.f};
+                                if (it0 + k * W < nI) {                                 // uniform in the wave
+                                    dot_rows<Q4, 2, CBD>(wr[k], a4, nchD, lane, 0, acc);
+                                    if (nchD > CBD * 64) {
+                                        const int r = it0 + k * W;
+                                        const WRow rows[2] = {wrow<Q4>(L.gate, L.sgate, r, dim), wrow<Q4>(L.up, L.sup, r, dim)};
+                                        dot_rows_tail<GL, Q4, 2, CBD>(rows, a4, nchD, lane, acc);
+                                    }
+                                    const float t = wave_sum2(acc[0], acc[1]);
+                                    acc[0] = lane_value(t, 0);
+                                    acc[1] = lane_value(t, 32);
+                                }
+                                if (lane == k) { g = acc[0]; u = acc[1]; }
+                            }
+                            g = g * sg; g = g * rs;
+                            u = u * su; u = u * rs;
+                            const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f));   // mongoose.cu:949-956
+                            if (it0 != gw) __syncthreads();             // outbuf is free again
+                            store_runs(g * sig * u, NIB, nI, it0 - gw, X + G.offM, nullptr);
                         }
-                        if (lane == k) { g = acc[0]; u = acc[1]; }
                     }
-                    g = g * sg; g = g * rs;
-                    u = u * su; u = u * rs;
-                    const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f));   // mongoose.cu:949-956
-                    if (it0 != gw) __syncthreads();             // outbuf is free again
-                    store_runs(g * sig * u, NIB, nI, it0 - gw, X + G.offM, nullptr);
                 }
-            }
-        }
 
-        FLOW_TRACE(8);
-        // ------------------------------------------------------------------ down + residual
-        {
-            const int nI = dim;
-            if constexpr (RING) {
-                if (blockIdx.x * FWAVES < nI) {
-                    constexpr int RD = 3, CB = 4;
-                    int4 ring[RD][1][CB];
-                    const int nItems = gw < nI ? (nI - gw + W - 1) / W : 0;
-                    const int nb = (nchF + 64 * CB - 1) / (64 * CB);
-                    const int T = nItems * nb;
-                    auto issueStep = [&](int4 (&set)[1][CB], int st) {
-                        const int sc = min(st, T - 1);
-                        const int k = sc / nb, b = sc - k * nb;
-                        ld_row<GL, Q4, CB>(wrow<Q4>(L.down, L.sdown, gw + k * W, ffn), nchF, lane, b * CB * 64, set[0]);
-                    };
-                    float e0 = 0.f, e1 = 0.f;
-                    if (T > 0) {
-                        if (lane < nItems) { const int r = gw + lane * W; e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r); e1 = poll1(X + G.offX1 + r, wt); }
+                FLOW_TRACE(8);
+                // ------------------------------------------------------------------ down + residual
+                {
+                    const int nI = dim;
+                    if constexpr (RING) {
+                        if (blockIdx.x * FWAVES < nI) {
+                            constexpr int RD = 3, CB = 4;
+                            int4 ring[RD][1][CB];
+                            const int nItems = gw < nI ? (nI - gw + W - 1) / W : 0;
+                            const int nb = (nchF + 64 * CB - 1) / (64 * CB);
+                            const int T = nItems * nb;
+                            auto issueStep = [&](int4 (&set)[1][CB], int st) {
+                                const int sc = min(st, T - 1);
+                                const int k = sc / nb, b = sc - k * nb;
+                                ld_row<GL, Q4, CB>(wrow<Q4>(L.down, L.sdown, gw + k * W, ffn), nchF, lane, b * CB * 64, set[0]);
+                            };
+                            float e0 = 0.f, e1 = 0.f;
+                            if (T > 0) {
+                                if (lane < nItems) { const int r = gw + lane * W; e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r); e1 = poll1(X + G.offX1 + r, wt); }
 #pragma unroll
-                        for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
-                    }
-                    stage_plain_w<Q4>(X + G.offM, ffn, a4, wt);
-                    FLOW_TRACE(9);
-                    float acc[1] = {0.f};
-                    float v = 0.f;
-                    for (int s0 = 0; s0 < T; s0 += RD) {
+                                for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
+                            }
+                            stage_plain_w<Q4>(X + G.offM, ffn, a4, wt);
+                            FLOW_TRACE(9);
+                            float acc[1] = {0.f};
+                            float v = 0.f;
+                            for (int s0 = 0; s0 < T; s0 += RD) {
 #pragma unroll
-                        for (int j = 0; j < RD; j++) {
-                            const int st = s0 + j;
-                            issueStep(ring[(j + RD - 1) % RD], st + RD - 1);
-                            if (st < T) {                                        // uniform in the wave
-                                const int k = st / nb, b = st - k * nb;
-                                dot_rows<Q4, 1, CB>(ring[j], a4, nchF, lane, b * CB * 64, acc);
-                                if (b == nb - 1) {
-                                    const float v0 = wave_sum(acc[0]);
-                                    if (lane == k) v = v0;
-                                    acc[0] = 0.f;
+                                for (int j = 0; j < RD; j++) {
+                                    const int st = s0 + j;
+                                    issueStep(ring[(j + RD - 1) % RD], st + RD - 1);
+                                    if (st < T) {                                        // uniform in the wave
+                                        const int k = st / nb, b = st - k * nb;
+                                        dot_rows<Q4, 1, CB>(ring[j], a4, nchF, lane, b * CB * 64, acc);
+                                        if (b == nb - 1) {
+                                            const float v0 = wave_sum(acc[0]);
+                                            if (lane == k) v = v0;
+                                            acc[0] = 0.f;
+                                        }
+                                    }
+                                }
+                            }
+                            store_runs(e1 + v * e0, (nI + W - 1) / W, nI, 0, X + G.offX2, l == p.l1 - 1 ? p.hidden : nullptr);
+                        }
+                    } else if (p.downSplit) {
+                        // Few rows (at most half as many as computing waves): a row is shared by two neighbouring waves of a
+                        // workgroup, each taking half of its chunks, and every workgroup with rows has half as many -- the
+                        // multiplications of this phase, its longest rows, take half as long (0.5B shape 0.366 -> 0.360 ms a
+                        // token).  One round.
+                        if ((int)blockIdx.x * (FWAVES / 2) < nI) {
+                            constexpr int CBH = CBF / 2;
+                            const int row = min(gw >> 1, nI - 1), hf = wave & 1;
+                            const int nHalf = (nchF + 1) >> 1;
+                            const int c0 = hf ? nHalf : 0, cHi = hf ? nchF : nHalf;
+                            const WRow rw = wrow<Q4>(L.down, L.sdown, row, ffn);
+                            int4 wr[CBH];
+                            ld_row_rng<GL, Q4, CBH>(rw, cHi, lane, c0, wr);
+                            float e0 = 0.f, e1 = 0.f;
+                            if (wave == 0 && lane < FWAVES / 2) {
+                                const int r = min((int)blockIdx.x * (FWAVES / 2) + lane, nI - 1);
+                                e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r);
+                                e1 = poll1(X + G.offX1 + r, wt);
+                            }
+                            stage_plain<Q4, false>(X + G.offM, ffn, a4, wt);
+                            FLOW_TRACE(9);
+                            float acc = dot_row_rng<Q4, CBH>(wr, a4, nchF, cHi, lane, c0, 0.f);
+                            for (int cc = c0 + CBH * 64; cc < cHi; cc += CBH * 64) {
+                                ld_row_rng<GL, Q4, CBH>(rw, cHi, lane, cc, wr);
+                                acc = dot_row_rng<Q4, CBH>(wr, a4, nchF, cHi, lane, cc, acc);
+                            }
+                            acc = wave_sum(acc);
+                            if (lane == 0) outbuf[0][wave] = acc;
+                            __syncthreads();
+                            if (wave == 0 && lane < FWAVES / 2) {
+                                const int r = (int)blockIdx.x * (FWAVES / 2) + lane;
+                                if (r < nI) {
+                                    const float o = e1 + (outbuf[0][2 * lane] + outbuf[0][2 * lane + 1]) * e0;
+                                    stx(X + G.offX2 + r, o);
+                                    if (l == p.l1 - 1) p.hidden[r] = o;
                                 }
                             }
                         }
-                    }
-                    store_runs(e1 + v * e0, (nI + W - 1) / W, nI, 0, X + G.offX2, l == p.l1 - 1 ? p.hidden : nullptr);
-                }
-            } else if (p.downSplit) {
-                // Few rows (at most half as many as computing waves): a row is shared by two neighbouring waves of a
-                // workgroup, each taking half of its chunks, and every workgroup with rows has half as many -- the
-                // multiplications of this phase, its longest rows, take half as long (0.5B shape 0.366 -> 0.360 ms a
-                // token).  One round.
-                if ((int)blockIdx.x * (FWAVES / 2) < nI) {
-                    constexpr int CBH = CBF / 2;
-                    const int row = min(gw >> 1, nI - 1), hf = wave & 1;
-                    const int nHalf = (nchF + 1) >> 1;
-                    const int c0 = hf ? nHalf : 0, cHi = hf ? nchF : nHalf;
-                    const WRow rw = wrow<Q4>(L.down, L.sdown, row, ffn);
-                    int4 wr[CBH];
-                    ld_row_rng<GL, Q4, CBH>(rw, cHi, lane, c0, wr);
-                    float e0 = 0.f, e1 = 0.f;
-                    if (wave == 0 && lane < FWAVES / 2) {
-                        const int r = min((int)blockIdx.x * (FWAVES / 2) + lane, nI - 1);
-                        e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r);
-                        e1 = poll1(X + G.offX1 + r, wt);
-                    }
-                    stage_plain<Q4, false>(X + G.offM, ffn, a4, wt);
-                    FLOW_TRACE(9);
-                    float acc = dot_row_rng<Q4, CBH>(wr, a4, nchF, cHi, lane, c0, 0.f);
-                    for (int cc = c0 + CBH * 64; cc < cHi; cc += CBH * 64) {
-                        ld_row_rng<GL, Q4, CBH>(rw, cHi, lane, cc, wr);
-                        acc = dot_row_rng<Q4, CBH>(wr, a4, nchF, cHi, lane, cc, acc);
-                    }
-                    acc = wave_sum(acc);
-                    if (lane == 0) outbuf[0][wave] = acc;
-                    __syncthreads();
-                    if (wave == 0 && lane < FWAVES / 2) {
-                        const int r = (int)blockIdx.x * (FWAVES / 2) + lane;
-                        if (r < nI) {
-                            const float o = e1 + (outbuf[0][2 * lane] + outbuf[0][2 * lane + 1]) * e0;
-                            stx(X + G.offX2 + r, o);
-                            if (l == p.l1 - 1) p.hidden[r] = o;
-                        }
-                    }
-                }
-            } else
-            if (blockIdx.x * FWAVES < nI) {
-                int4 wr[NID][1][CBF];
-                float e0 = 0.f, e1 = 0.f;
-                auto issue = [&](int it0) {
+                    } else
+                    if (blockIdx.x * FWAVES < nI) {
+                        int4 wr[NID][1][CBF];
+                        float e0 = 0.f, e1 = 0.f;
+                        auto issue = [&](int it0) {
 #pragma unroll
-                    for (int k = 0; k < NID; k++) {
-                        const int r = it0 + k * W;
-                        if (r < nI) ld_row<GL, Q4, CBF>(wrow<Q4>(L.down, L.sdown, r, ffn), nchF, lane, 0, wr[k][0]);      // uniform in the wave
-                    }
-                    if (lane < NID) { const int r = min(it0 + lane * W, nI - 1); e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r); e1 = poll1(X + G.offX1 + r, wt); }
-                };
-                if (gw < nI) issue(gw);
-                stage_plain<Q4, false>(X + G.offM, ffn, a4, wt);
-                FLOW_TRACE(9);
-                for (int it0 = gw; it0 < nI; it0 += NID * W) {
-                    if (it0 != gw) issue(it0);
-                    float v = 0.f;
-#pragma unroll
-                    for (int k = 0; k < NID; k++) {
-                        float acc[1] = {0.f};
-                        if (it0 + k * W < nI) {
-                            dot_rows<Q4, 1, CBF>(wr[k], a4, nchF, lane, 0, acc);
-                            if (nchF > CBF * 64) {
-                                const WRow rows[1] = {wrow<Q4>(L.down, L.sdown, it0 + k * W, ffn)};
-                                dot_rows_tail<GL, Q4, 1, CBF>(rows, a4, nchF, lane, acc);
+                            for (int k = 0; k < NID; k++) {
+                                const int r = it0 + k * W;
+                                if (r < nI) ld_row<GL, Q4, CBF>(wrow<Q4>(L.down, L.sdown, r, ffn), nchF, lane, 0, wr[k][0]);      // uniform in the wave
                             }
-                            acc[0] = wave_sum(acc[0]);
+                            if (lane < NID) { const int r = min(it0 + lane * W, nI - 1); e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r); e1 = poll1(X + G.offX1 + r, wt); }
+                        };
+                        if (gw < nI) issue(gw);
+                        stage_plain<Q4, false>(X + G.offM, ffn, a4, wt);
+                        FLOW_TRACE(9);
+                        for (int it0 = gw; it0 < nI; it0 += NID * W) {
+                            if (it0 != gw) issue(it0);
+                            float v = 0.f;
+#pragma unroll
+                            for (int k = 0; k < NID; k++) {
+                                float acc[1] = {0.f};
+                                if (it0 + k * W < nI) {
+                                    dot_rows<Q4, 1, CBF>(wr[k], a4, nchF, lane, 0, acc);
+                                    if (nchF > CBF * 64) {
+                                        const WRow rows[1] = {wrow<Q4>(L.down, L.sdown, it0 + k * W, ffn)};
+                                        dot_rows_tail<GL, Q4, 1, CBF>(rows, a4, nchF, lane, acc);
+                                    }
+                                    acc[0] = wave_sum(acc[0]);
+                                }
+                                if (lane == k) v = acc[0];
+                            }
+                            if (it0 != gw) __syncthreads();             // outbuf is free again
+                            store_runs(e1 + v * e0, NID, nI, it0 - gw, X + G.offX2, l == p.l1 - 1 ? p.hidden : nullptr);
                         }
-                        if (lane == k) v = acc[0];
                     }
-                    if (it0 != gw) __syncthreads();             // outbuf is free again
-                    store_runs(e1 + v * e0, NID, nI, it0 - gw, X + G.offX2, l == p.l1 - 1 ? p.hidden : nullptr);
                 }
+                FLOW_TRACE(10);
             }
         }
-        FLOW_TRACE(10);
+
+        if (tokens) {
+            // ---------------------------------------------------------------------------------------------- the tail
+            // All workgroups of the launch, the prefetching ones included.  Rows of the lm_head in items of NRT, item g to
+            // wave g % WA; a wave's items stream through a ring of register sets as gate | up's do.
+            const int l = p.l1;                             // (trace: the tail is recorded as one more layer)
+            FLOW_TRACE(0);
+            const int np = pos + 1;
+            const int gwA = blockIdx.x * FWAVES + wave, WA = (int)gridDim.x * FWAVES;
+            const signed char* lmW = TW_PTR(const signed char, lmW);
+            const float* lmAux = TW_PTR(const float, lmAux);
+            const int vocab = TW_INT(vocab);
+            float* logits = TW_PTR(float, logits);
+            float* amax = TW_PTR(float, amax);
+            constexpr int NRT = (RING || CBD > 1) ? 2 : 4, CBT = RING ? 2 : CBD, RDT = 3;
+            int4 ring[RDT][NRT][CBT];
+            float scl[RDT];
+            const int nItemsAll = (vocab + NRT - 1) / NRT;
+            float bestV = -INFINITY;
+            int bestI = INT_MAX;
+            float acc[NRT];
+#pragma unroll
+            for (int i = 0; i < NRT; i++) acc[i] = 0.f;
+            // an item's NRT sums -> logits and the lane's running best; lane i < NRT ends up with row r0 + i
+            auto finishItem = [&](int r0, float sc, float rs) {
+                float val;
+                if constexpr (NRT == 4) {
+                    const float t01 = wave_sum2(acc[0], acc[1]), t23 = wave_sum2(acc[2], acc[3]);
+                    val = lane_value(t01, 0);
+                    if (lane == 1) val = lane_value(t01, 32);
+                    if (lane == 2) val = lane_value(t23, 0);
+                    if (lane == 3) val = lane_value(t23, 32);
+                } else {
+                    const float t01 = wave_sum2(acc[0], acc[1]);
+                    val = lane_value(t01, 0);
+                    if (lane == 1) val = lane_value(t01, 32);
+                }
+                val = val * sc;
+                val = val * rs;
+                const int r = r0 + lane;
+                if (lane < NRT && r < vocab) {
+                    stg_f<true>(logits, (size_t)r, val);
+                    if (val > bestV || (val == bestV && r < bestI)) { bestV = val; bestI = r; }
+                }
+#pragma unroll
+                for (int i = 0; i < NRT; i++) acc[i] = 0.f;
+            };
+            auto resetOther = [&]() {
+                // the other half of the exchange area, and this workgroup's argmax slot there, for the token after this one
+                const f4 sent = {__builtin_bit_cast(float, XSENT), __builtin_bit_cast(float, XSENT), __builtin_bit_cast(float, XSENT), __builtin_bit_cast(float, XSENT)};
+                f4* o4 = reinterpret_cast<f4*>(p.xchg + (size_t)(np & 1) * halfFloats);
+                for (size_t i = (size_t)blockIdx.x * FWG + tid; i < halfFloats / 4; i += (size_t)gridDim.x * FWG)
+                    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(o4 + i), "v"(sent) : "memory");
+                if (tid == 0) {
+                    st_agent(amax + ((size_t)(np & 1) * gridDim.x + blockIdx.x) * FLOW_AMAX_STRIDE, sent.x);
+                    st_agent(amax + ((size_t)(np & 1) * gridDim.x + blockIdx.x) * FLOW_AMAX_STRIDE + 1, sent.x);
+                }
+            };
+            const float* xfin = xb + (size_t)(p.l1 - 1) * G.stride + G.offX2;
+            // A wave's items (item g to wave g % WA) stream through the ring in steps, as gate | up's rows do.  (Handing the
+            // items of a workgroup out to its waves as they fall free, from a counter in LDS, was measured: the waves of a
+            // workgroup then end together, but the launch ends when its slowest workgroup does, 2-3 us after the mean, as
+            // before -- 0.3511 against 0.3475 ms a token at the 0.5B shape.)
+            const int nItems = gwA < nItemsAll ? (nItemsAll - gwA + WA - 1) / WA : 0;
+            const int nb = (nchD + 64 * CBT - 1) / (64 * CBT);
+            const int Tn = nItems * nb;
+            auto issueStep = [&](int4 (&set)[NRT][CBT], float& sc, int st) {
+                const int s2 = min(st, Tn - 1);                      // past the end: the last step again (uniform loop)
+                const int k = s2 / nb, b = s2 - k * nb;
+                const int r0 = (gwA + k * WA) * NRT;
+#pragma unroll
+                for (int i = 0; i < NRT; i++)
+                    ld_row<GL, Q4, CBT>(wrow<Q4>(lmW, lmAux, min(r0 + i, vocab - 1), dim), nchD, lane, b * CBT * 64, set[i]);
+                sc = Q4 ? 1.f : ldg_f<GL>(lmAux, min(r0 + (lane < NRT ? lane : 0), vocab - 1));
+            };
+            if (Tn > 0) {
+#pragma unroll
+                for (int j = 0; j < RDT - 1; j++) issueStep(ring[j], scl[j], j);
+            }
+            resetOther();
+            const float rs = stage_rms<GL, Q4, !RING>(xfin, true, TW_PTR(const float, finalGain), dim, p.eps, a4, red, wt);
+            FLOW_TRACE(1);
+            for (int s0 = 0; s0 < Tn; s0 += RDT) {
+#pragma unroll
+                for (int j = 0; j < RDT; j++) {
+                    const int st = s0 + j;
+                    issueStep(ring[(j + RDT - 1) % RDT], scl[(j + RDT - 1) % RDT], st + RDT - 1);
+                    if (st < Tn) {                                       // uniform in the wave
+                        const int k = st / nb, b = st - k * nb;
+                        dot_rows<Q4, NRT, CBT>(ring[j], a4, nchD, lane, b * CBT * 64, acc);
+                        if (b == nb - 1) finishItem((gwA + k * WA) * NRT, scl[j], rs);
+                    }
+                }
+            }
+            FLOW_TRACE(2);
+            // argmax exchange: the workgroup's best (value, lowest index) goes out once its own stores (the reset above among
+            // them) have been acknowledged; then every workgroup reads all of them and picks the token for itself
+            wave_argmax(bestV, bestI);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (lane == 0) { tailV[wave] = bestV; tailI[wave] = bestI; }
+            __syncthreads();
+            FLOW_TRACE(4);
+            {
+                float v = tailV[0];
+                int ix = tailI[0];
+#pragma unroll
+                for (int k = 1; k < FWAVES; k++) argmax_pick(v, ix, tailV[k], tailI[k]);
+                if (tid == 0) {
+                    float* slot = amax + ((size_t)(pos & 1) * gridDim.x + blockIdx.x) * FLOW_AMAX_STRIDE;
+                    store_arg(slot, v, ix);
+                }
+            }
+            float pv = -INFINITY;
+            int pix = INT_MAX;
+            for (int i = tid; i < (int)gridDim.x; i += FWG) {
+                const ArgPart pr = poll_arg(amax + ((size_t)(pos & 1) * gridDim.x + i) * FLOW_AMAX_STRIDE, wt);
+                argmax_pick(pv, pix, pr.v, pr.i);
+            }
+            FLOW_TRACE(5);
+            wave_argmax(pv, pix);
+            __syncthreads();                                 // every thread has read the waves' bests above
+            if (lane == 0) { tailV[wave] = pv; tailI[wave] = pix; }
+            __syncthreads();
+            float tv = tailV[0];
+            int ti = tailI[0];
+#pragma unroll
+            for (int k = 1; k < FWAVES; k++) argmax_pick(tv, ti, tailV[k], tailI[k]);
+            if (ti < 0 || ti >= vocab) ti = 0;               // (a wait ran out: whatever it is, it stays a token)
+            FLOW_TRACE(3);
+            const int* prompt = TW_PTR(const int, prompt);
+            if (blockIdx.x == 0 && tid == 0) {
+                int* history = TW_PTR(int, history);
+                if (history && count0 + tk < TW_INT(historyCap)) history[count0 + tk] = ti;
+            }
+            tok = (prompt && np < nPrompt) ? prompt[np] : ti;
+            pos = np;
+        }
+    }   // tokens of the launch
+    if (tokens && blockIdx.x == 0) {
+        // the device state and the RoPE row of the next position, as the separate launches' last kernel leaves them
+        StepState* stw = TW_PTR(StepState, state);
+        float* rc = TW_PTR(float, ropeCur);
+        const int pr = pos < p.maxSeq ? pos : p.maxSeq - 1;
+        if (rc) {
+            for (int j = tid; j < half; j += FWG) {
+                rc[j] = TW_PTR(const float, cosTab)[(size_t)pr * half + j];
+                rc[half + j] = TW_PTR(const float, sinTab)[(size_t)pr * half + j];
+            }
+        }
+        if (tid == 0) { stw->pos = pos; stw->token = tok; stw->count = count0 + nTok; }
     }
 }
 
@@ -1309,7 +1539,10 @@ hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
         !flow_context_fits(p.maxSeq, p.geo) || !p.layers || !p.xchg || !p.err || !p.hidden ||
         !flow_grid_fits(p.ffn, p.nHeads, p.geo, nC) || (size_t)p.nLayersTotal * p.geo.stride * 4 >= (1ull << 31))
         return hipErrorInvalidValue;
-    const size_t lds = (size_t)(p.dim > p.ffn ? p.dim : p.ffn) * sizeof(float);
+    if (p.nTokens > 0 && (!p.tail || !p.state || p.l0 != 0 || p.l1 != p.nLayersTotal || p.nTokens > p.maxSeq ||
+                          flow_lds_bytes(p.dim, p.ffn, p.headDim, p.geo.gqa, true) > ((size_t)160 << 10)))
+        return hipErrorInvalidValue;
+    const size_t lds = (size_t)((p.dim > p.ffn ? p.dim : p.ffn) + (p.nTokens > 0 ? p.dim : 0)) * sizeof(float);
     const bool wide = p.dim > 1024, ring = p.dim > 2048, gqa = p.geo.gqa != 0;
 #define FLOW_LAUNCH(HDv, CBv, RGv, GQv, Q4v) hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v>), dim3(grid), dim3(FWG), lds, s, p)
 #define FLOW_LAUNCH_G(HDv, CBv, RGv) do { \
@@ -1341,6 +1574,21 @@ hipError_t launch_flow_reset(float* xchg, const FlowGeometry& g, int l0, int l1,
     hipLaunchKernelGGL(flow_reset_kernel, dim3((unsigned)blocks), dim3(WG), 0, s,
                        reinterpret_cast<uint4*>(xchg + (size_t)l0 * g.stride), n4);
     return hipGetLastError();
+}
+
+size_t flow_xchg_floats(const FlowGeometry& g, int nLayers, int grid) {
+    return (size_t)2 * nLayers * g.stride + (size_t)2 * grid * FLOW_AMAX_STRIDE;
+}
+hipError_t launch_flow_reset_all(float* xchg, const FlowGeometry& g, int nLayers, int grid, hipStream_t s) {
+    const size_t n4 = flow_xchg_floats(g, nLayers, grid) / 4;
+    size_t blocks = (n4 + WG - 1) / WG;
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(flow_reset_kernel, dim3((unsigned)blocks), dim3(WG), 0, s, reinterpret_cast<uint4*>(xchg), n4);
+    return hipGetLastError();
+}
+size_t flow_lds_bytes(int dim, int ffn, int headDim, int gqa, bool tokenMode) {
+    const size_t own = headDim == 64 ? (gqa ? (34u << 10) : (5u << 10)) : (gqa ? (53u << 10) : (8u << 10));
+    return own + (size_t)((dim > ffn ? dim : ffn) + (tokenMode ? dim : 0)) * sizeof(float);
 }
 
 }  // namespace mg

@@ -179,6 +179,15 @@ public:
     bool FlowInUse() const { return flowEligible(0, nLayers); }
     long long flowLimitTicks = 5000000;       // per wait of the persistent launch: 50 ms of the 100 MHz wall clock
     void SetFlowWaitLimit(long long ticks) { invalidateGraphs(); flowLimitTicks = ticks; }
+    // Whole tokens inside the persistent launch (embedding, layers, final norm, lm_head, argmax): on where the model
+    // allows it; tokensPerLaunch of them in one launch where a caller asks for a run of tokens (Generate, TimedDecode,
+    // GeneratePrefill), 1 = a launch (or a graph replay) per token.
+    bool flowTail = true;
+    int tokensPerLaunch = 64;
+    void SetFlowTail(int on) { invalidateGraphs(); flowTail = on != 0; }
+    int SetTokensPerLaunch(int n);
+    bool FlowTailInUse() const { return flowTailEligible(); }
+    int FlowTailTrace(long long* out, size_t cap, int* dims);
 private:
     FlowLayer* dFlowLayers = nullptr;
     int* dFlowErr = nullptr;
@@ -188,11 +197,17 @@ private:
     bool flowTableDirty = true;
     bool flowBroken = false;        // a wait ran into its limit once: the separate launches are used from then on
     bool flowEligible(int l0, int l1) const;
+    bool flowTailEligible() const;
+    FlowTail* dFlowTail = nullptr;
+    int enqueueTokensFlow(int nTokens);
+    int decodeRun(int nTokens, bool useGraph);      // nTokens decode steps from the device state
+    bool runsInLaunch(bool useGraph) const;         // ... as runs of tokens inside the persistent launch
+    int setState(int pos, int token, int count, int nPrompt);
     int flowComputeWgs(int cus) const;
     bool q4ActQuant = false;      // exec mode 0: Q4_0 matrices through the int8-activation matvecs
     void* q8Scratch = nullptr;    // (max(dim, ffnDim)/32)*40 bytes of activation blocks (cuda_fused_infer.go:175-179)
     int ensureFlow();
-    int enqueueLayersFlow(int l0, int l1, const StepState* st, int posImm, bool resetFirst);
+    int enqueueLayersFlow(int l0, int l1, const StepState* st, int posImm, bool resetFirst, int nTokens = 0);
     int checkFlowError();
     int enqueueToken(bool withHead);      // embed -> layers -> final(+argmax) / advance, all from device state
 

@@ -208,6 +208,7 @@ HIPFusedInference::~HIPFusedInference() {
     if (q8Scratch) (void)hipFree(q8Scratch);
     if (dFlowLayers) (void)hipFree(dFlowLayers);
     if (flowXchg) (void)hipFree(flowXchg);
+    if (dFlowTail) (void)hipFree(dFlowTail);
     if (dFlowErr) (void)hipFree(dFlowErr);
     if (hFlowErr) (void)hipHostFree(hFlowErr);
     if (hState) (void)hipHostFree(hState);
@@ -680,6 +681,7 @@ void HIPFusedInference::flowRegeometry() {
     if (stream) (void)hipStreamSynchronize(stream);
     (void)hipFree(dFlowLayers); dFlowLayers = nullptr;
     if (flowXchg) { (void)hipFree(flowXchg); flowXchg = nullptr; }
+    if (dFlowTail) { (void)hipFree(dFlowTail); dFlowTail = nullptr; }
     if (dFlowErr) { (void)hipFree(dFlowErr); dFlowErr = nullptr; }
     if (hFlowErr) { (void)hipHostFree(hFlowErr); hFlowErr = nullptr; }
     if (flowTrace) { (void)hipFree(flowTrace); flowTrace = nullptr; }
@@ -745,8 +747,11 @@ int HIPFusedInference::ensureFlow() {
         void* v = nullptr;
         HIPCHK(hipMalloc(&v, sizeof(FlowLayer) * (size_t)nLayers));
         dFlowLayers = static_cast<FlowLayer*>(v);
-        HIPCHK(hipMalloc(&v, sizeof(float) * (size_t)nLayers * flowGeo.stride));
+        HIPCHK(hipMalloc(&v, sizeof(float) * flow_xchg_floats(flowGeo, nLayers, flowGrid)));
         flowXchg = static_cast<float*>(v);
+        HIPCHK(launch_flow_reset_all(flowXchg, flowGeo, nLayers, flowGrid, stream));
+        HIPCHK(hipMalloc(&v, sizeof(FlowTail)));
+        dFlowTail = static_cast<FlowTail*>(v);
         HIPCHK(hipMalloc(&v, FLOW_ERR_BYTES));
         dFlowErr = static_cast<int*>(v);
         HIPCHK(hipMemsetAsync(dFlowErr, 0, FLOW_ERR_BYTES, stream));
@@ -774,8 +779,25 @@ int HIPFusedInference::ensureFlow() {
             F.bq = L.bq; F.bk = L.bk; F.bv = L.bv;
             F.Kc = kCache[l]; F.Vc = vCache[l];
         }
+        FlowTail T{};
+        if (finalNorm && lmHead.w) {
+            T.finalGain = finalNorm;
+            T.lmW = static_cast<const signed char*>(lmHead.w);
+            T.lmAux = lmHead.kind == WF_Q4P
+                          ? reinterpret_cast<const float*>(static_cast<const char*>(lmHead.w) + (size_t)lmHead.rows * (lmHead.cols >> 1))
+                          : lmHead.scales;
+            T.logits = logits;
+            if (embedKind == 1 || embedKind == 2) { T.embKind = embedKind; T.embTable = embedTable; }
+            else { T.embKind = lmHead.kind == WF_Q8 ? 0 : 3; T.embTable = lmHead.w; T.embScales = lmHead.scales; }
+            T.cosTab = cosTab; T.sinTab = sinTab;
+            T.state = dState; T.history = dHistory; T.historyCap = maxSeq + 1; T.prompt = dPrompt;
+            T.amax = flow_amax_area(flowXchg, flowGeo, nLayers);
+            T.ropeCur = ropeCur;
+            T.vocab = vocabSize;
+        }
         HIPCHK(hipStreamSynchronize(stream));
         HIPCHK(hipMemcpy(dFlowLayers, t.data(), sizeof(FlowLayer) * (size_t)nLayers, hipMemcpyHostToDevice));
+        HIPCHK(hipMemcpy(dFlowTail, &T, sizeof(FlowTail), hipMemcpyHostToDevice));
         flowTableDirty = false;
     }
     return MG_OK;
@@ -787,14 +809,15 @@ int HIPFusedInference::ensureFlow() {
 int HIPFusedInference::FlowTrace(int enable, long long* out, size_t cap, int* dims) {
     if (!flowEligible(0, nLayers)) { set_error("flow trace: the persistent launch is not in use for this model (exec mode, weight kinds, shape)"); return MG_E_STATE; }
     if (int rc = ensureFlow()) return rc;
-    const size_t n = (size_t)nLayers * FLOW_TRACE_SLOTS * (size_t)flowCompute;
+    // one more block than layers: the tail of a token (FlowTailTrace)
+    const size_t n = (size_t)nLayers * FLOW_TRACE_SLOTS * (size_t)flowCompute, nAll = (size_t)(nLayers + 1) * FLOW_TRACE_SLOTS * (size_t)flowCompute;
     HIPCHK(hipStreamSynchronize(stream));
     if (dims) { dims[0] = nLayers; dims[1] = FLOW_TRACE_SLOTS; dims[2] = flowCompute; }
     if (enable && !flowTrace) {
         void* v = nullptr;
-        HIPCHK(hipMalloc(&v, sizeof(long long) * n));
+        HIPCHK(hipMalloc(&v, sizeof(long long) * nAll));
         flowTrace = static_cast<long long*>(v);
-        HIPCHK(hipMemsetAsync(v, 0, sizeof(long long) * n, stream));
+        HIPCHK(hipMemsetAsync(v, 0, sizeof(long long) * nAll, stream));
         HIPCHK(hipStreamSynchronize(stream));
         invalidateGraphs();
     }
@@ -810,7 +833,20 @@ int HIPFusedInference::FlowTrace(int enable, long long* out, size_t cap, int* di
     return MG_OK;
 }
 
-int HIPFusedInference::enqueueLayersFlow(int l0, int l1, const StepState* st, int posImm, bool resetFirst) {
+// The tail's part of the trace (FLOW_TAIL_TRACE_NAMES: six points) of the last token a launch ran, while the trace is
+// enabled: ticks [point][workgroup]; dims gets {4, workgroups}.
+int HIPFusedInference::FlowTailTrace(long long* out, size_t cap, int* dims) {
+    if (!flowTrace || !flowTailEligible()) { set_error("flow tail trace: enable the trace first (and the launch must run whole tokens)"); return MG_E_STATE; }
+    const size_t n = (size_t)6 * flowCompute;
+    if (dims) { dims[0] = 6; dims[1] = flowCompute; }
+    if (!out) return MG_OK;
+    if (cap < n) { set_error("flow tail trace: buffer too small"); return MG_E_ARG; }
+    HIPCHK(hipStreamSynchronize(stream));
+    HIPCHK(hipMemcpy(out, flowTrace + (size_t)nLayers * FLOW_TRACE_SLOTS * (size_t)flowCompute, sizeof(long long) * n, hipMemcpyDeviceToHost));
+    return MG_OK;
+}
+
+int HIPFusedInference::enqueueLayersFlow(int l0, int l1, const StepState* st, int posImm, bool resetFirst, int nTokens) {
     if (l1 > nLayers) l1 = nLayers;
     FlowParams p{};
     p.layers = dFlowLayers; p.l0 = l0; p.l1 = l1; p.nLayersTotal = nLayers;
@@ -840,9 +876,64 @@ int HIPFusedInference::enqueueLayersFlow(int l0, int l1, const StepState* st, in
     p.err = dFlowErr;
     p.limitTicks = flowLimitTicks;
     p.trace = flowTrace;
+    if (nTokens > 0) { p.nTokens = nTokens; p.tail = dFlowTail; }
     if (resetFirst) HIPCHK(launch_flow_reset(flowXchg, flowGeo, l0, l1, stream));
     if (mark(1)) return MG_E_HIP;
     HIPCHK(launch_flow_layers(p, flowGrid, stream));
+    return MG_OK;
+}
+
+// nTokens whole tokens from the device state in one launch: embedding, layers, final norm, lm_head, argmax; the
+// exchange area must be in its reset state for the first token's position (setState), the launch leaves it so for
+// the position after its last.
+int HIPFusedInference::enqueueTokensFlow(int nTokens) {
+    return enqueueLayersFlow(0, nLayers, dState, 0, false, nTokens);
+}
+
+// Whole tokens in the launch need: the tail's operands set, the lm_head in the layers' format, room in LDS for the
+// embedding beside the staged vector.
+bool HIPFusedInference::flowTailEligible() const {
+    if (!flowTail || !flowEligible(0, nLayers)) return false;
+    if (!finalNorm || !lmHead.w || lmHead.kind != layers[0].wq.kind || lmHead.cols != dim || lmHead.rows != vocabSize) return false;
+    if (lmHead.kind == WF_Q4P && dim % 32) return false;
+    const FlowGeometry g = flowGrid ? flowGeo : flow_geometry(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim, maxSeq, 8);
+    const int gqa = flowGrid ? flowGeo.gqa : 1;        // before the launch is set up: the larger bound
+    (void)g;
+    return flow_lds_bytes(dim, ffnDim, headDim, gqa, true) <= ((size_t)160 << 10);
+}
+
+int HIPFusedInference::SetTokensPerLaunch(int n) {
+    if (n < 1 || n > 4096) { set_error("tokens per launch must be between 1 and 4096"); return MG_E_ARG; }
+    tokensPerLaunch = n;
+    return MG_OK;
+}
+
+// Sets the device-resident step state; where the persistent launch runs whole tokens, also leaves its exchange area
+// reset (a token expects the half of its position's parity so, and resets the other for its successor).
+int HIPFusedInference::setState(int pos, int token, int count, int nPrompt) {
+    HIPCHK(launch_set_state(dState, pos, token, count, nPrompt, ropeRef(), stream));
+    if (flowXchg && (execMode == 3 || execMode == 4)) HIPCHK(launch_flow_reset_all(flowXchg, flowGeo, nLayers, flowGrid, stream));
+    return MG_OK;
+}
+
+// nTokens decode steps from the device state: runs of tokens inside the persistent launch where that is in use, else
+// graph replays or eager launches of single tokens.
+bool HIPFusedInference::runsInLaunch(bool useGraph) const { return useGraph && tokensPerLaunch > 1 && flowTailEligible(); }
+
+int HIPFusedInference::decodeRun(int nTokens, bool useGraph) {
+    if (runsInLaunch(useGraph)) {
+        int rc = ensureFlow();
+        for (int done = 0; done < nTokens && rc == MG_OK;) {
+            const int n = std::min(tokensPerLaunch, nTokens - done);
+            rc = enqueueTokensFlow(n);
+            done += n;
+        }
+        return rc;
+    }
+    for (int i = 0; i < nTokens; i++) {
+        if (useGraph) HIPCHK(hipGraphLaunch(execFull, stream));
+        else { int rc = enqueueToken(true); if (rc) return rc; }
+    }
     return MG_OK;
 }
 
@@ -1074,14 +1165,15 @@ EmbedRef HIPFusedInference::embedRef() const {
     return e;
 }
 int HIPFusedInference::primeGraph() {
-    int rc = enqueueEmbed();
-    if (rc) return rc;
-    // a captured token leaves the exchange area reset for its successor; the first one finds it so here
-    if (graphsUseFlow) HIPCHK(launch_flow_reset(flowXchg, flowGeo, 0, nLayers, stream));
-    return MG_OK;
+    // (a captured token leaves the exchange area reset for its successor; the first one finds it so from setState)
+    return enqueueEmbed();
 }
 
 int HIPFusedInference::enqueueToken(bool withHead) {
+    if (withHead && flowTailEligible()) {          // the whole token is one launch
+        int rc = ensureFlow();
+        return rc ? rc : enqueueTokensFlow(1);
+    }
     int rc = fuseEmbed ? MG_OK : enqueueEmbed();
     if (rc) return rc;
     const bool flow = flowEligible(0, nLayers);
@@ -1097,7 +1189,9 @@ int HIPFusedInference::enqueueToken(bool withHead) {
     }
     if (withHead) return enqueueFinal(true);
     HIPCHK(launch_advance_prompt(dState, dPrompt, ropeRef(), embedRef(), stream));
-    if (flow && fuseEmbed) HIPCHK(launch_flow_reset(flowXchg, flowGeo, 0, nLayers, stream));    // captured prompt step: no lm_head launch to do it
+    // no lm_head launch to leave the exchange area reset for the next launch: a captured prompt step does it itself,
+    // and so does any prompt step where whole tokens run in the launch (they expect to find it so)
+    if (flow && (fuseEmbed || flowTailEligible())) HIPCHK(launch_flow_reset(flowXchg, flowGeo, 0, nLayers, stream));
     return MG_OK;
 }
 
@@ -1115,7 +1209,7 @@ int HIPFusedInference::DecodeToken(int token, int pos, int* nextToken, float* lo
     ARGCHK(pos >= 0 && pos < maxSeq && token >= 0 && token < vocabSize, "DecodeToken: token or pos out of range");
     int rc = checkReady(this);
     if (rc) return rc;
-    HIPCHK(launch_set_state(dState, pos, token, 0, 0, ropeRef(), stream));
+    { int rcs = setState(pos, token, 0, 0); if (rcs) return rcs; }
     if (execMode == 0) {
         rc = enqueueEmbed();
         if (rc) return rc;
@@ -1251,7 +1345,7 @@ int HIPFusedInference::GraphLaunch(int token, int pos, int* nextToken) {
     ARGCHK(pos >= 0 && pos < maxSeq && token >= 0 && token < vocabSize, "GraphLaunch: token or pos out of range");
     int rc = GraphCapture();
     if (rc) return rc;
-    HIPCHK(launch_set_state(dState, pos, token, 0, 0, ropeRef(), stream));
+    { int rcs = setState(pos, token, 0, 0); if (rcs) return rcs; }
     rc = primeGraph();
     if (rc) return rc;
     HIPCHK(hipGraphLaunch(execFull, stream));
@@ -1299,19 +1393,19 @@ int HIPFusedInference::Generate(const int* prompt, int nPrompt, int nDecode, int
         }
         return MG_OK;
     }
-    if (useGraph) { rc = GraphCapture(); if (rc) return rc; }
+    // (where runs of tokens go into one launch no graph is needed: the prompt steps are launched one by one)
+    const bool graphs = useGraph && !runsInLaunch(useGraph);
+    if (graphs) { rc = GraphCapture(); if (rc) return rc; }
     HIPCHK(hipStreamSynchronize(stream));
     HIPCHK(hipMemcpy(dPrompt, prompt, sizeof(int) * (size_t)nPrompt, hipMemcpyHostToDevice));
-    HIPCHK(launch_set_state(dState, 0, prompt[0], 0, nPrompt, ropeRef(), stream));
-    if (useGraph) { rc = primeGraph(); if (rc) return rc; }
+    { int rcs = setState(0, prompt[0], 0, nPrompt); if (rcs) return rcs; }
+    if (graphs) { rc = primeGraph(); if (rc) return rc; }
     for (int i = 0; i < nPrompt - 1; i++) {
-        if (useGraph) HIPCHK(hipGraphLaunch(execPrompt, stream));
+        if (graphs) HIPCHK(hipGraphLaunch(execPrompt, stream));
         else { rc = enqueueToken(false); if (rc) return rc; }
     }
-    for (int i = 0; i < nDecode; i++) {
-        if (useGraph) HIPCHK(hipGraphLaunch(execFull, stream));
-        else { rc = enqueueToken(true); if (rc) return rc; }
-    }
+    rc = decodeRun(nDecode, useGraph);
+    if (rc) return rc;
     if (nDecode > 0) HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int) * (size_t)nDecode, hipMemcpyDeviceToHost, stream));
     HIPCHK(hipStreamSynchronize(stream));
     for (int i = 0; i < nDecode; i++) outTokens[i] = hTokens[i];
@@ -1323,15 +1417,15 @@ int HIPFusedInference::TimedDecode(int token, int pos, int steps, bool useGraph,
     ARGCHK(steps >= 1 && pos >= 0 && pos + steps <= maxSeq && token >= 0 && token < vocabSize, "TimedDecode: bad arguments");
     int rc = checkReady(this);
     if (rc) return rc;
-    if (useGraph) { rc = GraphCapture(); if (rc) return rc; }
-    HIPCHK(launch_set_state(dState, pos, token, 0, 0, ropeRef(), stream));
-    if (useGraph) { rc = primeGraph(); if (rc) return rc; }
+    const bool graphs = useGraph && !runsInLaunch(useGraph);
+    if (graphs) { rc = GraphCapture(); if (rc) return rc; }
+    if (runsInLaunch(useGraph)) { rc = ensureFlow(); if (rc) return rc; }      // (allocations before the timed region)
+    { int rcs = setState(pos, token, 0, 0); if (rcs) return rcs; }
+    if (graphs) { rc = primeGraph(); if (rc) return rc; }
     HIPCHK(hipStreamSynchronize(stream));
     HIPCHK(hipEventRecord(ev0, stream));
-    for (int i = 0; i < steps; i++) {
-        if (useGraph) HIPCHK(hipGraphLaunch(execFull, stream));
-        else { rc = enqueueToken(true); if (rc) return rc; }
-    }
+    rc = decodeRun(steps, useGraph);
+    if (rc) return rc;
     HIPCHK(hipEventRecord(ev1, stream));
     HIPCHK(hipEventSynchronize(ev1));
     float ms = 0.f;
@@ -1358,7 +1452,7 @@ int HIPFusedInference::ProfileDecode(int token, int pos, int steps, unsigned cla
     profEvents.clear(); profClass.clear();
     int* gate = hGate;
     *reinterpret_cast<volatile int*>(gate) = 0;
-    HIPCHK(launch_set_state(dState, pos, token, 0, 0, ropeRef(), stream));
+    { int rcs = setState(pos, token, 0, 0); if (rcs) return rcs; }
     HIPCHK(launch_gate(gate, 100LL * 1000 * 500, stream));   // at most 0.5 s
     profiling = true;
     profMask = classMask ? classMask : 0xffu;
@@ -1510,7 +1604,7 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
     }
     // the last position continues on the decode path: final norm, lm_head, greedy token, state -> pos0 + T
     HIPCHK(hipMemcpyAsync(hidden[hiddenIdx], pfX + (size_t)(T - 1) * dim, (size_t)dim * 4, hipMemcpyDeviceToDevice, stream));
-    HIPCHK(launch_set_state(dState, pos0 + T - 1, tokens[T - 1], 0, 0, ropeRef(), stream));
+    { int rcs = setState(pos0 + T - 1, tokens[T - 1], 0, 0); if (rcs) return rcs; }
     rc = enqueueFinal(true);
     if (rc) return rc;
     HIPCHK(hipEventRecord(ev1, stream));
@@ -1527,12 +1621,14 @@ int HIPFusedInference::GeneratePrefill(const int* prompt, int nPrompt, int nDeco
     if (!built) return MG_E_NOT_BUILT;
     ARGCHK(prompt && nPrompt >= 1 && nDecode >= 1 && outTokens, "GeneratePrefill: bad arguments");
     ARGCHK(nPrompt + nDecode <= maxSeq + 1, "GeneratePrefill: prompt + decode exceeds maxSeq");
-    int rc = GraphCapture();
+    const bool graphs = !runsInLaunch(true);
+    int rc = graphs ? GraphCapture() : MG_OK;
     if (rc) return rc;
     rc = Prefill(prompt, nPrompt, 0, nullptr, nullptr, nullptr);
     if (rc) return rc;
-    if (nDecode > 1) { rc = primeGraph(); if (rc) return rc; }
-    for (int i = 1; i < nDecode; i++) HIPCHK(hipGraphLaunch(execFull, stream));
+    if (nDecode > 1 && graphs) { rc = primeGraph(); if (rc) return rc; }
+    rc = decodeRun(nDecode - 1, true);
+    if (rc) return rc;
     HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int) * (size_t)nDecode, hipMemcpyDeviceToHost, stream));
     HIPCHK(hipStreamSynchronize(stream));
     for (int i = 0; i < nDecode; i++) outTokens[i] = hTokens[i];
@@ -1693,6 +1789,14 @@ int mg_flow_in_use(mg_ctx* c) {
     if (!c || !c->f) return 0;
     return c->f->FlowInUse() ? 1 : 0;
 }
+int mg_flow_tail_in_use(mg_ctx* c) {
+    if (!c || !c->f) return 0;
+    return c->f->FlowTailInUse() ? 1 : 0;
+}
+int mg_set_flow_tail(mg_ctx* c, int on) { CTX(c); f->SetFlowTail(on); return MG_OK; }
+int mg_set_tokens_per_launch(mg_ctx* c, int n) { CTX(c); return f->SetTokensPerLaunch(n); }
+int mg_tokens_per_launch(mg_ctx* c) { return c && c->f ? c->f->tokensPerLaunch : 0; }
+int mg_flow_tail_trace(mg_ctx* c, long long* out, size_t cap, int* dims) { CTX(c); return f->FlowTailTrace(out, cap, dims); }
 int mg_flow_set_wait_limit(mg_ctx* c, long long ticks) {
     CTX(c);
     f->SetFlowWaitLimit(ticks);

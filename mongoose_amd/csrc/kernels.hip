@@ -1575,7 +1575,9 @@ hipError_t launch_fill_zero(void* ptr, size_t bytes, hipStream_t s) {
 // ---------------------------------------------------------------------------
 // Token-level stages that the reference leaves to its caller
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ void embed_element(int kind, const void* table, const float* scales, int tok, float* x, int dim, int vocab, int i);
+__device__ __forceinline__ void embed_element(int kind, const void* table, const float* scales, int tok, float* x, int dim, int vocab, int i) {
+    x[i] = embed_value(kind, table, scales, tok, dim, vocab, i);
+}
 // Row `tok` of the table into e.out, by the whole workgroup.
 __device__ __forceinline__ void embed_gather(const EmbedRef& e, int tok) {
     if (!e.out) return;
@@ -1591,25 +1593,6 @@ __global__ void embed_token_kernel(int kind, const void* table, const float* sca
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= dim) return;
     embed_element(kind, table, scales, tok, x, dim, vocab, i);
-}
-__device__ __forceinline__ void embed_element(int kind, const void* table, const float* scales, int tok, float* x, int dim, int vocab, int i) {
-    if (kind == 0) {
-        const signed char* q = static_cast<const signed char*>(table) + (size_t)tok * dim;
-        x[i] = (float)q[i] * scales[tok];
-    } else if (kind == 1) {
-        const unsigned short* t = static_cast<const unsigned short*>(table) + (size_t)tok * dim;
-        x[i] = half_bits_to_float(t[i]);
-    } else if (kind == 2) {
-        x[i] = static_cast<const float*>(table)[(size_t)tok * dim + i];
-    } else {
-        const unsigned char* base = static_cast<const unsigned char*>(table);
-        const unsigned char* qs = base + (size_t)tok * (dim >> 1);
-        const unsigned short* dpl = reinterpret_cast<const unsigned short*>(base + (size_t)vocab * (dim >> 1)) + (size_t)tok * (dim >> 5);
-        int b = i >> 5, j = i & 31;
-        unsigned char q = qs[b * 16 + (j & 15)];
-        int nib = j < 16 ? (q & 0x0f) : (q >> 4);
-        x[i] = (float)(nib - 8) * half_bits_to_float(dpl[b]);
-    }
 }
 hipError_t launch_embed_token(int kind, const void* table, const float* scales, const StepState* state, float* x,
                               int dim, int vocab, hipStream_t s) {

@@ -638,6 +638,31 @@ class HIPFusedInference:
         """True when a step over all layers goes through the persistent layer launch."""
         return lib.mg_flow_in_use(self._h) == 1
 
+    FLOW_TAIL_TRACE_POINTS = ("tail-top", "final-input-staged", "lm-head-done", "token-known", "all-waves-done", "partials-in")
+
+    def FlowTailInUse(self):
+        """True when whole tokens (embedding .. argmax) run inside the persistent launch."""
+        return lib.mg_flow_tail_in_use(self._h) == 1
+
+    def SetFlowTail(self, on):
+        return lib.mg_set_flow_tail(self._h, 1 if on else 0)
+
+    def SetTokensPerLaunch(self, n):
+        return lib.mg_set_tokens_per_launch(self._h, int(n))
+
+    def TokensPerLaunch(self):
+        return lib.mg_tokens_per_launch(self._h)
+
+    def FlowTailTrace(self):
+        """Ticks (10 ns) [point, workgroup] of the tail of the last token a launch ran (trace enabled)."""
+        dims = np.zeros(2, dtype=np.int32)
+        rc = lib.mg_flow_tail_trace(self._h, None, 0, _ip(dims))
+        if rc != 0:
+            return rc, None
+        buf = np.zeros(int(dims[0]) * int(dims[1]), dtype=np.int64)
+        rc = lib.mg_flow_tail_trace(self._h, buf.ctypes.data_as(ctypes.POINTER(ctypes.c_longlong)), buf.size, _ip(dims))
+        return rc, buf.reshape(int(dims[0]), int(dims[1]))
+
     def SetFlowWaitLimit(self, ticks):
         """Per-wait time limit of the persistent layer launch in 10 ns ticks (negative: give up at once)."""
         return lib.mg_flow_set_wait_limit(self._h, int(ticks))

@@ -121,6 +121,11 @@ _sig("mg_generate_prefill", c_int, c_void_p, _i, c_int, c_int, _i)
 _sig("mg_bench_matvec", c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _f)
 _sig("mg_flow_exchange", c_int, c_void_p, c_int, _f, c_size_t, _i)
 _sig("mg_flow_in_use", c_int, c_void_p)
+_sig("mg_flow_tail_in_use", c_int, c_void_p)
+_sig("mg_set_flow_tail", c_int, c_void_p, c_int)
+_sig("mg_set_tokens_per_launch", c_int, c_void_p, c_int)
+_sig("mg_tokens_per_launch", c_int, c_void_p)
+_sig("mg_flow_tail_trace", c_int, c_void_p, ctypes.POINTER(ctypes.c_longlong), c_size_t, _i)
 _sig("mg_flow_set_wait_limit", c_int, c_void_p, ctypes.c_longlong)
 _sig("mg_flow_trace", c_int, c_void_p, c_int, ctypes.POINTER(ctypes.c_longlong), c_size_t, _i)
 _sig("mg_weight_bytes_per_token", c_uint64, c_void_p)
