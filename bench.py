@@ -4,8 +4,10 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME]
 
 A "step" is one batch-1 greedy decode token through the whole path (embedding
-gather -> layers -> final norm -> lm_head -> argmax), replayed from a captured
-hipGraph with the position and the token resident on the device.  The W warmup
+gather -> layers -> final norm -> lm_head -> argmax) with the position and the token
+resident on the device: by default inside the persistent launch, which runs up to 64
+such steps per launch and chooses every next token on the device (the same steps as
+replays of a captured one-launch hipGraph are timed beside it).  The W warmup
 steps are the W prompt positions; the K timed steps are the K decode positions
 after them.  Weights are synthetic (seeded N(0, 0.02), quantized on the host by
 the library's own loader) and resident in HBM before the timed region starts.
@@ -15,9 +17,10 @@ the kernel that takes most of the step's time (HIP events around its launches in
 the step), a per-launch table, the lm_head matvec's own bandwidth (the second half of
 the metric), the CPU oracle timed on this box's host cores as a baseline, and -- under
 "configs" -- the same measurements for the other benchmark configurations (toy,
-TinyLlama-1.1B shape, Qwen2.5-0.5B Q4_0, Llama-3-8B shape at a short context, at ~4k
-context and its 512-token batched prefill), each with its greedy tokens checked against
-the oracle on a bounded sample.
+TinyLlama-1.1B shape, Qwen2.5-0.5B Q4_0 with a leg through the weight-streaming front end,
+Llama-3-8B shape at a short context, at ~4k context with fp32 and with fp16 K/V rows, and
+its 512-token batched prefill), each with its greedy tokens checked against the oracle
+on a bounded sample (the ~4k-context runs against the fused launches on the same positions).
 """
 import argparse
 import json
@@ -33,11 +36,17 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
 
 # HBM bytes per launch from rocprofv3 --pmc runs of this script (FETCH_SIZE then WRITE_SIZE,
 # KiB per dispatch), each scaled by what the same counter reads for a 256 MiB device copy in
-# the same run (FETCH_SIZE reads 131102.4 KiB for the 262144 KiB copied -> x1.9995; WRITE_SIZE
-# reads 262144.0 -> x1.0).  Counts are a property of kernel and shape, so they are recorded
+# the same run (FETCH_SIZE reads 131090-131102 KiB for the 262144 KiB copied -> x1.9995-1.9997;
+# WRITE_SIZE reads 262144.0 -> x1.0).  Counts are a property of kernel and shape, so they are recorded
 # here, keyed by (configuration, launch); profiles/ holds the runs they come from.  They are
 # NOT measured by the run that prints them: "traffic_source" in the output says so.
 PMC_TRAFFIC_BYTES = {
+    # the launch that runs whole tokens: bytes a TOKEN (all timed launches' counters over their tokens)
+    ("qwen2.5-0.5b", "token"): int(((16440188.1 + 16839402.9 + 17246984.3 + 2182704.8) * (262144.0 / 131090.4)
+                                    + (166748.1 + 168323.0 + 173509.0 + 21708.8)) * 1024 / 200),
+    ("tinyllama-1.1b", "token"): int((26373655.1 * (262144.0 / 131090.4) + 144828.2) * 1024 / 50),
+    ("llama-3-8b", "token"): int((240153544.6 * (262144.0 / 131090.4) + 625353.5) * 1024 / 64),
+    # separate launches (--no-flow-tail, --exec-mode 1): bytes a launch
     ("qwen2.5-0.5b", "lm_head"): int((67135.1 * (262144.0 / 131102.4) + 660.5 * 1.0) * 1024),
     ("qwen2.5-0.5b", "flow"): int((190867.0 * (262144.0 / 131102.4) + 952.0 * 1.0) * 1024),
     ("llama-3-8b", "lm_head"): int((257245.0 * (262144.0 / 131102.4) + 715.6 * 1.0) * 1024),
@@ -288,7 +297,7 @@ def check_tokens(E, orc, prompt, toks, budget_s):
 
 def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_graph=True, exec_mode=None, kv_f16=False,
             prefill=0, oracle_threads=0, check_budget_s=8.0, want_mode1_table=True, keep=False, tokens_per_launch=None,
-            want_phases=True, flow_tail=True, stream_tokens=0):
+            want_phases=True, flow_tail=True, stream_tokens=0, lean=False):
     """One configuration: load, warm up on the W prompt positions, time K decode steps at each start position of
     `contexts` (0 = right after the prompt), per-launch table, optional batched prefill, optional token check."""
     from oracle import binding as ob
@@ -328,18 +337,18 @@ def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_gra
                "step_bytes": int(step_bytes), "step_GBps": round(step_bytes / (ms_step * 1e-3) / 1e9, 1),
                "step_roofline_frac": round(step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                "launches": (K + tpl - 1) // tpl}
-        if tail and tpl > 1:
+        if tail and tpl > 1 and not lean:
             # the same steps as replays of the captured one-token graph (one launch a token)
             assert f.SetTokensPerLaunch(1) == 0
             rc, msg = f.TimedDecode(int(first[0]), P0, K, useGraph=use_graph)
             assert rc == 0, E.last_error()
             assert f.SetTokensPerLaunch(tpl) == 0
             run["graph_replay_one_token_a_launch_ms_per_step"] = round(msg / K, 5)
-        if flow and want_phases:
+        if flow and want_phases and not lean:
             run["in_launch_phases"] = phase_table(f, np, configs, s, int(first[0]), P0 + K, kv_f16)
-        table = launch_table(f, configs, s, int(first[0]), P0 + K, profile_steps, ms_step, kv_f16)
+        table = [] if (lean and tail) else launch_table(f, configs, s, int(first[0]), P0 + K, profile_steps, ms_step, kv_f16)
         run["kernels"] = table
-        if flow and want_mode1_table:
+        if flow and want_mode1_table and not lean:
             assert f.SetExecMode(1) == 0
             rc, ms1 = f.TimedDecode(int(first[0]), P0, K, useGraph=use_graph)
             assert rc == 0, E.last_error()
@@ -347,7 +356,7 @@ def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_gra
             run["kernels_fused_launches"] = launch_table(f, configs, s, int(first[0]), P0 + K, profile_steps, ms1 / K, kv_f16)
             assert f.SetExecMode(3 if exec_mode is None else exec_mode) == 0
             table = run["kernels_fused_launches"]
-        if flow and P0 > W:
+        if flow and P0 > W and not lean:
             # a long context is beyond the oracle's budget: the tokens of the launch that was timed against the fused
             # launches' (whose attention kernel the tests check against the oracle at this geometry), same positions
             seqs = {}
@@ -396,7 +405,7 @@ def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_gra
                           "mfma_frac_of_bf16_peak": round(2 * flops / (pms * 1e-3) / 1e12 / 2500.0, 4),
                           "note": "model flops = 2*T*weights of the layer projections; each is issued twice (bf16 hi and lo activation terms)"}
     toks = None
-    if orc is not None or keep:
+    if (orc is not None or keep) and not lean:
         # the token check runs on a 4-token prompt, so that the oracle's budget goes into decoded tokens
         cprompt = prompt[:4] if orc is not None else prompt
         assert f.ResetKV() == 0
@@ -479,6 +488,9 @@ def main():
                     help="tokens the persistent launch runs per launch (0 = the library's default, 64; 1 = a launch per token)")
     ap.add_argument("--no-flow-tail", action="store_true",
                     help="lm_head and argmax as launches of their own behind the persistent layer launch (for comparisons)")
+    ap.add_argument("--lean", action="store_true",
+                    help="only the timed region of the configuration (no per-launch tables, no graph-replay leg, no trace, no "
+                         "token check): the run to put under rocprofv3")
     ap.add_argument("--no-configs", action="store_true",
                     help="only the configuration named by --config (no 'configs' object with the other benchmark configurations)")
     args = ap.parse_args()
@@ -502,8 +514,8 @@ def main():
     mode = None if args.exec_mode < 0 else args.exec_mode
     res, f, prompt, first, toks = measure(E, np, configs, eng, s, args.seed, W, K, [args.context], args.profile_steps,
                                           use_graph=use_graph, exec_mode=mode, kv_f16=kv_f16, prefill=args.prefill,
-                                          oracle_threads=0, keep=True, tokens_per_launch=args.tokens_per_launch or None,
-                                          flow_tail=not args.no_flow_tail)
+                                          oracle_threads=0, keep=not args.lean or True, tokens_per_launch=args.tokens_per_launch or None,
+                                          flow_tail=not args.no_flow_tail, lean=args.lean)
     run = res["runs"][0]
     P0 = run["start_position"]
     ms_per_step = run["ms_per_step"]
@@ -595,11 +607,11 @@ def main():
     f.Close()
 
     cpu = None
-    if args.cpu_budget > 0:
+    if args.cpu_budget > 0 and not args.lean:
         cpu = cpu_baseline(E, np, s, args.seed, prompt, toks, args.cpu_budget, kv_f16=kv_f16)
 
     others = None
-    if not args.no_configs and args.config == "qwen2.5-0.5b":
+    if not args.no_configs and not args.lean and args.config == "qwen2.5-0.5b":
         others = {}
         plan = [("toy", dict(K=200, contexts=[0], threads=8)),
                 ("tinyllama-1.1b", dict(K=50, contexts=[0], threads=16)),
@@ -610,6 +622,10 @@ def main():
             others[name] = measure(E, np, configs, eng, configs.BY_NAME[name], args.seed + 1, 16, o["K"], o["contexts"],
                                    10, use_graph=True, prefill=o.get("prefill", 0), oracle_threads=o["threads"],
                                    check_budget_s=10.0, stream_tokens=o.get("stream", 0))
+        # the 8B shape's long-context leg once more with fp16 K/V rows (this backend's option, mg_set_kv_format)
+        print("bench.py: configuration llama-3-8b, fp16 K/V rows", file=sys.stderr, flush=True)
+        others["llama-3-8b-kv-f16"] = measure(E, np, configs, eng, configs.BY_NAME["llama-3-8b"], args.seed + 1, 16, 64, [4000],
+                                              10, use_graph=True, kv_f16=True, oracle_threads=0, want_mode1_table=False)
 
     out = {
         "metric": "Q8 decode tok/s (bs=1, Qwen2.5-0.5B shape) + matvec HBM GB/s % of peak" if s.name == "qwen2.5-0.5b"

@@ -22,7 +22,7 @@ struct FlowLayer {
     const float* sq; const float* sk; const float* sv; const float* so;
     const float* sgate; const float* sup; const float* sdown;
     const float* bq; const float* bk; const float* bv;      // optional (NULL)
-    float* Kc; float* Vc;                                    // fp32 caches [maxSeq, kvDim]
+    float* Kc; float* Vc;                                    // caches [maxSeq, kvDim]: fp32, or fp16 (FlowParams::kvHalf)
 };
 
 // Operands of the tail of a token (final norm, lm_head, greedy argmax, the next token's embedding), a struct in device
@@ -74,6 +74,7 @@ struct FlowParams {
     int q4;                      // 0: Q8 matrices, 1: Q4_0 matrices in the split layout
     int idleWoRows, idleGateUpRows;   // leading rows of Wo / of gate and up that workgroups idle during the attention read into the L2s
     int downSplit;               // the down projection's rows are shared by two waves each (few rows, long ones)
+    int kvHalf;                  // the caches hold fp16 rows (rounded where written, widened where read)
     int nCompute;                // workgroups 0 .. nCompute-1 compute (geo is laid out for them), the rest of the grid prefetches
     float eps;
     const StepState* state;      // position source (NULL -> posImm)

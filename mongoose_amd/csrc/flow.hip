@@ -685,7 +685,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     // the K / V rows of the earlier positions (the attention workgroups of every XCD read them; the row of the
                     // current position comes through the exchange area), while they are a small part of an L2: 0.5B shape at
                     // positions 16 .. 216 0.3766 -> 0.3710 ms a token
-                    const size_t kvBytes = (size_t)pos * kvDim * 4;
+                    const size_t kvBytes = (size_t)pos * kvDim * (p.kvHalf ? 2 : 4);
                     if (kvBytes <= ((size_t)512 << 10)) { pf.whole(L.Kc, kvBytes); pf.whole(L.Vc, kvBytes); }
                 }
                 release(G.offM);               // ... past its gate | up: gate | up of this one
@@ -772,8 +772,17 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                         stx(X + G.offQ + r, o);
                                     } else {                                              // mongoose.cu:1644-1647, and the hand-over copy
                                         // (write-through: the next token of the same launch reads the row on other XCDs)
-                                        st_agent((kk == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim + r, o);
-                                        stx(X + (kk == 1 ? G.offKc : G.offVc) + r, o);
+                                        float oc = o;
+                                        if (p.kvHalf) {           // fp16 rows: rounded where written; the hand-over copy carries the rounded value
+                                            const _Float16 hv = (_Float16)o;
+                                            oc = (float)hv;
+                                            const _Float16* dst = reinterpret_cast<const _Float16*>(kk == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim + r;
+                                            const unsigned bits = __builtin_bit_cast(unsigned short, hv);
+                                            asm volatile("global_store_short %0, %1, off sc1" : : "v"(dst), "v"(bits) : "memory");
+                                        } else {
+                                            st_agent((kk == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim + r, o);
+                                        }
+                                        stx(X + (kk == 1 ? G.offKc : G.offVc) + r, oc);
                                     }
                                 }
                             }
@@ -865,6 +874,28 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         // row has been written -- in token mode that row is written later in this same launch, by a workgroup of
                         // another XCD, and a line fetched early would be served stale from then on.
                         const float4* idle4 = reinterpret_cast<const float4*>(wt.idle) + dl;
+                        if (p.kvHalf) {
+                            // fp16 rows: a lane's piece is four halves (8 bytes), widened as it arrives
+                            typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+                            const int2* Kh = reinterpret_cast<const int2*>(L.Kc);
+                            const int2* Vh = reinterpret_cast<const int2*>(L.Vc);
+                            const int2* idle2 = reinterpret_cast<const int2*>(wt.idle) + dl;
+                            auto widen = [](int2 b) {
+                                const h4 h = __builtin_bit_cast(h4, b);
+                                return make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
+                            };
+#pragma unroll
+                            for (int u = 0; u < VU; u++) {
+                                const int row = t0 + tg + u * TG;
+                                const size_t ro = (size_t)row * rowStride + colOff;
+                                const int2* kp = row < pos ? Kh + ro : idle2;
+                                const int2* vp = row < pos ? Vh + ro : idle2;
+#pragma unroll
+                                for (int j = 0; j < NF; j++) kreg[u][j] = widen(ldg_i2<GL>(kp, j * 16));
+#pragma unroll
+                                for (int j = 0; j < NF; j++) vreg[u][j] = widen(ldg_i2<GL>(vp, j * 16));
+                            }
+                        } else {
 #pragma unroll
                         for (int u = 0; u < VU; u++) {
                             const int row = t0 + tg + u * TG;
@@ -875,6 +906,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             for (int j = 0; j < NF; j++) kreg[u][j] = ldg_f4<GL>(kp, j * 16);
 #pragma unroll
                             for (int j = 0; j < NF; j++) vreg[u][j] = ldg_f4<GL>(vp, j * 16);
+                        }
                         }
                         __syncthreads();
                         if (tid < (2 + QH) * (HD / 4)) {

@@ -708,7 +708,7 @@ int HIPFusedInference::flowComputeWgs(int cus) const {
 }
 
 bool HIPFusedInference::flowEligible(int l0, int l1) const {
-    if ((execMode != 3 && execMode != 4) || flowBroken || kvHalf) return false;
+    if ((execMode != 3 && execMode != 4) || flowBroken) return false;
     if (!flow_shape_supported(dim, kvDim, ffnDim, nHeads, nKVHeads, headDim)) return false;
     if (l1 > nLayers) l1 = nLayers;
     if (l0 < 0 || l0 >= l1) return false;
@@ -853,6 +853,7 @@ int HIPFusedInference::enqueueLayersFlow(int l0, int l1, const StepState* st, in
     p.dim = dim; p.kvDim = kvDim; p.ffn = ffnDim; p.nHeads = nHeads; p.nKVHeads = nKVHeads; p.headDim = headDim; p.maxSeq = maxSeq;
     p.q4 = layers[l0].wq.kind == WF_Q4P ? 1 : 0;
     p.nCompute = flowCompute;
+    p.kvHalf = kvHalf;
     p.downSplit = (dim <= 2048 && 2 * dim <= flowCompute * 8 && ffnDim >= 2048) ? 1 : 0;
     {
         // attention-idle prefetch: Wo where a wave holds only part of its rows ahead (rows of more than 2048 weights); of

@@ -10,7 +10,11 @@ their vectors over through an exchange area in device memory.
 * Q4_0 matrices (split layout, half-block chunks) through the same launch: every handed-over vector, tokens against
   the oracle, rows of one and of two chunks a lane, the ring variant, biases;
 * the widest FFN the launch takes, an FFN whose staged pieces come out uneven, row lengths between the tuned shapes;
-* a new context uses the launch; the trace diagnostic;
+* whole tokens inside the launch (embedding gather, layers, final norm, lm_head, argmax) and runs of tokens in one launch:
+  tokens against the oracle for every number of tokens a launch, bit-identical logits between one token a launch and
+  many, across a KV-split boundary inside a run (the K/V rows a run writes are read by its later tokens on other XCDs);
+* fp16 K/V rows through the launch;
+* a new context uses the launch; the trace diagnostic, the tail's included;
 * a wait that runs out: the launch still ends, the call reports it, the context continues with the fused launches.
 """
 import numpy as np
@@ -274,6 +278,37 @@ def test_heads_of_128_grouped_kv(hip):
     m.close()
 
 
+def test_fp16_kv_rows_in_the_launch(hip):
+    """fp16 K/V rows (SetKVFormat(1)) through the persistent launch: rounded where the q|k|v phase writes them (the
+    cache and the copy it hands to the attention workgroups), widened where the attention phase reads them.  Tokens
+    against the oracle with the same rounding (toy, and heads of 128 over several KV splits), then against the fused
+    launches -- tokens, logits and hidden state -- at the 8B attention geometry with grouped attention at positions
+    4040..4090."""
+    m = H.Model(configs.TOY, seed=44, maxSeq=72, eng=hip, threads=8, kv_f16=True)
+    prompt = m.prompt(8)
+    ref, _ = H.oracle_generate(m, prompt, 40)
+    rc, t = m.hip.Generate(prompt, 40, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert _in_use(m.hip) and m.hip.FlowTailInUse(), "fp16 rows should not keep a context out of the launch"
+    assert t.tolist() == ref.tolist(), H.first_divergence(t, ref)
+    m.close()
+    s = configs.Shape("l3-mini-f16", 2, 512, 4, 1, 128, 1024, 512, 1e-5, 5e5, False, True, "q8")
+    m = H.Model(s, seed=45, maxSeq=600, eng=hip, threads=8, kv_f16=True)
+    prompt = m.prompt(4)
+    ref, _ = H.oracle_generate(m, prompt, 300)
+    rc, t = m.hip.Generate(prompt, 300, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert _in_use(m.hip)
+    assert t.tolist() == ref.tolist(), H.first_divergence(t, ref)
+    _modes_agree(m, m.prompt(500), 40, "fp16 rows, heads of 128, 4-5 splits")
+    m.close()
+    s = H.with_layers(configs.LLAMA3_8B, 2)._replace(name="l3-geom-f16", ffnDim=1024, vocab=1024, tied=True)
+    m = H.Model(s, seed=46, maxSeq=4096, eng=hip, oracle=False, kv_f16=True)
+    print("flow: llama-3 geometry, fp16 rows, grouped attention, positions 4040..4090", flush=True)
+    _modes_agree(m, m.prompt(4040), 50, "fp16 rows, heads of 128, grouped")
+    m.close()
+
+
 @pytest.mark.parametrize("ffn", [15360, 9216])
 def test_streamed_rows_wide_ffn(hip, ffn):
     """Rows of 4096 weights with the widest FFN the launch takes (15360: seven or eight staged pieces a thread for the
@@ -314,6 +349,55 @@ def test_row_lengths_between_the_tuned_ones(hip, fmt, name, dim, heads, kv, hd, 
     m.close()
 
 
+@pytest.mark.parametrize("fmt", ["q8", "q4_0"])
+def test_runs_of_tokens_in_one_launch(hip, fmt):
+    """Whole tokens inside the persistent launch.  Toy model (8 + 64): the oracle's tokens whether a launch runs 1, 5 or 64
+    tokens, through Generate and GeneratePrefill, and with the lm_head and argmax as launches of their own
+    (SetFlowTail(0)).  0.5B geometry, 2 layers: a run of 80 tokens from position 90 crosses the boundary between the
+    first and the second KV split at position 128 inside one launch -- every K/V row the run writes is read by the
+    tokens after it -- and gives the tokens, and bit for bit the logits of the step after, of one token a launch."""
+    s = configs.TOY
+    m = H.Model(s, seed=41, maxSeq=80, eng=hip, threads=8, fmt=fmt)
+    prompt = m.prompt(8)
+    ref, _ = H.oracle_generate(m, prompt, 64)
+    assert m.hip.FlowTailInUse(), "whole tokens should run inside the launch"
+    for n in (1, 5, 64):
+        assert m.hip.SetTokensPerLaunch(n) == 0
+        assert m.hip.ResetKV() == 0
+        rc, t = m.hip.Generate(prompt, 64, useGraph=True)
+        assert rc == 0, E.last_error()
+        assert t.tolist() == ref.tolist(), (n, H.first_divergence(t, ref))
+    assert m.hip.ResetKV() == 0
+    rc, t = m.hip.GeneratePrefill(prompt, 64)
+    assert rc == 0, E.last_error()
+    H.assert_same_tokens_or_near_tie(m, prompt, t, ref, f"prefill then a run of tokens, {fmt}")
+    assert m.hip.SetFlowTail(False) == 0
+    assert m.hip.FlowInUse() and not m.hip.FlowTailInUse()
+    assert m.hip.ResetKV() == 0
+    rc, t = m.hip.Generate(prompt, 64, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert t.tolist() == ref.tolist()
+    m.close()
+
+    s = H.with_layers(configs.QWEN if fmt == "q8" else configs.QWEN_Q4, 2)._replace(name="qwen-geom-runs", vocab=2048)
+    m = H.Model(s, seed=42, maxSeq=200, eng=hip, oracle=False, fmt=fmt)
+    prompt = m.prompt(90)
+    res = {}
+    logits = np.empty(s.vocab, np.float32)
+    for n in (1, 64):
+        assert m.hip.SetTokensPerLaunch(n) == 0
+        assert m.hip.ResetKV() == 0
+        rc, t = m.hip.GeneratePrefill(prompt, 80)
+        assert rc == 0, E.last_error()
+        assert m.hip.FlowTailInUse()
+        rc, _ = m.hip.DecodeToken(int(t[-1]), 169, logits)
+        assert rc == 0, E.last_error()
+        res[n] = (t.tolist(), logits.copy())
+    assert res[1][0] == res[64][0], H.first_divergence(res[1][0], res[64][0])
+    assert np.array_equal(res[1][1], res[64][1])
+    m.close()
+
+
 def test_new_context_uses_the_launch_and_trace(hip):
     s = H.with_layers(configs.TOY, 8)
     m = H.Model(s, seed=5, maxSeq=40, eng=hip, threads=8)
@@ -332,6 +416,12 @@ def test_new_context_uses_the_launch_and_trace(hip):
     # every workgroup passed the top of every layer, later in every later layer
     tops = tr[:, 0, :]
     assert (tops > 0).all() and (np.diff(tops.astype(np.int64), axis=0) > 0).all()
+    # the tail of the token: after the last layer, in program order
+    rc, tt = m.hip.FlowTailTrace()
+    assert rc == 0 and tt.shape[0] == len(m.hip.FLOW_TAIL_TRACE_POINTS)
+    assert (tt[0] >= tr[-1, -1, :]).all()
+    top, staged, wave0, known, done, parts = [tt[i].astype(np.int64) for i in range(6)]
+    assert (staged >= top).all() and (wave0 >= staged).all() and (done >= wave0).all() and (parts >= done).all() and (known >= parts).all()
     assert m.hip.FlowTrace(False)[0] == 0
     # a context in another mode has no such launch to trace
     assert m.hip.SetExecMode(1) == 0

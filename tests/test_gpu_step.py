@@ -282,8 +282,8 @@ def test_streaming_matches_resident(hip):
 
 
 def test_fp16_kv_cache(hip):
-    """fp16 KV rows (mg_set_kv_format 1) against the oracle with the same rounding; fused launches,
-    graph replay and the per-op launches.  Hidden-state bar 5e-4 instead of 1e-4: two correct fp32
+    """fp16 KV rows (mg_set_kv_format 1) against the oracle with the same rounding; the persistent launch (what a new
+    context runs), fused launches, graph replay and the per-op launches.  Hidden-state bar 5e-4 instead of 1e-4: two correct fp32
     evaluations of a K/V element differ in the last bit, which now and then lands on either side of
     an fp16 rounding boundary, and that element then differs by one fp16 ulp (4.9e-4 relative) --
     at position 0 the attention output *is* the V row.  Logits 1e-3 and identical tokens as always."""
