@@ -137,9 +137,8 @@ __device__ __forceinline__ void poll_partial(const f4* pa, const float* pm, cons
         else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
     }
 }
-// A layer's table entry, read one layer ahead: lane i loads word i, and the fields are picked out of the lanes into
-// scalar registers when the layer starts (the entry is in HBM and cold; read at the top of its layer it would
-// hold up every wave of the launch).
+// A layer's table entry, read one layer ahead: lane i loads word i (the entry is in HBM and cold; read at the top of
+// its layer it would hold up every wave of the launch).
 __device__ __forceinline__ unsigned layer_words(const FlowLayer* t, int l, int lane) {
     static_assert(sizeof(FlowLayer) <= 64 * 4, "one word a lane");
     const unsigned* q = reinterpret_cast<const unsigned*>(t + l);
@@ -150,20 +149,22 @@ __device__ __forceinline__ T* lane_ptr(unsigned v, int word) {
     const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)v, word), hi = (unsigned)__builtin_amdgcn_readlane((int)v, word + 1);
     return reinterpret_cast<T*>(((unsigned long long)hi << 32) | lo);
 }
-#define FL_PTR(T, field) lane_ptr<T>(v, (int)(offsetof(FlowLayer, field) / 4))
-__device__ __forceinline__ FlowLayer unpack_layer(unsigned v) {
-    FlowLayer L;
-    L.g1 = FL_PTR(const float, g1); L.g2 = FL_PTR(const float, g2);
-    L.wq = FL_PTR(const signed char, wq); L.wk = FL_PTR(const signed char, wk); L.wv = FL_PTR(const signed char, wv);
-    L.wo = FL_PTR(const signed char, wo); L.gate = FL_PTR(const signed char, gate); L.up = FL_PTR(const signed char, up);
-    L.down = FL_PTR(const signed char, down);
-    L.sq = FL_PTR(const float, sq); L.sk = FL_PTR(const float, sk); L.sv = FL_PTR(const float, sv); L.so = FL_PTR(const float, so);
-    L.sgate = FL_PTR(const float, sgate); L.sup = FL_PTR(const float, sup); L.sdown = FL_PTR(const float, sdown);
-    L.bq = FL_PTR(const float, bq); L.bk = FL_PTR(const float, bk); L.bv = FL_PTR(const float, bv);
-    L.Kc = FL_PTR(float, Kc); L.Vc = FL_PTR(float, Vc);
-    return L;
-}
-#undef FL_PTR
+// The fields of a layer's entry are picked out of the lanes where they are used, two readlanes a pointer, not all at the
+// top of the layer: 21 pointers held in scalar registers across a layer's phases, on top of the launch's parameters, are
+// more than the scalar file has, and the compiler then parks them in lanes of a vector register of its own and fetches
+// them back one by one -- some 60 lane writes and over 100 lane reads a layer and wave.
+struct LayerView {
+    unsigned v;
+#define FL_FIELD(T, field) __device__ __forceinline__ T* field() const { return lane_ptr<T>(v, (int)(offsetof(FlowLayer, field) / 4)); }
+    FL_FIELD(const float, g1) FL_FIELD(const float, g2)
+    FL_FIELD(const signed char, wq) FL_FIELD(const signed char, wk) FL_FIELD(const signed char, wv) FL_FIELD(const signed char, wo)
+    FL_FIELD(const signed char, gate) FL_FIELD(const signed char, up) FL_FIELD(const signed char, down)
+    FL_FIELD(const float, sq) FL_FIELD(const float, sk) FL_FIELD(const float, sv) FL_FIELD(const float, so)
+    FL_FIELD(const float, sgate) FL_FIELD(const float, sup) FL_FIELD(const float, sdown)
+    FL_FIELD(const float, bq) FL_FIELD(const float, bk) FL_FIELD(const float, bv)
+    FL_FIELD(float, Kc) FL_FIELD(float, Vc)
+#undef FL_FIELD
+};
 // The tail's operands (FlowTail), read the same way: one word a lane, fields picked out where they are used.
 __device__ __forceinline__ unsigned tail_words(const FlowTail* t, int lane) {
     static_assert(sizeof(FlowTail) <= 64 * 4, "one word a lane");
@@ -542,7 +543,9 @@ constexpr int NID = 8 / FWAVES;    // down rows a wave holds in flight
 // RING: gate | up and down stream their rows through a ring of register sets (rows of more than 2048 weights)
 // GQA: an attention workgroup takes all query heads of a KV head (contexts too long for one workgroup a query head)
 // Q4: the seven matrices of a layer are Q4_0 in the split layout (the table's scale pointers then hold the d planes)
-template <int HD, int CBD, bool RING, bool GQA, bool Q4>
+// TRACE: the launch records its per-workgroup timeline (FlowParams::trace); the variants without it carry neither the
+//        trace points' instructions nor their scalar registers (1.2 % of the step at the 0.5B and 1.1B shapes)
+template <int HD, int CBD, bool RING, bool GQA, bool Q4, bool TRACE>
 __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     extern __shared__ float4 a4[];                     // the staged activation vector, max(dim, ffn) floats
     __shared__ float red[FWAVES];
@@ -597,8 +600,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     const int half = HD >> 1;
 
     // timing trace (diagnostic): slot b of layer l, per workgroup, in ticks of the 100 MHz wall clock
-#define FLOW_TRACE(b) do { if (p.trace && tid == 0 && (int)blockIdx.x < nC) \
-        p.trace[((size_t)(l - p.l0) * FLOW_TRACE_SLOTS + (b)) * nC + blockIdx.x] = wall_clock64(); } while (0)
+#define FLOW_TRACE(b) do { if constexpr (TRACE) { if (p.trace && tid == 0 && (int)blockIdx.x < nC) \
+        p.trace[((size_t)(l - p.l0) * FLOW_TRACE_SLOTS + (b)) * nC + blockIdx.x] = wall_clock64(); } } while (0)
     // the exchange area as a buffer resource: agent-scope loads that the compiler keeps track of (used where many are
     // wanted in flight together)
     const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(p.xchg, 0, (int)((size_t)p.nLayersTotal * G.stride * 4 * (p.nTokens > 0 ? 2 : 1)), 0x00020000);
@@ -647,7 +650,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             const size_t rdD = dim >> 4, rdF = ffn >> 4;                             // ... of its fp16 d values (Q4_0)
             const int halfHd = HD >> 1;
             for (int l = p.l0; l < p.l1; l++) {
-                const FlowLayer L = unpack_layer(lw);
+                LayerView L{lw};
                 if (l + 1 < p.l1) lw = layer_words(p.layers, l + 1, lane);
                 else if (tk + 1 < nTok) lw = layer_words(p.layers, p.l0, lane);
                 const float* Xp = xb + (size_t)(l - 1) * G.stride;               // the layer before (not for the first)
@@ -665,9 +668,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     for (int g = pf.x + 8 * pf.rank; g * 8 < nI; g += 8 * pf.nRank) {
                         const int item = g * 8;
                         const signed char* Wm; const float* aux; int a0, a1;
-                        if (item < nq) { Wm = L.wq; aux = L.sq; const int jj = item % halfHd; a0 = (item - jj) * 2 + jj; a1 = a0 + halfHd; }
-                        else if (item < nq + nk) { Wm = L.wk; aux = L.sk; const int i2 = item - nq; const int jj = i2 % halfHd; a0 = (i2 - jj) * 2 + jj; a1 = a0 + halfHd; }
-                        else { Wm = L.wv; aux = L.sv; a0 = (item - nq - nk) * 2; a1 = a0 + 8; }
+                        if (item < nq) { Wm = L.wq(); aux = L.sq(); const int jj = item % halfHd; a0 = (item - jj) * 2 + jj; a1 = a0 + halfHd; }
+                        else if (item < nq + nk) { Wm = L.wk(); aux = L.sk(); const int i2 = item - nq; const int jj = i2 % halfHd; a0 = (i2 - jj) * 2 + jj; a1 = a0 + halfHd; }
+                        else { Wm = L.wv(); aux = L.sv(); a0 = (item - nq - nk) * 2; a1 = a0 + 8; }
                         const char* wb = reinterpret_cast<const char*>(Wm);
                         pf.span(wb, (size_t)a0 * rbD, (size_t)(a0 + 8) * rbD);
                         pf.span(wb, (size_t)a1 * rbD, (size_t)(a1 + 8) * rbD);
@@ -677,27 +680,27 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             pf.span(db, ((size_t)a1 * rdD) & ~(size_t)15, (size_t)(a1 + 8) * rdD);
                         }
                     }
-                    if (!Q4) { pf.whole(L.sq, (size_t)dim * 4); pf.whole(L.sk, (size_t)kvDim * 4); pf.whole(L.sv, (size_t)kvDim * 4); }
-                    pf.whole(L.bq, (size_t)dim * 4); pf.whole(L.bk, (size_t)kvDim * 4); pf.whole(L.bv, (size_t)kvDim * 4);
-                    pf.whole(L.g1, (size_t)dim * 4);
-                    pf.rows(L.wo, rbD, dim, 8);
-                    if (Q4) pf.rows(L.so, rdD, dim, 8); else pf.whole(L.so, (size_t)dim * 4);
+                    if (!Q4) { pf.whole(L.sq(), (size_t)dim * 4); pf.whole(L.sk(), (size_t)kvDim * 4); pf.whole(L.sv(), (size_t)kvDim * 4); }
+                    pf.whole(L.bq(), (size_t)dim * 4); pf.whole(L.bk(), (size_t)kvDim * 4); pf.whole(L.bv(), (size_t)kvDim * 4);
+                    pf.whole(L.g1(), (size_t)dim * 4);
+                    pf.rows(L.wo(), rbD, dim, 8);
+                    if (Q4) pf.rows(L.so(), rdD, dim, 8); else pf.whole(L.so(), (size_t)dim * 4);
                     // the K / V rows of the earlier positions (the attention workgroups of every XCD read them; the row of the
                     // current position comes through the exchange area), while they are a small part of an L2: 0.5B shape at
                     // positions 16 .. 216 0.3766 -> 0.3710 ms a token
                     const size_t kvBytes = (size_t)pos * kvDim * (p.kvHalf ? 2 : 4);
-                    if (kvBytes <= ((size_t)512 << 10)) { pf.whole(L.Kc, kvBytes); pf.whole(L.Vc, kvBytes); }
+                    if (kvBytes <= ((size_t)512 << 10)) { pf.whole(L.Kc(), kvBytes); pf.whole(L.Vc(), kvBytes); }
                 }
                 release(G.offM);               // ... past its gate | up: gate | up of this one
-                pf.rows(L.gate, rbD, ffn, 8);
-                pf.rows(L.up, rbD, ffn, 8);
-                if (Q4) { pf.rows(L.sgate, rdD, ffn, 8); pf.rows(L.sup, rdD, ffn, 8); }
-                else { pf.whole(L.sgate, (size_t)ffn * 4); pf.whole(L.sup, (size_t)ffn * 4); }
-                pf.whole(L.g2, (size_t)dim * 4);
+                pf.rows(L.gate(), rbD, ffn, 8);
+                pf.rows(L.up(), rbD, ffn, 8);
+                if (Q4) { pf.rows(L.sgate(), rdD, ffn, 8); pf.rows(L.sup(), rdD, ffn, 8); }
+                else { pf.whole(L.sgate(), (size_t)ffn * 4); pf.whole(L.sup(), (size_t)ffn * 4); }
+                pf.whole(L.g2(), (size_t)dim * 4);
                 release(G.offX2);              // ... done: the down projection of this one
                 const int drun = p.downSplit ? FWAVES / 2 : FWAVES;      // rows of the down projection a workgroup takes
-                pf.rows(L.down, rbF, dim, drun);
-                if (Q4) pf.rows(L.sdown, rdF, dim, drun); else pf.whole(L.sdown, (size_t)dim * 4);
+                pf.rows(L.down(), rbF, dim, drun);
+                if (Q4) pf.rows(L.sdown(), rdF, dim, drun); else pf.whole(L.sdown(), (size_t)dim * 4);
             }
             pf.drain();
         } else {
@@ -706,7 +709,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 // the phases' own working sets then no longer fit the registers)
                 asm volatile("" : "+v"(tid), "+v"(lane));
                 asm volatile("" : "+s"(wave), "+s"(gw), "+s"(dim), "+s"(kvDim), "+s"(ffn), "+s"(nchD), "+s"(nchF));
-                const FlowLayer L = unpack_layer(lw);
+                LayerView L{lw};
                 if (l + 1 < p.l1) lw = layer_words(p.layers, l + 1, lane);
                 else if (tk + 1 < nTok) lw = layer_words(p.layers, p.l0, lane);
                 FLOW_TRACE(0);
@@ -727,9 +730,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         float e0[NPI], e1[NPI];                  // per-lane epilogue operands: lanes 0/1 scale and bias, lane 2 cos and sin
                         auto resolve = [&](int4 (&w)[2][CBQ], WRow (&rw)[2], int& kd, int& a0, int& a1, float& f0, float& f1, int item) {
                             const signed char* Wm; const float* sc; const float* bias;
-                            if (item < nq) { kd = 0; Wm = L.wq; sc = L.sq; bias = L.bq; const int jj = item % half; a0 = (item - jj) * 2 + jj; a1 = a0 + half; }
-                            else if (item < nq + nk) { kd = 1; Wm = L.wk; sc = L.sk; bias = L.bk; const int i2 = item - nq; const int jj = i2 % half; a0 = (i2 - jj) * 2 + jj; a1 = a0 + half; }
-                            else { kd = 2; Wm = L.wv; sc = L.sv; bias = L.bv; a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
+                            if (item < nq) { kd = 0; Wm = L.wq(); sc = L.sq(); bias = L.bq(); const int jj = item % half; a0 = (item - jj) * 2 + jj; a1 = a0 + half; }
+                            else if (item < nq + nk) { kd = 1; Wm = L.wk(); sc = L.sk(); bias = L.bk(); const int i2 = item - nq; const int jj = i2 % half; a0 = (i2 - jj) * 2 + jj; a1 = a0 + half; }
+                            else { kd = 2; Wm = L.wv(); sc = L.sv(); bias = L.bv(); a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
                             rw[0] = wrow<Q4>(Wm, sc, a0, dim); rw[1] = wrow<Q4>(Wm, sc, a1, dim);
                             ld_row<GL, Q4, CBQ>(rw[0], nchD, lane, 0, w[0]);
                             ld_row<GL, Q4, CBQ>(rw[1], nchD, lane, 0, w[1]);
@@ -776,11 +779,11 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                         if (p.kvHalf) {           // fp16 rows: rounded where written; the hand-over copy carries the rounded value
                                             const _Float16 hv = (_Float16)o;
                                             oc = (float)hv;
-                                            const _Float16* dst = reinterpret_cast<const _Float16*>(kk == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim + r;
+                                            const _Float16* dst = reinterpret_cast<const _Float16*>(kk == 1 ? L.Kc() : L.Vc()) + (size_t)pos * kvDim + r;
                                             const unsigned bits = __builtin_bit_cast(unsigned short, hv);
                                             asm volatile("global_store_short %0, %1, off sc1" : : "v"(dst), "v"(bits) : "memory");
                                         } else {
-                                            st_agent((kk == 1 ? L.Kc : L.Vc) + (size_t)pos * kvDim + r, o);
+                                            st_agent((kk == 1 ? L.Kc() : L.Vc()) + (size_t)pos * kvDim + r, o);
                                         }
                                         stx(X + (kk == 1 ? G.offKc : G.offVc) + r, oc);
                                     }
@@ -789,10 +792,10 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         };
 #pragma unroll
                         for (int q = 0; q < NPI; q++) {
-                            kind[q] = 0; r0[q] = 0; r1[q] = 0; e0[q] = 0.f; e1[q] = 0.f; rows[q][0] = wrow<Q4>(L.wq, L.sq, 0, dim); rows[q][1] = rows[q][0];
+                            kind[q] = 0; r0[q] = 0; r1[q] = 0; e0[q] = 0.f; e1[q] = 0.f; rows[q][0] = wrow<Q4>(L.wq(), L.sq(), 0, dim); rows[q][1] = rows[q][0];
                             if (gw + q * W < nI) resolve(wr[q], rows[q], kind[q], r0[q], r1[q], e0[q], e1[q], gw + q * W);
                         }
-                        const float rs = stage_rms<GL, Q4, !RING>(xin, !first, L.g1, dim, p.eps, a4, red, wt);
+                        const float rs = stage_rms<GL, Q4, !RING>(xin, !first, L.g1(), dim, p.eps, a4, red, wt);
                         FLOW_TRACE(1);
 #pragma unroll
                         for (int q = 0; q < NPI; q++)
@@ -846,13 +849,13 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             // (a workgroup without q | k | v rows gets here at the top of the layer; holding it back until q | k | v is
                             // through measures slower: 1.1B shape 0.453 against 0.435 ms a token)
                             if (p.idleWoRows > 0) {
-                                pf.rows(L.wo, rbD, p.idleWoRows, 8);
-                                if (Q4) pf.rows(L.so, rdD, p.idleWoRows, 8);
+                                pf.rows(L.wo(), rbD, p.idleWoRows, 8);
+                                if (Q4) pf.rows(L.so(), rdD, p.idleWoRows, 8);
                             }
                             if (p.idleGateUpRows > 0) {
-                                pf.rows(L.gate, rbD, p.idleGateUpRows, 8);
-                                pf.rows(L.up, rbD, p.idleGateUpRows, 8);
-                                if (Q4) { pf.rows(L.sgate, rdD, p.idleGateUpRows, 8); pf.rows(L.sup, rdD, p.idleGateUpRows, 8); }
+                                pf.rows(L.gate(), rbD, p.idleGateUpRows, 8);
+                                pf.rows(L.up(), rbD, p.idleGateUpRows, 8);
+                                if (Q4) { pf.rows(L.sgate(), rdD, p.idleGateUpRows, 8); pf.rows(L.sup(), rdD, p.idleGateUpRows, 8); }
                             }
                             pf.drain();
                         }
@@ -866,8 +869,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         const int t1 = min(len, t0 + TILE);
                         const size_t rowStride = (size_t)kvDim / 4;
                         const size_t colOff = (size_t)(kvh * HD) / 4 + dl;
-                        const float4* Kc4 = reinterpret_cast<const float4*>(L.Kc);
-                        const float4* Vc4 = reinterpret_cast<const float4*>(L.Vc);
+                        const float4* Kc4 = reinterpret_cast<const float4*>(L.Kc());
+                        const float4* Vc4 = reinterpret_cast<const float4*>(L.Vc());
                         float4 kreg[VU][NF], vreg[VU][NF];
                         // Only rows of earlier positions are read from the caches (the current one comes through the exchange
                         // area, the loads of later ones go to the idle line): a cache line is never fetched into an L2 before its
@@ -877,8 +880,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         if (p.kvHalf) {
                             // fp16 rows: a lane's piece is four halves (8 bytes), widened as it arrives
                             typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-                            const int2* Kh = reinterpret_cast<const int2*>(L.Kc);
-                            const int2* Vh = reinterpret_cast<const int2*>(L.Vc);
+                            const int2* Kh = reinterpret_cast<const int2*>(L.Kc());
+                            const int2* Vh = reinterpret_cast<const int2*>(L.Vc());
                             const int2* idle2 = reinterpret_cast<const int2*>(wt.idle) + dl;
                             auto widen = [](int2 b) {
                                 const h4 h = __builtin_bit_cast(h4, b);
@@ -1068,13 +1071,13 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     if (blockIdx.x * FWAVES < nI) {
                         int it = gw;
                         int4 wr[1][CBD];
-                        WRow rows[1] = {wrow<Q4>(L.wo, L.so, 0, dim)};
+                        WRow rows[1] = {wrow<Q4>(L.wo(), L.so(), 0, dim)};
                         float e0 = 0.f, e1 = 0.f;
                         auto resolve = [&](int item) {
-                            rows[0] = wrow<Q4>(L.wo, L.so, item, dim);
+                            rows[0] = wrow<Q4>(L.wo(), L.so(), item, dim);
                             ld_row<GL, Q4, CBD>(rows[0], nchD, lane, 0, wr[0]);
                             if (lane == 0) {
-                                e0 = Q4 ? 1.f : ldg_f<GL>(L.so, item);
+                                e0 = Q4 ? 1.f : ldg_f<GL>(L.so(), item);
                                 e1 = first ? xin[item] : poll1(xin + item, wt);         // there already if this workgroup staged it for q | k | v
                             }
                         };
@@ -1147,16 +1150,16 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                 const int sc = min(st, T - 1);                       // past the end: the last step again (uniform loop)
                                 const int k = sc / nb, b = sc - k * nb;
                                 const int row = gw + k * W;
-                                ld_row<GL, Q4, CB>(wrow<Q4>(L.gate, L.sgate, row, dim), nchD, lane, b * CB * 64, set[0]);
-                                ld_row<GL, Q4, CB>(wrow<Q4>(L.up, L.sup, row, dim), nchD, lane, b * CB * 64, set[1]);
+                                ld_row<GL, Q4, CB>(wrow<Q4>(L.gate(), L.sgate(), row, dim), nchD, lane, b * CB * 64, set[0]);
+                                ld_row<GL, Q4, CB>(wrow<Q4>(L.up(), L.sup(), row, dim), nchD, lane, b * CB * 64, set[1]);
                             };
                             float sg = 0.f, su = 0.f;
                             if (T > 0) {
 #pragma unroll
                                 for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
-                                if (lane < nItems) { const int r = gw + lane * W; sg = Q4 ? 1.f : ldg_f<GL>(L.sgate, r); su = Q4 ? 1.f : ldg_f<GL>(L.sup, r); }
+                                if (lane < nItems) { const int r = gw + lane * W; sg = Q4 ? 1.f : ldg_f<GL>(L.sgate(), r); su = Q4 ? 1.f : ldg_f<GL>(L.sup(), r); }
                             }
-                            const float rs = stage_rms<GL, Q4, !RING>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                            const float rs = stage_rms<GL, Q4, !RING>(X + G.offX1, true, L.g2(), dim, p.eps, a4, red, wt);
                             FLOW_TRACE(7);
                             float acc[2] = {0.f, 0.f};
                             float g = 0.f, u = 0.f;
@@ -1191,14 +1194,14 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             for (int k = 0; k < NIB; k++) {
                                 const int r = it0 + k * W;
                                 if (r < nI) {                                           // uniform in the wave
-                                    ld_row<GL, Q4, CBD>(wrow<Q4>(L.gate, L.sgate, r, dim), nchD, lane, 0, wr[k][0]);
-                                    ld_row<GL, Q4, CBD>(wrow<Q4>(L.up, L.sup, r, dim), nchD, lane, 0, wr[k][1]);
+                                    ld_row<GL, Q4, CBD>(wrow<Q4>(L.gate(), L.sgate(), r, dim), nchD, lane, 0, wr[k][0]);
+                                    ld_row<GL, Q4, CBD>(wrow<Q4>(L.up(), L.sup(), r, dim), nchD, lane, 0, wr[k][1]);
                                 }
                             }
-                            if (lane < NIB) { const int r = min(it0 + lane * W, nI - 1); sg = Q4 ? 1.f : ldg_f<GL>(L.sgate, r); su = Q4 ? 1.f : ldg_f<GL>(L.sup, r); }
+                            if (lane < NIB) { const int r = min(it0 + lane * W, nI - 1); sg = Q4 ? 1.f : ldg_f<GL>(L.sgate(), r); su = Q4 ? 1.f : ldg_f<GL>(L.sup(), r); }
                         };
                         if (gw < nI) issue(gw);
-                        const float rs = stage_rms<GL, Q4, !RING>(X + G.offX1, true, L.g2, dim, p.eps, a4, red, wt);
+                        const float rs = stage_rms<GL, Q4, !RING>(X + G.offX1, true, L.g2(), dim, p.eps, a4, red, wt);
                         FLOW_TRACE(7);
                         for (int it0 = gw; it0 < nI; it0 += NIB * W) {
                             if (it0 != gw) issue(it0);
@@ -1210,7 +1213,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                     dot_rows<Q4, 2, CBD>(wr[k], a4, nchD, lane, 0, acc);
                                     if (nchD > CBD * 64) {
                                         const int r = it0 + k * W;
-                                        const WRow rows[2] = {wrow<Q4>(L.gate, L.sgate, r, dim), wrow<Q4>(L.up, L.sup, r, dim)};
+                                        const WRow rows[2] = {wrow<Q4>(L.gate(), L.sgate(), r, dim), wrow<Q4>(L.up(), L.sup(), r, dim)};
                                         dot_rows_tail<GL, Q4, 2, CBD>(rows, a4, nchD, lane, acc);
                                     }
                                     const float t = wave_sum2(acc[0], acc[1]);
@@ -1242,11 +1245,11 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             auto issueStep = [&](int4 (&set)[1][CB], int st) {
                                 const int sc = min(st, T - 1);
                                 const int k = sc / nb, b = sc - k * nb;
-                                ld_row<GL, Q4, CB>(wrow<Q4>(L.down, L.sdown, gw + k * W, ffn), nchF, lane, b * CB * 64, set[0]);
+                                ld_row<GL, Q4, CB>(wrow<Q4>(L.down(), L.sdown(), gw + k * W, ffn), nchF, lane, b * CB * 64, set[0]);
                             };
                             float e0 = 0.f, e1 = 0.f;
                             if (T > 0) {
-                                if (lane < nItems) { const int r = gw + lane * W; e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r); e1 = poll1(X + G.offX1 + r, wt); }
+                                if (lane < nItems) { const int r = gw + lane * W; e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown(), r); e1 = poll1(X + G.offX1 + r, wt); }
 #pragma unroll
                                 for (int j = 0; j < RD - 1; j++) issueStep(ring[j], j);
                             }
@@ -1282,13 +1285,13 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             const int row = min(gw >> 1, nI - 1), hf = wave & 1;
                             const int nHalf = (nchF + 1) >> 1;
                             const int c0 = hf ? nHalf : 0, cHi = hf ? nchF : nHalf;
-                            const WRow rw = wrow<Q4>(L.down, L.sdown, row, ffn);
+                            const WRow rw = wrow<Q4>(L.down(), L.sdown(), row, ffn);
                             int4 wr[CBH];
                             ld_row_rng<GL, Q4, CBH>(rw, cHi, lane, c0, wr);
                             float e0 = 0.f, e1 = 0.f;
                             if (wave == 0 && lane < FWAVES / 2) {
                                 const int r = min((int)blockIdx.x * (FWAVES / 2) + lane, nI - 1);
-                                e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r);
+                                e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown(), r);
                                 e1 = poll1(X + G.offX1 + r, wt);
                             }
                             stage_plain<Q4, false>(X + G.offM, ffn, a4, wt);
@@ -1318,9 +1321,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
 #pragma unroll
                             for (int k = 0; k < NID; k++) {
                                 const int r = it0 + k * W;
-                                if (r < nI) ld_row<GL, Q4, CBF>(wrow<Q4>(L.down, L.sdown, r, ffn), nchF, lane, 0, wr[k][0]);      // uniform in the wave
+                                if (r < nI) ld_row<GL, Q4, CBF>(wrow<Q4>(L.down(), L.sdown(), r, ffn), nchF, lane, 0, wr[k][0]);      // uniform in the wave
                             }
-                            if (lane < NID) { const int r = min(it0 + lane * W, nI - 1); e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown, r); e1 = poll1(X + G.offX1 + r, wt); }
+                            if (lane < NID) { const int r = min(it0 + lane * W, nI - 1); e0 = Q4 ? 1.f : ldg_f<GL>(L.sdown(), r); e1 = poll1(X + G.offX1 + r, wt); }
                         };
                         if (gw < nI) issue(gw);
                         stage_plain<Q4, false>(X + G.offM, ffn, a4, wt);
@@ -1334,7 +1337,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                 if (it0 + k * W < nI) {
                                     dot_rows<Q4, 1, CBF>(wr[k], a4, nchF, lane, 0, acc);
                                     if (nchF > CBF * 64) {
-                                        const WRow rows[1] = {wrow<Q4>(L.down, L.sdown, it0 + k * W, ffn)};
+                                        const WRow rows[1] = {wrow<Q4>(L.down(), L.sdown(), it0 + k * W, ffn)};
                                         dot_rows_tail<GL, Q4, 1, CBF>(rows, a4, nchF, lane, acc);
                                     }
                                     acc[0] = wave_sum(acc[0]);
@@ -1408,10 +1411,17 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 }
             };
             const float* xfin = xb + (size_t)(p.l1 - 1) * G.stride + G.offX2;
-            // A wave's items (item g to wave g % WA) stream through the ring in steps, as gate | up's rows do.  (Handing the
-            // items of a workgroup out to its waves as they fall free, from a counter in LDS, was measured: the waves of a
-            // workgroup then end together, but the launch ends when its slowest workgroup does, 2-3 us after the mean, as
-            // before -- 0.3511 against 0.3475 ms a token at the 0.5B shape.)
+            // A wave's items (item g to wave g % WA) stream through the ring in steps, as gate | up's rows do, through
+            // explicitly global loads whatever the layers' phases use: the ring's loads stay in flight across the LDS reads
+            // of the steps before them, and the hand-over before the loop does not wait for the first steps' rows (generic
+            // loads here cost the 0.5B shape 2.5 % of its step).
+            // Measured and not kept, both at the 0.5B shape: handing the items of a workgroup out to its waves as they fall
+            // free, from a counter in LDS (the waves of a workgroup then end together, but the launch ends when its slowest
+            // workgroup does, 2-3 us after the mean, as before: 0.3511 against 0.3475 ms a token); and handing the last fifth
+            // of the items out across workgroups, from counters bumped by atomics that stay in an XCD's L2, one claim an item
+            // made a step ahead of its use.  Atomics on one address complete at some 40 a microsecond: one counter an XCD
+            // (256 waves) made the phase 15 us longer, eight an XCD brought the last workgroup 1.5 us closer to the median
+            // and still cost 1.7 % of the step against this static mapping (0.3481 against 0.3422 ms).
             const int nItems = gwA < nItemsAll ? (nItemsAll - gwA + WA - 1) / WA : 0;
             const int nb = (nchD + 64 * CBT - 1) / (64 * CBT);
             const int Tn = nItems * nb;
@@ -1421,8 +1431,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 const int r0 = (gwA + k * WA) * NRT;
 #pragma unroll
                 for (int i = 0; i < NRT; i++)
-                    ld_row<GL, Q4, CBT>(wrow<Q4>(lmW, lmAux, min(r0 + i, vocab - 1), dim), nchD, lane, b * CBT * 64, set[i]);
-                sc = Q4 ? 1.f : ldg_f<GL>(lmAux, min(r0 + (lane < NRT ? lane : 0), vocab - 1));
+                    ld_row<true, Q4, CBT>(wrow<Q4>(lmW, lmAux, min(r0 + i, vocab - 1), dim), nchD, lane, b * CBT * 64, set[i]);
+                sc = Q4 ? 1.f : ldg_f<true>(lmAux, min(r0 + (lane < NRT ? lane : 0), vocab - 1));
             };
             if (Tn > 0) {
 #pragma unroll
@@ -1576,7 +1586,9 @@ hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
         return hipErrorInvalidValue;
     const size_t lds = (size_t)((p.dim > p.ffn ? p.dim : p.ffn) + (p.nTokens > 0 ? p.dim : 0)) * sizeof(float);
     const bool wide = p.dim > 1024, ring = p.dim > 2048, gqa = p.geo.gqa != 0;
-#define FLOW_LAUNCH(HDv, CBv, RGv, GQv, Q4v) hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v>), dim3(grid), dim3(FWG), lds, s, p)
+#define FLOW_LAUNCH(HDv, CBv, RGv, GQv, Q4v) do { \
+        if (p.trace) hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v, true>), dim3(grid), dim3(FWG), lds, s, p); \
+        else hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v, false>), dim3(grid), dim3(FWG), lds, s, p); } while (0)
 #define FLOW_LAUNCH_G(HDv, CBv, RGv) do { \
         if (p.q4) { if (gqa) FLOW_LAUNCH(HDv, CBv, RGv, true, true); else FLOW_LAUNCH(HDv, CBv, RGv, false, true); } \
         else { if (gqa) FLOW_LAUNCH(HDv, CBv, RGv, true, false); else FLOW_LAUNCH(HDv, CBv, RGv, false, false); } } while (0)

@@ -466,4 +466,19 @@ def test_a_wait_that_runs_out_is_reported_and_the_context_goes_on(hip):
     rc, t = m.hip.Generate(prompt, 12, useGraph=True)
     assert rc == 0, E.last_error()
     assert t.tolist() == ref.tolist()
+    # asking for the mode by name arms the launch again; the same with a run of tokens in one launch: every workgroup
+    # gives up its waits, runs through all the run's tokens and exits, and the call reports it
+    assert m.hip.SetExecMode(3) == 0
+    assert _in_use(m.hip) and m.hip.FlowTailInUse()
+    assert m.hip.SetFlowWaitLimit(-1) == 0
+    assert m.hip.ResetKV() == 0
+    rc, _ = m.hip.Generate(prompt, 12, useGraph=True)
+    assert rc != 0 and "persistent" in E.last_error(), (rc, E.last_error())
+    assert not _in_use(m.hip)
+    assert m.hip.SetFlowWaitLimit(5_000_000) == 0
+    assert m.hip.SetExecMode(3) == 0
+    assert m.hip.ResetKV() == 0
+    rc, t = m.hip.Generate(prompt, 12, useGraph=True)
+    assert rc == 0, E.last_error()
+    assert _in_use(m.hip) and t.tolist() == ref.tolist()
     m.close()
