@@ -206,7 +206,9 @@ constexpr int PB = 3;        // float4 pieces a thread polls at once (a round of
 // that one line while its producers are still storing to it.
 // SINGLE (fixed where the kernel variant is chosen): the vector has at most one piece a thread (512 pieces), and the
 // loop asks for one.
-template <bool SINGLE>
+// PAUSE: whether attempts are spaced (see below); the merge of attention partials, which a few lines' worth of threads
+// wait for, asks again at once.
+template <bool SINGLE, bool PAUSE = true>
 __device__ __forceinline__ void poll_batch(const f4* const (&ptr)[PB], f4 (&v)[PB], int n, Waiter& w) {
     static_assert(PB == 3, "the readiness word below names three pieces");
     long long t0 = 0;
@@ -230,10 +232,28 @@ __device__ __forceinline__ void poll_batch(const f4* const (&ptr)[PB], f4 (&v)[P
         else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
         // 256 workgroups re-reading a vector load the lines its producers are still storing to: a pause of ~0.4 us
         // between attempts measures 1 % faster on the whole step than none, and than twice as much
-        for (int z = 0; z < 8; z++) __builtin_amdgcn_s_sleep(2);
+        if (PAUSE) for (int z = 0; z < 8; z++) __builtin_amdgcn_s_sleep(2);
     }
 }
 
+// Maxima and sums of up to PB KV splits of one head, all asked for in one round trip (a thread with fewer splits points
+// the rest at the idle line and ignores them).
+__device__ __forceinline__ void poll_ml(const float* const (&pm)[PB], const float* const (&pl)[PB], float (&m)[PB], float (&l)[PB], int n, Waiter& w) {
+    static_assert(PB == 3, "three splits a round");
+    long long t0 = 0;
+    bool timing = false;
+    for (;;) {
+        asm volatile("global_load_dword %0, %6, off sc1\n\tglobal_load_dword %1, %7, off sc1\n\tglobal_load_dword %2, %8, off sc1\n\t"
+                     "global_load_dword %3, %9, off sc1\n\tglobal_load_dword %4, %10, off sc1\n\tglobal_load_dword %5, %11, off sc1\n\t"
+                     "s_waitcnt vmcnt(0)"
+                     : "=&v"(m[0]), "=&v"(m[1]), "=&v"(m[2]), "=&v"(l[0]), "=&v"(l[1]), "=&v"(l[2])
+                     : "v"(pm[0]), "v"(pm[1]), "v"(pm[2]), "v"(pl[0]), "v"(pl[1]), "v"(pl[2]) : "memory");
+        const unsigned missing = unset1(m[0]) | unset1(l[0]) | (n > 1 ? unset1(m[1]) | unset1(l[1]) : 0u) | (n > 2 ? unset1(m[2]) | unset1(l[2]) : 0u);
+        if (!missing || w.dead) break;
+        if (!timing) { timing = true; t0 = wall_clock64(); }
+        else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
+    }
+}
 // The same for up to eight pieces (the 8B shape's down projection takes 14336 staged values: seven pieces a thread,
 // three rounds of poll_batch -- three dependent round trips; this is one).
 constexpr int PBW = 8;
@@ -1103,16 +1123,41 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                     num.z = num.z * c + wgt * a.z; num.w = num.w * c + wgt * a.w;
                                     M = Mn;
                                 };
-                                for (int s = 0; s < ns; s++) {
+                                // Up to PB splits a round: their accumulator pieces are waited for together (they are spread
+                                // over many lines), then their maxima and sums are fetched together, once the accumulators are
+                                // there -- all heads' maxima and sums of a split share a line, and a line that 50,000 threads
+                                // keep re-reading takes its producer's store late (asked for in the same round as the
+                                // accumulators, by every thread and every attempt, they cost the 0.5B shape 2 us a layer).
+                                // Two round trips after the last partial has landed, however many splits (one by one they
+                                // were one more per split: 4 % of the step at 1000 positions).
+                                const float* idle1 = reinterpret_cast<const float*>(wt.idle);
+                                if (ns == 1) {                             // uniform in the launch; one split: no loads to spare
                                     f4 a;
                                     float ms, ls;
-                                    const f4* pa = reinterpret_cast<const f4*>(X + G.offPacc + (size_t)s * dim) + i;
-                                    // The split everybody has to wait for is waited for on the accumulator pieces alone: they are
-                                    // spread over many lines, while the maxima and sums of all heads share one, and a line that
-                                    // 50,000 threads keep re-reading takes its producer's store late.
-                                    if (s == 0) a = poll4(pa, wt);
-                                    poll_partial(pa, X + G.offPm + s * p.nHeads + h, X + G.offPl + s * p.nHeads + h, a, ms, ls, wt);
+                                    const f4* pa = reinterpret_cast<const f4*>(X + G.offPacc) + i;
+                                    a = poll4(pa, wt);
+                                    poll_partial(pa, X + G.offPm + h, X + G.offPl + h, a, ms, ls, wt);
                                     mergeIn(a, ms, ls);
+                                } else
+                                for (int s0 = 0; s0 < ns; s0 += PB) {
+                                    const int nbt = min(PB, ns - s0);
+                                    const f4* pa[PB];
+                                    const float* pm[PB];
+                                    const float* pl[PB];
+                                    f4 a[PB];
+                                    float ms[PB], ls[PB];
+#pragma unroll
+                                    for (int u = 0; u < PB; u++) {
+                                        const bool on = u < nbt;
+                                        pa[u] = on ? reinterpret_cast<const f4*>(X + G.offPacc + (size_t)(s0 + u) * dim) + i : wt.idle;
+                                        pm[u] = on ? X + G.offPm + (s0 + u) * p.nHeads + h : idle1;
+                                        pl[u] = on ? X + G.offPl + (s0 + u) * p.nHeads + h : idle1;
+                                        a[u] = f4{0.f, 0.f, 0.f, 0.f};
+                                    }
+                                    poll_batch<false, false>(pa, a, nbt, wt);
+                                    poll_ml(pm, pl, ms, ls, nbt, wt);
+#pragma unroll
+                                    for (int u = 0; u < PB; u++) if (u < nbt) mergeIn(a[u], ms[u], ls[u]);
                                 }
                                 const float il = __builtin_amdgcn_rcpf(den);
                                 a4[slot4<Q4>(i, nchD)] = make_float4(num.x * il, num.y * il, num.z * il, num.w * il);
