@@ -220,7 +220,7 @@ __device__ __forceinline__ void poll_batch(const f4* const (&ptr)[PB], f4 (&v)[P
             if (!unset4(v[0]) || w.dead) break;
             if (!timing) { timing = true; t0 = wall_clock64(); }
             else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
-            for (int z = 0; z < 8; z++) __builtin_amdgcn_s_sleep(2);
+            for (int z = 0; z < 4; z++) __builtin_amdgcn_s_sleep(2);
         }
         return;
     }
@@ -230,9 +230,11 @@ __device__ __forceinline__ void poll_batch(const f4* const (&ptr)[PB], f4 (&v)[P
         if (!missing || w.dead) break;
         if (!timing) { timing = true; t0 = wall_clock64(); }
         else if (wall_clock64() - t0 > w.limit) { w.fail(); break; }
-        // 256 workgroups re-reading a vector load the lines its producers are still storing to: a pause of ~0.4 us
-        // between attempts measures 1 % faster on the whole step than none, and than twice as much
-        if (PAUSE) for (int z = 0; z < 8; z++) __builtin_amdgcn_s_sleep(2);
+        // 256 workgroups re-reading a vector load the lines its producers are still storing to, so attempts are spaced;
+        // the space is also the spread of the moments at which the workgroups notice the vector, and the phase ends with
+        // the last of them.  512 clocks (~0.25 us): against 1024, 1.9 % of the step at the 0.5B shape (Q8), 0.45 % at 8B,
+        // nothing at 0.5B Q4_0, -0.3 % at 1.1B; none at all and 256 are within 0.3 % of it at the 0.5B shape.
+        if (PAUSE) for (int z = 0; z < 4; z++) __builtin_amdgcn_s_sleep(2);
     }
 }
 
