@@ -766,20 +766,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             }
                             if (lane == 2 && kd < 2) { const int jj = a0 % half; f0 = cosRow[jj]; f1 = sinRow[jj]; }
                         };
-                        // one item of every wave of the workgroup: dot, epilogue, the results out as runs by wave 0
-                        auto finish = [&](const int4 (&w)[2][CBQ], const WRow (&rw)[2], int kd, float f0, float f1, float rs, int it) {
-                            float acc[2] = {0.f, 0.f};
-                            dot_rows<Q4, 2, CBQ>(w, a4, nchD, lane, 0, acc);
-                            if (nchD > CBQ * 64) dot_rows_tail<GL, Q4, 2, CBQ>(rw, a4, nchD, lane, acc);
-                            const float t = wave_sum2(acc[0], acc[1]);
-                            float v = lane == 1 ? lane_value(t, 32) : t;
-                            v = v * f0;                                                  // row scale (lanes 0 and 1)
-                            v = v * rs;
-                            v = v + f1;
-                            const float v1 = dpp_f<0x101>(v);                            // lane 0 reads lane 1: the pair's second row
-                            const float cs = dpp_f<0x102>(f0), sn = dpp_f<0x102>(f1);    // lane 0 reads lane 2
-                            float o0 = v, o1 = v1;
-                            if (kd < 2) { o0 = v * cs - v1 * sn; o1 = v * sn + v1 * cs; }            // mongoose.cu:991-1006
+                        // the pair of every wave of the workgroup (lane 0: both values) out as runs by wave 0; `it` the wave's item
+                        auto put_pair = [&](float o0, float o1, int it) {
                             // the eight waves' rows are consecutive (first rows of the pairs, and second rows)
                             if (it != gw) __syncthreads();              // outbuf is free again
                             if (lane == 0) { outbuf[0][wave] = o0; outbuf[1][wave] = o1; }
@@ -812,6 +800,90 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                 }
                             }
                         };
+                        // one item of every wave of the workgroup: dot, epilogue, the results out as runs by wave 0
+                        auto finish = [&](const int4 (&w)[2][CBQ], const WRow (&rw)[2], int kd, float f0, float f1, float rs, int it) {
+                            float acc[2] = {0.f, 0.f};
+                            dot_rows<Q4, 2, CBQ>(w, a4, nchD, lane, 0, acc);
+                            if (nchD > CBQ * 64) dot_rows_tail<GL, Q4, 2, CBQ>(rw, a4, nchD, lane, acc);
+                            const float t = wave_sum2(acc[0], acc[1]);
+                            float v = lane == 1 ? lane_value(t, 32) : t;
+                            v = v * f0;                                                  // row scale (lanes 0 and 1)
+                            v = v * rs;
+                            v = v + f1;
+                            const float v1 = dpp_f<0x101>(v);                            // lane 0 reads lane 1: the pair's second row
+                            const float cs = dpp_f<0x102>(f0), sn = dpp_f<0x102>(f1);    // lane 0 reads lane 2
+                            float o0 = v, o1 = v1;
+                            if (kd < 2) { o0 = v * cs - v1 * sn; o1 = v * sn + v1 * cs; }            // mongoose.cu:991-1006
+                            put_pair(o0, o1, it);
+                        };
+                        if constexpr (RING) {
+                            // Rows of more than 2048 weights: a wave's items (one or two row pairs of 16 KB at the 8B shape) stream
+                            // through a ring of register sets in steps of 2 x 128 chunks, as gate | up's rows do, two steps
+                            // requested before the input is waited for and every later one two steps ahead of its use.  Requested
+                            // whole-or-not-at-all (half of the first pair ahead, the rest where it is used) the phase ran into one
+                            // HBM latency after the other: 2 % of the 8B shape's step.
+                            // (Measured and not kept: single rows as items, dealt round the waves evenly -- three rows a wave at
+                            // the 8B shape instead of two pairs on half the waves and one on the others -- with the pairs' halves
+                            // meeting in LDS for the rotation.  HBM is shared by the whole chip, so the waves with two pairs speed
+                            // up once the others are done, and a third round of barriers and stores costs more than the balance
+                            // brings: 1.648 against 1.638 ms a token at 8B, +5 % at the 1.1B shape, whose pairs fit one round and
+                            // whose rows need two.)
+                            constexpr int RD = 3, CB = 2;
+                            int4 ring[RD][2][CB];
+                            float ef0[RD], ef1[RD];                  // the step's item's epilogue operands, as e0 / e1 above
+                            const int nRounds = (nI - (int)blockIdx.x * FWAVES + W - 1) / W;      // items of the workgroup's first wave
+                            const int nb = (nchD + 64 * CB - 1) / (64 * CB);
+                            const int T = nRounds * nb;
+                            auto issueStep = [&](int4 (&set)[2][CB], float& f0, float& f1, int st) {
+                                const int sc2 = min(st, T - 1);                      // past the end: the last step again (uniform loop)
+                                const int k = sc2 / nb, b = sc2 - k * nb;
+                                const int item = min(gw + k * W, nI - 1);            // (a wave past the last item repeats it and stores nothing)
+                                const signed char* Wm; const float* sc; const float* bias; int kd, a0, a1;
+                                if (item < nq) { kd = 0; Wm = L.wq(); sc = L.sq(); bias = L.bq(); const int jj = item % half; a0 = (item - jj) * 2 + jj; a1 = a0 + half; }
+                                else if (item < nq + nk) { kd = 1; Wm = L.wk(); sc = L.sk(); bias = L.bk(); const int i2 = item - nq; const int jj = i2 % half; a0 = (i2 - jj) * 2 + jj; a1 = a0 + half; }
+                                else { kd = 2; Wm = L.wv(); sc = L.sv(); bias = L.bv(); a0 = (item - nq - nk) * 2; a1 = a0 + 1; }
+                                ld_row<true, Q4, CB>(wrow<Q4>(Wm, sc, a0, dim), nchD, lane, b * CB * 64, set[0]);
+                                ld_row<true, Q4, CB>(wrow<Q4>(Wm, sc, a1, dim), nchD, lane, b * CB * 64, set[1]);
+                                f0 = 1.f; f1 = 0.f;
+                                if (lane < 2) {
+                                    const int r = lane ? a1 : a0;
+                                    if (!Q4) f0 = ldg_f<true>(sc, r);
+                                    if (bias) f1 = ldg_f<true>(bias, r);
+                                }
+                                if (lane == 2 && kd < 2) { const int jj = a0 % half; f0 = ldg_f<true>(cosRow, jj); f1 = ldg_f<true>(sinRow, jj); }
+                            };
+#pragma unroll
+                            for (int j = 0; j < RD - 1; j++) issueStep(ring[j], ef0[j], ef1[j], j);
+                            const float rs = stage_rms<GL, Q4, false>(xin, !first, L.g1(), dim, p.eps, a4, red, wt);
+                            FLOW_TRACE(1);
+                            float acc[2] = {0.f, 0.f};
+                            for (int s0 = 0; s0 < T; s0 += RD) {
+#pragma unroll
+                                for (int j = 0; j < RD; j++) {
+                                    const int st = s0 + j;
+                                    issueStep(ring[(j + RD - 1) % RD], ef0[(j + RD - 1) % RD], ef1[(j + RD - 1) % RD], st + RD - 1);
+                                    if (st < T) {                                        // uniform in the workgroup
+                                        const int k = st / nb, b = st - k * nb;
+                                        dot_rows<Q4, 2, CB>(ring[j], a4, nchD, lane, b * CB * 64, acc);
+                                        if (b == nb - 1) {
+                                            const int it = gw + k * W;
+                                            const int kd = it < nq ? 0 : (it < nq + nk ? 1 : 2);
+                                            const float t = wave_sum2(acc[0], acc[1]);
+                                            acc[0] = 0.f; acc[1] = 0.f;
+                                            float v = lane == 1 ? lane_value(t, 32) : t;
+                                            v = v * ef0[j];
+                                            v = v * rs;
+                                            v = v + ef1[j];
+                                            const float v1 = dpp_f<0x101>(v);
+                                            const float cs = dpp_f<0x102>(ef0[j]), sn = dpp_f<0x102>(ef1[j]);
+                                            float o0 = v, o1 = v1;
+                                            if (kd < 2) { o0 = v * cs - v1 * sn; o1 = v * sn + v1 * cs; }            // mongoose.cu:991-1006
+                                            put_pair(o0, o1, it);
+                                        }
+                                    }
+                                }
+                            }
+                        } else {
 #pragma unroll
                         for (int q = 0; q < NPI; q++) {
                             kind[q] = 0; r0[q] = 0; r1[q] = 0; e0[q] = 0.f; e1[q] = 0.f; rows[q][0] = wrow<Q4>(L.wq(), L.sq(), 0, dim); rows[q][1] = rows[q][0];
@@ -825,6 +897,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         for (int it = gw + NPI * W; it - wave < nI; it += W) {         // it - wave: the same for all waves of the workgroup
                             if (it < nI) resolve(wr[0], rows[0], kind[0], r0[0], r1[0], e0[0], e1[0], it);
                             finish(wr[0], rows[0], kind[0], e0[0], e1[0], rs, it);
+                        }
                         }
                     }
                 }
