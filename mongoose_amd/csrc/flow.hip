@@ -583,6 +583,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     __shared__ int4 pfScrap[64];                       // where the prefetching loads land (never read)
     __shared__ float tailV[FWAVES];                    // the tail's argmax: the waves' best values and indices
     __shared__ int tailI[FWAVES];
+    __shared__ unsigned tailCtr;                       // the tail's lm_head: next item of the workgroup to hand out (long rows)
 
     int tid = threadIdx.x, lane = tid & 63;
     int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1176,6 +1177,9 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                 e1 = first ? xin[item] : poll1(xin + item, wt);         // there already if this workgroup staged it for q | k | v
                             }
                         };
+                        // (Long rows streamed through a register ring here as in q | k | v, two steps requested ahead of the merge,
+                        // measure 1.6 % slower at the 8B shape: the merge's polls wait for every load issued before them, and a
+                        // whole row in flight from HBM holds them up longer than the half row does.)
                         if (it < nI) resolve(it);
                         // stage the attention output: merge the KV splits' partials (running maximum, as the split-KV combine)
                         if (grouped) {
@@ -1542,8 +1546,60 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             // made a step ahead of its use.  Atomics on one address complete at some 40 a microsecond: one counter an XCD
             // (256 waves) made the phase 15 us longer, eight an XCD brought the last workgroup 1.5 us closer to the median
             // and still cost 1.7 % of the step against this static mapping (0.3481 against 0.3422 ms).
-            const int nItems = gwA < nItemsAll ? (nItemsAll - gwA + WA - 1) / WA : 0;
             const int nb = (nchD + 64 * CBT - 1) / (64 * CBT);
+            if constexpr (RING) {
+                // Rows of more than 2048 weights (8B shape: 100 us of lm_head): the items of a workgroup -- its waves' first,
+                // second, ... items by the mapping above, numbered q = 8 round + slot -- are handed to its waves as they fall
+                // free, from a counter in LDS, after the two that every wave requests before the input is waited for.  The
+                // waves of a workgroup then end within one item of each other; by the fixed mapping the last wave of the
+                // median workgroup ended 13 us after its first.
+                if (tid == 0) tailCtr = 2 * FWAVES;                   // (stage_rms below has a barrier before any wave claims)
+                auto itemOf = [&](int q) { return (int)blockIdx.x * FWAVES + (q & (FWAVES - 1)) + (q / FWAVES) * WA; };
+                int gI = itemOf(wave), bI = 0, taken = 1;             // the step to issue next: item, block of columns
+                int gS[RDT], bS[RDT];
+                auto issueStep = [&](int4 (&set)[NRT][CBT], float& sc, int& gs, int& bs) {
+                    gs = gI; bs = bI;
+                    const int r0 = min(gI, nItemsAll - 1) * NRT;      // past the end: the last item again (uniform loop)
+#pragma unroll
+                    for (int i = 0; i < NRT; i++)
+                        ld_row<true, Q4, CBT>(wrow<Q4>(lmW, lmAux, min(r0 + i, vocab - 1), dim), nchD, lane, bI * CBT * 64, set[i]);
+                    sc = Q4 ? 1.f : ldg_f<true>(lmAux, min(r0 + (lane < NRT ? lane : 0), vocab - 1));
+                    if (++bI == nb) {
+                        bI = 0;
+                        if (gI < nItemsAll) {                             // (a wave stops at its first item past the end: later claims are later items)
+                            int q = FWAVES * taken + wave;
+                            if (taken >= 2) {
+                                unsigned c = 0;
+                                if (lane == 0) c = __hip_atomic_fetch_add(&tailCtr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                                q = __builtin_amdgcn_readfirstlane((int)c);
+                            }
+                            gI = itemOf(q);
+                            taken++;
+                        }
+                    }
+                };
+#pragma unroll
+                for (int j = 0; j < RDT - 1; j++) issueStep(ring[j], scl[j], gS[j], bS[j]);
+                resetOther();
+                const float rs = stage_rms<GL, Q4, false>(xfin, true, TW_PTR(const float, finalGain), dim, p.eps, a4, red, wt);
+                FLOW_TRACE(1);
+                // (The loop is left at the bottom of a whole round of the ring only: with a way out after every step, the
+                // compiler's count of the loads in flight at the top of a round would be that of the shortest way there, and
+                // its waits would drain the ring.  A wave whose items end inside a round issues the round's other steps idle.)
+                for (bool more = true; more;) {
+#pragma unroll
+                    for (int j = 0; j < RDT; j++) {
+                        constexpr int RDTm = RDT - 1;
+                        issueStep(ring[(j + RDTm) % RDT], scl[(j + RDTm) % RDT], gS[(j + RDTm) % RDT], bS[(j + RDTm) % RDT]);
+                        if (gS[j] < nItemsAll) {                             // uniform in the wave
+                            dot_rows<Q4, NRT, CBT>(ring[j], a4, nchD, lane, bS[j] * CBT * 64, acc);
+                            if (bS[j] == nb - 1) finishItem(gS[j] * NRT, scl[j], rs);
+                        }
+                    }
+                    more = gS[RDT - 1] < nItemsAll;
+                }
+            } else {
+            const int nItems = gwA < nItemsAll ? (nItemsAll - gwA + WA - 1) / WA : 0;
             const int Tn = nItems * nb;
             auto issueStep = [&](int4 (&set)[NRT][CBT], float& sc, int st) {
                 const int s2 = min(st, Tn - 1);                      // past the end: the last step again (uniform loop)
@@ -1559,7 +1615,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 for (int j = 0; j < RDT - 1; j++) issueStep(ring[j], scl[j], j);
             }
             resetOther();
-            const float rs = stage_rms<GL, Q4, !RING>(xfin, true, TW_PTR(const float, finalGain), dim, p.eps, a4, red, wt);
+            const float rs = stage_rms<GL, Q4, true>(xfin, true, TW_PTR(const float, finalGain), dim, p.eps, a4, red, wt);
             FLOW_TRACE(1);
             for (int s0 = 0; s0 < Tn; s0 += RDT) {
 #pragma unroll
@@ -1572,6 +1628,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         if (b == nb - 1) finishItem((gwA + k * WA) * NRT, scl[j], rs);
                     }
                 }
+            }
             }
             FLOW_TRACE(2);
             // argmax exchange: the workgroup's best (value, lowest index) goes out once its own stores (the reset above among
