@@ -92,6 +92,9 @@ struct FlowParams {
     int nTokens;                 // 0: layers [l0, l1) of one step, hidden in and out; n >= 1: token mode -- n whole tokens from the
                                  // device state on (all layers; xchg holds two halves and the argmax exchange; state != NULL)
     const FlowTail* tail;        // token mode
+    int gqaCode;                 // geo.gqa only: 1 = a position of this launch may need the grouped attention (the variant that can do
+                                 // it is launched); 0 = none does (positions below nCompute / nHeads tiles): the plain variant, which
+                                 // is faster there, runs on the same geometry and reports a position past its reach as error 3
 };
 #define FLOW_TAIL_TRACE_NAMES "tail-top", "final-input-staged", "lm-head-done", "token-known", "all-waves-done", "partials-in"
 

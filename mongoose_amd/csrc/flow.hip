@@ -651,6 +651,12 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
         asm volatile("" : "+s"(wave), "+s"(gw), "+s"(dim), "+s"(kvDim), "+s"(ffn), "+s"(nchD), "+s"(nchF));
         float* const xb = p.xchg + (tokens ? (size_t)(pos & 1) * halfFloats : (size_t)0);
         const unsigned xoff = tokens ? (unsigned)((size_t)(pos & 1) * halfFloats) : 0u;
+        if constexpr (!GQA) {
+            // the plain variant on a geometry laid out for grouped attention: a position past what a workgroup per query head
+            // and split covers is the host's mistake, and is reported instead of computed wrongly
+            if (G.gqa && p.nHeads * (pos / TILE + 1) > nC && blockIdx.x == 0 && tid == 0)
+                __hip_atomic_store(p.err, 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         const float* cosRow = p.cosRow;
         const float* sinRow = p.sinRow;
         if (tokens) {
@@ -1762,7 +1768,7 @@ hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
                           flow_lds_bytes(p.dim, p.ffn, p.headDim, p.geo.gqa, true) > ((size_t)160 << 10)))
         return hipErrorInvalidValue;
     const size_t lds = (size_t)((p.dim > p.ffn ? p.dim : p.ffn) + (p.nTokens > 0 ? p.dim : 0)) * sizeof(float);
-    const bool wide = p.dim > 1024, ring = p.dim > 2048, gqa = p.geo.gqa != 0;
+    const bool wide = p.dim > 1024, ring = p.dim > 2048, gqa = p.geo.gqa != 0 && p.gqaCode != 0;
 #define FLOW_LAUNCH(HDv, CBv, RGv, GQv, Q4v) do { \
         if (p.trace) hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v, true>), dim3(grid), dim3(FWG), lds, s, p); \
         else hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v, false>), dim3(grid), dim3(FWG), lds, s, p); } while (0)

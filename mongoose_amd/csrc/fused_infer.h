@@ -179,6 +179,8 @@ public:
     bool FlowInUse() const { return flowEligible(0, nLayers); }
     long long flowLimitTicks = 5000000;       // per wait of the persistent launch: 50 ms of the 100 MHz wall clock
     void SetFlowWaitLimit(long long ticks) { invalidateGraphs(); flowLimitTicks = ticks; }
+    int statePosHost = -1;                    // the device state's position where the host knows it (set with the state, advanced
+                                              // with whole tokens run in the persistent launch), else -1
     // Whole tokens inside the persistent launch (embedding, layers, final norm, lm_head, argmax): on where the model
     // allows it; tokensPerLaunch of them in one launch where a caller asks for a run of tokens (Generate, TimedDecode,
     // GeneratePrefill), 1 = a launch (or a graph replay) per token.

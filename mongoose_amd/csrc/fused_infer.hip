@@ -876,6 +876,16 @@ int HIPFusedInference::enqueueLayersFlow(int l0, int l1, const StepState* st, in
     p.xchg = flowXchg; p.geo = flowGeo;
     p.err = dFlowErr;
     p.limitTicks = flowLimitTicks;
+    {
+        // the last position this launch can reach, where the host knows it: the plain attention variant serves while a
+        // workgroup per query head and KV split fits the launch, also in a context laid out for grouped attention
+        long long posMax = -1;
+        if (!st) posMax = posImm;
+        else if (statePosHost >= 0) posMax = (long long)statePosHost + (nTokens > 0 ? nTokens - 1 : 0);
+        p.gqaCode = (posMax < 0 || (long long)nHeads * (posMax / FLOW_TILE + 1) > flowCompute) ? 1 : 0;
+        if (st && nTokens > 0 && statePosHost >= 0) statePosHost += nTokens;          // whole tokens advance the device state
+        else if (st) statePosHost = -1;                                               // (what follows this launch advances it)
+    }
     p.trace = flowTrace;
     if (nTokens > 0) { p.nTokens = nTokens; p.tail = dFlowTail; }
     if (resetFirst) HIPCHK(launch_flow_reset(flowXchg, flowGeo, l0, l1, stream));
@@ -913,6 +923,7 @@ int HIPFusedInference::SetTokensPerLaunch(int n) {
 // reset (a token expects the half of its position's parity so, and resets the other for its successor).
 int HIPFusedInference::setState(int pos, int token, int count, int nPrompt) {
     HIPCHK(launch_set_state(dState, pos, token, count, nPrompt, ropeRef(), stream));
+    statePosHost = pos;
     if (flowXchg && (execMode == 3 || execMode == 4)) HIPCHK(launch_flow_reset_all(flowXchg, flowGeo, nLayers, flowGrid, stream));
     return MG_OK;
 }
@@ -932,6 +943,7 @@ int HIPFusedInference::decodeRun(int nTokens, bool useGraph) {
         return rc;
     }
     for (int i = 0; i < nTokens; i++) {
+        statePosHost = -1;                          // (advanced on the device by launches that do not tell the host)
         if (useGraph) HIPCHK(hipGraphLaunch(execFull, stream));
         else { int rc = enqueueToken(true); if (rc) return rc; }
     }
@@ -945,14 +957,19 @@ int HIPFusedInference::checkFlowError() {
     if (!dFlowErr) return MG_OK;
     HIPCHK(hipMemcpy(hFlowErr, dFlowErr, sizeof(int), hipMemcpyDeviceToHost));
     if (*hFlowErr == 0) return MG_OK;
+    const int code = *hFlowErr;
     *hFlowErr = 0;
     HIPCHK(hipMemsetAsync(dFlowErr, 0, sizeof(int), stream));
     HIPCHK(hipStreamSynchronize(stream));
     flowBroken = true;
     releaseFlow();
     invalidateGraphs();
-    set_error("persistent layer launch: a wait between phases ran into its time limit (workgroups not all resident at once?); "
-              "this step's results are invalid, later steps use the separate launches");
+    if (code == 3)
+        set_error("persistent layer launch: the variant without grouped attention was given a position it does not cover; "
+                  "this step's results are invalid, later steps use the separate launches");
+    else
+        set_error("persistent layer launch: a wait between phases ran into its time limit (workgroups not all resident at once?); "
+                  "this step's results are invalid, later steps use the separate launches");
     return MG_E_HIP;
 }
 
@@ -971,6 +988,7 @@ int HIPFusedInference::enqueueLayer(const LayerWeights& L, int layer, const Step
 // Final norm + lm_head (cuda_fused_infer.go:446-448) with the per-workgroup
 // argmax folded into the matvec epilogue.
 int HIPFusedInference::enqueueFinal(bool withArgmax) {
+    if (withArgmax) statePosHost = -1;              // (the argmax's last kernel advances the device state)
     if (!finalNorm || !lmHead.w) { set_error("final norm / lm_head not set"); return MG_E_STATE; }
     if (execMode == 0 && q4ActQuant && lmHead.kind == WF_Q4P) {
         // the reference's tail with its integer matvec (cuda_fused_infer_q4.go:600-601): norm, quantize, lm_head; then
@@ -1189,6 +1207,7 @@ int HIPFusedInference::enqueueToken(bool withHead) {
         }
     }
     if (withHead) return enqueueFinal(true);
+    statePosHost = -1;
     HIPCHK(launch_advance_prompt(dState, dPrompt, ropeRef(), embedRef(), stream));
     // no lm_head launch to leave the exchange area reset for the next launch: a captured prompt step does it itself,
     // and so does any prompt step where whole tokens run in the launch (they expect to find it so)
@@ -1240,6 +1259,7 @@ int HIPFusedInference::GraphCapture() {
     graphsUseFlow = flow;
     if (flow) { rc = ensureFlow(); if (rc) return rc; }     // allocations and uploads come before the capture
     HIPCHK(hipStreamSynchronize(stream));
+    statePosHost = -1;                              // a captured launch is replayed at any position: the variant that covers all
     for (int which = 0; which < 2; which++) {
         HIPCHK(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));
         fuseEmbed = true;
@@ -1271,6 +1291,7 @@ int HIPFusedInference::LayerGraphCapture(LayerGraph& lg) {
     const bool flow = flowEligible(lg.l0, lg.l1);
     if (flow) { int rc = ensureFlow(); if (rc) return rc; }          // allocations and uploads come before the capture
     HIPCHK(hipStreamSynchronize(stream));
+    statePosHost = -1;                              // (replayed at any position)
     HIPCHK(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));
     int rc = MG_OK;
     if (flow) rc = enqueueLayersFlow(lg.l0, lg.l1, dState, 0, true);
@@ -1295,6 +1316,7 @@ int HIPFusedInference::LayerGraphLaunch(LayerGraph& lg, int pos) {
         if (rc) return rc;
     }
     HIPCHK(launch_set_state(dState, pos, 0, 0, 0, ropeRef(), stream));
+    statePosHost = -1;
     HIPCHK(hipGraphLaunch(lg.ex, stream));
     return MG_OK;
 }
@@ -1349,6 +1371,7 @@ int HIPFusedInference::GraphLaunch(int token, int pos, int* nextToken) {
     { int rcs = setState(pos, token, 0, 0); if (rcs) return rcs; }
     rc = primeGraph();
     if (rc) return rc;
+    statePosHost = -1;
     HIPCHK(hipGraphLaunch(execFull, stream));
     HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int), hipMemcpyDeviceToHost, stream));
     HIPCHK(hipStreamSynchronize(stream));
@@ -1405,6 +1428,7 @@ int HIPFusedInference::Generate(const int* prompt, int nPrompt, int nDecode, int
         if (graphs) HIPCHK(hipGraphLaunch(execPrompt, stream));
         else { rc = enqueueToken(false); if (rc) return rc; }
     }
+    statePosHost = nPrompt - 1;                     // one position a prompt step since setState(0, ..)
     rc = decodeRun(nDecode, useGraph);
     if (rc) return rc;
     if (nDecode > 0) HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int) * (size_t)nDecode, hipMemcpyDeviceToHost, stream));
@@ -1608,6 +1632,7 @@ int HIPFusedInference::Prefill(const int* tokens, int nTokens, int pos0, int* ne
     { int rcs = setState(pos0 + T - 1, tokens[T - 1], 0, 0); if (rcs) return rcs; }
     rc = enqueueFinal(true);
     if (rc) return rc;
+    statePosHost = pos0 + T;                        // where the argmax's last kernel leaves the state
     HIPCHK(hipEventRecord(ev1, stream));
     HIPCHK(hipMemcpyAsync(hTokens, dHistory, sizeof(int), hipMemcpyDeviceToHost, stream));
     HIPCHK(hipStreamSynchronize(stream));

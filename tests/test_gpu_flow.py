@@ -170,6 +170,13 @@ def test_kv_splits_heads_of_64(hip):
     _modes_agree(m, m.prompt(100), 30, "grouped, 1 split")
     _modes_agree(m, m.prompt(2990), 30, "grouped, 24 splits")
     _modes_agree(m, m.prompt(5950), 40, "grouped, 47 splits")
+    # The launch is handed the attention variant its positions need: the plain one (a workgroup per query head and split)
+    # while 14 heads x splits fit the 256 workgroups, i.e. up to position 2303, the grouped one from there on.  Launches of
+    # 8 tokens from position 2290: the first is plain, the second crosses the boundary inside the launch, the rest are
+    # grouped; the same run as launches of 64 tokens is grouped throughout.
+    for n in (8, 64):
+        assert m.hip.SetTokensPerLaunch(n) == 0
+        _modes_agree(m, m.prompt(2290), 40, f"plain to grouped at position 2304, {n} tokens a launch")
     m.close()
     # 2 KV heads x 128 positions x 128 workgroup rows = 16384 positions at most
     m = H.Model(s, seed=11, maxSeq=16385, eng=hip, oracle=False)
