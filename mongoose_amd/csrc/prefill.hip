@@ -480,7 +480,8 @@ constexpr int B_STRIDE = BK + 16;   // bytes per LDS row of int8 weights (80)
 
 __device__ __forceinline__ unsigned pack_bf16_exact(float lo, float hi) {
     // both floats hold small integers: their low 16 bits are zero, truncation is exact
-    return (__builtin_bit_cast(unsigned, lo) >> 16) | (__builtin_bit_cast(unsigned, hi) & 0xffff0000u);
+    // (one v_perm_b32: bytes 2, 3 of lo, then bytes 2, 3 of hi)
+    return __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, hi), __builtin_bit_cast(unsigned, lo), 0x07060302u);
 }
 
 // Workgroup tile BM x BN with NT threads: NT/64 waves as (NT/64)/(BN/64) x (BN/64), each wave
@@ -770,6 +771,11 @@ constexpr int RK = 32, RS = 3;
 constexpr int RING_PLANE = 256 * 64;                      // 256 rows x 32 bf16
 constexpr int RING_STAGE_BYTES = 3 * RING_PLANE;          // A hi, A lo, W as bf16
 
+// the 32-bit LDS address of a pointer into __shared__ memory
+__device__ __forceinline__ unsigned lds_offset(const void* p) {
+    return (unsigned)(size_t)(__attribute__((address_space(3))) const void*)p;
+}
+
 __device__ __forceinline__ bf16x8_t cvt8_i8_bf16(int lo, int hi) {
     uint4 u;
     u.x = pack_bf16_exact((float)(signed char)(lo), (float)(signed char)(lo >> 8));
@@ -835,10 +841,25 @@ __global__ __launch_bounds__(512) void gemm_q8_ring_kernel(GemmParams p) {
         const int st = min(step, ksteps - 1);            // past the end: a harmless reload that keeps the counters uniform
         unsigned char* base = ring + stage * RING_STAGE_BYTES + wave * 2048;
         const size_t ko = (size_t)(st >> 1) * 8192 + (st & 1) * 32;
-        __builtin_amdgcn_global_load_lds(p.Ahi + aOff[0] + ko, reinterpret_cast<int4*>(base), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(p.Ahi + aOff[1] + ko, reinterpret_cast<int4*>(base + 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(p.Alo + aOff[0] + ko, reinterpret_cast<int4*>(base + RING_PLANE), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(p.Alo + aOff[1] + ko, reinterpret_cast<int4*>(base + RING_PLANE + 1024), 16, 0, 0);
+        if constexpr (MODE == 3) {
+            // A uniform base in scalar registers and a 32-bit byte offset a lane that never changes: written out, because the
+            // compiler's own form of this load adds the two in vector registers for every load (the matrix pipe and the other
+            // vector instructions of a SIMD do not overlap, so those additions came out of the multiplications' time).  M0
+            // carries the LDS address of the wave's first slot.
+            const unsigned short* ah = p.Ahi + ko;
+            const unsigned short* al = p.Alo + ko;
+            const unsigned l0 = lds_offset(base);
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(l0), "v"(aOff[0] * 2u), "s"(ah));
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(l0 + 1024u), "v"(aOff[1] * 2u), "s"(ah));
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(l0 + (unsigned)RING_PLANE), "v"(aOff[0] * 2u), "s"(al));
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(l0 + (unsigned)RING_PLANE + 1024u), "v"(aOff[1] * 2u), "s"(al));
+        } else {
+            // (K split or short launches: the compiler's form of the same loads schedules better there -- measured)
+            __builtin_amdgcn_global_load_lds(p.Ahi + aOff[0] + ko, reinterpret_cast<int4*>(base), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(p.Ahi + aOff[1] + ko, reinterpret_cast<int4*>(base + 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(p.Alo + aOff[0] + ko, reinterpret_cast<int4*>(base + RING_PLANE), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(p.Alo + aOff[1] + ko, reinterpret_cast<int4*>(base + RING_PLANE + 1024), 16, 0, 0);
+        }
     };
     auto loadW = [&](int step) __attribute__((always_inline)) {
         return *reinterpret_cast<const int4*>(bG + (size_t)min(step, ksteps - 1) * RK);
@@ -903,6 +924,50 @@ __global__ __launch_bounds__(512) void gemm_q8_ring_kernel(GemmParams p) {
 
     // C layout of the 16 x 16 blocks: lane l holds column l%16, rows 4*(l/16) + e
     const int mrow = m0 + wm * 64 + 4 * (lane >> 4);
+    if (MODE == 3 && n0 + 128 <= N) {
+        // A whole tile of columns: the 256 x 128 results are the four 128-row x 64-k blocks (rb, kb) of each split plane,
+        // 16 KB of consecutive addresses each.  They are gathered in the ring's LDS in that order (the 32-byte pair of
+        // pieces of a row XOR-ed with row bits, so that the four row groups of a wave's store fall into different banks)
+        // and leave as whole rows of 128 bytes, 16 bytes a lane -- not as 2-byte stores to four rows an instruction.
+        __syncthreads();                                  // every wave is through with the last stage
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const int jg = (jj >> 1) * 4 + (jj & 1);      // gate blocks 0, 1, 4, 5; the up values of the same columns in jg + 2
+            const int c = (wn * 2 + (jj >> 1)) * 32 + (jj & 1) * 16 + (lane & 15);
+            const int n = n0 + c;
+            const float scg = p.seg[0].scales[n], scu = p.seg[1].scales[n];
+            const float big = p.seg[0].bias ? p.seg[0].bias[n] : 0.f, biu = p.seg[1].bias ? p.seg[1].bias[n] : 0.f;
+            const int kb = c >> 6, pc = (c & 63) >> 3;    // 64-k block of the column, its 16-byte piece there
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int r = wm * 64 + i * 16 + 4 * (lane >> 4) + e;          // row of the tile
+                    const float g = acc[i][jg][e] * scg + big, u = acc[i][jg + 2][e] * scu + biu;
+                    const float a = g * (1.0f / (1.0f + expf(-g))) * u;            // mongoose.cu:949-956
+                    const unsigned short h = f32_to_bf16_rne(a);
+                    const int rl = r & 127;
+                    const unsigned o = ((r >> 7) * 2 + kb) * 16384 + rl * 128 + ((((pc >> 1) ^ ((rl >> 2) & 3)) << 1) | (pc & 1)) * 16 + (c & 7) * 2;
+                    *reinterpret_cast<unsigned short*>(ring + o) = h;
+                    *reinterpret_cast<unsigned short*>(ring + 65536 + o) = f32_to_bf16_rne(a - bf16_to_f32(h));
+                }
+        }
+        __syncthreads();
+        const int ksN = (N + 63) >> 6;
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            const int ch = q * 512 + tid;                 // 16-byte chunk: plane, block, row, piece
+            const int plane = ch >> 12, blk = (ch >> 10) & 3, off = ch & 1023;
+            const int rl = off >> 3, pc = off & 7;
+            const int rbG = (m0 >> 7) + (blk >> 1);
+            if (rbG * 128 >= planeRows) continue;         // (uniform in the wave: a chunk row is 8 lanes)
+            const uint4 v = *reinterpret_cast<const uint4*>(ring + plane * 65536 + blk * 16384 + rl * 128 +
+                                                            ((((pc >> 1) ^ ((rl >> 2) & 3)) << 1) | (pc & 1)) * 16);
+            unsigned short* dst = (plane ? p.nextLo : p.nextHi) + ((size_t)rbG * ksN + (n0 >> 6) + (blk & 1)) * 8192 + (size_t)off * 8;
+            *reinterpret_cast<uint4*>(dst) = v;
+        }
+        return;
+    }
     if (MODE == 3) {
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
