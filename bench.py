@@ -42,10 +42,10 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
 # NOT measured by the run that prints them: "traffic_source" in the output says so.
 PMC_TRAFFIC_BYTES = {
     # the launch that runs whole tokens: bytes a TOKEN (all timed launches' counters over their tokens)
-    ("qwen2.5-0.5b", "token"): int(((16440188.1 + 16839402.9 + 17246984.3 + 2182704.8) * (262144.0 / 131090.4)
-                                    + (166748.1 + 168323.0 + 173509.0 + 21708.8)) * 1024 / 200),
-    ("tinyllama-1.1b", "token"): int((26373655.1 * (262144.0 / 131090.4) + 144828.2) * 1024 / 50),
-    ("llama-3-8b", "token"): int((240153544.6 * (262144.0 / 131090.4) + 625353.5) * 1024 / 64),
+    ("qwen2.5-0.5b", "token"): int(((16432663.6 + 16825804.6 + 17254655.8 + 2184860.8) * (262144.0 / 131090.0)
+                                    + (167463.2 + 168969.3 + 174229.8 + 21776.3)) * 1024 / 200),
+    ("tinyllama-1.1b", "token"): int((26419379.1 * (262144.0 / 131090.0) + 144818.5) * 1024 / 50),
+    ("llama-3-8b", "token"): int((239340691.1 * (262144.0 / 131090.0) + 621317.0) * 1024 / 64),
     # separate launches (--no-flow-tail, --exec-mode 1): bytes a launch
     ("qwen2.5-0.5b", "lm_head"): int((67135.1 * (262144.0 / 131102.4) + 660.5 * 1.0) * 1024),
     ("qwen2.5-0.5b", "flow"): int((190867.0 * (262144.0 / 131102.4) + 952.0 * 1.0) * 1024),
