@@ -153,6 +153,15 @@ def test_prefill_llama3_shape_two_row_tiles(hip):
     m.close()
 
 
+def test_prefill_wide_ffn_with_a_partial_column_tile(hip):
+    """An FFN of 80.5 tiles of 128 columns at 300 rows: the gate|up GEMM runs unsplit on the 256 x 256 tiles and forms
+    silu(gate)*up itself.  Whole tiles leave through LDS as 128-byte rows (row blocks past the planes' 384 rows are
+    skipped), the last tile has 64 columns and stores element by element; the down projection then reads both."""
+    s = configs.Shape("ffn-edge", 1, 256, 4, 2, 64, 10304, 512, 1e-5, 1e4, False, True, "q8")
+    m, _, _ = _prefill_case(hip, s, seed=21, nPrompt=300, nDecode=2, maxSeq=320)
+    m.close()
+
+
 def test_prefill_fp16_kv(hip):
     """Prefill writing fp16 KV rows (head sizes 64 and 128) against the oracle with the same rounding."""
     m, _, _ = _prefill_case(hip, H.with_layers(configs.QWEN, 2), seed=7, nPrompt=70, nDecode=6, maxSeq=96, kv_f16=True)
