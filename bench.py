@@ -38,8 +38,11 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
 # KiB per dispatch), each scaled by what the same counter reads for a 256 MiB device copy in
 # the same run (FETCH_SIZE reads 131090-131102 KiB for the 262144 KiB copied -> x1.9995-1.9997;
 # WRITE_SIZE reads 262144.0 -> x1.0).  Counts are a property of kernel and shape, so they are recorded
-# here, keyed by (configuration, launch); profiles/ holds the runs they come from.  They are
-# NOT measured by the run that prints them: "traffic_source" in the output says so.
+# here, keyed by (configuration, launch); profiles/ holds the runs they come from.  The default run
+# measures the headline launch's traffic itself (live_pmc_traffic: the same two passes as children of this
+# process) and reports the recorded figure beside it; where it cannot (a flag that leaves the default path,
+# no rocprofv3, a pass that fails) and for the other configurations the recorded figures are reported, and
+# "traffic_source" / "traffic_note" in the output say which it was.
 PMC_TRAFFIC_BYTES = {
     # the launch that runs whole tokens: bytes a TOKEN (all timed launches' counters over their tokens)
     ("qwen2.5-0.5b", "token"): int(((16432663.6 + 16825804.6 + 17254655.8 + 2184860.8) * (262144.0 / 131090.0)
@@ -53,6 +56,63 @@ PMC_TRAFFIC_BYTES = {
     ("llama-3-8b", "flow"): int((3510548.2 * (262144.0 / 131102.4) + 4432.0 * 1.0) * 1024),
 }
 PMC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script recorded in profiles/ (constants in bench.py, not measured by this run)"
+
+
+
+def live_pmc_traffic(config, steps, warmup, timeout_s=150):
+    """HBM bytes of the token launches of THIS build on THIS box: two rocprofv3 --pmc passes (FETCH_SIZE, then WRITE_SIZE --
+    together they need more counters of one block than a pass holds) over `bench.py --lean --pmc-copy`, run as child
+    processes before this process touches the GPU.  Returns (dict, None) or (None, reason)."""
+    import csv
+    import shutil
+    import signal
+    import subprocess
+    import tempfile
+    exe = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    if not os.path.exists(exe):
+        return None, "rocprofv3 not found"
+    tmp = tempfile.mkdtemp(prefix="mg_pmc_", dir="/tmp")
+    env = dict(os.environ, TMPDIR="/tmp")
+    got = {}
+    try:
+        for ctr in ("FETCH_SIZE", "WRITE_SIZE"):
+            cmd = [exe, "--pmc", ctr, "--output-format", "csv", "-d", tmp, "-o", ctr.lower(), "--",
+                   sys.executable, os.path.join(ROOT, "bench.py"), "--lean", "--pmc-copy", "--config", config,
+                   "--steps", str(steps), "--warmup", str(warmup)]
+            print(f"bench.py: rocprofv3 --pmc {ctr} pass", file=sys.stderr, flush=True)
+            proc = subprocess.Popen(cmd, cwd=ROOT, env=env, stdout=subprocess.DEVNULL, stderr=subprocess.PIPE,
+                                    start_new_session=True, text=True)
+            try:
+                _, err = proc.communicate(timeout=timeout_s)
+            except subprocess.TimeoutExpired:
+                os.killpg(proc.pid, signal.SIGKILL)
+                proc.communicate()
+                return None, f"rocprofv3 --pmc {ctr} pass did not end within {timeout_s} s"
+            if proc.returncode != 0:
+                return None, f"rocprofv3 --pmc {ctr} pass ended with status {proc.returncode}: {(err or '').strip()[-200:]}"
+            path = None
+            for dp, _, files in os.walk(tmp):
+                for fn in files:
+                    if fn == f"{ctr.lower()}_counter_collection.csv":
+                        path = os.path.join(dp, fn)
+            if path is None:
+                return None, f"no counter file from the {ctr} pass"
+            launch, copies = [], []
+            for r in csv.DictReader(open(path)):
+                if r.get("Counter_Name") != ctr:
+                    continue
+                v = float(r["Counter_Value"])
+                if "flow_layers_kernel" in r["Kernel_Name"]:
+                    launch.append(v)
+                elif "copyBuffer" in r["Kernel_Name"] and v > 65536:
+                    copies.append(v)
+            if not launch or not copies:
+                return None, f"{ctr} pass: no dispatch of the launch or of the 256 MiB copies in the counter file"
+            got[ctr] = (launch, 262144.0 / (sum(copies) / len(copies)))
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    return got, None
+
 
 LAUNCH_NAMES = {0: "embed_gather", 1: "norm+qkv", 2: "rope+kvwrite+attention", 3: "wo+residual", 4: "norm+gate_up+swiglu",
                 5: "down+residual", 6: "norm+lm_head+argmax_partials", 7: "argmax_finish"}
@@ -491,6 +551,9 @@ def main():
     ap.add_argument("--lean", action="store_true",
                     help="only the timed region of the configuration (no per-launch tables, no graph-replay leg, no trace, no "
                          "token check): the run to put under rocprofv3")
+    ap.add_argument("--no-live-pmc", action="store_true",
+                    help="do not run the two rocprofv3 --pmc passes that measure the launch's HBM traffic (the figures recorded "
+                         "from profiles/ are reported instead)")
     ap.add_argument("--no-configs", action="store_true",
                     help="only the configuration named by --config (no 'configs' object with the other benchmark configurations)")
     args = ap.parse_args()
@@ -498,6 +561,14 @@ def main():
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
               "the decode path is batch-1 on a single device", file=sys.stderr)
         sys.exit(2)
+
+    # HBM traffic of the run's own launches, from counters: before anything here touches the GPU (the profiler runs
+    # children of this process).  Only for the default path, whose dispatches the passes can pick out.
+    pmc_live, pmc_why = None, "not the default path (flags)"
+    default_path = (not args.lean and args.exec_mode < 0 and not args.no_flow_tail and args.context == 0 and args.kv == "f32"
+                    and not args.tokens_per_launch and not args.no_graph and not args.pmc_copy)
+    if default_path and not args.no_live_pmc:
+        pmc_live, pmc_why = live_pmc_traffic(args.config, args.steps, max(args.warmup, 1))
 
     import numpy as np
     from mongoose_amd import configs
@@ -547,6 +618,21 @@ def main():
                     "traffic": int(tr_b * K / launches) if tr_b else None,
                     "traffic_source": PMC_SOURCE if tr_b else None,
                     "traffic_note": None if tr_b else "not collected for this kernel"}
+        if pmc_live and all(len(pmc_live[c][0]) >= launches for c in pmc_live):
+            # the timed launches are the last `launches` dispatches of the kernel in each pass (the same command line)
+            fe, ff = pmc_live["FETCH_SIZE"]
+            wr, wf = pmc_live["WRITE_SIZE"]
+            tb = (sum(fe[-launches:]) * ff + sum(wr[-launches:]) * wf) * 1024.0 / launches
+            roofline["traffic_recorded"] = roofline["traffic"]
+            roofline["traffic"] = int(tb)
+            roofline["traffic_over_algorithmic"] = round(tb / b, 4)
+            roofline["traffic_source"] = ("measured by this run: rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE passes over `bench.py --lean "
+                                          "--pmc-copy` with this configuration, made before the timing (same build, same box); KiB per dispatch of "
+                                          f"the timed launches, scaled by what the same counters read for 256 MiB device copies (x{ff:.4f} / x{wf:.4f})")
+            roofline["traffic_note"] = None
+        elif not args.lean:
+            roofline["traffic_note"] = ((roofline["traffic_note"] + "; ") if roofline["traffic_note"] else "") + \
+                f"no live counter passes: {pmc_why or 'fewer dispatches in the counter files than timed launches'}"
         ph = run.get("in_launch_phases") or {}
         lmh = ph.get("lm_head")
         sep = [e for e in (run.get("kernels_fused_launches") or []) if e["cls"] == 6]
