@@ -59,7 +59,7 @@ PMC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script record
 
 
 
-def live_pmc_traffic(config, steps, warmup, timeout_s=150):
+def live_pmc_traffic(config, steps, warmup, timeout_s=100):
     """HBM bytes of the token launches of THIS build on THIS box: two rocprofv3 --pmc passes (FETCH_SIZE, then WRITE_SIZE --
     together they need more counters of one block than a pass holds) over `bench.py --lean --pmc-copy`, run as child
     processes before this process touches the GPU.  Returns (dict, None) or (None, reason)."""
