@@ -357,7 +357,7 @@ def check_tokens(E, orc, prompt, toks, budget_s):
 
 def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_graph=True, exec_mode=None, kv_f16=False,
             prefill=0, oracle_threads=0, check_budget_s=8.0, want_mode1_table=True, keep=False, tokens_per_launch=None,
-            want_phases=True, flow_tail=True, stream_tokens=0, lean=False):
+            want_phases=True, flow_tail=True, stream_tokens=0, lean=False, flow_generic=False):
     """One configuration: load, warm up on the W prompt positions, time K decode steps at each start position of
     `contexts` (0 = right after the prompt), per-launch table, optional batched prefill, optional token check."""
     from oracle import binding as ob
@@ -368,6 +368,8 @@ def measure(E, np, configs, eng, s, seed, W, K, contexts, profile_steps, use_gra
     f = load_model(E, np, s, seed, maxSeq, eng, oracle=orc, kv_f16=kv_f16)
     if exec_mode is not None and f.SetExecMode(exec_mode) != 0:
         raise SystemExit("bench.py: " + E.last_error())
+    if flow_generic:
+        assert f.SetFlowGeneric(True) == 0
     if not flow_tail:
         f.SetFlowTail(False)
     t_load = time.perf_counter() - t_load
@@ -551,6 +553,9 @@ def main():
     ap.add_argument("--lean", action="store_true",
                     help="only the timed region of the configuration (no per-launch tables, no graph-replay leg, no trace, no "
                          "token check): the run to put under rocprofv3")
+    ap.add_argument("--flow-generic", action="store_true",
+                    help="only the persistent launch's variants whose sizes come with the launch (for comparisons with the "
+                         "variants that have a known shape's sizes compiled in)")
     ap.add_argument("--no-live-pmc", action="store_true",
                     help="do not run the two rocprofv3 --pmc passes that measure the launch's HBM traffic (the figures recorded "
                          "from profiles/ are reported instead)")
@@ -566,7 +571,7 @@ def main():
     # children of this process).  Only for the default path, whose dispatches the passes can pick out.
     pmc_live, pmc_why = None, "not the default path (flags)"
     default_path = (not args.lean and args.exec_mode < 0 and not args.no_flow_tail and args.context == 0 and args.kv == "f32"
-                    and not args.tokens_per_launch and not args.no_graph and not args.pmc_copy)
+                    and not args.tokens_per_launch and not args.no_graph and not args.pmc_copy and not args.flow_generic)
     if default_path and not args.no_live_pmc:
         pmc_live, pmc_why = live_pmc_traffic(args.config, args.steps, max(args.warmup, 1))
 
@@ -586,7 +591,7 @@ def main():
     res, f, prompt, first, toks = measure(E, np, configs, eng, s, args.seed, W, K, [args.context], args.profile_steps,
                                           use_graph=use_graph, exec_mode=mode, kv_f16=kv_f16, prefill=args.prefill,
                                           oracle_threads=0, keep=not args.lean or True, tokens_per_launch=args.tokens_per_launch or None,
-                                          flow_tail=not args.no_flow_tail, lean=args.lean)
+                                          flow_tail=not args.no_flow_tail, lean=args.lean, flow_generic=args.flow_generic)
     run = res["runs"][0]
     P0 = run["start_position"]
     ms_per_step = run["ms_per_step"]

@@ -416,6 +416,11 @@ int mg_flow_trace(mg_ctx* ctx, int enable, long long* out, size_t cap, int* dims
  * {6, workgroups}.  No counterparts in the reference. */
 int mg_set_flow_tail(mg_ctx* ctx, int on);
 int mg_set_tokens_per_launch(mg_ctx* ctx, int n);
+/* The persistent launch has variants with the sizes of known model shapes compiled in (Qwen2.5-0.5B, TinyLlama-1.1B,
+ * Llama-3-8B: hidden size, K/V row, FFN width, head counts as constants instead of launch parameters); a context of
+ * exactly such a shape takes them: same formulas over the same rows (results agree to rounding), 1-2 % faster.  on != 0: this context only takes
+ * the variants whose sizes come with the launch (comparisons, tests).  No counterpart in the reference. */
+int mg_set_flow_generic(mg_ctx* ctx, int on);
 int mg_tokens_per_launch(mg_ctx* ctx);
 int mg_flow_tail_in_use(mg_ctx* ctx);
 int mg_flow_tail_trace(mg_ctx* ctx, long long* out, size_t cap, int* dims);

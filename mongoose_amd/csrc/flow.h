@@ -95,6 +95,7 @@ struct FlowParams {
     int gqaCode;                 // geo.gqa only: 1 = a position of this launch may need the grouped attention (the variant that can do
                                  // it is launched); 0 = none does (positions below nCompute / nHeads tiles): the plain variant, which
                                  // is faster there, runs on the same geometry and reports a position past its reach as error 3
+    int generic;                 // 1: never a variant with a known shape's sizes compiled in (comparisons, tests)
 };
 #define FLOW_TAIL_TRACE_NAMES "tail-top", "final-input-staged", "lm-head-done", "token-known", "all-waves-done", "partials-in"
 

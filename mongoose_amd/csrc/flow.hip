@@ -567,7 +567,18 @@ constexpr int NID = 8 / FWAVES;    // down rows a wave holds in flight
 // Q4: the seven matrices of a layer are Q4_0 in the split layout (the table's scale pointers then hold the d planes)
 // TRACE: the launch records its per-workgroup timeline (FlowParams::trace); the variants without it carry neither the
 //        trace points' instructions nor their scalar registers (1.2 % of the step at the 0.5B and 1.1B shapes)
-template <int HD, int CBD, bool RING, bool GQA, bool Q4, bool TRACE>
+// FIX: 0 = the sizes come with the launch; 1, 2, 3 = the sizes of a known model shape (FlowFixedShape) are constants of the
+//      variant instead of launch parameters held in scalar registers and laundered at every token and layer: addresses,
+//      trip counts and divisions fold (0.5B shape: 0.3294 -> 0.3231 ms a token).  Same formulas over the same rows; results
+//      agree with the other variants' to rounding (the compiler contracts and schedules differently).
+struct FlowFixedShape { int dim, kvDim, ffn, nHeads, nKVHeads, headDim; };
+__host__ __device__ constexpr FlowFixedShape flow_fixed_shape(int fix) {
+    return fix == 1 ? FlowFixedShape{896, 128, 4864, 14, 2, 64}            // Qwen2.5-0.5B
+         : fix == 2 ? FlowFixedShape{2048, 256, 5632, 32, 4, 64}           // TinyLlama-1.1B
+         : fix == 3 ? FlowFixedShape{4096, 1024, 14336, 32, 8, 128}        // Llama-3-8B
+                    : FlowFixedShape{0, 0, 0, 0, 0, 0};
+}
+template <int HD, int CBD, bool RING, bool GQA, bool Q4, bool TRACE, int FIX = 0>
 __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     extern __shared__ float4 a4[];                     // the staged activation vector, max(dim, ffn) floats
     __shared__ float red[FWAVES];
@@ -608,7 +619,11 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             }
         }
     };
-    int dim = p.dim, kvDim = p.kvDim, ffn = p.ffn;
+    constexpr bool FX = FIX != 0;
+    constexpr FlowFixedShape FS = flow_fixed_shape(FIX);
+    static_assert(!FX || FS.headDim == HD, "the fixed shape's head size is the variant's");
+    int dim = FX ? FS.dim : p.dim, kvDim = FX ? FS.kvDim : p.kvDim, ffn = FX ? FS.ffn : p.ffn;
+    const int nHeadsV = FX ? FS.nHeads : p.nHeads, nKVHeadsV = FX ? FS.nKVHeads : p.nKVHeads;
     int nchD = dim >> 4, nchF = ffn >> 4;
     const FlowGeometry G = p.geo;
     // (the idle lines follow the error word's 256 bytes: 16 lines of 128 bytes, two workgroups of an XCD on each)
@@ -648,13 +663,14 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
         // Nothing that depends on the thread or on the shape is to be computed once for all tokens and kept in registers
         // across the whole launch (hundreds of addresses and offsets otherwise are): every token derives them again.
         asm volatile("" : "+v"(tid), "+v"(lane));
-        asm volatile("" : "+s"(wave), "+s"(gw), "+s"(dim), "+s"(kvDim), "+s"(ffn), "+s"(nchD), "+s"(nchF));
+        if constexpr (FX) asm volatile("" : "+s"(wave), "+s"(gw));
+        else asm volatile("" : "+s"(wave), "+s"(gw), "+s"(dim), "+s"(kvDim), "+s"(ffn), "+s"(nchD), "+s"(nchF));
         float* const xb = p.xchg + (tokens ? (size_t)(pos & 1) * halfFloats : (size_t)0);
         const unsigned xoff = tokens ? (unsigned)((size_t)(pos & 1) * halfFloats) : 0u;
         if constexpr (!GQA) {
             // the plain variant on a geometry laid out for grouped attention: a position past what a workgroup per query head
             // and split covers is the host's mistake, and is reported instead of computed wrongly
-            if (G.gqa && p.nHeads * (pos / TILE + 1) > nC && blockIdx.x == 0 && tid == 0)
+            if (G.gqa && nHeadsV * (pos / TILE + 1) > nC && blockIdx.x == 0 && tid == 0)
                 __hip_atomic_store(p.err, 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         const float* cosRow = p.cosRow;
@@ -737,7 +753,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 // (the same per layer: offsets that do not depend on the layer would otherwise be kept across all phases, and
                 // the phases' own working sets then no longer fit the registers)
                 asm volatile("" : "+v"(tid), "+v"(lane));
-                asm volatile("" : "+s"(wave), "+s"(gw), "+s"(dim), "+s"(kvDim), "+s"(ffn), "+s"(nchD), "+s"(nchF));
+                if constexpr (FX) asm volatile("" : "+s"(wave), "+s"(gw));
+        else asm volatile("" : "+s"(wave), "+s"(gw), "+s"(dim), "+s"(kvDim), "+s"(ffn), "+s"(nchD), "+s"(nchF));
                 LayerView L{lw};
                 if (l + 1 < p.l1) lw = layer_words(p.layers, l + 1, lane);
                 else if (tk + 1 < nTok) lw = layer_words(p.layers, p.l0, lane);
@@ -912,23 +929,23 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 FLOW_TRACE(2);
                 // ------------------------------------------------------------------ attention: one (head, KV split) per workgroup
                 // grouped only while a workgroup per query head and split would not fit the launch (positions far into a long context)
-                const bool grouped = GQA && p.nHeads * (pos / TILE + 1) > nC;
+                const bool grouped = GQA && nHeadsV * (pos / TILE + 1) > nC;
                 {
                     const int nsplit = pos / TILE + 1;
                     // Grouped: the query heads of a KV head are shared out over as many workgroups as the launch has left for
                     // them at this position (each loads the K / V rows once and takes its heads in turn), so a workgroup takes as
                     // few heads as possible: qhMax heads a workgroup, `sub` workgroups a KV head and split.
-                    const int Gq = p.nHeads / p.nKVHeads;
+                    const int Gq = nHeadsV / nKVHeadsV;
                     int qhMax = 1, sub = Gq;
                     if (grouped) {
                         qhMax = Gq; sub = 1;
                         const int live = nsplit < G.smax ? nsplit : G.smax;
                         for (int q = 2; q < Gq; q++) {
                             const int sb = (Gq + q - 1) / q;
-                            if (p.nKVHeads * sb * live <= nC) { qhMax = q; sub = sb; break; }
+                            if (nKVHeadsV * sb * live <= nC) { qhMax = q; sub = sb; break; }
                         }
                     }
-                    const int unit = grouped ? p.nKVHeads * sub : p.nHeads;
+                    const int unit = grouped ? nKVHeadsV * sub : nHeadsV;
                     const int split = blockIdx.x / unit, hu = blockIdx.x % unit;
                     const int hg = grouped ? hu % sub : 0;                         // which of the KV head's groups of query heads
                     const int QH = grouped ? min(qhMax, Gq - hg * qhMax) : 1;      // query heads of this workgroup
@@ -943,7 +960,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     if ((p.idleWoRows > 0 || p.idleGateUpRows > 0) && nC == (int)gridDim.x) {
                         const int live = nsplit < G.smax ? nsplit : G.smax;
                         int nBusy = unit * live;
-                        if (grouped && nBusy < p.nHeads) nBusy = p.nHeads;
+                        if (grouped && nBusy < nHeadsV) nBusy = nHeadsV;
                         nBusy = (nBusy + 7) & ~7;
                         if ((int)blockIdx.x >= nBusy && 2 * ((int)gridDim.x - nBusy) >= (int)gridDim.x) {
                             Prefetcher pf{(int)blockIdx.x & 7, ((int)blockIdx.x - nBusy) >> 3, ((int)gridDim.x - nBusy) >> 3, tid, pfScrap};
@@ -1094,8 +1111,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             }
                             stx4(reinterpret_cast<f4*>(X + G.offPacc + (size_t)split * dim + h * HD) + i, r);
                             if (i == 0) {
-                                stx(X + G.offPm + split * p.nHeads + h, mg_);
-                                stx(X + G.offPl + split * p.nHeads + h, lg);
+                                stx(X + G.offPm + split * nHeadsV + h, mg_);
+                                stx(X + G.offPl + split * nHeadsV + h, lg);
                             }
                         }
                     }
@@ -1105,7 +1122,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     // Long contexts, tens of KV splits: merged once per head, by workgroup h for head h (every thread a 16-byte piece
                     // and every eighth split, eight splits' loads in flight together, then combined through LDS), and handed on as
                     // one vector -- every consumer merging all partials itself re-reads tens of KB per workgroup and layer.
-                    if ((int)blockIdx.x < p.nHeads) {
+                    if ((int)blockIdx.x < nHeadsV) {
                         constexpr int P4 = HD / 4, SG = FWG / P4;          // pieces of a head, split groups (thread = piece x group)
                         __shared__ float4 mnum[SG][P4];
                         __shared__ float mM[SG][P4], mden[SG][P4];
@@ -1126,8 +1143,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                 for (int j = 0; j < MBG; j++) {
                                     const int sj = min(s1 + j * SG, ns - 1);
                                     a[j] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (Xo + G.offPacc + (unsigned)sj * dim + h * HD + i * 4) * 4u, 0, 16));
-                                    ms[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, (Xo + G.offPm + sj * p.nHeads + h) * 4u, 0, 16));
-                                    ls[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, (Xo + G.offPl + sj * p.nHeads + h) * 4u, 0, 16));
+                                    ms[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, (Xo + G.offPm + sj * nHeadsV + h) * 4u, 0, 16));
+                                    ls[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, (Xo + G.offPl + sj * nHeadsV + h) * 4u, 0, 16));
                                 }
 #pragma unroll
                                 for (int j = 0; j < MBG; j++) missing |= unset4(a[j]) | unset1(ms[j]) | unset1(ls[j]);
@@ -1235,8 +1252,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                     for (int u = 0; u < PB; u++) {
                                         const bool on = u < nbt;
                                         pa[u] = on ? reinterpret_cast<const f4*>(X + G.offPacc + (size_t)(s0 + u) * dim) + i : wt.idle;
-                                        pm[u] = on ? X + G.offPm + (s0 + u) * p.nHeads + h : idle1;
-                                        pl[u] = on ? X + G.offPl + (s0 + u) * p.nHeads + h : idle1;
+                                        pm[u] = on ? X + G.offPm + (s0 + u) * nHeadsV + h : idle1;
+                                        pl[u] = on ? X + G.offPl + (s0 + u) * nHeadsV + h : idle1;
                                         a[u] = f4{0.f, 0.f, 0.f, 0.f};
                                     }
                                     poll_batch<false, false>(pa, a, nbt, wt);
@@ -1776,7 +1793,26 @@ hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
 #define FLOW_LAUNCH_G(HDv, CBv, RGv) do { \
         if (p.q4) { if (gqa) FLOW_LAUNCH(HDv, CBv, RGv, true, true); else FLOW_LAUNCH(HDv, CBv, RGv, false, true); } \
         else { if (gqa) FLOW_LAUNCH(HDv, CBv, RGv, true, false); else FLOW_LAUNCH(HDv, CBv, RGv, false, false); } } while (0)
-    if (p.headDim == 64) {
+    // the variants with a known shape's sizes compiled in (launches of exactly that shape, unless switched off)
+    int fix = 0;
+    if (!p.generic)
+        for (int k = 1; k <= 3 && !fix; k++) {
+            const FlowFixedShape fs = flow_fixed_shape(k);
+            if (p.dim == fs.dim && p.kvDim == fs.kvDim && p.ffn == fs.ffn && p.nHeads == fs.nHeads && p.nKVHeads == fs.nKVHeads &&
+                p.headDim == fs.headDim) fix = k;
+        }
+#define FLOW_LAUNCH_F(HDv, CBv, RGv, GQv, Q4v, FXv) do { \
+        if (p.trace) hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v, true, FXv>), dim3(grid), dim3(FWG), lds, s, p); \
+        else hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v, false, FXv>), dim3(grid), dim3(FWG), lds, s, p); } while (0)
+    if (fix == 1 && !gqa) {
+        if (p.q4) FLOW_LAUNCH_F(64, 1, false, false, true, 1);
+        else FLOW_LAUNCH_F(64, 1, false, false, false, 1);
+    } else if (fix == 2 && !gqa && !p.q4) {
+        FLOW_LAUNCH_F(64, 2, false, false, false, 2);
+    } else if (fix == 3 && !p.q4) {
+        if (gqa) FLOW_LAUNCH_F(128, 2, true, true, false, 3);
+        else FLOW_LAUNCH_F(128, 2, true, false, false, 3);
+    } else if (p.headDim == 64) {
         if (ring) FLOW_LAUNCH_G(64, 2, true);
         else if (wide) FLOW_LAUNCH_G(64, 2, false);
         else FLOW_LAUNCH_G(64, 1, false);
@@ -1785,6 +1821,7 @@ hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
         else if (wide) FLOW_LAUNCH_G(128, 2, false);
         else FLOW_LAUNCH_G(128, 1, false);
     }
+#undef FLOW_LAUNCH_F
 #undef FLOW_LAUNCH_G
 #undef FLOW_LAUNCH
     return hipGetLastError();

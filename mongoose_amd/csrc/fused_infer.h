@@ -187,6 +187,8 @@ public:
     bool flowTail = true;
     int tokensPerLaunch = 64;
     void SetFlowTail(int on) { invalidateGraphs(); flowTail = on != 0; }
+    bool flowGeneric = false;    // never the persistent launch's variants with a known shape's sizes compiled in
+    void SetFlowGeneric(int on) { invalidateGraphs(); flowGeneric = on != 0; }
     int SetTokensPerLaunch(int n);
     bool FlowTailInUse() const { return flowTailEligible(); }
     int FlowTailTrace(long long* out, size_t cap, int* dims);

@@ -883,6 +883,7 @@ int HIPFusedInference::enqueueLayersFlow(int l0, int l1, const StepState* st, in
         if (!st) posMax = posImm;
         else if (statePosHost >= 0) posMax = (long long)statePosHost + (nTokens > 0 ? nTokens - 1 : 0);
         p.gqaCode = (posMax < 0 || (long long)nHeads * (posMax / FLOW_TILE + 1) > flowCompute) ? 1 : 0;
+        p.generic = flowGeneric ? 1 : 0;
         if (st && nTokens > 0 && statePosHost >= 0) statePosHost += nTokens;          // whole tokens advance the device state
         else if (st) statePosHost = -1;                                               // (what follows this launch advances it)
     }
@@ -1820,6 +1821,7 @@ int mg_flow_tail_in_use(mg_ctx* c) {
     return c->f->FlowTailInUse() ? 1 : 0;
 }
 int mg_set_flow_tail(mg_ctx* c, int on) { CTX(c); f->SetFlowTail(on); return MG_OK; }
+int mg_set_flow_generic(mg_ctx* c, int on) { CTX(c); f->SetFlowGeneric(on); return MG_OK; }
 int mg_set_tokens_per_launch(mg_ctx* c, int n) { CTX(c); return f->SetTokensPerLaunch(n); }
 int mg_tokens_per_launch(mg_ctx* c) { return c && c->f ? c->f->tokensPerLaunch : 0; }
 int mg_flow_tail_trace(mg_ctx* c, long long* out, size_t cap, int* dims) { CTX(c); return f->FlowTailTrace(out, cap, dims); }

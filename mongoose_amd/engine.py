@@ -647,6 +647,10 @@ class HIPFusedInference:
     def SetFlowTail(self, on):
         return lib.mg_set_flow_tail(self._h, 1 if on else 0)
 
+    def SetFlowGeneric(self, on):
+        """on: only the persistent launch's variants whose sizes come with the launch (none with a known shape's compiled in)."""
+        return lib.mg_set_flow_generic(self._h, 1 if on else 0)
+
     def SetTokensPerLaunch(self, n):
         return lib.mg_set_tokens_per_launch(self._h, int(n))
 

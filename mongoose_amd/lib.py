@@ -123,6 +123,7 @@ _sig("mg_flow_exchange", c_int, c_void_p, c_int, _f, c_size_t, _i)
 _sig("mg_flow_in_use", c_int, c_void_p)
 _sig("mg_flow_tail_in_use", c_int, c_void_p)
 _sig("mg_set_flow_tail", c_int, c_void_p, c_int)
+_sig("mg_set_flow_generic", c_int, c_void_p, c_int)
 _sig("mg_set_tokens_per_launch", c_int, c_void_p, c_int)
 _sig("mg_tokens_per_launch", c_int, c_void_p)
 _sig("mg_flow_tail_trace", c_int, c_void_p, ctypes.POINTER(ctypes.c_longlong), c_size_t, _i)

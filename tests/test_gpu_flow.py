@@ -262,6 +262,43 @@ def test_prefetching_workgroups_change_nothing(hip, fmt):
     m.close()
 
 
+@pytest.mark.parametrize("name,positions", [("qwen2.5-0.5b", 300), ("qwen2.5-0.5b-q4_0", 300), ("tinyllama-1.1b", 300),
+                                            ("llama-3-8b", 1100)])
+def test_variants_with_a_shape_compiled_in_change_nothing(hip, name, positions):
+    """A context of exactly the 0.5B, 1.1B or 8B shape takes a variant of the persistent launch with that shape's sizes as
+    constants; mg_set_flow_generic keeps it on the variants whose sizes come with the launch.  Same formulas over the same
+    rows; the compiler contracts and schedules the two differently, so logits agree to rounding (1e-5 of their largest, the
+    bar between launches elsewhere in this file) and the greedy tokens are the same, token by token across the first KV
+    split boundary and in runs of tokens inside one launch (8B shape: to past position 1024, where the launch changes to
+    the grouped attention)."""
+    s = H.with_layers(configs.BY_NAME[name], 2)._replace(vocab=2048)
+    m = H.Model(s, seed=41, maxSeq=positions + 40, eng=hip, oracle=False)
+    prompt = m.prompt(8)
+    outs = {}
+    for generic in (0, 1):
+        assert m.hip.SetFlowGeneric(generic) == 0
+        assert m.hip.ResetKV() == 0
+        assert _in_use(m.hip)
+        rc, toks = m.hip.Generate(prompt, positions, useGraph=True)         # runs of 64 tokens a launch
+        assert rc == 0, E.last_error()
+        assert m.hip.FlowInUse()
+        stream = list(prompt) + [int(t) for t in toks]
+        assert m.hip.ResetKV() == 0
+        logits = np.empty(s.vocab, np.float32)
+        res = []
+        for pos in range(140):                                              # a launch a token, logits read back
+            last = pos in (0, 1, 127, 128, 139)
+            rc, nxt = m.hip.DecodeToken(stream[pos], pos, logits if last else None)
+            assert rc == 0, E.last_error()
+            if last:
+                res.append((nxt, logits.copy()))
+        outs[generic] = (toks.tolist(), res)
+    assert outs[0][0] == outs[1][0]
+    for (n0, l0), (n1, l1) in zip(outs[0][1], outs[1][1]):
+        assert n0 == n1 and H.rel_err(l0, l1) < 1e-5
+    m.close()
+
+
 def test_heads_of_128_grouped_kv(hip):
     """Llama-3-8B attention geometry (32 query heads of 128 on 8 KV heads, dim 4096: rows of two chunks a lane), 2
     layers, FFN and vocabulary cut: 8 partial slots, tile 128."""
