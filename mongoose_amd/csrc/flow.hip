@@ -578,6 +578,22 @@ __host__ __device__ constexpr FlowFixedShape flow_fixed_shape(int fix) {
          : fix == 3 ? FlowFixedShape{4096, 1024, 14336, 32, 8, 128}        // Llama-3-8B
                     : FlowFixedShape{0, 0, 0, 0, 0, 0};
 }
+// The part of a layer's exchange area whose layout follows from the sizes alone: q, current K row, current V row, hidden
+// after attention, SwiGLU vector, layer output, merged attention output, and where the KV splits' partial slots begin.
+__host__ __device__ constexpr FlowGeometry flow_geometry_head(int dim, int kvDim, int ffn) {
+    FlowGeometry g{};
+    int o = 0;
+    g.offQ = o; o += (dim + 63) & ~63;
+    g.offKc = o; o += (kvDim + 63) & ~63;
+    g.offVc = o; o += (kvDim + 63) & ~63;
+    g.offX1 = o; o += (dim + 63) & ~63;
+    g.offM = o; o += (ffn + 63) & ~63;
+    g.offX2 = o; o += (dim + 63) & ~63;
+    g.offAttn = o; o += (dim + 63) & ~63;          // attention output merged over the splits (grouped attention only)
+    g.offPacc = o;
+    return g;
+}
+
 template <int HD, int CBD, bool RING, bool GQA, bool Q4, bool TRACE, int FIX = 0>
 __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     extern __shared__ float4 a4[];                     // the staged activation vector, max(dim, ffn) floats
@@ -625,7 +641,14 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     int dim = FX ? FS.dim : p.dim, kvDim = FX ? FS.kvDim : p.kvDim, ffn = FX ? FS.ffn : p.ffn;
     const int nHeadsV = FX ? FS.nHeads : p.nHeads, nKVHeadsV = FX ? FS.nKVHeads : p.nKVHeads;
     int nchD = dim >> 4, nchF = ffn >> 4;
-    const FlowGeometry G = p.geo;
+    FlowGeometry G = p.geo;
+    // (A known shape: these are constants, not scalar registers -- 0.5B Q4_0 0.330 -> 0.3235 ms a token, 1.1B 0.3755 -> 0.372,
+    // 0.5B Q8 and 8B unchanged.)
+    if constexpr (FX) {
+        constexpr FlowGeometry GH = flow_geometry_head(FS.dim, FS.kvDim, FS.ffn);
+        G.offQ = GH.offQ; G.offKc = GH.offKc; G.offVc = GH.offVc; G.offX1 = GH.offX1; G.offM = GH.offM; G.offX2 = GH.offX2;
+        G.offAttn = GH.offAttn; G.offPacc = GH.offPacc;
+    }
     // (the idle lines follow the error word's 256 bytes: 16 lines of 128 bytes, two workgroups of an XCD on each)
     Waiter wt{p.limitTicks, p.err, false, reinterpret_cast<const f4*>(reinterpret_cast<const char*>(p.err) + 256 + ((blockIdx.x >> 3) & 15) * 128)};
 
@@ -1724,18 +1747,15 @@ FlowGeometry flow_geometry(int dim, int kvDim, int ffn, int nHeads, int nKVHeads
     g.smax = want;
     if (unit > 0 && g.smax > grid / unit) g.smax = grid / unit;
     if (g.smax < 1) g.smax = 1;
+    // the vectors whose place depends on the sizes alone come first (a variant with a known shape has them as constants),
+    // the partial slots, which grow with the context, last
     auto up64 = [](int v) { return (v + 63) & ~63; };
-    int o = 0;
-    g.offQ = o; o += up64(dim);
-    g.offKc = o; o += up64(kvDim);
-    g.offVc = o; o += up64(kvDim);
-    g.offPacc = o; o += up64(g.smax * dim);
+    const FlowGeometry h = flow_geometry_head(dim, kvDim, ffn);
+    g.offQ = h.offQ; g.offKc = h.offKc; g.offVc = h.offVc; g.offX1 = h.offX1; g.offM = h.offM; g.offX2 = h.offX2;
+    g.offAttn = h.offAttn; g.offPacc = h.offPacc;
+    int o = g.offPacc + up64(g.smax * dim);
     g.offPm = o; o += up64(g.smax * nHeads);
     g.offPl = o; o += up64(g.smax * nHeads);
-    g.offX1 = o; o += up64(dim);
-    g.offM = o; o += up64(ffn);
-    g.offX2 = o; o += up64(dim);
-    g.offAttn = o; o += up64(dim);          // attention output merged over the splits (grouped attention only)
     g.stride = o;
     return g;
 }
