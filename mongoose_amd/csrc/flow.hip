@@ -571,12 +571,12 @@ constexpr int NID = 8 / FWAVES;    // down rows a wave holds in flight
 //      variant instead of launch parameters held in scalar registers and laundered at every token and layer: addresses,
 //      trip counts and divisions fold (0.5B shape: 0.3294 -> 0.3231 ms a token).  Same formulas over the same rows; results
 //      agree with the other variants' to rounding (the compiler contracts and schedules differently).
-struct FlowFixedShape { int dim, kvDim, ffn, nHeads, nKVHeads, headDim; };
+struct FlowFixedShape { int dim, kvDim, ffn, nHeads, nKVHeads, headDim, downSplit; };
 __host__ __device__ constexpr FlowFixedShape flow_fixed_shape(int fix) {
-    return fix == 1 ? FlowFixedShape{896, 128, 4864, 14, 2, 64}            // Qwen2.5-0.5B
-         : fix == 2 ? FlowFixedShape{2048, 256, 5632, 32, 4, 64}           // TinyLlama-1.1B
-         : fix == 3 ? FlowFixedShape{4096, 1024, 14336, 32, 8, 128}        // Llama-3-8B
-                    : FlowFixedShape{0, 0, 0, 0, 0, 0};
+    return fix == 1 ? FlowFixedShape{896, 128, 4864, 14, 2, 64, 1}         // Qwen2.5-0.5B
+         : fix == 2 ? FlowFixedShape{2048, 256, 5632, 32, 4, 64, 0}        // TinyLlama-1.1B
+         : fix == 3 ? FlowFixedShape{4096, 1024, 14336, 32, 8, 128, 0}     // Llama-3-8B
+                    : FlowFixedShape{0, 0, 0, 0, 0, 0, 0};
 }
 // The part of a layer's exchange area whose layout follows from the sizes alone: q, current K row, current V row, hidden
 // after attention, SwiGLU vector, layer output, merged attention output, and where the KV splits' partial slots begin.
@@ -636,10 +636,17 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
         }
     };
     constexpr bool FX = FIX != 0;
-    constexpr FlowFixedShape FS = flow_fixed_shape(FIX);
+    constexpr FlowFixedShape FS = flow_fixed_shape(FIX & 7);
     static_assert(!FX || FS.headDim == HD, "the fixed shape's head size is the variant's");
     int dim = FX ? FS.dim : p.dim, kvDim = FX ? FS.kvDim : p.kvDim, ffn = FX ? FS.ffn : p.ffn;
     const int nHeadsV = FX ? FS.nHeads : p.nHeads, nKVHeadsV = FX ? FS.nKVHeads : p.nKVHeads;
+    // (known shapes: whether two waves share a row of the down projection follows from the sizes and the launch's 2048
+    // waves; the caches hold fp32 rows unless the variant's code says fp16 -- both are branches between whole code paths)
+    // Measured per variant, ms a token with / without: 0.5B Q8 0.3141 / 0.3230, 8B 1.558 / 1.561 (fp16 rows at 4,000
+    // positions 1.841 / 1.847), 0.5B Q4_0 0.3235 / 0.3230, 1.1B 0.378 / 0.372 -- the last two keep them in registers.
+    constexpr bool FXF = FX && (((FIX & 7) == 1 && !Q4) || (FIX & 7) == 3);
+    const bool downSplitV = FXF ? FS.downSplit != 0 : p.downSplit != 0;
+    const bool kvHalfV = FXF ? (FIX & 8) != 0 : p.kvHalf != 0;
     int nchD = dim >> 4, nchF = ffn >> 4;
     FlowGeometry G = p.geo;
     // (A known shape: these are constants, not scalar registers -- 0.5B Q4_0 0.330 -> 0.3235 ms a token, 1.1B 0.3755 -> 0.372,
@@ -756,7 +763,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     // the K / V rows of the earlier positions (the attention workgroups of every XCD read them; the row of the
                     // current position comes through the exchange area), while they are a small part of an L2: 0.5B shape at
                     // positions 16 .. 216 0.3766 -> 0.3710 ms a token
-                    const size_t kvBytes = (size_t)pos * kvDim * (p.kvHalf ? 2 : 4);
+                    const size_t kvBytes = (size_t)pos * kvDim * (kvHalfV ? 2 : 4);
                     if (kvBytes <= ((size_t)512 << 10)) { pf.whole(L.Kc(), kvBytes); pf.whole(L.Vc(), kvBytes); }
                 }
                 release(G.offM);               // ... past its gate | up: gate | up of this one
@@ -766,7 +773,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                 else { pf.whole(L.sgate(), (size_t)ffn * 4); pf.whole(L.sup(), (size_t)ffn * 4); }
                 pf.whole(L.g2(), (size_t)dim * 4);
                 release(G.offX2);              // ... done: the down projection of this one
-                const int drun = p.downSplit ? FWAVES / 2 : FWAVES;      // rows of the down projection a workgroup takes
+                const int drun = downSplitV ? FWAVES / 2 : FWAVES;      // rows of the down projection a workgroup takes
                 pf.rows(L.down(), rbF, dim, drun);
                 if (Q4) pf.rows(L.sdown(), rdF, dim, drun); else pf.whole(L.sdown(), (size_t)dim * 4);
             }
@@ -833,7 +840,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                                     } else {                                              // mongoose.cu:1644-1647, and the hand-over copy
                                         // (write-through: the next token of the same launch reads the row on other XCDs)
                                         float oc = o;
-                                        if (p.kvHalf) {           // fp16 rows: rounded where written; the hand-over copy carries the rounded value
+                                        if (kvHalfV) {           // fp16 rows: rounded where written; the hand-over copy carries the rounded value
                                             const _Float16 hv = (_Float16)o;
                                             oc = (float)hv;
                                             const _Float16* dst = reinterpret_cast<const _Float16*>(kk == 1 ? L.Kc() : L.Vc()) + (size_t)pos * kvDim + r;
@@ -1019,7 +1026,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                         // row has been written -- in token mode that row is written later in this same launch, by a workgroup of
                         // another XCD, and a line fetched early would be served stale from then on.
                         const float4* idle4 = reinterpret_cast<const float4*>(wt.idle) + dl;
-                        if (p.kvHalf) {
+                        if (kvHalfV) {
                             // fp16 rows: a lane's piece is four halves (8 bytes), widened as it arrives
                             typedef _Float16 h4 __attribute__((ext_vector_type(4)));
                             const int2* Kh = reinterpret_cast<const int2*>(L.Kc());
@@ -1445,7 +1452,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                             }
                             store_runs(e1 + v * e0, (nI + W - 1) / W, nI, 0, X + G.offX2, l == p.l1 - 1 ? p.hidden : nullptr);
                         }
-                    } else if (p.downSplit) {
+                    } else if (downSplitV) {
                         // Few rows (at most half as many as computing waves): a row is shared by two neighbouring waves of a
                         // workgroup, each taking half of its chunks, and every workgroup with rows has half as many -- the
                         // multiplications of this phase, its longest rows, take half as long (0.5B shape 0.366 -> 0.360 ms a
@@ -1819,19 +1826,21 @@ hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
         for (int k = 1; k <= 3 && !fix; k++) {
             const FlowFixedShape fs = flow_fixed_shape(k);
             if (p.dim == fs.dim && p.kvDim == fs.kvDim && p.ffn == fs.ffn && p.nHeads == fs.nHeads && p.nKVHeads == fs.nKVHeads &&
-                p.headDim == fs.headDim) fix = k;
+                p.headDim == fs.headDim && (p.downSplit != 0) == (fs.downSplit != 0)) fix = k;
         }
 #define FLOW_LAUNCH_F(HDv, CBv, RGv, GQv, Q4v, FXv) do { \
         if (p.trace) hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v, true, FXv>), dim3(grid), dim3(FWG), lds, s, p); \
         else hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v, false, FXv>), dim3(grid), dim3(FWG), lds, s, p); } while (0)
-    if (fix == 1 && !gqa) {
+    if (fix == 1 && !gqa && !p.kvHalf) {
         if (p.q4) FLOW_LAUNCH_F(64, 1, false, false, true, 1);
         else FLOW_LAUNCH_F(64, 1, false, false, false, 1);
-    } else if (fix == 2 && !gqa && !p.q4) {
+    } else if (fix == 2 && !gqa && !p.q4 && !p.kvHalf) {
         FLOW_LAUNCH_F(64, 2, false, false, false, 2);
-    } else if (fix == 3 && !p.q4) {
+    } else if (fix == 3 && !p.q4 && !p.kvHalf) {
         if (gqa) FLOW_LAUNCH_F(128, 2, true, true, false, 3);
         else FLOW_LAUNCH_F(128, 2, true, false, false, 3);
+    } else if (fix == 3 && !p.q4 && gqa) {              // fp16 K / V rows at a long context
+        FLOW_LAUNCH_F(128, 2, true, true, false, 11);
     } else if (p.headDim == 64) {
         if (ring) FLOW_LAUNCH_G(64, 2, true);
         else if (wide) FLOW_LAUNCH_G(64, 2, false);

@@ -262,17 +262,18 @@ def test_prefetching_workgroups_change_nothing(hip, fmt):
     m.close()
 
 
-@pytest.mark.parametrize("name,positions", [("qwen2.5-0.5b", 300), ("qwen2.5-0.5b-q4_0", 300), ("tinyllama-1.1b", 300),
-                                            ("llama-3-8b", 1100)])
-def test_variants_with_a_shape_compiled_in_change_nothing(hip, name, positions):
+@pytest.mark.parametrize("name,positions,kv_f16", [("qwen2.5-0.5b", 300, False), ("qwen2.5-0.5b-q4_0", 300, False),
+                                                   ("tinyllama-1.1b", 300, False), ("llama-3-8b", 1100, False),
+                                                   ("llama-3-8b", 1100, True)])
+def test_variants_with_a_shape_compiled_in_change_nothing(hip, name, positions, kv_f16):
     """A context of exactly the 0.5B, 1.1B or 8B shape takes a variant of the persistent launch with that shape's sizes as
     constants; mg_set_flow_generic keeps it on the variants whose sizes come with the launch.  Same formulas over the same
     rows; the compiler contracts and schedules the two differently, so logits agree to rounding (1e-5 of their largest, the
     bar between launches elsewhere in this file) and the greedy tokens are the same, token by token across the first KV
     split boundary and in runs of tokens inside one launch (8B shape: to past position 1024, where the launch changes to
-    the grouped attention)."""
+    the grouped attention, with fp32 and with fp16 K/V rows)."""
     s = H.with_layers(configs.BY_NAME[name], 2)._replace(vocab=2048)
-    m = H.Model(s, seed=41, maxSeq=positions + 40, eng=hip, oracle=False)
+    m = H.Model(s, seed=41, maxSeq=positions + 40, eng=hip, oracle=False, kv_f16=kv_f16)
     prompt = m.prompt(8)
     outs = {}
     for generic in (0, 1):
