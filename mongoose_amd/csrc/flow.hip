@@ -571,12 +571,12 @@ constexpr int NID = 8 / FWAVES;    // down rows a wave holds in flight
 //      variant instead of launch parameters held in scalar registers and laundered at every token and layer: addresses,
 //      trip counts and divisions fold (0.5B shape: 0.3294 -> 0.3231 ms a token).  Same formulas over the same rows; results
 //      agree with the other variants' to rounding (the compiler contracts and schedules differently).
-struct FlowFixedShape { int dim, kvDim, ffn, nHeads, nKVHeads, headDim, downSplit; };
+struct FlowFixedShape { int dim, kvDim, ffn, nHeads, nKVHeads, headDim, downSplit, dedicated; };
 __host__ __device__ constexpr FlowFixedShape flow_fixed_shape(int fix) {
-    return fix == 1 ? FlowFixedShape{896, 128, 4864, 14, 2, 64, 1}         // Qwen2.5-0.5B
-         : fix == 2 ? FlowFixedShape{2048, 256, 5632, 32, 4, 64, 0}        // TinyLlama-1.1B
-         : fix == 3 ? FlowFixedShape{4096, 1024, 14336, 32, 8, 128, 0}     // Llama-3-8B
-                    : FlowFixedShape{0, 0, 0, 0, 0, 0, 0};
+    return fix == 1 ? FlowFixedShape{896, 128, 4864, 14, 2, 64, 1, 1}      // Qwen2.5-0.5B
+         : fix == 2 ? FlowFixedShape{2048, 256, 5632, 32, 4, 64, 0, 0}     // TinyLlama-1.1B
+         : fix == 3 ? FlowFixedShape{4096, 1024, 14336, 32, 8, 128, 0, 0}  // Llama-3-8B
+                    : FlowFixedShape{0, 0, 0, 0, 0, 0, 0, 0};
 }
 // The part of a layer's exchange area whose layout follows from the sizes alone: q, current K row, current V row, hidden
 // after attention, SwiGLU vector, layer output, merged attention output, and where the KV splits' partial slots begin.
@@ -645,6 +645,10 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     // Measured per variant, ms a token with / without: 0.5B Q8 0.3141 / 0.3230, 8B 1.558 / 1.561 (fp16 rows at 4,000
     // positions 1.841 / 1.847), 0.5B Q4_0 0.3235 / 0.3230, 1.1B 0.378 / 0.372 -- the last two keep them in registers.
     constexpr bool FXF = FX && (((FIX & 7) == 1 && !Q4) || (FIX & 7) == 3);
+    constexpr bool FXD = FX && (FIX & 7) == 1;        // (0.5B Q4_0 0.3267 -> 0.3204 ms a token, Q8 0.3141 -> 0.3138; the others gain nothing)
+    // whether workgroups past the computing ones prefetch (then none prefetches while idle during the attention): of the
+    // two roles a known shape has one, the other's code is not in its variant
+    const bool hasPrefetchers = FXD ? FS.dedicated != 0 : nC != (int)gridDim.x;
     const bool downSplitV = FXF ? FS.downSplit != 0 : p.downSplit != 0;
     const bool kvHalfV = FXF ? (FIX & 8) != 0 : p.kvHalf != 0;
     int nchD = dim >> 4, nchF = ffn >> 4;
@@ -717,7 +721,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
             __syncthreads();
         }
 
-        if ((int)blockIdx.x >= nC) {
+        if (hasPrefetchers && (int)blockIdx.x >= nC) {
             // ---- prefetch role (see Prefetcher): per layer three jobs, each released by a vector of the layer before ----
             const int pi = (int)blockIdx.x - nC;
             Prefetcher pf{pi & 7, pi >> 3, ((int)gridDim.x - nC) >> 3, tid, pfScrap};
@@ -987,7 +991,7 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
                     // 0.470), else half of the first round of rows, which is what a phase waits for before it streams (8B shape
                     // with both: 1.845 -> 1.790; the whole first round 1.804, a quarter 1.800).
                     // Only while at least half the launch is idle (short contexts), and only without dedicated prefetchers.
-                    if ((p.idleWoRows > 0 || p.idleGateUpRows > 0) && nC == (int)gridDim.x) {
+                    if (!hasPrefetchers && (p.idleWoRows > 0 || p.idleGateUpRows > 0)) {
                         const int live = nsplit < G.smax ? nsplit : G.smax;
                         int nBusy = unit * live;
                         if (grouped && nBusy < nHeadsV) nBusy = nHeadsV;
@@ -1826,7 +1830,7 @@ hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
         for (int k = 1; k <= 3 && !fix; k++) {
             const FlowFixedShape fs = flow_fixed_shape(k);
             if (p.dim == fs.dim && p.kvDim == fs.kvDim && p.ffn == fs.ffn && p.nHeads == fs.nHeads && p.nKVHeads == fs.nKVHeads &&
-                p.headDim == fs.headDim && (p.downSplit != 0) == (fs.downSplit != 0)) fix = k;
+                p.headDim == fs.headDim && (p.downSplit != 0) == (fs.downSplit != 0) && (k != 1 || (nC != grid) == (fs.dedicated != 0))) fix = k;
         }
 #define FLOW_LAUNCH_F(HDv, CBv, RGv, GQv, Q4v, FXv) do { \
         if (p.trace) hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v, true, FXv>), dim3(grid), dim3(FWG), lds, s, p); \
