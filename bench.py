@@ -45,10 +45,10 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
 # "traffic_source" / "traffic_note" in the output say which it was.
 PMC_TRAFFIC_BYTES = {
     # the launch that runs whole tokens: bytes a TOKEN (all timed launches' counters over their tokens)
-    ("qwen2.5-0.5b", "token"): int(((16432663.6 + 16825804.6 + 17254655.8 + 2184860.8) * (262144.0 / 131090.0)
-                                    + (167463.2 + 168969.3 + 174229.8 + 21776.3)) * 1024 / 200),
-    ("tinyllama-1.1b", "token"): int((26419379.1 * (262144.0 / 131090.0) + 144818.5) * 1024 / 50),
-    ("llama-3-8b", "token"): int((239340691.1 * (262144.0 / 131090.0) + 621317.0) * 1024 / 64),
+    ("qwen2.5-0.5b", "token"): int(((16441105.4 + 16837552.8 + 17269667.3 + 2186685.6) * (262144.0 / 131090.0)
+                                    + (168650.8 + 170183.7 + 175082.7 + 22744.8)) * 1024 / 200),
+    ("tinyllama-1.1b", "token"): int((26422361.4 * (262144.0 / 131090.0) + 144851.5) * 1024 / 50),
+    ("llama-3-8b", "token"): int((239270332.8 * (262144.0 / 131090.0) + 622790.0) * 1024 / 64),
     # separate launches (--no-flow-tail, --exec-mode 1): bytes a launch
     ("qwen2.5-0.5b", "lm_head"): int((67135.1 * (262144.0 / 131102.4) + 660.5 * 1.0) * 1024),
     ("qwen2.5-0.5b", "flow"): int((190867.0 * (262144.0 / 131102.4) + 952.0 * 1.0) * 1024),
