@@ -685,7 +685,8 @@ __global__ __launch_bounds__(FWG) void flow_layers_kernel(FlowParams p) {
     // then has two halves, used by even and by odd positions: during a token's tail all workgroups reset the other
     // half for the token after it.  (Nothing of the token before is read any more once a workgroup has got there:
     // every workgroup reads every workgroup's argmax partial, so a token starts only when all are through the last.)
-    const bool tokens = p.nTokens > 0;
+    // (known shapes, bit 16 of FIX: the launch runs whole tokens -- the layers-only form's code is not in the variant)
+    const bool tokens = (FIX & 16) ? true : p.nTokens > 0;
     const int nTok = tokens ? p.nTokens : 1;
     const unsigned tw = tokens ? tail_words(p.tail, lane) : 0u;
     int pos = p.state ? p.state->pos : p.posImm;
@@ -1837,6 +1838,8 @@ hipError_t launch_flow_layers(const FlowParams& p, int grid, hipStream_t s) {
         else hipLaunchKernelGGL((flow_layers_kernel<HDv, CBv, RGv, GQv, Q4v, false, FXv>), dim3(grid), dim3(FWG), lds, s, p); } while (0)
     if (fix == 1 && !gqa && !p.kvHalf) {
         if (p.q4) FLOW_LAUNCH_F(64, 1, false, false, true, 1);
+        else if (p.nTokens > 0 && !p.trace)             // (whole tokens as a constant: 0.3140 -> 0.3130 ms a token; slower in the other variants)
+            hipLaunchKernelGGL((flow_layers_kernel<64, 1, false, false, false, false, 17>), dim3(grid), dim3(FWG), lds, s, p);
         else FLOW_LAUNCH_F(64, 1, false, false, false, 1);
     } else if (fix == 2 && !gqa && !p.q4 && !p.kvHalf) {
         FLOW_LAUNCH_F(64, 2, false, false, false, 2);
