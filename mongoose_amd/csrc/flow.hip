@@ -567,10 +567,11 @@ constexpr int NID = 8 / FWAVES;    // down rows a wave holds in flight
 // Q4: the seven matrices of a layer are Q4_0 in the split layout (the table's scale pointers then hold the d planes)
 // TRACE: the launch records its per-workgroup timeline (FlowParams::trace); the variants without it carry neither the
 //        trace points' instructions nor their scalar registers (1.2 % of the step at the 0.5B and 1.1B shapes)
-// FIX: 0 = the sizes come with the launch; 1, 2, 3 = the sizes of a known model shape (FlowFixedShape) are constants of the
-//      variant instead of launch parameters held in scalar registers and laundered at every token and layer: addresses,
-//      trip counts and divisions fold (0.5B shape: 0.3294 -> 0.3231 ms a token).  Same formulas over the same rows; results
-//      agree with the other variants' to rounding (the compiler contracts and schedules differently).
+// FIX: 0 = the sizes come with the launch; low three bits 1, 2, 3 = the sizes of a known model shape (FlowFixedShape) are
+//      constants of the variant instead of launch parameters held in scalar registers and laundered at every token and layer:
+//      addresses, trip counts and divisions fold (0.5B shape: 0.3294 -> 0.3231 ms a token).  Bit 8: the caches hold fp16 rows;
+//      bit 16: the launch runs whole tokens (FlowParams::nTokens > 0).  Same formulas over the same rows; results agree with
+//      the other variants' to rounding (the compiler contracts and schedules differently).  launch_flow_layers picks them.
 struct FlowFixedShape { int dim, kvDim, ffn, nHeads, nKVHeads, headDim, downSplit, dedicated; };
 __host__ __device__ constexpr FlowFixedShape flow_fixed_shape(int fix) {
     return fix == 1 ? FlowFixedShape{896, 128, 4864, 14, 2, 64, 1, 1}      // Qwen2.5-0.5B
