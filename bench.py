@@ -47,7 +47,7 @@ PMC_TRAFFIC_BYTES = {
     # the launch that runs whole tokens: bytes a TOKEN (all timed launches' counters over their tokens)
     ("qwen2.5-0.5b", "token"): int(((16442513.9 + 16834705.5 + 17266254.7 + 2186297.5) * (262144.0 / 131090.0)
                                     + (168980.9 + 170548.5 + 175650.0 + 22851.3)) * 1024 / 200),
-    ("tinyllama-1.1b", "token"): int((26422361.4 * (262144.0 / 131090.0) + 144851.5) * 1024 / 50),
+    ("tinyllama-1.1b", "token"): int((26410817.8 * (262144.0 / 131090.0) + 144870.5) * 1024 / 50),
     ("llama-3-8b", "token"): int((239270332.8 * (262144.0 / 131090.0) + 622790.0) * 1024 / 64),
     # separate launches (--no-flow-tail, --exec-mode 1): bytes a launch
     ("qwen2.5-0.5b", "lm_head"): int((67135.1 * (262144.0 / 131102.4) + 660.5 * 1.0) * 1024),
